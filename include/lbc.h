@@ -1,0 +1,151 @@
+/*
+ * lbc.h - C ABI of the MI355X (gfx950) low-bit communication codec.
+ *
+ * Plain pointers and sizes only; every pointer is a DEVICE pointer on the
+ * current HIP device unless stated otherwise, every launch is asynchronous on
+ * the `stream` argument (a hipStream_t passed as void*; NULL = the null
+ * stream), nothing here allocates, frees, synchronises or keeps global state
+ * besides a per-thread error string.  Inputs are never written.
+ *
+ * Wire format ("format A", the reference's portable codec,
+ * ccdl_comm/quantization/torch_fallback.py:24-36): for a flat tensor of n
+ * elements and group size g, G = ceil(n/g) groups;
+ *   codes  int8[G*g]   natural element order, the tail group zero padded;
+ *   scales float[G]    max(absmax/127, 2^-23) per group, IEEE division.
+ * A packed payload is uint8[codes || scales] (ccdl_comm/communication/
+ * payload_packing.py:63-68); passing codes = base and
+ * scales = base + G*g writes or reads that layout with no copy.
+ *
+ * Return values: LBC_OK (0) the work was enqueued (or there was nothing to
+ * do); LBC_UNSUPPORTED (1) the arguments are valid but this build has no
+ * kernel for them - the caller should take its own fallback, as with the
+ * reference's `return false` (ccdl_comm/csrc/quantization/
+ * quant_pack_kernel.cu:231-239); negative = contract violation, text in
+ * lbc_last_error() - the reference raises through TORCH_CHECK there.
+ */
+#ifndef LBC_H
+#define LBC_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LBC_ABI_VERSION 1
+
+enum { LBC_OK = 0, LBC_UNSUPPORTED = 1, LBC_EINVAL = -1, LBC_ELAUNCH = -2 };
+
+/* element types: ccdl_comm/csrc/pybind.cpp:148-165 (DType) */
+enum { LBC_F32 = 0, LBC_F16 = 1, LBC_BF16 = 2, LBC_NONE = -1 };
+
+/* ccdl_comm/csrc/pybind.cpp:148-165 (ReduceOP) */
+enum { LBC_REDUCE_NONE = 0, LBC_REDUCE_SUM = 1, LBC_REDUCE_MAX = 2, LBC_REDUCE_MIN = 3 };
+
+#define LBC_MAX_PAYLOADS 8 /* ccdl_comm/csrc/quantization/dequant_reduce_kernel.cu:73-80,251 */
+
+int lbc_abi_version(void);
+
+/* Text of the last negative return on the calling thread ("" if none). */
+const char *lbc_last_error(void);
+
+/*
+ * Quantize + pack, optionally fused with error feedback.
+ * Replaces: quantize_tensor_fallback (ccdl_comm/quantization/torch_fallback.py:10-36),
+ * native inplace_quantize_pack (ccdl_comm/csrc/quantization/quant_pack_kernel.cu:220-275),
+ * and, with the optional outputs, the local round trip of DDPBucketProcessor.process
+ * (ccdl_comm/communication/ddp.py:69-97) plus ErrorFeedbackState.compensate/update
+ * (ccdl_comm/quantization/error_feedback.py:27-41).
+ *
+ *   p        = x                       (residual == NULL)
+ *            = x + residual            (torch promotion: any fp32 operand -> fp32 sum;
+ *                                       two equal 16-bit types -> sum rounded to that type)
+ *   scale_g  = max(absmax_g(p)/127, 2^-23);  code = sat8(rint(p/scale_g)), NaN -> 0
+ *   restored = code*scale_g rounded to restored_dtype          (written if restored != NULL)
+ *   new_residual = p - restored, rounded to new_residual_dtype (written if new_residual != NULL)
+ *
+ * new_residual may alias residual (in-place update).  codes must hold G*g bytes
+ * and scales G floats (4-byte aligned).  Supported: group_size in {16,32,64};
+ * x_dtype any; residual_dtype in {LBC_NONE, LBC_F32, x_dtype}; restored_dtype in
+ * {LBC_F32, x_dtype}; new_residual_dtype must equal the torch promotion of p's
+ * type and restored_dtype.  Other combinations return LBC_UNSUPPORTED.
+ */
+int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residual_dtype,
+                   int64_t numel, int group_size, int8_t *codes, float *scales,
+                   void *new_residual, int new_residual_dtype, void *restored, int restored_dtype,
+                   void *stream);
+
+/*
+ * Quantize `world` equal destination chunks of one flat bucket in a single
+ * launch.  Replaces the per-chunk loop of the compressed reduce-scatter
+ * transport (ccdl_comm/communication/reduce_scatter_transport.py:252-276,
+ * 499-519) over the chunk plan of ccdl_comm/cuda/transports/
+ * compressed_reduce_scatter.py:72-94: shard_numel = ceil(numel/world); the
+ * bucket is treated as zero padded to world*shard_numel; chunk d covers
+ * [d*shard_numel, (d+1)*shard_numel) and its groups restart at its first
+ * element.  Payload d is written packed at payloads + d*payload_stride:
+ * int8 codes[Gs*g] then float scales[Gs], Gs = ceil(shard_numel/g).
+ * payload_stride >= Gs*(g+4) and a multiple of 4.
+ */
+int lbc_quant_pack_chunks(const void *x, int x_dtype, int64_t numel, int world, int group_size,
+                          uint8_t *payloads, int64_t payload_stride, void *stream);
+
+/*
+ * Decode one payload: out[i] (op)= float(code[i]) * scale[i/g], rounded to out_dtype.
+ * Replaces: dequantize_tensor_fallback (ccdl_comm/quantization/torch_fallback.py:39-53)
+ * and native inplace_dequantize with its ReduceOP (ccdl_comm/csrc/quantization/
+ * dequant_kernel_fp32.cuh:106-120).  reduce_op NONE overwrites; SUM/MAX/MIN combine
+ * with the value already in out (in out_dtype arithmetic).  numel need not be a
+ * multiple of group_size; exactly numel elements are written.
+ */
+int lbc_dequant(const int8_t *codes, const float *scales, int64_t numel, int group_size,
+                void *out, int out_dtype, int reduce_op, void *stream);
+
+/*
+ * Fused dequant-reduce of `world` payloads (1..8) into one tensor, in the
+ * order given, optionally fused with mean and error-feedback update.
+ * Replaces: CompressedAllGatherReduce.run + _sum_tensors (ccdl_comm/communication/
+ * gather_reduce.py:27-45); native try_inplace_dequantize_reduce_fused,
+ * inplace_dequantize_reduce_mean and
+ * inplace_dequantize_reduce_mean_update_error_feedback (ccdl_comm/csrc/quantization/
+ * dequant_reduce_kernel.cu:71-134,150-221,315-430).
+ *
+ *   t_r   = float(code_r[i]) * scale_r[i/g]   rounded to out_dtype
+ *   acc   = t_0;  acc = acc + t_r             each sum rounded to out_dtype, r = 1..world-1
+ *   out   = acc                                (divisor == 1)
+ *         = acc / divisor                      IEEE division in out_dtype arithmetic
+ *   new_residual[i] = prepared[i] - out[i]     (if prepared != NULL; prepared_dtype must
+ *                                               equal out_dtype, as must new_residual's)
+ *
+ * codes[] / scales[] are HOST arrays of `world` device pointers (copied by value
+ * into the launch).  divisor must be > 0.  world > 8 returns LBC_UNSUPPORTED.
+ */
+int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, int world,
+                       int64_t numel, int group_size, float divisor, void *out, int out_dtype,
+                       const void *prepared, void *new_residual, void *stream);
+
+/*
+ * Decode `world` payloads into `world` consecutive shards of one flat tensor in a
+ * single launch (the all-gather leg: ccdl_comm/communication/topology_transport.py:
+ * 866-894 decodes every gathered shard payload into its slot).  Payload d is
+ * packed at payloads + d*payload_stride as written by lbc_quant_pack_chunks for a
+ * shard of shard_numel elements; shard d lands at out + d*shard_numel; only the
+ * first total_numel elements of the concatenation are written.
+ */
+int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world,
+                       int64_t shard_numel, int64_t total_numel, int group_size, void *out,
+                       int out_dtype, void *stream);
+
+/*
+ * residual = prepared - restored, element-wise, subtraction in fp32, rounded to
+ * residual_dtype.  Replaces native inplace_error_feedback_update (ccdl_comm/csrc/
+ * quantization/dequant_reduce_kernel.cu:136-148,223-233,266-313) and
+ * ErrorFeedbackState.update (ccdl_comm/quantization/error_feedback.py:38-41).
+ */
+int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored, int restored_dtype,
+                  void *residual, int residual_dtype, int64_t numel, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LBC_H */

@@ -1,0 +1,368 @@
+// Decode-side kernels for gfx950: fused dequant-reduce of up to 8 payloads
+// (optionally with mean and error-feedback update), single/multi-chunk decode
+// with a reduce op, and the standalone error-feedback update.
+//
+// Mapping.  One lane owns VEC consecutive output elements: 4 for fp32 output
+// (one dword of codes per payload in, one 16-byte store out) and 8 for 16-bit
+// output (8 bytes of codes in, 16 bytes out), so every wavefront load and store
+// is one contiguous run and the output - the largest stream - leaves as 1 KiB
+// per wavefront instruction.  The lanes of one group read its scale from the
+// same address (a broadcast load).  The payload pointers travel by value in the
+// kernel argument block; all loads of an unrolled step are issued before the
+// arithmetic starts.
+//
+// Semantics follow the reference's portable path: decode each payload with one
+// rounding (ccdl_comm/quantization/torch_fallback.py:48-53) and add them left to
+// right in list order (ccdl_comm/communication/gather_reduce.py:39-45) in the
+// output dtype; "mean" is a true division.  The translation unit is compiled
+// with -ffp-contract=off so that no product/sum pair is fused into an FMA.
+#include "device_utils.h"
+#include "launch.h"
+
+namespace lbc {
+namespace {
+
+template <typename OT> struct decode_tiling {
+    static constexpr int VEC = sizeof(OT) == 4 ? 4 : 8;
+    static constexpr int TILE = kWave * VEC;
+    static constexpr int UNROLL = 4;
+    static constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock * UNROLL;
+};
+
+template <int VEC, bool ALIGNED>
+__device__ __forceinline__ void load_codes(const int8_t *__restrict__ p, uint32_t (&w)[VEC / 4]) {
+    if constexpr (ALIGNED) {
+        load_vec<uint32_t, VEC / 4, true>(reinterpret_cast<const uint32_t *>(p), w);
+    } else {
+#pragma unroll
+        for (int k = 0; k < VEC / 4; ++k) {
+            const uint8_t *b = reinterpret_cast<const uint8_t *>(p) + 4 * k;
+            w[k] = static_cast<uint32_t>(b[0]) | (static_cast<uint32_t>(b[1]) << 8) |
+                   (static_cast<uint32_t>(b[2]) << 16) | (static_cast<uint32_t>(b[3]) << 24);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// fused dequant-reduce
+// ---------------------------------------------------------------------------
+template <typename OT, int G, int W, bool ALIGNED>
+__global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs a) {
+    using T = decode_tiling<OT>;
+    constexpr int VEC = T::VEC;
+    constexpr int UNROLL = T::UNROLL;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t block_first = static_cast<int64_t>(blockIdx.x) * T::BLOCK_ELEMS;
+    OT *__restrict__ out = static_cast<OT *>(a.out);
+    const OT *prepared = static_cast<const OT *>(a.prepared);  // may alias new_r
+    OT *new_r = static_cast<OT *>(a.new_residual);
+    const bool mean = a.divisor != 1.0f;
+
+    if (block_first + T::BLOCK_ELEMS <= a.numel) {
+        // ---- interior block ---------------------------------------------------
+        uint32_t words[UNROLL][W][VEC / 4];
+        float scale[UNROLL][W];
+        int64_t e0[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            e0[u] = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
+            const int64_t g = e0[u] / G;
+#pragma unroll
+            for (int r = 0; r < W; ++r) {
+                load_codes<VEC, ALIGNED>(a.codes[r] + e0[u], words[u][r]);
+                scale[u][r] = a.scales[r][g];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            float acc[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = round_through<OT>(code_to_float(words[u][0][i / 4], i % 4) * scale[u][0]);
+#pragma unroll
+            for (int r = 1; r < W; ++r) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const float t = round_through<OT>(code_to_float(words[u][r][i / 4], i % 4) * scale[u][r]);
+                    acc[i] = round_through<OT>(acc[i] + t);
+                }
+            }
+            if (mean) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[i] = round_through<OT>(acc[i] / a.divisor);
+            }
+            OT o[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) o[i] = narrow<OT>(acc[i]);
+            store_vec<OT, VEC, ALIGNED>(out + e0[u], o);
+            if (new_r != nullptr) {
+                OT pv[VEC], d[VEC];
+                load_vec<OT, VEC, ALIGNED>(prepared + e0[u], pv);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) d[i] = narrow<OT>(widen(pv[i]) - acc[i]);
+                store_vec<OT, VEC, ALIGNED>(new_r + e0[u], d);
+            }
+        }
+        return;
+    }
+
+    // ---- edge block: element-wise, stores guarded by numel ----------------------
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t e0 = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
+        for (int i = 0; i < VEC; ++i) {
+            const int64_t e = e0 + i;
+            if (e >= a.numel) break;
+            const int64_t g = e / G;
+            float acc = 0.0f;
+#pragma unroll
+            for (int r = 0; r < W; ++r) {
+                const float t = round_through<OT>(static_cast<float>(a.codes[r][e]) * a.scales[r][g]);
+                acc = r == 0 ? t : round_through<OT>(acc + t);
+            }
+            if (mean) acc = round_through<OT>(acc / a.divisor);
+            out[e] = narrow<OT>(acc);
+            if (new_r != nullptr) new_r[e] = narrow<OT>(widen(prepared[e]) - acc);
+        }
+    }
+}
+
+template <typename OT, int G, int W>
+hipError_t launch_reduce_w(bool aligned, const ReduceArgs &a, hipStream_t stream) {
+    using T = decode_tiling<OT>;
+    const int64_t blocks = (a.numel + T::BLOCK_ELEMS - 1) / T::BLOCK_ELEMS;
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    if (aligned)
+        hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, true>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a);
+    else
+        hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, false>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+template <typename OT, int G>
+hipError_t launch_reduce_g(int world, bool aligned, const ReduceArgs &a, hipStream_t s) {
+    switch (world) {
+        case 1: return launch_reduce_w<OT, G, 1>(aligned, a, s);
+        case 2: return launch_reduce_w<OT, G, 2>(aligned, a, s);
+        case 3: return launch_reduce_w<OT, G, 3>(aligned, a, s);
+        case 4: return launch_reduce_w<OT, G, 4>(aligned, a, s);
+        case 5: return launch_reduce_w<OT, G, 5>(aligned, a, s);
+        case 6: return launch_reduce_w<OT, G, 6>(aligned, a, s);
+        case 7: return launch_reduce_w<OT, G, 7>(aligned, a, s);
+        case 8: return launch_reduce_w<OT, G, 8>(aligned, a, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
+template <typename OT>
+hipError_t launch_reduce_t(int g, int world, bool aligned, const ReduceArgs &a, hipStream_t s) {
+    switch (g) {
+        case 64: return launch_reduce_g<OT, 64>(world, aligned, a, s);
+        case 32: return launch_reduce_g<OT, 32>(world, aligned, a, s);
+        case 16: return launch_reduce_g<OT, 16>(world, aligned, a, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// decode of one payload, or of `world` shard payloads into consecutive shards
+// ---------------------------------------------------------------------------
+template <int OP> __device__ __forceinline__ float combine(float old, float v) {
+    if constexpr (OP == 1) return old + v;
+    else if constexpr (OP == 2) return old > v ? old : v;
+    else if constexpr (OP == 3) return old < v ? old : v;
+    else return v;
+}
+
+template <typename OT, int G, int OP, bool ALIGNED>
+__global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
+    using T = decode_tiling<OT>;
+    constexpr int VEC = T::VEC;
+    constexpr int UNROLL = T::UNROLL;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t chunk = blockIdx.y;
+    const int64_t chunk_start = chunk * a.shard_numel;
+    int64_t valid = a.total_numel - chunk_start;
+    valid = valid < 0 ? 0 : (valid > a.shard_numel ? a.shard_numel : valid);
+    const int8_t *__restrict__ codes = reinterpret_cast<const int8_t *>(a.codes_base + chunk * a.payload_stride);
+    const float *__restrict__ scales = reinterpret_cast<const float *>(a.scales_base + chunk * a.payload_stride);
+    OT *__restrict__ out = static_cast<OT *>(a.out) + chunk_start;
+    const int64_t block_first = static_cast<int64_t>(blockIdx.x) * T::BLOCK_ELEMS;
+    if (block_first >= valid) return;
+
+    if (block_first + T::BLOCK_ELEMS <= valid) {
+        uint32_t words[UNROLL][VEC / 4];
+        float scale[UNROLL];
+        int64_t e0[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            e0[u] = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
+            load_codes<VEC, ALIGNED>(codes + e0[u], words[u]);
+            scale[u] = scales[e0[u] / G];
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            OT o[VEC];
+            if constexpr (OP != 0) load_vec<OT, VEC, ALIGNED>(out + e0[u], o);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                float v = round_through<OT>(code_to_float(words[u][i / 4], i % 4) * scale[u]);
+                if constexpr (OP != 0) v = round_through<OT>(combine<OP>(widen(o[i]), v));
+                o[i] = narrow<OT>(v);
+            }
+            store_vec<OT, VEC, ALIGNED>(out + e0[u], o);
+        }
+        return;
+    }
+
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t e0 = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
+        for (int i = 0; i < VEC; ++i) {
+            const int64_t e = e0 + i;
+            if (e >= valid) break;
+            float v = round_through<OT>(static_cast<float>(codes[e]) * scales[e / G]);
+            if constexpr (OP != 0) v = round_through<OT>(combine<OP>(widen(out[e]), v));
+            out[e] = narrow<OT>(v);
+        }
+    }
+}
+
+template <typename OT, int G, int OP>
+hipError_t launch_decode_op(bool aligned, const DecodeArgs &a, int world, hipStream_t stream) {
+    using T = decode_tiling<OT>;
+    const int64_t blocks = (a.shard_numel + T::BLOCK_ELEMS - 1) / T::BLOCK_ELEMS;
+    if (blocks == 0 || world == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFFLL || world > 65535) return hipErrorInvalidValue;
+    dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(world));
+    if (aligned)
+        hipLaunchKernelGGL((decode_kernel<OT, G, OP, true>), grid, dim3(kBlock), 0, stream, a);
+    else
+        hipLaunchKernelGGL((decode_kernel<OT, G, OP, false>), grid, dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+template <typename OT, int G>
+hipError_t launch_decode_g(int op, bool aligned, const DecodeArgs &a, int world, hipStream_t s) {
+    switch (op) {
+        case 0: return launch_decode_op<OT, G, 0>(aligned, a, world, s);
+        case 1: return launch_decode_op<OT, G, 1>(aligned, a, world, s);
+        case 2: return launch_decode_op<OT, G, 2>(aligned, a, world, s);
+        case 3: return launch_decode_op<OT, G, 3>(aligned, a, world, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
+template <typename OT>
+hipError_t launch_decode_t(int g, int op, bool aligned, const DecodeArgs &a, int world, hipStream_t s) {
+    switch (g) {
+        case 64: return launch_decode_g<OT, 64>(op, aligned, a, world, s);
+        case 32: return launch_decode_g<OT, 32>(op, aligned, a, world, s);
+        case 16: return launch_decode_g<OT, 16>(op, aligned, a, world, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// residual = prepared - restored
+// ---------------------------------------------------------------------------
+template <typename PT, typename TT, typename RT, bool ALIGNED>
+__global__ __launch_bounds__(kBlock) void ef_update_kernel(const EfArgs a) {
+    constexpr int VEC = 4;
+    constexpr int UNROLL = 4;
+    constexpr int BLOCK_ELEMS = kBlock * VEC * UNROLL;
+    const PT *__restrict__ prepared = static_cast<const PT *>(a.prepared);
+    const TT *__restrict__ restored = static_cast<const TT *>(a.restored);
+    RT *__restrict__ residual = static_cast<RT *>(a.residual);
+    const int64_t block_first = static_cast<int64_t>(blockIdx.x) * BLOCK_ELEMS;
+    if (block_first + BLOCK_ELEMS <= a.numel) {
+        PT pv[UNROLL][VEC];
+        TT tv[UNROLL][VEC];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t e0 = block_first + (static_cast<int64_t>(u) * kBlock + threadIdx.x) * VEC;
+            load_vec<PT, VEC, ALIGNED>(prepared + e0, pv[u]);
+            load_vec<TT, VEC, ALIGNED>(restored + e0, tv[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t e0 = block_first + (static_cast<int64_t>(u) * kBlock + threadIdx.x) * VEC;
+            RT d[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) d[i] = narrow<RT>(widen(pv[u][i]) - widen(tv[u][i]));
+            store_vec<RT, VEC, ALIGNED>(residual + e0, d);
+        }
+        return;
+    }
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t e0 = block_first + (static_cast<int64_t>(u) * kBlock + threadIdx.x) * VEC;
+        for (int i = 0; i < VEC; ++i) {
+            const int64_t e = e0 + i;
+            if (e >= a.numel) break;
+            residual[e] = narrow<RT>(widen(prepared[e]) - widen(restored[e]));
+        }
+    }
+}
+
+template <typename PT, typename TT, typename RT>
+hipError_t launch_ef(bool aligned, const EfArgs &a, hipStream_t stream) {
+    constexpr int BLOCK_ELEMS = kBlock * 4 * 4;
+    const int64_t blocks = (a.numel + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    if (aligned)
+        hipLaunchKernelGGL((ef_update_kernel<PT, TT, RT, true>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a);
+    else
+        hipLaunchKernelGGL((ef_update_kernel<PT, TT, RT, false>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+// Supported combinations: restored has prepared's type or either is float; the
+// residual has their torch promotion.  Anything else is reported unsupported.
+template <typename PT, typename TT, typename RT>
+hipError_t launch_ef_checked(int r_dtype, int want, bool aligned, const EfArgs &a, hipStream_t s) {
+    if (r_dtype != want) return hipErrorNotSupported;
+    return launch_ef<PT, TT, RT>(aligned, a, s);
+}
+
+hipError_t launch_ef_any(int p, int t, int r, bool aligned, const EfArgs &a, hipStream_t s) {
+    if (p == kF32 && t == kF32) return launch_ef_checked<float, float, float>(r, kF32, aligned, a, s);
+    if (p == kF32 && t == kF16) return launch_ef_checked<float, f16, float>(r, kF32, aligned, a, s);
+    if (p == kF32 && t == kBF16) return launch_ef_checked<float, bf16, float>(r, kF32, aligned, a, s);
+    if (p == kF16 && t == kF32) return launch_ef_checked<f16, float, float>(r, kF32, aligned, a, s);
+    if (p == kBF16 && t == kF32) return launch_ef_checked<bf16, float, float>(r, kF32, aligned, a, s);
+    if (p == kF16 && t == kF16) return launch_ef_checked<f16, f16, f16>(r, kF16, aligned, a, s);
+    if (p == kBF16 && t == kBF16) return launch_ef_checked<bf16, bf16, bf16>(r, kBF16, aligned, a, s);
+    return hipErrorNotSupported;
+}
+
+}  // namespace
+
+hipError_t launch_dequant_reduce(int out_dtype, int group_size, int world, bool aligned,
+                                 const ReduceArgs &args, hipStream_t stream) {
+    switch (out_dtype) {
+        case kF32: return launch_reduce_t<float>(group_size, world, aligned, args, stream);
+        case kF16: return launch_reduce_t<f16>(group_size, world, aligned, args, stream);
+        case kBF16: return launch_reduce_t<bf16>(group_size, world, aligned, args, stream);
+        default: return hipErrorNotSupported;
+    }
+}
+
+hipError_t launch_decode(int out_dtype, int group_size, int reduce_op, bool aligned,
+                         const DecodeArgs &args, int world, hipStream_t stream) {
+    switch (out_dtype) {
+        case kF32: return launch_decode_t<float>(group_size, reduce_op, aligned, args, world, stream);
+        case kF16: return launch_decode_t<f16>(group_size, reduce_op, aligned, args, world, stream);
+        case kBF16: return launch_decode_t<bf16>(group_size, reduce_op, aligned, args, world, stream);
+        default: return hipErrorNotSupported;
+    }
+}
+
+hipError_t launch_ef_update(int p_dtype, int t_dtype, int r_dtype, bool aligned, const EfArgs &args,
+                            hipStream_t stream) {
+    return launch_ef_any(p_dtype, t_dtype, r_dtype, aligned, args, stream);
+}
+
+}  // namespace lbc

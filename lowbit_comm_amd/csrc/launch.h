@@ -1,0 +1,64 @@
+// Host-side launch interface between the C ABI (lbc_api.hip) and the kernel
+// translation units.  The ABI validates; these only pick an instantiation.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lbc {
+
+constexpr int kMaxPayloads = 8;
+
+// dtype tags shared with include/lbc.h
+constexpr int kF32 = 0, kF16 = 1, kBF16 = 2, kNone = -1;
+
+struct QuantArgs {
+    const void *x;
+    const void *residual;    // may be null
+    uint8_t *codes_base;     // chunk d: codes at codes_base + d * payload_stride
+    uint8_t *scales_base;    // chunk d: scales at scales_base + d * payload_stride
+    void *new_residual;      // may be null
+    void *restored;          // may be null
+    int64_t numel;           // valid elements in the whole tensor
+    int64_t shard_numel;     // elements per chunk (== numel for a single payload)
+    int64_t payload_stride;  // bytes
+};
+
+struct ReduceArgs {
+    const int8_t *codes[kMaxPayloads];
+    const float *scales[kMaxPayloads];
+    void *out;
+    const void *prepared;  // may be null
+    void *new_residual;    // may be null
+    int64_t numel;
+    float divisor;
+};
+
+struct DecodeArgs {
+    const uint8_t *codes_base;   // chunk d: codes at codes_base + d * payload_stride
+    const uint8_t *scales_base;  // chunk d: scales at scales_base + d * payload_stride
+    void *out;                   // chunk d lands at out + d * shard_numel elements
+    int64_t shard_numel;
+    int64_t total_numel;
+    int64_t payload_stride;
+};
+
+struct EfArgs {
+    const void *prepared;
+    const void *restored;
+    void *residual;
+    int64_t numel;
+};
+
+// Each returns hipSuccess/last launch error, or hipErrorNotSupported when no
+// instantiation exists for the type combination.
+hipError_t launch_quant_pack(int x_dtype, int r_dtype, int d_dtype, int group_size, bool aligned,
+                             const QuantArgs &args, int world, hipStream_t stream);
+hipError_t launch_dequant_reduce(int out_dtype, int group_size, int world, bool aligned,
+                                 const ReduceArgs &args, hipStream_t stream);
+hipError_t launch_decode(int out_dtype, int group_size, int reduce_op, bool aligned,
+                         const DecodeArgs &args, int world, hipStream_t stream);
+hipError_t launch_ef_update(int p_dtype, int t_dtype, int r_dtype, bool aligned, const EfArgs &args,
+                            hipStream_t stream);
+
+}  // namespace lbc

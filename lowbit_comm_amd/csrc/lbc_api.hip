@@ -1,0 +1,243 @@
+// C ABI of the codec library (declared in include/lbc.h): argument validation,
+// alignment probing and dispatch.  No allocation, no synchronisation, no state
+// besides a per-thread error string.
+#include "../../include/lbc.h"
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "launch.h"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool valid_dtype(int d) { return d == LBC_F32 || d == LBC_F16 || d == LBC_BF16; }
+int dtype_size(int d) { return d == LBC_F32 ? 4 : 2; }
+bool valid_group(int g) { return g == 16 || g == 32 || g == 64; }
+
+bool aligned_to(const void *p, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; }
+
+// torch promotion of two of {f32, f16, bf16}
+int promote(int a, int b) { return a == b ? a : LBC_F32; }
+
+int finish(hipError_t err, const char *what) {
+    if (err == hipSuccess) return LBC_OK;
+    if (err == hipErrorNotSupported) return LBC_UNSUPPORTED;
+    return fail(LBC_ELAUNCH, "%s: %s", what, hipGetErrorString(err));
+}
+
+}  // namespace
+
+extern "C" {
+
+int lbc_abi_version(void) { return LBC_ABI_VERSION; }
+
+const char *lbc_last_error(void) { return g_error; }
+
+int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel,
+                   int group_size, int8_t *codes, float *scales, void *new_residual, int new_residual_dtype,
+                   void *restored, int restored_dtype, void *stream) {
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (!valid_dtype(x_dtype)) return fail(LBC_EINVAL, "unsupported input dtype %d", x_dtype);
+    if (residual != nullptr && !valid_dtype(residual_dtype))
+        return fail(LBC_EINVAL, "unsupported residual dtype %d", residual_dtype);
+    if (!valid_group(group_size)) return LBC_UNSUPPORTED;
+    if (numel == 0) return LBC_OK;
+    if (x == nullptr) return fail(LBC_EINVAL, "input must not be null");
+    if (codes == nullptr || scales == nullptr) return fail(LBC_EINVAL, "codes and scales must not be null");
+    if (!aligned_to(scales, 4)) return fail(LBC_EINVAL, "scales must be 4-byte aligned");
+    if (!aligned_to(x, dtype_size(x_dtype))) return fail(LBC_EINVAL, "input is not aligned to its element size");
+
+    const int r_dtype = residual ? residual_dtype : LBC_NONE;
+    const int p_dtype = residual ? promote(x_dtype, r_dtype) : x_dtype;
+    const bool wants_outputs = new_residual != nullptr || restored != nullptr;
+    int d_dtype = LBC_F32;
+    if (wants_outputs) {
+        if (!valid_dtype(restored_dtype)) return fail(LBC_EINVAL, "unsupported restored dtype %d", restored_dtype);
+        d_dtype = restored_dtype;
+        if (new_residual != nullptr) {
+            if (!valid_dtype(new_residual_dtype))
+                return fail(LBC_EINVAL, "unsupported new-residual dtype %d", new_residual_dtype);
+            if (new_residual_dtype != promote(p_dtype, d_dtype))
+                return fail(LBC_EINVAL, "new residual must have the promoted dtype of (input+residual) and restored");
+        }
+    }
+    if (r_dtype != LBC_NONE && r_dtype != LBC_F32 && r_dtype != x_dtype) return LBC_UNSUPPORTED;
+    if (d_dtype != LBC_F32 && d_dtype != x_dtype) return LBC_UNSUPPORTED;
+
+    const int vec = 16 / dtype_size(x_dtype);
+    bool aligned = aligned_to(x, 16) && aligned_to(codes, vec);
+    if (residual) aligned = aligned && aligned_to(residual, 16);
+    if (new_residual) aligned = aligned && aligned_to(new_residual, 16);
+    if (restored) aligned = aligned && aligned_to(restored, 16);
+
+    lbc::QuantArgs a{};
+    a.x = x;
+    a.residual = residual;
+    a.codes_base = reinterpret_cast<uint8_t *>(codes);
+    a.scales_base = reinterpret_cast<uint8_t *>(scales);
+    a.new_residual = new_residual;
+    a.restored = restored;
+    a.numel = numel;
+    a.shard_numel = numel;
+    a.payload_stride = 0;
+    return finish(lbc::launch_quant_pack(x_dtype, r_dtype, d_dtype, group_size, aligned, a, 1,
+                                         static_cast<hipStream_t>(stream)),
+                  "lbc_quant_pack");
+}
+
+int lbc_quant_pack_chunks(const void *x, int x_dtype, int64_t numel, int world, int group_size,
+                          uint8_t *payloads, int64_t payload_stride, void *stream) {
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
+    if (!valid_dtype(x_dtype)) return fail(LBC_EINVAL, "unsupported input dtype %d", x_dtype);
+    if (!valid_group(group_size)) return LBC_UNSUPPORTED;
+    if (world > 65535) return LBC_UNSUPPORTED;
+    const int64_t shard = (numel + world - 1) / world;
+    if (shard == 0) return LBC_OK;
+    const int64_t groups = (shard + group_size - 1) / group_size;
+    const int64_t payload_bytes = groups * (group_size + 4);
+    if (x == nullptr || payloads == nullptr) return fail(LBC_EINVAL, "input and payloads must not be null");
+    if (payload_stride < payload_bytes || (payload_stride & 3) != 0)
+        return fail(LBC_EINVAL, "payload_stride must be a multiple of 4 and >= %lld", (long long)payload_bytes);
+    if (!aligned_to(payloads, 4)) return fail(LBC_EINVAL, "payloads must be 4-byte aligned");
+    if (!aligned_to(x, dtype_size(x_dtype))) return fail(LBC_EINVAL, "input is not aligned to its element size");
+
+    const int vec = 16 / dtype_size(x_dtype);
+    const bool aligned = aligned_to(x, 16) && (shard * dtype_size(x_dtype)) % 16 == 0 && aligned_to(payloads, vec) &&
+                         payload_stride % vec == 0;
+    lbc::QuantArgs a{};
+    a.x = x;
+    a.codes_base = payloads;
+    a.scales_base = payloads + groups * group_size;
+    a.numel = numel;
+    a.shard_numel = shard;
+    a.payload_stride = payload_stride;
+    return finish(lbc::launch_quant_pack(x_dtype, LBC_NONE, LBC_F32, group_size, aligned, a, world,
+                                         static_cast<hipStream_t>(stream)),
+                  "lbc_quant_pack_chunks");
+}
+
+int lbc_dequant(const int8_t *codes, const float *scales, int64_t numel, int group_size, void *out,
+                int out_dtype, int reduce_op, void *stream) {
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (!valid_dtype(out_dtype)) return fail(LBC_EINVAL, "unsupported output dtype %d", out_dtype);
+    if (reduce_op < LBC_REDUCE_NONE || reduce_op > LBC_REDUCE_MIN)
+        return fail(LBC_EINVAL, "unsupported reduce op %d", reduce_op);
+    if (!valid_group(group_size)) return LBC_UNSUPPORTED;
+    if (numel == 0) return LBC_OK;
+    if (codes == nullptr || scales == nullptr || out == nullptr)
+        return fail(LBC_EINVAL, "codes, scales and out must not be null");
+    if (!aligned_to(scales, 4)) return fail(LBC_EINVAL, "scales must be 4-byte aligned");
+    if (!aligned_to(out, dtype_size(out_dtype))) return fail(LBC_EINVAL, "out is not aligned to its element size");
+    const int vec = out_dtype == LBC_F32 ? 4 : 8;
+    const bool aligned = aligned_to(codes, vec) && aligned_to(out, 16);
+    lbc::DecodeArgs a{};
+    a.codes_base = reinterpret_cast<const uint8_t *>(codes);
+    a.scales_base = reinterpret_cast<const uint8_t *>(scales);
+    a.out = out;
+    a.shard_numel = numel;
+    a.total_numel = numel;
+    a.payload_stride = 0;
+    return finish(lbc::launch_decode(out_dtype, group_size, reduce_op, aligned, a, 1, static_cast<hipStream_t>(stream)),
+                  "lbc_dequant");
+}
+
+int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world, int64_t shard_numel,
+                       int64_t total_numel, int group_size, void *out, int out_dtype, void *stream) {
+    if (shard_numel < 0 || total_numel < 0) return fail(LBC_EINVAL, "element counts must be >= 0");
+    if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
+    if (total_numel > shard_numel * world) return fail(LBC_EINVAL, "total_numel exceeds world * shard_numel");
+    if (!valid_dtype(out_dtype)) return fail(LBC_EINVAL, "unsupported output dtype %d", out_dtype);
+    if (!valid_group(group_size)) return LBC_UNSUPPORTED;
+    if (world > 65535) return LBC_UNSUPPORTED;
+    if (shard_numel == 0 || total_numel == 0) return LBC_OK;
+    const int64_t groups = (shard_numel + group_size - 1) / group_size;
+    const int64_t payload_bytes = groups * (group_size + 4);
+    if (payloads == nullptr || out == nullptr) return fail(LBC_EINVAL, "payloads and out must not be null");
+    if (payload_stride < payload_bytes || (payload_stride & 3) != 0)
+        return fail(LBC_EINVAL, "payload_stride must be a multiple of 4 and >= %lld", (long long)payload_bytes);
+    if (!aligned_to(payloads, 4)) return fail(LBC_EINVAL, "payloads must be 4-byte aligned");
+    if (!aligned_to(out, dtype_size(out_dtype))) return fail(LBC_EINVAL, "out is not aligned to its element size");
+    const int vec = out_dtype == LBC_F32 ? 4 : 8;
+    const bool aligned = aligned_to(payloads, vec) && payload_stride % vec == 0 && aligned_to(out, 16) &&
+                         (shard_numel * dtype_size(out_dtype)) % 16 == 0;
+    lbc::DecodeArgs a{};
+    a.codes_base = payloads;
+    a.scales_base = payloads + groups * group_size;
+    a.out = out;
+    a.shard_numel = shard_numel;
+    a.total_numel = total_numel;
+    a.payload_stride = payload_stride;
+    return finish(lbc::launch_decode(out_dtype, group_size, LBC_REDUCE_NONE, aligned, a, world,
+                                     static_cast<hipStream_t>(stream)),
+                  "lbc_dequant_chunks");
+}
+
+int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, int world, int64_t numel,
+                       int group_size, float divisor, void *out, int out_dtype, const void *prepared,
+                       void *new_residual, void *stream) {
+    if (world <= 0) return fail(LBC_EINVAL, "inputs must not be empty");
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (!(divisor > 0.0f)) return fail(LBC_EINVAL, "divisor must be > 0");
+    if (!valid_dtype(out_dtype)) return fail(LBC_EINVAL, "unsupported output dtype %d", out_dtype);
+    if ((prepared == nullptr) != (new_residual == nullptr))
+        return fail(LBC_EINVAL, "prepared and new_residual must be given together");
+    if (world > LBC_MAX_PAYLOADS || !valid_group(group_size)) return LBC_UNSUPPORTED;
+    if (numel == 0) return LBC_OK;
+    if (codes == nullptr || scales == nullptr || out == nullptr)
+        return fail(LBC_EINVAL, "codes, scales and out must not be null");
+    const int vec = out_dtype == LBC_F32 ? 4 : 8;
+    bool aligned = aligned_to(out, 16);
+    if (!aligned_to(out, dtype_size(out_dtype))) return fail(LBC_EINVAL, "out is not aligned to its element size");
+    lbc::ReduceArgs a{};
+    for (int r = 0; r < world; ++r) {
+        if (codes[r] == nullptr || scales[r] == nullptr) return fail(LBC_EINVAL, "payload %d has a null pointer", r);
+        if (!aligned_to(scales[r], 4)) return fail(LBC_EINVAL, "scales of payload %d must be 4-byte aligned", r);
+        aligned = aligned && aligned_to(codes[r], vec);
+        a.codes[r] = codes[r];
+        a.scales[r] = scales[r];
+    }
+    if (prepared != nullptr) {
+        if (!aligned_to(prepared, dtype_size(out_dtype)) || !aligned_to(new_residual, dtype_size(out_dtype)))
+            return fail(LBC_EINVAL, "prepared/new_residual are not aligned to their element size");
+        aligned = aligned && aligned_to(prepared, 16) && aligned_to(new_residual, 16);
+    }
+    a.out = out;
+    a.prepared = prepared;
+    a.new_residual = new_residual;
+    a.numel = numel;
+    a.divisor = divisor;
+    return finish(lbc::launch_dequant_reduce(out_dtype, group_size, world, aligned, a, static_cast<hipStream_t>(stream)),
+                  "lbc_dequant_reduce");
+}
+
+int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored, int restored_dtype,
+                  void *residual, int residual_dtype, int64_t numel, void *stream) {
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (!valid_dtype(prepared_dtype) || !valid_dtype(restored_dtype) || !valid_dtype(residual_dtype))
+        return fail(LBC_EINVAL, "unsupported dtype");
+    if (numel == 0) return LBC_OK;
+    if (prepared == nullptr || restored == nullptr || residual == nullptr)
+        return fail(LBC_EINVAL, "prepared, restored and residual must not be null");
+    if (!aligned_to(prepared, dtype_size(prepared_dtype)) || !aligned_to(restored, dtype_size(restored_dtype)) ||
+        !aligned_to(residual, dtype_size(residual_dtype)))
+        return fail(LBC_EINVAL, "a tensor is not aligned to its element size");
+    const bool aligned = aligned_to(prepared, 16) && aligned_to(restored, 16) && aligned_to(residual, 16);
+    lbc::EfArgs a{prepared, restored, residual, numel};
+    return finish(lbc::launch_ef_update(prepared_dtype, restored_dtype, residual_dtype, aligned, a,
+                                        static_cast<hipStream_t>(stream)),
+                  "lbc_ef_update");
+}
+
+}  // extern "C"

@@ -1,0 +1,70 @@
+"""ctypes binding of ``liblbc_hip.so`` (the C ABI declared in ``include/lbc.h``).
+
+The library is built in-tree by ``lowbit_comm_amd/csrc/Makefile``.  Loading never falls back to
+anything else: if the shared object is missing or a symbol is absent, :func:`load_library` raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+
+from lowbit_comm_amd.exceptions import CCDLUnavailableError
+
+LIBRARY_PATH = Path(__file__).resolve().parent.parent / "liblbc_hip.so"
+ABI_VERSION = 1
+
+LBC_OK = 0
+LBC_UNSUPPORTED = 1
+
+_c_ptr = ctypes.c_void_p
+_c_i64 = ctypes.c_int64
+_c_int = ctypes.c_int
+
+# symbol -> (restype, argtypes); one entry per declaration in include/lbc.h
+SIGNATURES = {
+    "lbc_abi_version": (_c_int, []),
+    "lbc_last_error": (ctypes.c_char_p, []),
+    "lbc_quant_pack": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_ptr, _c_ptr,
+                                _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr]),
+    "lbc_quant_pack_chunks": (_c_int, [_c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_ptr, _c_i64, _c_ptr]),
+    "lbc_dequant": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
+    "lbc_dequant_chunks": (_c_int, [_c_ptr, _c_i64, _c_int, _c_i64, _c_i64, _c_int, _c_ptr, _c_int, _c_ptr]),
+    "lbc_dequant_reduce": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_ptr, _c_int,
+                                    _c_ptr, _c_ptr, _c_ptr]),
+    "lbc_ef_update": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr]),
+}
+
+_library: ctypes.CDLL | None = None
+
+
+def load_library(path: str | Path | None = None) -> ctypes.CDLL:
+    """Load the shared object once and type every entry point."""
+    global _library
+    if _library is not None and path is None:
+        return _library
+    target = Path(path) if path is not None else LIBRARY_PATH
+    if not target.exists():
+        raise CCDLUnavailableError(
+            f"{target.name} is not built (run `make -C lowbit_comm_amd/csrc` or __graft_entry__.build())")
+    try:
+        lib = ctypes.CDLL(str(target))
+    except OSError as exc:
+        raise CCDLUnavailableError(f"cannot load {target}: {exc}") from exc
+    for name, (restype, argtypes) in SIGNATURES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as exc:
+            raise CCDLUnavailableError(f"{target.name} missing required symbol: {name}") from exc
+        fn.restype = restype
+        fn.argtypes = argtypes
+    version = lib.lbc_abi_version()
+    if version != ABI_VERSION:
+        raise CCDLUnavailableError(f"{target.name} has ABI version {version}, expected {ABI_VERSION}")
+    if path is None:
+        _library = lib
+    return lib
+
+
+def last_error(lib: ctypes.CDLL) -> str:
+    raw = lib.lbc_last_error()
+    return raw.decode("utf-8", "replace") if raw else ""

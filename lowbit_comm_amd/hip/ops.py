@@ -1,0 +1,274 @@
+"""Tensor-level entry points over the C ABI.
+
+Every function takes torch tensors that already live on the GPU, checks the contract the C ABI
+cannot see (device, contiguity, element counts), and enqueues on torch's current stream of the
+tensors' device.  Functions named ``*_into`` write only into caller-owned tensors and return
+``True`` (enqueued) or ``False`` (valid request this build has no kernel for - take a fallback),
+mirroring the reference's native ``inplace_*`` functions (ccdl_comm/csrc/pybind.cpp:39-131);
+contract violations raise ``RuntimeError`` like the reference's ``TORCH_CHECK``.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Sequence
+
+import torch
+
+from lowbit_comm_amd.hip.library import LBC_OK, LBC_UNSUPPORTED, last_error, load_library
+
+DTYPE_CODES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+DTYPE_NAMES = {torch.float32: "fp32", torch.float16: "fp16", torch.bfloat16: "bf16"}
+TORCH_DTYPES = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
+REDUCE_OPS = {"none": 0, "sum": 1, "max": 2, "min": 3}
+MAX_PAYLOADS = 8
+_NONE = -1
+
+
+def num_groups(numel: int, group_size: int) -> int:
+    return -(-numel // group_size) if numel else 0
+
+
+def payload_nbytes(numel: int, group_size: int = 64) -> int:
+    """Bytes of one packed payload ``[int8 codes || fp32 scales]``."""
+    return num_groups(numel, group_size) * (group_size + 4)
+
+
+def split_payload(payload: torch.Tensor, numel: int, group_size: int = 64):
+    """Zero-copy ``(codes int8[G*g], scales float32[G])`` views of a packed uint8 payload."""
+    groups = num_groups(numel, group_size)
+    code_bytes = groups * group_size
+    if payload.dtype != torch.uint8 or payload.dim() != 1 or payload.numel() != code_bytes + 4 * groups:
+        raise RuntimeError(
+            f"payload must be a flat uint8 tensor of {code_bytes + 4 * groups} bytes; got "
+            f"{payload.dtype} with {payload.numel()} elements")
+    return payload[:code_bytes].view(torch.int8), payload[code_bytes:].view(torch.float32)
+
+
+def promote(a: torch.dtype, b: torch.dtype) -> torch.dtype:
+    return a if a == b else torch.float32
+
+
+# --------------------------------------------------------------------------- #
+def _require(cond: bool, message: str) -> None:
+    if not cond:
+        raise RuntimeError(message)
+
+
+def _device_tensor(t: torch.Tensor, name: str, device: torch.device | None = None) -> None:
+    _require(isinstance(t, torch.Tensor), f"{name} must be a tensor")
+    _require(t.is_cuda, f"{name} must be a GPU tensor")
+    _require(t.is_contiguous(), f"{name} must be contiguous")
+    if device is not None:
+        _require(t.device == device, f"{name} must be on {device}")
+
+
+def _float_tensor(t: torch.Tensor, name: str, device: torch.device | None = None) -> int:
+    _device_tensor(t, name, device)
+    _require(t.dtype in DTYPE_CODES, f"{name} must be fp16, bf16 or fp32; got {t.dtype}")
+    return DTYPE_CODES[t.dtype]
+
+
+def _ptr(t: torch.Tensor | None):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+class _Launch:
+    """Device guard + current stream of ``device`` for one ABI call."""
+
+    def __init__(self, device: torch.device) -> None:
+        self._guard = None if device.index in (None, torch.cuda.current_device()) else torch.cuda.device(device)
+        self.device = device
+
+    def __enter__(self):
+        if self._guard is not None:
+            self._guard.__enter__()
+        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def __exit__(self, *exc):
+        if self._guard is not None:
+            self._guard.__exit__(*exc)
+        return False
+
+
+def _finish(rc: int, lib) -> bool:
+    if rc == LBC_OK:
+        return True
+    if rc == LBC_UNSUPPORTED:
+        return False
+    raise RuntimeError(last_error(lib) or f"lbc call failed with code {rc}")
+
+
+# --------------------------------------------------------------------------- #
+# quantize + pack
+# --------------------------------------------------------------------------- #
+def quant_pack_into(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, *, group_size: int = 64,
+                    residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
+                    restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None) -> bool:
+    """``codes, scales <- quant(x + residual)``; optionally ``restored`` and ``new_residual = p - restored``."""
+    lib = load_library()
+    x_code = _float_tensor(x, "input")
+    device = x.device
+    n = x.numel()
+    groups = num_groups(n, group_size)
+    _device_tensor(codes, "codes", device)
+    _device_tensor(scales, "scales", device)
+    _require(codes.dtype in (torch.int8, torch.uint8), "codes must have int8 or uint8 dtype")
+    _require(scales.dtype == torch.float32, "scales must have float32 dtype")
+    _require(codes.numel() == groups * group_size, "codes has an invalid quantized payload size")
+    _require(scales.numel() == groups, "scales has an invalid group count")
+    r_code = _NONE
+    if residual is not None:
+        r_code = _float_tensor(residual, "residual", device)
+        _require(residual.numel() == n, "input and residual must have the same number of elements")
+    p_dtype = x.dtype if residual is None else promote(x.dtype, residual.dtype)
+    d_dtype = restored.dtype if restored is not None else (restored_dtype or torch.float32)
+    d_code = DTYPE_CODES.get(d_dtype)
+    _require(d_code is not None, f"restored dtype must be fp16, bf16 or fp32; got {d_dtype}")
+    n_code = _NONE
+    if restored is not None:
+        _float_tensor(restored, "restored", device)
+        _require(restored.numel() >= n, "restored must have at least input.numel() elements")
+    if new_residual is not None:
+        n_code = _float_tensor(new_residual, "new_residual", device)
+        _require(new_residual.numel() == n, "input and new_residual must have the same number of elements")
+        _require(new_residual.dtype == promote(p_dtype, d_dtype),
+                 f"new_residual must have dtype {promote(p_dtype, d_dtype)}")
+    with _Launch(device) as stream:
+        rc = lib.lbc_quant_pack(_ptr(x), x_code, _ptr(residual), r_code, n, group_size, _ptr(codes), _ptr(scales),
+                                _ptr(new_residual), n_code, _ptr(restored), d_code, stream)
+    return _finish(rc, lib)
+
+
+def quant_pack_payload_into(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64, **kwargs) -> bool:
+    """Same as :func:`quant_pack_into`, writing the packed ``uint8[codes || scales]`` wire layout."""
+    codes, scales = split_payload(payload, x.numel(), group_size)
+    return quant_pack_into(x, codes, scales, group_size=group_size, **kwargs)
+
+
+def quant_pack(x: torch.Tensor, *, group_size: int = 64, residual: torch.Tensor | None = None):
+    """Allocating convenience wrapper: returns ``(codes int8[G*g], scales float32[G])``."""
+    groups = num_groups(x.numel(), group_size)
+    codes = torch.empty(groups * group_size, dtype=torch.int8, device=x.device)
+    scales = torch.empty(groups, dtype=torch.float32, device=x.device)
+    if not quant_pack_into(x.contiguous().reshape(-1), codes, scales, group_size=group_size, residual=residual):
+        raise RuntimeError(f"quant_pack has no kernel for dtype {x.dtype} / group_size {group_size}")
+    return codes, scales
+
+
+def quant_pack_chunks_into(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64) -> bool:
+    """Quantize the ``world`` destination chunks of ``x`` into the rows of ``payloads`` (uint8 [world, stride])."""
+    lib = load_library()
+    x_code = _float_tensor(x, "input")
+    _device_tensor(payloads, "payloads", x.device)
+    _require(payloads.dtype == torch.uint8 and payloads.dim() == 2, "payloads must be a 2-D uint8 tensor")
+    _require(payloads.shape[0] == world, "payloads must have one row per destination rank")
+    shard = -(-x.numel() // world)
+    _require(payloads.shape[1] >= payload_nbytes(shard, group_size), "payload rows are too small")
+    with _Launch(x.device) as stream:
+        rc = lib.lbc_quant_pack_chunks(_ptr(x), x_code, x.numel(), world, group_size, _ptr(payloads),
+                                       payloads.stride(0), stream)
+    return _finish(rc, lib)
+
+
+# --------------------------------------------------------------------------- #
+# decode
+# --------------------------------------------------------------------------- #
+def dequant_into(codes: torch.Tensor, scales: torch.Tensor, out: torch.Tensor, *, numel: int | None = None,
+                 group_size: int = 64, reduce_op: str = "none") -> bool:
+    """``out[:numel] (op)= float(code) * scale``."""
+    lib = load_library()
+    o_code = _float_tensor(out, "output")
+    device = out.device
+    n = out.numel() if numel is None else int(numel)
+    _require(0 <= n <= out.numel(), "numel exceeds the output size")
+    groups = num_groups(n, group_size)
+    _device_tensor(codes, "codes", device)
+    _device_tensor(scales, "scales", device)
+    _require(codes.dtype in (torch.int8, torch.uint8), "codes must have int8 or uint8 dtype")
+    _require(scales.dtype == torch.float32, "scales must have float32 dtype")
+    _require(codes.numel() >= groups * group_size, "codes is smaller than the padded element count")
+    _require(scales.numel() >= groups, "scales is smaller than the group count")
+    _require(reduce_op in REDUCE_OPS, f"unsupported reduce op {reduce_op!r}")
+    with _Launch(device) as stream:
+        rc = lib.lbc_dequant(_ptr(codes), _ptr(scales), n, group_size, _ptr(out), o_code, REDUCE_OPS[reduce_op], stream)
+    return _finish(rc, lib)
+
+
+def dequant(codes: torch.Tensor, scales: torch.Tensor, numel: int, *, group_size: int = 64,
+            dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    out = torch.empty(numel, dtype=dtype, device=codes.device)
+    if not dequant_into(codes, scales, out, group_size=group_size):
+        raise RuntimeError(f"dequant has no kernel for dtype {dtype} / group_size {group_size}")
+    return out
+
+
+def dequant_chunks_into(payloads: torch.Tensor, out: torch.Tensor, shard_numel: int, *, group_size: int = 64) -> bool:
+    """Decode row ``d`` of ``payloads`` into ``out[d*shard : (d+1)*shard]`` (clipped to ``out.numel()``)."""
+    lib = load_library()
+    o_code = _float_tensor(out, "output")
+    _device_tensor(payloads, "payloads", out.device)
+    _require(payloads.dtype == torch.uint8 and payloads.dim() == 2, "payloads must be a 2-D uint8 tensor")
+    world = payloads.shape[0]
+    _require(payloads.shape[1] >= payload_nbytes(shard_numel, group_size), "payload rows are too small")
+    _require(out.numel() <= world * shard_numel, "output is larger than world * shard_numel")
+    with _Launch(out.device) as stream:
+        rc = lib.lbc_dequant_chunks(_ptr(payloads), payloads.stride(0), world, shard_numel, out.numel(), group_size,
+                                    _ptr(out), o_code, stream)
+    return _finish(rc, lib)
+
+
+def dequant_reduce_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out: torch.Tensor, *,
+                        numel: int | None = None, group_size: int = 64, divisor: float = 1.0,
+                        prepared: torch.Tensor | None = None, new_residual: torch.Tensor | None = None) -> bool:
+    """``out[:numel] = (sum_r decode(payload_r)) / divisor`` in list order; optional ``new_residual = prepared - out``.
+
+    ``payloads`` is a sequence of ``(codes, scales)`` pairs.  More than 8 payloads returns ``False``.
+    """
+    lib = load_library()
+    _require(len(payloads) > 0, "inputs must not be empty")
+    _require(divisor > 0, "divisor must be > 0")
+    o_code = _float_tensor(out, "output")
+    device = out.device
+    n = out.numel() if numel is None else int(numel)
+    _require(0 <= n <= out.numel(), "numel exceeds the output size")
+    if len(payloads) > MAX_PAYLOADS:
+        return False
+    groups = num_groups(n, group_size)
+    world = len(payloads)
+    code_ptrs = (ctypes.c_void_p * world)()
+    scale_ptrs = (ctypes.c_void_p * world)()
+    for r, (codes, scales) in enumerate(payloads):
+        _device_tensor(codes, f"codes[{r}]", device)
+        _device_tensor(scales, f"scales[{r}]", device)
+        _require(codes.dtype in (torch.int8, torch.uint8), f"codes[{r}] must have int8 or uint8 dtype")
+        _require(scales.dtype == torch.float32, f"scales[{r}] must have float32 dtype")
+        _require(codes.numel() >= groups * group_size, f"codes[{r}] is smaller than the padded element count")
+        _require(scales.numel() >= groups, f"scales[{r}] is smaller than the group count")
+        code_ptrs[r] = codes.data_ptr()
+        scale_ptrs[r] = scales.data_ptr()
+    _require((prepared is None) == (new_residual is None), "prepared and new_residual must be given together")
+    if prepared is not None:
+        _float_tensor(prepared, "prepared", device)
+        _float_tensor(new_residual, "residual", device)
+        _require(prepared.dtype == out.dtype, "prepared and restored must have the same dtype")
+        _require(new_residual.dtype == out.dtype, "prepared and residual must have the same dtype")
+        _require(prepared.numel() == n, "prepared must have numel elements")
+        _require(new_residual.numel() == n, "prepared and residual must have the same number of elements")
+    with _Launch(device) as stream:
+        rc = lib.lbc_dequant_reduce(code_ptrs, scale_ptrs, world, n, group_size, float(divisor), _ptr(out), o_code,
+                                    _ptr(prepared), _ptr(new_residual), stream)
+    return _finish(rc, lib)
+
+
+def ef_update_into(prepared: torch.Tensor, restored: torch.Tensor, residual: torch.Tensor) -> bool:
+    """``residual = prepared - restored`` (fp32 subtraction, rounded to the residual's dtype)."""
+    lib = load_library()
+    p_code = _float_tensor(prepared, "prepared")
+    t_code = _float_tensor(restored, "restored", prepared.device)
+    r_code = _float_tensor(residual, "residual", prepared.device)
+    _require(prepared.numel() == restored.numel(), "prepared and restored must have the same number of elements")
+    _require(prepared.numel() == residual.numel(), "prepared and residual must have the same number of elements")
+    with _Launch(prepared.device) as stream:
+        rc = lib.lbc_ef_update(_ptr(prepared), p_code, _ptr(restored), t_code, _ptr(residual), r_code,
+                               prepared.numel(), stream)
+    return _finish(rc, lib)

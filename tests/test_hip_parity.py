@@ -1,0 +1,445 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle on the same seeded inputs.
+
+Bar: int8 codes, fp32 scales and packed bytes bit-exact; decode / reduce / residual outputs bit-exact
+(the kernels use the oracle's accumulation order and no FMA contraction), which is stricter than the
+stated rtol 1e-6 / atol 1e-7.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import codec_np, codec_torch
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def ops(hip_device):
+    from lowbit_comm_amd.hip import ops as hip_ops
+
+    return hip_ops
+
+
+def gradient_like(n, dtype, seed, device, sigma=1e-3, outliers=True):
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    x = torch.randn(n, generator=gen) * sigma
+    if outliers and n:
+        mask = torch.rand(n, generator=gen) < 1e-3
+        x = torch.where(mask, torch.randn(n, generator=gen) * 1e-1, x)
+    return x.to(dtype).to(device)
+
+
+def bits(t: torch.Tensor) -> torch.Tensor:
+    t = t.detach().cpu().contiguous()
+    return t.view(torch.int32) if t.dtype == torch.float32 else t.view(torch.int16)
+
+
+def assert_same_bits(got: torch.Tensor, want: torch.Tensor, what: str):
+    assert got.dtype == want.dtype, what
+    assert got.shape == want.shape, what
+    same = torch.equal(bits(got), bits(want))
+    if not same:
+        bad = (bits(got) != bits(want)).nonzero().flatten()
+        i = int(bad[0])
+        raise AssertionError(f"{what}: {bad.numel()} mismatches, first at {i}: got {got.flatten()[i].item()!r} "
+                             f"want {want.flatten()[i].item()!r}")
+
+
+# --------------------------------------------------------------------------- #
+# quantize + pack
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("dtype", ["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("n", [1, 63, 64, 65, 4096, 4097, 16384 + 256 * 3 + 17, 1_000_003])
+def test_quant_pack_bit_exact(ops, hip_device, dtype, n):
+    x = gradient_like(n, DTYPES[dtype], 1000 + n, hip_device)
+    codes, scales = ops.quant_pack(x, group_size=64)
+    want_codes, want_scales = codec_torch.quantize(x.cpu(), 64)
+    assert torch.equal(codes.cpu(), want_codes)
+    assert_same_bits(scales, want_scales, "scales")
+
+
+@pytest.mark.parametrize("g", [16, 32, 64])
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_quant_pack_group_sizes(ops, hip_device, g, dtype):
+    n = 70_001
+    x = gradient_like(n, DTYPES[dtype], 77 + g, hip_device)
+    codes, scales = ops.quant_pack(x, group_size=g)
+    want_codes, want_scales = codec_torch.quantize(x.cpu(), g)
+    assert torch.equal(codes.cpu(), want_codes)
+    assert_same_bits(scales, want_scales, "scales")
+
+
+def test_quant_pack_config1_bucket(ops, hip_device):
+    """25 MiB fp32 DDP bucket, N(0,1e-3) with 0.1% N(0,1e-1) outliers: full size against the oracle."""
+    n = 6_553_600
+    x = gradient_like(n, torch.float32, 1234, hip_device)
+    codes, scales = ops.quant_pack(x)
+    want_codes, want_scales = codec_torch.quantize(x.cpu(), 64)
+    assert torch.equal(codes.cpu(), want_codes)
+    assert_same_bits(scales, want_scales, "scales")
+    restored = ops.dequant(codes, scales, n)
+    assert_same_bits(restored, codec_torch.dequantize(want_codes, want_scales, n), "round trip")
+    rel = float((x - restored).norm() / x.norm())
+    assert rel < 0.02
+
+
+def test_quant_pack_special_values(ops, hip_device):
+    x = torch.zeros(64 * 8, dtype=torch.float32)
+    x[0:9] = torch.tensor([127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5, 126.5])   # exact ties, scale 1.0
+    x[64] = 1e-3                                                                    # next group: one value
+    x[128:131] = torch.tensor([6e-7, -3.1e-7, 1.0e-7])                              # eps-clamped scale
+    x[192:256] = 1e-40                                                              # denormals
+    x[192] = 8e-8
+    x[256] = float("nan")
+    x[257] = 1.0
+    x[320] = float("inf")
+    x[321] = 2.0
+    x[384] = 3.4e38                                                                 # near FLT_MAX
+    x[385] = -1.7e38
+    # group 7 stays all zero
+    codes, scales = ops.quant_pack(x.to(hip_device))
+    want_codes, want_scales = codec_np.quantize(x.numpy(), 64)
+    got_scales = scales.cpu().numpy()
+    finite = np.isfinite(want_scales)
+    assert np.array_equal(got_scales[finite].view(np.uint32), want_scales[finite].view(np.uint32))
+    assert np.isnan(got_scales[4]) and np.isinf(got_scales[5])
+    assert np.array_equal(codes.cpu().numpy(), want_codes)
+    assert codes[:9].tolist() == [127, 0, 2, 2, 0, -2, -2, 4, 126]
+    assert int(scales[7].view(torch.int32)) == 0x34000000
+
+
+def test_quant_pack_near_tie_quotients(ops, hip_device):
+    """Values built so that value/scale lands on or next to k + 0.5 - where a reciprocal multiply goes wrong."""
+    rng = np.random.default_rng(5)
+    groups = 4096
+    x = np.zeros((groups, 64), dtype=np.float32)
+    peak = rng.uniform(1e-4, 1e-2, size=groups).astype(np.float32)
+    x[:, 0] = peak
+    scale = np.maximum(peak / np.float32(127.0), np.float32(2.0 ** -23))
+    k = rng.integers(-126, 126, size=(groups, 63)).astype(np.float32)
+    base = (k + np.float32(0.5)) * scale[:, None]
+    ulps = rng.integers(-2, 3, size=(groups, 63)).astype(np.int32)
+    x[:, 1:] = (base.view(np.int32) + ulps).view(np.float32)
+    x = np.where(np.abs(x) <= peak[:, None], x, 0).astype(np.float32).reshape(-1)
+    codes, scales = ops.quant_pack(torch.from_numpy(x).to(hip_device))
+    want_codes, want_scales = codec_np.quantize(x, 64)
+    assert np.array_equal(scales.cpu().numpy().view(np.uint32), want_scales.view(np.uint32))
+    assert np.array_equal(codes.cpu().numpy(), want_codes)
+
+
+def test_quant_pack_unaligned_views_and_untouched_input(ops, hip_device):
+    base = gradient_like(20_000, torch.float32, 9, hip_device)
+    view = base[3:3 + 12_345]          # 12-byte offset: not 16-byte aligned
+    keep = base.clone()
+    storage = torch.empty(ops.payload_nbytes(view.numel()) + 1, dtype=torch.uint8, device=hip_device)
+    groups = ops.num_groups(view.numel(), 64)
+    codes = torch.empty(groups * 64 + 1, dtype=torch.int8, device=hip_device)[1:]   # odd address
+    scales = torch.empty(groups, dtype=torch.float32, device=hip_device)
+    assert ops.quant_pack_into(view, codes, scales)
+    want_codes, want_scales = codec_torch.quantize(view.cpu(), 64)
+    assert torch.equal(codes.cpu(), want_codes)
+    assert_same_bits(scales, want_scales, "scales")
+    assert torch.equal(base, keep)
+    del storage
+
+
+def test_packed_payload_bytes_match_the_wire_format(ops, hip_device):
+    n = 10_000
+    x = gradient_like(n, torch.float32, 21, hip_device)
+    payload = torch.empty(ops.payload_nbytes(n), dtype=torch.uint8, device=hip_device)
+    assert ops.quant_pack_payload_into(x, payload)
+    want = codec_torch.pack(*codec_torch.quantize(x.cpu(), 64))
+    assert payload.numel() == 157 * 68
+    assert torch.equal(payload.cpu(), want)
+    assert np.array_equal(payload.cpu().numpy(), codec_np.pack(*codec_np.quantize(x.cpu().numpy(), 64)))
+
+
+def test_quantize_is_idempotent_and_scale_equivariant_at_full_size(ops, hip_device):
+    """Size-independent properties on a 100 MiB fp32 bucket (too large to run the oracle on comfortably)."""
+    n = 26_214_400
+    x = gradient_like(n, torch.float32, 31, hip_device, outliers=False)
+    codes, scales = ops.quant_pack(x)
+    codes8, scales8 = ops.quant_pack(x * 8.0)
+    assert torch.equal(codes, codes8)
+    assert torch.equal(scales * 8.0, scales8)
+    decoded = ops.dequant(codes, scales, n)
+    codes2, _ = ops.quant_pack(decoded)
+    assert torch.equal(codes, codes2)
+    peak = codes.view(-1, 64).abs().amax(dim=1)
+    assert int(peak.min()) == 127 and int(peak.max()) == 127
+    err = (x - decoded).abs().view(-1, 64)
+    assert bool((err <= scales[:, None] * 0.50005).all())
+
+
+# --------------------------------------------------------------------------- #
+# decode and fused dequant-reduce
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("out_dtype", ["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("n", [1, 64, 100, 16_384, 200_003])
+def test_dequant_bit_exact(ops, hip_device, out_dtype, n):
+    x = gradient_like(n, torch.float32, 300 + n, hip_device)
+    codes, scales = ops.quant_pack(x)
+    got = ops.dequant(codes, scales, n, dtype=DTYPES[out_dtype])
+    want = codec_torch.dequantize(codes.cpu(), scales.cpu(), n, 64, out_dtype)
+    assert_same_bits(got, want, "decoded")
+
+
+def test_fp16_decode_rounds_twice_like_the_reference(ops, hip_device):
+    """code*scale is rounded to fp32 and then to fp16 (two roundings).  A fused multiply-convert that rounds
+    once differs on rare (code, scale) pairs; this payload is made only of such pairs."""
+    rng = np.random.default_rng(77)
+    picked_codes, picked_scales = [], []
+    while len(picked_codes) < 4096:
+        c = rng.integers(-127, 128, size=1 << 20).astype(np.int8)
+        s = (rng.uniform(1e-6, 1e-3, size=1 << 20)).astype(np.float32)
+        exact = c.astype(np.float64) * s.astype(np.float64)           # exact: 8 + 24 significant bits
+        once = exact.astype(np.float16)
+        twice = (c.astype(np.float32) * s).astype(np.float16)
+        differs = once != twice
+        picked_codes.extend(c[differs].tolist())
+        picked_scales.extend(s[differs].tolist())
+    groups = 4096
+    codes = np.zeros((groups, 64), dtype=np.int8)
+    codes[:, 0] = picked_codes[:groups]
+    codes[:, 37] = picked_codes[:groups]
+    scales = np.array(picked_scales[:groups], dtype=np.float32)
+    t_codes = torch.from_numpy(codes.reshape(-1)).to(hip_device)
+    t_scales = torch.from_numpy(scales).to(hip_device)
+    n = groups * 64
+    want = codec_torch.dequantize(t_codes.cpu(), t_scales.cpu(), n, 64, "fp16")
+    assert_same_bits(ops.dequant(t_codes, t_scales, n, dtype=torch.float16), want, "decode")
+    out = torch.empty(n, dtype=torch.float16, device=hip_device)
+    assert ops.dequant_reduce_into([(t_codes, t_scales)], out)
+    assert_same_bits(out, want, "reduce W=1")
+    # and through the fused error-feedback quantize: restored = fp16(code*scale) of the payload just made
+    x = want.float().to(hip_device)
+    c2 = torch.empty(n, dtype=torch.int8, device=hip_device)
+    s2 = torch.empty(groups, dtype=torch.float32, device=hip_device)
+    restored = torch.empty(n, dtype=torch.float16, device=hip_device)
+    half_in = x.half()
+    assert ops.quant_pack_into(half_in, c2, s2, restored=restored)
+    w_codes, w_scales, w_restored, _ = codec_torch.ef_round_trip(half_in.cpu(), None, 64, "fp16")
+    assert torch.equal(c2.cpu(), w_codes)
+    assert_same_bits(restored, w_restored, "restored")
+
+
+@pytest.mark.parametrize("op", ["sum", "max", "min"])
+def test_dequant_with_reduce_op_combines_with_existing_output(ops, hip_device, op):
+    n = 70_000
+    x = gradient_like(n, torch.float32, 41, hip_device)
+    codes, scales = ops.quant_pack(x)
+    before = gradient_like(n, torch.float32, 42, hip_device)
+    out = before.clone()
+    assert ops.dequant_into(codes, scales, out, reduce_op=op)
+    decoded = codec_torch.dequantize(codes.cpu(), scales.cpu(), n)
+    want = {"sum": before.cpu() + decoded, "max": torch.maximum(before.cpu(), decoded),
+            "min": torch.minimum(before.cpu(), decoded)}[op]
+    assert_same_bits(out, want, op)
+
+
+def make_payloads(ops, world, n, device, seed, g=64):
+    payloads = []
+    for r in range(world):
+        payloads.append(ops.quant_pack(gradient_like(n, torch.float32, seed + r, device, outliers=False), group_size=g))
+    return payloads
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 5, 8])
+@pytest.mark.parametrize("n", [64, 1000, 16_384 * 3 + 5])
+def test_dequant_reduce_sum_bit_exact(ops, hip_device, world, n):
+    payloads = make_payloads(ops, world, n, hip_device, 500)
+    out = torch.empty(n, dtype=torch.float32, device=hip_device)
+    assert ops.dequant_reduce_into(payloads, out)
+    want = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in payloads], n, 64, "fp32", "sum")
+    assert_same_bits(out, want, "reduced")
+
+
+@pytest.mark.parametrize("world", [3, 8])
+@pytest.mark.parametrize("out_dtype", ["fp32", "fp16", "bf16"])
+def test_dequant_reduce_mean_and_16bit_accumulation(ops, hip_device, world, out_dtype):
+    n = 50_001
+    payloads = make_payloads(ops, world, n, hip_device, 600)
+    out = torch.empty(n, dtype=DTYPES[out_dtype], device=hip_device)
+    assert ops.dequant_reduce_into(payloads, out, divisor=world)
+    want = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in payloads], n, 64, out_dtype, "mean")
+    assert_same_bits(out, want, "mean")
+
+
+def test_dequant_reduce_order_follows_the_list(ops, hip_device):
+    n = 64 * 2000
+    payloads = make_payloads(ops, 8, n, hip_device, 700)
+    fwd = torch.empty(n, dtype=torch.float32, device=hip_device)
+    rev = torch.empty_like(fwd)
+    assert ops.dequant_reduce_into(payloads, fwd)
+    assert ops.dequant_reduce_into(payloads[::-1], rev)
+    cpu = [(c.cpu(), s.cpu()) for c, s in payloads]
+    assert_same_bits(fwd, codec_torch.reduce_payloads(cpu, n), "forward")
+    assert_same_bits(rev, codec_torch.reduce_payloads(cpu[::-1], n), "reverse")
+    assert not torch.equal(fwd, rev)
+
+
+def test_dequant_reduce_config2_shard(ops, hip_device):
+    """W=8 payloads of a 3,276,800-element shard (100 MiB fp32 bucket split 8 ways), fixed rank order."""
+    n = 3_276_800
+    payloads = make_payloads(ops, 8, n, hip_device, 1234)
+    out = torch.empty(n, dtype=torch.float32, device=hip_device)
+    assert ops.dequant_reduce_into(payloads, out)
+    want = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in payloads], n)
+    assert_same_bits(out, want, "shard")
+
+
+def test_dequant_reduce_linearity_at_full_bucket_size(ops, hip_device):
+    """All-gather-reduce shape (8 payloads x 26,214,400): the W-way sum equals decode-and-add one by one."""
+    n = 26_214_400
+    x = gradient_like(n, torch.float32, 55, hip_device, outliers=False)
+    payloads = []
+    for r in range(8):
+        payloads.append(ops.quant_pack(torch.roll(x, 4099 * r) * (1.0 + 0.25 * r)))
+    fused = torch.empty(n, dtype=torch.float32, device=hip_device)
+    assert ops.dequant_reduce_into(payloads, fused)
+    chained = torch.empty_like(fused)
+    for r, (codes, scales) in enumerate(payloads):
+        assert ops.dequant_into(codes, scales, chained, reduce_op="none" if r == 0 else "sum")
+    assert torch.equal(fused, chained)
+
+
+def test_dequant_reduce_with_error_feedback_update(ops, hip_device):
+    n = 40_000
+    world = 4
+    payloads = make_payloads(ops, world, n, hip_device, 800)
+    prepared = gradient_like(n, torch.float32, 801, hip_device)
+    restored = torch.empty(n, dtype=torch.float32, device=hip_device)
+    residual = torch.empty_like(restored)
+    assert ops.dequant_reduce_into(payloads, restored, divisor=world, prepared=prepared, new_residual=residual)
+    want = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in payloads], n, 64, "fp32", "mean")
+    assert_same_bits(restored, want, "restored")
+    assert_same_bits(residual, prepared.cpu() - want, "residual")
+
+
+def test_more_than_eight_payloads_is_unsupported_not_an_error(ops, hip_device):
+    payloads = make_payloads(ops, 9, 128, hip_device, 900)
+    out = torch.empty(128, dtype=torch.float32, device=hip_device)
+    assert ops.dequant_reduce_into(payloads, out) is False
+
+
+def test_contract_violations_raise(ops, hip_device):
+    x = gradient_like(128, torch.float32, 1, hip_device)
+    codes, scales = ops.quant_pack(x)
+    out = torch.empty(128, dtype=torch.float32, device=hip_device)
+    with pytest.raises(RuntimeError, match="divisor must be > 0"):
+        ops.dequant_reduce_into([(codes, scales)], out, divisor=0)
+    with pytest.raises(RuntimeError, match="inputs must not be empty"):
+        ops.dequant_reduce_into([], out)
+    with pytest.raises(RuntimeError, match="invalid quantized payload size"):
+        ops.quant_pack_into(x, codes[:64], scales)
+    with pytest.raises(RuntimeError, match="must be a GPU tensor"):
+        ops.quant_pack_into(x.cpu(), codes, scales)
+    with pytest.raises(RuntimeError, match="must be contiguous"):
+        ops.quant_pack_into(torch.empty(128, 2, device=hip_device)[:, 0], codes, scales)
+
+
+def test_empty_input_is_a_no_op(ops, hip_device):
+    x = torch.empty(0, dtype=torch.float32, device=hip_device)
+    codes, scales = ops.quant_pack(x)
+    assert codes.numel() == 0 and scales.numel() == 0
+
+
+# --------------------------------------------------------------------------- #
+# error feedback
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("grad_dtype,res_dtype,restored_dtype", [
+    ("bf16", "fp32", "fp32"), ("bf16", "fp32", "bf16"), ("fp16", "fp32", "fp16"), ("fp32", "fp32", "fp32"),
+    ("bf16", "bf16", "bf16"), ("bf16", None, "bf16"), ("fp32", None, "fp32"), ("fp16", "fp16", "fp32"),
+])
+@pytest.mark.parametrize("n", [2048 * 5, 30_011])
+def test_ef_quant_pack_matches_the_processor_round_trip(ops, hip_device, grad_dtype, res_dtype, restored_dtype, n):
+    grad = gradient_like(n, DTYPES[grad_dtype], 1100 + n, hip_device)
+    residual = None if res_dtype is None else gradient_like(n, DTYPES[res_dtype], 1101, hip_device, sigma=1e-5,
+                                                             outliers=False)
+    p_dtype = grad.dtype if residual is None else ops.promote(grad.dtype, residual.dtype)
+    n_dtype = ops.promote(p_dtype, DTYPES[restored_dtype])
+    groups = ops.num_groups(n, 64)
+    codes = torch.empty(groups * 64, dtype=torch.int8, device=hip_device)
+    scales = torch.empty(groups, dtype=torch.float32, device=hip_device)
+    restored = torch.empty(n, dtype=DTYPES[restored_dtype], device=hip_device)
+    new_residual = torch.empty(n, dtype=n_dtype, device=hip_device)
+    assert ops.quant_pack_into(grad, codes, scales, residual=residual, new_residual=new_residual, restored=restored)
+    w_codes, w_scales, w_restored, w_residual = codec_torch.ef_round_trip(
+        grad.cpu(), None if residual is None else residual.cpu(), 64, restored_dtype)
+    assert torch.equal(codes.cpu(), w_codes)
+    assert_same_bits(scales, w_scales, "scales")
+    assert_same_bits(restored, w_restored, "restored")
+    assert_same_bits(new_residual, w_residual, "residual")
+
+
+def test_ef_in_place_residual_over_ten_steps_config3_shape_scaled(ops, hip_device):
+    """Config 3 at 1/16 size (3,276,800 bf16 values), 10 steps, residual updated in place."""
+    n = 3_276_800
+    residual = gradient_like(n, torch.float32, 1234, hip_device, sigma=1e-5, outliers=False)
+    cpu_residual = residual.cpu()
+    groups = ops.num_groups(n, 64)
+    codes = torch.empty(groups * 64, dtype=torch.int8, device=hip_device)
+    scales = torch.empty(groups, dtype=torch.float32, device=hip_device)
+    for step in range(10):
+        grad = gradient_like(n, torch.bfloat16, 2000 + step, hip_device, outliers=False)
+        assert ops.quant_pack_into(grad, codes, scales, residual=residual, new_residual=residual)
+        w_codes, w_scales, _w_restored, cpu_residual = codec_torch.ef_round_trip(grad.cpu(), cpu_residual, 64, "fp32")
+        assert torch.equal(codes.cpu(), w_codes), f"step {step}"
+        assert_same_bits(scales, w_scales, f"scales step {step}")
+        assert_same_bits(residual, cpu_residual, f"residual step {step}")
+
+
+@pytest.mark.parametrize("p,t", [("fp32", "fp32"), ("fp32", "bf16"), ("bf16", "bf16"), ("fp16", "fp32")])
+def test_standalone_ef_update(ops, hip_device, p, t):
+    n = 33_333
+    prepared = gradient_like(n, DTYPES[p], 1, hip_device)
+    restored = gradient_like(n, DTYPES[t], 2, hip_device)
+    residual = torch.empty(n, dtype=ops.promote(DTYPES[p], DTYPES[t]), device=hip_device)
+    assert ops.ef_update_into(prepared, restored, residual)
+    assert_same_bits(residual, prepared.cpu() - restored.cpu(), "residual")
+
+
+# --------------------------------------------------------------------------- #
+# chunked plan (reduce-scatter leg + requantize + all-gather leg)
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("n,world", [(64 * 8 * 100, 8), (64 * 9 + 30, 4), (1_000_003, 8), (5, 8)])
+def test_chunked_quantize_restarts_groups_per_chunk(ops, hip_device, n, world):
+    x = gradient_like(n, torch.float32, 1300 + n, hip_device)
+    shard = -(-n // world)
+    stride = (ops.payload_nbytes(shard) + 15) // 16 * 16
+    payloads = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+    assert ops.quant_pack_chunks_into(x, payloads, world)
+    want = codec_np.quantize_chunks(x.cpu().numpy(), world, 64)
+    for d, (codes, scales) in enumerate(want):
+        row = payloads[d, :ops.payload_nbytes(shard)].cpu().numpy()
+        assert np.array_equal(row, codec_np.pack(codes, scales)), f"chunk {d}"
+
+
+def test_full_plan_config4_scaled(ops, hip_device):
+    """Config 4 at 1/32 size: quantize 8 chunks per peer, reduce, requantize, decode all shards."""
+    world, n = 8, 1_638_400 + 40          # ragged: shard = 204_805
+    peers = [gradient_like(n, torch.float32, 1234 + r, hip_device, outliers=False) for r in range(world)]
+    shard = -(-n // world)
+    nbytes = ops.payload_nbytes(shard)
+    stride = (nbytes + 15) // 16 * 16
+    sent = []
+    for x in peers:
+        rows = torch.empty(world, stride, dtype=torch.uint8, device=hip_device)
+        assert ops.quant_pack_chunks_into(x, rows, world)
+        sent.append(rows)
+    gathered = torch.empty(world, stride, dtype=torch.uint8, device=hip_device)
+    shards = []
+    for dest in range(world):
+        received = [ops.split_payload(sent[src][dest, :nbytes], shard) for src in range(world)]
+        out = torch.empty(shard, dtype=torch.float32, device=hip_device)
+        assert ops.dequant_reduce_into(received, out)
+        shards.append(out)
+        assert ops.quant_pack_payload_into(out, gathered[dest, :nbytes])
+    restored = torch.empty(n, dtype=torch.float32, device=hip_device)
+    assert ops.dequant_chunks_into(gathered, restored, shard)
+    want_shards, want_restored = codec_np.reduce_scatter_all_gather_plan([p.cpu().numpy() for p in peers], 64, "sum")
+    for d in range(world):
+        assert np.array_equal(shards[d].cpu().numpy().view(np.uint32), want_shards[d].view(np.uint32)), f"shard {d}"
+    assert np.array_equal(restored.cpu().numpy().view(np.uint32), want_restored.view(np.uint32))
