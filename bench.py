@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the compression hot path on one MI355X.
+
+One "step" pushes one 100 MiB fp32 gradient bucket through the compressed reduce-scatter hot path
+of one rank at simulated world size 8 (BASELINE config 2): quantize+pack the bucket's 8 destination
+chunks (one launch), then the fused dequant-reduce of the 8 peer payloads of this rank's shard in
+fixed rank order (one launch).  Peer payloads are synthesised in HBM before the timed region; there
+are no collectives.  `value` is GB/s of gradient input consumed per step.
+
+The line also carries, for the dominant kernel (quantize+pack of the 100 MiB bucket), the HBM
+roofline: algorithmic bytes per launch / average launch duration measured with HIP events around
+back-to-back launches on the launch stream; and a CPU baseline: the torch-op restatement of the
+reference codec timed on this host for the same step.  `kernels` adds the same roofline figures for
+the other kernels of the path (shard reduce, full-bucket all-gather-reduce shape, EF quantize).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12          # MI355X published HBM3E bandwidth, bytes/s
+BUCKET_NUMEL = 26_214_400  # 100 MiB of fp32
+WORLD = 8
+GROUP = 64
+SEED = 1234
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), or None
+MEASURED_TRAFFIC = {"quant_pack_chunks": None}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--sets", type=int, default=6, help="distinct buffer sets rotated through (defeats the LLC)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default="", help="comma list of kernel legs to time (for profiling one kernel)")
+    return ap.parse_args()
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU's share of the path; --gpus {args.gpus} is not supported "
+              "(this build has no collectives or multi-GPU sharding)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from lowbit_comm_amd.hip import ops
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream(dev)
+
+    n, world, g = BUCKET_NUMEL, WORLD, GROUP
+    shard = n // world
+    payload_bytes = ops.payload_nbytes(shard, g)
+    stride = (payload_bytes + 255) // 256 * 256
+    only = {k for k in args.only.split(",") if k}
+
+    def gen(seed, numel, sigma, dtype=torch.float32):
+        gen_ = torch.Generator(device=dev).manual_seed(seed)
+        return (torch.randn(numel, generator=gen_, device=dev) * sigma).to(dtype)
+
+    # ---- synthetic inputs, resident in HBM before any timing -----------------------------------
+    sets = []
+    for s in range(args.sets):
+        bucket = gen(SEED + 100 * s, n, 1e-3)                       # this rank's bucket
+        sent = torch.empty(world, stride, dtype=torch.uint8, device=dev)
+        received = torch.empty(world, stride, dtype=torch.uint8, device=dev)
+        for r in range(world):                                      # peer r's chunk for this rank's shard
+            peer_chunk = gen(SEED + 100 * s + 1 + r, shard, 1e-3)
+            assert ops.quant_pack_payload_into(peer_chunk, received[r, :payload_bytes], group_size=g)
+        out = torch.empty(shard, dtype=torch.float32, device=dev)
+        pairs = [ops.split_payload(received[r, :payload_bytes], shard, g) for r in range(world)]
+        sets.append({
+            "bucket": bucket, "sent": sent, "received": received, "out": out,
+            "quant": ops.bind_quant_pack_chunks(bucket, sent, world, group_size=g),
+            "reduce": ops.bind_dequant_reduce(pairs, out, group_size=g),
+        })
+    torch.cuda.synchronize()
+
+    def step(i):
+        s = sets[i % len(sets)]
+        s["quant"]()
+        s["reduce"]()
+
+    def timed(fn, count, warmup):
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        for i in range(count):
+            fn(i)
+        stop.record(stream)
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) * 1e-3  # seconds
+
+    # ---- the step ---------------------------------------------------------------------------------
+    result = {}
+    if not only or "step" in only:
+        total = timed(step, args.steps, args.warmup)
+        result["ms_per_step"] = total / args.steps * 1e3
+        result["value"] = n * 4 * args.steps / total / 1e9
+
+    # ---- per-kernel launch durations ---------------------------------------------------------------
+    kernels = {}
+
+    def leg(name, fn, algorithmic_bytes, launches=None, warmup=None):
+        if only and name not in only:
+            return
+        launches = launches or args.steps
+        seconds = timed(fn, launches, warmup if warmup is not None else args.warmup) / launches
+        kernels[name] = {
+            "us_per_launch": seconds * 1e6, "algorithmic_bytes": algorithmic_bytes,
+            "achieved_GBps": algorithmic_bytes / seconds / 1e9, "frac_of_hbm_peak": algorithmic_bytes / seconds / HBM_PEAK,
+        }
+
+    quant_bytes = n * 4 + world * payload_bytes
+    leg("quant_pack_chunks", lambda i: sets[i % len(sets)]["quant"](), quant_bytes)
+    leg("dequant_reduce_shard", lambda i: sets[i % len(sets)]["reduce"](), world * payload_bytes + shard * 4)
+
+    if "copy_calibration" in only:
+        # a plain device copy of known size (100 MiB read + 100 MiB written) to scale the HBM counters by
+        srcs = [sets[i]["bucket"] for i in range(len(sets))]
+        dsts = [torch.empty_like(srcs[0]) for _ in range(2)]
+        leg("copy_calibration", lambda i: dsts[i % 2].copy_(srcs[i % len(srcs)]), 2 * n * 4)
+
+    if not only or "dequant_reduce_full" in only or "ef_quant_pack" in only:
+        # all-gather-reduce shape: 8 payloads of the whole bucket -> fp32 bucket
+        full_sets = []
+        if not only or "dequant_reduce_full" in only:
+            for s in range(2):
+                pairs = [ops.quant_pack(gen(SEED + 7000 + 10 * s + r, n, 1e-3), group_size=g) for r in range(world)]
+                out = torch.empty(n, dtype=torch.float32, device=dev)
+                full_sets.append(ops.bind_dequant_reduce(pairs, out, group_size=g))
+            leg("dequant_reduce_full", lambda i: full_sets[i % 2](), world * ops.payload_nbytes(n, g) + n * 4,
+                launches=max(20, args.steps // 4), warmup=5)
+            del full_sets
+        if not only or "ef_quant_pack" in only:
+            # config 3: 100 MiB bf16 gradient + fp32 residual, residual updated in place
+            n3 = 52_428_800
+            groups3 = ops.num_groups(n3, g)
+            ef_sets = []
+            for s in range(2):
+                grad = gen(SEED + 9000 + s, n3, 1e-3, torch.bfloat16)
+                residual = gen(SEED + 9100 + s, n3, 1e-5)
+                codes = torch.empty(groups3 * g, dtype=torch.int8, device=dev)
+                scales = torch.empty(groups3, dtype=torch.float32, device=dev)
+                ef_sets.append(ops.bind_quant_pack(grad, codes, scales, group_size=g, residual=residual,
+                                                   new_residual=residual))
+            leg("ef_quant_pack", lambda i: ef_sets[i % 2](), n3 * (2 + 4 + 4) + groups3 * (g + 4),
+                launches=max(20, args.steps // 4), warmup=5)
+            del ef_sets
+        torch.cuda.empty_cache()
+
+    # ---- parity of the timed workload + CPU baseline (oracle, checker only) -------------------
+    cpu_baseline = None
+    parity = None
+    if not args.no_cpu_baseline and not only:
+        from oracle import codec_torch
+
+        s0 = sets[0]
+        s0["quant"](); s0["reduce"]()
+        torch.cuda.synchronize()
+        bucket_cpu = s0["bucket"].cpu()
+        received_cpu = s0["received"].cpu()
+
+        def cpu_step():
+            payloads = [codec_torch.quantize(bucket_cpu[d * shard:(d + 1) * shard], g) for d in range(world)]
+            peers = []
+            for r in range(world):
+                row = received_cpu[r, :payload_bytes]
+                peers.append((row[:shard].view(torch.int8), row[shard:].view(torch.float32)))
+            return payloads, codec_torch.reduce_payloads(peers, shard, g, "fp32", "sum")
+
+        payloads, reduced = cpu_step()
+        sent_cpu = s0["sent"].cpu()
+        ok = all(torch.equal(sent_cpu[d, :payload_bytes], codec_torch.pack(*payloads[d])) for d in range(world))
+        ok = ok and torch.equal(s0["out"].cpu().view(torch.int32), reduced.view(torch.int32))
+        parity = "bit-exact" if ok else "MISMATCH"
+        times = []
+        deadline = time.perf_counter() + 25.0
+        for i in range(12):
+            t0 = time.perf_counter()
+            cpu_step()
+            times.append(time.perf_counter() - t0)
+            if time.perf_counter() > deadline:
+                break
+        times = sorted(times[2:] or times)
+        median = times[len(times) // 2]
+        cpu_baseline = {
+            "value": n * 4 / median / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{len(times)} timed repeats of the full step (8x quantize of 3,276,800-element chunks + "
+                      f"8-payload left-fold reduce of one shard) with torch CPU ops, median {median * 1e3:.1f} ms; "
+                      f"host has {os.cpu_count()} logical CPUs",
+        }
+
+    dominant = kernels.get("quant_pack_chunks")
+    line = {
+        "metric": "quant-pack & fused dequant-reduce GB/s on 1 MI355X; % of HBM roofline",
+        "value": result.get("value"),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": result.get("ms_per_step"),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "config 2: 100 MiB fp32 bucket ~N(0,1e-3 std), W=8, group 64: quant-pack of the 8 chunks + "
+                        "fused dequant-reduce of one rank's shard (8 payloads x 3,276,800 codes), fixed rank order",
+            "bucket_numel": n, "world_size": world, "group_size": g, "buffer_sets": args.sets,
+            "value_is": "bucket bytes (104,857,600) consumed per step / step time",
+        },
+        "roofline": None if dominant is None else {
+            "bound": "hbm", "kernel": "quant_pack_kernel (100 MiB fp32 bucket, 8 chunks, one launch)",
+            "achieved": dominant["achieved_GBps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": dominant["frac_of_hbm_peak"], "traffic": MEASURED_TRAFFIC["quant_pack_chunks"],
+            "algorithmic_bytes": dominant["algorithmic_bytes"], "us_per_launch": dominant["us_per_launch"],
+        },
+        "cpu_baseline": cpu_baseline,
+        "parity": parity,
+        "kernels": kernels,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -50,6 +50,15 @@ int lbc_abi_version(void);
 const char *lbc_last_error(void);
 
 /*
+ * Tuning knob with no counterpart in the reference: calls that move at least
+ * `min_bytes` use non-temporal (streaming) loads and stores, smaller ones plain
+ * vector access.  Process-wide; the initial value is 96 MiB or the environment
+ * variable LBC_STREAM_MIN_BYTES.  Returns the previous threshold.  Results do not
+ * depend on it.
+ */
+int64_t lbc_set_stream_min_bytes(int64_t min_bytes);
+
+/*
  * Quantize + pack, optionally fused with error feedback.
  * Replaces: quantize_tensor_fallback (ccdl_comm/quantization/torch_fallback.py:10-36),
  * native inplace_quantize_pack (ccdl_comm/csrc/quantization/quant_pack_kernel.cu:220-275),
@@ -138,7 +147,8 @@ int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int worl
 
 /*
  * residual = prepared - restored, element-wise, subtraction in fp32, rounded to
- * residual_dtype.  Replaces native inplace_error_feedback_update (ccdl_comm/csrc/
+ * residual_dtype.  Supported: restored_dtype equal to prepared_dtype or either of
+ * them LBC_F32, and residual_dtype their torch promotion; else LBC_UNSUPPORTED.  Replaces native inplace_error_feedback_update (ccdl_comm/csrc/
  * quantization/dequant_reduce_kernel.cu:136-148,223-233,266-313) and
  * ErrorFeedbackState.update (ccdl_comm/quantization/error_feedback.py:38-41).
  */

@@ -25,14 +25,17 @@ namespace {
 template <typename OT> struct decode_tiling {
     static constexpr int VEC = sizeof(OT) == 4 ? 4 : 8;
     static constexpr int TILE = kWave * VEC;
-    static constexpr int UNROLL = 4;
+#ifndef LBC_DECODE_UNROLL
+#define LBC_DECODE_UNROLL 1
+#endif
+    static constexpr int UNROLL = LBC_DECODE_UNROLL;
     static constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock * UNROLL;
 };
 
-template <int VEC, bool ALIGNED>
+template <int VEC, int MODE>
 __device__ __forceinline__ void load_codes(const int8_t *__restrict__ p, uint32_t (&w)[VEC / 4]) {
-    if constexpr (ALIGNED) {
-        load_vec<uint32_t, VEC / 4, true>(reinterpret_cast<const uint32_t *>(p), w);
+    if constexpr (MODE != kScalar) {
+        load_vec<uint32_t, VEC / 4, MODE>(reinterpret_cast<const uint32_t *>(p), w);
     } else {
 #pragma unroll
         for (int k = 0; k < VEC / 4; ++k) {
@@ -46,7 +49,7 @@ __device__ __forceinline__ void load_codes(const int8_t *__restrict__ p, uint32_
 // ---------------------------------------------------------------------------
 // fused dequant-reduce
 // ---------------------------------------------------------------------------
-template <typename OT, int G, int W, bool ALIGNED>
+template <typename OT, int G, int W, int MODE>
 __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs a) {
     using T = decode_tiling<OT>;
     constexpr int VEC = T::VEC;
@@ -60,7 +63,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
     OT *new_r = static_cast<OT *>(a.new_residual);
     const bool mean = a.divisor != 1.0f;
 
-    if (block_first + T::BLOCK_ELEMS <= a.numel) {
+    if (MODE != kScalar && block_first + T::BLOCK_ELEMS <= a.numel) {
         // ---- interior block ---------------------------------------------------
         uint32_t words[UNROLL][W][VEC / 4];
         float scale[UNROLL][W];
@@ -71,7 +74,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
             const int64_t g = e0[u] / G;
 #pragma unroll
             for (int r = 0; r < W; ++r) {
-                load_codes<VEC, ALIGNED>(a.codes[r] + e0[u], words[u][r]);
+                load_codes<VEC, MODE>(a.codes[r] + e0[u], words[u][r]);
                 scale[u][r] = a.scales[r][g];
             }
         }
@@ -95,13 +98,13 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
             OT o[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) o[i] = narrow<OT>(acc[i]);
-            store_vec<OT, VEC, ALIGNED>(out + e0[u], o);
+            store_vec<OT, VEC, MODE>(out + e0[u], o);
             if (new_r != nullptr) {
                 OT pv[VEC], d[VEC];
-                load_vec<OT, VEC, ALIGNED>(prepared + e0[u], pv);
+                load_vec<OT, VEC, MODE>(prepared + e0[u], pv);
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) d[i] = narrow<OT>(widen(pv[i]) - acc[i]);
-                store_vec<OT, VEC, ALIGNED>(new_r + e0[u], d);
+                store_vec<OT, VEC, MODE>(new_r + e0[u], d);
             }
         }
         return;
@@ -128,39 +131,40 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
 }
 
 template <typename OT, int G, int W>
-hipError_t launch_reduce_w(bool aligned, const ReduceArgs &a, hipStream_t stream) {
+hipError_t launch_reduce_w(int mode, const ReduceArgs &a, hipStream_t stream) {
     using T = decode_tiling<OT>;
     const int64_t blocks = (a.numel + T::BLOCK_ELEMS - 1) / T::BLOCK_ELEMS;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-    if (aligned)
-        hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, true>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a);
-    else
-        hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, false>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a);
+    switch (mode) {
+        case kStream: hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, kStream>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a); break;
+        case kVector: hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, kVector>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a); break;
+        default: hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, kScalar>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a); break;
+    }
     return hipGetLastError();
 }
 
 template <typename OT, int G>
-hipError_t launch_reduce_g(int world, bool aligned, const ReduceArgs &a, hipStream_t s) {
+hipError_t launch_reduce_g(int world, int mode, const ReduceArgs &a, hipStream_t s) {
     switch (world) {
-        case 1: return launch_reduce_w<OT, G, 1>(aligned, a, s);
-        case 2: return launch_reduce_w<OT, G, 2>(aligned, a, s);
-        case 3: return launch_reduce_w<OT, G, 3>(aligned, a, s);
-        case 4: return launch_reduce_w<OT, G, 4>(aligned, a, s);
-        case 5: return launch_reduce_w<OT, G, 5>(aligned, a, s);
-        case 6: return launch_reduce_w<OT, G, 6>(aligned, a, s);
-        case 7: return launch_reduce_w<OT, G, 7>(aligned, a, s);
-        case 8: return launch_reduce_w<OT, G, 8>(aligned, a, s);
+        case 1: return launch_reduce_w<OT, G, 1>(mode, a, s);
+        case 2: return launch_reduce_w<OT, G, 2>(mode, a, s);
+        case 3: return launch_reduce_w<OT, G, 3>(mode, a, s);
+        case 4: return launch_reduce_w<OT, G, 4>(mode, a, s);
+        case 5: return launch_reduce_w<OT, G, 5>(mode, a, s);
+        case 6: return launch_reduce_w<OT, G, 6>(mode, a, s);
+        case 7: return launch_reduce_w<OT, G, 7>(mode, a, s);
+        case 8: return launch_reduce_w<OT, G, 8>(mode, a, s);
         default: return hipErrorNotSupported;
     }
 }
 
 template <typename OT>
-hipError_t launch_reduce_t(int g, int world, bool aligned, const ReduceArgs &a, hipStream_t s) {
+hipError_t launch_reduce_t(int g, int world, int mode, const ReduceArgs &a, hipStream_t s) {
     switch (g) {
-        case 64: return launch_reduce_g<OT, 64>(world, aligned, a, s);
-        case 32: return launch_reduce_g<OT, 32>(world, aligned, a, s);
-        case 16: return launch_reduce_g<OT, 16>(world, aligned, a, s);
+        case 64: return launch_reduce_g<OT, 64>(world, mode, a, s);
+        case 32: return launch_reduce_g<OT, 32>(world, mode, a, s);
+        case 16: return launch_reduce_g<OT, 16>(world, mode, a, s);
         default: return hipErrorNotSupported;
     }
 }
@@ -175,7 +179,7 @@ template <int OP> __device__ __forceinline__ float combine(float old, float v) {
     else return v;
 }
 
-template <typename OT, int G, int OP, bool ALIGNED>
+template <typename OT, int G, int OP, int MODE>
 __global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
     using T = decode_tiling<OT>;
     constexpr int VEC = T::VEC;
@@ -193,27 +197,27 @@ __global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
     const int64_t block_first = static_cast<int64_t>(blockIdx.x) * T::BLOCK_ELEMS;
     if (block_first >= valid) return;
 
-    if (block_first + T::BLOCK_ELEMS <= valid) {
+    if (MODE != kScalar && block_first + T::BLOCK_ELEMS <= valid) {
         uint32_t words[UNROLL][VEC / 4];
         float scale[UNROLL];
         int64_t e0[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             e0[u] = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
-            load_codes<VEC, ALIGNED>(codes + e0[u], words[u]);
+            load_codes<VEC, MODE>(codes + e0[u], words[u]);
             scale[u] = scales[e0[u] / G];
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             OT o[VEC];
-            if constexpr (OP != 0) load_vec<OT, VEC, ALIGNED>(out + e0[u], o);
+            if constexpr (OP != 0) load_vec<OT, VEC, MODE>(out + e0[u], o);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
                 float v = round_through<OT>(code_to_float(words[u][i / 4], i % 4) * scale[u]);
                 if constexpr (OP != 0) v = round_through<OT>(combine<OP>(widen(o[i]), v));
                 o[i] = narrow<OT>(v);
             }
-            store_vec<OT, VEC, ALIGNED>(out + e0[u], o);
+            store_vec<OT, VEC, MODE>(out + e0[u], o);
         }
         return;
     }
@@ -231,36 +235,37 @@ __global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
 }
 
 template <typename OT, int G, int OP>
-hipError_t launch_decode_op(bool aligned, const DecodeArgs &a, int world, hipStream_t stream) {
+hipError_t launch_decode_op(int mode, const DecodeArgs &a, int world, hipStream_t stream) {
     using T = decode_tiling<OT>;
     const int64_t blocks = (a.shard_numel + T::BLOCK_ELEMS - 1) / T::BLOCK_ELEMS;
     if (blocks == 0 || world == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL || world > 65535) return hipErrorInvalidValue;
     dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(world));
-    if (aligned)
-        hipLaunchKernelGGL((decode_kernel<OT, G, OP, true>), grid, dim3(kBlock), 0, stream, a);
-    else
-        hipLaunchKernelGGL((decode_kernel<OT, G, OP, false>), grid, dim3(kBlock), 0, stream, a);
+    switch (mode) {
+        case kStream: hipLaunchKernelGGL((decode_kernel<OT, G, OP, kStream>), grid, dim3(kBlock), 0, stream, a); break;
+        case kVector: hipLaunchKernelGGL((decode_kernel<OT, G, OP, kVector>), grid, dim3(kBlock), 0, stream, a); break;
+        default: hipLaunchKernelGGL((decode_kernel<OT, G, OP, kScalar>), grid, dim3(kBlock), 0, stream, a); break;
+    }
     return hipGetLastError();
 }
 
 template <typename OT, int G>
-hipError_t launch_decode_g(int op, bool aligned, const DecodeArgs &a, int world, hipStream_t s) {
+hipError_t launch_decode_g(int op, int mode, const DecodeArgs &a, int world, hipStream_t s) {
     switch (op) {
-        case 0: return launch_decode_op<OT, G, 0>(aligned, a, world, s);
-        case 1: return launch_decode_op<OT, G, 1>(aligned, a, world, s);
-        case 2: return launch_decode_op<OT, G, 2>(aligned, a, world, s);
-        case 3: return launch_decode_op<OT, G, 3>(aligned, a, world, s);
+        case 0: return launch_decode_op<OT, G, 0>(mode, a, world, s);
+        case 1: return launch_decode_op<OT, G, 1>(mode, a, world, s);
+        case 2: return launch_decode_op<OT, G, 2>(mode, a, world, s);
+        case 3: return launch_decode_op<OT, G, 3>(mode, a, world, s);
         default: return hipErrorNotSupported;
     }
 }
 
 template <typename OT>
-hipError_t launch_decode_t(int g, int op, bool aligned, const DecodeArgs &a, int world, hipStream_t s) {
+hipError_t launch_decode_t(int g, int op, int mode, const DecodeArgs &a, int world, hipStream_t s) {
     switch (g) {
-        case 64: return launch_decode_g<OT, 64>(op, aligned, a, world, s);
-        case 32: return launch_decode_g<OT, 32>(op, aligned, a, world, s);
-        case 16: return launch_decode_g<OT, 16>(op, aligned, a, world, s);
+        case 64: return launch_decode_g<OT, 64>(op, mode, a, world, s);
+        case 32: return launch_decode_g<OT, 32>(op, mode, a, world, s);
+        case 16: return launch_decode_g<OT, 16>(op, mode, a, world, s);
         default: return hipErrorNotSupported;
     }
 }
@@ -268,7 +273,7 @@ hipError_t launch_decode_t(int g, int op, bool aligned, const DecodeArgs &a, int
 // ---------------------------------------------------------------------------
 // residual = prepared - restored
 // ---------------------------------------------------------------------------
-template <typename PT, typename TT, typename RT, bool ALIGNED>
+template <typename PT, typename TT, typename RT, int MODE>
 __global__ __launch_bounds__(kBlock) void ef_update_kernel(const EfArgs a) {
     constexpr int VEC = 4;
     constexpr int UNROLL = 4;
@@ -277,14 +282,14 @@ __global__ __launch_bounds__(kBlock) void ef_update_kernel(const EfArgs a) {
     const TT *__restrict__ restored = static_cast<const TT *>(a.restored);
     RT *__restrict__ residual = static_cast<RT *>(a.residual);
     const int64_t block_first = static_cast<int64_t>(blockIdx.x) * BLOCK_ELEMS;
-    if (block_first + BLOCK_ELEMS <= a.numel) {
+    if (MODE != kScalar && block_first + BLOCK_ELEMS <= a.numel) {
         PT pv[UNROLL][VEC];
         TT tv[UNROLL][VEC];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int64_t e0 = block_first + (static_cast<int64_t>(u) * kBlock + threadIdx.x) * VEC;
-            load_vec<PT, VEC, ALIGNED>(prepared + e0, pv[u]);
-            load_vec<TT, VEC, ALIGNED>(restored + e0, tv[u]);
+            load_vec<PT, VEC, MODE>(prepared + e0, pv[u]);
+            load_vec<TT, VEC, MODE>(restored + e0, tv[u]);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
@@ -292,7 +297,7 @@ __global__ __launch_bounds__(kBlock) void ef_update_kernel(const EfArgs a) {
             RT d[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) d[i] = narrow<RT>(widen(pv[u][i]) - widen(tv[u][i]));
-            store_vec<RT, VEC, ALIGNED>(residual + e0, d);
+            store_vec<RT, VEC, MODE>(residual + e0, d);
         }
         return;
     }
@@ -307,62 +312,63 @@ __global__ __launch_bounds__(kBlock) void ef_update_kernel(const EfArgs a) {
 }
 
 template <typename PT, typename TT, typename RT>
-hipError_t launch_ef(bool aligned, const EfArgs &a, hipStream_t stream) {
+hipError_t launch_ef(int mode, const EfArgs &a, hipStream_t stream) {
     constexpr int BLOCK_ELEMS = kBlock * 4 * 4;
     const int64_t blocks = (a.numel + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-    if (aligned)
-        hipLaunchKernelGGL((ef_update_kernel<PT, TT, RT, true>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a);
-    else
-        hipLaunchKernelGGL((ef_update_kernel<PT, TT, RT, false>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a);
+    switch (mode) {
+        case kStream: hipLaunchKernelGGL((ef_update_kernel<PT, TT, RT, kStream>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a); break;
+        case kVector: hipLaunchKernelGGL((ef_update_kernel<PT, TT, RT, kVector>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a); break;
+        default: hipLaunchKernelGGL((ef_update_kernel<PT, TT, RT, kScalar>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a); break;
+    }
     return hipGetLastError();
 }
 
 // Supported combinations: restored has prepared's type or either is float; the
 // residual has their torch promotion.  Anything else is reported unsupported.
 template <typename PT, typename TT, typename RT>
-hipError_t launch_ef_checked(int r_dtype, int want, bool aligned, const EfArgs &a, hipStream_t s) {
+hipError_t launch_ef_checked(int r_dtype, int want, int mode, const EfArgs &a, hipStream_t s) {
     if (r_dtype != want) return hipErrorNotSupported;
-    return launch_ef<PT, TT, RT>(aligned, a, s);
+    return launch_ef<PT, TT, RT>(mode, a, s);
 }
 
-hipError_t launch_ef_any(int p, int t, int r, bool aligned, const EfArgs &a, hipStream_t s) {
-    if (p == kF32 && t == kF32) return launch_ef_checked<float, float, float>(r, kF32, aligned, a, s);
-    if (p == kF32 && t == kF16) return launch_ef_checked<float, f16, float>(r, kF32, aligned, a, s);
-    if (p == kF32 && t == kBF16) return launch_ef_checked<float, bf16, float>(r, kF32, aligned, a, s);
-    if (p == kF16 && t == kF32) return launch_ef_checked<f16, float, float>(r, kF32, aligned, a, s);
-    if (p == kBF16 && t == kF32) return launch_ef_checked<bf16, float, float>(r, kF32, aligned, a, s);
-    if (p == kF16 && t == kF16) return launch_ef_checked<f16, f16, f16>(r, kF16, aligned, a, s);
-    if (p == kBF16 && t == kBF16) return launch_ef_checked<bf16, bf16, bf16>(r, kBF16, aligned, a, s);
+hipError_t launch_ef_any(int p, int t, int r, int mode, const EfArgs &a, hipStream_t s) {
+    if (p == kF32 && t == kF32) return launch_ef_checked<float, float, float>(r, kF32, mode, a, s);
+    if (p == kF32 && t == kF16) return launch_ef_checked<float, f16, float>(r, kF32, mode, a, s);
+    if (p == kF32 && t == kBF16) return launch_ef_checked<float, bf16, float>(r, kF32, mode, a, s);
+    if (p == kF16 && t == kF32) return launch_ef_checked<f16, float, float>(r, kF32, mode, a, s);
+    if (p == kBF16 && t == kF32) return launch_ef_checked<bf16, float, float>(r, kF32, mode, a, s);
+    if (p == kF16 && t == kF16) return launch_ef_checked<f16, f16, f16>(r, kF16, mode, a, s);
+    if (p == kBF16 && t == kBF16) return launch_ef_checked<bf16, bf16, bf16>(r, kBF16, mode, a, s);
     return hipErrorNotSupported;
 }
 
 }  // namespace
 
-hipError_t launch_dequant_reduce(int out_dtype, int group_size, int world, bool aligned,
+hipError_t launch_dequant_reduce(int out_dtype, int group_size, int world, int mode,
                                  const ReduceArgs &args, hipStream_t stream) {
     switch (out_dtype) {
-        case kF32: return launch_reduce_t<float>(group_size, world, aligned, args, stream);
-        case kF16: return launch_reduce_t<f16>(group_size, world, aligned, args, stream);
-        case kBF16: return launch_reduce_t<bf16>(group_size, world, aligned, args, stream);
+        case kF32: return launch_reduce_t<float>(group_size, world, mode, args, stream);
+        case kF16: return launch_reduce_t<f16>(group_size, world, mode, args, stream);
+        case kBF16: return launch_reduce_t<bf16>(group_size, world, mode, args, stream);
         default: return hipErrorNotSupported;
     }
 }
 
-hipError_t launch_decode(int out_dtype, int group_size, int reduce_op, bool aligned,
+hipError_t launch_decode(int out_dtype, int group_size, int reduce_op, int mode,
                          const DecodeArgs &args, int world, hipStream_t stream) {
     switch (out_dtype) {
-        case kF32: return launch_decode_t<float>(group_size, reduce_op, aligned, args, world, stream);
-        case kF16: return launch_decode_t<f16>(group_size, reduce_op, aligned, args, world, stream);
-        case kBF16: return launch_decode_t<bf16>(group_size, reduce_op, aligned, args, world, stream);
+        case kF32: return launch_decode_t<float>(group_size, reduce_op, mode, args, world, stream);
+        case kF16: return launch_decode_t<f16>(group_size, reduce_op, mode, args, world, stream);
+        case kBF16: return launch_decode_t<bf16>(group_size, reduce_op, mode, args, world, stream);
         default: return hipErrorNotSupported;
     }
 }
 
-hipError_t launch_ef_update(int p_dtype, int t_dtype, int r_dtype, bool aligned, const EfArgs &args,
+hipError_t launch_ef_update(int p_dtype, int t_dtype, int r_dtype, int mode, const EfArgs &args,
                             hipStream_t stream) {
-    return launch_ef_any(p_dtype, t_dtype, r_dtype, aligned, args, stream);
+    return launch_ef_any(p_dtype, t_dtype, r_dtype, mode, args, stream);
 }
 
 }  // namespace lbc

@@ -16,6 +16,15 @@ constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr uint32_t kEpsBits = 0x34000000u;  // 2^-23, torch.finfo(float32).eps
 
+// Access modes of the bulk loads and stores.  kScalar: element by element (any
+// alignment).  kVector: one vector instruction per lane (the caller guarantees
+// N*sizeof(T) alignment).  kStream: vector instructions carrying the
+// non-temporal hint - every tensor here is read once and written once, and on
+// working sets well beyond the last-level cache the hint raises achieved
+// bandwidth; small working sets do better without it because the producer's
+// lines are still cached.
+enum AccessMode { kScalar = 0, kVector = 1, kStream = 2 };
+
 template <typename T, int N>
 using vec_t = T __attribute__((ext_vector_type(N)));
 
@@ -37,13 +46,13 @@ template <typename T> __device__ __forceinline__ float round_through(float v) {
 }
 
 // ---- N-element contiguous load / store --------------------------------------
-// ALIGNED: one vector instruction (the caller guarantees N*sizeof(T) alignment);
-// otherwise element by element.
-template <typename T, int N, bool ALIGNED>
+template <typename T, int N, int MODE>
 __device__ __forceinline__ void load_vec(const T *__restrict__ p, T (&dst)[N]) {
-    if constexpr (ALIGNED) {
+    if constexpr (MODE != kScalar) {
         using V = vec_t<T, N>;
-        V v = *reinterpret_cast<const V *>(p);
+        V v;
+        if constexpr (MODE == kStream) v = __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+        else v = *reinterpret_cast<const V *>(p);
 #pragma unroll
         for (int i = 0; i < N; ++i) dst[i] = v[i];
     } else {
@@ -52,17 +61,53 @@ __device__ __forceinline__ void load_vec(const T *__restrict__ p, T (&dst)[N]) {
     }
 }
 
-template <typename T, int N, bool ALIGNED>
+template <typename T, int N, int MODE>
 __device__ __forceinline__ void store_vec(T *__restrict__ p, const T (&src)[N]) {
-    if constexpr (ALIGNED) {
+    if constexpr (MODE != kScalar) {
         using V = vec_t<T, N>;
         V v;
 #pragma unroll
         for (int i = 0; i < N; ++i) v[i] = src[i];
-        *reinterpret_cast<V *>(p) = v;
+        if constexpr (MODE == kStream) __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
+        else *reinterpret_cast<V *>(p) = v;
     } else {
 #pragma unroll
         for (int i = 0; i < N; ++i) p[i] = src[i];
+    }
+}
+
+// Loads / stores N elements as ceil(N*sizeof(T)/16) instructions of at most 16 bytes.
+template <typename T, int N, int MODE>
+__device__ __forceinline__ void load_wide(const T *__restrict__ p, T (&dst)[N]) {
+    constexpr int PER = 16 / sizeof(T);
+    if constexpr (N <= PER) {
+        load_vec<T, N, MODE>(p, dst);
+    } else {
+        static_assert(N % PER == 0, "whole 16-byte pieces");
+#pragma unroll
+        for (int k = 0; k < N / PER; ++k) {
+            T piece[PER];
+            load_vec<T, PER, MODE>(p + k * PER, piece);
+#pragma unroll
+            for (int i = 0; i < PER; ++i) dst[k * PER + i] = piece[i];
+        }
+    }
+}
+
+template <typename T, int N, int MODE>
+__device__ __forceinline__ void store_wide(T *__restrict__ p, const T (&src)[N]) {
+    constexpr int PER = 16 / sizeof(T);
+    if constexpr (N <= PER) {
+        store_vec<T, N, MODE>(p, src);
+    } else {
+        static_assert(N % PER == 0, "whole 16-byte pieces");
+#pragma unroll
+        for (int k = 0; k < N / PER; ++k) {
+            T piece[PER];
+#pragma unroll
+            for (int i = 0; i < PER; ++i) piece[i] = src[k * PER + i];
+            store_vec<T, PER, MODE>(p + k * PER, piece);
+        }
     }
 }
 
@@ -88,27 +133,67 @@ template <int LANES> __device__ __forceinline__ uint32_t group_max_bits(uint32_t
     return v;
 }
 
-// scale = max(absmax / 127, 2^-23) with a true IEEE division; a NaN absmax
-// stays NaN (the comparison is false), matching torch.clamp(min=eps).
+// scale = max(absmax / 127, 2^-23), bit-identical to an IEEE division.
+// absmax/127 is evaluated as q0 = a*c, r = fma(-q0, 127, a), q1 = fma(r, c, q0)
+// with c = RN(1/127): an exhaustive sweep over every finite non-negative float
+// shows q1 == RN(a/127) (tests/native/check_scale127.c).  +Inf would turn the
+// residual into NaN and is passed through; a NaN absmax stays NaN because the
+// final comparison is false, matching torch.clamp(min=eps).
 __device__ __forceinline__ float scale_from_absmax(float absmax) {
-    float s = absmax / 127.0f;
+    const float c = as_f32(0x3C010204u);
+    const float q0 = absmax * c;
+    const float r = __builtin_fmaf(-q0, 127.0f, absmax);
+    float s = __builtin_fmaf(r, c, q0);
+    s = as_u32(absmax) == 0x7F800000u ? absmax : s;
     return s < as_f32(kEpsBits) ? as_f32(kEpsBits) : s;
 }
 
-// code = saturate(rint(p / scale)) with NaN -> 0.  rintf is round-half-even
-// (v_rndne_f32); the float -> int conversion instruction returns 0 for NaN and
-// saturates infinities, after which the integer clamp applies +-127.
-__device__ __forceinline__ int encode(float p, float scale) {
-    float q = __builtin_rintf(p / scale);
+__device__ __forceinline__ int cvt_i32(float v) {  // NaN -> 0, saturating
     int c;
-    asm("v_cvt_i32_f32 %0, %1" : "=v"(c) : "v"(q));
-    c = c < -127 ? -127 : c;
-    return c > 127 ? 127 : c;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(c) : "v"(v));
+    return c;
 }
 
+// codes[i] = rint(p[i] / scale) as the reference computes it (IEEE division,
+// then round-half-even), NaN -> 0.
+//
+// Fast path: q~ = p * rcp(scale).  v_rcp_f32 is accurate to 1 ulp and |q| <=
+// 127.0001, so |q~ - p/scale| < 2.3e-5, and the correctly rounded quotient is
+// within 2^-18 of p/scale.  rint(q~) can differ from rint(RN(p/scale)) only if a
+// half-integer lies within 2.7e-5 of q~.  Lanes whose q~ comes within 2^-14
+// (6.1e-5) of a half-integer redo their elements with the exact division; this
+// happens for about 1 element in 8000.
+//
+// No +-127 clamp is needed: |p| <= absmax and scale >= RN(absmax/127), hence
+// |p/scale| <= 127 * (1 + 2^-23) and the rounded quotient is at most 127; an
+// infinite scale gives quotient 0 or NaN.
+template <int N>
+__device__ __forceinline__ void encode_group(const float (&p)[N], float scale, int (&codes)[N]) {
+    const float inv = __builtin_amdgcn_rcpf(scale);
+    float r[N];
+    float worst = 0.0f;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const float q = p[i] * inv;
+        r[i] = __builtin_rintf(q);
+        worst = __builtin_fmaxf(worst, __builtin_fabsf(q - r[i]));
+    }
+    if (worst > 0.5f - 0x1p-14f) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) r[i] = __builtin_rintf(p[i] / scale);
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i) codes[i] = cvt_i32(r[i]);
+}
+
+// Single-element form for the ragged edge.
+__device__ __forceinline__ int encode(float p, float scale) { return cvt_i32(__builtin_rintf(p / scale)); }
+
+// Low bytes of four ints -> one little-endian word (three v_perm_b32).
 __device__ __forceinline__ uint32_t pack4(int c0, int c1, int c2, int c3) {
-    return (static_cast<uint32_t>(c0) & 0xFFu) | ((static_cast<uint32_t>(c1) & 0xFFu) << 8) |
-           ((static_cast<uint32_t>(c2) & 0xFFu) << 16) | (static_cast<uint32_t>(c3) << 24);
+    const uint32_t lo = __builtin_amdgcn_perm(static_cast<uint32_t>(c1), static_cast<uint32_t>(c0), 0x0C0C0400u);
+    const uint32_t hi = __builtin_amdgcn_perm(static_cast<uint32_t>(c3), static_cast<uint32_t>(c2), 0x04000C0Cu);
+    return lo | hi;
 }
 
 // signed byte k of a packed word -> float

@@ -52,13 +52,16 @@ struct EfArgs {
 
 // Each returns hipSuccess/last launch error, or hipErrorNotSupported when no
 // instantiation exists for the type combination.
-hipError_t launch_quant_pack(int x_dtype, int r_dtype, int d_dtype, int group_size, bool aligned,
+// `mode` is an lbc::AccessMode: 0 element-wise (any alignment), 1 vector, 2 vector + non-temporal.
+hipError_t launch_quant_pack(int x_dtype, int r_dtype, int d_dtype, bool outputs, int group_size, int mode,
                              const QuantArgs &args, int world, hipStream_t stream);
-hipError_t launch_dequant_reduce(int out_dtype, int group_size, int world, bool aligned,
+// Elements one lane owns for that combination (decides the alignment the vector modes need).
+int quant_pack_vec(int x_dtype, int r_dtype, int d_dtype, bool outputs);
+hipError_t launch_dequant_reduce(int out_dtype, int group_size, int world, int mode,
                                  const ReduceArgs &args, hipStream_t stream);
-hipError_t launch_decode(int out_dtype, int group_size, int reduce_op, bool aligned,
+hipError_t launch_decode(int out_dtype, int group_size, int reduce_op, int mode,
                          const DecodeArgs &args, int world, hipStream_t stream);
-hipError_t launch_ef_update(int p_dtype, int t_dtype, int r_dtype, bool aligned, const EfArgs &args,
+hipError_t launch_ef_update(int p_dtype, int t_dtype, int r_dtype, int mode, const EfArgs &args,
                             hipStream_t stream);
 
 }  // namespace lbc

@@ -6,6 +6,9 @@
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
+
+#include <atomic>
 
 #include "launch.h"
 
@@ -30,6 +33,28 @@ bool aligned_to(const void *p, uintptr_t bytes) { return (reinterpret_cast<uintp
 // torch promotion of two of {f32, f16, bf16}
 int promote(int a, int b) { return a == b ? a : LBC_F32; }
 
+// Streaming (non-temporal) access pays off once a call moves far more bytes than
+// the last-level cache holds; below that the producer's lines are still cached and
+// plain vector access is faster.  The threshold is a process-wide tuning knob:
+// LBC_STREAM_MIN_BYTES at first use, or lbc_set_stream_min_bytes().
+std::atomic<int64_t> g_stream_min{-1};
+
+int64_t stream_threshold() {
+    int64_t value = g_stream_min.load(std::memory_order_relaxed);
+    if (value < 0) {
+        const char *env = getenv("LBC_STREAM_MIN_BYTES");
+        value = env != nullptr ? atoll(env) : (int64_t{96} << 20);
+        if (value < 0) value = 0;
+        g_stream_min.store(value, std::memory_order_relaxed);
+    }
+    return value;
+}
+
+int pick_mode(bool aligned, int64_t bytes_moved) {
+    if (!aligned) return 0;
+    return bytes_moved >= stream_threshold() ? 2 : 1;
+}
+
 int finish(hipError_t err, const char *what) {
     if (err == hipSuccess) return LBC_OK;
     if (err == hipErrorNotSupported) return LBC_UNSUPPORTED;
@@ -43,6 +68,12 @@ extern "C" {
 int lbc_abi_version(void) { return LBC_ABI_VERSION; }
 
 const char *lbc_last_error(void) { return g_error; }
+
+int64_t lbc_set_stream_min_bytes(int64_t min_bytes) {
+    const int64_t previous = stream_threshold();
+    g_stream_min.store(min_bytes < 0 ? 0 : min_bytes, std::memory_order_relaxed);
+    return previous;
+}
 
 int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel,
                    int group_size, int8_t *codes, float *scales, void *new_residual, int new_residual_dtype,
@@ -75,11 +106,15 @@ int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residua
     if (r_dtype != LBC_NONE && r_dtype != LBC_F32 && r_dtype != x_dtype) return LBC_UNSUPPORTED;
     if (d_dtype != LBC_F32 && d_dtype != x_dtype) return LBC_UNSUPPORTED;
 
-    const int vec = 16 / dtype_size(x_dtype);
+    const int vec = lbc::quant_pack_vec(x_dtype, r_dtype, d_dtype, wants_outputs);
     bool aligned = aligned_to(x, 16) && aligned_to(codes, vec);
     if (residual) aligned = aligned && aligned_to(residual, 16);
     if (new_residual) aligned = aligned && aligned_to(new_residual, 16);
     if (restored) aligned = aligned && aligned_to(restored, 16);
+    int64_t moved = numel * (dtype_size(x_dtype) + 1);
+    if (residual) moved += numel * dtype_size(r_dtype);
+    if (new_residual) moved += numel * dtype_size(new_residual_dtype);
+    if (restored) moved += numel * dtype_size(d_dtype);
 
     lbc::QuantArgs a{};
     a.x = x;
@@ -91,8 +126,8 @@ int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residua
     a.numel = numel;
     a.shard_numel = numel;
     a.payload_stride = 0;
-    return finish(lbc::launch_quant_pack(x_dtype, r_dtype, d_dtype, group_size, aligned, a, 1,
-                                         static_cast<hipStream_t>(stream)),
+    return finish(lbc::launch_quant_pack(x_dtype, r_dtype, d_dtype, wants_outputs, group_size,
+                                         pick_mode(aligned, moved), a, 1, static_cast<hipStream_t>(stream)),
                   "lbc_quant_pack");
 }
 
@@ -113,7 +148,7 @@ int lbc_quant_pack_chunks(const void *x, int x_dtype, int64_t numel, int world, 
     if (!aligned_to(payloads, 4)) return fail(LBC_EINVAL, "payloads must be 4-byte aligned");
     if (!aligned_to(x, dtype_size(x_dtype))) return fail(LBC_EINVAL, "input is not aligned to its element size");
 
-    const int vec = 16 / dtype_size(x_dtype);
+    const int vec = lbc::quant_pack_vec(x_dtype, LBC_NONE, LBC_F32, false);
     const bool aligned = aligned_to(x, 16) && (shard * dtype_size(x_dtype)) % 16 == 0 && aligned_to(payloads, vec) &&
                          payload_stride % vec == 0;
     lbc::QuantArgs a{};
@@ -123,7 +158,8 @@ int lbc_quant_pack_chunks(const void *x, int x_dtype, int64_t numel, int world, 
     a.numel = numel;
     a.shard_numel = shard;
     a.payload_stride = payload_stride;
-    return finish(lbc::launch_quant_pack(x_dtype, LBC_NONE, LBC_F32, group_size, aligned, a, world,
+    return finish(lbc::launch_quant_pack(x_dtype, LBC_NONE, LBC_F32, false, group_size,
+                                         pick_mode(aligned, numel * (dtype_size(x_dtype) + 1)), a, world,
                                          static_cast<hipStream_t>(stream)),
                   "lbc_quant_pack_chunks");
 }
@@ -149,7 +185,8 @@ int lbc_dequant(const int8_t *codes, const float *scales, int64_t numel, int gro
     a.shard_numel = numel;
     a.total_numel = numel;
     a.payload_stride = 0;
-    return finish(lbc::launch_decode(out_dtype, group_size, reduce_op, aligned, a, 1, static_cast<hipStream_t>(stream)),
+    return finish(lbc::launch_decode(out_dtype, group_size, reduce_op, pick_mode(aligned, numel * (dtype_size(out_dtype) + 1)),
+                                     a, 1, static_cast<hipStream_t>(stream)),
                   "lbc_dequant");
 }
 
@@ -179,7 +216,8 @@ int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int worl
     a.shard_numel = shard_numel;
     a.total_numel = total_numel;
     a.payload_stride = payload_stride;
-    return finish(lbc::launch_decode(out_dtype, group_size, LBC_REDUCE_NONE, aligned, a, world,
+    return finish(lbc::launch_decode(out_dtype, group_size, LBC_REDUCE_NONE,
+                                     pick_mode(aligned, total_numel * (dtype_size(out_dtype) + 1)), a, world,
                                      static_cast<hipStream_t>(stream)),
                   "lbc_dequant_chunks");
 }
@@ -218,7 +256,10 @@ int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, i
     a.new_residual = new_residual;
     a.numel = numel;
     a.divisor = divisor;
-    return finish(lbc::launch_dequant_reduce(out_dtype, group_size, world, aligned, a, static_cast<hipStream_t>(stream)),
+    int64_t moved = numel * (world + dtype_size(out_dtype));
+    if (prepared != nullptr) moved += 2 * numel * dtype_size(out_dtype);
+    return finish(lbc::launch_dequant_reduce(out_dtype, group_size, world, pick_mode(aligned, moved), a,
+                                             static_cast<hipStream_t>(stream)),
                   "lbc_dequant_reduce");
 }
 
@@ -235,7 +276,8 @@ int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored
         return fail(LBC_EINVAL, "a tensor is not aligned to its element size");
     const bool aligned = aligned_to(prepared, 16) && aligned_to(restored, 16) && aligned_to(residual, 16);
     lbc::EfArgs a{prepared, restored, residual, numel};
-    return finish(lbc::launch_ef_update(prepared_dtype, restored_dtype, residual_dtype, aligned, a,
+    const int64_t moved = numel * (dtype_size(prepared_dtype) + dtype_size(restored_dtype) + dtype_size(residual_dtype));
+    return finish(lbc::launch_ef_update(prepared_dtype, restored_dtype, residual_dtype, pick_mode(aligned, moved), a,
                                         static_cast<hipStream_t>(stream)),
                   "lbc_ef_update");
 }

@@ -24,6 +24,7 @@ _c_int = ctypes.c_int
 SIGNATURES = {
     "lbc_abi_version": (_c_int, []),
     "lbc_last_error": (ctypes.c_char_p, []),
+    "lbc_set_stream_min_bytes": (_c_i64, [_c_i64]),
     "lbc_quant_pack": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_ptr, _c_ptr,
                                 _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr]),
     "lbc_quant_pack_chunks": (_c_int, [_c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_ptr, _c_i64, _c_ptr]),

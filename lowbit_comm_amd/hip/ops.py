@@ -90,6 +90,33 @@ class _Launch:
         return False
 
 
+class BoundLaunch:
+    """One ABI call with every argument validated and marshalled ahead of time.
+
+    Calling it enqueues the kernel on torch's current stream of the tensors' device and returns
+    ``True``/``False`` like the ``*_into`` function it was made from.  The bound tensors are kept
+    alive by the object; their addresses must not change (no resize, no reallocation).  This is
+    the per-bucket fast path: a DDP hook binds once per bucket shape and replays every step.
+    """
+
+    __slots__ = ("_fn", "_args", "_device", "_lib", "_keep")
+
+    def __init__(self, fn, args: tuple, device: torch.device, lib, keep: tuple) -> None:
+        self._fn = fn
+        self._args = args
+        self._device = device
+        self._lib = lib
+        self._keep = keep
+
+    def __call__(self) -> bool:
+        if self._device.index not in (None, torch.cuda.current_device()):
+            with _Launch(self._device) as stream:
+                return _finish(self._fn(*self._args, stream), self._lib)
+        stream = torch.cuda.current_stream(self._device).cuda_stream
+        rc = self._fn(*self._args, stream)
+        return True if rc == LBC_OK else _finish(rc, self._lib)
+
+
 def _finish(rc: int, lib) -> bool:
     if rc == LBC_OK:
         return True
@@ -105,6 +132,14 @@ def quant_pack_into(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, 
                     residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
                     restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None) -> bool:
     """``codes, scales <- quant(x + residual)``; optionally ``restored`` and ``new_residual = p - restored``."""
+    return bind_quant_pack(x, codes, scales, group_size=group_size, residual=residual, new_residual=new_residual,
+                           restored=restored, restored_dtype=restored_dtype)()
+
+
+def bind_quant_pack(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, *, group_size: int = 64,
+                    residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
+                    restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None) -> BoundLaunch:
+    """Validate once; the returned :class:`BoundLaunch` replays :func:`quant_pack_into` on the same tensors."""
     lib = load_library()
     x_code = _float_tensor(x, "input")
     device = x.device
@@ -133,10 +168,9 @@ def quant_pack_into(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, 
         _require(new_residual.numel() == n, "input and new_residual must have the same number of elements")
         _require(new_residual.dtype == promote(p_dtype, d_dtype),
                  f"new_residual must have dtype {promote(p_dtype, d_dtype)}")
-    with _Launch(device) as stream:
-        rc = lib.lbc_quant_pack(_ptr(x), x_code, _ptr(residual), r_code, n, group_size, _ptr(codes), _ptr(scales),
-                                _ptr(new_residual), n_code, _ptr(restored), d_code, stream)
-    return _finish(rc, lib)
+    args = (_ptr(x), x_code, _ptr(residual), r_code, n, group_size, _ptr(codes), _ptr(scales),
+            _ptr(new_residual), n_code, _ptr(restored), d_code)
+    return BoundLaunch(lib.lbc_quant_pack, args, device, lib, (x, codes, scales, residual, new_residual, restored))
 
 
 def quant_pack_payload_into(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64, **kwargs) -> bool:
@@ -157,6 +191,10 @@ def quant_pack(x: torch.Tensor, *, group_size: int = 64, residual: torch.Tensor 
 
 def quant_pack_chunks_into(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64) -> bool:
     """Quantize the ``world`` destination chunks of ``x`` into the rows of ``payloads`` (uint8 [world, stride])."""
+    return bind_quant_pack_chunks(x, payloads, world, group_size=group_size)()
+
+
+def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64) -> BoundLaunch:
     lib = load_library()
     x_code = _float_tensor(x, "input")
     _device_tensor(payloads, "payloads", x.device)
@@ -164,10 +202,8 @@ def quant_pack_chunks_into(x: torch.Tensor, payloads: torch.Tensor, world: int, 
     _require(payloads.shape[0] == world, "payloads must have one row per destination rank")
     shard = -(-x.numel() // world)
     _require(payloads.shape[1] >= payload_nbytes(shard, group_size), "payload rows are too small")
-    with _Launch(x.device) as stream:
-        rc = lib.lbc_quant_pack_chunks(_ptr(x), x_code, x.numel(), world, group_size, _ptr(payloads),
-                                       payloads.stride(0), stream)
-    return _finish(rc, lib)
+    args = (_ptr(x), x_code, x.numel(), world, group_size, _ptr(payloads), payloads.stride(0))
+    return BoundLaunch(lib.lbc_quant_pack_chunks, args, x.device, lib, (x, payloads))
 
 
 # --------------------------------------------------------------------------- #
@@ -176,6 +212,11 @@ def quant_pack_chunks_into(x: torch.Tensor, payloads: torch.Tensor, world: int, 
 def dequant_into(codes: torch.Tensor, scales: torch.Tensor, out: torch.Tensor, *, numel: int | None = None,
                  group_size: int = 64, reduce_op: str = "none") -> bool:
     """``out[:numel] (op)= float(code) * scale``."""
+    return bind_dequant(codes, scales, out, numel=numel, group_size=group_size, reduce_op=reduce_op)()
+
+
+def bind_dequant(codes: torch.Tensor, scales: torch.Tensor, out: torch.Tensor, *, numel: int | None = None,
+                 group_size: int = 64, reduce_op: str = "none") -> BoundLaunch:
     lib = load_library()
     o_code = _float_tensor(out, "output")
     device = out.device
@@ -189,9 +230,8 @@ def dequant_into(codes: torch.Tensor, scales: torch.Tensor, out: torch.Tensor, *
     _require(codes.numel() >= groups * group_size, "codes is smaller than the padded element count")
     _require(scales.numel() >= groups, "scales is smaller than the group count")
     _require(reduce_op in REDUCE_OPS, f"unsupported reduce op {reduce_op!r}")
-    with _Launch(device) as stream:
-        rc = lib.lbc_dequant(_ptr(codes), _ptr(scales), n, group_size, _ptr(out), o_code, REDUCE_OPS[reduce_op], stream)
-    return _finish(rc, lib)
+    args = (_ptr(codes), _ptr(scales), n, group_size, _ptr(out), o_code, REDUCE_OPS[reduce_op])
+    return BoundLaunch(lib.lbc_dequant, args, device, lib, (codes, scales, out))
 
 
 def dequant(codes: torch.Tensor, scales: torch.Tensor, numel: int, *, group_size: int = 64,
@@ -204,6 +244,10 @@ def dequant(codes: torch.Tensor, scales: torch.Tensor, numel: int, *, group_size
 
 def dequant_chunks_into(payloads: torch.Tensor, out: torch.Tensor, shard_numel: int, *, group_size: int = 64) -> bool:
     """Decode row ``d`` of ``payloads`` into ``out[d*shard : (d+1)*shard]`` (clipped to ``out.numel()``)."""
+    return bind_dequant_chunks(payloads, out, shard_numel, group_size=group_size)()
+
+
+def bind_dequant_chunks(payloads: torch.Tensor, out: torch.Tensor, shard_numel: int, *, group_size: int = 64) -> BoundLaunch:
     lib = load_library()
     o_code = _float_tensor(out, "output")
     _device_tensor(payloads, "payloads", out.device)
@@ -211,10 +255,8 @@ def dequant_chunks_into(payloads: torch.Tensor, out: torch.Tensor, shard_numel: 
     world = payloads.shape[0]
     _require(payloads.shape[1] >= payload_nbytes(shard_numel, group_size), "payload rows are too small")
     _require(out.numel() <= world * shard_numel, "output is larger than world * shard_numel")
-    with _Launch(out.device) as stream:
-        rc = lib.lbc_dequant_chunks(_ptr(payloads), payloads.stride(0), world, shard_numel, out.numel(), group_size,
-                                    _ptr(out), o_code, stream)
-    return _finish(rc, lib)
+    args = (_ptr(payloads), payloads.stride(0), world, shard_numel, out.numel(), group_size, _ptr(out), o_code)
+    return BoundLaunch(lib.lbc_dequant_chunks, args, out.device, lib, (payloads, out))
 
 
 def dequant_reduce_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out: torch.Tensor, *,
@@ -224,6 +266,16 @@ def dequant_reduce_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], o
 
     ``payloads`` is a sequence of ``(codes, scales)`` pairs.  More than 8 payloads returns ``False``.
     """
+    bound = bind_dequant_reduce(payloads, out, numel=numel, group_size=group_size, divisor=divisor,
+                                prepared=prepared, new_residual=new_residual)
+    return False if bound is None else bound()
+
+
+def bind_dequant_reduce(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out: torch.Tensor, *,
+                        numel: int | None = None, group_size: int = 64, divisor: float = 1.0,
+                        prepared: torch.Tensor | None = None,
+                        new_residual: torch.Tensor | None = None) -> BoundLaunch | None:
+    """Bound form of :func:`dequant_reduce_into`; ``None`` when there are more than 8 payloads."""
     lib = load_library()
     _require(len(payloads) > 0, "inputs must not be empty")
     _require(divisor > 0, "divisor must be > 0")
@@ -232,7 +284,7 @@ def dequant_reduce_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], o
     n = out.numel() if numel is None else int(numel)
     _require(0 <= n <= out.numel(), "numel exceeds the output size")
     if len(payloads) > MAX_PAYLOADS:
-        return False
+        return None
     groups = num_groups(n, group_size)
     world = len(payloads)
     code_ptrs = (ctypes.c_void_p * world)()
@@ -254,10 +306,10 @@ def dequant_reduce_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], o
         _require(new_residual.dtype == out.dtype, "prepared and residual must have the same dtype")
         _require(prepared.numel() == n, "prepared must have numel elements")
         _require(new_residual.numel() == n, "prepared and residual must have the same number of elements")
-    with _Launch(device) as stream:
-        rc = lib.lbc_dequant_reduce(code_ptrs, scale_ptrs, world, n, group_size, float(divisor), _ptr(out), o_code,
-                                    _ptr(prepared), _ptr(new_residual), stream)
-    return _finish(rc, lib)
+    args = (code_ptrs, scale_ptrs, world, n, group_size, float(divisor), _ptr(out), o_code,
+            _ptr(prepared), _ptr(new_residual))
+    keep = (tuple(payloads), out, prepared, new_residual)
+    return BoundLaunch(lib.lbc_dequant_reduce, args, device, lib, keep)
 
 
 def ef_update_into(prepared: torch.Tensor, restored: torch.Tensor, residual: torch.Tensor) -> bool:
@@ -268,7 +320,5 @@ def ef_update_into(prepared: torch.Tensor, restored: torch.Tensor, residual: tor
     r_code = _float_tensor(residual, "residual", prepared.device)
     _require(prepared.numel() == restored.numel(), "prepared and restored must have the same number of elements")
     _require(prepared.numel() == residual.numel(), "prepared and residual must have the same number of elements")
-    with _Launch(prepared.device) as stream:
-        rc = lib.lbc_ef_update(_ptr(prepared), p_code, _ptr(restored), t_code, _ptr(residual), r_code,
-                               prepared.numel(), stream)
-    return _finish(rc, lib)
+    args = (_ptr(prepared), p_code, _ptr(restored), t_code, _ptr(residual), r_code, prepared.numel())
+    return BoundLaunch(lib.lbc_ef_update, args, prepared.device, lib, (prepared, restored, residual))()

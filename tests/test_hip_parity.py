@@ -15,11 +15,18 @@ pytestmark = pytest.mark.gpu
 DTYPES = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
 
 
-@pytest.fixture(scope="module")
-def ops(hip_device):
+@pytest.fixture(scope="module", params=["vector", "stream", "default"])
+def ops(request, hip_device):
+    """The tensor-level ops with the bulk access mode forced to plain vector, to non-temporal, or left to
+    the size threshold - results must not depend on it."""
     from lowbit_comm_amd.hip import ops as hip_ops
+    from lowbit_comm_amd.hip.library import load_library
 
-    return hip_ops
+    lib = load_library()
+    wanted = {"vector": 1 << 62, "stream": 0, "default": 96 << 20}[request.param]
+    previous = lib.lbc_set_stream_min_bytes(wanted)
+    yield hip_ops
+    lib.lbc_set_stream_min_bytes(previous)
 
 
 def gradient_like(n, dtype, seed, device, sigma=1e-3, outliers=True):
