@@ -33,7 +33,7 @@ WORLD = 8
 GROUP = 64
 SEED = 1234
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), or None
-MEASURED_TRAFFIC = {"quant_pack_chunks": None}
+MEASURED_TRAFFIC = {"quant_pack_chunks": 132_750_000}
 
 
 def parse_args():
