@@ -1,0 +1,283 @@
+"""PyTorch DDP communication hook over the compressed bucket path.
+
+``create_ddp_comm_hook`` keeps the keyword surface of the reference's
+``ccdl_comm/communication/ddp_hook.py:48-81`` so call sites port unchanged.  What runs here is the
+compute of that hook - error-feedback compensate, quantize+pack, fused dequant-reduce, residual
+update - on HIP kernels; the collectives themselves are *injected* (``all_gather=``, ``all_reduce=``,
+``reduce_scatter_all_gather=`` ...).  This build ships no collective transport of its own: a
+strategy whose transport is not injected raises :class:`UnsupportedCollective`, as do the
+asynchronous gather pipelines.
+"""
+from __future__ import annotations
+
+from collections.abc import Callable
+from typing import Any
+
+from lowbit_comm_amd.communication.collectives import CompressedPayload
+from lowbit_comm_amd.communication.ddp import DDPBucketProcessor
+from lowbit_comm_amd.communication.gather_reduce import CompressedAllGatherReduce, GatheredPayloads
+from lowbit_comm_amd.communication.payload_packing import (
+    DEFAULT_FUSED_PAYLOAD_MIN_NUMEL,
+    make_fused_payload_all_gather,
+    should_fuse_payload,
+)
+from lowbit_comm_amd.communication.workspace import DequantizedWorkspaceCache
+from lowbit_comm_amd.config import CompressionConfig
+from lowbit_comm_amd.exceptions import UnsupportedCollective
+from lowbit_comm_amd.quantization.codec import (
+    allocate_dequantized_buffer,
+    dequantize_reduce_tensors,
+    dequantize_tensor,
+    inplace_dequantize_reduce_mean_update_error_feedback,
+    quantize_tensor,
+)
+from lowbit_comm_amd.quantization.error_feedback import ErrorFeedbackState
+from lowbit_comm_amd.quantization.error_feedback_policy import ErrorFeedbackPolicy
+
+STRATEGIES = ("auto", "all_gather", "all_reduce", "reduce_scatter", "hierarchical", "topology")
+
+
+def _torch_future() -> Any:
+    import torch
+
+    return torch.futures.Future()
+
+
+def resolve_dtype(dtype: str, tensor: Any) -> str:
+    """``"auto"`` -> ``fp16`` / ``bf16`` / ``fp32`` from the bucket tensor's dtype."""
+    if dtype != "auto":
+        return dtype
+    text = str(getattr(tensor, "dtype", ""))
+    if "bfloat16" in text:
+        return "bf16"
+    if "float16" in text or text.endswith("half"):
+        return "fp16"
+    if "float32" in text or text.endswith("float"):
+        return "fp32"
+    raise ValueError(f"cannot infer CCDL dtype from bucket tensor dtype: {text!r}")
+
+
+def coerce_payload(value: Any, *, shape: tuple[int, ...], dtype: str) -> CompressedPayload:
+    """Accept a :class:`CompressedPayload`, a ``{"buffer": ...}`` dict or a bare buffer from a quantizer."""
+    if isinstance(value, CompressedPayload):
+        return value
+    if isinstance(value, dict) and "buffer" in value:
+        return CompressedPayload(buffer=value["buffer"], shape=tuple(value.get("shape", shape)),
+                                 dtype=str(value.get("dtype", dtype)), metadata=dict(value.get("metadata", {})))
+    return CompressedPayload(buffer=value, shape=shape, dtype=dtype)
+
+
+def _buffer_of(payload: Any) -> Any:
+    return payload.buffer if hasattr(payload, "buffer") else payload
+
+
+def _numel(tensor: Any) -> int:
+    count = getattr(tensor, "numel", None)
+    if callable(count):
+        return int(count())
+    total = 1
+    for dim in getattr(tensor, "shape", ()):
+        total *= int(dim)
+    return total
+
+
+def _single_process_all_reduce(tensor: Any, reduce: str) -> Any:
+    """Bypass for uncompressed small buckets when no ``bypass_all_reduce`` is injected: the identity,
+    which is the all-reduce of a one-rank world.  With an initialised process group the caller must
+    inject the collective."""
+    try:
+        import torch.distributed as dist
+
+        if dist.is_available() and dist.is_initialized() and dist.get_world_size() > 1:
+            raise UnsupportedCollective("all_reduce", reason="inject bypass_all_reduce= for uncompressed buckets; "
+                                                             "this build ships no collective transport")
+    except ImportError:
+        pass
+    del reduce
+    return tensor
+
+
+def _annotate(hook: Callable[[Any, Any], Any], provider: Callable[[], dict[str, Any]] | None) -> None:
+    def default() -> dict[str, Any]:
+        import torch
+        import torch.distributed as dist
+
+        return {"state": object, "bucket": dist.GradBucket, "return": torch.futures.Future[torch.Tensor]}
+
+    try:
+        hook.__annotations__ = (provider or default)()
+    except (ImportError, ModuleNotFoundError, AttributeError):
+        pass
+
+
+def create_ddp_comm_hook(
+    config: CompressionConfig,
+    *,
+    dtype: str = "auto",
+    strategy: str = "all_reduce",
+    reduce: str = "mean",
+    quantize: Callable[[Any, CompressionConfig], Any] | None = None,
+    dequantize: Callable[[Any, tuple[int, ...], CompressionConfig, str], Any] | None = None,
+    all_reduce: Callable[[CompressedPayload, str], CompressedPayload] | None = None,
+    all_gather: Callable[[Any], GatheredPayloads] | None = None,
+    async_gather: bool = False,
+    async_error_feedback: bool = False,
+    synchronize_async_feedback_completion: bool = True,
+    async_all_gather: Callable[[Any], Any] | None = None,
+    native_error_feedback_update: Callable[[Any, Any, Any], Any] | None = None,
+    native_dequantize_reduce_update_feedback: Callable[..., Any] | None = None,
+    native_inplace_dequantize_reduce_update_feedback: Callable[..., bool] | None = None,
+    reduce_scatter_all_gather: Callable[..., Any] | None = None,
+    hierarchical_all_reduce: Callable[..., Any] | None = None,
+    topology_all_reduce: Callable[..., Any] | None = None,
+    topology_method: str | None = None,
+    allocate_dequantized_workspace: Callable[[Any, tuple[int, ...], CompressionConfig], Any] | None = None,
+    workspace_cache_max_entries: int | None = 1,
+    workspace_cache_max_bytes: int | None = None,
+    completion_manager: Any | None = None,
+    fuse_payload: bool = False,
+    fuse_payload_min_numel: int = DEFAULT_FUSED_PAYLOAD_MIN_NUMEL,
+    min_compress_numel: int = 0,
+    bypass_all_reduce: Callable[[Any, str], Any] | None = None,
+    error_feedback: ErrorFeedbackState | None = None,
+    extension_status: Any | None = None,
+    future_factory: Callable[[], Any] = _torch_future,
+    annotation_provider: Callable[[], dict[str, Any]] | None = None,
+) -> Callable[[Any, Any], Any]:
+    """Build ``hook(state, bucket) -> Future`` for ``DistributedDataParallel.register_comm_hook``."""
+    del async_error_feedback, synchronize_async_feedback_completion, async_all_gather, completion_manager
+    del native_dequantize_reduce_update_feedback, topology_method
+    requested = strategy.strip().lower()
+    if requested not in STRATEGIES:
+        raise UnsupportedCollective(strategy, reason="explicit strategy is unknown and no fallback was declared")
+    if async_gather:
+        raise UnsupportedCollective("async_gather", reason="asynchronous gather pipelines are not part of this build")
+    injected = {"reduce_scatter": reduce_scatter_all_gather, "hierarchical": hierarchical_all_reduce,
+                "topology": topology_all_reduce}
+    if requested in injected and injected[requested] is None:
+        raise UnsupportedCollective(requested, reason=f"{requested} transport unavailable for explicit strategy")
+    effective = requested
+    if requested == "auto":
+        effective = "reduce_scatter" if reduce_scatter_all_gather is not None else "all_gather"
+
+    def active_quantize(tensor: Any, active: CompressionConfig) -> Any:
+        if quantize is not None:
+            return quantize(tensor, active)
+        return quantize_tensor(tensor, active, extension_status=extension_status)
+
+    def active_dequantize(payload: Any, shape: tuple[int, ...], active: CompressionConfig, active_dtype: str) -> Any:
+        if dequantize is not None:
+            return dequantize(payload, shape, active, active_dtype)
+        return dequantize_tensor(_buffer_of(payload), shape, active, dtype=active_dtype,
+                                 extension_status=extension_status)
+
+    feedback = error_feedback or ErrorFeedbackState()
+    policy = ErrorFeedbackPolicy(config)
+    uncompressed = bypass_all_reduce or _single_process_all_reduce
+    inplace_reduce_feedback = (native_inplace_dequantize_reduce_update_feedback
+                               or inplace_dequantize_reduce_mean_update_error_feedback)
+    workspaces = DequantizedWorkspaceCache(
+        allocator=allocate_dequantized_workspace or allocate_dequantized_buffer,
+        max_entries=workspace_cache_max_entries, max_cached_bytes=workspace_cache_max_bytes)
+
+    def small(tensor: Any) -> bool:
+        return min_compress_numel > 0 and _numel(tensor) < min_compress_numel
+
+    def clone(tensor: Any) -> Any:
+        return tensor.clone() if callable(getattr(tensor, "clone", None)) else tensor
+
+    if effective in injected:
+        transport = injected[effective]
+
+        def process_bucket(bucket: Any) -> Any:
+            tensor = bucket.buffer()
+            if small(tensor):
+                return uncompressed(clone(tensor), reduce)
+            return transport(tensor, config=config, op=reduce, async_op=False, dtype=resolve_dtype(dtype, tensor),
+                             extension_status=extension_status)
+
+    elif effective == "all_gather":
+        if all_gather is None:
+            raise UnsupportedCollective("all_gather", reason="inject all_gather=; this build ships no collective transport")
+        plain_gather = all_gather
+        packed_gather = all_gather
+
+        def process_bucket(bucket: Any) -> Any:
+            key = bucket.index() if callable(getattr(bucket, "index", None)) else id(bucket)
+            original = bucket.buffer()
+            if small(original):
+                return uncompressed(clone(original), reduce)
+            decision = policy.decide(key, numel=_numel(original))
+            prepared = feedback.compensate(key, original) if decision.apply else original
+            active_dtype = resolve_dtype(dtype, prepared)
+            shape = tuple(prepared.shape)
+            gather = (packed_gather if should_fuse_payload(prepared, enabled=fuse_payload,
+                                                           min_numel=fuse_payload_min_numel) else plain_gather)
+            if dequantize is None and reduce in ("mean", "sum"):
+                # facade path: flat uint8 buffers, fused decode+reduce (+ residual update) on the GPU
+                local = coerce_payload(active_quantize(prepared, config), shape=shape, dtype=active_dtype)
+                buffers = [_buffer_of(p) for p in gather(local).payloads]
+                restored = None
+                residual = feedback.get(key) if decision.update else None
+                if residual is not None and getattr(residual, "dtype", None) == getattr(prepared, "dtype", None):
+                    workspace = workspaces.get(key, prepared, shape, config)
+                    try:
+                        if inplace_reduce_feedback(buffers, prepared, workspace, residual, config,
+                                                   extension_status=extension_status, reduce=reduce):
+                            restored = workspace.reshape(-1)[:_numel(prepared)].reshape(shape)
+                    except RuntimeError:
+                        restored = None
+                if restored is None:
+                    restored = dequantize_reduce_tensors(buffers, shape, config, dtype=active_dtype,
+                                                         extension_status=extension_status, reduce=reduce)
+                    if decision.update:
+                        latest = feedback.get(key)
+                        if native_error_feedback_update is not None and latest is not None:
+                            native_error_feedback_update(prepared, restored, latest)
+                        else:
+                            feedback.update(key, original=prepared, transmitted=restored)
+                policy.advance(key)
+                return restored
+            collective = CompressedAllGatherReduce(
+                config=config,
+                compress=lambda tensor, active: coerce_payload(active_quantize(tensor, active),
+                                                               shape=tuple(tensor.shape), dtype=active_dtype),
+                all_gather=gather,
+                decompress=active_dequantize,
+            )
+            restored = collective.run(prepared, shape=shape, dtype=active_dtype, reduce=reduce)
+            if decision.update:
+                feedback.update(key, original=prepared, transmitted=restored)
+            policy.advance(key)
+            return restored
+
+    else:  # all_reduce
+        if all_reduce is None:
+            raise UnsupportedCollective("all_reduce", reason="inject all_reduce=; this build ships no collective transport")
+        processor = DDPBucketProcessor(config=config, quantize=active_quantize, dequantize=active_dequantize,
+                                       all_reduce=all_reduce, error_feedback=feedback)
+
+        def process_bucket(bucket: Any) -> Any:
+            tensor = bucket.buffer()
+            if small(tensor):
+                return uncompressed(clone(tensor), reduce)
+            return processor.process(bucket, dtype=resolve_dtype(dtype, tensor))
+
+    def hook(state: Any, bucket: Any) -> Any:
+        del state
+        result = process_bucket(bucket)
+        if hasattr(result, "set_result"):
+            return result
+        future = future_factory()
+        future.set_result(result)
+        return future
+
+    hook._ccdl_requested_strategy = requested
+    hook._ccdl_effective_strategy = effective
+    _annotate(hook, annotation_provider)
+    return hook
+
+
+def make_fused_all_gather(byte_all_gather: Callable[[Any], GatheredPayloads]):
+    """Convenience re-export: wrap a byte all-gather so payloads travel packed (one collective per bucket)."""
+    return make_fused_payload_all_gather(byte_all_gather)

@@ -1,0 +1,164 @@
+"""Small LRU caches for decode and shard workspaces keyed by bucket
+(behaviour of ``ccdl_comm/communication/workspace.py:35-196``).  They hand back the *same* tensor for
+the same key and layout so steady-state steps allocate nothing and addresses stay stable; a layout
+change under a key replaces the entry.  Budgets: number of entries and estimated bytes, oldest first.
+"""
+from __future__ import annotations
+
+from collections import OrderedDict
+from math import prod
+from typing import Any, Callable
+
+from lowbit_comm_amd.config import CompressionConfig
+
+_DTYPE_BYTES = {"float64": 8, "double": 8, "int64": 8, "float32": 4, "float": 4, "int32": 4,
+                "float16": 2, "half": 2, "fp16": 2, "bfloat16": 2, "bf16": 2, "int16": 2}
+
+
+def _bytes_per_element(dtype: Any) -> int:
+    return _DTYPE_BYTES.get(str(dtype).lower().removeprefix("torch."), 1)
+
+
+def _tensor_bytes(tensor: Any) -> int:
+    nbytes = getattr(tensor, "nbytes", None)
+    if nbytes is not None:
+        return int(nbytes)
+    numel, size = getattr(tensor, "numel", None), getattr(tensor, "element_size", None)
+    if callable(numel) and callable(size):
+        return int(numel()) * int(size())
+    shape = tuple(getattr(tensor, "shape", ()))
+    return prod(shape) * _bytes_per_element(getattr(tensor, "dtype", "")) if shape else 0
+
+
+def _signature(tensor: Any) -> tuple:
+    return (tuple(getattr(tensor, "shape", ())), str(getattr(tensor, "dtype", "")), str(getattr(tensor, "device", "")))
+
+
+def _policy_signature(config: CompressionConfig) -> tuple:
+    return (config.bit, config.group_size, config.topk, config.quant_type, config.stochastic, config.compact)
+
+
+class _LruStore:
+    """``key -> (layout, tensor, bytes)`` with entry and byte budgets."""
+
+    def __init__(self, max_entries: int | None, max_cached_bytes: int | None) -> None:
+        if max_entries is not None and max_entries < 1:
+            raise ValueError("max_entries must be >= 1 or None")
+        if max_cached_bytes is not None and max_cached_bytes < 0:
+            raise ValueError("max_cached_bytes must be >= 0 or None")
+        self.max_entries = max_entries
+        self.max_cached_bytes = max_cached_bytes
+        self.items: OrderedDict[Any, tuple[Any, Any, int]] = OrderedDict()
+        self.cached_bytes = 0
+
+    def lookup(self, key: Any, layout: Any) -> Any | None:
+        entry = self.items.get(key)
+        if entry is None or entry[0] != layout:
+            return None
+        self.items.move_to_end(key)
+        return entry[1]
+
+    def insert(self, key: Any, layout: Any, tensor: Any, nbytes: int) -> None:
+        old = self.items.pop(key, None)
+        if old is not None:
+            self.cached_bytes -= old[2]
+        self.items[key] = (layout, tensor, nbytes)
+        self.cached_bytes += nbytes
+        while self.items and (
+                (self.max_entries is not None and len(self.items) > self.max_entries)
+                or (self.max_cached_bytes is not None and self.cached_bytes > self.max_cached_bytes)):
+            _key, (_layout, _tensor, dropped) = self.items.popitem(last=False)
+            self.cached_bytes -= dropped
+
+    def clear(self) -> None:
+        self.items.clear()
+        self.cached_bytes = 0
+
+
+def _default_decode_allocator(tensor: Any, shape: tuple[int, ...], config: CompressionConfig) -> Any:
+    from lowbit_comm_amd.quantization.codec import allocate_dequantized_buffer
+
+    return allocate_dequantized_buffer(tensor, shape, config)
+
+
+class DequantizedWorkspaceCache:
+    """Per-hook cache of decode workspaces, one per bucket key."""
+
+    def __init__(self, *, allocator: Callable[[Any, tuple[int, ...], CompressionConfig], Any] | None = None,
+                 max_entries: int | None = None, max_cached_bytes: int | None = None) -> None:
+        self._allocator = allocator or _default_decode_allocator
+        self._store = _LruStore(max_entries, max_cached_bytes)
+
+    def get(self, key: Any, tensor: Any, shape: tuple[int, ...], config: CompressionConfig) -> Any:
+        g = config.group_size
+        numel = prod(shape) if shape else 0
+        padded = -(-numel // g) * g if numel else 0
+        dtype = str(getattr(tensor, "dtype", ""))
+        layout = (tuple(shape), dtype, str(getattr(tensor, "device", "")), padded)
+        found = self._store.lookup(key, layout)
+        if found is not None:
+            return found
+        workspace = self._allocator(tensor, shape, config)
+        self._store.insert(key, layout, workspace, padded * _bytes_per_element(dtype))
+        return workspace
+
+    def clear(self) -> None:
+        self._store.clear()
+
+    @property
+    def cached_bytes(self) -> int:
+        return self._store.cached_bytes
+
+    def __len__(self) -> int:
+        return len(self._store.items)
+
+
+def _default_quantized_allocator(tensor: Any, config: CompressionConfig, dtype: str) -> Any:
+    from lowbit_comm_amd.quantization.codec import allocate_quantized_buffer
+
+    return allocate_quantized_buffer(tensor, config, dtype=dtype)
+
+
+class ShardCommunicationWorkspaceCache:
+    """Send (quantized chunk), receive (peer payload) and reduced-shard workspaces of a shard collective."""
+
+    def __init__(self, *, quantized_allocator: Callable[[Any, CompressionConfig, str], Any] | None = None,
+                 reduced_allocator: Callable[[Any, tuple[int, ...], CompressionConfig], Any] | None = None,
+                 max_entries: int | None = None, max_cached_bytes: int | None = None) -> None:
+        self._quantized_allocator = quantized_allocator or _default_quantized_allocator
+        self._reduced_allocator = reduced_allocator or _default_decode_allocator
+        self._store = _LruStore(max_entries, max_cached_bytes)
+
+    def _get(self, key: tuple, allocate: Callable[[], Any]) -> Any:
+        found = self._store.lookup(key, None)
+        if found is not None:
+            return found
+        workspace = allocate()
+        self._store.insert(key, None, workspace, _tensor_bytes(workspace))
+        return workspace
+
+    def get_quantized_chunk(self, bucket_key: Any, chunk_index: int, tensor: Any, config: CompressionConfig, *,
+                            dtype: str, world_size: int) -> Any:
+        key = ("send", bucket_key, chunk_index, world_size, _signature(tensor), _policy_signature(config), dtype)
+        return self._get(key, lambda: self._quantized_allocator(tensor, config, dtype))
+
+    def get_received_payload(self, bucket_key: Any, payload_template: Any, index: int, *, world_size: int,
+                             config: CompressionConfig) -> Any:
+        key = ("recv", bucket_key, index, world_size, _signature(payload_template), _policy_signature(config))
+        return self._get(key, lambda: payload_template.new_empty(tuple(payload_template.shape)))
+
+    def get_reduced_shard(self, bucket_key: Any, tensor: Any, shape: tuple[int, ...], config: CompressionConfig, *,
+                          dtype: str, world_size: int, rank: int) -> Any:
+        key = ("reduced", bucket_key, rank, world_size, tuple(shape), _signature(tensor), _policy_signature(config),
+               dtype)
+        return self._get(key, lambda: self._reduced_allocator(tensor, shape, config))
+
+    def clear(self) -> None:
+        self._store.clear()
+
+    @property
+    def cached_bytes(self) -> int:
+        return self._store.cached_bytes
+
+    def __len__(self) -> int:
+        return len(self._store.items)

@@ -1,0 +1,25 @@
+"""HIP (gfx950) backend: C-ABI binding, tensor-level ops, native-module shim, codec callables, workspace pool."""
+from .loader import CudaExtensionStatus, HipExtensionStatus, load_cuda_extension, load_hip_extension
+from .workspace import (
+    CudaOutputLease,
+    CudaShardWorkspaceProvider,
+    CudaShardWorkspaceSession,
+    CudaWorkspacePool,
+    EventCompletion,
+    EventCompletionManager,
+    HipOutputLease,
+    HipWorkspacePool,
+    ShardWorkspaceProvider,
+    ShardWorkspaceSession,
+    WorkspaceKey,
+    WorkspaceLease,
+    WorkspaceStats,
+    create_torch_workspace_pool,
+)
+
+__all__ = [
+    "CudaExtensionStatus", "CudaOutputLease", "CudaShardWorkspaceProvider", "CudaShardWorkspaceSession",
+    "CudaWorkspacePool", "EventCompletion", "EventCompletionManager", "HipExtensionStatus", "HipOutputLease",
+    "HipWorkspacePool", "ShardWorkspaceProvider", "ShardWorkspaceSession", "WorkspaceKey", "WorkspaceLease",
+    "WorkspaceStats", "create_torch_workspace_pool", "load_cuda_extension", "load_hip_extension",
+]

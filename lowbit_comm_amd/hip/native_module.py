@@ -1,0 +1,268 @@
+"""The duck-typed native module the codec facade talks to.
+
+It exposes the names and positional argument orders of the reference's pybind module
+(``ccdl_comm/csrc/pybind.cpp:133-166``; orders from ``ccdl_comm/csrc/quantization/quant_api.cuh:5-17``
+and ``dequant_api.cuh:5-12``) over this package's C ABI.  Buffers are flat ``uint8`` tensors holding
+the portable wire format ``[int8 codes || fp32 scales]`` (68 bytes per group of 64 for every source
+dtype; size them with ``estimate_payload_size``).
+
+Conventions kept from the reference: ``inplace_*`` never allocate and never touch their inputs;
+unsupported *policy* (4-bit, top-k, stochastic, non-linear, more than 8 payloads for the fused calls)
+returns ``False`` so the caller can fall back; contract violations raise ``RuntimeError``; launches go
+to torch's current stream of the tensors' device and do not synchronise.  ``compact`` is accepted
+and ignored: the portable format has a single layout.
+"""
+from __future__ import annotations
+
+import enum
+from typing import Sequence
+
+import torch
+
+from lowbit_comm_amd.hip import ops
+from lowbit_comm_amd.hip.library import load_library
+
+
+class QuantType(enum.IntEnum):
+    Linear = 0
+    Normal = 1
+    Uniform = 2
+    E3M0 = 3
+    E2M1 = 4
+
+
+class DType(enum.IntEnum):
+    FP16 = 1
+    BF16 = 2
+    FP32 = 0
+
+
+class ReduceOP(enum.IntEnum):
+    NONE = 0
+    SUM = 1
+    MAX = 2
+    MIN = 3
+
+
+_TORCH_OF = {DType.FP16: torch.float16, DType.BF16: torch.bfloat16, DType.FP32: torch.float32}
+_OP_NAME = {ReduceOP.NONE: "none", ReduceOP.SUM: "sum", ReduceOP.MAX: "max", ReduceOP.MIN: "min"}
+
+
+def _policy_supported(group_size: int, topk: int, stochastic: bool, bit: int, quant_type) -> bool:
+    return (group_size in (16, 32, 64) and topk == 0 and not stochastic and bit == 8
+            and int(quant_type) == int(QuantType.Linear))
+
+
+def _require_policy(group_size, topk, stochastic, bit, quant_type) -> None:
+    if not _policy_supported(group_size, topk, stochastic, bit, quant_type):
+        raise RuntimeError(
+            "the HIP codec supports linear 8-bit quantization with group_size 16/32/64, topk=0, no stochastic "
+            f"rounding; got group_size={group_size} topk={topk} stochastic={stochastic} bit={bit} "
+            f"quant_type={getattr(quant_type, 'name', quant_type)}")
+
+
+def _check_payload(buffer: torch.Tensor, name: str) -> None:
+    if not isinstance(buffer, torch.Tensor) or buffer.dtype != torch.uint8:
+        raise RuntimeError(f"{name} must be uint8")
+    if not buffer.is_cuda:
+        raise RuntimeError(f"{name} must be a GPU tensor")
+    if not buffer.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _padded_numel_of(buffer: torch.Tensor, group_size: int, name: str = "input") -> int:
+    nbytes = buffer.numel()
+    if nbytes % (group_size + 4) != 0:
+        raise RuntimeError(f"{name} has an invalid quantized payload size")
+    return nbytes // (group_size + 4) * group_size
+
+
+def _views(buffer: torch.Tensor, group_size: int):
+    padded = _padded_numel_of(buffer, group_size)
+    flat = buffer.reshape(-1)
+    return flat[:padded].view(torch.int8), flat[padded:].view(torch.float32)
+
+
+class HipNativeModule:
+    """Instance with the reference extension's symbols; constructing it loads (and type-checks) the library."""
+
+    QuantType = QuantType
+    DType = DType
+    ReduceOP = ReduceOP
+    NATIVE_WIRE_FORMAT = "portable"
+
+    def __init__(self) -> None:
+        self._lib = load_library()
+
+    # ---- quantize ------------------------------------------------------------------------------
+    def quantize(self, input, group_size, topk, stochastic, bit, quant_type, compact):
+        _require_policy(group_size, topk, stochastic, bit, quant_type)
+        output = torch.empty(ops.payload_nbytes(input.numel(), group_size), dtype=torch.uint8, device=input.device)
+        self.inplace_quantize(input, output, group_size, topk, stochastic, bit, quant_type, compact)
+        return output
+
+    def inplace_quantize(self, input, output, group_size, topk, stochastic, bit, quant_type, compact) -> None:
+        _require_policy(group_size, topk, stochastic, bit, quant_type)
+        if not self.inplace_quantize_pack(input, output, None, group_size, topk, stochastic, bit, quant_type, compact):
+            raise RuntimeError(f"no HIP quantize kernel for input dtype {input.dtype}")
+
+    def inplace_quantize_pack(self, input, output, residual, group_size, topk, stochastic, bit, quant_type,
+                              compact) -> bool:
+        """Fused ``(input + residual) -> quantize -> pack`` into ``output``; ``False`` for unsupported policy."""
+        if not _policy_supported(group_size, topk, stochastic, bit, quant_type):
+            return False
+        _check_payload(output, "output")
+        if not isinstance(input, torch.Tensor) or not input.is_cuda:
+            raise RuntimeError("input must be a GPU tensor")
+        if output.device != input.device:
+            raise RuntimeError("input and output must be on the same device")
+        if output.numel() != ops.payload_nbytes(input.numel(), group_size):
+            raise RuntimeError("output has an invalid quantized payload size")
+        if input.numel() == 0:
+            return True
+        if residual is not None and residual.numel() != input.numel():
+            raise RuntimeError("input and residual must have the same number of elements")
+        flat = input.reshape(-1)
+        if not flat.is_contiguous():
+            raise RuntimeError("input must be contiguous")
+        flat_residual = None if residual is None else residual.reshape(-1)
+        return ops.quant_pack_payload_into(flat, output.reshape(-1), group_size=group_size, residual=flat_residual)
+
+    # ---- dequantize -----------------------------------------------------------------------------
+    def dequantize(self, input, group_size, topk, bit, reduce_op, quant_type, dtype, compact):
+        _require_policy(group_size, topk, False, bit, quant_type)
+        _check_payload(input, "input")
+        output = torch.empty(_padded_numel_of(input, group_size), dtype=_TORCH_OF[DType(int(dtype))],
+                             device=input.device)
+        if int(reduce_op) != int(ReduceOP.NONE):
+            output.zero_()
+        self.inplace_dequantize(input, output, group_size, topk, bit, reduce_op, quant_type, compact)
+        return output
+
+    def inplace_dequantize(self, input, output, group_size, topk, bit, reduce_op, quant_type, compact) -> None:
+        _require_policy(group_size, topk, False, bit, quant_type)
+        _check_payload(input, "input")
+        codes, scales = _views(input, group_size)
+        flat = output.reshape(-1)
+        numel = min(flat.numel(), codes.numel())
+        if not ops.dequant_into(codes, scales, flat, numel=numel, group_size=group_size,
+                                reduce_op=_OP_NAME[ReduceOP(int(reduce_op))]):
+            raise RuntimeError(f"no HIP dequantize kernel for output dtype {output.dtype}")
+
+    # ---- dequantize + reduce ------------------------------------------------------------------
+    def _pairs(self, inputs: Sequence[torch.Tensor], group_size: int):
+        if len(inputs) == 0:
+            raise RuntimeError("inputs must not be empty")
+        for i, buffer in enumerate(inputs):
+            _check_payload(buffer, f"inputs[{i}]" if i else "input")
+        return [_views(buffer, group_size) for buffer in inputs]
+
+    def dequantize_reduce(self, inputs, group_size, topk, bit, quant_type, dtype, compact):
+        _require_policy(group_size, topk, False, bit, quant_type)
+        pairs = self._pairs(inputs, group_size)
+        output = torch.empty(pairs[0][0].numel(), dtype=_TORCH_OF[DType(int(dtype))], device=inputs[0].device)
+        self.inplace_dequantize_reduce(inputs, output, group_size, topk, bit, quant_type, compact)
+        return output
+
+    def inplace_dequantize_reduce(self, inputs, output, group_size, topk, bit, quant_type, compact) -> None:
+        """Sum of all payloads into ``output`` in list order; any number of payloads (8 per fused launch)."""
+        _require_policy(group_size, topk, False, bit, quant_type)
+        pairs = self._pairs(inputs, group_size)
+        flat = output.reshape(-1)
+        numel = min(flat.numel(), pairs[0][0].numel())
+        if len(pairs) <= ops.MAX_PAYLOADS:
+            if not ops.dequant_reduce_into(pairs, flat, numel=numel, group_size=group_size):
+                raise RuntimeError(f"no HIP dequantize-reduce kernel for output dtype {output.dtype}")
+            return
+        # More than 8 payloads: keep the left fold exact by chaining decode-and-add one payload at a time.
+        for r, (codes, scales) in enumerate(pairs):
+            if not ops.dequant_into(codes, scales, flat, numel=numel, group_size=group_size,
+                                    reduce_op="none" if r == 0 else "sum"):
+                raise RuntimeError(f"no HIP dequantize kernel for output dtype {output.dtype}")
+
+    def _fused_eligible(self, inputs, output, group_size, topk, bit, quant_type) -> bool:
+        if not _policy_supported(group_size, topk, False, bit, quant_type):
+            return False
+        if not 1 <= len(inputs) <= ops.MAX_PAYLOADS:
+            return False
+        if not isinstance(output, torch.Tensor) or not output.is_cuda or not output.is_contiguous():
+            return False
+        if output.dtype not in ops.DTYPE_CODES or output.numel() == 0:
+            return False
+        expected = ops.payload_nbytes(output.numel(), group_size)
+        for buffer in inputs:
+            if not isinstance(buffer, torch.Tensor) or buffer.dtype != torch.uint8 or not buffer.is_cuda:
+                return False
+            if not buffer.is_contiguous() or buffer.device != output.device or buffer.numel() != expected:
+                return False
+        return True
+
+    def inplace_dequantize_reduce_mean(self, inputs, output, group_size, topk, bit, quant_type, compact,
+                                       divisor) -> bool:
+        if divisor <= 0:
+            raise RuntimeError("divisor must be > 0")
+        if not self._fused_eligible(inputs, output, group_size, topk, bit, quant_type):
+            return False
+        pairs = [_views(buffer, group_size) for buffer in inputs]
+        return ops.dequant_reduce_into(pairs, output.reshape(-1), group_size=group_size, divisor=float(divisor))
+
+    # ---- error feedback -------------------------------------------------------------------------
+    def inplace_error_feedback_update(self, prepared, restored, residual) -> None:
+        if prepared.numel() != restored.numel():
+            raise RuntimeError("prepared and restored must have the same number of elements")
+        if prepared.numel() != residual.numel():
+            raise RuntimeError("prepared and residual must have the same number of elements")
+        if not ops.ef_update_into(prepared.reshape(-1), restored.reshape(-1), residual.reshape(-1)):
+            raise RuntimeError("unsupported dtype for inplace_error_feedback_update")
+
+    def dequantize_reduce_update_error_feedback(self, inputs, prepared, residual, group_size, topk, bit, quant_type,
+                                                dtype, compact, divisor):
+        if len(inputs) == 0:
+            raise RuntimeError("inputs must not be empty")
+        if divisor <= 0:
+            raise RuntimeError("divisor must be > 0")
+        restored = torch.empty(_padded_numel_of(inputs[0], group_size), dtype=_TORCH_OF[DType(int(dtype))],
+                               device=inputs[0].device)
+        trimmed = restored[:prepared.numel()]
+        if not self.inplace_dequantize_reduce_mean_update_error_feedback(
+                inputs, prepared, trimmed, residual, group_size, topk, bit, quant_type, compact, divisor):
+            self.inplace_dequantize_reduce(inputs, trimmed, group_size, topk, bit, quant_type, compact)
+            if divisor != 1:
+                ops.true_divide_(trimmed, divisor)
+            self.inplace_error_feedback_update(prepared, trimmed, residual)
+        return restored
+
+    def inplace_dequantize_reduce_mean_update_error_feedback(self, inputs, prepared, restored, residual, group_size,
+                                                             topk, bit, quant_type, compact, divisor) -> bool:
+        """One launch: ``restored = mean/sum of payloads``, ``residual = prepared - restored``."""
+        if divisor <= 0:
+            raise RuntimeError("divisor must be > 0")
+        for name, t in (("prepared", prepared), ("restored", restored), ("residual", residual)):
+            if not isinstance(t, torch.Tensor) or not t.is_cuda:
+                raise RuntimeError(f"{name} must be a GPU tensor")
+            if not t.is_contiguous():
+                raise RuntimeError(f"{name} must be contiguous")
+        if prepared.numel() != residual.numel():
+            raise RuntimeError("prepared and residual must have the same number of elements")
+        if restored.numel() < prepared.numel():
+            raise RuntimeError("restored must have at least prepared.numel() elements")
+        if prepared.dtype != restored.dtype:
+            raise RuntimeError("prepared and restored must have the same dtype")
+        if prepared.dtype != residual.dtype:
+            raise RuntimeError("prepared and residual must have the same dtype")
+        if prepared.device != restored.device or prepared.device != residual.device:
+            raise RuntimeError("prepared, restored and residual must be on the same device")
+        numel = prepared.numel()
+        if not _policy_supported(group_size, topk, False, bit, quant_type):
+            return False
+        if not 1 <= len(inputs) <= ops.MAX_PAYLOADS or numel == 0:
+            return False
+        expected = ops.payload_nbytes(numel, group_size)
+        for buffer in inputs:
+            if (not isinstance(buffer, torch.Tensor) or buffer.dtype != torch.uint8 or not buffer.is_cuda
+                    or not buffer.is_contiguous() or buffer.device != prepared.device or buffer.numel() != expected):
+                return False
+        pairs = [_views(buffer, group_size) for buffer in inputs]
+        return ops.dequant_reduce_into(pairs, restored.reshape(-1), numel=numel, group_size=group_size,
+                                       divisor=float(divisor), prepared=prepared.reshape(-1),
+                                       new_residual=residual.reshape(-1))

@@ -48,6 +48,15 @@ def promote(a: torch.dtype, b: torch.dtype) -> torch.dtype:
     return a if a == b else torch.float32
 
 
+def true_divide_(tensor: torch.Tensor, divisor: float) -> torch.Tensor:
+    """In-place IEEE division by a scalar.  ``tensor.div_(python_number)`` on a GPU tensor multiplies by
+    the reciprocal, which differs from the CPU codec's true division in the last bit for divisors that
+    are not powers of two; dividing by a 0-dim device tensor takes the exact path."""
+    if tensor.is_cuda:
+        return tensor.div_(torch.full((), float(divisor), dtype=torch.float32, device=tensor.device))
+    return tensor.div_(divisor)
+
+
 # --------------------------------------------------------------------------- #
 def _require(cond: bool, message: str) -> None:
     if not cond:

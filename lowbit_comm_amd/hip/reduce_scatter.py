@@ -1,0 +1,191 @@
+"""Compute steps of the compressed reduce-scatter (+ requantized all-gather) on one GPU.
+
+The reference's transport (``ccdl_comm/communication/reduce_scatter_transport.py:186-377``) pads the
+flattened bucket to ``W * shard_numel``, quantizes each destination chunk separately, exchanges the
+payloads with an all-to-all, and reduces the ``W`` received payloads into this rank's shard; the
+topology family then requantizes the shard, all-gathers the payloads and decodes every shard into
+its slot (``ccdl_comm/communication/topology_transport.py:866-894``).  Here the exchange callables are
+injected (or synthesised by a test / benchmark) and every compute step is one launch:
+
+    quantize W chunks   -> lbc_quant_pack_chunks    (one launch for all W chunks)
+    reduce W payloads   -> lbc_dequant_reduce        (fused, fixed rank order)
+    requantize shard    -> lbc_quant_pack            (into row ``rank`` of the gather buffer)
+    decode W shards     -> lbc_dequant_chunks        (one launch for all W shards)
+
+Workspaces are allocated once per plan and reused, so a steady-state bucket allocates nothing.
+"""
+from __future__ import annotations
+
+from collections.abc import Callable
+from typing import Any
+
+import torch
+
+from lowbit_comm_amd.config import CompressionConfig
+from lowbit_comm_amd.hip import ops
+from lowbit_comm_amd.hip.chunk_plan import ChunkPlan, compile_chunk_plan
+from lowbit_comm_amd.hip.codec import ccdl_dtype, torch_dtype
+from lowbit_comm_amd.shard import ReducedShard
+
+_ROW_ALIGN = 256
+
+
+class ReduceScatterPlan:
+    """Pre-bound compute of one bucket shape at world size ``W`` for rank ``rank``."""
+
+    def __init__(self, numel: int, dtype: torch.dtype, *, world_size: int, rank: int, config: CompressionConfig,
+                 device: torch.device | str, reduced_dtype: torch.dtype | None = None,
+                 shape: tuple[int, ...] | None = None) -> None:
+        if config.bit != 8 or config.quant_type != "linear" or config.topk != 0 or config.stochastic:
+            raise ValueError("the HIP reduce-scatter plan supports linear 8-bit quantization without top-k / stochastic")
+        if not 0 <= rank < world_size:
+            raise ValueError(f"rank must be in [0, {world_size})")
+        self.config = config
+        self.world_size = world_size
+        self.rank = rank
+        self.numel = int(numel)
+        self.shape = tuple(shape) if shape is not None else (self.numel,)
+        self.dtype = dtype
+        self.reduced_dtype = reduced_dtype or dtype
+        self.device = torch.device(device)
+        self.chunks: ChunkPlan = compile_chunk_plan(original_numel=self.numel, world_size=world_size)
+        shard = self.chunks.shard_numel
+        g = config.group_size
+        self.payload_bytes = ops.payload_nbytes(shard, g)
+        self.row_stride = -(-self.payload_bytes // _ROW_ALIGN) * _ROW_ALIGN
+        rows = (world_size, self.row_stride)
+        self.send = torch.empty(rows, dtype=torch.uint8, device=self.device)       # my chunk for every rank
+        self.received = torch.empty(rows, dtype=torch.uint8, device=self.device)   # every rank's chunk for me
+        self.gathered = torch.empty(rows, dtype=torch.uint8, device=self.device)   # every rank's requantized shard
+        self.shard = torch.empty(shard, dtype=self.reduced_dtype, device=self.device)
+        self._bound: dict[Any, ops.BoundLaunch] = {}   # launches bound to tensor addresses seen so far
+
+    def _remember(self, key: Any, make: Callable[[], ops.BoundLaunch]) -> ops.BoundLaunch:
+        bound = self._bound.get(key)
+        if bound is None:
+            if len(self._bound) >= 32:      # addresses keep changing: do not grow without bound
+                self._bound.clear()
+            bound = self._bound[key] = make()
+        return bound
+
+    # ---- payload views ---------------------------------------------------------------------------
+    def payload(self, rows: torch.Tensor, index: int) -> torch.Tensor:
+        """Row ``index`` of a payload matrix, trimmed to the exact payload size (a view)."""
+        return rows[index, :self.payload_bytes]
+
+    def _pairs(self, rows: torch.Tensor):
+        shard, g = self.chunks.shard_numel, self.config.group_size
+        return [ops.split_payload(self.payload(rows, r), shard, g) for r in range(self.world_size)]
+
+    # ---- compute steps ---------------------------------------------------------------------------
+    def quantize_chunks(self, tensor: torch.Tensor) -> torch.Tensor:
+        """Quantize the ``W`` destination chunks of ``tensor`` into ``self.send`` (one launch)."""
+        flat = tensor.reshape(-1)
+        if flat.numel() != self.numel or flat.dtype != self.dtype:
+            raise ValueError("tensor does not match the planned bucket")
+        bound = self._remember(("q", flat.data_ptr()), lambda: ops.bind_quant_pack_chunks(
+            flat, self.send, self.world_size, group_size=self.config.group_size))
+        if self.numel and not bound():
+            raise ValueError(f"no HIP quantize kernel for dtype {flat.dtype}")
+        return self.send
+
+    def reduce_received(self, received: torch.Tensor | None = None, *, op: str = "sum",
+                        out: torch.Tensor | None = None) -> ReducedShard:
+        """Fused dequant-reduce of the ``W`` received payloads (rank order) into this rank's shard."""
+        if op not in ("sum", "mean"):
+            raise ValueError(f"unsupported reduce-scatter mode: {op}")
+        rows = self.received if received is None else received
+        target = self.shard if out is None else out
+        shard = self.chunks.shard_numel
+        fused = self.world_size <= ops.MAX_PAYLOADS
+        if shard:
+            if fused:
+                bound = self._remember(("r", rows.data_ptr(), target.data_ptr(), op), lambda: ops.bind_dequant_reduce(
+                    self._pairs(rows), target, numel=shard, group_size=self.config.group_size,
+                    divisor=float(self.world_size) if op == "mean" else 1.0))
+                fused = bool(bound())
+            if not fused:
+                for r, (codes, scales) in enumerate(self._pairs(rows)):
+                    ops.dequant_into(codes, scales, target, numel=shard, group_size=self.config.group_size,
+                                     reduce_op="none" if r == 0 else "sum")
+                if op == "mean":
+                    ops.true_divide_(target, self.world_size)
+        metadata = {
+            "compression_bit": self.config.bit, "group_size": self.config.group_size, "workspace_output": True,
+            "workspace_shape": (shard,), "quantized_workspace_output": True, "received_workspace_output": True,
+            "workspace_cache": True, "output_ownership": "plan" if out is None else "caller",
+            "fused_dequant_reduce": fused, "chunk_plan_precompiled": True,
+            "received_payload_numel": self.world_size * self.payload_bytes,
+        }
+        if not fused:
+            metadata["fused_dequant_reduce_reason"] = (
+                f"fused dequant supports at most {ops.MAX_PAYLOADS} input ranks; received {self.world_size}")
+        return ReducedShard(shard=target, shard_index=self.rank, shard_numel=shard, original_shape=self.shape,
+                            original_numel=self.numel, world_size=self.world_size, reduce=op,
+                            padded_numel=self.chunks.padded_numel, dtype=ops.DTYPE_NAMES[self.reduced_dtype],
+                            transport="compressed_all_to_all", metadata=metadata)
+
+    def requantize_shard(self, shard: torch.Tensor | None = None) -> torch.Tensor:
+        """Quantize the reduced shard into row ``rank`` of ``self.gathered``; returns that payload view."""
+        source = self.shard if shard is None else shard
+        row = self.payload(self.gathered, self.rank)
+
+        def make() -> ops.BoundLaunch:
+            codes, scales = ops.split_payload(row, self.chunks.shard_numel, self.config.group_size)
+            return ops.bind_quant_pack(source, codes, scales, group_size=self.config.group_size)
+
+        bound = self._remember(("g", source.data_ptr()), make)
+        if self.chunks.shard_numel and not bound():
+            raise ValueError(f"no HIP quantize kernel for dtype {source.dtype}")
+        return row
+
+    def decode_gathered(self, gathered: torch.Tensor | None = None, *, out: torch.Tensor | None = None) -> torch.Tensor:
+        """Decode the ``W`` gathered shard payloads into one flat tensor of the bucket's size (one launch)."""
+        rows = self.gathered if gathered is None else gathered
+        target = out if out is not None else torch.empty(self.numel, dtype=self.reduced_dtype, device=self.device)
+        make = lambda: ops.bind_dequant_chunks(rows, target.reshape(-1), self.chunks.shard_numel,  # noqa: E731
+                                               group_size=self.config.group_size)
+        bound = self._remember(("d", rows.data_ptr(), target.data_ptr()), make) if out is not None else make()
+        if self.numel and not bound():
+            raise ValueError(f"no HIP decode kernel for dtype {target.dtype}")
+        return target.reshape(self.shape)
+
+
+def compressed_reduce_scatter_shard(tensor: torch.Tensor, *, config: CompressionConfig, world_size: int, rank: int,
+                                    all_to_all: Callable[[torch.Tensor, torch.Tensor], None], op: str = "sum",
+                                    plan: ReduceScatterPlan | None = None) -> ReducedShard:
+    """Quantize per-destination chunks, exchange, reduce: returns this rank's :class:`ReducedShard`.
+
+    ``all_to_all(received_rows, send_rows)`` must fill row ``r`` of ``received_rows`` with rank ``r``'s
+    payload for this rank (row ``rank`` of ``send_rows`` of that rank) - the one collective of the leg.
+    """
+    if plan is None:
+        plan = ReduceScatterPlan(tensor.numel(), tensor.dtype, world_size=world_size, rank=rank, config=config,
+                                 device=tensor.device, shape=tuple(tensor.shape))
+    send = plan.quantize_chunks(tensor)
+    all_to_all(plan.received, send)
+    return plan.reduce_received(op=op)
+
+
+def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: CompressionConfig, world_size: int,
+                                             rank: int, all_to_all: Callable[[torch.Tensor, torch.Tensor], None],
+                                             all_gather: Callable[[torch.Tensor, torch.Tensor], None],
+                                             op: str = "sum", plan: ReduceScatterPlan | None = None,
+                                             out: torch.Tensor | None = None) -> torch.Tensor:
+    """Full plan: reduce-scatter leg, requantize, all-gather leg, decode every shard.
+
+    ``all_gather(gathered_rows, my_payload)`` must fill row ``r`` of ``gathered_rows`` with rank ``r``'s
+    requantized shard payload (row ``rank`` is already in place).
+    """
+    if plan is None:
+        plan = ReduceScatterPlan(tensor.numel(), tensor.dtype, world_size=world_size, rank=rank, config=config,
+                                 device=tensor.device, shape=tuple(tensor.shape))
+    compressed_reduce_scatter_shard(tensor, config=config, world_size=world_size, rank=rank, all_to_all=all_to_all,
+                                    op=op, plan=plan)
+    mine = plan.requantize_shard()
+    all_gather(plan.gathered, mine)
+    return plan.decode_gathered(out=out)
+
+
+__all__ = ["ReduceScatterPlan", "compressed_all_reduce_via_reduce_scatter", "compressed_reduce_scatter_shard",
+           "ccdl_dtype", "torch_dtype"]

@@ -1,0 +1,499 @@
+"""GPU tests of the host layer over the HIP kernels: the native-module shim behind the codec facade, the
+codec callables, the bucket processor and comm hook, the precollected-payload executor, the
+reduce-scatter plan and the workspace pool with real device events.  Expected values come from the CPU
+oracle on the same inputs; integer/byte results and fp32 results are compared bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+from lowbit_comm_amd import CompressionConfig
+from lowbit_comm_amd.communication import FusedPayloadPacker, GatheredPayloads, PackedPayload, make_fused_payload_all_gather
+from lowbit_comm_amd.communication.ddp import DDPBucketProcessor
+from lowbit_comm_amd.communication.ddp_hook import create_ddp_comm_hook
+from lowbit_comm_amd.quantization import ErrorFeedbackState, Quantizer, codec
+from oracle import codec_np, codec_torch
+
+pytestmark = pytest.mark.gpu
+CFG = CompressionConfig()
+
+
+@pytest.fixture(scope="module")
+def dev(hip_device):
+    return hip_device
+
+
+@pytest.fixture(scope="module")
+def status(dev):
+    from lowbit_comm_amd.hip.loader import load_hip_extension
+
+    found = load_hip_extension()
+    assert found.available, found.reason
+    return found
+
+
+def grad(n, dtype, seed, dev, sigma=1e-3):
+    gen = torch.Generator().manual_seed(seed)
+    return (torch.randn(n, generator=gen) * sigma).to(dtype).to(dev)
+
+
+def same_bits(a, b):
+    a, b = a.detach().cpu().contiguous(), b.detach().cpu().contiguous()
+    assert a.dtype == b.dtype and a.shape == b.shape, (a.dtype, b.dtype, a.shape, b.shape)
+    view = torch.int32 if a.dtype == torch.float32 else torch.int16
+    return torch.equal(a.view(view), b.view(view))
+
+
+def oracle_packed(x_cpu, g=64):
+    return codec_torch.pack(*codec_torch.quantize(x_cpu, g))
+
+
+class Bucket:
+    def __init__(self, tensor, index=0):
+        self._tensor, self._index = tensor, index
+
+    def buffer(self):
+        return self._tensor
+
+    def index(self):
+        return self._index
+
+
+# --------------------------------------------------------------------------- #
+# facade over the native module
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("dtype,name", [(torch.float32, "fp32"), (torch.bfloat16, "bf16"), (torch.float16, "fp16")])
+@pytest.mark.parametrize("n", [64, 1000, 65_537])
+def test_facade_quantize_dequantize_round_trip(status, dev, dtype, name, n):
+    x = grad(n, dtype, 10 + n, dev).reshape(-1)
+    buffer = codec.quantize_tensor(x, CFG, extension_status=status)
+    assert buffer.dtype == torch.uint8 and torch.equal(buffer.cpu(), oracle_packed(x.cpu()))
+    restored = codec.dequantize_tensor(buffer, (n,), CFG, dtype=name, extension_status=status)
+    want = codec_torch.dequantize(*codec_torch.quantize(x.cpu()), n, 64, name)
+    assert same_bits(restored, want)
+    out = codec.allocate_quantized_buffer(x, CFG, dtype=name)
+    meta = {}
+    assert codec.quantize_tensor(x, CFG, extension_status=status, output=out, metadata=meta) is out
+    assert meta["fused_quant_pack"] is True and meta["original_numel"] == n
+    assert torch.equal(out, buffer)
+    q = Quantizer(CFG, dtype=name, extension_status=status)
+    assert torch.equal(q.quantize(x, q.allocate_q(x)), buffer)
+    assert same_bits(q.dequantize(buffer, (n,)), want)
+
+
+def test_inplace_calls_do_not_allocate_or_touch_inputs(status, dev):
+    n = 1 << 20
+    x = grad(n, torch.float32, 1, dev)
+    residual = grad(n, torch.float32, 2, dev, sigma=1e-5)
+    keep_x, keep_r = x.clone(), residual.clone()
+    out = codec.allocate_quantized_buffer(x, CFG, dtype="fp32")
+    workspace = codec.allocate_dequantized_buffer(x, (n,), CFG)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    pointers = (out.data_ptr(), workspace.data_ptr())
+    for _ in range(3):
+        assert codec.inplace_quantize_pack(x, out, residual, CFG, extension_status=status)
+        assert codec.inplace_dequantize_reduce_mean([out, out], workspace, CFG, extension_status=status, reduce="mean")
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert (out.data_ptr(), workspace.data_ptr()) == pointers
+    assert torch.equal(x, keep_x) and torch.equal(residual, keep_r)
+    assert torch.equal(out.cpu(), oracle_packed(keep_x.cpu() + keep_r.cpu()))
+
+
+@pytest.mark.parametrize("world", [2, 8, 11])
+@pytest.mark.parametrize("reduce", ["sum", "mean"])
+def test_facade_dequantize_reduce_matches_the_left_fold(status, dev, world, reduce):
+    n = 40_000
+    peers = [grad(n, torch.float32, 100 + r, dev) for r in range(world)]
+    buffers = [codec.quantize_tensor(p, CFG, extension_status=status) for p in peers]
+    payloads = [codec_torch.quantize(p.cpu()) for p in peers]
+    want = codec_torch.reduce_payloads(payloads, n, 64, "fp32", reduce)
+    got = codec.dequantize_reduce_tensors(buffers, (n,), CFG, dtype="fp32", extension_status=status, reduce=reduce)
+    assert same_bits(got, want)
+    workspace = codec.allocate_dequantized_buffer(peers[0], (n,), CFG)
+    got = codec.dequantize_reduce_tensors(buffers, (n,), CFG, dtype="fp32", extension_status=status,
+                                          output=workspace, reduce=reduce)
+    assert same_bits(got, want) and got.data_ptr() == workspace.data_ptr()
+    fused = codec.inplace_dequantize_reduce_mean(buffers, workspace, CFG, extension_status=status, reduce=reduce)
+    assert fused is (world <= 8)
+
+
+def test_facade_error_feedback_calls(status, dev):
+    n, world = 30_016, 4
+    peers = [grad(n, torch.float32, 200 + r, dev) for r in range(world)]
+    buffers = [codec.quantize_tensor(p, CFG, extension_status=status) for p in peers]
+    prepared = grad(n, torch.float32, 250, dev)
+    restored = torch.empty(n, device=dev)
+    residual = torch.empty(n, device=dev)
+    assert codec.inplace_dequantize_reduce_mean_update_error_feedback(
+        buffers, prepared, restored, residual, CFG, extension_status=status, reduce="mean")
+    want = codec_torch.reduce_payloads([codec_torch.quantize(p.cpu()) for p in peers], n, 64, "fp32", "mean")
+    assert same_bits(restored, want) and same_bits(residual, prepared.cpu() - want)
+    residual2 = torch.zeros(n, device=dev)
+    got = codec.dequantize_reduce_update_error_feedback(buffers, prepared, residual2, (n,), CFG, dtype="fp32",
+                                                        extension_status=status, reduce="mean")
+    assert same_bits(got, want) and same_bits(residual2, prepared.cpu() - want)
+    residual3 = torch.zeros(n, device=dev)
+    codec.update_error_feedback_residual(prepared, restored, residual3, extension_status=status)
+    assert same_bits(residual3, prepared.cpu() - want)
+    with pytest.raises(RuntimeError, match="divisor must be > 0"):
+        status.module.inplace_dequantize_reduce_mean(buffers, restored, 64, 0, 8, status.module.QuantType.Linear, False, 0)
+    with pytest.raises(RuntimeError, match="same number of elements"):
+        codec.inplace_dequantize_reduce_mean_update_error_feedback(
+            buffers, prepared, restored, residual[:-1], CFG, extension_status=status)
+
+
+def test_unsupported_policies_decline_instead_of_failing(status, dev):
+    x = grad(1024, torch.float32, 3, dev)
+    out = torch.empty(1024 // 64 * 68, dtype=torch.uint8, device=dev)
+    for cfg in (CompressionConfig(topk=1), CompressionConfig(stochastic=True), CompressionConfig(quant_type="normal"),
+                CompressionConfig(bit=4, allow_experimental=True)):
+        assert codec.inplace_quantize_pack(x, out, None, cfg, extension_status=status) is False
+        if not cfg.stochastic:                      # decoding does not depend on how rounding was done
+            assert codec.inplace_dequantize_reduce_mean([out], torch.empty_like(x), cfg, extension_status=status) is False
+    with pytest.raises(RuntimeError, match="invalid quantized payload size"):
+        codec.inplace_quantize_pack(x, out[:-1], None, CFG, extension_status=status)
+
+
+# --------------------------------------------------------------------------- #
+# codec callables + packer + hook
+# --------------------------------------------------------------------------- #
+def test_hip_codec_callables_produce_the_portable_payload_and_pack_without_a_copy(dev):
+    from lowbit_comm_amd.hip.codec import dequantize_tensor_hip, quantize_tensor_hip
+
+    x = grad(10_000, torch.bfloat16, 7, dev).reshape(100, 100)
+    payload = quantize_tensor_hip(x, CFG)
+    w_codes, w_scales = codec_torch.quantize(x.cpu())
+    assert isinstance(payload, PackedPayload) and payload.shape == (100, 100) and payload.dtype == "bf16"
+    assert payload.buffer.dtype == torch.int8 and torch.equal(payload.buffer.cpu(), w_codes)
+    assert same_bits(payload.metadata["scales"], w_scales) and payload.metadata["original_numel"] == 10_000
+    packer = FusedPayloadPacker.from_payload(payload)
+    packed = packer.pack(payload)
+    assert packed.data_ptr() == payload.packed.data_ptr() and torch.equal(packed.cpu(), codec_torch.pack(w_codes, w_scales))
+    again = packer.unpack(packed, shape=payload.shape, dtype="bf16")
+    restored = dequantize_tensor_hip(again, (100, 100), CFG, "bf16")
+    assert same_bits(restored, codec_torch.dequantize(w_codes, w_scales, 10_000, 64, "bf16").reshape(100, 100))
+    with pytest.raises(ValueError, match="linear"):
+        quantize_tensor_hip(x, CompressionConfig(quant_type="normal"))
+    with pytest.raises(ValueError, match="bit=8"):
+        quantize_tensor_hip(x, CompressionConfig(bit=4, allow_experimental=True))
+
+
+def _peer_gather(peers_cpu_payloads, dev):
+    """all_gather stand-in: rank 0 is the local payload, the others are synthesised peers."""
+    def all_gather(local):
+        others = [CompressedPayloadOn(dev, codes, scales, local) for codes, scales in peers_cpu_payloads]
+        return GatheredPayloads([local] + others, 1 + len(others))
+    return all_gather
+
+
+def CompressedPayloadOn(dev, codes, scales, like):
+    from lowbit_comm_amd.communication import CompressedPayload
+
+    return CompressedPayload(buffer=codes.to(dev), shape=like.shape, dtype=like.dtype,
+                             metadata={"scales": scales.to(dev), "original_numel": like.metadata["original_numel"]})
+
+
+@pytest.mark.parametrize("reduce", ["mean", "sum"])
+def test_all_gather_hook_with_hip_callables_matches_the_reference_sequence(dev, reduce):
+    from lowbit_comm_amd.hip.codec import dequantize_tensor_hip, quantize_tensor_hip
+
+    n, world = 20_000, 4
+    peers = [codec_torch.quantize(grad(n, torch.float32, 300 + r, "cpu")) for r in range(world - 1)]
+    state = ErrorFeedbackState()
+    hook = create_ddp_comm_hook(CFG, strategy="all_gather", reduce=reduce, quantize=quantize_tensor_hip,
+                                dequantize=dequantize_tensor_hip, all_gather=_peer_gather(peers, dev),
+                                error_feedback=state)
+    cpu_residual = None
+    for step in range(3):
+        g = grad(n, torch.float32, 400 + step, dev)
+        restored = hook(None, Bucket(g, index=5)).wait()
+        prepared = g.cpu() if cpu_residual is None else g.cpu() + cpu_residual
+        payloads = [codec_torch.quantize(prepared)] + peers
+        want = codec_torch.reduce_payloads(payloads, n, 64, "fp32", reduce)
+        cpu_residual = prepared - want
+        assert same_bits(restored, want), f"step {step}"
+        assert same_bits(state.get(5), cpu_residual), f"residual step {step}"
+
+
+def test_all_gather_hook_facade_path_uses_the_fused_kernels(status, dev):
+    """dequantize=None: flat uint8 buffers, fused decode+reduce, and from the second step on the fused
+    decode+reduce+residual-update kernel into a cached workspace."""
+    n, world = 50_000, 8
+    peers = [oracle_packed(grad(n, torch.float32, 500 + r, "cpu")).to(dev) for r in range(world - 1)]
+    peer_payloads = [codec_torch.quantize(grad(n, torch.float32, 500 + r, "cpu")) for r in range(world - 1)]
+
+    def all_gather(local):
+        return GatheredPayloads([local.buffer] + peers, world)
+
+    state = ErrorFeedbackState()
+    hook = create_ddp_comm_hook(CFG, strategy="all_gather", reduce="mean", all_gather=all_gather,
+                                error_feedback=state, extension_status=status)
+    cpu_residual = None
+    outputs = []
+    for step in range(4):
+        g = grad(n, torch.float32, 600 + step, dev)
+        restored = hook(None, Bucket(g, index=1)).wait()
+        outputs.append(restored.data_ptr())
+        prepared = g.cpu() if cpu_residual is None else g.cpu() + cpu_residual
+        want = codec_torch.reduce_payloads([codec_torch.quantize(prepared)] + peer_payloads, n, 64, "fp32", "mean")
+        cpu_residual = prepared - want
+        assert same_bits(restored, want), f"step {step}"
+        assert same_bits(state.get(1), cpu_residual), f"residual step {step}"
+    assert outputs[1] == outputs[2] == outputs[3]          # cached decode workspace from step 1 on
+
+
+def test_fused_all_gather_adapter_ships_one_packed_tensor(dev):
+    from lowbit_comm_amd.hip.codec import dequantize_reduce_hip, quantize_tensor_hip
+
+    n = 8192
+    local = quantize_tensor_hip(grad(n, torch.float32, 1, dev), CFG)
+    remote = quantize_tensor_hip(grad(n, torch.float32, 2, dev), CFG)
+    seen = []
+
+    def byte_all_gather(packed):
+        seen.append((packed.data_ptr(), packed.numel()))
+        return GatheredPayloads([packed, remote.packed], 2)
+
+    gathered = make_fused_payload_all_gather(byte_all_gather)(local)
+    assert seen == [(local.packed.data_ptr(), n // 64 * 68)]
+    got = dequantize_reduce_hip(gathered.payloads, (n,), CFG, "fp32", "sum")
+    want = codec_torch.reduce_payloads([(p.buffer.cpu(), p.metadata["scales"].cpu()) for p in (local, remote)], n)
+    assert same_bits(got, want)
+    assert dequantize_reduce_hip([local] * 9, (n,), CFG, "fp32", "sum") is None
+
+
+# --------------------------------------------------------------------------- #
+# fused local round trip (config 3 semantics)
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("dtype,name", [(torch.bfloat16, "bf16"), (torch.float32, "fp32"), (torch.float16, "fp16")])
+def test_fused_bucket_processor_equals_the_unfused_reference_sequence(dev, dtype, name):
+    n = 100_032
+    fused = DDPBucketProcessor.from_hip_codec(CFG, fused=True)
+    unfused = DDPBucketProcessor.from_hip_codec(CFG, fused=False)
+    if dtype != torch.float32:                      # config 3: an fp32 residual already exists
+        seed = grad(n, torch.float32, 9, dev, sigma=1e-5)
+        fused.error_feedback.put(0, seed.clone())
+        unfused.error_feedback.put(0, seed.clone())
+        cpu_residual = seed.cpu()
+    else:
+        cpu_residual = None
+    for step in range(4):
+        g = grad(n, dtype, 700 + step, dev)
+        torch.cuda.synchronize()
+        out_fused = fused.process(Bucket(g), dtype=name)
+        out_plain = unfused.process(Bucket(g), dtype=name)
+        _c, _s, want, cpu_residual = codec_torch.ef_round_trip(g.cpu(), cpu_residual, 64, name)
+        assert out_fused.dtype == dtype and same_bits(out_fused, want), f"step {step}"
+        assert same_bits(out_plain, want), f"unfused step {step}"
+        assert same_bits(fused.error_feedback.get(0), cpu_residual), f"residual step {step}"
+        assert same_bits(unfused.error_feedback.get(0), cpu_residual), f"unfused residual step {step}"
+
+
+def test_fused_codec_steady_state_allocates_nothing(dev):
+    from lowbit_comm_amd.hip.codec import FusedErrorFeedbackCodec
+
+    n = 1 << 20
+    fused = FusedErrorFeedbackCodec(CFG)
+    g = grad(n, torch.bfloat16, 1, dev)
+    fused.error_feedback.put("b", torch.zeros(n, device=dev))
+    fused.step("b", g, "bf16")
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    residual_ptr = fused.error_feedback.get("b").data_ptr()
+    for _ in range(5):
+        payload, restored = fused.step("b", g, "bf16")
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert fused.error_feedback.get("b").data_ptr() == residual_ptr
+    assert payload.packed.numel() == n // 64 * 68 and restored.dtype == torch.bfloat16
+
+
+# --------------------------------------------------------------------------- #
+# precollected payloads (the reference's own "payloads already in device memory" entry)
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("world,fused", [(1, True), (8, True), (9, False)])
+def test_precollected_payload_executor(status, dev, world, fused):
+    from lowbit_comm_amd.hip.executors import FUSED_FAST_PATH, PrecollectedPayloadExecutor
+
+    n = 64 * 500
+    executor = PrecollectedPayloadExecutor(CFG, shape=(n,), dtype="fp32", extension_status=status)
+    peers = [grad(n, torch.float32, 800 + r, "cpu") for r in range(world)]
+    payloads = [oracle_packed(p).to(dev) for p in peers]
+    prepared = grad(n, torch.float32, 850, dev)
+    output = torch.empty(n, device=dev)
+    residual = torch.empty(n, device=dev)
+    assert executor.run_precollected_payloads(payloads, prepared, output, residual) is output
+    want = codec_torch.reduce_payloads([codec_torch.quantize(p) for p in peers], n, 64, "fp32", "mean")
+    assert same_bits(output, want) and same_bits(residual, prepared.cpu() - want)
+    info = executor.last_execution_info
+    assert info.fallback_used is (not fused)
+    assert info.fast_path == (FUSED_FAST_PATH if fused else "python_fallback")
+    if not fused:
+        assert "at most 8 payloads" in info.fallback_reason
+    assert executor.execution_counters.snapshot().completed_runs == 1
+    with pytest.raises(ValueError, match="must contain"):
+        executor.run_precollected_payloads([payloads[0][:-4]], prepared, output, residual)
+    with pytest.raises(ValueError, match="must not be empty"):
+        executor.run_precollected_payloads([], prepared, output, residual)
+    assert executor.execution_counters.snapshot().failed_runs == 2
+
+
+# --------------------------------------------------------------------------- #
+# reduce-scatter plan with every rank simulated on one device (config 4 structure)
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("n,world", [(64 * 8 * 40, 8), (100_003, 4), (70_000, 3)])
+def test_reduce_scatter_all_gather_plan_matches_the_oracle(dev, n, world):
+    from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan, compressed_all_reduce_via_reduce_scatter
+
+    buckets = [grad(n, torch.float32, 900 + r, dev) for r in range(world)]
+    plans = [ReduceScatterPlan(n, torch.float32, world_size=world, rank=r, config=CFG, device=dev) for r in range(world)]
+    for plan, bucket in zip(plans, buckets):
+        plan.quantize_chunks(bucket)
+
+    def all_to_all_for(rank):
+        def exchange(received, send):
+            for src in range(world):
+                received[src].copy_(plans[src].send[rank])
+        return exchange
+
+    shards = []
+    for r, plan in enumerate(plans):
+        all_to_all_for(r)(plan.received, plan.send)
+        reduced = plan.reduce_received(op="sum")
+        assert reduced.metadata["fused_dequant_reduce"] and reduced.shard_index == r
+        shards.append(reduced)
+        plan.requantize_shard()
+
+    def all_gather(gathered, mine):
+        for src in range(world):
+            gathered[src].copy_(plans[src].gathered[src])
+
+    full = []
+    for plan in plans:
+        all_gather(plan.gathered, None)
+        full.append(plan.decode_gathered())
+    want_shards, want_full = codec_np.reduce_scatter_all_gather_plan([b.cpu().numpy() for b in buckets], 64, "sum")
+    for r in range(world):
+        assert np.array_equal(shards[r].shard.cpu().numpy().view(np.uint32), want_shards[r].view(np.uint32)), r
+        assert np.array_equal(full[r].cpu().numpy().view(np.uint32), want_full.view(np.uint32)), r
+    # the one-call form on rank 0, reusing its plan
+    out = compressed_all_reduce_via_reduce_scatter(buckets[0], config=CFG, world_size=world, rank=0,
+                                                   all_to_all=all_to_all_for(0), all_gather=all_gather, plan=plans[0])
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want_full.view(np.uint32))
+
+
+def test_reduce_scatter_plan_beyond_eight_ranks_chains_exactly(dev):
+    from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
+
+    n, world = 64 * 12 * 10, 12
+    buckets = [grad(n, torch.float32, 950 + r, dev) for r in range(world)]
+    plans = [ReduceScatterPlan(n, torch.float32, world_size=world, rank=r, config=CFG, device=dev) for r in range(world)]
+    for plan, bucket in zip(plans, buckets):
+        plan.quantize_chunks(bucket)
+    for src in range(world):
+        plans[0].received[src].copy_(plans[src].send[0])
+    reduced = plans[0].reduce_received(op="mean")
+    assert reduced.metadata["fused_dequant_reduce"] is False and "at most 8" in reduced.metadata["fused_dequant_reduce_reason"]
+    shard = n // world
+    payloads = [codec_np.quantize_chunks(b.cpu().numpy(), world, 64)[0] for b in buckets]
+    want = codec_np.reduce_payloads(payloads, shard, 64, "fp32", "mean")
+    assert np.array_equal(reduced.shard.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+# --------------------------------------------------------------------------- #
+# workspace pool with real streams and events
+# --------------------------------------------------------------------------- #
+def test_pool_reuses_buffers_across_streams_without_host_sync(dev):
+    from lowbit_comm_amd.hip import EventCompletion, WorkspaceKey, create_torch_workspace_pool
+
+    pool = create_torch_workspace_pool()
+    key = WorkspaceKey(backend="hip", collective="reduce_scatter", strategy="compressed", shape_class=(1 << 22,),
+                       dtype="float32", world_size=8, bit=8, group_size=64, chunk_config=(0,), workspace_kind="reduced",
+                       device=str(dev))
+    producer, consumer = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(producer):
+        lease = pool.acquire(key, producer)
+        lease.buffer.fill_(1.0)
+        for _ in range(20):
+            lease.buffer.mul_(1.0000001)
+        lease.release(completion=EventCompletion(producer))
+    with torch.cuda.stream(consumer):
+        taken = pool.acquire(key, consumer)            # same buffer: handed off (or idle if the work already ended)
+        assert taken.buffer.data_ptr() == lease.buffer.data_ptr()
+        total = taken.buffer.sum()
+        taken.release(completion=EventCompletion(consumer))
+    torch.cuda.synchronize()
+    assert abs(float(total) / (1 << 22) - 1.0) < 1e-3
+    stats = pool.stats
+    assert (stats.hits, stats.misses) == (1, 1) and stats.in_flight_bytes == 0 and stats.cached_bytes == 4 << 22
+    before = torch.cuda.memory_allocated()
+    for _ in range(10):
+        again = pool.acquire(key, torch.cuda.current_stream())
+        again.release(completion=EventCompletion())
+        torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before and pool.stats.misses == 1
+
+
+def test_llama_shaped_bucket_stream_through_the_pool(dev):
+    """Config 5 structure at 1/64 scale: bf16 parameter tensors of a Llama-3-8B-shaped layer stack, flattened in
+    reverse registration order into fixed-size buckets with a ragged tail; per bucket EF quant-pack and a W=8
+    shard reduce with pooled workspaces.  Checks: bit parity of sampled buckets and of the ragged tail, pool
+    misses == distinct workspace keys, zero allocations after the first pass."""
+    from lowbit_comm_amd.hip import EventCompletion, ShardWorkspaceProvider, create_torch_workspace_pool
+    from lowbit_comm_amd.hip import ops
+    from lowbit_comm_amd.hip.codec import FusedErrorFeedbackCodec
+
+    hidden, ffn, kv, vocab, layers = 512, 1792, 128, 16_032, 2
+    shapes = [(vocab, hidden)]
+    for _ in range(layers):
+        shapes += [(hidden, hidden), (kv, hidden), (kv, hidden), (hidden, hidden), (ffn, hidden), (ffn, hidden),
+                   (hidden, ffn), (hidden,), (hidden,)]
+    shapes += [(hidden,), (vocab, hidden), (1001,)]      # the odd-sized last tensor makes the tail ragged
+    total = sum(int(np.prod(s)) for s in shapes)
+    bucket_numel = 1 << 20
+    stream = torch.cat([grad(int(np.prod(s)), torch.bfloat16, 1000 + i, dev) for i, s in enumerate(reversed(shapes))])
+    assert stream.numel() == total
+    bounds = [(a, min(a + bucket_numel, total)) for a in range(0, total, bucket_numel)]
+    assert (bounds[-1][1] - bounds[-1][0]) % 64 != 0          # ragged tail
+    world = 8
+    pool = create_torch_workspace_pool()
+    provider = ShardWorkspaceProvider(pool, backend="hip", collective="reduce_scatter", strategy="compressed",
+                                      device=str(dev))
+    codec_ef = FusedErrorFeedbackCodec(CFG)
+    cpu_residuals = {}
+
+    def one_pass(check):
+        for index, (a, b) in enumerate(bounds):
+            bucket = stream[a:b]
+            payload, _restored = codec_ef.step(index, bucket, "bf16")
+            shard = -(-(b - a) // world)
+            session = provider.begin(stream=torch.cuda.current_stream())
+            received = [session.get_received_tensor_payload(index, r, bucket[:shard], CFG, dtype="bf16", world_size=world)
+                        for r in range(world)]
+            out = session.get_reduced_shard(index, torch.empty(0, dtype=torch.float32, device=dev), (shard,), CFG,
+                                            dtype="fp32", world_size=world, rank=0)
+            first = bucket[:shard].float()
+            for r, row in enumerate(received):               # synthetic peers: scaled copies of this rank's chunk
+                assert ops.quant_pack_payload_into(first * (1.0 + 0.125 * r), row)
+            pairs = [ops.split_payload(row, shard) for row in received]
+            assert ops.dequant_reduce_into(pairs, out, numel=shard)
+            if check and index in (0, len(bounds) // 2, len(bounds) - 1):
+                w_codes, w_scales, _r, cpu_residuals[index] = codec_torch.ef_round_trip(
+                    bucket.cpu(), cpu_residuals.get(index), 64, "bf16")
+                assert torch.equal(payload.buffer.cpu(), w_codes), index
+                assert same_bits(payload.metadata["scales"], w_scales), index
+                assert same_bits(codec_ef.error_feedback.get(index), cpu_residuals[index]), index
+                peers = [codec_torch.quantize(first.cpu() * (1.0 + 0.125 * r)) for r in range(world)]
+                assert same_bits(out[:shard], codec_torch.reduce_payloads(peers, shard)), index
+            session.release(completion=EventCompletion())
+
+    one_pass(check=True)
+    torch.cuda.synchronize()
+    distinct_keys = 2 * (world + 1)                           # full-size and tail shapes: W recv rows + 1 reduced each
+    assert pool.stats.misses == distinct_keys
+    before = torch.cuda.memory_allocated()
+    one_pass(check=False)
+    torch.cuda.synchronize()
+    assert pool.stats.misses == distinct_keys
+    assert torch.cuda.memory_allocated() <= before
