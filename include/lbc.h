@@ -4,8 +4,9 @@
  * Plain pointers and sizes only; every pointer is a DEVICE pointer on the
  * current HIP device unless stated otherwise, every launch is asynchronous on
  * the `stream` argument (a hipStream_t passed as void*; NULL = the null
- * stream), nothing here allocates, frees, synchronises or keeps global state
- * besides a per-thread error string.  Inputs are never written.
+ * stream), nothing here allocates, frees or synchronises, and the only state is a
+ * per-thread error string and one process-wide tuning threshold
+ * (lbc_set_stream_min_bytes).  Inputs are never written.
  *
  * Wire format ("format A", the reference's portable codec,
  * ccdl_comm/quantization/torch_fallback.py:24-36): for a flat tensor of n
