@@ -2,7 +2,7 @@
 """Benchmark of the compression hot path on one MI355X.
 
 One "step" pushes one 100 MiB fp32 gradient bucket through the compressed reduce-scatter hot path
-of one rank at simulated world size 8 (BASELINE config 2): quantize+pack the bucket's 8 destination
+of one rank at simulated world size 8 (the "config 2" workload): quantize+pack the bucket's 8 destination
 chunks (one launch), then the fused dequant-reduce of the 8 peer payloads of this rank's shard in
 fixed rank order (one launch).  Peer payloads are synthesised in HBM before the timed region; there
 are no collectives.  `value` is GB/s of gradient input consumed per step.
