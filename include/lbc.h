@@ -87,18 +87,23 @@ int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residua
 
 /*
  * Quantize `world` equal destination chunks of one flat bucket in a single
- * launch.  Replaces the per-chunk loop of the compressed reduce-scatter
- * transport (ccdl_comm/communication/reduce_scatter_transport.py:252-276,
- * 499-519) over the chunk plan of ccdl_comm/cuda/transports/
+ * launch, optionally fused with error feedback exactly as lbc_quant_pack
+ * (residual, new_residual, restored are flat tensors of `numel` elements that
+ * are indexed like x).  Replaces the per-chunk loop of the compressed
+ * reduce-scatter transport (ccdl_comm/communication/reduce_scatter_transport.py:
+ * 252-276,499-519) over the chunk plan of ccdl_comm/cuda/transports/
  * compressed_reduce_scatter.py:72-94: shard_numel = ceil(numel/world); the
  * bucket is treated as zero padded to world*shard_numel; chunk d covers
  * [d*shard_numel, (d+1)*shard_numel) and its groups restart at its first
  * element.  Payload d is written packed at payloads + d*payload_stride:
  * int8 codes[Gs*g] then float scales[Gs], Gs = ceil(shard_numel/g).
- * payload_stride >= Gs*(g+4) and a multiple of 4.
+ * payload_stride >= Gs*(g+4) and a multiple of 4.  Pass residual =
+ * new_residual = restored = NULL (dtypes ignored) for a plain quantize.
  */
-int lbc_quant_pack_chunks(const void *x, int x_dtype, int64_t numel, int world, int group_size,
-                          uint8_t *payloads, int64_t payload_stride, void *stream);
+int lbc_quant_pack_chunks(const void *x, int x_dtype, const void *residual, int residual_dtype,
+                          int64_t numel, int world, int group_size, uint8_t *payloads,
+                          int64_t payload_stride, void *new_residual, int new_residual_dtype,
+                          void *restored, int restored_dtype, void *stream);
 
 /*
  * Decode one payload: out[i] (op)= float(code[i]) * scale[i/g], rounded to out_dtype.

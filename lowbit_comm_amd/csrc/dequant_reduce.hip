@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
         int64_t e0[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            e0[u] = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
+            e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
             const int64_t g = e0[u] / G;
 #pragma unroll
             for (int r = 0; r < W; ++r) {
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
 
     // ---- edge block: element-wise, stores guarded by numel ----------------------
     for (int u = 0; u < UNROLL; ++u) {
-        const int64_t e0 = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
+        const int64_t e0 = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
         for (int i = 0; i < VEC; ++i) {
             const int64_t e = e0 + i;
             if (e >= a.numel) break;
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
         int64_t e0[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            e0[u] = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
+            e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
             load_codes<VEC, MODE>(codes + e0[u], words[u]);
             scale[u] = scales[e0[u] / G];
         }
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
     }
 
     for (int u = 0; u < UNROLL; ++u) {
-        const int64_t e0 = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
+        const int64_t e0 = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
         for (int i = 0; i < VEC; ++i) {
             const int64_t e = e0 + i;
             if (e >= valid) break;

@@ -11,9 +11,22 @@ namespace lbc {
 using f16 = _Float16;
 using bf16 = __bf16;
 
+#ifndef LBC_BLOCK
+#define LBC_BLOCK 256
+#endif
+#ifndef LBC_TILE_ORDER
+#define LBC_TILE_ORDER 0
+#endif
 constexpr int kWave = 64;
-constexpr int kBlock = 256;
+constexpr int kBlock = LBC_BLOCK;
 constexpr int kWavesPerBlock = kBlock / kWave;
+
+// Index of the u-th tile a wavefront handles inside its block.  Order 0: the block's
+// wavefronts sweep the block's span together (tile = u * waves + wave); order 1: each
+// wavefront owns UNROLL consecutive tiles.
+template <int UNROLL> __device__ __forceinline__ int tile_in_block(int u, int wave) {
+    return LBC_TILE_ORDER == 0 ? u * kWavesPerBlock + wave : wave * UNROLL + u;
+}
 constexpr uint32_t kEpsBits = 0x34000000u;  // 2^-23, torch.finfo(float32).eps
 
 // Access modes of the bulk loads and stores.  kScalar: element by element (any

@@ -63,6 +63,61 @@ int finish(hipError_t err, const char *what) {
 
 }  // namespace
 
+namespace {
+
+// Shared body of lbc_quant_pack (world == 1, separate codes/scales pointers) and
+// lbc_quant_pack_chunks (world >= 1, packed rows).
+int quant_pack_common(const char *what, const void *x, int x_dtype, const void *residual, int residual_dtype,
+                      int64_t numel, int world, int group_size, uint8_t *codes_base, uint8_t *scales_base,
+                      int64_t payload_stride, int64_t shard_numel, void *new_residual, int new_residual_dtype,
+                      void *restored, int restored_dtype, bool rows_aligned, void *stream) {
+    const int r_dtype = residual ? residual_dtype : LBC_NONE;
+    const int p_dtype = residual ? promote(x_dtype, r_dtype) : x_dtype;
+    const bool wants_outputs = new_residual != nullptr || restored != nullptr;
+    int d_dtype = LBC_F32;
+    if (wants_outputs) {
+        if (!valid_dtype(restored_dtype)) return fail(LBC_EINVAL, "unsupported restored dtype %d", restored_dtype);
+        d_dtype = restored_dtype;
+        if (new_residual != nullptr) {
+            if (!valid_dtype(new_residual_dtype))
+                return fail(LBC_EINVAL, "unsupported new-residual dtype %d", new_residual_dtype);
+            if (new_residual_dtype != promote(p_dtype, d_dtype))
+                return fail(LBC_EINVAL, "new residual must have the promoted dtype of (input+residual) and restored");
+        }
+    }
+    if (r_dtype != LBC_NONE && r_dtype != LBC_F32 && r_dtype != x_dtype) return LBC_UNSUPPORTED;
+    if (d_dtype != LBC_F32 && d_dtype != x_dtype) return LBC_UNSUPPORTED;
+
+    const int vec = lbc::quant_pack_vec(x_dtype, r_dtype, d_dtype, wants_outputs);
+    bool aligned = rows_aligned && aligned_to(x, 16) && aligned_to(codes_base, vec) && payload_stride % vec == 0;
+    int64_t moved = numel * (dtype_size(x_dtype) + 1);
+    auto side = [&](const void *p, int dtype) {
+        if (p == nullptr) return;
+        aligned = aligned && aligned_to(p, 16) && (world == 1 || (shard_numel * dtype_size(dtype)) % 16 == 0);
+        moved += numel * dtype_size(dtype);
+    };
+    if (world > 1) aligned = aligned && (shard_numel * dtype_size(x_dtype)) % 16 == 0;
+    side(residual, r_dtype);
+    side(new_residual, new_residual_dtype);
+    side(restored, d_dtype);
+
+    lbc::QuantArgs a{};
+    a.x = x;
+    a.residual = residual;
+    a.codes_base = codes_base;
+    a.scales_base = scales_base;
+    a.new_residual = new_residual;
+    a.restored = restored;
+    a.numel = numel;
+    a.shard_numel = shard_numel;
+    a.payload_stride = payload_stride;
+    return finish(lbc::launch_quant_pack(x_dtype, r_dtype, d_dtype, wants_outputs, group_size,
+                                         pick_mode(aligned, moved), a, world, static_cast<hipStream_t>(stream)),
+                  what);
+}
+
+}  // namespace
+
 extern "C" {
 
 int lbc_abi_version(void) { return LBC_ABI_VERSION; }
@@ -88,54 +143,19 @@ int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residua
     if (codes == nullptr || scales == nullptr) return fail(LBC_EINVAL, "codes and scales must not be null");
     if (!aligned_to(scales, 4)) return fail(LBC_EINVAL, "scales must be 4-byte aligned");
     if (!aligned_to(x, dtype_size(x_dtype))) return fail(LBC_EINVAL, "input is not aligned to its element size");
-
-    const int r_dtype = residual ? residual_dtype : LBC_NONE;
-    const int p_dtype = residual ? promote(x_dtype, r_dtype) : x_dtype;
-    const bool wants_outputs = new_residual != nullptr || restored != nullptr;
-    int d_dtype = LBC_F32;
-    if (wants_outputs) {
-        if (!valid_dtype(restored_dtype)) return fail(LBC_EINVAL, "unsupported restored dtype %d", restored_dtype);
-        d_dtype = restored_dtype;
-        if (new_residual != nullptr) {
-            if (!valid_dtype(new_residual_dtype))
-                return fail(LBC_EINVAL, "unsupported new-residual dtype %d", new_residual_dtype);
-            if (new_residual_dtype != promote(p_dtype, d_dtype))
-                return fail(LBC_EINVAL, "new residual must have the promoted dtype of (input+residual) and restored");
-        }
-    }
-    if (r_dtype != LBC_NONE && r_dtype != LBC_F32 && r_dtype != x_dtype) return LBC_UNSUPPORTED;
-    if (d_dtype != LBC_F32 && d_dtype != x_dtype) return LBC_UNSUPPORTED;
-
-    const int vec = lbc::quant_pack_vec(x_dtype, r_dtype, d_dtype, wants_outputs);
-    bool aligned = aligned_to(x, 16) && aligned_to(codes, vec);
-    if (residual) aligned = aligned && aligned_to(residual, 16);
-    if (new_residual) aligned = aligned && aligned_to(new_residual, 16);
-    if (restored) aligned = aligned && aligned_to(restored, 16);
-    int64_t moved = numel * (dtype_size(x_dtype) + 1);
-    if (residual) moved += numel * dtype_size(r_dtype);
-    if (new_residual) moved += numel * dtype_size(new_residual_dtype);
-    if (restored) moved += numel * dtype_size(d_dtype);
-
-    lbc::QuantArgs a{};
-    a.x = x;
-    a.residual = residual;
-    a.codes_base = reinterpret_cast<uint8_t *>(codes);
-    a.scales_base = reinterpret_cast<uint8_t *>(scales);
-    a.new_residual = new_residual;
-    a.restored = restored;
-    a.numel = numel;
-    a.shard_numel = numel;
-    a.payload_stride = 0;
-    return finish(lbc::launch_quant_pack(x_dtype, r_dtype, d_dtype, wants_outputs, group_size,
-                                         pick_mode(aligned, moved), a, 1, static_cast<hipStream_t>(stream)),
-                  "lbc_quant_pack");
+    return quant_pack_common("lbc_quant_pack", x, x_dtype, residual, residual_dtype, numel, 1, group_size,
+                             reinterpret_cast<uint8_t *>(codes), reinterpret_cast<uint8_t *>(scales), 0, numel,
+                             new_residual, new_residual_dtype, restored, restored_dtype, true, stream);
 }
 
-int lbc_quant_pack_chunks(const void *x, int x_dtype, int64_t numel, int world, int group_size,
-                          uint8_t *payloads, int64_t payload_stride, void *stream) {
+int lbc_quant_pack_chunks(const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel,
+                          int world, int group_size, uint8_t *payloads, int64_t payload_stride, void *new_residual,
+                          int new_residual_dtype, void *restored, int restored_dtype, void *stream) {
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
     if (!valid_dtype(x_dtype)) return fail(LBC_EINVAL, "unsupported input dtype %d", x_dtype);
+    if (residual != nullptr && !valid_dtype(residual_dtype))
+        return fail(LBC_EINVAL, "unsupported residual dtype %d", residual_dtype);
     if (!valid_group(group_size)) return LBC_UNSUPPORTED;
     if (world > 65535) return LBC_UNSUPPORTED;
     const int64_t shard = (numel + world - 1) / world;
@@ -147,21 +167,9 @@ int lbc_quant_pack_chunks(const void *x, int x_dtype, int64_t numel, int world, 
         return fail(LBC_EINVAL, "payload_stride must be a multiple of 4 and >= %lld", (long long)payload_bytes);
     if (!aligned_to(payloads, 4)) return fail(LBC_EINVAL, "payloads must be 4-byte aligned");
     if (!aligned_to(x, dtype_size(x_dtype))) return fail(LBC_EINVAL, "input is not aligned to its element size");
-
-    const int vec = lbc::quant_pack_vec(x_dtype, LBC_NONE, LBC_F32, false);
-    const bool aligned = aligned_to(x, 16) && (shard * dtype_size(x_dtype)) % 16 == 0 && aligned_to(payloads, vec) &&
-                         payload_stride % vec == 0;
-    lbc::QuantArgs a{};
-    a.x = x;
-    a.codes_base = payloads;
-    a.scales_base = payloads + groups * group_size;
-    a.numel = numel;
-    a.shard_numel = shard;
-    a.payload_stride = payload_stride;
-    return finish(lbc::launch_quant_pack(x_dtype, LBC_NONE, LBC_F32, false, group_size,
-                                         pick_mode(aligned, numel * (dtype_size(x_dtype) + 1)), a, world,
-                                         static_cast<hipStream_t>(stream)),
-                  "lbc_quant_pack_chunks");
+    return quant_pack_common("lbc_quant_pack_chunks", x, x_dtype, residual, residual_dtype, numel, world, group_size,
+                             payloads, payloads + groups * group_size, payload_stride, shard, new_residual,
+                             new_residual_dtype, restored, restored_dtype, true, stream);
 }
 
 int lbc_dequant(const int8_t *codes, const float *scales, int64_t numel, int group_size, void *out,

@@ -18,7 +18,7 @@
 #include "launch.h"
 
 #ifndef LBC_QUANT_UNROLL
-#define LBC_QUANT_UNROLL 2
+#define LBC_QUANT_UNROLL 4
 #endif
 
 namespace lbc {
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
         int64_t e0[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            e0[u] = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
+            e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
             load_wide<XT, VEC, MODE>(x + e0[u], xv[u]);
             if constexpr (HAS_R) load_wide<RLoad, VEC, MODE>(r + e0[u], rv[u]);
         }
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
 
     // ---- edge block: ragged tail and zero padding, element-wise and guarded ----
     for (int u = 0; u < UNROLL; ++u) {
-        const int64_t e0 = block_first + static_cast<int64_t>(u * kWavesPerBlock + wave) * T::TILE + lane * VEC;
+        const int64_t e0 = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
         if (e0 - lane * VEC >= padded) break;  // wavefront-uniform
         float p[VEC];
 #pragma unroll

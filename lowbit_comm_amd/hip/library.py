@@ -27,7 +27,8 @@ SIGNATURES = {
     "lbc_set_stream_min_bytes": (_c_i64, [_c_i64]),
     "lbc_quant_pack": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_ptr, _c_ptr,
                                 _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr]),
-    "lbc_quant_pack_chunks": (_c_int, [_c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_ptr, _c_i64, _c_ptr]),
+    "lbc_quant_pack_chunks": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_ptr, _c_i64,
+                                       _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr]),
     "lbc_dequant": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
     "lbc_dequant_chunks": (_c_int, [_c_ptr, _c_i64, _c_int, _c_i64, _c_i64, _c_int, _c_ptr, _c_int, _c_ptr]),
     "lbc_dequant_reduce": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_ptr, _c_int,

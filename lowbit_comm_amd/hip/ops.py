@@ -134,6 +134,29 @@ def _finish(rc: int, lib) -> bool:
     raise RuntimeError(last_error(lib) or f"lbc call failed with code {rc}")
 
 
+def _side_tensors(x: torch.Tensor, residual, new_residual, restored, restored_dtype):
+    """Validate the optional error-feedback tensors of a quantize call; returns their dtype codes."""
+    device, n = x.device, x.numel()
+    r_code = _NONE
+    if residual is not None:
+        r_code = _float_tensor(residual, "residual", device)
+        _require(residual.numel() == n, "input and residual must have the same number of elements")
+    p_dtype = x.dtype if residual is None else promote(x.dtype, residual.dtype)
+    d_dtype = restored.dtype if restored is not None else (restored_dtype or torch.float32)
+    d_code = DTYPE_CODES.get(d_dtype)
+    _require(d_code is not None, f"restored dtype must be fp16, bf16 or fp32; got {d_dtype}")
+    n_code = _NONE
+    if restored is not None:
+        _float_tensor(restored, "restored", device)
+        _require(restored.numel() >= n, "restored must have at least input.numel() elements")
+    if new_residual is not None:
+        n_code = _float_tensor(new_residual, "new_residual", device)
+        _require(new_residual.numel() == n, "input and new_residual must have the same number of elements")
+        _require(new_residual.dtype == promote(p_dtype, d_dtype),
+                 f"new_residual must have dtype {promote(p_dtype, d_dtype)}")
+    return r_code, n_code, d_code
+
+
 # --------------------------------------------------------------------------- #
 # quantize + pack
 # --------------------------------------------------------------------------- #
@@ -160,23 +183,7 @@ def bind_quant_pack(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, 
     _require(scales.dtype == torch.float32, "scales must have float32 dtype")
     _require(codes.numel() == groups * group_size, "codes has an invalid quantized payload size")
     _require(scales.numel() == groups, "scales has an invalid group count")
-    r_code = _NONE
-    if residual is not None:
-        r_code = _float_tensor(residual, "residual", device)
-        _require(residual.numel() == n, "input and residual must have the same number of elements")
-    p_dtype = x.dtype if residual is None else promote(x.dtype, residual.dtype)
-    d_dtype = restored.dtype if restored is not None else (restored_dtype or torch.float32)
-    d_code = DTYPE_CODES.get(d_dtype)
-    _require(d_code is not None, f"restored dtype must be fp16, bf16 or fp32; got {d_dtype}")
-    n_code = _NONE
-    if restored is not None:
-        _float_tensor(restored, "restored", device)
-        _require(restored.numel() >= n, "restored must have at least input.numel() elements")
-    if new_residual is not None:
-        n_code = _float_tensor(new_residual, "new_residual", device)
-        _require(new_residual.numel() == n, "input and new_residual must have the same number of elements")
-        _require(new_residual.dtype == promote(p_dtype, d_dtype),
-                 f"new_residual must have dtype {promote(p_dtype, d_dtype)}")
+    r_code, n_code, d_code = _side_tensors(x, residual, new_residual, restored, restored_dtype)
     args = (_ptr(x), x_code, _ptr(residual), r_code, n, group_size, _ptr(codes), _ptr(scales),
             _ptr(new_residual), n_code, _ptr(restored), d_code)
     return BoundLaunch(lib.lbc_quant_pack, args, device, lib, (x, codes, scales, residual, new_residual, restored))
@@ -198,21 +205,33 @@ def quant_pack(x: torch.Tensor, *, group_size: int = 64, residual: torch.Tensor 
     return codes, scales
 
 
-def quant_pack_chunks_into(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64) -> bool:
-    """Quantize the ``world`` destination chunks of ``x`` into the rows of ``payloads`` (uint8 [world, stride])."""
-    return bind_quant_pack_chunks(x, payloads, world, group_size=group_size)()
+def quant_pack_chunks_into(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64,
+                           residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
+                           restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None) -> bool:
+    """Quantize the ``world`` destination chunks of ``x`` (+ ``residual``) into the rows of ``payloads``
+    (uint8 ``[world, stride]``) in one launch; optional fused error-feedback outputs as in
+    :func:`quant_pack_into`."""
+    return bind_quant_pack_chunks(x, payloads, world, group_size=group_size, residual=residual,
+                                  new_residual=new_residual, restored=restored, restored_dtype=restored_dtype)()
 
 
-def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64) -> BoundLaunch:
+def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64,
+                           residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
+                           restored: torch.Tensor | None = None,
+                           restored_dtype: torch.dtype | None = None) -> BoundLaunch:
     lib = load_library()
     x_code = _float_tensor(x, "input")
-    _device_tensor(payloads, "payloads", x.device)
+    device = x.device
+    n = x.numel()
+    _device_tensor(payloads, "payloads", device)
     _require(payloads.dtype == torch.uint8 and payloads.dim() == 2, "payloads must be a 2-D uint8 tensor")
     _require(payloads.shape[0] == world, "payloads must have one row per destination rank")
-    shard = -(-x.numel() // world)
+    shard = -(-n // world)
     _require(payloads.shape[1] >= payload_nbytes(shard, group_size), "payload rows are too small")
-    args = (_ptr(x), x_code, x.numel(), world, group_size, _ptr(payloads), payloads.stride(0))
-    return BoundLaunch(lib.lbc_quant_pack_chunks, args, x.device, lib, (x, payloads))
+    r_code, n_code, d_code = _side_tensors(x, residual, new_residual, restored, restored_dtype)
+    args = (_ptr(x), x_code, _ptr(residual), r_code, n, world, group_size, _ptr(payloads), payloads.stride(0),
+            _ptr(new_residual), n_code, _ptr(restored), d_code)
+    return BoundLaunch(lib.lbc_quant_pack_chunks, args, device, lib, (x, payloads, residual, new_residual, restored))
 
 
 # --------------------------------------------------------------------------- #

@@ -78,15 +78,23 @@ class ReduceScatterPlan:
         return [ops.split_payload(self.payload(rows, r), shard, g) for r in range(self.world_size)]
 
     # ---- compute steps ---------------------------------------------------------------------------
-    def quantize_chunks(self, tensor: torch.Tensor) -> torch.Tensor:
-        """Quantize the ``W`` destination chunks of ``tensor`` into ``self.send`` (one launch)."""
+    def quantize_chunks(self, tensor: torch.Tensor, *, residual: torch.Tensor | None = None,
+                        new_residual: torch.Tensor | None = None) -> torch.Tensor:
+        """Quantize the ``W`` destination chunks of ``tensor`` (+ ``residual``) into ``self.send`` (one launch).
+
+        With ``new_residual`` the same launch also stores what quantization dropped,
+        ``(tensor + residual) - decode(payload)``; it may be the ``residual`` tensor itself."""
         flat = tensor.reshape(-1)
         if flat.numel() != self.numel or flat.dtype != self.dtype:
             raise ValueError("tensor does not match the planned bucket")
-        bound = self._remember(("q", flat.data_ptr()), lambda: ops.bind_quant_pack_chunks(
-            flat, self.send, self.world_size, group_size=self.config.group_size))
+        key = ("q", flat.data_ptr(), None if residual is None else residual.data_ptr(),
+               None if new_residual is None else new_residual.data_ptr())
+        bound = self._remember(key, lambda: ops.bind_quant_pack_chunks(
+            flat, self.send, self.world_size, group_size=self.config.group_size,
+            residual=None if residual is None else residual.reshape(-1),
+            new_residual=None if new_residual is None else new_residual.reshape(-1)))
         if self.numel and not bound():
-            raise ValueError(f"no HIP quantize kernel for dtype {flat.dtype}")
+            raise ValueError(f"no HIP quantize kernel for dtype {flat.dtype} with this residual")
         return self.send
 
     def reduce_received(self, received: torch.Tensor | None = None, *, op: str = "sum",

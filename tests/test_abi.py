@@ -44,7 +44,8 @@ def test_argument_validation_happens_before_any_device_work():
     assert lib.lbc_dequant_reduce(none, none, 9, 64, 64, 1.0, none, 0, none, none, none) == 1          # > 8 payloads
     assert lib.lbc_dequant_reduce(none, none, 2, 64, 64, 0.0, none, 0, none, none, none) == -1
     assert library.last_error(lib) == "divisor must be > 0"
-    assert lib.lbc_quant_pack_chunks(none, 0, 640, 0, 64, none, 0, none) == -1
+    assert lib.lbc_quant_pack_chunks(none, 0, none, -1, 640, 0, 64, none, 0, none, -1, none, 0, none) == -1
+    assert library.last_error(lib) == "world must be > 0"
     assert lib.lbc_dequant(none, none, 64, 64, none, 0, 9, none) == -1
     previous = lib.lbc_set_stream_min_bytes(123)
     assert lib.lbc_set_stream_min_bytes(previous) == 123

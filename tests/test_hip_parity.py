@@ -424,6 +424,33 @@ def test_chunked_quantize_restarts_groups_per_chunk(ops, hip_device, n, world):
         assert np.array_equal(row, codec_np.pack(codes, scales)), f"chunk {d}"
 
 
+@pytest.mark.parametrize("grad_dtype,res_dtype", [("bf16", "fp32"), ("fp32", "fp32"), ("bf16", "bf16"), ("fp16", None)])
+@pytest.mark.parametrize("n,world", [(64 * 8 * 64, 8), (100_003, 4)])
+def test_chunked_quantize_with_fused_error_feedback(ops, hip_device, grad_dtype, res_dtype, n, world):
+    """One launch: p = g + r, every destination chunk of p quantized on its own, r' = p - decode(q) in place."""
+    grad = gradient_like(n, DTYPES[grad_dtype], 1400 + n, hip_device)
+    residual = None if res_dtype is None else gradient_like(n, DTYPES[res_dtype], 1401, hip_device, sigma=1e-5,
+                                                             outliers=False)
+    keep = None if residual is None else residual.clone()
+    p_dtype = grad.dtype if residual is None else ops.promote(grad.dtype, residual.dtype)
+    new_residual = residual if (residual is not None and residual.dtype == ops.promote(p_dtype, torch.float32)) \
+        else torch.empty(n, dtype=ops.promote(p_dtype, torch.float32), device=hip_device)
+    shard = -(-n // world)
+    nbytes = ops.payload_nbytes(shard)
+    stride = (nbytes + 15) // 16 * 16
+    payloads = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+    assert ops.quant_pack_chunks_into(grad, payloads, world, residual=residual, new_residual=new_residual)
+    prepared = grad.cpu() if keep is None else grad.cpu() + keep.cpu()
+    padded = torch.cat([prepared.float(), torch.zeros(shard * world - n)])
+    want_residual = torch.empty(shard * world)
+    for d in range(world):
+        chunk = padded[d * shard:(d + 1) * shard].to(prepared.dtype)
+        codes, scales = codec_torch.quantize(chunk, 64)
+        assert torch.equal(payloads[d, :nbytes].cpu(), codec_torch.pack(codes, scales)), f"chunk {d}"
+        want_residual[d * shard:(d + 1) * shard] = (chunk - codec_torch.dequantize(codes, scales, shard, 64, "fp32")).float()
+    assert_same_bits(new_residual, want_residual[:n].to(new_residual.dtype), "residual")
+
+
 def test_full_plan_config4_scaled(ops, hip_device):
     """Config 4 at 1/32 size: quantize 8 chunks per peer, reduce, requantize, decode all shards."""
     world, n = 8, 1_638_400 + 40          # ragged: shard = 204_805
