@@ -22,13 +22,15 @@
 namespace lbc {
 namespace {
 
-template <typename OT> struct decode_tiling {
-    static constexpr int VEC = sizeof(OT) == 4 ? 4 : 8;
-    static constexpr int TILE = kWave * VEC;
 #ifndef LBC_DECODE_UNROLL
 #define LBC_DECODE_UNROLL 1
 #endif
-    static constexpr int UNROLL = LBC_DECODE_UNROLL;
+// W payloads give 2*W loads per tile; with one or two payloads a second tile in
+// flight per wavefront is needed to cover the memory latency.
+template <typename OT, int W = 8> struct decode_tiling {
+    static constexpr int VEC = sizeof(OT) == 4 ? 4 : 8;
+    static constexpr int TILE = kWave * VEC;
+    static constexpr int UNROLL = W <= 2 ? 2 * LBC_DECODE_UNROLL : LBC_DECODE_UNROLL;
     static constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock * UNROLL;
 };
 
@@ -51,7 +53,7 @@ __device__ __forceinline__ void load_codes(const int8_t *__restrict__ p, uint32_
 // ---------------------------------------------------------------------------
 template <typename OT, int G, int W, int MODE>
 __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs a) {
-    using T = decode_tiling<OT>;
+    using T = decode_tiling<OT, W>;
     constexpr int VEC = T::VEC;
     constexpr int UNROLL = T::UNROLL;
 
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
 
 template <typename OT, int G, int W>
 hipError_t launch_reduce_w(int mode, const ReduceArgs &a, hipStream_t stream) {
-    using T = decode_tiling<OT>;
+    using T = decode_tiling<OT, W>;
     const int64_t blocks = (a.numel + T::BLOCK_ELEMS - 1) / T::BLOCK_ELEMS;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
@@ -179,9 +181,19 @@ template <int OP> __device__ __forceinline__ float combine(float old, float v) {
     else return v;
 }
 
+#ifndef LBC_DECODE1_UNROLL
+#define LBC_DECODE1_UNROLL 2
+#endif
+template <typename OT> struct decode1_tiling {
+    static constexpr int VEC = decode_tiling<OT>::VEC;
+    static constexpr int TILE = kWave * VEC;
+    static constexpr int UNROLL = LBC_DECODE1_UNROLL;   // a single payload has few loads per tile: keep more tiles in flight
+    static constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock * UNROLL;
+};
+
 template <typename OT, int G, int OP, int MODE>
 __global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
-    using T = decode_tiling<OT>;
+    using T = decode1_tiling<OT>;
     constexpr int VEC = T::VEC;
     constexpr int UNROLL = T::UNROLL;
 
@@ -236,7 +248,7 @@ __global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
 
 template <typename OT, int G, int OP>
 hipError_t launch_decode_op(int mode, const DecodeArgs &a, int world, hipStream_t stream) {
-    using T = decode_tiling<OT>;
+    using T = decode1_tiling<OT>;
     const int64_t blocks = (a.shard_numel + T::BLOCK_ELEMS - 1) / T::BLOCK_ELEMS;
     if (blocks == 0 || world == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL || world > 65535) return hipErrorInvalidValue;

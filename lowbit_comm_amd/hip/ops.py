@@ -117,11 +117,14 @@ class BoundLaunch:
         self._lib = lib
         self._keep = keep
 
-    def __call__(self) -> bool:
-        if self._device.index not in (None, torch.cuda.current_device()):
-            with _Launch(self._device) as stream:
-                return _finish(self._fn(*self._args, stream), self._lib)
-        stream = torch.cuda.current_stream(self._device).cuda_stream
+    def __call__(self, stream: int | None = None) -> bool:
+        """Enqueue.  ``stream``: raw ``hipStream_t`` handle (``torch.cuda.Stream.cuda_stream``) of a stream on
+        the tensors' device, which must be the current device; ``None`` looks up torch's current stream."""
+        if stream is None:
+            if self._device.index not in (None, torch.cuda.current_device()):
+                with _Launch(self._device) as guarded:
+                    return _finish(self._fn(*self._args, guarded), self._lib)
+            stream = torch.cuda.current_stream(self._device).cuda_stream
         rc = self._fn(*self._args, stream)
         return True if rc == LBC_OK else _finish(rc, self._lib)
 
