@@ -311,9 +311,7 @@ def main() -> int:
                     backend="hip", collective="reduce_scatter", strategy="compressed", shape_class=(world, stride),
                     dtype="uint8", world_size=world, bit=8, group_size=G, chunk_config=(size,), workspace_kind="send",
                     device=str(dev))
-            lease = provider.pool.acquire(key, stream)
-            session._leases.append(lease)
-            return lease.buffer
+            return session.acquire(key)
 
         bound_cache = {}
         raw_stream = stream.cuda_stream

@@ -488,6 +488,12 @@ class ShardWorkspaceSession:
         self._leases.append(lease)
         return lease.buffer
 
+    def acquire(self, key: WorkspaceKey) -> Any:
+        """Lease a buffer for an explicit key on this session's stream; released with the others."""
+        lease = self._provider.pool.acquire(key, self._stream)
+        self._leases.append(lease)
+        return lease.buffer
+
     def _payload_bytes(self, tensor: Any, config: CompressionConfig, dtype: str) -> int:
         return estimate_quantized_size(int(tensor.numel()), dtype=dtype, config=config,
                                        wire_format="portable").quantized_bytes

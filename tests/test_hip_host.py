@@ -497,3 +497,48 @@ def test_llama_shaped_bucket_stream_through_the_pool(dev):
     torch.cuda.synchronize()
     assert pool.stats.misses == distinct_keys
     assert torch.cuda.memory_allocated() <= before
+
+
+# --------------------------------------------------------------------------- #
+# HIP graph capture: the launches allocate nothing and never synchronise, so a bucket step can be captured
+# --------------------------------------------------------------------------- #
+def test_bucket_step_replays_from_a_hip_graph(dev):
+    from lowbit_comm_amd.hip import ops
+    from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
+
+    n, world = 64 * 8 * 500, 8
+    plan = ReduceScatterPlan(n, torch.float32, world_size=world, rank=0, config=CFG, device=dev)
+    bucket = torch.zeros(n, device=dev)
+    residual = torch.zeros(n, device=dev)
+    peers = [grad(n, torch.float32, 1500 + r, dev) for r in range(world)]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                      # warm up on a side stream, as graph capture requires
+        plan.quantize_chunks(bucket, residual=residual, new_residual=residual)
+        plan.reduce_received(op="mean")
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.quantize_chunks(bucket, residual=residual, new_residual=residual)
+        plan.reduce_received(op="mean")
+    cpu_residual = torch.zeros(n)
+    shard = n // world
+    for step in range(4):                              # replays interleaved with eager work and synchronisation
+        g = grad(n, torch.float32, 1600 + step, dev)
+        bucket.copy_(g)
+        for src in range(world):                        # synthetic exchange: peers' chunk 0 payloads
+            row = plan.received[src, :plan.payload_bytes]
+            assert ops.quant_pack_payload_into(peers[src][:shard] * (1.0 + 0.01 * step), row)
+        if step == 0:
+            residual.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        prepared = g.cpu() + cpu_residual
+        want_rows = [codec_torch.quantize(prepared[d * shard:(d + 1) * shard]) for d in range(world)]
+        for d in range(world):
+            assert torch.equal(plan.send[d, :plan.payload_bytes].cpu(), codec_torch.pack(*want_rows[d])), (step, d)
+        cpu_residual = prepared - torch.cat([codec_torch.dequantize(c, s, shard) for c, s in want_rows])
+        assert same_bits(residual, cpu_residual), step
+        received = [codec_torch.quantize(peers[src][:shard].cpu() * (1.0 + 0.01 * step)) for src in range(world)]
+        assert same_bits(plan.shard, codec_torch.reduce_payloads(received, shard, 64, "fp32", "mean")), step
