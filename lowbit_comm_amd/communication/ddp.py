@@ -7,7 +7,6 @@ with ``fused=True`` and no collective the whole local round trip is a single ker
 from __future__ import annotations
 
 from collections.abc import Callable, Hashable
-from dataclasses import dataclass, field
 from typing import Any
 
 from lowbit_comm_amd.communication.collectives import CompressedAllReduce, CompressedPayload
@@ -27,63 +26,73 @@ def bucket_tensor(bucket: Any) -> Any:
     return buffer()
 
 
-@dataclass
 class DDPBucketProcessor:
-    config: CompressionConfig
-    quantize: Callable[[Any, CompressionConfig], Any]
-    dequantize: Callable[[Any, tuple[int, ...], CompressionConfig, str], Any]
-    all_reduce: Callable[[CompressedPayload, str], CompressedPayload] | None = None
-    error_feedback: ErrorFeedbackState = field(default_factory=ErrorFeedbackState)
-    fused_codec: Any | None = None  # a FusedErrorFeedbackCodec, used when there is no collective
+    """One bucket at a time: ``compensate -> quantize -> [all_reduce] -> dequantize -> residual update``.
 
+    ``quantize(tensor, config)`` and ``dequantize(payload, shape, config, dtype)`` are positional callables;
+    ``all_reduce(payload, op)`` is optional (``None`` = local round trip); ``fused_codec`` (a
+    ``FusedErrorFeedbackCodec``) replaces the whole local round trip by one kernel.
+    """
+
+    def __init__(self, config: CompressionConfig, quantize: Callable[[Any, CompressionConfig], Any],
+                 dequantize: Callable[[Any, tuple[int, ...], CompressionConfig, str], Any],
+                 all_reduce: Callable[[CompressedPayload, str], CompressedPayload] | None = None,
+                 error_feedback: ErrorFeedbackState | None = None, fused_codec: Any | None = None) -> None:
+        self.config = config
+        self.quantize = quantize
+        self.dequantize = dequantize
+        self.all_reduce = all_reduce
+        self.error_feedback = ErrorFeedbackState() if error_feedback is None else error_feedback
+        self.fused_codec = fused_codec
+
+    # ---- constructors ----------------------------------------------------------------------------
     @classmethod
     def from_cuda_codec(cls, config: CompressionConfig, *, extension_status: Any | None = None,
                         error_feedback: ErrorFeedbackState | None = None) -> "DDPBucketProcessor":
-        """Bind the codec facade (flat ``uint8`` buffers) - the reference's constructor name."""
-        from lowbit_comm_amd.quantization.codec import dequantize_tensor, quantize_tensor
+        """Codec facade with flat ``uint8`` buffers (the reference's constructor name)."""
+        from lowbit_comm_amd.quantization import codec
 
-        def quantize(tensor: Any, active: CompressionConfig) -> Any:
-            return quantize_tensor(tensor, active, extension_status=extension_status)
-
-        def dequantize(payload: Any, shape: tuple[int, ...], active: CompressionConfig, dtype: str) -> Any:
-            return dequantize_tensor(payload, shape, active, dtype=dtype, extension_status=extension_status)
-
-        return cls(config=config, quantize=quantize, dequantize=dequantize,
-                   error_feedback=error_feedback or ErrorFeedbackState())
+        return cls(
+            config,
+            quantize=lambda tensor, active: codec.quantize_tensor(tensor, active, extension_status=extension_status),
+            dequantize=lambda payload, shape, active, dtype: codec.dequantize_tensor(
+                payload, shape, active, dtype=dtype, extension_status=extension_status),
+            error_feedback=error_feedback,
+        )
 
     @classmethod
     def from_hip_codec(cls, config: CompressionConfig, *, error_feedback: ErrorFeedbackState | None = None,
                        fused: bool = True) -> "DDPBucketProcessor":
-        """Bind the GPU codec callables; ``fused`` runs the local round trip as one kernel per bucket."""
-        from lowbit_comm_amd.hip.codec import FusedErrorFeedbackCodec, dequantize_tensor_hip, quantize_tensor_hip
+        """GPU codec callables; with ``fused`` the local round trip is one kernel per bucket."""
+        from lowbit_comm_amd.hip import codec as hip_codec
 
-        state = error_feedback or ErrorFeedbackState()
-        return cls(config=config, quantize=quantize_tensor_hip, dequantize=dequantize_tensor_hip,
-                   error_feedback=state,
-                   fused_codec=FusedErrorFeedbackCodec(config, error_feedback=state) if fused else None)
+        state = ErrorFeedbackState() if error_feedback is None else error_feedback
+        one_kernel = hip_codec.FusedErrorFeedbackCodec(config, error_feedback=state) if fused else None
+        return cls(config, hip_codec.quantize_tensor_hip, hip_codec.dequantize_tensor_hip, error_feedback=state,
+                   fused_codec=one_kernel)
 
-    def process(self, bucket: Any, *, dtype: str) -> Any:
-        key = bucket_key(bucket)
-        original = bucket_tensor(bucket)
-        use_feedback = self.config.error_feedback
-
-        if self.all_reduce is None and self.fused_codec is not None:
-            _payload, restored = self.fused_codec.step(key, original, dtype, update=use_feedback, apply=use_feedback)
-            return restored
-
-        prepared = self.error_feedback.compensate(key, original) if use_feedback else original
+    # ---- the step ----------------------------------------------------------------------------------
+    def _round_trip(self, prepared: Any, dtype: str) -> Any:
         shape = tuple(getattr(prepared, "shape", ()))
         if self.all_reduce is None:
-            restored = self.dequantize(self.quantize(prepared, self.config), shape, self.config, dtype)
-        else:
-            restored = CompressedAllReduce(
-                config=self.config,
-                compress=lambda tensor, active: CompressedPayload(
-                    buffer=self.quantize(tensor, active), shape=tuple(getattr(tensor, "shape", ())), dtype=dtype),
-                all_reduce=self.all_reduce,
-                decompress=lambda payload, active: self.dequantize(payload.buffer, payload.shape, active,
-                                                                   payload.dtype),
-            ).run(prepared, op="sum")
-        if use_feedback:
+            return self.dequantize(self.quantize(prepared, self.config), shape, self.config, dtype)
+
+        def compress(tensor: Any, active: CompressionConfig) -> CompressedPayload:
+            return CompressedPayload(buffer=self.quantize(tensor, active), shape=tuple(getattr(tensor, "shape", ())),
+                                     dtype=dtype)
+
+        def decompress(payload: CompressedPayload, active: CompressionConfig) -> Any:
+            return self.dequantize(payload.buffer, payload.shape, active, payload.dtype)
+
+        return CompressedAllReduce(self.config, compress, self.all_reduce, decompress).run(prepared, op="sum")
+
+    def process(self, bucket: Any, *, dtype: str) -> Any:
+        key, original = bucket_key(bucket), bucket_tensor(bucket)
+        feedback_on = self.config.error_feedback
+        if self.all_reduce is None and self.fused_codec is not None:
+            return self.fused_codec.step(key, original, dtype, update=feedback_on, apply=feedback_on)[1]
+        prepared = self.error_feedback.compensate(key, original) if feedback_on else original
+        restored = self._round_trip(prepared, dtype)
+        if feedback_on:
             self.error_feedback.update(key, original=prepared, transmitted=restored)
         return restored

@@ -1,26 +1,29 @@
-"""Compression policy.  Field names, defaults and validation messages mirror the reference's
-``ccdl_comm/config.py:22-77`` so configs move between the two packages unchanged."""
+"""``CompressionConfig`` - the user-facing compression policy.
+
+Fields, defaults and the wording of validation errors follow the reference's dataclass
+(``ccdl_comm/config.py:22-77``), so a config written for either package constructs in both.  The HIP
+kernels implement the default policy (linear, 8 bit, group 16/32/64, no top-k, deterministic
+rounding); other valid policies are reported as unsupported by the codec, not rejected here.
+"""
 from __future__ import annotations
 
 from dataclasses import dataclass
 
-_CHOICES = {
-    "bit": (4, 8),
-    "group_size": (16, 32, 64),
-    "topk": (0, 1, 2),
-}
-_NAMED_CHOICES = {
+# field -> allowed values; the first table prints values bare, the second quoted (as the reference does)
+_NUMERIC_DOMAINS = {"bit": (4, 8), "group_size": (16, 32, 64), "topk": (0, 1, 2)}
+_NAMED_DOMAINS = {
     "quant_type": ("e2m1", "e3m0", "linear", "normal", "uniform"),
     "target": ("collective", "ddp_gradient_bucket", "p2p", "tensor"),
     "error_feedback_policy": ("always", "large_bucket_only", "none", "periodic", "warmup_then_enable"),
 }
-_STABLE_BITS = (8,)
+_NON_EXPERIMENTAL_BITS = frozenset({8})
+_LOWER_BOUNDS = (("error_feedback_min_numel", 0, "must be >= 0"),
+                 ("error_feedback_warmup_steps", 0, "must be >= 0"),
+                 ("error_feedback_period", 1, "must be > 0"))
 
 
 @dataclass(frozen=True)
 class CompressionConfig:
-    """User-facing compression policy; the default is linear 8-bit, group 64, error feedback on."""
-
     bit: int = 8
     group_size: int = 64
     topk: int = 0
@@ -38,23 +41,20 @@ class CompressionConfig:
     error_feedback_period: int = 1
 
     def __post_init__(self) -> None:
-        for name, allowed in _CHOICES.items():
+        for name, domain in _NUMERIC_DOMAINS.items():
             value = getattr(self, name)
-            if value not in allowed:
-                raise ValueError(f"Unsupported {name}={value}; expected one of {sorted(allowed)}")
-            if name == "bit" and value not in _STABLE_BITS and not self.allow_experimental:
-                raise ValueError(f"bit={value} is experimental; set allow_experimental=True to opt in")
-        for name, allowed in _NAMED_CHOICES.items():
+            if value not in domain:
+                raise ValueError(f"Unsupported {name}={value}; expected one of {sorted(domain)}")
+        if self.bit not in _NON_EXPERIMENTAL_BITS and not self.allow_experimental:
+            raise ValueError(f"bit={self.bit} is experimental; set allow_experimental=True to opt in")
+        for name, domain in _NAMED_DOMAINS.items():
             value = getattr(self, name)
-            if value not in allowed:
-                raise ValueError(f"Unsupported {name}={value!r}; expected one of {sorted(allowed)}")
-        if self.error_feedback_min_numel < 0:
-            raise ValueError("error_feedback_min_numel must be >= 0")
-        if self.error_feedback_warmup_steps < 0:
-            raise ValueError("error_feedback_warmup_steps must be >= 0")
-        if self.error_feedback_period <= 0:
-            raise ValueError("error_feedback_period must be > 0")
+            if value not in domain:
+                raise ValueError(f"Unsupported {name}={value!r}; expected one of {sorted(domain)}")
+        for name, minimum, rule in _LOWER_BOUNDS:
+            if getattr(self, name) < minimum:
+                raise ValueError(f"{name} {rule}")
 
     def effective_error_feedback_policy(self) -> str:
-        """``"none"`` when error feedback is switched off, else the configured policy."""
+        """The configured policy, or ``"none"`` when ``error_feedback`` is off."""
         return self.error_feedback_policy if self.error_feedback else "none"

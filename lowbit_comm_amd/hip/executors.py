@@ -9,7 +9,7 @@ divide -> residual update and records why.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, replace
+from dataclasses import dataclass
 from math import prod
 from typing import Any
 
@@ -86,12 +86,9 @@ class PrecollectedPayloadExecutor:
         estimate = estimate_quantized_size(numel, dtype=dtype, config=config, wire_format=wire_format)
         self.expected_payload_bytes = estimate.quantized_bytes
         self._static_reason = fused_dequant_fallback_reason(config)
-        self.execution_info = ExecutionInfo(
-            requested_strategy="all_gather", executed_strategy="all_gather", backend="hip", fallback_used=False,
-            fallback_reason=None, stage_names=("dequant_reduce_mean_ef",), original_bytes=estimate.original_bytes,
-            compressed_bytes=estimate.quantized_bytes,
-            compression_ratio=estimate.compression_ratio if estimate.compression_ratio > 0 else 1.0,
-            workspace_cache_hit=True, async_capable=False, fast_path=FUSED_FAST_PATH)
+        self.execution_info = ExecutionInfo.for_fused_path(
+            strategy="all_gather", fast_path=FUSED_FAST_PATH, stage="dequant_reduce_mean_ef",
+            original_bytes=estimate.original_bytes, compressed_bytes=estimate.quantized_bytes)
         self.last_execution_info = self.execution_info
         self.execution_counters = ExecutionCounters()
 
@@ -132,7 +129,6 @@ class PrecollectedPayloadExecutor:
         if execution.fused:
             self.last_execution_info = self.execution_info
         else:
-            self.last_execution_info = replace(self.execution_info, fallback_used=True,
-                                               fallback_reason=execution.fallback_reason, fast_path="python_fallback")
+            self.last_execution_info = self.execution_info.with_fallback(execution.fallback_reason)
         self.execution_counters._record_completed()
         return execution.output

@@ -56,6 +56,22 @@ class ErrorFeedbackState:
         else:
             self._residuals.pop(key, None)
 
+    def keys(self) -> list[Hashable]:
+        """Bucket keys that currently hold a residual."""
+        return list(self._residuals)
+
+    def __len__(self) -> int:
+        return len(self._residuals)
+
+    def state_dict(self) -> dict[Hashable, Any]:
+        """Residuals by bucket key, for the host framework's checkpoint (the tensors themselves, not copies)."""
+        return dict(self._residuals)
+
+    def load_state_dict(self, state: dict[Hashable, Any]) -> None:
+        """Replace all residuals with ``state`` (as produced by :meth:`state_dict`)."""
+        self._residuals.clear()
+        self._residuals.update(state)
+
     def __eq__(self, other: object) -> bool:
         return isinstance(other, ErrorFeedbackState) and self._residuals == other._residuals
 

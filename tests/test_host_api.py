@@ -608,3 +608,23 @@ def test_strategies_without_an_injected_transport_are_unsupported():
     assert hook._ccdl_effective_strategy == "reduce_scatter"
     assert hook(None, Bucket(torch.ones(4))).value == "RS"
     assert calls[0]["op"] == "mean" and calls[0]["dtype"] == "fp32" and calls[0]["async_op"] is False
+
+
+def test_error_feedback_state_checkpoint_round_trip():
+    state = ErrorFeedbackState()
+    state.put("a", torch.ones(3))
+    state.put(7, torch.zeros(2))
+    saved = state.state_dict()
+    assert sorted(map(str, state.keys())) == ["7", "a"] and len(state) == 2
+    other = ErrorFeedbackState()
+    other.load_state_dict(saved)
+    assert torch.equal(other.get("a"), torch.ones(3)) and other.get(7) is saved[7]
+
+
+def test_payload_conveniences():
+    p = _payload([1, 2, 3, 4], [1.0, 2.0])
+    assert p.original_numel == 4
+    assert CompressedPayload(buffer=None, shape=(2, 3), dtype="fp32").original_numel == 6
+    q = Quantizer(CompressionConfig(), dtype="bf16")
+    assert q.payload_bytes(128) == 136 and q.payload_bytes(128, wire_format="native") == 132
+    assert "group_size=64" in repr(q)
