@@ -171,7 +171,7 @@ def create_ddp_comm_hook(
         return dequantize_tensor(_buffer_of(payload), shape, active, dtype=active_dtype,
                                  extension_status=extension_status)
 
-    feedback = error_feedback or ErrorFeedbackState()
+    feedback = ErrorFeedbackState() if error_feedback is None else error_feedback
     policy = ErrorFeedbackPolicy(config)
     uncompressed = bypass_all_reduce or _single_process_all_reduce
     inplace_reduce_feedback = (native_inplace_dequantize_reduce_update_feedback
