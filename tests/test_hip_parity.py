@@ -180,6 +180,38 @@ def test_quantize_is_idempotent_and_scale_equivariant_at_full_size(ops, hip_devi
     assert bool((err <= scales[:, None] * 0.50005).all())
 
 
+def test_more_than_2_to_the_31_elements(ops, hip_device):
+    """Indexing is 64-bit: a 4.3 GB bf16 tensor with a ragged tail; group-aligned windows at the start, across
+    the 2^31 boundary and at the tail are compared with the oracle (quantization is local to a group)."""
+    n = (1 << 31) + 64 * 1000 + 5
+    x = torch.empty(n, dtype=torch.bfloat16, device=hip_device)
+    step = 1 << 28
+    for i, a in enumerate(range(0, n, step)):
+        b = min(a + step, n)
+        gen = torch.Generator(device=hip_device).manual_seed(4242 + i)
+        x[a:b] = (torch.randn(b - a, generator=gen, device=hip_device) * 1e-3).to(torch.bfloat16)
+    codes, scales = ops.quant_pack(x)
+    assert codes.numel() == ops.num_groups(n, 64) * 64 and scales.numel() == ops.num_groups(n, 64)
+    restored = ops.dequant(codes, scales, n, dtype=torch.bfloat16)
+    windows = [(0, 1 << 20), ((1 << 31) - 64 * 2000, (1 << 31) + 64 * 500), (n - 64 * 3000 - 5, n)]
+    for a, b in windows:
+        assert a % 64 == 0
+        w_codes, w_scales = codec_torch.quantize(x[a:b].cpu(), 64)
+        padded = ops.num_groups(b - a, 64) * 64
+        assert torch.equal(codes[a:a + padded].cpu(), w_codes), (a, b)
+        assert_same_bits(scales[a // 64:a // 64 + padded // 64], w_scales, f"scales {a}")
+        assert_same_bits(restored[a:b], codec_torch.dequantize(w_codes, w_scales, b - a, 64, "bf16"), f"restored {a}")
+    del restored
+    # W=2 reduce across the boundary: x + x decodes to exactly twice the single decode
+    out = torch.empty(n, dtype=torch.float32, device=hip_device)
+    assert ops.dequant_reduce_into([(codes, scales), (codes, scales)], out)
+    a, b = windows[1]
+    single = codec_torch.dequantize(codes[a:b].cpu(), scales[a // 64:b // 64].cpu(), b - a, 64, "fp32")
+    assert_same_bits(out[a:b], single + single, "reduce across 2^31")
+    assert_same_bits(out[n - 1000:], codec_torch.dequantize(codes[windows[2][0]:].cpu(), scales[windows[2][0] // 64:].cpu(),
+                                                            n - windows[2][0], 64, "fp32")[-1000:] * 2, "reduce tail")
+
+
 # --------------------------------------------------------------------------- #
 # decode and fused dequant-reduce
 # --------------------------------------------------------------------------- #
