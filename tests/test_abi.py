@@ -68,3 +68,25 @@ def test_scale_formula_is_exact_for_every_finite_float(tmp_path):
     assert done.returncode == 0, done.stdout
     assert "mismatches with result >= 2^-24: 0 ; below (clamped region): 0" in done.stdout
     assert "0x3C010204" in done.stdout
+
+
+def test_device_code_has_no_instruction_that_changes_the_rounding_contract(tmp_path):
+    """The parity argument rests on build flags: products and sums round separately.  Compile the two kernel
+    files to assembly with the Makefile's flags and check that no packed-fp32 arithmetic and no
+    fused multiply-convert (`v_fma_mix*`, which rounds a product straight to fp16) was selected."""
+    makefile = (ROOT / "lowbit_comm_amd" / "csrc" / "Makefile").read_text()
+    flags = re.search(r"HIPFLAGS\s*:=\s*((?:.*\\\n)*.*)", makefile).group(1).replace("\\\n", " ").split()
+    flags = [f.replace("$(ARCH)", "gfx950") for f in flags if f != "-fPIC"]
+    assert "-ffp-contract=off" in flags
+    procs = []
+    for name in ("quant_pack", "dequant_reduce"):
+        out = tmp_path / f"{name}.s"
+        procs.append((out, subprocess.Popen(
+            ["/opt/rocm/bin/hipcc", *flags, "--cuda-device-only", "-S", str(ROOT / "lowbit_comm_amd" / "csrc" / f"{name}.hip"),
+             "-o", str(out)], stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)))
+    for out, proc in procs:
+        assert proc.wait(timeout=900) == 0
+        text = out.read_text()
+        assert "gfx950" in text
+        for forbidden in ("v_fma_mix", "v_mad_mix", "v_pk_mul_f32", "v_pk_add_f32", "v_pk_fma_f32"):
+            assert forbidden not in text, (out.name, forbidden)

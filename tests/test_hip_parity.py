@@ -509,3 +509,55 @@ def test_full_plan_config4_scaled(ops, hip_device):
     for d in range(world):
         assert np.array_equal(shards[d].cpu().numpy().view(np.uint32), want_shards[d].view(np.uint32)), f"shard {d}"
     assert np.array_equal(restored.cpu().numpy().view(np.uint32), want_restored.view(np.uint32))
+
+
+# --------------------------------------------------------------------------- #
+# randomized sweep over shapes, dtypes, groups, alignments and payload counts
+# --------------------------------------------------------------------------- #
+def test_randomized_parity_sweep(ops, hip_device):
+    rng = np.random.default_rng(20261125)
+    names = ["fp32", "fp16", "bf16"]
+    for case in range(60):
+        g = int(rng.choice([16, 32, 64]))
+        n = int(rng.integers(1, 200_000))
+        x_name = names[int(rng.integers(0, 3))]
+        offset = int(rng.integers(0, 4))                     # element offset: exercises unaligned base pointers
+        sigma = float(10.0 ** rng.uniform(-6, 2))
+        base = gradient_like(n + offset, DTYPES[x_name], 5000 + case, hip_device, sigma=sigma)
+        x = base[offset:]
+        label = f"case {case}: n={n} g={g} {x_name} offset={offset} sigma={sigma:.3g}"
+        # plain quantize + decode to a random dtype
+        codes, scales = ops.quant_pack(x, group_size=g)
+        w_codes, w_scales = codec_torch.quantize(x.cpu(), g)
+        assert torch.equal(codes.cpu(), w_codes), label
+        assert_same_bits(scales, w_scales, label)
+        o_name = names[int(rng.integers(0, 3))]
+        assert_same_bits(ops.dequant(codes, scales, n, group_size=g, dtype=DTYPES[o_name]),
+                         codec_torch.dequantize(w_codes, w_scales, n, g, o_name), label + f" decode {o_name}")
+        # fused error feedback with a residual of a supported dtype
+        r_name = [None, "fp32", x_name][int(rng.integers(0, 3))]
+        d_name = ["fp32", x_name][int(rng.integers(0, 2))]
+        residual = None if r_name is None else gradient_like(n, DTYPES[r_name], 6000 + case, hip_device, sigma=sigma * 1e-2)
+        p_dtype = x.dtype if residual is None else ops.promote(x.dtype, residual.dtype)
+        new_residual = torch.empty(n, dtype=ops.promote(p_dtype, DTYPES[d_name]), device=hip_device)
+        restored = torch.empty(n, dtype=DTYPES[d_name], device=hip_device)
+        groups = ops.num_groups(n, g)
+        c2 = torch.empty(groups * g, dtype=torch.int8, device=hip_device)
+        s2 = torch.empty(groups, dtype=torch.float32, device=hip_device)
+        assert ops.quant_pack_into(x, c2, s2, group_size=g, residual=residual, new_residual=new_residual,
+                                   restored=restored), label
+        e_codes, e_scales, e_restored, e_residual = codec_torch.ef_round_trip(
+            x.cpu(), None if residual is None else residual.cpu(), g, d_name)
+        assert torch.equal(c2.cpu(), e_codes), label + " ef codes"
+        assert_same_bits(s2, e_scales, label + " ef scales")
+        assert_same_bits(restored, e_restored, label + " ef restored")
+        assert_same_bits(new_residual, e_residual, label + " ef residual")
+        # fused reduce of W payloads of this shape
+        world = int(rng.integers(1, 9))
+        payloads = [(codes, scales)] + [ops.quant_pack(gradient_like(n, torch.float32, 7000 + 10 * case + r, hip_device,
+                                                                     sigma=sigma), group_size=g) for r in range(world - 1)]
+        mode = ["sum", "mean"][int(rng.integers(0, 2))]
+        out = torch.empty(n, dtype=DTYPES[o_name], device=hip_device)
+        assert ops.dequant_reduce_into(payloads, out, group_size=g, divisor=float(world) if mode == "mean" else 1.0), label
+        want = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in payloads], n, g, o_name, mode)
+        assert_same_bits(out, want, label + f" reduce W={world} {mode} {o_name}")
