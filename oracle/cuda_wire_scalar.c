@@ -1,0 +1,204 @@
+/*
+ * Scalar C restatement of the reference's CUDA wire format.  TEST INFRASTRUCTURE ONLY.
+ *
+ * One element at a time, reading and writing payload bytes at the offsets the
+ * reference kernels compute, with hand-written fp16/bf16 conversions so that
+ * nothing is shared with the numpy restatement.  Compiled with
+ * -ffp-contract=off; the fused multiply-add variant of the reduce calls fmaf
+ * explicitly.  The product never links this file.
+ *
+ * Reference lines followed (paths under the upstream repository):
+ *   lbw_quantize    ccdl_comm/csrc/quantization/quant_pack_kernel.cu:45-162
+ *                   (non-compact offsets: quant_kernel_fp32.cuh:266-303)
+ *   lbw_dequantize  ccdl_comm/csrc/quantization/dequant_kernel_fp32.cuh:81-120,
+ *                   dequant_kernel.cuh:15-60
+ *   lbw_reduce      ccdl_comm/csrc/quantization/dequant_reduce_kernel.cu:27-134,150-221
+ *
+ * dtype: 0 fp32, 1 fp16, 2 bf16 (16-bit values travel as uint16 bit patterns).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+
+enum { LBW_F32 = 0, LBW_F16 = 1, LBW_BF16 = 2 };
+
+static float bits_to_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static uint32_t f32_to_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+static float bf16_to_f32(uint16_t h) { return bits_to_f32((uint32_t)h << 16); }
+static uint16_t f32_to_bf16(float f) {
+    uint32_t u = f32_to_bits(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+static float f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    if (exp == 0x1Fu) return bits_to_f32(sign | 0x7F800000u | (man << 13));
+    if (exp == 0) {
+        float v = (float)man * 0x1p-24f; /* subnormal: man * 2^-24, exact */
+        return sign ? -v : v;
+    }
+    return bits_to_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+static uint16_t f32_to_f16(float f) { /* round to nearest, ties to even */
+    uint32_t u = f32_to_bits(f);
+    uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u | ((a >> 13) & 0x3FFu));
+    if (a >= 0x47800000u) return (uint16_t)(sign | 0x7C00u);          /* >= 65536 (incl. inf) */
+    if (a < 0x38800000u) {                                            /* below the smallest normal half */
+        float scaled = fabsf(f) * 0x1p24f;                            /* exact scaling; < 1024 */
+        float r = rintf(scaled);                                      /* nearest-even in units of 2^-24 */
+        return (uint16_t)(sign | (uint16_t)r);                        /* r == 1024 lands on the first normal */
+    }
+    uint32_t lsb = (a >> 13) & 1u;
+    a += 0xFFFu + lsb;
+    uint32_t h = (a >> 13) - (112u << 10);
+    if (h >= 0x7C00u) h = 0x7C00u;                                    /* rounded up to infinity */
+    return (uint16_t)(sign | h);
+}
+
+static int item_size(int dtype) { return dtype == LBW_F32 ? 4 : 2; }
+
+static float load_as_f32(const void *base, int64_t index, int dtype) {
+    if (dtype == LBW_F32) return ((const float *)base)[index];
+    uint16_t h = ((const uint16_t *)base)[index];
+    return dtype == LBW_F16 ? f16_to_f32(h) : bf16_to_f32(h);
+}
+
+static float round_to(float v, int dtype) {
+    if (dtype == LBW_F16) return f16_to_f32(f32_to_f16(v));
+    if (dtype == LBW_BF16) return bf16_to_f32(f32_to_bf16(v));
+    return v;
+}
+
+static void store_from_f32(void *base, int64_t index, int dtype, float v) {
+    if (dtype == LBW_F32) ((float *)base)[index] = v;
+    else ((uint16_t *)base)[index] = dtype == LBW_F16 ? f32_to_f16(v) : f32_to_bf16(v);
+}
+
+static int64_t group_count(int64_t numel, int g) { return numel ? (numel + g - 1) / g : 0; }
+static int64_t code_offset(int64_t group, int g, int item, int compact) {
+    return compact ? group * (g + item) : group * g;
+}
+static int64_t scale_offset(int64_t group, int64_t groups, int g, int item, int compact) {
+    return compact ? group * (g + item) + g : groups * g + group * item;
+}
+
+/* position of element k of a group inside the group's code bytes */
+static int byte_slot(int k, int item) { return (k / item) * item + (item - 1 - k % item); }
+
+void lbw_quantize(const void *x, const void *residual, int dtype, int64_t numel, int g, int compact,
+                  uint8_t *payload) {
+    const int item = item_size(dtype);
+    const int64_t groups = group_count(numel, g);
+    float prepared[256];
+    for (int64_t group = 0; group < groups; ++group) {
+        float max_abs = 0.0f;
+        for (int k = 0; k < g; ++k) {
+            const int64_t e = group * g + k;
+            float v = 0.0f;
+            if (e < numel) {
+                v = load_as_f32(x, e, dtype);
+                if (residual) v = round_to(v + load_as_f32(residual, e, dtype), dtype);
+            }
+            prepared[k] = v;
+            max_abs = fmaxf(max_abs, fabsf(v));
+        }
+        const float stored = round_to(max_abs, dtype);
+        const float scale = fmaxf(stored, 1.0e-6f);
+        const float multiplier = 127.0f / scale;
+        uint8_t *codes = payload + code_offset(group, g, item, compact);
+        for (int k = 0; k < g; ++k) {
+            float q = rintf(prepared[k] * multiplier);
+            int c = q != q ? 0 : (q > 127.0f ? 127 : (q < -127.0f ? -127 : (int)q));
+            codes[byte_slot(k, item)] = (uint8_t)(int8_t)c;
+        }
+        uint8_t *where = payload + scale_offset(group, groups, g, item, compact);
+        if (dtype == LBW_F32) memcpy(where, &stored, 4);
+        else {
+            uint16_t h = dtype == LBW_F16 ? f32_to_f16(stored) : f32_to_bf16(stored);
+            memcpy(where, &h, 2);
+        }
+    }
+}
+
+static float payload_step(const uint8_t *payload, int64_t group, int64_t groups, int g, int dtype, int compact) {
+    const int item = item_size(dtype);
+    const uint8_t *where = payload + scale_offset(group, groups, g, item, compact);
+    float stored;
+    if (dtype == LBW_F32) memcpy(&stored, where, 4);
+    else {
+        uint16_t h;
+        memcpy(&h, where, 2);
+        stored = dtype == LBW_F16 ? f16_to_f32(h) : bf16_to_f32(h);
+    }
+    return stored / 127.0f;
+}
+
+static float payload_code(const uint8_t *payload, int64_t e, int g, int dtype, int compact) {
+    const int item = item_size(dtype);
+    const int64_t group = e / g;
+    const int k = (int)(e - group * g);
+    return (float)(int8_t)payload[code_offset(group, g, item, compact) + byte_slot(k, item)];
+}
+
+/* correctly rounded a + b in a 16-bit dtype: the double sum is exact (or, for far-apart bf16 operands,
+ * off by far less than the rounding step) and is rounded once */
+static float add_in_dtype(float a, float b, int dtype) {
+    if (dtype == LBW_F32) return a + b;
+    double wide = (double)a + (double)b;
+    float near = (float)wide;
+    double err = wide - (double)near;
+    if (err != 0.0 && isfinite(near)) {
+        uint32_t u = f32_to_bits(near);
+        if ((u & 1u) == 0) {
+            int up = (err > 0.0) == (near > 0.0f);
+            u = up ? u + 1u : u - 1u;
+            near = bits_to_f32(u);
+        }
+    }
+    return round_to(near, dtype);
+}
+
+/* op: 0 none, 1 sum, 2 max, 3 min; out is read for op != 0 */
+void lbw_dequantize(const uint8_t *payload, int64_t numel, int g, int compact, int dtype, int op, void *out) {
+    const int64_t groups = group_count(numel, g);
+    for (int64_t e = 0; e < numel; ++e) {
+        const float step = payload_step(payload, e / g, groups, g, dtype, compact);
+        float v = round_to(payload_code(payload, e, g, dtype, compact) * step, dtype);
+        if (op != 0) {
+            const float old = load_as_f32(out, e, dtype);
+            if (op == 1) v = add_in_dtype(old, v, dtype);
+            else if (op == 2) v = old > v ? old : v;
+            else v = old > v ? v : old;
+        }
+        store_from_f32(out, e, dtype, v);
+    }
+}
+
+/* out = T(sum_r code_r * step_r * inv_divisor); with `prepared`, residual = T(prepared - unrounded mean) */
+void lbw_reduce(const uint8_t *const *payloads, int world, int64_t numel, int g, int compact, int dtype,
+                float inv_divisor, int use_fma, const void *prepared, void *out, void *residual) {
+    const int64_t groups = group_count(numel, g);
+    for (int64_t e = 0; e < numel; ++e) {
+        float sum = 0.0f;
+        for (int r = 0; r < world; ++r) {
+            const float step = payload_step(payloads[r], e / g, groups, g, dtype, compact);
+            const float code = payload_code(payloads[r], e, g, dtype, compact);
+            if (use_fma) sum = fmaf(code, step, sum);
+            else {
+                const float term = code * step;
+                sum = sum + term;
+            }
+        }
+        const float value = sum * inv_divisor;
+        store_from_f32(out, e, dtype, value);
+        if (prepared && residual) store_from_f32(residual, e, dtype, load_as_f32(prepared, e, dtype) - value);
+    }
+}
