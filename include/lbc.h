@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define LBC_ABI_VERSION 1
+#define LBC_ABI_VERSION 2
 
 enum { LBC_OK = 0, LBC_UNSUPPORTED = 1, LBC_EINVAL = -1, LBC_ELAUNCH = -2 };
 
@@ -160,6 +160,67 @@ int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int worl
  */
 int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored, int restored_dtype,
                   void *residual, int residual_dtype, int64_t numel, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Payload format of the reference's CUDA extension ("format B", the bytes ccdl_cuda_ops
+ * produces and consumes), for fleets that mix ranks running that extension with gfx950 ranks.
+ * `dtype` is the element type of the tensor AND of the stored scales; G = ceil(n/g) groups:
+ *   scale  = max |p| over the group, stored as `dtype` (NaNs are skipped);
+ *   code   = rint(p * (127 / max(float(scale), 1e-6f))), NaN -> 0
+ *            (ccdl_comm/csrc/quantization/quant_pack_kernel.cu:86-103,111-143);
+ *   bytes  = codes with the byte order reversed inside every sizeof(dtype)-byte word;
+ *   compact != 0: per group [g code bytes][scale]  (quant_pack_kernel.cu:104-106,160-162)
+ *   compact == 0: all code bytes, then all scales  (quant_kernel_fp32.cuh:266-303);
+ *   decode = float(code) * (float(scale) / 127), rounded to `dtype`
+ *            (dequant_reduce_kernel.cu:38-69, dequant_kernel_fp32.cuh:81-104).
+ * A payload holds G * (g + sizeof(dtype)) bytes and must be aligned to sizeof(dtype).
+ * No golden bytes of an NVIDIA build exist in the reference, so byte equality with such a
+ * build is argued from the source, not measured.
+ */
+
+/* Bytes of one payload (quant_pack_kernel.cu:247-249); -1 for invalid arguments. */
+int64_t lbc_wire_payload_nbytes(int64_t numel, int group_size, int dtype);
+
+/*
+ * Quantize x (+ residual, added in fp32 and rounded to dtype first) into one payload.
+ * Replaces native inplace_quantize_pack and inplace_quantize for 8-bit linear codes
+ * (quant_pack_kernel.cu:220-275, ccdl_comm/csrc/pybind.cpp:36-63).  Ragged numel is zero padded.
+ */
+int lbc_wire_quant_pack(const void *x, const void *residual, int dtype, int64_t numel, int group_size,
+                        int compact, uint8_t *payload, void *stream);
+
+/* As lbc_quant_pack_chunks, in this format: chunk d of ceil(numel/world) elements becomes the
+ * payload at payloads + d*payload_stride (ccdl_comm/cuda/transports/compressed_reduce_scatter.py:72-94). */
+int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, int64_t numel, int world,
+                               int group_size, int compact, uint8_t *payloads, int64_t payload_stride,
+                               void *stream);
+
+/*
+ * Decode one payload into out (reduce_op NONE) or combine it with the values already in out:
+ * SUM adds in `dtype` with one rounding, MAX/MIN keep `(old > new) ? old : new` resp. its
+ * opposite.  Replaces native inplace_dequantize (dequant_kernel_fp32.cuh:106-120,
+ * dequant_kernel.cuh:46-60, pybind.cpp:64-90).
+ */
+int lbc_wire_dequant(const uint8_t *payload, int64_t numel, int group_size, int compact, void *out, int dtype,
+                     int reduce_op, void *stream);
+
+/* As lbc_dequant_chunks, in this format (ccdl_comm/communication/topology_transport.py:866-894). */
+int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world, int64_t shard_numel,
+                            int64_t total_numel, int group_size, int compact, void *out, int dtype,
+                            int reduce_op, void *stream);
+
+/*
+ * out = dtype(sum_r float(code_r) * (scale_r / 127) * inv_divisor), payloads added in list order in
+ * fp32 starting from 0; with prepared/new_residual: new_residual = dtype(float(prepared) - the
+ * unrounded fp32 value).  Replaces native try_inplace_dequantize_reduce_fused and
+ * inplace_dequantize_reduce_mean_update_error_feedback (dequant_reduce_kernel.cu:71-134,150-221,
+ * 315-430), which support group_size 64 and world <= 8 only; so does this.
+ * fused_multiply_add != 0 accumulates with fma(code, step, sum), which is what nvcc's default
+ * contraction makes of the reference's `sum += code * step`; 0 rounds the product first.
+ */
+int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t numel, int group_size,
+                            int compact, float inv_divisor, int fused_multiply_add, void *out, int dtype,
+                            const void *prepared, void *new_residual, void *stream);
 
 #ifdef __cplusplus
 }

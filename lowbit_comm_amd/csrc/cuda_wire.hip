@@ -1,0 +1,525 @@
+// Kernels for the payload format of the reference's CUDA extension (ccdl_cuda_ops), so that
+// gfx950 ranks can exchange payloads with ranks running that extension.
+//
+// Format (ccdl_comm/csrc/quantization/quant_pack_kernel.cu:101-162 writes it,
+// dequant_reduce_kernel.cu:27-69 reads it), for element type T of the tensor:
+//   scale of a group  = max |p| over the group, stored as T (NaNs skipped, fmaxf);
+//   code              = rint(p * (127 / max(float(scale), 1e-6f))), NaN -> 0;
+//   bytes of a group  = codes with the byte order reversed inside every sizeof(T)-byte word
+//                       (2-byte words for fp16/bf16, 4-byte words for fp32);
+//   compact layout    = per group [G code bytes][scale]; otherwise all code bytes, then all scales;
+//   decode            = float(code) * (float(scale) / 127), rounded to T.
+//
+// Mapping: as in the portable-format kernels, one lane owns 16 bytes of the tensor (4 fp32 or
+// 8 half elements), a group sits in adjacent lanes of one DPP row, and every tile's loads are
+// issued before the arithmetic.  Group strides of 66 or 68 bytes leave code words only 2- or
+// 4-byte aligned; gfx950 global memory instructions accept that, so all accesses here are typed
+// with element alignment only and there is no separate path for unaligned tensors.
+#include "device_utils.h"
+#include "launch.h"
+
+namespace lbc {
+namespace {
+
+constexpr int kPlain = 0, kNonTemporal = 1;
+
+// N 32-bit words at an address aligned to ALIGN bytes.
+template <int N, int ALIGN> struct words_at {
+    typedef vec_t<uint32_t, N> type __attribute__((aligned(ALIGN)));
+};
+
+template <int N, int ALIGN, int NT>
+__device__ __forceinline__ void load_words(const uint8_t *p, uint32_t (&w)[N]) {
+    using V = typename words_at<N, ALIGN>::type;
+    vec_t<uint32_t, N> v;
+    if constexpr (NT == kNonTemporal) v = __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+    else v = *reinterpret_cast<const V *>(p);
+#pragma unroll
+    for (int i = 0; i < N; ++i) w[i] = v[i];
+}
+
+template <int N, int ALIGN, int NT>
+__device__ __forceinline__ void store_words(uint8_t *p, const uint32_t (&w)[N]) {
+    using V = typename words_at<N, ALIGN>::type;
+    vec_t<uint32_t, N> v;
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = w[i];
+    if constexpr (NT == kNonTemporal) __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
+    else *reinterpret_cast<V *>(p) = v;
+}
+
+// VEC elements of T at an address aligned to sizeof(T) only.
+template <typename T, int VEC, int NT>
+__device__ __forceinline__ void load_elems(const T *p, T (&dst)[VEC]) {
+    typedef vec_t<T, VEC> V __attribute__((aligned(sizeof(T))));
+    vec_t<T, VEC> v;
+    if constexpr (NT == kNonTemporal) v = __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+    else v = *reinterpret_cast<const V *>(p);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) dst[i] = v[i];
+}
+
+template <typename T, int VEC, int NT>
+__device__ __forceinline__ void store_elems(T *p, const T (&src)[VEC]) {
+    typedef vec_t<T, VEC> V __attribute__((aligned(sizeof(T))));
+    vec_t<T, VEC> v;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = src[i];
+    if constexpr (NT == kNonTemporal) __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
+    else *reinterpret_cast<V *>(p) = v;
+}
+
+template <typename T> struct wire {
+    static constexpr int ITEM = sizeof(T);
+    static constexpr int VEC = 16 / ITEM;       // elements per lane
+    static constexpr int WORDS = VEC / 4;       // 32-bit code words per lane
+    static constexpr int TILE = kWave * VEC;
+};
+
+// Byte position of element k (0..3) inside its 32-bit word: fp32 payloads reverse all four
+// bytes, 16-bit payloads swap byte pairs.
+template <typename T> __device__ __forceinline__ constexpr int byte_in_word(int k) {
+    return sizeof(T) == 4 ? 3 - k : (k ^ 1);
+}
+// Byte position of element k of a group inside the group's code bytes.
+template <typename T> __device__ __forceinline__ int byte_in_group(int k) {
+    constexpr int ITEM = sizeof(T);
+    return (k / ITEM) * ITEM + (ITEM - 1 - k % ITEM);
+}
+
+template <typename T, int G> struct group_layout {
+    static constexpr int ITEM = sizeof(T);
+    const int64_t groups;
+    const bool compact;
+    __device__ __forceinline__ int64_t codes(int64_t group) const { return compact ? group * (G + ITEM) : group * G; }
+    __device__ __forceinline__ int64_t scale(int64_t group) const {
+        return compact ? group * (G + ITEM) + G : groups * G + group * ITEM;
+    }
+};
+
+// float(scale) / 127 with IEEE rounding: the three-operation form proven exhaustively for
+// every finite float (tests/native/check_scale127.c); an infinite scale passes through.
+__device__ __forceinline__ float div127(float a) {
+    const float c = as_f32(0x3C010204u);
+    const float q0 = a * c;
+    const float r = __builtin_fmaf(-q0, 127.0f, a);
+    const float q = __builtin_fmaf(r, c, q0);
+    return (as_u32(a) & 0x7FFFFFFFu) == 0x7F800000u ? a : q;
+}
+
+// a + b rounded once to T (what a native half / bfloat16 add returns): the float sum is turned
+// into a round-to-odd result with the exact error term, then rounded to T.
+template <typename T> __device__ __forceinline__ float add_rounded_once(float a, float b) {
+    float s = a + b;
+    if constexpr (same_t<T, float>::value) return s;
+    const float bb = s - a;
+    const float err = (a - (s - bb)) + (b - bb);
+    uint32_t u = as_u32(s);
+    const bool finite = (u & 0x7F800000u) != 0x7F800000u;
+    if (err != 0.0f && finite && (u & 1u) == 0) {
+        const bool larger_magnitude = (err > 0.0f) == (s > 0.0f);
+        u = larger_magnitude ? u + 1u : u - 1u;
+        s = as_f32(u);
+    }
+    return round_through<T>(s);
+}
+
+// ---------------------------------------------------------------------------
+// quantize + pack (optionally x + residual), `world` chunks via blockIdx.y
+// ---------------------------------------------------------------------------
+template <typename T, int G, bool HAS_R, int NT>
+__global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs a) {
+    using W = wire<T>;
+    constexpr int VEC = W::VEC;
+    constexpr int LPG = G / VEC;
+    constexpr int UNROLL = 4;
+    constexpr int BLOCK_ELEMS = W::TILE * kWavesPerBlock * UNROLL;
+    static_assert(LPG >= 1 && LPG <= 16, "a group must fit one DPP row");
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t chunk = blockIdx.y;
+    const int64_t chunk_start = chunk * a.shard_numel;
+    int64_t valid = a.numel - chunk_start;
+    valid = valid < 0 ? 0 : (valid > a.shard_numel ? a.shard_numel : valid);
+    const int64_t groups = (a.shard_numel + G - 1) / G;
+    const int64_t padded = groups * G;
+    const group_layout<T, G> at{groups, a.compact != 0};
+
+    const T *__restrict__ x = static_cast<const T *>(a.x) + chunk_start;
+    const T *__restrict__ r = HAS_R ? static_cast<const T *>(a.residual) + chunk_start : nullptr;
+    uint8_t *__restrict__ payload = a.payloads + chunk * a.payload_stride;
+
+    const int64_t block_first = static_cast<int64_t>(blockIdx.x) * BLOCK_ELEMS;
+    if (block_first >= padded) return;
+
+    auto group_multiplier = [](uint32_t absmax_bits, float &absmax) {
+        absmax = as_f32(group_max_bits<LPG>(absmax_bits));
+        const float scale = absmax < 1.0e-6f ? 1.0e-6f : absmax;
+        return 127.0f / scale;
+    };
+
+    if (block_first + BLOCK_ELEMS <= valid) {
+        T xv[UNROLL][VEC];
+        T rv[UNROLL][VEC];
+        int64_t e0[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
+            load_elems<T, VEC, NT>(x + e0[u], xv[u]);
+            if constexpr (HAS_R) load_elems<T, VEC, NT>(r + e0[u], rv[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            float p[VEC];
+            uint32_t m = 0;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                float v = widen(xv[u][i]);
+                if constexpr (HAS_R) v = round_through<T>(v + widen(rv[u][i]));
+                p[i] = v;
+                uint32_t bits = as_u32(v) & 0x7FFFFFFFu;
+                bits = bits > 0x7F800000u ? 0u : bits;   // fmaxf skips NaN
+                m = bits > m ? bits : m;
+            }
+            float absmax;
+            const float multiplier = group_multiplier(m, absmax);
+            int c[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) c[i] = cvt_i32(__builtin_rintf(p[i] * multiplier));
+            uint32_t words[W::WORDS];
+#pragma unroll
+            for (int k = 0; k < W::WORDS; ++k) {
+                if constexpr (sizeof(T) == 4) words[k] = pack4(c[4 * k + 3], c[4 * k + 2], c[4 * k + 1], c[4 * k]);
+                else words[k] = pack4(c[4 * k + 1], c[4 * k], c[4 * k + 3], c[4 * k + 2]);
+            }
+            const int64_t group = e0[u] / G;
+            const int k0 = static_cast<int>(e0[u] - group * G);
+            store_words<W::WORDS, sizeof(T), NT>(payload + at.codes(group) + k0, words);
+            if ((lane & (LPG - 1)) == 0) *reinterpret_cast<T *>(payload + at.scale(group)) = narrow<T>(absmax);
+        }
+        return;
+    }
+
+    // ---- edge block: ragged tail and zero padding, element-wise ----------------
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t e0 = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
+        if (e0 - lane * VEC >= padded) break;  // wavefront-uniform
+        float p[VEC];
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const int64_t e = e0 + i;
+            float v = 0.0f;
+            if (e < valid) {
+                v = widen(x[e]);
+                if constexpr (HAS_R) v = round_through<T>(v + widen(r[e]));
+            }
+            p[i] = v;
+            uint32_t bits = as_u32(v) & 0x7FFFFFFFu;
+            bits = bits > 0x7F800000u ? 0u : bits;
+            m = bits > m ? bits : m;
+        }
+        float absmax;
+        const float multiplier = group_multiplier(m, absmax);   // every lane of the row takes part
+        if (e0 < padded) {
+            const int64_t group = e0 / G;
+            const int k0 = static_cast<int>(e0 - group * G);
+            uint8_t *codes = payload + at.codes(group);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i)
+                codes[byte_in_group<T>(k0 + i)] = static_cast<uint8_t>(cvt_i32(__builtin_rintf(p[i] * multiplier)));
+            if ((lane & (LPG - 1)) == 0) *reinterpret_cast<T *>(payload + at.scale(group)) = narrow<T>(absmax);
+        }
+    }
+}
+
+template <typename T, int G, bool HAS_R>
+hipError_t launch_wire_quant_r(int mode, const WireQuantArgs &a, int world, hipStream_t stream) {
+    constexpr int BLOCK_ELEMS = wire<T>::TILE * kWavesPerBlock * 4;
+    const int64_t groups = (a.shard_numel + G - 1) / G;
+    const int64_t blocks = (groups * G + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
+    if (blocks == 0 || world == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFFLL || world > 65535) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(world));
+    if (mode == kStream) hipLaunchKernelGGL((wire_quant_kernel<T, G, HAS_R, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
+    else hipLaunchKernelGGL((wire_quant_kernel<T, G, HAS_R, kPlain>), grid, dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_wire_quant_t(int g, int mode, const WireQuantArgs &a, int world, hipStream_t s) {
+    const bool has_r = a.residual != nullptr;
+    switch (g) {
+        case 64: return has_r ? launch_wire_quant_r<T, 64, true>(mode, a, world, s) : launch_wire_quant_r<T, 64, false>(mode, a, world, s);
+        case 32: return has_r ? launch_wire_quant_r<T, 32, true>(mode, a, world, s) : launch_wire_quant_r<T, 32, false>(mode, a, world, s);
+        case 16: return has_r ? launch_wire_quant_r<T, 16, true>(mode, a, world, s) : launch_wire_quant_r<T, 16, false>(mode, a, world, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// fused dequant-reduce of up to 8 payloads (+ mean, + error-feedback update)
+// ---------------------------------------------------------------------------
+template <typename T, int G, int WORLD, bool FMA, int NT>
+__global__ __launch_bounds__(kBlock) void wire_reduce_kernel(const WireReduceArgs a) {
+    using W = wire<T>;
+    constexpr int VEC = W::VEC;
+    constexpr int UNROLL = WORLD <= 2 ? 2 : 1;
+    constexpr int BLOCK_ELEMS = W::TILE * kWavesPerBlock * UNROLL;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t block_first = static_cast<int64_t>(blockIdx.x) * BLOCK_ELEMS;
+    const int64_t groups = (a.numel + G - 1) / G;
+    const group_layout<T, G> at{groups, a.compact != 0};
+    T *__restrict__ out = static_cast<T *>(a.out);
+    const T *prepared = static_cast<const T *>(a.prepared);  // may alias new_r
+    T *new_r = static_cast<T *>(a.new_residual);
+
+    auto accumulate = [](float acc, float code, float step) {
+        if constexpr (FMA) return __builtin_fmaf(code, step, acc);
+        else return acc + code * step;
+    };
+
+    if (block_first + BLOCK_ELEMS <= a.numel) {
+        uint32_t words[UNROLL][WORLD][W::WORDS];
+        T stored[UNROLL][WORLD];
+        int64_t e0[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
+            const int64_t group = e0[u] / G;
+            const int k0 = static_cast<int>(e0[u] - group * G);
+            const int64_t code_at = at.codes(group) + k0;
+            const int64_t scale_at = at.scale(group);
+#pragma unroll
+            for (int r = 0; r < WORLD; ++r) {
+                load_words<W::WORDS, sizeof(T), NT>(a.payloads[r] + code_at, words[u][r]);
+                stored[u][r] = *reinterpret_cast<const T *>(a.payloads[r] + scale_at);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            float acc[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+#pragma unroll
+            for (int r = 0; r < WORLD; ++r) {
+                const float step = div127(widen(stored[u][r]));
+#pragma unroll
+                for (int i = 0; i < VEC; ++i)
+                    acc[i] = accumulate(acc[i], code_to_float(words[u][r][i / 4], byte_in_word<T>(i % 4)), step);
+            }
+            T o[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                acc[i] = acc[i] * a.inv_divisor;
+                o[i] = narrow<T>(acc[i]);
+            }
+            store_elems<T, VEC, NT>(out + e0[u], o);
+            if (new_r != nullptr) {
+                T pv[VEC], d[VEC];
+                load_elems<T, VEC, NT>(prepared + e0[u], pv);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) d[i] = narrow<T>(widen(pv[i]) - acc[i]);
+                store_elems<T, VEC, NT>(new_r + e0[u], d);
+            }
+        }
+        return;
+    }
+
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t e0 = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
+        for (int i = 0; i < VEC; ++i) {
+            const int64_t e = e0 + i;
+            if (e >= a.numel) break;
+            const int64_t group = e / G;
+            const int k = static_cast<int>(e - group * G);
+            float acc = 0.0f;
+#pragma unroll
+            for (int r = 0; r < WORLD; ++r) {
+                const float step = div127(widen(*reinterpret_cast<const T *>(a.payloads[r] + at.scale(group))));
+                const float code = static_cast<float>(static_cast<int8_t>(a.payloads[r][at.codes(group) + byte_in_group<T>(k)]));
+                acc = accumulate(acc, code, step);
+            }
+            acc = acc * a.inv_divisor;
+            out[e] = narrow<T>(acc);
+            if (new_r != nullptr) new_r[e] = narrow<T>(widen(prepared[e]) - acc);
+        }
+    }
+}
+
+template <typename T, int G, int WORLD, bool FMA>
+hipError_t launch_wire_reduce_w(int mode, const WireReduceArgs &a, hipStream_t stream) {
+    constexpr int BLOCK_ELEMS = wire<T>::TILE * kWavesPerBlock * (WORLD <= 2 ? 2 : 1);
+    const int64_t blocks = (a.numel + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks));
+    if (mode == kStream) hipLaunchKernelGGL((wire_reduce_kernel<T, G, WORLD, FMA, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
+    else hipLaunchKernelGGL((wire_reduce_kernel<T, G, WORLD, FMA, kPlain>), grid, dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+template <typename T, int G, bool FMA>
+hipError_t launch_wire_reduce_f(int world, int mode, const WireReduceArgs &a, hipStream_t s) {
+    switch (world) {
+        case 1: return launch_wire_reduce_w<T, G, 1, FMA>(mode, a, s);
+        case 2: return launch_wire_reduce_w<T, G, 2, FMA>(mode, a, s);
+        case 3: return launch_wire_reduce_w<T, G, 3, FMA>(mode, a, s);
+        case 4: return launch_wire_reduce_w<T, G, 4, FMA>(mode, a, s);
+        case 5: return launch_wire_reduce_w<T, G, 5, FMA>(mode, a, s);
+        case 6: return launch_wire_reduce_w<T, G, 6, FMA>(mode, a, s);
+        case 7: return launch_wire_reduce_w<T, G, 7, FMA>(mode, a, s);
+        case 8: return launch_wire_reduce_w<T, G, 8, FMA>(mode, a, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
+template <typename T>
+hipError_t launch_wire_reduce_t(int g, int world, bool fma, int mode, const WireReduceArgs &a, hipStream_t s) {
+    if (g != 64) return hipErrorNotSupported;   // as the reference: dequant_reduce_kernel.cu:17,252
+    return fma ? launch_wire_reduce_f<T, 64, true>(world, mode, a, s) : launch_wire_reduce_f<T, 64, false>(world, mode, a, s);
+}
+
+// ---------------------------------------------------------------------------
+// decode of one payload (optionally combined into `out`), or of `world` shard payloads
+// ---------------------------------------------------------------------------
+template <typename T, int OP> __device__ __forceinline__ float combine_in(float old, float v) {
+    if constexpr (OP == 1) return add_rounded_once<T>(old, v);
+    else if constexpr (OP == 2) return old > v ? old : v;
+    else if constexpr (OP == 3) return old > v ? v : old;
+    else return v;
+}
+
+template <typename T, int G, int OP, int NT>
+__global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArgs a) {
+    using W = wire<T>;
+    constexpr int VEC = W::VEC;
+    constexpr int UNROLL = 2;
+    constexpr int BLOCK_ELEMS = W::TILE * kWavesPerBlock * UNROLL;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t chunk = blockIdx.y;
+    const int64_t chunk_start = chunk * a.shard_numel;
+    int64_t valid = a.total_numel - chunk_start;
+    valid = valid < 0 ? 0 : (valid > a.shard_numel ? a.shard_numel : valid);
+    const int64_t groups = (a.shard_numel + G - 1) / G;
+    const group_layout<T, G> at{groups, a.compact != 0};
+    const uint8_t *__restrict__ payload = a.payloads + chunk * a.payload_stride;
+    T *__restrict__ out = static_cast<T *>(a.out) + chunk_start;
+    const int64_t block_first = static_cast<int64_t>(blockIdx.x) * BLOCK_ELEMS;
+    if (block_first >= valid) return;
+
+    if (block_first + BLOCK_ELEMS <= valid) {
+        uint32_t words[UNROLL][W::WORDS];
+        T stored[UNROLL];
+        int64_t e0[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
+            const int64_t group = e0[u] / G;
+            const int k0 = static_cast<int>(e0[u] - group * G);
+            load_words<W::WORDS, sizeof(T), NT>(payload + at.codes(group) + k0, words[u]);
+            stored[u] = *reinterpret_cast<const T *>(payload + at.scale(group));
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            T o[VEC];
+            if constexpr (OP != 0) load_elems<T, VEC, NT>(out + e0[u], o);
+            const float step = div127(widen(stored[u]));
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                float v = round_through<T>(code_to_float(words[u][i / 4], byte_in_word<T>(i % 4)) * step);
+                if constexpr (OP != 0) v = combine_in<T, OP>(widen(o[i]), v);
+                o[i] = narrow<T>(v);
+            }
+            store_elems<T, VEC, NT>(out + e0[u], o);
+        }
+        return;
+    }
+
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t e0 = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
+        for (int i = 0; i < VEC; ++i) {
+            const int64_t e = e0 + i;
+            if (e >= valid) break;
+            const int64_t group = e / G;
+            const int k = static_cast<int>(e - group * G);
+            const float step = div127(widen(*reinterpret_cast<const T *>(payload + at.scale(group))));
+            const float code = static_cast<float>(static_cast<int8_t>(payload[at.codes(group) + byte_in_group<T>(k)]));
+            float v = round_through<T>(code * step);
+            if constexpr (OP != 0) v = combine_in<T, OP>(widen(out[e]), v);
+            out[e] = narrow<T>(v);
+        }
+    }
+}
+
+template <typename T, int G, int OP>
+hipError_t launch_wire_decode_op(int mode, const WireDecodeArgs &a, int world, hipStream_t stream) {
+    constexpr int BLOCK_ELEMS = wire<T>::TILE * kWavesPerBlock * 2;
+    const int64_t blocks = (a.shard_numel + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
+    if (blocks == 0 || world == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFFLL || world > 65535) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(world));
+    if (mode == kStream) hipLaunchKernelGGL((wire_decode_kernel<T, G, OP, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
+    else hipLaunchKernelGGL((wire_decode_kernel<T, G, OP, kPlain>), grid, dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+template <typename T, int G>
+hipError_t launch_wire_decode_g(int op, int mode, const WireDecodeArgs &a, int world, hipStream_t s) {
+    switch (op) {
+        case 0: return launch_wire_decode_op<T, G, 0>(mode, a, world, s);
+        case 1: return launch_wire_decode_op<T, G, 1>(mode, a, world, s);
+        case 2: return launch_wire_decode_op<T, G, 2>(mode, a, world, s);
+        case 3: return launch_wire_decode_op<T, G, 3>(mode, a, world, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
+template <typename T>
+hipError_t launch_wire_decode_t(int g, int op, int mode, const WireDecodeArgs &a, int world, hipStream_t s) {
+    switch (g) {
+        case 64: return launch_wire_decode_g<T, 64>(op, mode, a, world, s);
+        case 32: return launch_wire_decode_g<T, 32>(op, mode, a, world, s);
+        case 16: return launch_wire_decode_g<T, 16>(op, mode, a, world, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_wire_quant(int dtype, int group_size, int mode, const WireQuantArgs &args, int world,
+                             hipStream_t stream) {
+    switch (dtype) {
+        case kF32: return launch_wire_quant_t<float>(group_size, mode, args, world, stream);
+        case kF16: return launch_wire_quant_t<f16>(group_size, mode, args, world, stream);
+        case kBF16: return launch_wire_quant_t<bf16>(group_size, mode, args, world, stream);
+        default: return hipErrorNotSupported;
+    }
+}
+
+hipError_t launch_wire_reduce(int dtype, int group_size, int world, bool fused_multiply_add, int mode,
+                              const WireReduceArgs &args, hipStream_t stream) {
+    switch (dtype) {
+        case kF32: return launch_wire_reduce_t<float>(group_size, world, fused_multiply_add, mode, args, stream);
+        case kF16: return launch_wire_reduce_t<f16>(group_size, world, fused_multiply_add, mode, args, stream);
+        case kBF16: return launch_wire_reduce_t<bf16>(group_size, world, fused_multiply_add, mode, args, stream);
+        default: return hipErrorNotSupported;
+    }
+}
+
+hipError_t launch_wire_decode(int dtype, int group_size, int reduce_op, int mode, const WireDecodeArgs &args,
+                              int world, hipStream_t stream) {
+    switch (dtype) {
+        case kF32: return launch_wire_decode_t<float>(group_size, reduce_op, mode, args, world, stream);
+        case kF16: return launch_wire_decode_t<f16>(group_size, reduce_op, mode, args, world, stream);
+        case kBF16: return launch_wire_decode_t<bf16>(group_size, reduce_op, mode, args, world, stream);
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace lbc

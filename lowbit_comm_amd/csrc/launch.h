@@ -50,6 +50,36 @@ struct EfArgs {
     int64_t numel;
 };
 
+// ---- payload format of the reference's CUDA extension (cuda_wire.hip) ----------
+struct WireQuantArgs {
+    const void *x;
+    const void *residual;    // may be null; same dtype as x
+    uint8_t *payloads;       // chunk d starts at payloads + d * payload_stride
+    int64_t numel;           // valid elements in the whole tensor
+    int64_t shard_numel;     // elements per chunk (== numel for a single payload)
+    int64_t payload_stride;  // bytes
+    int compact;             // scales interleaved after each group's codes
+};
+
+struct WireReduceArgs {
+    const uint8_t *payloads[kMaxPayloads];
+    void *out;
+    const void *prepared;  // may be null
+    void *new_residual;    // may be null
+    int64_t numel;
+    float inv_divisor;
+    int compact;
+};
+
+struct WireDecodeArgs {
+    const uint8_t *payloads;  // chunk d starts at payloads + d * payload_stride
+    void *out;                // chunk d lands at out + d * shard_numel elements
+    int64_t shard_numel;
+    int64_t total_numel;
+    int64_t payload_stride;
+    int compact;
+};
+
 // Each returns hipSuccess/last launch error, or hipErrorNotSupported when no
 // instantiation exists for the type combination.
 // `mode` is an lbc::AccessMode: 0 element-wise (any alignment), 1 vector, 2 vector + non-temporal.
@@ -63,5 +93,14 @@ hipError_t launch_decode(int out_dtype, int group_size, int reduce_op, int mode,
                          const DecodeArgs &args, int world, hipStream_t stream);
 hipError_t launch_ef_update(int p_dtype, int t_dtype, int r_dtype, int mode, const EfArgs &args,
                             hipStream_t stream);
+
+// Wire-format launches take mode 1 (plain) or 2 (non-temporal); they have no alignment demands
+// beyond element alignment.
+hipError_t launch_wire_quant(int dtype, int group_size, int mode, const WireQuantArgs &args, int world,
+                             hipStream_t stream);
+hipError_t launch_wire_reduce(int dtype, int group_size, int world, bool fused_multiply_add, int mode,
+                              const WireReduceArgs &args, hipStream_t stream);
+hipError_t launch_wire_decode(int dtype, int group_size, int reduce_op, int mode, const WireDecodeArgs &args,
+                              int world, hipStream_t stream);
 
 }  // namespace lbc

@@ -290,4 +290,116 @@ int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored
                   "lbc_ef_update");
 }
 
+// ---- payload format of the reference's CUDA extension -------------------------------------
+int64_t lbc_wire_payload_nbytes(int64_t numel, int group_size, int dtype) {
+    if (numel < 0 || !valid_group(group_size) || !valid_dtype(dtype)) return -1;
+    const int64_t groups = numel == 0 ? 0 : (numel + group_size - 1) / group_size;
+    return groups * (group_size + dtype_size(dtype));
+}
+
+int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, int64_t numel, int world,
+                               int group_size, int compact, uint8_t *payloads, int64_t payload_stride, void *stream) {
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
+    if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported dtype %d", dtype);
+    if (!valid_group(group_size) || world > 65535) return LBC_UNSUPPORTED;
+    const int64_t shard = (numel + world - 1) / world;
+    if (shard == 0) return LBC_OK;
+    const int item = dtype_size(dtype);
+    const int64_t payload_bytes = lbc_wire_payload_nbytes(shard, group_size, dtype);
+    if (x == nullptr || payloads == nullptr) return fail(LBC_EINVAL, "input and payloads must not be null");
+    if (world > 1 && (payload_stride < payload_bytes || payload_stride % item != 0))
+        return fail(LBC_EINVAL, "payload_stride must be a multiple of %d and >= %lld", item, (long long)payload_bytes);
+    if (!aligned_to(payloads, item)) return fail(LBC_EINVAL, "payloads must be aligned to the element size");
+    if (!aligned_to(x, item) || !aligned_to(residual, item))
+        return fail(LBC_EINVAL, "input/residual are not aligned to their element size");
+    lbc::WireQuantArgs a{};
+    a.x = x;
+    a.residual = residual;
+    a.payloads = payloads;
+    a.numel = numel;
+    a.shard_numel = shard;
+    a.payload_stride = world > 1 ? payload_stride : 0;
+    a.compact = compact != 0;
+    const int64_t moved = numel * (item * (residual ? 2 : 1) + 1);
+    return finish(lbc::launch_wire_quant(dtype, group_size, pick_mode(true, moved), a, world,
+                                         static_cast<hipStream_t>(stream)),
+                  "lbc_wire_quant_pack");
+}
+
+int lbc_wire_quant_pack(const void *x, const void *residual, int dtype, int64_t numel, int group_size, int compact,
+                        uint8_t *payload, void *stream) {
+    return lbc_wire_quant_pack_chunks(x, residual, dtype, numel, 1, group_size, compact, payload, 0, stream);
+}
+
+int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world, int64_t shard_numel,
+                            int64_t total_numel, int group_size, int compact, void *out, int dtype, int reduce_op,
+                            void *stream) {
+    if (shard_numel < 0 || total_numel < 0) return fail(LBC_EINVAL, "element counts must be >= 0");
+    if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
+    if (total_numel > shard_numel * world) return fail(LBC_EINVAL, "total_numel exceeds world * shard_numel");
+    if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported dtype %d", dtype);
+    if (reduce_op < LBC_REDUCE_NONE || reduce_op > LBC_REDUCE_MIN)
+        return fail(LBC_EINVAL, "unsupported reduce op %d", reduce_op);
+    if (!valid_group(group_size) || world > 65535) return LBC_UNSUPPORTED;
+    if (shard_numel == 0 || total_numel == 0) return LBC_OK;
+    const int item = dtype_size(dtype);
+    const int64_t payload_bytes = lbc_wire_payload_nbytes(shard_numel, group_size, dtype);
+    if (payloads == nullptr || out == nullptr) return fail(LBC_EINVAL, "payloads and out must not be null");
+    if (world > 1 && (payload_stride < payload_bytes || payload_stride % item != 0))
+        return fail(LBC_EINVAL, "payload_stride must be a multiple of %d and >= %lld", item, (long long)payload_bytes);
+    if (!aligned_to(payloads, item) || !aligned_to(out, item))
+        return fail(LBC_EINVAL, "payloads/out must be aligned to the element size");
+    lbc::WireDecodeArgs a{};
+    a.payloads = payloads;
+    a.out = out;
+    a.shard_numel = shard_numel;
+    a.total_numel = total_numel;
+    a.payload_stride = world > 1 ? payload_stride : 0;
+    a.compact = compact != 0;
+    const int64_t moved = total_numel * (item * (reduce_op == LBC_REDUCE_NONE ? 1 : 2) + 1);
+    return finish(lbc::launch_wire_decode(dtype, group_size, reduce_op, pick_mode(true, moved), a, world,
+                                          static_cast<hipStream_t>(stream)),
+                  "lbc_wire_dequant");
+}
+
+int lbc_wire_dequant(const uint8_t *payload, int64_t numel, int group_size, int compact, void *out, int dtype,
+                     int reduce_op, void *stream) {
+    return lbc_wire_dequant_chunks(payload, 0, 1, numel, numel, group_size, compact, out, dtype, reduce_op, stream);
+}
+
+int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t numel, int group_size, int compact,
+                            float inv_divisor, int fused_multiply_add, void *out, int dtype, const void *prepared,
+                            void *new_residual, void *stream) {
+    if (world <= 0) return fail(LBC_EINVAL, "inputs must not be empty");
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (!(inv_divisor > 0.0f)) return fail(LBC_EINVAL, "inv_divisor must be > 0");
+    if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported dtype %d", dtype);
+    if ((prepared == nullptr) != (new_residual == nullptr))
+        return fail(LBC_EINVAL, "prepared and new_residual must be given together");
+    if (world > LBC_MAX_PAYLOADS || group_size != 64) return LBC_UNSUPPORTED;
+    if (numel == 0) return LBC_OK;
+    if (payloads == nullptr || out == nullptr) return fail(LBC_EINVAL, "payloads and out must not be null");
+    const int item = dtype_size(dtype);
+    if (!aligned_to(out, item) || !aligned_to(prepared, item) || !aligned_to(new_residual, item))
+        return fail(LBC_EINVAL, "out/prepared/new_residual are not aligned to their element size");
+    lbc::WireReduceArgs a{};
+    for (int r = 0; r < world; ++r) {
+        if (payloads[r] == nullptr) return fail(LBC_EINVAL, "payload %d is null", r);
+        if (!aligned_to(payloads[r], item)) return fail(LBC_EINVAL, "payload %d must be aligned to the element size", r);
+        a.payloads[r] = payloads[r];
+    }
+    a.out = out;
+    a.prepared = prepared;
+    a.new_residual = new_residual;
+    a.numel = numel;
+    a.inv_divisor = inv_divisor;
+    a.compact = compact != 0;
+    int64_t moved = numel * (world + item);
+    if (prepared != nullptr) moved += 2 * numel * item;
+    return finish(lbc::launch_wire_reduce(dtype, group_size, world, fused_multiply_add != 0, pick_mode(true, moved), a,
+                                          static_cast<hipStream_t>(stream)),
+                  "lbc_wire_dequant_reduce");
+}
+
 }  // extern "C"
