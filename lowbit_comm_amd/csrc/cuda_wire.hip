@@ -87,15 +87,20 @@ template <typename T> __device__ __forceinline__ int byte_in_group(int k) {
     return (k / ITEM) * ITEM + (ITEM - 1 - k % ITEM);
 }
 
-template <typename T, int G> struct group_layout {
+// COMPACT payloads interleave [G code bytes][scale] per group, so a 128-byte line is shared by
+// neighbouring wavefront instructions and payload accesses must stay cacheable even when the tensors
+// stream with the non-temporal hint (the hint would drop the line between its two uses).  Otherwise
+// the policy measured for the portable format applies: code stores follow the tensors' hint, code
+// loads are non-temporal only from four payloads on.
+template <typename T, int G, bool COMPACT> struct group_layout {
     static constexpr int ITEM = sizeof(T);
     const int64_t groups;
-    const bool compact;
-    __device__ __forceinline__ int64_t codes(int64_t group) const { return compact ? group * (G + ITEM) : group * G; }
+    __device__ __forceinline__ int64_t codes(int64_t group) const { return COMPACT ? group * (G + ITEM) : group * G; }
     __device__ __forceinline__ int64_t scale(int64_t group) const {
-        return compact ? group * (G + ITEM) + G : groups * G + group * ITEM;
+        return COMPACT ? group * (G + ITEM) + G : groups * G + group * ITEM;
     }
 };
+template <bool COMPACT, int NT, int WORLD> constexpr int payload_load_hint() { return COMPACT || WORLD < 4 ? kPlain : NT; }
 
 // float(scale) / 127 with IEEE rounding: the three-operation form proven exhaustively for
 // every finite float (tests/native/check_scale127.c); an infinite scale passes through.
@@ -127,8 +132,9 @@ template <typename T> __device__ __forceinline__ float add_rounded_once(float a,
 // ---------------------------------------------------------------------------
 // quantize + pack (optionally x + residual), `world` chunks via blockIdx.y
 // ---------------------------------------------------------------------------
-template <typename T, int G, bool HAS_R, int NT>
+template <typename T, int G, bool HAS_R, bool COMPACT, int NT>
 __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs a) {
+    constexpr int PNT = COMPACT ? kPlain : NT;
     using W = wire<T>;
     constexpr int VEC = W::VEC;
     constexpr int LPG = G / VEC;
@@ -144,7 +150,7 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
     valid = valid < 0 ? 0 : (valid > a.shard_numel ? a.shard_numel : valid);
     const int64_t groups = (a.shard_numel + G - 1) / G;
     const int64_t padded = groups * G;
-    const group_layout<T, G> at{groups, a.compact != 0};
+    const group_layout<T, G, COMPACT> at{groups};
 
     const T *__restrict__ x = static_cast<const T *>(a.x) + chunk_start;
     const T *__restrict__ r = HAS_R ? static_cast<const T *>(a.residual) + chunk_start : nullptr;
@@ -195,7 +201,7 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
             }
             const int64_t group = e0[u] / G;
             const int k0 = static_cast<int>(e0[u] - group * G);
-            store_words<W::WORDS, sizeof(T), NT>(payload + at.codes(group) + k0, words);
+            store_words<W::WORDS, sizeof(T), PNT>(payload + at.codes(group) + k0, words);
             if ((lane & (LPG - 1)) == 0) *reinterpret_cast<T *>(payload + at.scale(group)) = narrow<T>(absmax);
         }
         return;
@@ -234,17 +240,23 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
     }
 }
 
-template <typename T, int G, bool HAS_R>
-hipError_t launch_wire_quant_r(int mode, const WireQuantArgs &a, int world, hipStream_t stream) {
+template <typename T, int G, bool HAS_R, bool COMPACT>
+hipError_t launch_wire_quant_c(int mode, const WireQuantArgs &a, int world, hipStream_t stream) {
     constexpr int BLOCK_ELEMS = wire<T>::TILE * kWavesPerBlock * 4;
     const int64_t groups = (a.shard_numel + G - 1) / G;
     const int64_t blocks = (groups * G + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
     if (blocks == 0 || world == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL || world > 65535) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(world));
-    if (mode == kStream) hipLaunchKernelGGL((wire_quant_kernel<T, G, HAS_R, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
-    else hipLaunchKernelGGL((wire_quant_kernel<T, G, HAS_R, kPlain>), grid, dim3(kBlock), 0, stream, a);
+    if (mode == kStream) hipLaunchKernelGGL((wire_quant_kernel<T, G, HAS_R, COMPACT, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
+    else hipLaunchKernelGGL((wire_quant_kernel<T, G, HAS_R, COMPACT, kPlain>), grid, dim3(kBlock), 0, stream, a);
     return hipGetLastError();
+}
+
+template <typename T, int G, bool HAS_R>
+hipError_t launch_wire_quant_r(int mode, const WireQuantArgs &a, int world, hipStream_t stream) {
+    return a.compact ? launch_wire_quant_c<T, G, HAS_R, true>(mode, a, world, stream)
+                     : launch_wire_quant_c<T, G, HAS_R, false>(mode, a, world, stream);
 }
 
 template <typename T>
@@ -261,8 +273,9 @@ hipError_t launch_wire_quant_t(int g, int mode, const WireQuantArgs &a, int worl
 // ---------------------------------------------------------------------------
 // fused dequant-reduce of up to 8 payloads (+ mean, + error-feedback update)
 // ---------------------------------------------------------------------------
-template <typename T, int G, int WORLD, bool FMA, int NT>
+template <typename T, int G, int WORLD, bool FMA, bool COMPACT, int NT>
 __global__ __launch_bounds__(kBlock) void wire_reduce_kernel(const WireReduceArgs a) {
+    constexpr int PNT = payload_load_hint<COMPACT, NT, WORLD>();
     using W = wire<T>;
     constexpr int VEC = W::VEC;
     constexpr int UNROLL = WORLD <= 2 ? 2 : 1;
@@ -272,7 +285,7 @@ __global__ __launch_bounds__(kBlock) void wire_reduce_kernel(const WireReduceArg
     const int wave = threadIdx.x >> 6;
     const int64_t block_first = static_cast<int64_t>(blockIdx.x) * BLOCK_ELEMS;
     const int64_t groups = (a.numel + G - 1) / G;
-    const group_layout<T, G> at{groups, a.compact != 0};
+    const group_layout<T, G, COMPACT> at{groups};
     T *__restrict__ out = static_cast<T *>(a.out);
     const T *prepared = static_cast<const T *>(a.prepared);  // may alias new_r
     T *new_r = static_cast<T *>(a.new_residual);
@@ -295,7 +308,7 @@ __global__ __launch_bounds__(kBlock) void wire_reduce_kernel(const WireReduceArg
             const int64_t scale_at = at.scale(group);
 #pragma unroll
             for (int r = 0; r < WORLD; ++r) {
-                load_words<W::WORDS, sizeof(T), NT>(a.payloads[r] + code_at, words[u][r]);
+                load_words<W::WORDS, sizeof(T), PNT>(a.payloads[r] + code_at, words[u][r]);
                 stored[u][r] = *reinterpret_cast<const T *>(a.payloads[r] + scale_at);
             }
         }
@@ -350,16 +363,22 @@ __global__ __launch_bounds__(kBlock) void wire_reduce_kernel(const WireReduceArg
     }
 }
 
-template <typename T, int G, int WORLD, bool FMA>
-hipError_t launch_wire_reduce_w(int mode, const WireReduceArgs &a, hipStream_t stream) {
+template <typename T, int G, int WORLD, bool FMA, bool COMPACT>
+hipError_t launch_wire_reduce_c(int mode, const WireReduceArgs &a, hipStream_t stream) {
     constexpr int BLOCK_ELEMS = wire<T>::TILE * kWavesPerBlock * (WORLD <= 2 ? 2 : 1);
     const int64_t blocks = (a.numel + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks));
-    if (mode == kStream) hipLaunchKernelGGL((wire_reduce_kernel<T, G, WORLD, FMA, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
-    else hipLaunchKernelGGL((wire_reduce_kernel<T, G, WORLD, FMA, kPlain>), grid, dim3(kBlock), 0, stream, a);
+    if (mode == kStream) hipLaunchKernelGGL((wire_reduce_kernel<T, G, WORLD, FMA, COMPACT, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
+    else hipLaunchKernelGGL((wire_reduce_kernel<T, G, WORLD, FMA, COMPACT, kPlain>), grid, dim3(kBlock), 0, stream, a);
     return hipGetLastError();
+}
+
+template <typename T, int G, int WORLD, bool FMA>
+hipError_t launch_wire_reduce_w(int mode, const WireReduceArgs &a, hipStream_t stream) {
+    return a.compact ? launch_wire_reduce_c<T, G, WORLD, FMA, true>(mode, a, stream)
+                     : launch_wire_reduce_c<T, G, WORLD, FMA, false>(mode, a, stream);
 }
 
 template <typename T, int G, bool FMA>
@@ -393,8 +412,9 @@ template <typename T, int OP> __device__ __forceinline__ float combine_in(float 
     else return v;
 }
 
-template <typename T, int G, int OP, int NT>
+template <typename T, int G, int OP, bool COMPACT, int NT>
 __global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArgs a) {
+    constexpr int PNT = payload_load_hint<COMPACT, NT, 1>();
     using W = wire<T>;
     constexpr int VEC = W::VEC;
     constexpr int UNROLL = 2;
@@ -407,7 +427,7 @@ __global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArg
     int64_t valid = a.total_numel - chunk_start;
     valid = valid < 0 ? 0 : (valid > a.shard_numel ? a.shard_numel : valid);
     const int64_t groups = (a.shard_numel + G - 1) / G;
-    const group_layout<T, G> at{groups, a.compact != 0};
+    const group_layout<T, G, COMPACT> at{groups};
     const uint8_t *__restrict__ payload = a.payloads + chunk * a.payload_stride;
     T *__restrict__ out = static_cast<T *>(a.out) + chunk_start;
     const int64_t block_first = static_cast<int64_t>(blockIdx.x) * BLOCK_ELEMS;
@@ -422,7 +442,7 @@ __global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArg
             e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
             const int64_t group = e0[u] / G;
             const int k0 = static_cast<int>(e0[u] - group * G);
-            load_words<W::WORDS, sizeof(T), NT>(payload + at.codes(group) + k0, words[u]);
+            load_words<W::WORDS, sizeof(T), PNT>(payload + at.codes(group) + k0, words[u]);
             stored[u] = *reinterpret_cast<const T *>(payload + at.scale(group));
         }
 #pragma unroll
@@ -457,16 +477,22 @@ __global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArg
     }
 }
 
-template <typename T, int G, int OP>
-hipError_t launch_wire_decode_op(int mode, const WireDecodeArgs &a, int world, hipStream_t stream) {
+template <typename T, int G, int OP, bool COMPACT>
+hipError_t launch_wire_decode_c(int mode, const WireDecodeArgs &a, int world, hipStream_t stream) {
     constexpr int BLOCK_ELEMS = wire<T>::TILE * kWavesPerBlock * 2;
     const int64_t blocks = (a.shard_numel + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
     if (blocks == 0 || world == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL || world > 65535) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(world));
-    if (mode == kStream) hipLaunchKernelGGL((wire_decode_kernel<T, G, OP, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
-    else hipLaunchKernelGGL((wire_decode_kernel<T, G, OP, kPlain>), grid, dim3(kBlock), 0, stream, a);
+    if (mode == kStream) hipLaunchKernelGGL((wire_decode_kernel<T, G, OP, COMPACT, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
+    else hipLaunchKernelGGL((wire_decode_kernel<T, G, OP, COMPACT, kPlain>), grid, dim3(kBlock), 0, stream, a);
     return hipGetLastError();
+}
+
+template <typename T, int G, int OP>
+hipError_t launch_wire_decode_op(int mode, const WireDecodeArgs &a, int world, hipStream_t stream) {
+    return a.compact ? launch_wire_decode_c<T, G, OP, true>(mode, a, world, stream)
+                     : launch_wire_decode_c<T, G, OP, false>(mode, a, world, stream);
 }
 
 template <typename T, int G>

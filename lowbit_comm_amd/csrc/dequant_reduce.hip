@@ -34,6 +34,13 @@ template <typename OT, int W = 8> struct decode_tiling {
     static constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock * UNROLL;
 };
 
+// Cache policy of the code loads in streaming mode, from measurement on 100 MiB buckets: with one to
+// three payloads the output dominates the traffic and cacheable code loads are ~13 % faster; from
+// four payloads on the codes dominate and the non-temporal hint wins by ~9 %.
+template <int W> __device__ __forceinline__ constexpr int code_load_mode(int mode) {
+    return mode == kStream && W < 4 ? kVector : mode;
+}
+
 template <int VEC, int MODE>
 __device__ __forceinline__ void load_codes(const int8_t *__restrict__ p, uint32_t (&w)[VEC / 4]) {
     if constexpr (MODE != kScalar) {
@@ -76,7 +83,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
             const int64_t g = e0[u] / G;
 #pragma unroll
             for (int r = 0; r < W; ++r) {
-                load_codes<VEC, MODE>(a.codes[r] + e0[u], words[u][r]);
+                load_codes<VEC, code_load_mode<W>(MODE)>(a.codes[r] + e0[u], words[u][r]);
                 scale[u][r] = a.scales[r][g];
             }
         }
@@ -216,7 +223,7 @@ __global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
-            load_codes<VEC, MODE>(codes + e0[u], words[u]);
+            load_codes<VEC, code_load_mode<1>(MODE)>(codes + e0[u], words[u]);
             scale[u] = scales[e0[u] / G];
         }
 #pragma unroll
