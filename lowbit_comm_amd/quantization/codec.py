@@ -82,9 +82,11 @@ def _zero_padded(tensor: Any, group_size: int) -> Any:
     return torch.cat((flat, flat.new_zeros((missing,))), dim=0)
 
 
-def _divide(decoded: Any, count: int, *, in_place: bool) -> Any:
-    """``decoded / count`` as a true division (GPU tensors: not the reciprocal multiply torch would use)."""
-    if getattr(decoded, "is_cuda", False):
+def _divide(decoded: Any, count: int, *, in_place: bool, exact: bool = True) -> Any:
+    """``decoded / count``.  ``exact``: a true division on GPU tensors, as the portable CPU codec computes it,
+    instead of the reciprocal multiply torch uses there; the CUDA byte format keeps torch's own division because
+    that is what a rank running the CUDA extension computes (ccdl_comm/quantization/codec.py:339-343)."""
+    if exact and getattr(decoded, "is_cuda", False):
         from lowbit_comm_amd.hip.ops import true_divide_
 
         return true_divide_(decoded if in_place else decoded.clone(), count)
@@ -213,7 +215,8 @@ def dequantize_reduce_tensors(buffers: list[object], shape: tuple[int, ...], con
                                                          config.bit, quant_type, config.compact)
         decoded = output
     if reduce == "mean" and not fused:
-        decoded = _divide(decoded, len(buffers), in_place=output is not None)
+        decoded = _divide(decoded, len(buffers), in_place=output is not None,
+                          exact=_wire_format(module) == "portable")
     return _trim_to_shape(decoded, shape)
 
 

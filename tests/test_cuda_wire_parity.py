@@ -246,3 +246,113 @@ def test_cross_format_round_trip_is_consistent(hip, hip_device):
         codes_a, _ = wire.split(to_numpy(payload), x.numel(), name)
         codes_b, _ = wire.split(to_numpy(again), x.numel(), name)
         assert np.abs(codes_a.astype(np.int16) - codes_b.astype(np.int16)).max() <= 1
+
+
+# --------------------------------------------------------------------------- #
+# the drop-in module (names and argument orders of the reference's pybind module) and the facade over it
+# --------------------------------------------------------------------------- #
+@pytest.fixture(scope="module")
+def wire_status(hip_device):
+    from lowbit_comm_amd.hip.loader import load_hip_extension
+
+    status = load_hip_extension(wire_format="native")
+    assert status.available, status.reason
+    assert status.module.NATIVE_WIRE_FORMAT == "native"
+    return status
+
+
+def test_module_round_trip_like_the_reference_smoke_test(wire_status, hip_device):
+    """tests/test_cuda_extension_smoke.py:15-34 upstream: 4096 fp16 randn, 8-bit linear, group 64, rel-L2 < 0.02."""
+    from lowbit_comm_amd.config import CompressionConfig
+    from lowbit_comm_amd.quantization.codec import dequantize_tensor, quantize_tensor
+
+    tensor = make(4096, "fp16", 1, hip_device)
+    config = CompressionConfig(bit=8, group_size=64, quant_type="linear")
+    quantized = quantize_tensor(tensor, config, extension_status=wire_status)
+    same(quantized, wire.quantize(to_numpy(tensor), "fp16", 64, config.compact))
+    restored = dequantize_tensor(quantized, tensor.shape, config, dtype="fp16", extension_status=wire_status)
+    assert restored.shape == tensor.shape and bool(torch.isfinite(restored).all())
+    rel = float((tensor.float() - restored.float()).norm() / tensor.float().norm())
+    assert rel < 0.02
+    same(restored, wire.dequantize(to_numpy(quantized), 4096, "fp16", 64, config.compact))
+
+
+@pytest.mark.parametrize("name", list(NAMES))
+def test_module_fused_pack_equals_the_padded_chain(wire_status, hip_device, name):
+    """tests/cuda/test_fused_quant_pack.py:27-70 upstream: uneven input, with and without residual; sizes from the
+    facade's allocator; metadata as the reference records it."""
+    from lowbit_comm_amd.config import CompressionConfig
+    from lowbit_comm_amd.quantization.codec import allocate_quantized_buffer, inplace_quantize_pack, quantize_tensor
+
+    for g in (16, 32, 64):
+        config = CompressionConfig(bit=8, group_size=g, compact=True)
+        tensor = torch.linspace(-3.0, 3.0, g + 7, device=hip_device, dtype=NAMES[name])
+        for residual in (None, torch.linspace(-0.2, 0.2, g + 7, device=hip_device, dtype=NAMES[name])):
+            reference_input = tensor if residual is None else tensor + residual
+            chained = quantize_tensor(reference_input, config, extension_status=wire_status)
+            output = allocate_quantized_buffer(tensor, config, dtype=name, wire_format="native")
+            metadata = {}
+            assert inplace_quantize_pack(tensor, output, residual, config, metadata, extension_status=wire_status)
+            assert torch.equal(output, chained)
+            assert metadata == {"original_numel": g + 7, "padded_numel": 2 * g, "padding_numel": g - 7,
+                                "fused_quant_pack": True}
+
+
+@pytest.mark.parametrize("name", list(NAMES))
+def test_module_reduce_paths(wire_status, hip_device, name):
+    """Fused path for whole groups; decode-and-add chain in the tensor dtype otherwise (pybind.cpp:39-56 upstream)."""
+    module = wire_status.module
+    linear, dtype_member = module.QuantType.Linear, {"fp32": module.DType.FP32, "fp16": module.DType.FP16,
+                                                     "bf16": module.DType.BF16}[name]
+    n = 64 * 50
+    grads = [make(n, name, 900 + r, hip_device) for r in range(4)]
+    payloads = [module.quantize(g_, 64, 0, False, 8, linear, True) for g_ in grads]
+    host = [to_numpy(p) for p in payloads]
+    fused = module.dequantize_reduce(payloads, 64, 0, 8, linear, dtype_member, True)
+    same(fused, wire.reduce_payloads(host, n, name))
+    out = torch.empty(n, dtype=NAMES[name], device=hip_device)
+    assert module.inplace_dequantize_reduce_mean(payloads, out, 64, 0, 8, linear, True, 4)
+    same(out, wire.reduce_payloads(host, n, name, inv_divisor=0.25))
+    # nine payloads: no fused kernel, the chain adds in the tensor dtype
+    nine = payloads + payloads + payloads[:1]
+    assert module.inplace_dequantize_reduce_mean(nine, out, 64, 0, 8, linear, True, 9) is False
+    module.inplace_dequantize_reduce(nine, out, 64, 0, 8, linear, True)
+    want = wire.dequantize(host[0], n, name)
+    for p in (host + host + host[:1])[1:]:
+        want = wire.dequantize(p, n, name, reduce_op="sum", out=want)
+    same(out, want)
+    # group size 32: chain as well
+    p32 = [module.quantize(g_, 32, 0, False, 8, linear, True) for g_ in grads[:2]]
+    got = module.dequantize_reduce(p32, 32, 0, 8, linear, dtype_member, True)
+    want = wire.dequantize(to_numpy(p32[1]), n, name, 32, reduce_op="sum", out=wire.dequantize(to_numpy(p32[0]), n, name, 32))
+    same(got, want)
+
+
+def test_module_error_feedback_paths(wire_status, hip_device):
+    """tests/test_cuda_extension_smoke.py:37-100 upstream: residual update, fused mean + feedback, ragged prepared."""
+    module = wire_status.module
+    linear = module.QuantType.Linear
+    prepared = make(4096, "fp32", 3, hip_device)
+    restored = make(4096, "fp32", 4, hip_device)
+    residual = torch.empty_like(prepared)
+    module.inplace_error_feedback_update(prepared, restored, residual)
+    assert torch.equal(residual, prepared - restored)
+
+    n = 131                                                       # ragged: restored workspace is padded to 192
+    grads = [make(n, "fp16", 20 + r, hip_device) for r in range(2)]
+    payloads = [module.quantize(torch.cat((g_, g_.new_zeros(192 - n))), 64, 0, False, 8, linear, True) for g_ in grads]
+    prepared = make(n, "fp16", 30, hip_device)
+    residual = torch.empty_like(prepared)
+    restored = module.dequantize_reduce_update_error_feedback(payloads, prepared, residual, 64, 0, 8, linear,
+                                                              module.DType.FP16, True, 2)
+    assert restored.numel() == 192
+    want_restored, want_residual = wire.reduce_mean_error_feedback([to_numpy(p) for p in payloads], to_numpy(prepared),
+                                                                   n, "fp16", divisor=2)
+    same(restored[:n], want_restored)
+    same(residual, want_residual)
+    with pytest.raises(RuntimeError):
+        module.inplace_dequantize_reduce_mean_update_error_feedback(payloads, prepared, restored, residual, 64, 0, 8,
+                                                                    linear, True, 0)
+    with pytest.raises(RuntimeError):
+        module.quantize(prepared, 64, 0, False, 4, linear, True)          # 4-bit codes have no kernel
+    assert module.inplace_quantize_pack(prepared, payloads[0], None, 64, 1, False, 8, linear, True) is False

@@ -393,6 +393,21 @@ def test_default_extension_status_is_unavailable_without_a_gpu_and_never_falls_b
     assert not broken.available and "cannot load" in broken.reason
 
 
+def test_loader_wire_format_choice():
+    with pytest.raises(ValueError, match="wire_format"):
+        load_hip_extension(wire_format="format-b")
+    if not torch.cuda.is_available():
+        assert not load_hip_extension(wire_format="native").available
+    from lowbit_comm_amd.hip.cuda_wire_module import HipCudaWireModule
+    from lowbit_comm_amd.hip.native_module import HipNativeModule
+
+    portable = load_hip_extension(factory=HipNativeModule)      # constructing only loads the library
+    native = load_hip_extension(factory=HipCudaWireModule)
+    assert portable.module.NATIVE_WIRE_FORMAT == "portable" and native.module.NATIVE_WIRE_FORMAT == "native"
+    names = [n for n in dir(HipNativeModule) if not n.startswith("_")]
+    assert set(names) <= set(dir(HipCudaWireModule))             # same surface as the reference's pybind module
+
+
 def test_workspace_allocators():
     x = torch.ones(100, dtype=torch.bfloat16)
     assert codec.allocate_quantized_buffer(x, CFG, dtype="bf16").shape == (136,)
