@@ -11,10 +11,12 @@ object per configuration plus a summary table on stderr:
   4  full compressed reduce-scatter + all-gather plan of a 200 MiB fp32 bucket at W=8
   5  Llama-3-8B-shaped bf16 gradient stream in 25 MiB buckets: EF quant-pack + W=8 shard reduce per
      bucket through the workspace pool
+  6  the same bucket shapes in the byte format of the reference's CUDA extension (scales in the tensor
+     dtype, interleaved or appended): quantize+pack, W=8 fused reduce, mean + error-feedback reduce
 
 "~N(0, s)" is read as standard deviation s.  Times are HIP-event averages over back-to-back launches.
 
-    python bench_configs.py [--configs 1,2,3,4,5] [--no-parity] [--llama-layers 32]
+    python bench_configs.py [--configs 1,2,3,4,5,6] [--no-parity] [--llama-layers 32]
 """
 from __future__ import annotations
 
@@ -35,7 +37,7 @@ G = 64
 
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--configs", default="1,2,3,4,5")
+    ap.add_argument("--configs", default="1,2,3,4,5,6")
     ap.add_argument("--no-parity", action="store_true", help="skip the CPU oracle comparisons")
     ap.add_argument("--llama-layers", type=int, default=32, help="config 5: number of transformer layers (32 = full model)")
     ap.add_argument("--iters", type=int, default=50)
@@ -385,6 +387,57 @@ def main() -> int:
              host_enqueue_s=host1 - host0, pool_misses=stats.misses, pool_misses_after_first_pass=misses_after_first,
              pool_hits=stats.hits, steady_state_allocation_bytes=torch.cuda.memory_allocated() - allocated,
              distinct_workspace_keys=2 * 2)
+
+    # ------------------------------------------------------------------------------------------ 6
+    if 6 in wanted:
+        from lowbit_comm_amd.hip import cuda_wire
+
+        if parity:
+            from oracle import cuda_wire_scalar as wire_c
+
+        def host(t):
+            t = t.detach().cpu().contiguous()
+            return t.view(torch.int16).numpy().view("uint16") if t.dtype == torch.bfloat16 else t.numpy()
+
+        world, n = 8, 26_214_400
+        for name, dtype in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+            item = 4 if name == "fp32" else 2
+            for compact in (True, False):
+                layout = "interleaved scales" if compact else "appended scales"
+                pbytes = cuda_wire.payload_nbytes(n, dtype)
+                xs = [gen(SEED + 600 + s, n, 1e-3, dtype) for s in range(4)]
+                outs = [torch.empty(pbytes, dtype=torch.uint8, device=dev) for _ in range(4)]
+                quant = [cuda_wire.bind_quant_pack(xs[s], outs[s], compact=compact) for s in range(4)]
+                check = None
+                if parity:
+                    quant[0]()
+                    check = "bit-exact" if host(outs[0]).tobytes() == wire_c.quantize(host(xs[0]), name, 64, compact).tobytes() else "MISMATCH"
+                emit(6, f"quantize+pack 26.2M {name}, {layout}", n * item + pbytes,
+                     timed(lambda i: quant[i % 4](), args.iters), n * item, check)
+                # W=8 fused reduce (+ mean + error feedback) of full-bucket payloads; parity on one shard-sized case
+                payloads = [[cuda_wire.quant_pack(gen(SEED + 700 + 10 * s + r, n, 1e-3, dtype), compact=compact)
+                             for r in range(world)] for s in range(2)]
+                res = [torch.empty(n, dtype=dtype, device=dev) for _ in range(2)]
+                prepared = [gen(SEED + 800 + s, n, 1e-3, dtype) for s in range(2)]
+                plain = [cuda_wire.bind_dequant_reduce(payloads[s], res[s], compact=compact, inv_divisor=0.125) for s in range(2)]
+                feedback = [cuda_wire.bind_dequant_reduce(payloads[s], res[s], compact=compact, inv_divisor=0.125,
+                                                          prepared=prepared[s], new_residual=prepared[s]) for s in range(2)]
+                check = None
+                if parity:
+                    m = n // world
+                    small = [cuda_wire.quant_pack(gen(SEED + 900 + r, m, 1e-3, dtype), compact=compact) for r in range(world)]
+                    got = torch.empty(m, dtype=dtype, device=dev)
+                    prep = gen(SEED + 950, m, 1e-3, dtype)
+                    new_r = torch.empty_like(prep)
+                    cuda_wire.dequant_reduce_into(small, got, compact=compact, inv_divisor=0.125, prepared=prep, new_residual=new_r)
+                    want, want_r = wire_c.reduce_payloads([host(p) for p in small], m, name, 64, compact, 0.125, True, prepared=host(prep))
+                    ok = host(got).tobytes() == want.tobytes() and host(new_r).tobytes() == want_r.tobytes()
+                    check = "bit-exact (one shard)" if ok else "MISMATCH"
+                emit(6, f"fused dequant-reduce W=8 -> 26.2M {name}, {layout}", world * pbytes + n * item,
+                     timed(lambda i: plain[i % 2](), max(10, args.iters // 2)), world * pbytes, check)
+                emit(6, f"fused reduce + mean + error feedback W=8, {name}, {layout}", world * pbytes + 3 * n * item,
+                     timed(lambda i: feedback[i % 2](), max(10, args.iters // 2)), world * pbytes, check)
+                del xs, outs, quant, payloads, res, prepared, plain, feedback
 
     print(f"\n{'cfg':>3} {'us':>10} {'GB/s alg.':>10} {'% of 8TB/s':>10} {'input GB/s':>10}  parity / op", file=sys.stderr)
     for r in rows_out:
