@@ -4,15 +4,17 @@
 ``ccdl_comm/communication/ddp_hook.py:48-81`` so call sites port unchanged.  What runs here is the
 compute of that hook - error-feedback compensate, quantize+pack, fused dequant-reduce, residual
 update - on HIP kernels; the collectives themselves are *injected* (``all_gather=``, ``all_reduce=``,
-``reduce_scatter_all_gather=`` ...).  This build ships no collective transport of its own: a
-strategy whose transport is not injected raises :class:`UnsupportedCollective`, as do the
-asynchronous gather pipelines.
+``reduce_scatter_all_gather=``, ``async_all_gather=`` ...).  This build ships no collective transport of
+its own: a strategy (or the asynchronous gather) whose transport is not injected raises
+:class:`UnsupportedCollective`.
 """
 from __future__ import annotations
 
 from collections.abc import Callable
+from dataclasses import dataclass, field
 from typing import Any
 
+from lowbit_comm_amd.communication.async_pipeline import AsyncBucketPipeline
 from lowbit_comm_amd.communication.collectives import CompressedPayload
 from lowbit_comm_amd.communication.ddp import DDPBucketProcessor
 from lowbit_comm_amd.communication.gather_reduce import CompressedAllGatherReduce, GatheredPayloads
@@ -27,6 +29,7 @@ from lowbit_comm_amd.exceptions import UnsupportedCollective
 from lowbit_comm_amd.quantization.codec import (
     allocate_dequantized_buffer,
     dequantize_reduce_tensors,
+    dequantize_reduce_update_error_feedback,
     dequantize_tensor,
     inplace_dequantize_reduce_mean_update_error_feedback,
     quantize_tensor,
@@ -35,6 +38,19 @@ from lowbit_comm_amd.quantization.error_feedback import ErrorFeedbackState
 from lowbit_comm_amd.quantization.error_feedback_policy import ErrorFeedbackPolicy
 
 STRATEGIES = ("auto", "all_gather", "all_reduce", "reduce_scatter", "hierarchical", "topology")
+
+
+@dataclass(frozen=True)
+class StrategyPlan:
+    """How the requested strategy was resolved (fields of ``ccdl_comm/communication/strategy.py:46-55``).
+    The resolution here only looks at which transports were injected; there is no topology planner."""
+
+    requested_strategy: str
+    strategy: str
+    fallback_strategy: str = "all_gather"
+    reason: str = ""
+    requires_fallback: bool = False
+    capability_flags: dict[str, bool] = field(default_factory=dict)
 
 
 def _torch_future() -> Any:
@@ -79,6 +95,22 @@ def _numel(tensor: Any) -> int:
     for dim in getattr(tensor, "shape", ()):
         total *= int(dim)
     return total
+
+
+def _shaped(workspace: Any, shape: tuple[int, ...]) -> Any:
+    """First ``prod(shape)`` elements of a (possibly padded) workspace, viewed as ``shape``; objects that cannot
+    be reshaped are passed through."""
+    if not hasattr(workspace, "reshape"):
+        return workspace
+    count = 1
+    for dim in shape:
+        count *= int(dim)
+    flat = workspace.reshape((-1,))
+    try:
+        flat = flat[:count]
+    except TypeError:
+        pass
+    return flat.reshape(shape)
 
 
 def _single_process_all_reduce(tensor: Any, reduce: str) -> Any:
@@ -145,20 +177,24 @@ def create_ddp_comm_hook(
     annotation_provider: Callable[[], dict[str, Any]] | None = None,
 ) -> Callable[[Any, Any], Any]:
     """Build ``hook(state, bucket) -> Future`` for ``DistributedDataParallel.register_comm_hook``."""
-    del async_error_feedback, synchronize_async_feedback_completion, async_all_gather, completion_manager
-    del native_dequantize_reduce_update_feedback, topology_method
+    del topology_method
     requested = strategy.strip().lower()
     if requested not in STRATEGIES:
         raise UnsupportedCollective(strategy, reason="explicit strategy is unknown and no fallback was declared")
-    if async_gather:
-        raise UnsupportedCollective("async_gather", reason="asynchronous gather pipelines are not part of this build")
+    if async_gather and async_all_gather is None:
+        raise UnsupportedCollective("async_gather", reason="inject async_all_gather=; this build ships no collective transport")
     injected = {"reduce_scatter": reduce_scatter_all_gather, "hierarchical": hierarchical_all_reduce,
                 "topology": topology_all_reduce}
     if requested in injected and injected[requested] is None:
         raise UnsupportedCollective(requested, reason=f"{requested} transport unavailable for explicit strategy")
     effective = requested
+    reason = "explicit strategy"
     if requested == "auto":
         effective = "reduce_scatter" if reduce_scatter_all_gather is not None else "all_gather"
+        reason = ("a reduce-scatter transport was injected" if effective == "reduce_scatter"
+                  else "no reduce-scatter transport was injected")
+    plan = StrategyPlan(requested_strategy=requested, strategy=effective, reason=reason,
+                        capability_flags={name: fn is not None for name, fn in injected.items()})
 
     def active_quantize(tensor: Any, active: CompressionConfig) -> Any:
         if quantize is not None:
@@ -176,6 +212,7 @@ def create_ddp_comm_hook(
     uncompressed = bypass_all_reduce or _single_process_all_reduce
     inplace_reduce_feedback = (native_inplace_dequantize_reduce_update_feedback
                                or inplace_dequantize_reduce_mean_update_error_feedback)
+    combined_reduce_feedback = native_dequantize_reduce_update_feedback or dequantize_reduce_update_error_feedback
     workspaces = DequantizedWorkspaceCache(
         allocator=allocate_dequantized_workspace or allocate_dequantized_buffer,
         max_entries=workspace_cache_max_entries, max_cached_bytes=workspace_cache_max_bytes)
@@ -197,10 +234,74 @@ def create_ddp_comm_hook(
                              extension_status=extension_status)
 
     elif effective == "all_gather":
-        if all_gather is None:
+        if all_gather is None and not async_gather:
             raise UnsupportedCollective("all_gather", reason="inject all_gather=; this build ships no collective transport")
-        plain_gather = all_gather
-        packed_gather = all_gather
+
+        def missing_gather(payload: Any) -> Any:
+            raise UnsupportedCollective("all_gather", reason="this bucket needs the synchronous gather: inject all_gather=")
+
+        plain_gather = packed_gather = all_gather or missing_gather
+
+        def gather_asynchronously(key: Any, prepared: Any, local: CompressedPayload, shape: tuple[int, ...],
+                                  active_dtype: str, decision: Any) -> Any:
+            """Start the gather, return the bucket's future, finish when the gather's own future fires
+            (ccdl_comm/communication/ddp_hook.py:211-311)."""
+            work = async_all_gather(_buffer_of(local))
+            outer = future_factory()
+            read_residual = getattr(feedback, "get", None)
+            residual = read_residual(key) if decision.update and callable(read_residual) else None
+            fused_update_done = [False]
+
+            def decode(gathered: Any) -> Any:
+                buffers = [_buffer_of(p) for p in gathered.payloads]
+                if decision.update and residual is not None:
+                    try:
+                        workspace = workspaces.get(key, prepared, shape, config)
+                        if inplace_reduce_feedback(buffers, prepared, workspace, residual, config,
+                                                   extension_status=extension_status, reduce=reduce):
+                            fused_update_done[0] = True
+                            return _shaped(workspace, shape)
+                    except Exception:
+                        pass
+                    try:
+                        restored = combined_reduce_feedback(buffers, prepared, residual, shape, config,
+                                                            dtype=active_dtype, extension_status=extension_status,
+                                                            reduce=reduce)
+                        fused_update_done[0] = True
+                        return restored
+                    except Exception:
+                        pass
+                return dequantize_reduce_tensors(buffers, shape, config, dtype=active_dtype,
+                                                 extension_status=extension_status, reduce=reduce)
+
+            def update(restored: Any) -> None:
+                if not decision.update or fused_update_done[0]:
+                    return
+                latest = read_residual(key) if callable(read_residual) else None
+                if native_error_feedback_update is not None and latest is not None:
+                    native_error_feedback_update(prepared, restored, latest)
+                else:
+                    feedback.update(key, original=prepared, transmitted=restored)
+
+            if decision.apply or decision.update:
+                return AsyncBucketPipeline(gather_work=work, future=outer, dequantize_reduce=decode,
+                                           update_feedback=update, advance_policy=lambda: policy.advance(key),
+                                           completion_manager=completion_manager,
+                                           synchronize_completion=synchronize_async_feedback_completion).run()
+
+            def complete(_unused: Any = None) -> Any:
+                restored = decode(work.wait())
+                policy.advance(key)
+                outer.set_result(restored)
+                return restored
+
+            get_future = getattr(work, "get_future", None)
+            inner = get_future() if callable(get_future) else None
+            if inner is not None and hasattr(inner, "then"):
+                inner.then(complete)
+            else:
+                complete()
+            return outer
 
         def process_bucket(bucket: Any) -> Any:
             key = bucket.index() if callable(getattr(bucket, "index", None)) else id(bucket)
@@ -216,22 +317,25 @@ def create_ddp_comm_hook(
             if dequantize is None and reduce in ("mean", "sum"):
                 # facade path: flat uint8 buffers, fused decode+reduce (+ residual update) on the GPU
                 local = coerce_payload(active_quantize(prepared, config), shape=shape, dtype=active_dtype)
+                needs_feedback = decision.apply or decision.update
+                if async_gather and (async_error_feedback or not needs_feedback):
+                    return gather_asynchronously(key, prepared, local, shape, active_dtype, decision)
                 buffers = [_buffer_of(p) for p in gather(local).payloads]
                 restored = None
-                residual = feedback.get(key) if decision.update else None
+                residual = feedback.get(key) if decision.update and callable(getattr(feedback, "get", None)) else None
                 if residual is not None and getattr(residual, "dtype", None) == getattr(prepared, "dtype", None):
                     workspace = workspaces.get(key, prepared, shape, config)
                     try:
                         if inplace_reduce_feedback(buffers, prepared, workspace, residual, config,
                                                    extension_status=extension_status, reduce=reduce):
-                            restored = workspace.reshape(-1)[:_numel(prepared)].reshape(shape)
+                            restored = _shaped(workspace, shape)
                     except RuntimeError:
                         restored = None
                 if restored is None:
                     restored = dequantize_reduce_tensors(buffers, shape, config, dtype=active_dtype,
                                                          extension_status=extension_status, reduce=reduce)
                     if decision.update:
-                        latest = feedback.get(key)
+                        latest = feedback.get(key) if callable(getattr(feedback, "get", None)) else None
                         if native_error_feedback_update is not None and latest is not None:
                             native_error_feedback_update(prepared, restored, latest)
                         else:
@@ -272,6 +376,7 @@ def create_ddp_comm_hook(
         future.set_result(result)
         return future
 
+    hook._ccdl_strategy_plan = plan
     hook._ccdl_requested_strategy = requested
     hook._ccdl_effective_strategy = effective
     _annotate(hook, annotation_provider)

@@ -301,6 +301,22 @@ CudaWorkspacePool = HipWorkspacePool
 # --------------------------------------------------------------------------- #
 # completions
 # --------------------------------------------------------------------------- #
+class NoopCompletion:
+    """Completion of work that needs no device ordering (host tensors, no GPU)."""
+
+    def query(self) -> bool:
+        return True
+
+    def wait(self) -> None:
+        return None
+
+    def wait_stream(self, stream: Any) -> None:
+        del stream
+
+    def synchronize(self) -> None:
+        return None
+
+
 class EventCompletion:
     """Completion of everything enqueued on ``stream`` so far, as a recorded device event."""
 
@@ -313,6 +329,10 @@ class EventCompletion:
     def query(self) -> bool:
         return bool(self._event.query())
 
+    def wait(self) -> None:
+        """Order torch's current stream after the event (device-side wait; the host does not block)."""
+        self._event.wait()
+
     def wait_stream(self, stream: Any) -> None:
         """Order ``stream`` after the event (device-side wait; the host does not block)."""
         stream.wait_event(self._event)
@@ -322,10 +342,16 @@ class EventCompletion:
 
 
 class EventCompletionManager:
-    """``record_for(value, stream=None)`` -> :class:`EventCompletion` (the protocol output leases consume)."""
+    """``record_for(value, stream=None)`` -> a completion (the protocol output leases and the asynchronous bucket
+    pipeline consume): an :class:`EventCompletion` for GPU values, a :class:`NoopCompletion` otherwise."""
 
-    def record_for(self, value: Any, *, stream: Any = None) -> EventCompletion:
-        del value
+    def record_for(self, value: Any, *, stream: Any = None) -> Any:
+        if stream is None and getattr(value, "is_cuda", None) is False:
+            return NoopCompletion()          # a host tensor: nothing on the device to order after
+        import torch
+
+        if not torch.cuda.is_available():
+            return NoopCompletion()
         return EventCompletion(stream)
 
 
