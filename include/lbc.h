@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define LBC_ABI_VERSION 2
+#define LBC_ABI_VERSION 3
 
 enum { LBC_OK = 0, LBC_UNSUPPORTED = 1, LBC_EINVAL = -1, LBC_ELAUNCH = -2 };
 
@@ -173,27 +173,30 @@ int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored
  *   compact == 0: all code bytes, then all scales  (quant_kernel_fp32.cuh:266-303);
  *   decode = float(code) * (float(scale) / 127), rounded to `dtype`
  *            (dequant_reduce_kernel.cu:38-69, dequant_kernel_fp32.cuh:81-104).
- * A payload holds G * (g + sizeof(dtype)) bytes and must be aligned to sizeof(dtype).
+ * `bit` = 4 selects 4-bit codes: multiplier 7 / max(scale, 1e-6), two's-complement nibbles packed
+ * 2*sizeof(dtype) to a word with the first code in the most significant nibble, decode by scale / 7
+ * (quant_pack_kernel.cu:103,120-130,145-158; ccdl_comm/csrc/quantization/inner.cuh:36-40,67-72).
+ * A payload holds G * (g*bit/8 + sizeof(dtype)) bytes and must be aligned to sizeof(dtype).
  * No golden bytes of an NVIDIA build exist in the reference, so byte equality with such a
  * build is argued from the source, not measured.
  */
 
 /* Bytes of one payload (quant_pack_kernel.cu:247-249); -1 for invalid arguments. */
-int64_t lbc_wire_payload_nbytes(int64_t numel, int group_size, int dtype);
+int64_t lbc_wire_payload_nbytes(int64_t numel, int group_size, int dtype, int bit);
 
 /*
  * Quantize x (+ residual, added in fp32 and rounded to dtype first) into one payload.
- * Replaces native inplace_quantize_pack and inplace_quantize for 8-bit linear codes
+ * Replaces native inplace_quantize_pack and inplace_quantize for linear 8- and 4-bit codes
  * (quant_pack_kernel.cu:220-275, ccdl_comm/csrc/pybind.cpp:36-63).  Ragged numel is zero padded.
  */
 int lbc_wire_quant_pack(const void *x, const void *residual, int dtype, int64_t numel, int group_size,
-                        int compact, uint8_t *payload, void *stream);
+                        int bit, int compact, uint8_t *payload, void *stream);
 
 /* As lbc_quant_pack_chunks, in this format: chunk d of ceil(numel/world) elements becomes the
  * payload at payloads + d*payload_stride (ccdl_comm/cuda/transports/compressed_reduce_scatter.py:72-94). */
 int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, int64_t numel, int world,
-                               int group_size, int compact, uint8_t *payloads, int64_t payload_stride,
-                               void *stream);
+                               int group_size, int bit, int compact, uint8_t *payloads,
+                               int64_t payload_stride, void *stream);
 
 /*
  * Decode one payload into out (reduce_op NONE) or combine it with the values already in out:
@@ -201,12 +204,12 @@ int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, i
  * opposite.  Replaces native inplace_dequantize (dequant_kernel_fp32.cuh:106-120,
  * dequant_kernel.cuh:46-60, pybind.cpp:64-90).
  */
-int lbc_wire_dequant(const uint8_t *payload, int64_t numel, int group_size, int compact, void *out, int dtype,
-                     int reduce_op, void *stream);
+int lbc_wire_dequant(const uint8_t *payload, int64_t numel, int group_size, int bit, int compact, void *out,
+                     int dtype, int reduce_op, void *stream);
 
 /* As lbc_dequant_chunks, in this format (ccdl_comm/communication/topology_transport.py:866-894). */
 int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world, int64_t shard_numel,
-                            int64_t total_numel, int group_size, int compact, void *out, int dtype,
+                            int64_t total_numel, int group_size, int bit, int compact, void *out, int dtype,
                             int reduce_op, void *stream);
 
 /*
@@ -214,7 +217,7 @@ int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int
  * fp32 starting from 0; with prepared/new_residual: new_residual = dtype(float(prepared) - the
  * unrounded fp32 value).  Replaces native try_inplace_dequantize_reduce_fused and
  * inplace_dequantize_reduce_mean_update_error_feedback (dequant_reduce_kernel.cu:71-134,150-221,
- * 315-430), which support group_size 64 and world <= 8 only; so does this.
+ * 315-430), which support 8-bit codes, group_size 64 and world <= 8 only; so does this.
  * fused_multiply_add != 0 accumulates with fma(code, step, sum), which is what nvcc's default
  * contraction makes of the reference's `sum += code * step`; 0 rounds the product first.
  */

@@ -9,6 +9,10 @@
 //                       (2-byte words for fp16/bf16, 4-byte words for fp32);
 //   compact layout    = per group [G code bytes][scale]; otherwise all code bytes, then all scales;
 //   decode            = float(code) * (float(scale) / 127), rounded to T.
+// 4-bit codes (BIT = 4; quant_pack_kernel.cu:103,120-130,145-158, inner.cuh:36-40): multiplier
+// 7 / max(scale, 1e-6), two's-complement nibbles, 2*sizeof(T) codes per word with the first code in
+// the most significant nibble, decode by scale / 7; quantize and single-payload decode only, as in
+// the reference (its fused reduce is 8-bit).
 //
 // Mapping: as in the portable-format kernels, one lane owns 16 bytes of the tensor (4 fp32 or
 // 8 half elements), a group sits in adjacent lanes of one DPP row, and every tile's loads are
@@ -69,11 +73,12 @@ __device__ __forceinline__ void store_elems(T *p, const T (&src)[VEC]) {
     else *reinterpret_cast<V *>(p) = v;
 }
 
-template <typename T> struct wire {
+template <typename T, int BIT = 8> struct wire {
     static constexpr int ITEM = sizeof(T);
-    static constexpr int VEC = 16 / ITEM;       // elements per lane
-    static constexpr int WORDS = VEC / 4;       // 32-bit code words per lane
+    static constexpr int VEC = BIT == 8 ? 16 / ITEM : 8;   // elements per lane (a 4-bit lane fills one 32-bit word)
+    static constexpr int WORDS = VEC * BIT / 32;            // 32-bit code words per lane
     static constexpr int TILE = kWave * VEC;
+    static constexpr float LEVELS = BIT == 8 ? 127.0f : 7.0f;
 };
 
 // Byte position of element k (0..3) inside its 32-bit word: fp32 payloads reverse all four
@@ -92,14 +97,65 @@ template <typename T> __device__ __forceinline__ int byte_in_group(int k) {
 // stream with the non-temporal hint (the hint would drop the line between its two uses).  Otherwise
 // the policy measured for the portable format applies: code stores follow the tensors' hint, code
 // loads are non-temporal only from four payloads on.
-template <typename T, int G, bool COMPACT> struct group_layout {
+template <typename T, int G, bool COMPACT, int BIT = 8> struct group_layout {
     static constexpr int ITEM = sizeof(T);
+    static constexpr int CB = G * BIT / 8;      // code bytes per group
     const int64_t groups;
-    __device__ __forceinline__ int64_t codes(int64_t group) const { return COMPACT ? group * (G + ITEM) : group * G; }
+    __device__ __forceinline__ int64_t codes(int64_t group) const { return COMPACT ? group * (CB + ITEM) : group * CB; }
     __device__ __forceinline__ int64_t scale(int64_t group) const {
-        return COMPACT ? group * (G + ITEM) + G : groups * G + group * ITEM;
+        return COMPACT ? group * (CB + ITEM) + CB : groups * CB + group * ITEM;
     }
 };
+
+// The VEC codes of one lane -> its 32-bit words, in the byte / nibble order of the format.
+template <typename T, int BIT, int VEC, int WORDS>
+__device__ __forceinline__ void pack_codes(const int (&c)[VEC], uint32_t (&words)[WORDS]) {
+    if constexpr (BIT == 8) {
+#pragma unroll
+        for (int k = 0; k < WORDS; ++k) {
+            if constexpr (sizeof(T) == 4) words[k] = pack4(c[4 * k + 3], c[4 * k + 2], c[4 * k + 1], c[4 * k]);
+            else words[k] = pack4(c[4 * k + 1], c[4 * k], c[4 * k + 3], c[4 * k + 2]);
+        }
+    } else {
+        static_assert(VEC == 8 && WORDS == 1, "a 4-bit lane owns one word");
+        uint32_t word = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            // fp32 payloads: one 32-bit word, first code on top; 16-bit payloads: two 16-bit words, low half first
+            const int shift = sizeof(T) == 4 ? 28 - 4 * i : 16 * (i / 4) + 12 - 4 * (i % 4);
+            word |= (static_cast<uint32_t>(c[i]) & 0xFu) << shift;
+        }
+        words[0] = word;
+    }
+}
+
+// Code i of the lane's words as a float.
+template <typename T, int BIT, int WORDS>
+__device__ __forceinline__ float unpack_code(const uint32_t (&words)[WORDS], int i) {
+    if constexpr (BIT == 8) {
+        return code_to_float(words[i / 4], byte_in_word<T>(i % 4));
+    } else {
+        const int top = sizeof(T) == 4 ? 4 * i : 16 - 16 * (i / 4) + 4 * (i % 4);   // left shift that puts the nibble on top
+        return static_cast<float>(static_cast<int32_t>(words[0] << top) >> 28);
+    }
+}
+
+// Code of element k of a group read from the group's code bytes (ragged-edge path).
+template <typename T, int BIT> __device__ __forceinline__ float code_at(const uint8_t *group_codes, int k) {
+    if constexpr (BIT == 8) {
+        return static_cast<float>(static_cast<int8_t>(group_codes[byte_in_group<T>(k)]));
+    } else {
+        constexpr int ITEM = sizeof(T), PER_WORD = 2 * ITEM;
+        const int in_word = k % PER_WORD;
+        const uint32_t byte = group_codes[(k / PER_WORD) * ITEM + (ITEM - 1 - in_word / 2)];
+        const uint32_t nibble = (in_word & 1) ? (byte & 0xFu) : (byte >> 4);
+        return static_cast<float>(static_cast<int32_t>(nibble << 28) >> 28);
+    }
+}
+
+// float(scale) / levels with IEEE rounding.
+template <int BIT> __device__ __forceinline__ float step_of(float stored);
+
 template <bool COMPACT, int NT, int WORLD> constexpr int payload_load_hint() { return COMPACT || WORLD < 4 ? kPlain : NT; }
 
 // float(scale) / 127 with IEEE rounding: the three-operation form proven exhaustively for
@@ -111,6 +167,9 @@ __device__ __forceinline__ float div127(float a) {
     const float q = __builtin_fmaf(r, c, q0);
     return (as_u32(a) & 0x7FFFFFFFu) == 0x7F800000u ? a : q;
 }
+
+template <> __device__ __forceinline__ float step_of<8>(float stored) { return div127(stored); }
+template <> __device__ __forceinline__ float step_of<4>(float stored) { return stored / 7.0f; }
 
 // a + b rounded once to T (what a native half / bfloat16 add returns): the float sum is turned
 // into a round-to-odd result with the exact error term, then rounded to T.
@@ -132,10 +191,10 @@ template <typename T> __device__ __forceinline__ float add_rounded_once(float a,
 // ---------------------------------------------------------------------------
 // quantize + pack (optionally x + residual), `world` chunks via blockIdx.y
 // ---------------------------------------------------------------------------
-template <typename T, int G, bool HAS_R, bool COMPACT, int NT>
+template <typename T, int G, int BIT, bool HAS_R, bool COMPACT, int NT>
 __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs a) {
     constexpr int PNT = COMPACT ? kPlain : NT;
-    using W = wire<T>;
+    using W = wire<T, BIT>;
     constexpr int VEC = W::VEC;
     constexpr int LPG = G / VEC;
     constexpr int UNROLL = 4;
@@ -150,7 +209,7 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
     valid = valid < 0 ? 0 : (valid > a.shard_numel ? a.shard_numel : valid);
     const int64_t groups = (a.shard_numel + G - 1) / G;
     const int64_t padded = groups * G;
-    const group_layout<T, G, COMPACT> at{groups};
+    const group_layout<T, G, COMPACT, BIT> at{groups};
 
     const T *__restrict__ x = static_cast<const T *>(a.x) + chunk_start;
     const T *__restrict__ r = HAS_R ? static_cast<const T *>(a.residual) + chunk_start : nullptr;
@@ -162,7 +221,7 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
     auto group_multiplier = [](uint32_t absmax_bits, float &absmax) {
         absmax = as_f32(group_max_bits<LPG>(absmax_bits));
         const float scale = absmax < 1.0e-6f ? 1.0e-6f : absmax;
-        return 127.0f / scale;
+        return W::LEVELS / scale;
     };
 
     if (block_first + BLOCK_ELEMS <= valid) {
@@ -194,14 +253,10 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
 #pragma unroll
             for (int i = 0; i < VEC; ++i) c[i] = cvt_i32(__builtin_rintf(p[i] * multiplier));
             uint32_t words[W::WORDS];
-#pragma unroll
-            for (int k = 0; k < W::WORDS; ++k) {
-                if constexpr (sizeof(T) == 4) words[k] = pack4(c[4 * k + 3], c[4 * k + 2], c[4 * k + 1], c[4 * k]);
-                else words[k] = pack4(c[4 * k + 1], c[4 * k], c[4 * k + 3], c[4 * k + 2]);
-            }
+            pack_codes<T, BIT, VEC, W::WORDS>(c, words);
             const int64_t group = e0[u] / G;
             const int k0 = static_cast<int>(e0[u] - group * G);
-            store_words<W::WORDS, sizeof(T), PNT>(payload + at.codes(group) + k0, words);
+            store_words<W::WORDS, sizeof(T), PNT>(payload + at.codes(group) + k0 * BIT / 8, words);
             if ((lane & (LPG - 1)) == 0) *reinterpret_cast<T *>(payload + at.scale(group)) = narrow<T>(absmax);
         }
         return;
@@ -228,44 +283,55 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
         }
         float absmax;
         const float multiplier = group_multiplier(m, absmax);   // every lane of the row takes part
-        if (e0 < padded) {
+        if (e0 < padded) {   // the lane's VEC elements lie inside the padded range together: whole words again
             const int64_t group = e0 / G;
             const int k0 = static_cast<int>(e0 - group * G);
-            uint8_t *codes = payload + at.codes(group);
+            int c[VEC];
 #pragma unroll
-            for (int i = 0; i < VEC; ++i)
-                codes[byte_in_group<T>(k0 + i)] = static_cast<uint8_t>(cvt_i32(__builtin_rintf(p[i] * multiplier)));
+            for (int i = 0; i < VEC; ++i) c[i] = cvt_i32(__builtin_rintf(p[i] * multiplier));
+            uint32_t words[W::WORDS];
+            pack_codes<T, BIT, VEC, W::WORDS>(c, words);
+            store_words<W::WORDS, sizeof(T), kPlain>(payload + at.codes(group) + k0 * BIT / 8, words);
             if ((lane & (LPG - 1)) == 0) *reinterpret_cast<T *>(payload + at.scale(group)) = narrow<T>(absmax);
         }
     }
 }
 
-template <typename T, int G, bool HAS_R, bool COMPACT>
+template <typename T, int G, int BIT, bool HAS_R, bool COMPACT>
 hipError_t launch_wire_quant_c(int mode, const WireQuantArgs &a, int world, hipStream_t stream) {
-    constexpr int BLOCK_ELEMS = wire<T>::TILE * kWavesPerBlock * 4;
+    constexpr int BLOCK_ELEMS = wire<T, BIT>::TILE * kWavesPerBlock * 4;
     const int64_t groups = (a.shard_numel + G - 1) / G;
     const int64_t blocks = (groups * G + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
     if (blocks == 0 || world == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL || world > 65535) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(world));
-    if (mode == kStream) hipLaunchKernelGGL((wire_quant_kernel<T, G, HAS_R, COMPACT, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
-    else hipLaunchKernelGGL((wire_quant_kernel<T, G, HAS_R, COMPACT, kPlain>), grid, dim3(kBlock), 0, stream, a);
+    if (mode == kStream) hipLaunchKernelGGL((wire_quant_kernel<T, G, BIT, HAS_R, COMPACT, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
+    else hipLaunchKernelGGL((wire_quant_kernel<T, G, BIT, HAS_R, COMPACT, kPlain>), grid, dim3(kBlock), 0, stream, a);
     return hipGetLastError();
 }
 
-template <typename T, int G, bool HAS_R>
-hipError_t launch_wire_quant_r(int mode, const WireQuantArgs &a, int world, hipStream_t stream) {
-    return a.compact ? launch_wire_quant_c<T, G, HAS_R, true>(mode, a, world, stream)
-                     : launch_wire_quant_c<T, G, HAS_R, false>(mode, a, world, stream);
+template <typename T, int G, int BIT>
+hipError_t launch_wire_quant_b(int mode, const WireQuantArgs &a, int world, hipStream_t stream) {
+    if (a.residual != nullptr)
+        return a.compact ? launch_wire_quant_c<T, G, BIT, true, true>(mode, a, world, stream)
+                         : launch_wire_quant_c<T, G, BIT, true, false>(mode, a, world, stream);
+    return a.compact ? launch_wire_quant_c<T, G, BIT, false, true>(mode, a, world, stream)
+                     : launch_wire_quant_c<T, G, BIT, false, false>(mode, a, world, stream);
+}
+
+template <typename T, int G>
+hipError_t launch_wire_quant_g(int bit, int mode, const WireQuantArgs &a, int world, hipStream_t stream) {
+    if (bit == 8) return launch_wire_quant_b<T, G, 8>(mode, a, world, stream);
+    if (bit == 4) return launch_wire_quant_b<T, G, 4>(mode, a, world, stream);
+    return hipErrorNotSupported;
 }
 
 template <typename T>
-hipError_t launch_wire_quant_t(int g, int mode, const WireQuantArgs &a, int world, hipStream_t s) {
-    const bool has_r = a.residual != nullptr;
+hipError_t launch_wire_quant_t(int g, int bit, int mode, const WireQuantArgs &a, int world, hipStream_t s) {
     switch (g) {
-        case 64: return has_r ? launch_wire_quant_r<T, 64, true>(mode, a, world, s) : launch_wire_quant_r<T, 64, false>(mode, a, world, s);
-        case 32: return has_r ? launch_wire_quant_r<T, 32, true>(mode, a, world, s) : launch_wire_quant_r<T, 32, false>(mode, a, world, s);
-        case 16: return has_r ? launch_wire_quant_r<T, 16, true>(mode, a, world, s) : launch_wire_quant_r<T, 16, false>(mode, a, world, s);
+        case 64: return launch_wire_quant_g<T, 64>(bit, mode, a, world, s);
+        case 32: return launch_wire_quant_g<T, 32>(bit, mode, a, world, s);
+        case 16: return launch_wire_quant_g<T, 16>(bit, mode, a, world, s);
         default: return hipErrorNotSupported;
     }
 }
@@ -412,10 +478,10 @@ template <typename T, int OP> __device__ __forceinline__ float combine_in(float 
     else return v;
 }
 
-template <typename T, int G, int OP, bool COMPACT, int NT>
+template <typename T, int G, int BIT, int OP, bool COMPACT, int NT>
 __global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArgs a) {
     constexpr int PNT = payload_load_hint<COMPACT, NT, 1>();
-    using W = wire<T>;
+    using W = wire<T, BIT>;
     constexpr int VEC = W::VEC;
     constexpr int UNROLL = 2;
     constexpr int BLOCK_ELEMS = W::TILE * kWavesPerBlock * UNROLL;
@@ -427,7 +493,7 @@ __global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArg
     int64_t valid = a.total_numel - chunk_start;
     valid = valid < 0 ? 0 : (valid > a.shard_numel ? a.shard_numel : valid);
     const int64_t groups = (a.shard_numel + G - 1) / G;
-    const group_layout<T, G, COMPACT> at{groups};
+    const group_layout<T, G, COMPACT, BIT> at{groups};
     const uint8_t *__restrict__ payload = a.payloads + chunk * a.payload_stride;
     T *__restrict__ out = static_cast<T *>(a.out) + chunk_start;
     const int64_t block_first = static_cast<int64_t>(blockIdx.x) * BLOCK_ELEMS;
@@ -442,17 +508,17 @@ __global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArg
             e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
             const int64_t group = e0[u] / G;
             const int k0 = static_cast<int>(e0[u] - group * G);
-            load_words<W::WORDS, sizeof(T), PNT>(payload + at.codes(group) + k0, words[u]);
+            load_words<W::WORDS, sizeof(T), PNT>(payload + at.codes(group) + k0 * BIT / 8, words[u]);
             stored[u] = *reinterpret_cast<const T *>(payload + at.scale(group));
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             T o[VEC];
             if constexpr (OP != 0) load_elems<T, VEC, NT>(out + e0[u], o);
-            const float step = div127(widen(stored[u]));
+            const float step = step_of<BIT>(widen(stored[u]));
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
-                float v = round_through<T>(code_to_float(words[u][i / 4], byte_in_word<T>(i % 4)) * step);
+                float v = round_through<T>(unpack_code<T, BIT, W::WORDS>(words[u], i) * step);
                 if constexpr (OP != 0) v = combine_in<T, OP>(widen(o[i]), v);
                 o[i] = narrow<T>(v);
             }
@@ -468,62 +534,68 @@ __global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArg
             if (e >= valid) break;
             const int64_t group = e / G;
             const int k = static_cast<int>(e - group * G);
-            const float step = div127(widen(*reinterpret_cast<const T *>(payload + at.scale(group))));
-            const float code = static_cast<float>(static_cast<int8_t>(payload[at.codes(group) + byte_in_group<T>(k)]));
-            float v = round_through<T>(code * step);
+            const float step = step_of<BIT>(widen(*reinterpret_cast<const T *>(payload + at.scale(group))));
+            float v = round_through<T>(code_at<T, BIT>(payload + at.codes(group), k) * step);
             if constexpr (OP != 0) v = combine_in<T, OP>(widen(out[e]), v);
             out[e] = narrow<T>(v);
         }
     }
 }
 
-template <typename T, int G, int OP, bool COMPACT>
+template <typename T, int G, int BIT, int OP, bool COMPACT>
 hipError_t launch_wire_decode_c(int mode, const WireDecodeArgs &a, int world, hipStream_t stream) {
-    constexpr int BLOCK_ELEMS = wire<T>::TILE * kWavesPerBlock * 2;
+    constexpr int BLOCK_ELEMS = wire<T, BIT>::TILE * kWavesPerBlock * 2;
     const int64_t blocks = (a.shard_numel + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
     if (blocks == 0 || world == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL || world > 65535) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(world));
-    if (mode == kStream) hipLaunchKernelGGL((wire_decode_kernel<T, G, OP, COMPACT, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
-    else hipLaunchKernelGGL((wire_decode_kernel<T, G, OP, COMPACT, kPlain>), grid, dim3(kBlock), 0, stream, a);
+    if (mode == kStream) hipLaunchKernelGGL((wire_decode_kernel<T, G, BIT, OP, COMPACT, kNonTemporal>), grid, dim3(kBlock), 0, stream, a);
+    else hipLaunchKernelGGL((wire_decode_kernel<T, G, BIT, OP, COMPACT, kPlain>), grid, dim3(kBlock), 0, stream, a);
     return hipGetLastError();
 }
 
-template <typename T, int G, int OP>
+template <typename T, int G, int BIT, int OP>
 hipError_t launch_wire_decode_op(int mode, const WireDecodeArgs &a, int world, hipStream_t stream) {
-    return a.compact ? launch_wire_decode_c<T, G, OP, true>(mode, a, world, stream)
-                     : launch_wire_decode_c<T, G, OP, false>(mode, a, world, stream);
+    return a.compact ? launch_wire_decode_c<T, G, BIT, OP, true>(mode, a, world, stream)
+                     : launch_wire_decode_c<T, G, BIT, OP, false>(mode, a, world, stream);
 }
 
-template <typename T, int G>
-hipError_t launch_wire_decode_g(int op, int mode, const WireDecodeArgs &a, int world, hipStream_t s) {
+template <typename T, int G, int BIT>
+hipError_t launch_wire_decode_b(int op, int mode, const WireDecodeArgs &a, int world, hipStream_t s) {
     switch (op) {
-        case 0: return launch_wire_decode_op<T, G, 0>(mode, a, world, s);
-        case 1: return launch_wire_decode_op<T, G, 1>(mode, a, world, s);
-        case 2: return launch_wire_decode_op<T, G, 2>(mode, a, world, s);
-        case 3: return launch_wire_decode_op<T, G, 3>(mode, a, world, s);
+        case 0: return launch_wire_decode_op<T, G, BIT, 0>(mode, a, world, s);
+        case 1: return launch_wire_decode_op<T, G, BIT, 1>(mode, a, world, s);
+        case 2: return launch_wire_decode_op<T, G, BIT, 2>(mode, a, world, s);
+        case 3: return launch_wire_decode_op<T, G, BIT, 3>(mode, a, world, s);
         default: return hipErrorNotSupported;
     }
 }
 
+template <typename T, int G>
+hipError_t launch_wire_decode_g(int bit, int op, int mode, const WireDecodeArgs &a, int world, hipStream_t s) {
+    if (bit == 8) return launch_wire_decode_b<T, G, 8>(op, mode, a, world, s);
+    if (bit == 4) return launch_wire_decode_b<T, G, 4>(op, mode, a, world, s);
+    return hipErrorNotSupported;
+}
+
 template <typename T>
-hipError_t launch_wire_decode_t(int g, int op, int mode, const WireDecodeArgs &a, int world, hipStream_t s) {
+hipError_t launch_wire_decode_t(int g, int bit, int op, int mode, const WireDecodeArgs &a, int world, hipStream_t s) {
     switch (g) {
-        case 64: return launch_wire_decode_g<T, 64>(op, mode, a, world, s);
-        case 32: return launch_wire_decode_g<T, 32>(op, mode, a, world, s);
-        case 16: return launch_wire_decode_g<T, 16>(op, mode, a, world, s);
+        case 64: return launch_wire_decode_g<T, 64>(bit, op, mode, a, world, s);
+        case 32: return launch_wire_decode_g<T, 32>(bit, op, mode, a, world, s);
+        case 16: return launch_wire_decode_g<T, 16>(bit, op, mode, a, world, s);
         default: return hipErrorNotSupported;
     }
 }
 
 }  // namespace
 
-hipError_t launch_wire_quant(int dtype, int group_size, int mode, const WireQuantArgs &args, int world,
+hipError_t launch_wire_quant(int dtype, int group_size, int bit, int mode, const WireQuantArgs &args, int world,
                              hipStream_t stream) {
     switch (dtype) {
-        case kF32: return launch_wire_quant_t<float>(group_size, mode, args, world, stream);
-        case kF16: return launch_wire_quant_t<f16>(group_size, mode, args, world, stream);
-        case kBF16: return launch_wire_quant_t<bf16>(group_size, mode, args, world, stream);
+        case kF32: return launch_wire_quant_t<float>(group_size, bit, mode, args, world, stream);
+        case kF16: return launch_wire_quant_t<f16>(group_size, bit, mode, args, world, stream);
+        case kBF16: return launch_wire_quant_t<bf16>(group_size, bit, mode, args, world, stream);
         default: return hipErrorNotSupported;
     }
 }
@@ -538,12 +610,12 @@ hipError_t launch_wire_reduce(int dtype, int group_size, int world, bool fused_m
     }
 }
 
-hipError_t launch_wire_decode(int dtype, int group_size, int reduce_op, int mode, const WireDecodeArgs &args,
+hipError_t launch_wire_decode(int dtype, int group_size, int bit, int reduce_op, int mode, const WireDecodeArgs &args,
                               int world, hipStream_t stream) {
     switch (dtype) {
-        case kF32: return launch_wire_decode_t<float>(group_size, reduce_op, mode, args, world, stream);
-        case kF16: return launch_wire_decode_t<f16>(group_size, reduce_op, mode, args, world, stream);
-        case kBF16: return launch_wire_decode_t<bf16>(group_size, reduce_op, mode, args, world, stream);
+        case kF32: return launch_wire_decode_t<float>(group_size, bit, reduce_op, mode, args, world, stream);
+        case kF16: return launch_wire_decode_t<f16>(group_size, bit, reduce_op, mode, args, world, stream);
+        case kBF16: return launch_wire_decode_t<bf16>(group_size, bit, reduce_op, mode, args, world, stream);
         default: return hipErrorNotSupported;
     }
 }

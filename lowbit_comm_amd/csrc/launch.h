@@ -96,11 +96,12 @@ hipError_t launch_ef_update(int p_dtype, int t_dtype, int r_dtype, int mode, con
 
 // Wire-format launches take mode 1 (plain) or 2 (non-temporal); they have no alignment demands
 // beyond element alignment.
-hipError_t launch_wire_quant(int dtype, int group_size, int mode, const WireQuantArgs &args, int world,
+// `bit` is 8 or 4 for quantize and decode; the fused reduce exists for 8-bit codes only.
+hipError_t launch_wire_quant(int dtype, int group_size, int bit, int mode, const WireQuantArgs &args, int world,
                              hipStream_t stream);
 hipError_t launch_wire_reduce(int dtype, int group_size, int world, bool fused_multiply_add, int mode,
                               const WireReduceArgs &args, hipStream_t stream);
-hipError_t launch_wire_decode(int dtype, int group_size, int reduce_op, int mode, const WireDecodeArgs &args,
+hipError_t launch_wire_decode(int dtype, int group_size, int bit, int reduce_op, int mode, const WireDecodeArgs &args,
                               int world, hipStream_t stream);
 
 }  // namespace lbc

@@ -291,22 +291,23 @@ int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored
 }
 
 // ---- payload format of the reference's CUDA extension -------------------------------------
-int64_t lbc_wire_payload_nbytes(int64_t numel, int group_size, int dtype) {
-    if (numel < 0 || !valid_group(group_size) || !valid_dtype(dtype)) return -1;
+int64_t lbc_wire_payload_nbytes(int64_t numel, int group_size, int dtype, int bit) {
+    if (numel < 0 || !valid_group(group_size) || !valid_dtype(dtype) || (bit != 8 && bit != 4)) return -1;
     const int64_t groups = numel == 0 ? 0 : (numel + group_size - 1) / group_size;
-    return groups * (group_size + dtype_size(dtype));
+    return groups * (group_size * bit / 8 + dtype_size(dtype));
 }
 
 int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, int64_t numel, int world,
-                               int group_size, int compact, uint8_t *payloads, int64_t payload_stride, void *stream) {
+                               int group_size, int bit, int compact, uint8_t *payloads, int64_t payload_stride,
+                               void *stream) {
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
     if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported dtype %d", dtype);
-    if (!valid_group(group_size) || world > 65535) return LBC_UNSUPPORTED;
+    if (!valid_group(group_size) || world > 65535 || (bit != 8 && bit != 4)) return LBC_UNSUPPORTED;
     const int64_t shard = (numel + world - 1) / world;
     if (shard == 0) return LBC_OK;
     const int item = dtype_size(dtype);
-    const int64_t payload_bytes = lbc_wire_payload_nbytes(shard, group_size, dtype);
+    const int64_t payload_bytes = lbc_wire_payload_nbytes(shard, group_size, dtype, bit);
     if (x == nullptr || payloads == nullptr) return fail(LBC_EINVAL, "input and payloads must not be null");
     if (world > 1 && (payload_stride < payload_bytes || payload_stride % item != 0))
         return fail(LBC_EINVAL, "payload_stride must be a multiple of %d and >= %lld", item, (long long)payload_bytes);
@@ -322,29 +323,29 @@ int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, i
     a.payload_stride = world > 1 ? payload_stride : 0;
     a.compact = compact != 0;
     const int64_t moved = numel * (item * (residual ? 2 : 1) + 1);
-    return finish(lbc::launch_wire_quant(dtype, group_size, pick_mode(true, moved), a, world,
+    return finish(lbc::launch_wire_quant(dtype, group_size, bit, pick_mode(true, moved), a, world,
                                          static_cast<hipStream_t>(stream)),
                   "lbc_wire_quant_pack");
 }
 
-int lbc_wire_quant_pack(const void *x, const void *residual, int dtype, int64_t numel, int group_size, int compact,
-                        uint8_t *payload, void *stream) {
-    return lbc_wire_quant_pack_chunks(x, residual, dtype, numel, 1, group_size, compact, payload, 0, stream);
+int lbc_wire_quant_pack(const void *x, const void *residual, int dtype, int64_t numel, int group_size, int bit,
+                        int compact, uint8_t *payload, void *stream) {
+    return lbc_wire_quant_pack_chunks(x, residual, dtype, numel, 1, group_size, bit, compact, payload, 0, stream);
 }
 
 int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world, int64_t shard_numel,
-                            int64_t total_numel, int group_size, int compact, void *out, int dtype, int reduce_op,
-                            void *stream) {
+                            int64_t total_numel, int group_size, int bit, int compact, void *out, int dtype,
+                            int reduce_op, void *stream) {
     if (shard_numel < 0 || total_numel < 0) return fail(LBC_EINVAL, "element counts must be >= 0");
     if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
     if (total_numel > shard_numel * world) return fail(LBC_EINVAL, "total_numel exceeds world * shard_numel");
     if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported dtype %d", dtype);
     if (reduce_op < LBC_REDUCE_NONE || reduce_op > LBC_REDUCE_MIN)
         return fail(LBC_EINVAL, "unsupported reduce op %d", reduce_op);
-    if (!valid_group(group_size) || world > 65535) return LBC_UNSUPPORTED;
+    if (!valid_group(group_size) || world > 65535 || (bit != 8 && bit != 4)) return LBC_UNSUPPORTED;
     if (shard_numel == 0 || total_numel == 0) return LBC_OK;
     const int item = dtype_size(dtype);
-    const int64_t payload_bytes = lbc_wire_payload_nbytes(shard_numel, group_size, dtype);
+    const int64_t payload_bytes = lbc_wire_payload_nbytes(shard_numel, group_size, dtype, bit);
     if (payloads == nullptr || out == nullptr) return fail(LBC_EINVAL, "payloads and out must not be null");
     if (world > 1 && (payload_stride < payload_bytes || payload_stride % item != 0))
         return fail(LBC_EINVAL, "payload_stride must be a multiple of %d and >= %lld", item, (long long)payload_bytes);
@@ -358,14 +359,15 @@ int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int
     a.payload_stride = world > 1 ? payload_stride : 0;
     a.compact = compact != 0;
     const int64_t moved = total_numel * (item * (reduce_op == LBC_REDUCE_NONE ? 1 : 2) + 1);
-    return finish(lbc::launch_wire_decode(dtype, group_size, reduce_op, pick_mode(true, moved), a, world,
+    return finish(lbc::launch_wire_decode(dtype, group_size, bit, reduce_op, pick_mode(true, moved), a, world,
                                           static_cast<hipStream_t>(stream)),
                   "lbc_wire_dequant");
 }
 
-int lbc_wire_dequant(const uint8_t *payload, int64_t numel, int group_size, int compact, void *out, int dtype,
-                     int reduce_op, void *stream) {
-    return lbc_wire_dequant_chunks(payload, 0, 1, numel, numel, group_size, compact, out, dtype, reduce_op, stream);
+int lbc_wire_dequant(const uint8_t *payload, int64_t numel, int group_size, int bit, int compact, void *out,
+                     int dtype, int reduce_op, void *stream) {
+    return lbc_wire_dequant_chunks(payload, 0, 1, numel, numel, group_size, bit, compact, out, dtype, reduce_op,
+                                   stream);
 }
 
 int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t numel, int group_size, int compact,

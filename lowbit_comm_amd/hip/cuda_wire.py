@@ -19,9 +19,9 @@ from lowbit_comm_amd.hip.ops import (MAX_PAYLOADS, REDUCE_OPS, BoundLaunch, _dev
                                      _require, num_groups)
 
 
-def payload_nbytes(numel: int, dtype: torch.dtype, group_size: int = 64) -> int:
-    """``G * (g + element size)`` (ccdl_comm/csrc/quantization/quant_pack_kernel.cu:247-249)."""
-    return num_groups(numel, group_size) * (group_size + torch.empty((), dtype=dtype).element_size())
+def payload_nbytes(numel: int, dtype: torch.dtype, group_size: int = 64, bit: int = 8) -> int:
+    """``G * (g*bit/8 + element size)`` (ccdl_comm/csrc/quantization/quant_pack_kernel.cu:247-249)."""
+    return num_groups(numel, group_size) * (group_size * bit // 8 + torch.empty((), dtype=dtype).element_size())
 
 
 def _payload_rows(t: torch.Tensor, device: torch.device) -> None:
@@ -37,78 +37,79 @@ def _payload(t: torch.Tensor, name: str, device: torch.device, nbytes: int) -> N
 
 
 def bind_quant_pack(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64, compact: bool = True,
-                    residual: torch.Tensor | None = None) -> BoundLaunch:
+                    residual: torch.Tensor | None = None, bit: int = 8) -> BoundLaunch:
     lib = load_library()
     code = _float_tensor(x, "input")
-    _payload(payload, "output", x.device, payload_nbytes(x.numel(), x.dtype, group_size))
+    _payload(payload, "output", x.device, payload_nbytes(x.numel(), x.dtype, group_size, bit))
     if residual is not None:
         _float_tensor(residual, "residual", x.device)
         _require(residual.dtype == x.dtype, "input and residual must have the same dtype")
         _require(residual.numel() == x.numel(), "input and residual must have the same number of elements")
-    args = (_ptr(x), _ptr(residual), code, x.numel(), group_size, int(compact), _ptr(payload))
+    args = (_ptr(x), _ptr(residual), code, x.numel(), group_size, int(bit), int(compact), _ptr(payload))
     return BoundLaunch(lib.lbc_wire_quant_pack, args, x.device, lib, (x, residual, payload))
 
 
 def quant_pack_into(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64, compact: bool = True,
-                    residual: torch.Tensor | None = None) -> bool:
+                    residual: torch.Tensor | None = None, bit: int = 8) -> bool:
     """``payload = encode(x [+ residual])``; replaces native ``inplace_quantize_pack`` / ``inplace_quantize``."""
-    return bind_quant_pack(x, payload, group_size=group_size, compact=compact, residual=residual)()
+    return bind_quant_pack(x, payload, group_size=group_size, compact=compact, residual=residual, bit=bit)()
 
 
 def quant_pack(x: torch.Tensor, *, group_size: int = 64, compact: bool = True,
-               residual: torch.Tensor | None = None) -> torch.Tensor:
-    payload = torch.empty(payload_nbytes(x.numel(), x.dtype, group_size), dtype=torch.uint8, device=x.device)
-    if not quant_pack_into(x, payload, group_size=group_size, compact=compact, residual=residual):
-        raise RuntimeError(f"no kernel for group_size={group_size}")
+               residual: torch.Tensor | None = None, bit: int = 8) -> torch.Tensor:
+    payload = torch.empty(payload_nbytes(x.numel(), x.dtype, group_size, bit), dtype=torch.uint8, device=x.device)
+    if not quant_pack_into(x, payload, group_size=group_size, compact=compact, residual=residual, bit=bit):
+        raise RuntimeError(f"no kernel for group_size={group_size}, bit={bit}")
     return payload
 
 
 def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64,
-                           compact: bool = True, residual: torch.Tensor | None = None) -> BoundLaunch:
+                           compact: bool = True, residual: torch.Tensor | None = None, bit: int = 8) -> BoundLaunch:
     """``payloads`` is a ``(world, stride)`` uint8 tensor; row d receives chunk d of ``ceil(numel/world)`` elements."""
     lib = load_library()
     code = _float_tensor(x, "input")
     _payload_rows(payloads, x.device)
     _require(payloads.shape[0] == world, "payloads must have one row per chunk")
     shard = -(-x.numel() // world) if x.numel() else 0
-    _require(payloads.shape[1] >= payload_nbytes(shard, x.dtype, group_size), "payload rows are too small")
+    _require(payloads.shape[1] >= payload_nbytes(shard, x.dtype, group_size, bit), "payload rows are too small")
     if residual is not None:
         _float_tensor(residual, "residual", x.device)
         _require(residual.dtype == x.dtype and residual.numel() == x.numel(),
                  "input and residual must have the same dtype and number of elements")
-    args = (_ptr(x), _ptr(residual), code, x.numel(), world, group_size, int(compact), _ptr(payloads),
+    args = (_ptr(x), _ptr(residual), code, x.numel(), world, group_size, int(bit), int(compact), _ptr(payloads),
             payloads.stride(0))
     return BoundLaunch(lib.lbc_wire_quant_pack_chunks, args, x.device, lib, (x, residual, payloads))
 
 
 def bind_dequant(payload: torch.Tensor, out: torch.Tensor, *, numel: int | None = None, group_size: int = 64,
-                 compact: bool = True, reduce_op: str = "none") -> BoundLaunch:
+                 compact: bool = True, reduce_op: str = "none", bit: int = 8) -> BoundLaunch:
     lib = load_library()
     code = _float_tensor(out, "output")
     n = out.numel() if numel is None else int(numel)
     _require(0 <= n <= out.numel(), "numel exceeds the output size")
     _require(reduce_op in REDUCE_OPS, f"unsupported reduce op {reduce_op!r}")
-    _payload(payload, "input", out.device, payload_nbytes(n, out.dtype, group_size))
-    args = (_ptr(payload), n, group_size, int(compact), _ptr(out), code, REDUCE_OPS[reduce_op])
+    _payload(payload, "input", out.device, payload_nbytes(n, out.dtype, group_size, bit))
+    args = (_ptr(payload), n, group_size, int(bit), int(compact), _ptr(out), code, REDUCE_OPS[reduce_op])
     return BoundLaunch(lib.lbc_wire_dequant, args, out.device, lib, (payload, out))
 
 
 def dequant_into(payload: torch.Tensor, out: torch.Tensor, *, numel: int | None = None, group_size: int = 64,
-                 compact: bool = True, reduce_op: str = "none") -> bool:
+                 compact: bool = True, reduce_op: str = "none", bit: int = 8) -> bool:
     """Decode into ``out`` or combine with it (``sum``/``max``/``min``); replaces native ``inplace_dequantize``."""
-    return bind_dequant(payload, out, numel=numel, group_size=group_size, compact=compact, reduce_op=reduce_op)()
+    return bind_dequant(payload, out, numel=numel, group_size=group_size, compact=compact, reduce_op=reduce_op,
+                        bit=bit)()
 
 
 def bind_dequant_chunks(payloads: torch.Tensor, out: torch.Tensor, shard_numel: int, *, group_size: int = 64,
-                        compact: bool = True) -> BoundLaunch:
+                        compact: bool = True, bit: int = 8) -> BoundLaunch:
     lib = load_library()
     code = _float_tensor(out, "output")
     _payload_rows(payloads, out.device)
     world = payloads.shape[0]
     _require(out.numel() <= world * shard_numel, "output is larger than world * shard_numel")
-    _require(payloads.shape[1] >= payload_nbytes(shard_numel, out.dtype, group_size), "payload rows are too small")
-    args = (_ptr(payloads), payloads.stride(0), world, shard_numel, out.numel(), group_size, int(compact), _ptr(out),
-            code, REDUCE_OPS["none"])
+    _require(payloads.shape[1] >= payload_nbytes(shard_numel, out.dtype, group_size, bit), "payload rows are too small")
+    args = (_ptr(payloads), payloads.stride(0), world, shard_numel, out.numel(), group_size, int(bit), int(compact),
+            _ptr(out), code, REDUCE_OPS["none"])
     return BoundLaunch(lib.lbc_wire_dequant_chunks, args, out.device, lib, (payloads, out))
 
 

@@ -10,8 +10,9 @@ load this module on gfx950 with ranks that load the CUDA extension.  The portabl
 Kept from the reference: the fused reduce runs only for group size 64, at most 8 payloads and an element
 count that is a multiple of 64 (``dequant_reduce_kernel.cu:243-262``); otherwise payloads are decoded one
 by one and added in the tensor dtype (``pybind.cpp:39-56``), which rounds differently, so eligibility is
-mirrored exactly.  4-bit codes, top-k side channels, stochastic rounding and the non-linear maps have no
-kernel here: ``inplace_quantize_pack`` and the fused calls return ``False`` for them, the others raise.
+mirrored exactly.  Linear 8- and 4-bit codes are implemented (4-bit: quantize and decode; reduces go through the
+decode-and-add chain, as in the reference).  Top-k side channels, stochastic rounding and the non-linear maps
+have no kernel here: ``inplace_quantize_pack`` and the fused calls return ``False`` for them, the others raise.
 """
 from __future__ import annotations
 
@@ -21,18 +22,31 @@ import torch
 
 from lowbit_comm_amd.hip import cuda_wire, ops
 from lowbit_comm_amd.hip.library import load_library
-from lowbit_comm_amd.hip.native_module import (DType, QuantType, ReduceOP, _OP_NAME, _TORCH_OF, _check_payload,
-                                               _policy_supported, _require_policy)
+from lowbit_comm_amd.hip.native_module import DType, QuantType, ReduceOP, _OP_NAME, _TORCH_OF, _check_payload
 
 FUSED_GROUP_SIZE = 64
+FUSED_BIT = 8
+
+
+def _policy_supported(group_size: int, topk: int, stochastic: bool, bit: int, quant_type) -> bool:
+    return (group_size in (16, 32, 64) and topk == 0 and not stochastic and bit in (4, 8)
+            and int(quant_type) == int(QuantType.Linear))
+
+
+def _require_policy(group_size, topk, stochastic, bit, quant_type) -> None:
+    if not _policy_supported(group_size, topk, stochastic, bit, quant_type):
+        raise RuntimeError(
+            "the HIP codec for the CUDA byte format supports linear 8- and 4-bit quantization with group_size "
+            f"16/32/64, topk=0, no stochastic rounding; got group_size={group_size} topk={topk} "
+            f"stochastic={stochastic} bit={bit} quant_type={getattr(quant_type, 'name', quant_type)}")
 
 
 def _item(dtype: torch.dtype) -> int:
     return 4 if dtype == torch.float32 else 2
 
 
-def _padded_numel(buffer: torch.Tensor, group_size: int, dtype: torch.dtype, name: str = "input") -> int:
-    per_group = group_size + _item(dtype)
+def _padded_numel(buffer: torch.Tensor, group_size: int, dtype: torch.dtype, bit: int = 8, name: str = "input") -> int:
+    per_group = group_size * bit // 8 + _item(dtype)
     if buffer.numel() % per_group != 0:
         raise RuntimeError(f"{name} has an invalid quantized payload size")
     return buffer.numel() // per_group * group_size
@@ -55,14 +69,14 @@ class HipCudaWireModule:
     # ---- quantize ------------------------------------------------------------------------------
     def quantize(self, input, group_size, topk, stochastic, bit, quant_type, compact):
         _require_policy(group_size, topk, stochastic, bit, quant_type)
-        output = torch.empty(cuda_wire.payload_nbytes(input.numel(), input.dtype, group_size), dtype=torch.uint8,
+        output = torch.empty(cuda_wire.payload_nbytes(input.numel(), input.dtype, group_size, bit), dtype=torch.uint8,
                              device=input.device)
         self.inplace_quantize(input, output, group_size, topk, stochastic, bit, quant_type, compact)
         return output
 
     def inplace_quantize(self, input, output, group_size, topk, stochastic, bit, quant_type, compact) -> None:
         _require_policy(group_size, topk, stochastic, bit, quant_type)
-        if not self._quantize(input, output, None, group_size, compact):
+        if not self._quantize(input, output, None, group_size, compact, bit):
             raise RuntimeError(f"no HIP quantize kernel for input dtype {input.dtype}")
 
     def inplace_quantize_pack(self, input, output, residual, group_size, topk, stochastic, bit, quant_type,
@@ -76,9 +90,9 @@ class HipCudaWireModule:
                 raise RuntimeError("input and residual must have the same dtype")
             if residual.numel() != input.numel():
                 raise RuntimeError("input and residual must have the same number of elements")
-        return self._quantize(input, output, residual, group_size, True)
+        return self._quantize(input, output, residual, group_size, True, bit)
 
-    def _quantize(self, input, output, residual, group_size, compact) -> bool:
+    def _quantize(self, input, output, residual, group_size, compact, bit) -> bool:
         _check_payload(output, "output")
         if not isinstance(input, torch.Tensor) or not input.is_cuda:
             raise RuntimeError("input must be a GPU tensor")
@@ -86,20 +100,21 @@ class HipCudaWireModule:
             raise RuntimeError("input must be contiguous")
         if output.device != input.device:
             raise RuntimeError("input and output must be on the same device")
-        if output.numel() != cuda_wire.payload_nbytes(input.numel(), input.dtype, group_size):
+        if output.numel() != cuda_wire.payload_nbytes(input.numel(), input.dtype, group_size, bit):
             raise RuntimeError("output has an invalid quantized payload size")
         if input.numel() == 0:
             return True
         flat_residual = None if residual is None else residual.reshape(-1)
         return cuda_wire.quant_pack_into(input.reshape(-1), output.reshape(-1), group_size=group_size,
-                                         compact=bool(compact), residual=flat_residual)
+                                         compact=bool(compact), residual=flat_residual, bit=bit)
 
     # ---- dequantize -----------------------------------------------------------------------------
     def dequantize(self, input, group_size, topk, bit, reduce_op, quant_type, dtype, compact):
         _require_policy(group_size, topk, False, bit, quant_type)
         _check_payload(input, "input")
         torch_dtype = _TORCH_OF[DType(int(dtype))]
-        output = torch.empty(_padded_numel(input, group_size, torch_dtype), dtype=torch_dtype, device=input.device)
+        output = torch.empty(_padded_numel(input, group_size, torch_dtype, bit), dtype=torch_dtype,
+                             device=input.device)
         if int(reduce_op) != int(ReduceOP.NONE):
             output.zero_()
         self.inplace_dequantize(input, output, group_size, topk, bit, reduce_op, quant_type, compact)
@@ -109,13 +124,13 @@ class HipCudaWireModule:
         _require_policy(group_size, topk, False, bit, quant_type)
         _check_payload(input, "input")
         flat = output.reshape(-1)
-        numel = min(flat.numel(), _padded_numel(input, group_size, output.dtype))
+        numel = min(flat.numel(), _padded_numel(input, group_size, output.dtype, bit))
         payload = input.reshape(-1)
-        expected = cuda_wire.payload_nbytes(numel, output.dtype, group_size)
+        expected = cuda_wire.payload_nbytes(numel, output.dtype, group_size, bit)
         if payload.numel() != expected:
             raise RuntimeError("input has an invalid quantized payload size")
         if not cuda_wire.dequant_into(payload, flat, numel=numel, group_size=group_size, compact=bool(compact),
-                                      reduce_op=_OP_NAME[ReduceOP(int(reduce_op))]):
+                                      reduce_op=_OP_NAME[ReduceOP(int(reduce_op))], bit=bit):
             raise RuntimeError(f"no HIP dequantize kernel for output dtype {output.dtype}")
 
     # ---- dequantize + reduce ------------------------------------------------------------------
@@ -123,7 +138,7 @@ class HipCudaWireModule:
         """``can_use_fused_dequant_reduce`` (dequant_reduce_kernel.cu:243-262)."""
         if not 1 <= len(inputs) <= ops.MAX_PAYLOADS:
             return False
-        if group_size != FUSED_GROUP_SIZE or not _policy_supported(group_size, topk, False, bit, quant_type):
+        if group_size != FUSED_GROUP_SIZE or bit != FUSED_BIT or not _policy_supported(group_size, topk, False, bit, quant_type):
             return False
         if not isinstance(output, torch.Tensor) or not output.is_cuda or not output.is_contiguous():
             return False
@@ -162,7 +177,7 @@ class HipCudaWireModule:
             raise RuntimeError("inputs must not be empty")
         _check_payload(inputs[0], "input")
         torch_dtype = _TORCH_OF[DType(int(dtype))]
-        output = torch.empty(_padded_numel(inputs[0], group_size, torch_dtype), dtype=torch_dtype,
+        output = torch.empty(_padded_numel(inputs[0], group_size, torch_dtype, bit), dtype=torch_dtype,
                              device=inputs[0].device)
         self.inplace_dequantize_reduce(inputs, output, group_size, topk, bit, quant_type, compact)
         return output
@@ -227,7 +242,7 @@ class HipCudaWireModule:
         if divisor <= 0:
             raise RuntimeError("divisor must be > 0")
         torch_dtype = _TORCH_OF[DType(int(dtype))]
-        restored = torch.empty(_padded_numel(inputs[0], group_size, torch_dtype), dtype=torch_dtype,
+        restored = torch.empty(_padded_numel(inputs[0], group_size, torch_dtype, bit), dtype=torch_dtype,
                                device=inputs[0].device)
         if self.inplace_dequantize_reduce_mean_update_error_feedback(
                 inputs, prepared, restored, residual, group_size, topk, bit, quant_type, compact, divisor):

@@ -33,6 +33,11 @@ CUDA device exists here, so agreement with an actual NVIDIA build is unpinned;
 the accumulate in ``reduce_payloads`` in particular depends on whether nvcc fuses
 ``sum += code * scale`` into an FMA (its default), which is why it is a switch.
 
+4-bit codes (``bit=4``; quant_pack_kernel.cu:103,120-130,145-158; inner.cuh:36-40,67-72): the multiplier is
+``7 / max(scale, 1e-6)``, codes are clamped to +-7 and stored as two's-complement nibbles, four to a 16-bit
+word or eight to a 32-bit word with the first element in the most significant nibble; decode multiplies the
+sign-extended nibble by ``scale / 7``.  The reference has no fused reduce for them.
+
 Arrays: fp32 -> ``float32``, fp16 -> ``float16``, bf16 -> ``uint16`` bit patterns.
 """
 from __future__ import annotations
@@ -70,9 +75,32 @@ def num_groups(numel: int, group_size: int) -> int:
     return -(-numel // group_size) if numel else 0
 
 
-def payload_nbytes(numel: int, group_size: int, dtype: str) -> int:
+def payload_nbytes(numel: int, group_size: int, dtype: str, bit: int = 8) -> int:
     """quant_pack_kernel.cu:247-249."""
-    return num_groups(numel, group_size) * (group_size + _ITEMSIZE[dtype])
+    return num_groups(numel, group_size) * (group_size * bit // 8 + _ITEMSIZE[dtype])
+
+
+def _levels(bit: int) -> np.float32:
+    if bit not in (4, 8):
+        raise ValueError(f"bit must be 4 or 8, got {bit}")
+    return np.float32(127.0 if bit == 8 else 7.0)
+
+
+def _pack_nibbles(codes: np.ndarray, word: int) -> np.ndarray:
+    """int8 codes in [-7, 7] -> bytes: ``2*word`` consecutive codes fill one ``word``-byte little-endian unit with
+    the first code in the most significant nibble (quant_pack_kernel.cu:123-129,149-157)."""
+    nibbles = (codes.astype(np.int16) & 0xF).astype(np.uint8).reshape(-1, 2 * word)
+    by_significance = (nibbles[:, 0::2] << 4) | nibbles[:, 1::2]        # most significant byte first
+    return np.ascontiguousarray(by_significance[:, ::-1]).reshape(-1)
+
+
+def _unpack_nibbles(code_bytes: np.ndarray, word: int) -> np.ndarray:
+    by_significance = code_bytes.reshape(-1, word)[:, ::-1]
+    nibbles = np.empty((by_significance.shape[0], 2 * word), dtype=np.uint8)
+    nibbles[:, 0::2] = by_significance >> 4
+    nibbles[:, 1::2] = by_significance & 0xF
+    signed = nibbles.astype(np.int8)
+    return np.where(signed >= 8, signed - 16, signed).astype(np.int8).reshape(-1)      # inner.cuh:36-40
 
 
 def _swap_words(codes: np.ndarray, word: int) -> np.ndarray:
@@ -82,7 +110,8 @@ def _swap_words(codes: np.ndarray, word: int) -> np.ndarray:
 
 
 def quantize(x: np.ndarray, dtype: str, group_size: int = 64, compact: bool = True,
-             residual: np.ndarray | None = None) -> np.ndarray:
+             residual: np.ndarray | None = None, bit: int = 8) -> np.ndarray:
+    levels = _levels(bit)
     xf = to_f32(x, dtype).reshape(-1)
     n = xf.size
     if residual is not None:
@@ -98,40 +127,45 @@ def quantize(x: np.ndarray, dtype: str, group_size: int = 64, compact: bool = Tr
         absmax = np.fmax.reduce(np.abs(rows), axis=1, initial=np.float32(0.0)).astype(np.float32)   # fmaxf skips NaN
         stored = from_f32(absmax, dtype)                                                           # :101
         scale = np.fmax(to_f32(stored, dtype), _FLOOR)                                             # :102
-        multiplier = (_F127 / scale).astype(np.float32)                                            # :103
+        multiplier = (levels / scale).astype(np.float32)                                           # :103
         product = (rows * multiplier[:, None]).astype(np.float32)
         rounded = np.rint(product)
     rounded = np.where(np.isnan(rounded), np.float32(0.0), rounded)                                # __float2int_rn(NaN) = 0
-    codes = np.clip(rounded, -127.0, 127.0).astype(np.int8).view(np.uint8)
-    swapped = _swap_words(codes.reshape(-1), _ITEMSIZE[dtype]).reshape(groups, group_size)
+    codes = np.clip(rounded, -levels, levels).astype(np.int8)
+    if bit == 8:
+        swapped = _swap_words(codes.view(np.uint8).reshape(-1), _ITEMSIZE[dtype]).reshape(groups, group_size)
+    else:
+        swapped = _pack_nibbles(codes.reshape(-1), _ITEMSIZE[dtype]).reshape(groups, group_size // 2)
     scale_bytes = _raw_bytes(stored).reshape(groups, _ITEMSIZE[dtype])
     if compact:
         return np.ascontiguousarray(np.concatenate([swapped, scale_bytes], axis=1)).reshape(-1)
     return np.concatenate([swapped.reshape(-1), scale_bytes.reshape(-1)])
 
 
-def split(payload: np.ndarray, numel: int, dtype: str, group_size: int = 64, compact: bool = True):
+def split(payload: np.ndarray, numel: int, dtype: str, group_size: int = 64, compact: bool = True, bit: int = 8):
     """Payload -> (int8 codes in element order [G*g], stored scales [G] in the payload dtype)."""
+    _levels(bit)
     item = _ITEMSIZE[dtype]
     groups = num_groups(numel, group_size)
+    per_group = group_size * bit // 8
     payload = np.ascontiguousarray(payload, dtype=np.uint8).reshape(-1)
-    assert payload.size == groups * (group_size + item), (payload.size, groups, group_size, item)
+    assert payload.size == groups * (per_group + item), (payload.size, groups, per_group, item)
     if compact:
-        table = payload.reshape(groups, group_size + item)
-        code_bytes = np.ascontiguousarray(table[:, :group_size]).reshape(-1)
-        scale_bytes = np.ascontiguousarray(table[:, group_size:]).reshape(-1)
+        table = payload.reshape(groups, per_group + item)
+        code_bytes = np.ascontiguousarray(table[:, :per_group]).reshape(-1)
+        scale_bytes = np.ascontiguousarray(table[:, per_group:]).reshape(-1)
     else:
-        code_bytes = payload[: groups * group_size]
-        scale_bytes = np.ascontiguousarray(payload[groups * group_size:])
-    codes = _swap_words(code_bytes, item).view(np.int8)
+        code_bytes = payload[: groups * per_group]
+        scale_bytes = np.ascontiguousarray(payload[groups * per_group:])
+    codes = _swap_words(code_bytes, item).view(np.int8) if bit == 8 else _unpack_nibbles(code_bytes, item)
     view = {"fp32": np.float32, "fp16": np.float16, "bf16": np.uint16}[dtype]
     return codes, scale_bytes.view(view)
 
 
-def _decode_f32(payload, numel, dtype, group_size, compact):
-    codes, stored = split(payload, numel, dtype, group_size, compact)
+def _decode_f32(payload, numel, dtype, group_size, compact, bit=8):
+    codes, stored = split(payload, numel, dtype, group_size, compact, bit)
     with np.errstate(invalid="ignore", over="ignore"):
-        step = (to_f32(stored, dtype) / _F127).astype(np.float32)          # scale / 127 (IEEE)
+        step = (to_f32(stored, dtype) / _levels(bit)).astype(np.float32)   # scale / 127 or scale / 7 (IEEE)
         values = codes.astype(np.float32).reshape(-1, group_size) * step[:, None]
     return values.astype(np.float32).reshape(-1)[:numel]
 
@@ -164,9 +198,9 @@ def _f64_to_bf16(values: np.ndarray) -> np.ndarray:
 
 
 def dequantize(payload: np.ndarray, numel: int, dtype: str, group_size: int = 64, compact: bool = True,
-               reduce_op: str = "none", out: np.ndarray | None = None) -> np.ndarray:
+               reduce_op: str = "none", out: np.ndarray | None = None, bit: int = 8) -> np.ndarray:
     """Decode one payload into ``dtype``; SUM/MAX/MIN combine with the existing ``out`` in that dtype."""
-    value = from_f32(_decode_f32(payload, numel, dtype, group_size, compact), dtype)
+    value = from_f32(_decode_f32(payload, numel, dtype, group_size, compact, bit), dtype)
     if reduce_op == "none":
         return value
     assert out is not None

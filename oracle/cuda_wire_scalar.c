@@ -83,19 +83,31 @@ static void store_from_f32(void *base, int64_t index, int dtype, float v) {
 }
 
 static int64_t group_count(int64_t numel, int g) { return numel ? (numel + g - 1) / g : 0; }
-static int64_t code_offset(int64_t group, int g, int item, int compact) {
-    return compact ? group * (g + item) : group * g;
+/* cb = code bytes per group (g for 8-bit codes, g/2 for 4-bit codes) */
+static int64_t code_offset(int64_t group, int cb, int item, int compact) {
+    return compact ? group * (cb + item) : group * cb;
 }
-static int64_t scale_offset(int64_t group, int64_t groups, int g, int item, int compact) {
-    return compact ? group * (g + item) + g : groups * g + group * item;
+static int64_t scale_offset(int64_t group, int64_t groups, int cb, int item, int compact) {
+    return compact ? group * (cb + item) + cb : groups * cb + group * item;
 }
 
 /* position of element k of a group inside the group's code bytes */
 static int byte_slot(int k, int item) { return (k / item) * item + (item - 1 - k % item); }
 
-void lbw_quantize(const void *x, const void *residual, int dtype, int64_t numel, int g, int compact,
+/* 4-bit codes: element k of a group lives in a word of `item` bytes holding 2*item elements, first element in
+ * the most significant nibble; the word is stored little-endian (quant_pack_kernel.cu:120-130,145-158). */
+static int nibble_byte(int k, int item) {
+    const int per_word = 2 * item;
+    const int in_word = k % per_word;
+    return (k / per_word) * item + (item - 1 - in_word / 2);
+}
+static int nibble_is_high(int k) { return (k % 2) == 0; }
+
+void lbw_quantize(const void *x, const void *residual, int dtype, int64_t numel, int g, int compact, int bit,
                   uint8_t *payload) {
     const int item = item_size(dtype);
+    const int cb = g * bit / 8;
+    const float levels = bit == 8 ? 127.0f : 7.0f;
     const int64_t groups = group_count(numel, g);
     float prepared[256];
     for (int64_t group = 0; group < groups; ++group) {
@@ -112,14 +124,16 @@ void lbw_quantize(const void *x, const void *residual, int dtype, int64_t numel,
         }
         const float stored = round_to(max_abs, dtype);
         const float scale = fmaxf(stored, 1.0e-6f);
-        const float multiplier = 127.0f / scale;
-        uint8_t *codes = payload + code_offset(group, g, item, compact);
+        const float multiplier = levels / scale;
+        uint8_t *codes = payload + code_offset(group, cb, item, compact);
+        if (bit == 4) memset(codes, 0, (size_t)cb);
         for (int k = 0; k < g; ++k) {
             float q = rintf(prepared[k] * multiplier);
-            int c = q != q ? 0 : (q > 127.0f ? 127 : (q < -127.0f ? -127 : (int)q));
-            codes[byte_slot(k, item)] = (uint8_t)(int8_t)c;
+            int c = q != q ? 0 : (q > levels ? (int)levels : (q < -levels ? -(int)levels : (int)q));
+            if (bit == 8) codes[byte_slot(k, item)] = (uint8_t)(int8_t)c;
+            else codes[nibble_byte(k, item)] |= (uint8_t)((c & 0xF) << (nibble_is_high(k) ? 4 : 0));
         }
-        uint8_t *where = payload + scale_offset(group, groups, g, item, compact);
+        uint8_t *where = payload + scale_offset(group, groups, cb, item, compact);
         if (dtype == LBW_F32) memcpy(where, &stored, 4);
         else {
             uint16_t h = dtype == LBW_F16 ? f32_to_f16(stored) : f32_to_bf16(stored);
@@ -128,9 +142,10 @@ void lbw_quantize(const void *x, const void *residual, int dtype, int64_t numel,
     }
 }
 
-static float payload_step(const uint8_t *payload, int64_t group, int64_t groups, int g, int dtype, int compact) {
+static float payload_step(const uint8_t *payload, int64_t group, int64_t groups, int g, int dtype, int compact,
+                          int bit) {
     const int item = item_size(dtype);
-    const uint8_t *where = payload + scale_offset(group, groups, g, item, compact);
+    const uint8_t *where = payload + scale_offset(group, groups, g * bit / 8, item, compact);
     float stored;
     if (dtype == LBW_F32) memcpy(&stored, where, 4);
     else {
@@ -138,14 +153,17 @@ static float payload_step(const uint8_t *payload, int64_t group, int64_t groups,
         memcpy(&h, where, 2);
         stored = dtype == LBW_F16 ? f16_to_f32(h) : bf16_to_f32(h);
     }
-    return stored / 127.0f;
+    return stored / (bit == 8 ? 127.0f : 7.0f);
 }
 
-static float payload_code(const uint8_t *payload, int64_t e, int g, int dtype, int compact) {
+static float payload_code(const uint8_t *payload, int64_t e, int g, int dtype, int compact, int bit) {
     const int item = item_size(dtype);
     const int64_t group = e / g;
     const int k = (int)(e - group * g);
-    return (float)(int8_t)payload[code_offset(group, g, item, compact) + byte_slot(k, item)];
+    const uint8_t *codes = payload + code_offset(group, g * bit / 8, item, compact);
+    if (bit == 8) return (float)(int8_t)codes[byte_slot(k, item)];
+    int nibble = (codes[nibble_byte(k, item)] >> (nibble_is_high(k) ? 4 : 0)) & 0xF;
+    return (float)(nibble >= 8 ? nibble - 16 : nibble);
 }
 
 /* correctly rounded a + b in a 16-bit dtype: the double sum is exact (or, for far-apart bf16 operands,
@@ -167,11 +185,12 @@ static float add_in_dtype(float a, float b, int dtype) {
 }
 
 /* op: 0 none, 1 sum, 2 max, 3 min; out is read for op != 0 */
-void lbw_dequantize(const uint8_t *payload, int64_t numel, int g, int compact, int dtype, int op, void *out) {
+void lbw_dequantize(const uint8_t *payload, int64_t numel, int g, int compact, int dtype, int op, int bit,
+                    void *out) {
     const int64_t groups = group_count(numel, g);
     for (int64_t e = 0; e < numel; ++e) {
-        const float step = payload_step(payload, e / g, groups, g, dtype, compact);
-        float v = round_to(payload_code(payload, e, g, dtype, compact) * step, dtype);
+        const float step = payload_step(payload, e / g, groups, g, dtype, compact, bit);
+        float v = round_to(payload_code(payload, e, g, dtype, compact, bit) * step, dtype);
         if (op != 0) {
             const float old = load_as_f32(out, e, dtype);
             if (op == 1) v = add_in_dtype(old, v, dtype);
@@ -189,8 +208,8 @@ void lbw_reduce(const uint8_t *const *payloads, int world, int64_t numel, int g,
     for (int64_t e = 0; e < numel; ++e) {
         float sum = 0.0f;
         for (int r = 0; r < world; ++r) {
-            const float step = payload_step(payloads[r], e / g, groups, g, dtype, compact);
-            const float code = payload_code(payloads[r], e, g, dtype, compact);
+            const float step = payload_step(payloads[r], e / g, groups, g, dtype, compact, 8);
+            const float code = payload_code(payloads[r], e, g, dtype, compact, 8);
             if (use_fma) sum = fmaf(code, step, sum);
             else {
                 const float term = code * step;

@@ -28,21 +28,21 @@ def _typed(values, dtype):
     return np.ascontiguousarray(values, dtype=_NUMPY[dtype]).reshape(-1)
 
 
-def quantize(x, dtype: str, group_size: int = 64, compact: bool = True, residual=None) -> np.ndarray:
+def quantize(x, dtype: str, group_size: int = 64, compact: bool = True, residual=None, bit: int = 8) -> np.ndarray:
     x = _typed(x, dtype)
     residual = None if residual is None else _typed(residual, dtype)
-    payload = np.zeros(payload_nbytes(x.size, group_size, dtype), dtype=np.uint8)
+    payload = np.zeros(payload_nbytes(x.size, group_size, dtype, bit), dtype=np.uint8)
     _lib().lbw_quantize(_ptr(x), _ptr(residual), ctypes.c_int(_DTYPE[dtype]), ctypes.c_int64(x.size),
-                        ctypes.c_int(group_size), ctypes.c_int(int(compact)), _ptr(payload))
+                        ctypes.c_int(group_size), ctypes.c_int(int(compact)), ctypes.c_int(bit), _ptr(payload))
     return payload
 
 
 def dequantize(payload, numel: int, dtype: str, group_size: int = 64, compact: bool = True,
-               reduce_op: str = "none", out=None) -> np.ndarray:
+               reduce_op: str = "none", out=None, bit: int = 8) -> np.ndarray:
     payload = np.ascontiguousarray(payload, dtype=np.uint8)
     result = np.zeros(numel, dtype=_NUMPY[dtype]) if out is None else _typed(out, dtype).copy()
     _lib().lbw_dequantize(_ptr(payload), ctypes.c_int64(numel), ctypes.c_int(group_size), ctypes.c_int(int(compact)),
-                          ctypes.c_int(_DTYPE[dtype]), ctypes.c_int(_OPS[reduce_op]), _ptr(result))
+                          ctypes.c_int(_DTYPE[dtype]), ctypes.c_int(_OPS[reduce_op]), ctypes.c_int(bit), _ptr(result))
     return result
 
 

@@ -315,3 +315,96 @@ def test_round_trip_error_statistics_match_the_reference_reports():
     x = make(rng, 4096, "fp16")
     back = wire.to_f32(wire.dequantize(wire.quantize(x, "fp16"), 4096, "fp16"), "fp16")
     assert 0.004 < rel_l2(back, wire.to_f32(x, "fp16")) < 0.009
+
+
+# --------------------------------------------------------------------------- #
+# 4-bit codes
+# --------------------------------------------------------------------------- #
+def reader_nibble(payload: np.ndarray, e: int, g: int, item: int, compact: bool, groups: int) -> int:
+    """The generic decode loop of the reference walks a word from its last element to its first, shifting right by
+    four each time (dequant_kernel_fp32.cuh:94-104, dequant_kernel.cuh:36-41): element j of a word of W elements is
+    ``(word >> 4*(W-1-j)) & 15``; the table int4_to_float (inner.cuh:36-40) is two's complement."""
+    per_group = g // 2
+    group, k = divmod(e, g)
+    per_word = 2 * item
+    base = (group * (per_group + item) if compact else group * per_group) + (k // per_word) * item
+    word = sum(int(payload[base + b]) << (8 * b) for b in range(item))
+    nibble = (word >> (4 * (per_word - 1 - k % per_word))) & 15
+    return [0, 1, 2, 3, 4, 5, 6, 7, -8, -7, -6, -5, -4, -3, -2, -1][nibble]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("compact", (True, False))
+@pytest.mark.parametrize("g", (16, 32, 64))
+def test_four_bit_writer_layout_is_what_the_reader_expects(dtype, compact, g):
+    rng = np.random.default_rng(41)
+    n = 5 * g
+    x = make(rng, n, dtype)
+    payload = wire.quantize(x, dtype, g, compact, bit=4)
+    item = 4 if dtype == "fp32" else 2
+    assert payload.size == wire.payload_nbytes(n, g, dtype, 4) == 5 * (g // 2 + item)
+    codes, stored = wire.split(payload, n, dtype, g, compact, bit=4)
+    assert np.abs(codes).max() == 7
+    for e in range(n):
+        assert reader_nibble(payload, e, g, item, compact, 5) == int(codes[e]), e
+    raw = np.ascontiguousarray(stored).view(np.uint8).reshape(5, item)
+    for group in range(5):
+        at = group * (g // 2 + item) + g // 2 if compact else 5 * (g // 2) + group * item
+        assert payload[at:at + item].tobytes() == raw[group].tobytes()
+
+
+def test_four_bit_literal_bytes():
+    x = np.array([7, -7, 1, 2, 3, 4, 5, 6, -1, -2, -3, -4, 0, 0, 6, -6], dtype=np.float32)
+    payload = wire.quantize(x, "fp32", 16, True, bit=4)
+    # words (first element in the top nibble): 0x79123456 and 0xFEDC006A, each stored little-endian
+    assert payload[:8].tolist() == [0x56, 0x34, 0x12, 0x79, 0x6A, 0x00, 0xDC, 0xFE]
+    assert payload[8:].tobytes() == np.float32(7.0).tobytes()
+    half = wire.quantize(x.astype(np.float16), "fp16", 16, True, bit=4)
+    # 16-bit words 0x7912, 0x3456, 0xFEDC, 0x006A
+    assert half[:8].tolist() == [0x12, 0x79, 0x56, 0x34, 0xDC, 0xFE, 0x6A, 0x00]
+    assert half[8:].tobytes() == np.float16(7.0).tobytes()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_four_bit_codes_match_exact_rational_arithmetic(dtype):
+    rng = np.random.default_rng(43)
+    g = 16
+    x = make(rng, 8 * g, dtype, 0.02)
+    codes, stored = wire.split(wire.quantize(x, dtype, g, True, bit=4), 8 * g, dtype, g, True, bit=4)
+    xf = wire.to_f32(x, dtype)
+    for group in range(8):
+        exact = [Fraction(float(v)) for v in xf[group * g:(group + 1) * g]]
+        absmax = max(abs(v) for v in exact)
+        multiplier = Fraction(float(_round_to_f32(Fraction(7) / max(absmax, Fraction(float(np.float32(1.0e-6)))))))
+        want = [max(-7, min(7, _rint_half_even(Fraction(float(_round_to_f32(v * multiplier)))))) for v in exact]
+        assert codes[group * g:(group + 1) * g].tolist() == want
+        step = _round_to_f32(absmax / 7)
+        decoded = wire.to_f32(wire.dequantize(wire.quantize(x, dtype, g, True, bit=4), 8 * g, dtype, g, True, bit=4), dtype)
+        for k in range(g):
+            product = _round_to_f32(Fraction(want[k]) * Fraction(float(step)))
+            assert decoded[group * g + k] == wire.to_f32(wire.from_f32(np.array([product], dtype=np.float32), dtype), dtype)[0]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("compact", (True, False))
+@pytest.mark.parametrize("g", (16, 32, 64))
+@pytest.mark.parametrize("n", (1, 63, 200, 4099))
+def test_four_bit_numpy_and_c_restatements_agree(dtype, compact, g, n):
+    rng = np.random.default_rng(n * 11 + g)
+    x = make(rng, n, dtype, 10.0 ** rng.uniform(-7, 3))
+    r = make(rng, n, dtype, 1e-2)
+    for residual in (None, r):
+        assert same_bits(wire.quantize(x, dtype, g, compact, residual, bit=4),
+                         wire_c.quantize(x, dtype, g, compact, residual, bit=4))
+    payload = wire.quantize(x, dtype, g, compact, bit=4)
+    base = make(rng, n, dtype)
+    for op in ("none", "sum", "max", "min"):
+        assert same_bits(wire.dequantize(payload, n, dtype, g, compact, op, base, bit=4),
+                         wire_c.dequantize(payload, n, dtype, g, compact, op, base, bit=4)), op
+    decoded = wire.to_f32(wire.dequantize(payload, n, dtype, g, compact, bit=4), dtype)
+    xf = wire.to_f32(x, dtype)
+    pad = -n % g
+    absmax = np.abs(np.concatenate([xf, np.zeros(pad, dtype=np.float32)])).reshape(-1, g).max(axis=1)
+    spread = np.repeat(absmax, g)[:n]
+    above_floor = spread >= 1.0e-6          # below it the encoder uses 7e6 as multiplier and decode no longer inverts it
+    assert np.all(np.abs(decoded - xf)[above_floor] <= (spread * (0.5 / 7 + 2.0 ** -7))[above_floor])

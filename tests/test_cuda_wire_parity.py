@@ -354,5 +354,73 @@ def test_module_error_feedback_paths(wire_status, hip_device):
         module.inplace_dequantize_reduce_mean_update_error_feedback(payloads, prepared, restored, residual, 64, 0, 8,
                                                                     linear, True, 0)
     with pytest.raises(RuntimeError):
-        module.quantize(prepared, 64, 0, False, 4, linear, True)          # 4-bit codes have no kernel
+        module.quantize(prepared, 64, 2, False, 8, linear, True)          # top-k side channels have no kernel
     assert module.inplace_quantize_pack(prepared, payloads[0], None, 64, 1, False, 8, linear, True) is False
+
+
+# --------------------------------------------------------------------------- #
+# 4-bit codes
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("name", list(NAMES))
+@pytest.mark.parametrize("compact", (True, False))
+@pytest.mark.parametrize("g", (16, 32, 64))
+@pytest.mark.parametrize("n", (1, 63, 131, 8192, 70_001))
+def test_four_bit_quantize_and_decode(hip, hip_device, access, name, compact, g, n):
+    x = make(n, name, 1100 + n + g, hip_device, sigma=10.0 ** ((n % 7) - 4))
+    r = make(n, name, 1200 + n + g, hip_device, sigma=1e-3)
+    payload = hip.quant_pack(x, group_size=g, compact=compact, bit=4)
+    assert payload.numel() == hip.payload_nbytes(n, x.dtype, g, 4)
+    same(payload, wire.quantize(to_numpy(x), name, g, compact, bit=4), "plain")
+    same(hip.quant_pack(x, group_size=g, compact=compact, residual=r, bit=4),
+         wire.quantize(to_numpy(x), name, g, compact, residual=to_numpy(r), bit=4), "with residual")
+    base = make(n, name, 1300 + n, hip_device, sigma=5.0)
+    for op in ("none", "sum", "max", "min"):
+        out = base.clone()
+        assert hip.dequant_into(payload, out, group_size=g, compact=compact, reduce_op=op, bit=4)
+        same(out, wire.dequantize(to_numpy(payload), n, name, g, compact, op, to_numpy(base), bit=4), op)
+
+
+def test_four_bit_full_bucket_and_chunks(hip, hip_device, access):
+    n, world = 26_214_400, 8
+    x = make(n, "bf16", 77, hip_device, sigma=1e-3)
+    payload = hip.quant_pack(x, bit=4)
+    same(payload, wire_c.quantize(to_numpy(x), "bf16", bit=4))
+    back = torch.empty_like(x)
+    assert hip.dequant_into(payload, back, bit=4)
+    same(back, wire_c.dequantize(to_numpy(payload), n, "bf16", bit=4))
+    shard = n // world
+    row = hip.payload_nbytes(shard, x.dtype, 64, 4)
+    rows = torch.empty(world, row, dtype=torch.uint8, device=hip_device)
+    assert hip.bind_quant_pack_chunks(x, rows, world, bit=4)()
+    xs = to_numpy(x)
+    for d in (0, 3, 7):
+        same(rows[d], wire_c.quantize(xs[d * shard:(d + 1) * shard], "bf16", bit=4), f"chunk {d}")
+    out = torch.empty_like(x)
+    assert hip.bind_dequant_chunks(rows, out, shard, bit=4)()
+    same(out, np.concatenate([wire_c.dequantize(to_numpy(rows[d]), shard, "bf16", bit=4) for d in range(world)]))
+
+
+def test_four_bit_through_the_module(wire_status, hip_device):
+    """4-bit codes are experimental upstream (allow_experimental); quantize and decode run natively, reduces chain."""
+    from lowbit_comm_amd.config import CompressionConfig
+    from lowbit_comm_amd.quantization.codec import allocate_quantized_buffer, dequantize_tensor, quantize_tensor
+
+    module = wire_status.module
+    linear = module.QuantType.Linear
+    config = CompressionConfig(bit=4, group_size=64, compact=True, allow_experimental=True)
+    tensor = make(64 * 30 + 5, "fp16", 8, hip_device)
+    buffer = allocate_quantized_buffer(tensor, config, dtype="fp16", wire_format="native")
+    assert buffer.numel() == 31 * (32 + 2)
+    quantize_tensor(tensor, config, extension_status=wire_status, output=buffer)
+    same(buffer, wire.quantize(to_numpy(tensor), "fp16", 64, True, bit=4))
+    restored = dequantize_tensor(buffer, tensor.shape, config, dtype="fp16", extension_status=wire_status)
+    same(restored, wire.dequantize(to_numpy(buffer), tensor.numel(), "fp16", bit=4))
+    grads = [make(64 * 20, "fp16", 40 + r, hip_device) for r in range(3)]
+    payloads = [module.quantize(g_, 64, 0, False, 4, linear, True) for g_ in grads]
+    out = torch.empty(64 * 20, dtype=torch.float16, device=hip_device)
+    assert module.inplace_dequantize_reduce_mean(payloads, out, 64, 0, 4, linear, True, 3) is False   # no fused 4-bit reduce
+    module.inplace_dequantize_reduce(payloads, out, 64, 0, 4, linear, True)
+    want = wire.dequantize(to_numpy(payloads[0]), 64 * 20, "fp16", bit=4)
+    for p in payloads[1:]:
+        want = wire.dequantize(to_numpy(p), 64 * 20, "fp16", reduce_op="sum", out=want, bit=4)
+    same(out, want)
