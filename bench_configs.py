@@ -438,6 +438,27 @@ def main() -> int:
                 emit(6, f"fused reduce + mean + error feedback W=8, {name}, {layout}", world * pbytes + 3 * n * item,
                      timed(lambda i: feedback[i % 2](), max(10, args.iters // 2)), world * pbytes, check)
                 del xs, outs, quant, payloads, res, prepared, plain, feedback
+            # 4-bit codes (experimental upstream): quantize+pack and decode of one payload, interleaved scales
+            p4 = cuda_wire.payload_nbytes(n, dtype, 64, 4)
+            xs = [gen(SEED + 1000 + s, n, 1e-3, dtype) for s in range(4)]
+            outs = [torch.empty(p4, dtype=torch.uint8, device=dev) for _ in range(4)]
+            back = [torch.empty(n, dtype=dtype, device=dev) for _ in range(4)]
+            quant = [cuda_wire.bind_quant_pack(xs[s], outs[s], bit=4) for s in range(4)]
+            decode = [cuda_wire.bind_dequant(outs[s], back[s], bit=4) for s in range(4)]
+            check = None
+            if parity:
+                quant[0](); decode[0]()
+                want = wire_c.quantize(host(xs[0]), name, 64, True, bit=4)
+                ok = host(outs[0]).tobytes() == want.tobytes()
+                ok = ok and host(back[0]).tobytes() == wire_c.dequantize(want, n, name, 64, True, bit=4).tobytes()
+                check = "bit-exact" if ok else "MISMATCH"
+            for s in range(4):
+                quant[s]()
+            emit(6, f"4-bit quantize+pack 26.2M {name}, interleaved scales", n * item + p4,
+                 timed(lambda i: quant[i % 4](), args.iters), n * item, check)
+            emit(6, f"4-bit decode 26.2M {name}, interleaved scales", n * item + p4,
+                 timed(lambda i: decode[i % 4](), args.iters), p4, check)
+            del xs, outs, back, quant, decode
 
     print(f"\n{'cfg':>3} {'us':>10} {'GB/s alg.':>10} {'% of 8TB/s':>10} {'input GB/s':>10}  parity / op", file=sys.stderr)
     for r in rows_out:

@@ -75,8 +75,9 @@ __device__ __forceinline__ void store_elems(T *p, const T (&src)[VEC]) {
 
 template <typename T, int BIT = 8> struct wire {
     static constexpr int ITEM = sizeof(T);
-    static constexpr int VEC = BIT == 8 ? 16 / ITEM : 8;   // elements per lane (a 4-bit lane fills one 32-bit word)
-    static constexpr int WORDS = VEC * BIT / 32;            // 32-bit code words per lane
+    static constexpr int VEC = 16 / ITEM;                  // elements per lane: 16 bytes of the tensor
+    static constexpr int CODE_BYTES = VEC * BIT / 8;        // 8, 4 or (4-bit codes of an fp32 tensor) 2
+    static constexpr int WORDS = CODE_BYTES >= 4 ? CODE_BYTES / 4 : 1;   // 32-bit registers holding them
     static constexpr int TILE = kWave * VEC;
     static constexpr float LEVELS = BIT == 8 ? 127.0f : 7.0f;
 };
@@ -117,16 +118,35 @@ __device__ __forceinline__ void pack_codes(const int (&c)[VEC], uint32_t (&words
             else words[k] = pack4(c[4 * k + 1], c[4 * k], c[4 * k + 3], c[4 * k + 2]);
         }
     } else {
-        static_assert(VEC == 8 && WORDS == 1, "a 4-bit lane owns one word");
+        // Four codes make one 16-bit unit with the first code on top.  A 16-bit tensor's lane holds two
+        // such units, low half first; an fp32 tensor's lane holds one (half of a 32-bit payload word).
+        static_assert(WORDS == 1 && (VEC == 8 || VEC == 4), "a 4-bit lane owns at most one register");
         uint32_t word = 0;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            // fp32 payloads: one 32-bit word, first code on top; 16-bit payloads: two 16-bit words, low half first
-            const int shift = sizeof(T) == 4 ? 28 - 4 * i : 16 * (i / 4) + 12 - 4 * (i % 4);
-            word |= (static_cast<uint32_t>(c[i]) & 0xFu) << shift;
-        }
+        for (int i = 0; i < VEC; ++i)
+            word |= (static_cast<uint32_t>(c[i]) & 0xFu) << (16 * (i / 4) + 12 - 4 * (i % 4));
         words[0] = word;
     }
+}
+
+// Byte offset, inside a group's code bytes, of the piece owned by the lane whose first element is k0.
+// An fp32 payload word holds eight 4-bit codes, elements 0-3 in its upper half: the two lanes sharing a
+// word write its halves swapped, which keeps a wavefront's 2-byte accesses one contiguous run.
+template <typename T, int BIT> __device__ __forceinline__ int piece_offset(int k0) {
+    if constexpr (BIT == 4 && sizeof(T) == 4) return (k0 / 8) * 4 + ((k0 & 4) ? 0 : 2);
+    else return k0 * BIT / 8;
+}
+
+template <typename T, int BIT, int PNT, int WORDS>
+__device__ __forceinline__ void store_piece(uint8_t *p, const uint32_t (&words)[WORDS]) {
+    if constexpr (wire<T, BIT>::CODE_BYTES == 2) *reinterpret_cast<uint16_t *>(p) = static_cast<uint16_t>(words[0]);
+    else store_words<WORDS, sizeof(T), PNT>(p, words);
+}
+
+template <typename T, int BIT, int PNT, int WORDS>
+__device__ __forceinline__ void load_piece(const uint8_t *p, uint32_t (&words)[WORDS]) {
+    if constexpr (wire<T, BIT>::CODE_BYTES == 2) words[0] = *reinterpret_cast<const uint16_t *>(p);
+    else load_words<WORDS, sizeof(T), PNT>(p, words);
 }
 
 // Code i of the lane's words as a float.
@@ -135,7 +155,7 @@ __device__ __forceinline__ float unpack_code(const uint32_t (&words)[WORDS], int
     if constexpr (BIT == 8) {
         return code_to_float(words[i / 4], byte_in_word<T>(i % 4));
     } else {
-        const int top = sizeof(T) == 4 ? 4 * i : 16 - 16 * (i / 4) + 4 * (i % 4);   // left shift that puts the nibble on top
+        const int top = 16 - 16 * (i / 4) + 4 * (i % 4);   // left shift that puts the nibble on top
         return static_cast<float>(static_cast<int32_t>(words[0] << top) >> 28);
     }
 }
@@ -256,7 +276,7 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
             pack_codes<T, BIT, VEC, W::WORDS>(c, words);
             const int64_t group = e0[u] / G;
             const int k0 = static_cast<int>(e0[u] - group * G);
-            store_words<W::WORDS, sizeof(T), PNT>(payload + at.codes(group) + k0 * BIT / 8, words);
+            store_piece<T, BIT, PNT, W::WORDS>(payload + at.codes(group) + piece_offset<T, BIT>(k0), words);
             if ((lane & (LPG - 1)) == 0) *reinterpret_cast<T *>(payload + at.scale(group)) = narrow<T>(absmax);
         }
         return;
@@ -291,7 +311,7 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
             for (int i = 0; i < VEC; ++i) c[i] = cvt_i32(__builtin_rintf(p[i] * multiplier));
             uint32_t words[W::WORDS];
             pack_codes<T, BIT, VEC, W::WORDS>(c, words);
-            store_words<W::WORDS, sizeof(T), kPlain>(payload + at.codes(group) + k0 * BIT / 8, words);
+            store_piece<T, BIT, kPlain, W::WORDS>(payload + at.codes(group) + piece_offset<T, BIT>(k0), words);
             if ((lane & (LPG - 1)) == 0) *reinterpret_cast<T *>(payload + at.scale(group)) = narrow<T>(absmax);
         }
     }
@@ -508,7 +528,7 @@ __global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArg
             e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
             const int64_t group = e0[u] / G;
             const int k0 = static_cast<int>(e0[u] - group * G);
-            load_words<W::WORDS, sizeof(T), PNT>(payload + at.codes(group) + k0 * BIT / 8, words[u]);
+            load_piece<T, BIT, PNT, W::WORDS>(payload + at.codes(group) + piece_offset<T, BIT>(k0), words[u]);
             stored[u] = *reinterpret_cast<const T *>(payload + at.scale(group));
         }
 #pragma unroll
