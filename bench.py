@@ -204,11 +204,33 @@ def main() -> int:
                 break
         times = sorted(times[2:] or times)
         median = times[len(times) // 2]
+        threads = torch.get_num_threads()
+        single = None
+        if threads > 1:                                   # the same step on one thread, a few repeats
+            torch.set_num_threads(1)
+            one = []
+            stop_at = time.perf_counter() + 8.0
+            for i in range(4):
+                t0 = time.perf_counter()
+                cpu_step()
+                one.append(time.perf_counter() - t0)
+                if time.perf_counter() > stop_at:
+                    break
+            torch.set_num_threads(threads)
+            single = sorted(one[1:] or one)[0]
+        model = "unknown"
+        try:
+            with open("/proc/cpuinfo") as info:
+                model = next((line.split(":", 1)[1].strip() for line in info if line.startswith("model name")), model)
+        except OSError:
+            pass
         cpu_baseline = {
-            "value": n * 4 / median / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "value": n * 4 / median / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"{len(times)} timed repeats of the full step (8x quantize of 3,276,800-element chunks + "
                       f"8-payload left-fold reduce of one shard) with torch CPU ops, median {median * 1e3:.1f} ms; "
                       f"host has {os.cpu_count()} logical CPUs",
+            "single_thread_value": None if single is None else n * 4 / single / 1e9,
+            "cpu_model": model,
         }
 
     dominant = kernels.get("quant_pack_chunks")

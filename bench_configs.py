@@ -240,9 +240,20 @@ def main() -> int:
         plan = plans[0]
         pb = plan.payload_bytes
         b_quant, b_reduce, b_requant, b_decode = n * 4 + world * pb, world * pb + shard * 4, shard * 4 + pb, world * pb + n * 4
+        # stage times use launches bound once to the plans' buffers (what the plan caches internally), so the
+        # short stages measure the kernels and not the Python bookkeeping of the plan methods
+        def stage_launches(p):
+            pairs = p._pairs(p.received)
+            row = p.payload(p.gathered, p.rank)
+            row_codes, row_scales = ops.split_payload(row, shard, G)
+            return (ops.bind_dequant_reduce(pairs, p.shard, numel=shard, group_size=G),
+                    ops.bind_quant_pack(p.shard, row_codes, row_scales, group_size=G),
+                    ops.bind_dequant_reduce_quant(pairs, row_codes, row_scales, shard, group_size=G))
+
+        bound = [stage_launches(p) for p in plans]
         t_quant = timed(lambda i: plans[i % world].quantize_chunks(peers[i % world]), 24)
-        t_reduce = timed(lambda i: plans[i % world].reduce_received(op="sum"), 24)
-        t_requant = timed(lambda i: plans[i % world].requantize_shard(), 24)
+        t_reduce = timed(lambda i: bound[i % world][0](), 48)
+        t_requant = timed(lambda i: bound[i % world][1](), 48)
         outs = [out, torch.empty_like(out)]
         t_decode = timed(lambda i: plans[i % world].decode_gathered(out=outs[i % 2]), 24)
 
@@ -252,11 +263,30 @@ def main() -> int:
             p.decode_gathered(out=outs[i % 2])
 
         t_plan = timed(whole, 24)
+        # variant for callers that only forward the requantized payload: (ii)+(iii) as one launch, the fp32
+        # shard is never written
+        fused_check = None
+        if parity:
+            reference_row = plans[0].payload(plans[0].gathered, 0).clone()
+            plans[0].gathered[0].zero_()
+            fused_row = plans[0].reduce_and_requantize(op="sum")
+            fused_check = "bit-exact vs (ii)+(iii)" if torch.equal(fused_row, reference_row) else "MISMATCH"
+        t_fused = timed(lambda i: bound[i % world][2](), 48)
+
+        def whole_fused(i):
+            p = plans[i % world]
+            p.quantize_chunks(peers[i % world]); p.reduce_and_requantize(op="sum")
+            p.decode_gathered(out=outs[i % 2])
+
+        t_plan_fused = timed(whole_fused, 24)
         emit(4, "(i) quant-pack 8 chunks of 200 MiB fp32", b_quant, t_quant, n * 4, check)
         emit(4, "(ii) fused dequant-reduce W=8 -> 25 MiB shard", b_reduce, t_reduce, world * pb, check)
         emit(4, "(iii) requantize shard", b_requant, t_requant, shard * 4, check)
         emit(4, "(iv) decode 8 shard payloads -> 200 MiB", b_decode, t_decode, world * pb, check)
         emit(4, "whole plan (4 launches)", b_quant + b_reduce + b_requant + b_decode, t_plan, n * 4, check)
+        emit(4, "(ii+iii) fused reduce + requantize, shard not written", world * pb + pb, t_fused, world * pb, fused_check)
+        emit(4, "whole plan, fused variant (3 launches)", b_quant + world * pb + pb + b_decode, t_plan_fused, n * 4,
+             fused_check)
         del peers, plans, outs, out
         torch.cuda.empty_cache()
 

@@ -152,6 +152,21 @@ int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int worl
                        int out_dtype, void *stream);
 
 /*
+ * Fused reduce + requantize for the reduce-scatter -> all-gather hand-over: the payload of
+ * quantize(reduce(payloads)) without writing the reduced shard.  The reduce is the one of
+ * lbc_dequant_reduce for an output of type mid_dtype (list order, every partial sum rounded to
+ * mid_dtype, true division by divisor), the quantize the one of lbc_quant_pack on that result,
+ * elements past numel counting as zeros.  Replaces the two steps
+ * `_dequantize_reduce_payloads` + `_quantize_chunk` of the topology transport when no caller needs
+ * the full-precision shard (ccdl_comm/communication/topology_transport.py:866-894 gathers and decodes
+ * only the requantized payloads).  out_codes holds ceil(numel/g)*g codes, out_scales ceil(numel/g)
+ * floats; neither may alias an input.  world > 8: LBC_UNSUPPORTED.
+ */
+int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *scales, int world,
+                             int64_t numel, int group_size, float divisor, int mid_dtype,
+                             int8_t *out_codes, float *out_scales, void *stream);
+
+/*
  * residual = prepared - restored, element-wise, subtraction in fp32, rounded to
  * residual_dtype.  Supported: restored_dtype equal to prepared_dtype or either of
  * them LBC_F32, and residual_dtype their torch promotion; else LBC_UNSUPPORTED.  Replaces native inplace_error_feedback_update (ccdl_comm/csrc/

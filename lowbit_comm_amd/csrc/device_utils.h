@@ -161,6 +161,18 @@ __device__ __forceinline__ float scale_from_absmax(float absmax) {
     return s < as_f32(kEpsBits) ? as_f32(kEpsBits) : s;
 }
 
+// Scale of the group that the VEC values of LPG adjacent lanes form; every lane gets it.
+template <int VEC, int LPG>
+__device__ __forceinline__ float group_scale(const float (&p)[VEC]) {
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        const uint32_t a = as_u32(p[i]) & 0x7FFFFFFFu;
+        m = a > m ? a : m;
+    }
+    return scale_from_absmax(as_f32(group_max_bits<LPG>(m)));
+}
+
 __device__ __forceinline__ int cvt_i32(float v) {  // NaN -> 0, saturating
     int c;
     asm("v_cvt_i32_f32 %0, %1" : "=v"(c) : "v"(v));

@@ -34,6 +34,15 @@ struct ReduceArgs {
     float divisor;
 };
 
+struct ReduceQuantArgs {
+    const int8_t *codes[kMaxPayloads];
+    const float *scales[kMaxPayloads];
+    int8_t *out_codes;     // padded: ceil(numel/g)*g codes
+    float *out_scales;
+    int64_t numel;
+    float divisor;
+};
+
 struct DecodeArgs {
     const uint8_t *codes_base;   // chunk d: codes at codes_base + d * payload_stride
     const uint8_t *scales_base;  // chunk d: scales at scales_base + d * payload_stride
@@ -89,6 +98,9 @@ hipError_t launch_quant_pack(int x_dtype, int r_dtype, int d_dtype, bool outputs
 int quant_pack_vec(int x_dtype, int r_dtype, int d_dtype, bool outputs);
 hipError_t launch_dequant_reduce(int out_dtype, int group_size, int world, int mode,
                                  const ReduceArgs &args, hipStream_t stream);
+// Reduce of `world` payloads in `mid_dtype` arithmetic, requantized without leaving the chip.
+hipError_t launch_dequant_reduce_quant(int mid_dtype, int group_size, int world, int mode,
+                                       const ReduceQuantArgs &args, hipStream_t stream);
 hipError_t launch_decode(int out_dtype, int group_size, int reduce_op, int mode,
                          const DecodeArgs &args, int world, hipStream_t stream);
 hipError_t launch_ef_update(int p_dtype, int t_dtype, int r_dtype, int mode, const EfArgs &args,

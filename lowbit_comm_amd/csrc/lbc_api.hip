@@ -271,6 +271,38 @@ int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, i
                   "lbc_dequant_reduce");
 }
 
+int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *scales, int world, int64_t numel,
+                             int group_size, float divisor, int mid_dtype, int8_t *out_codes, float *out_scales,
+                             void *stream) {
+    if (world <= 0) return fail(LBC_EINVAL, "inputs must not be empty");
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (!(divisor > 0.0f)) return fail(LBC_EINVAL, "divisor must be > 0");
+    if (!valid_dtype(mid_dtype)) return fail(LBC_EINVAL, "unsupported intermediate dtype %d", mid_dtype);
+    if (world > LBC_MAX_PAYLOADS || !valid_group(group_size)) return LBC_UNSUPPORTED;
+    if (numel == 0) return LBC_OK;
+    if (codes == nullptr || scales == nullptr || out_codes == nullptr || out_scales == nullptr)
+        return fail(LBC_EINVAL, "codes, scales, out_codes and out_scales must not be null");
+    if (!aligned_to(out_scales, 4)) return fail(LBC_EINVAL, "out_scales must be 4-byte aligned");
+    bool aligned = aligned_to(out_codes, 4);
+    lbc::ReduceQuantArgs a{};
+    for (int r = 0; r < world; ++r) {
+        if (codes[r] == nullptr || scales[r] == nullptr) return fail(LBC_EINVAL, "payload %d has a null pointer", r);
+        if (!aligned_to(scales[r], 4)) return fail(LBC_EINVAL, "scales of payload %d must be 4-byte aligned", r);
+        if (codes[r] == out_codes || scales[r] == out_scales)
+            return fail(LBC_EINVAL, "the output payload must not alias input payload %d", r);
+        aligned = aligned && aligned_to(codes[r], 4);
+        a.codes[r] = codes[r];
+        a.scales[r] = scales[r];
+    }
+    a.out_codes = out_codes;
+    a.out_scales = out_scales;
+    a.numel = numel;
+    a.divisor = divisor;
+    return finish(lbc::launch_dequant_reduce_quant(mid_dtype, group_size, world, pick_mode(aligned, numel * (world + 1)),
+                                                   a, static_cast<hipStream_t>(stream)),
+                  "lbc_dequant_reduce_quant");
+}
+
 int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored, int restored_dtype,
                   void *residual, int residual_dtype, int64_t numel, void *stream) {
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");

@@ -38,17 +38,6 @@ template <int VEC> struct quant_tiling {
     static constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock * UNROLL;
 };
 
-template <int VEC, int LPG>
-__device__ __forceinline__ float group_scale(const float (&p)[VEC]) {
-    uint32_t m = 0;
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-        const uint32_t a = as_u32(p[i]) & 0x7FFFFFFFu;
-        m = a > m ? a : m;
-    }
-    return scale_from_absmax(as_f32(group_max_bits<LPG>(m)));
-}
-
 // XT input, RT residual (void = none), DT type `restored` is rounded to.
 template <typename XT, typename RT, typename DT, int G, int VEC, int MODE>
 __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {

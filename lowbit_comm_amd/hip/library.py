@@ -33,6 +33,8 @@ SIGNATURES = {
     "lbc_dequant_chunks": (_c_int, [_c_ptr, _c_i64, _c_int, _c_i64, _c_i64, _c_int, _c_ptr, _c_int, _c_ptr]),
     "lbc_dequant_reduce": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_ptr, _c_int,
                                     _c_ptr, _c_ptr, _c_ptr]),
+    "lbc_dequant_reduce_quant": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_int, _c_ptr,
+                                          _c_ptr, _c_ptr]),
     "lbc_ef_update": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr]),
     "lbc_wire_payload_nbytes": (_c_i64, [_c_i64, _c_int, _c_int, _c_int]),
     "lbc_wire_quant_pack": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),

@@ -343,6 +343,50 @@ def bind_dequant_reduce(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], o
     return BoundLaunch(lib.lbc_dequant_reduce, args, device, lib, keep)
 
 
+def bind_dequant_reduce_quant(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out_codes: torch.Tensor,
+                              out_scales: torch.Tensor, numel: int, *, group_size: int = 64, divisor: float = 1.0,
+                              mid_dtype: torch.dtype = torch.float32) -> BoundLaunch | None:
+    """Bound form of :func:`dequant_reduce_quant_into`; ``None`` when there are more than 8 payloads."""
+    lib = load_library()
+    _require(len(payloads) > 0, "inputs must not be empty")
+    _require(divisor > 0, "divisor must be > 0")
+    _require(mid_dtype in DTYPE_CODES, f"intermediate dtype must be fp16, bf16 or fp32; got {mid_dtype}")
+    _device_tensor(out_codes, "out_codes")
+    device = out_codes.device
+    _device_tensor(out_scales, "out_scales", device)
+    n = int(numel)
+    groups = num_groups(n, group_size)
+    _require(out_codes.dtype in (torch.int8, torch.uint8), "out_codes must have int8 or uint8 dtype")
+    _require(out_scales.dtype == torch.float32, "out_scales must have float32 dtype")
+    _require(out_codes.numel() >= groups * group_size, "out_codes is smaller than the padded element count")
+    _require(out_scales.numel() >= groups, "out_scales is smaller than the group count")
+    if len(payloads) > MAX_PAYLOADS:
+        return None
+    world = len(payloads)
+    code_ptrs = (ctypes.c_void_p * world)()
+    scale_ptrs = (ctypes.c_void_p * world)()
+    for r, (codes, scales) in enumerate(payloads):
+        _device_tensor(codes, f"codes[{r}]", device)
+        _device_tensor(scales, f"scales[{r}]", device)
+        _require(codes.dtype in (torch.int8, torch.uint8), f"codes[{r}] must have int8 or uint8 dtype")
+        _require(scales.dtype == torch.float32, f"scales[{r}] must have float32 dtype")
+        _require(codes.numel() >= groups * group_size, f"codes[{r}] is smaller than the padded element count")
+        _require(scales.numel() >= groups, f"scales[{r}] is smaller than the group count")
+        code_ptrs[r] = codes.data_ptr()
+        scale_ptrs[r] = scales.data_ptr()
+    args = (code_ptrs, scale_ptrs, world, n, group_size, float(divisor), DTYPE_CODES[mid_dtype], _ptr(out_codes),
+            _ptr(out_scales))
+    return BoundLaunch(lib.lbc_dequant_reduce_quant, args, device, lib, (tuple(payloads), out_codes, out_scales))
+
+
+def dequant_reduce_quant_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out_codes: torch.Tensor,
+                              out_scales: torch.Tensor, numel: int, **kwargs) -> bool:
+    """``(out_codes, out_scales) = quantize((sum_r decode(payload_r)) / divisor)`` in one launch, the reduce carried
+    out in ``mid_dtype`` exactly as :func:`dequant_reduce_into` would for an output of that dtype."""
+    bound = bind_dequant_reduce_quant(payloads, out_codes, out_scales, numel, **kwargs)
+    return False if bound is None else bound()
+
+
 def ef_update_into(prepared: torch.Tensor, restored: torch.Tensor, residual: torch.Tensor) -> bool:
     """``residual = prepared - restored`` (fp32 subtraction, rounded to the residual's dtype)."""
     lib = load_library()

@@ -147,6 +147,33 @@ class ReduceScatterPlan:
             raise ValueError(f"no HIP quantize kernel for dtype {source.dtype}")
         return row
 
+    def reduce_and_requantize(self, received: torch.Tensor | None = None, *, op: str = "sum") -> torch.Tensor:
+        """The two steps above in one launch, for callers that only forward the requantized payload: row ``rank``
+        of ``self.gathered`` receives ``quantize(reduce(received))`` and the full-precision shard is never written.
+        Bit-identical to ``requantize_shard(reduce_received(...).shard)``.  Falls back to the two steps beyond 8
+        ranks."""
+        if op not in ("sum", "mean"):
+            raise ValueError(f"unsupported reduce-scatter mode: {op}")
+        rows = self.received if received is None else received
+        row = self.payload(self.gathered, self.rank)
+        shard = self.chunks.shard_numel
+        if not shard:
+            return row
+        if self.world_size > ops.MAX_PAYLOADS:
+            self.reduce_received(rows, op=op)
+            return self.requantize_shard()
+
+        def make() -> ops.BoundLaunch:
+            codes, scales = ops.split_payload(row, shard, self.config.group_size)
+            return ops.bind_dequant_reduce_quant(self._pairs(rows), codes, scales, shard,
+                                                 group_size=self.config.group_size,
+                                                 divisor=float(self.world_size) if op == "mean" else 1.0,
+                                                 mid_dtype=self.reduced_dtype)
+
+        if not self._remember(("rq", rows.data_ptr(), op), make)():
+            raise ValueError(f"no HIP reduce-requantize kernel for dtype {self.reduced_dtype}")
+        return row
+
     def decode_gathered(self, gathered: torch.Tensor | None = None, *, out: torch.Tensor | None = None) -> torch.Tensor:
         """Decode the ``W`` gathered shard payloads into one flat tensor of the bucket's size (one launch)."""
         rows = self.gathered if gathered is None else gathered
@@ -179,8 +206,11 @@ def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: Co
                                              rank: int, all_to_all: Callable[[torch.Tensor, torch.Tensor], None],
                                              all_gather: Callable[[torch.Tensor, torch.Tensor], None],
                                              op: str = "sum", plan: ReduceScatterPlan | None = None,
-                                             out: torch.Tensor | None = None) -> torch.Tensor:
+                                             out: torch.Tensor | None = None, keep_shard: bool = False) -> torch.Tensor:
     """Full plan: reduce-scatter leg, requantize, all-gather leg, decode every shard.
+
+    Reduce and requantize run as one launch unless ``keep_shard`` asks for the full-precision shard in
+    ``plan.shard`` as well.
 
     ``all_gather(gathered_rows, my_payload)`` must fill row ``r`` of ``gathered_rows`` with rank ``r``'s
     requantized shard payload (row ``rank`` is already in place).
@@ -188,9 +218,14 @@ def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: Co
     if plan is None:
         plan = ReduceScatterPlan(tensor.numel(), tensor.dtype, world_size=world_size, rank=rank, config=config,
                                  device=tensor.device, shape=tuple(tensor.shape))
-    compressed_reduce_scatter_shard(tensor, config=config, world_size=world_size, rank=rank, all_to_all=all_to_all,
-                                    op=op, plan=plan)
-    mine = plan.requantize_shard()
+    if keep_shard:
+        compressed_reduce_scatter_shard(tensor, config=config, world_size=world_size, rank=rank,
+                                        all_to_all=all_to_all, op=op, plan=plan)
+        mine = plan.requantize_shard()
+    else:
+        send = plan.quantize_chunks(tensor)
+        all_to_all(plan.received, send)
+        mine = plan.reduce_and_requantize(op=op)
     all_gather(plan.gathered, mine)
     return plan.decode_gathered(out=out)
 

@@ -383,6 +383,51 @@ def test_reduce_scatter_all_gather_plan_matches_the_oracle(dev, n, world):
     assert np.array_equal(out.cpu().numpy().view(np.uint32), want_full.view(np.uint32))
 
 
+def test_reduce_scatter_plan_fused_requantize_matches_the_two_steps(hip_device):
+    from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan, compressed_all_reduce_via_reduce_scatter
+
+    world, n = 8, 8 * 64 * 500 + 1234
+    config = CompressionConfig(error_feedback=False)
+    buckets = [torch.randn(n, device=hip_device) * 1e-3 for _ in range(world)]
+    plans = [ReduceScatterPlan(n, torch.float32, world_size=world, rank=r, config=config, device=hip_device)
+             for r in range(world)]
+
+    def all_to_all_for(rank):
+        def exchange(received, send):
+            for r in range(world):
+                received[r].copy_(plans[r].send[rank])
+        return exchange
+
+    for r in range(world):
+        plans[r].quantize_chunks(buckets[r])
+    for mode in ("sum", "mean"):
+        for r in (0, world - 1):
+            all_to_all_for(r)(plans[r].received, plans[r].send)
+            reduced = plans[r].reduce_received(op=mode)
+            two_step = plans[r].requantize_shard(reduced.shard).clone()
+            plans[r].gathered.zero_()
+            fused = plans[r].reduce_and_requantize(op=mode)
+            assert torch.equal(fused, two_step), (mode, r)
+
+    def all_gather_for(rank):
+        def gather(gathered, mine):
+            for r in range(world):
+                if r != rank:
+                    all_to_all_for(r)(plans[r].received, plans[r].send)
+                    gathered[r, :plans[r].payload_bytes].copy_(plans[r].reduce_and_requantize(op="mean"))
+        return gather
+
+    full_fused = compressed_all_reduce_via_reduce_scatter(buckets[0], config=config, world_size=world, rank=0,
+                                                          all_to_all=all_to_all_for(0), all_gather=all_gather_for(0),
+                                                          op="mean", plan=plans[0]).clone()
+    full_kept = compressed_all_reduce_via_reduce_scatter(buckets[0], config=config, world_size=world, rank=0,
+                                                         all_to_all=all_to_all_for(0), all_gather=all_gather_for(0),
+                                                         op="mean", plan=plans[0], keep_shard=True)
+    assert torch.equal(full_fused, full_kept)
+    exact = torch.stack(buckets).mean(dim=0)
+    assert float((full_fused - exact).norm() / exact.norm()) < 0.02
+
+
 def test_reduce_scatter_plan_beyond_eight_ranks_chains_exactly(dev):
     from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
 

@@ -561,3 +561,57 @@ def test_randomized_parity_sweep(ops, hip_device):
         assert ops.dequant_reduce_into(payloads, out, group_size=g, divisor=float(world) if mode == "mean" else 1.0), label
         want = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in payloads], n, g, o_name, mode)
         assert_same_bits(out, want, label + f" reduce W={world} {mode} {o_name}")
+
+
+# --------------------------------------------------------------------------- #
+# fused reduce + requantize
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("mid", ["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("world", (1, 2, 5, 8))
+@pytest.mark.parametrize("mode", ("sum", "mean"))
+def test_reduce_requantize_equals_the_two_steps_and_the_oracle(ops, hip_device, mid, world, mode):
+    for g, n in ((64, 64 * 300), (64, 100_003), (32, 4099), (16, 1), (64, 2_000_000)):
+        peers = [gradient_like(n, torch.float32, 9000 + 7 * world + r, hip_device, sigma=10.0 ** (r % 3 - 3))
+                 for r in range(world)]
+        payloads = [ops.quant_pack(p, group_size=g) for p in peers]
+        groups = ops.num_groups(n, g)
+        codes = torch.empty(groups * g, dtype=torch.int8, device=hip_device)
+        scales = torch.empty(groups, dtype=torch.float32, device=hip_device)
+        divisor = float(world) if mode == "mean" else 1.0
+        assert ops.dequant_reduce_quant_into(payloads, codes, scales, n, group_size=g, divisor=divisor,
+                                             mid_dtype=DTYPES[mid])
+        # against the oracle: reduce in `mid`, then quantize
+        reduced = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in payloads], n, g, mid, mode)
+        want_codes, want_scales = codec_torch.quantize(reduced, g)
+        assert torch.equal(codes.cpu(), want_codes), (mid, world, mode, g, n)
+        assert_same_bits(scales, want_scales, f"{mid} W={world} {mode} g={g} n={n}")
+        # against the two launches
+        shard = torch.empty(n, dtype=DTYPES[mid], device=hip_device)
+        assert ops.dequant_reduce_into(payloads, shard, group_size=g, divisor=divisor)
+        two_codes, two_scales = ops.quant_pack(shard, group_size=g)
+        assert torch.equal(codes, two_codes) and torch.equal(scales.view(torch.int32), two_scales.view(torch.int32))
+
+
+def test_reduce_requantize_contract(ops, hip_device):
+    x = gradient_like(640, torch.float32, 1, hip_device)
+    payload = ops.quant_pack(x)
+    codes = torch.empty(640, dtype=torch.int8, device=hip_device)
+    scales = torch.empty(10, dtype=torch.float32, device=hip_device)
+    assert ops.dequant_reduce_quant_into([payload] * 9, codes, scales, 640) is False
+    with pytest.raises(RuntimeError):
+        ops.dequant_reduce_quant_into([], codes, scales, 640)
+    with pytest.raises(RuntimeError):
+        ops.dequant_reduce_quant_into([payload], codes[:100], scales, 640)
+    with pytest.raises(RuntimeError):
+        ops.dequant_reduce_quant_into([payload], payload[0], scales, 640)          # output aliases an input
+    # a peer whose tail-group scale is not finite must not leak into the zero padding
+    n = 70
+    a, b = ops.quant_pack(gradient_like(n, torch.float32, 2, hip_device)), ops.quant_pack(gradient_like(n, torch.float32, 3, hip_device))
+    b[1][1] = float("inf")
+    c2 = torch.empty(128, dtype=torch.int8, device=hip_device)
+    s2 = torch.empty(2, dtype=torch.float32, device=hip_device)
+    assert ops.dequant_reduce_quant_into([a, b], c2, s2, n)
+    reduced = codec_torch.reduce_payloads([(a[0].cpu(), a[1].cpu()), (b[0].cpu(), b[1].cpu())], n, 64, "fp32", "sum")
+    want_codes, want_scales = codec_torch.quantize(reduced, 64)
+    assert torch.equal(c2.cpu(), want_codes) and torch.equal(c2[n:].cpu(), torch.zeros(128 - n, dtype=torch.int8))
+    assert_same_bits(s2, want_scales, "non-finite tail")
