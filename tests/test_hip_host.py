@@ -587,3 +587,21 @@ def test_bucket_step_replays_from_a_hip_graph(dev):
         assert same_bits(residual, cpu_residual), step
         received = [codec_torch.quantize(peers[src][:shard].cpu() * (1.0 + 0.01 * step)) for src in range(world)]
         assert same_bits(plan.shard, codec_torch.reduce_payloads(received, shard, 64, "fp32", "mean")), step
+
+
+@pytest.mark.parametrize("wire_format", ["portable", "native"])
+def test_hook_on_a_real_distributed_data_parallel_model(hip_device, wire_format):
+    """register_comm_hook on torch's own DDP (one rank, RCCL): real GradBucket objects and futures, gradients within
+    the quantization error of the uncompressed model.  Runs in a child process under a time limit so that trouble in
+    process-group set-up cannot stall the test run."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    worker = Path(__file__).resolve().parent / "workers" / "ddp_single_rank.py"
+    done = subprocess.run([sys.executable, str(worker), wire_format], capture_output=True, text=True, timeout=240)
+    assert done.returncode == 0, done.stderr[-2000:]
+    report = json.loads([line for line in done.stdout.splitlines() if line.startswith("{")][-1])
+    assert report["finite"] and report["buckets"] >= 3
+    assert all(0.0 < e < 0.02 for e in report["errors"]), report
