@@ -135,11 +135,13 @@ def main() -> int:
     leg("quant_pack_chunks", lambda i: sets[i % len(sets)]["quant"](), quant_bytes)
     leg("dequant_reduce_shard", lambda i: sets[i % len(sets)]["reduce"](), world * payload_bytes + shard * 4)
 
-    if "copy_calibration" in only:
-        # a plain device copy of known size (100 MiB read + 100 MiB written) to scale the HBM counters by
+    if not only or "copy_calibration" in only:
+        # a plain device copy of known size (100 MiB read + 100 MiB written): scales the HBM counters, and shows
+        # what this box sustains on the simplest possible streaming kernel next to the codec kernels
         srcs = [sets[i]["bucket"] for i in range(len(sets))]
         dsts = [torch.empty_like(srcs[0]) for _ in range(2)]
         leg("copy_calibration", lambda i: dsts[i % 2].copy_(srcs[i % len(srcs)]), 2 * n * 4)
+        del dsts
 
     if not only or "dequant_reduce_full" in only or "ef_quant_pack" in only:
         # all-gather-reduce shape: 8 payloads of the whole bucket -> fp32 bucket
