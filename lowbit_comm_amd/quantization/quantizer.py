@@ -52,6 +52,18 @@ class Quantizer:
         return estimate_quantized_size(numel, dtype="fp32" if name == "auto" else name, config=self.config,
                                        wire_format=wire_format).quantized_bytes
 
+    def dequantize_reduce(self, buffers: list, shape: tuple[int, ...], output: Any | None = None, *,
+                          reduce: str = "sum", dtype: str | None = None) -> Any:
+        """Decode every buffer and reduce them in list order (``sum`` or ``mean``); fused on the GPU when an
+        ``output`` workspace is given and there are at most eight buffers."""
+        return _codec.dequantize_reduce_tensors(buffers, shape, self.config, dtype=self._dtype(dtype),
+                                                extension_status=self.extension_status, output=output, reduce=reduce)
+
+    def update_residual(self, prepared: Any, restored: Any, residual: Any) -> Any:
+        """``residual <- prepared - restored`` on the device; returns ``residual``."""
+        return _codec.update_error_feedback_residual(prepared, restored, residual,
+                                                     extension_status=self.extension_status)
+
     def is_quantized(self) -> bool:
         return self.config.bit < 16
 
