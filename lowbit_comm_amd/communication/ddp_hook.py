@@ -425,3 +425,4 @@ def create_ddp_comm_hook(
 def make_fused_all_gather(byte_all_gather: Callable[[Any], GatheredPayloads]):
     """Convenience re-export: wrap a byte all-gather so payloads travel packed (one collective per bucket)."""
     return make_fused_payload_all_gather(byte_all_gather)
+
