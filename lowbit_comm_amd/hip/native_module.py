@@ -111,22 +111,22 @@ class HipNativeModule:
         """Fused ``(input + residual) -> quantize -> pack`` into ``output``; ``False`` for unsupported policy."""
         if not _policy_supported(group_size, topk, stochastic, bit, quant_type):
             return False
-        _check_payload(output, "output")
         if not isinstance(input, torch.Tensor) or not input.is_cuda:
             raise RuntimeError("input must be a GPU tensor")
-        if output.device != input.device:
+        if not input.is_contiguous():
+            raise RuntimeError("input must be contiguous")
+        if isinstance(output, torch.Tensor) and output.device != input.device:
             raise RuntimeError("input and output must be on the same device")
-        if output.numel() != ops.payload_nbytes(input.numel(), group_size):
-            raise RuntimeError("output has an invalid quantized payload size")
-        if input.numel() == 0:
-            return True
         if residual is not None and residual.numel() != input.numel():
             raise RuntimeError("input and residual must have the same number of elements")
-        flat = input.reshape(-1)
-        if not flat.is_contiguous():
-            raise RuntimeError("input must be contiguous")
-        flat_residual = None if residual is None else residual.reshape(-1)
-        return ops.quant_pack_payload_into(flat, output.reshape(-1), group_size=group_size, residual=flat_residual)
+        if input.numel() == 0:
+            _check_payload(output, "output")
+            if output.numel() != 0:
+                raise RuntimeError("output has an invalid quantized payload size")
+            return True
+        # payload dtype / contiguity / size are checked where the addresses are taken
+        return ops.quant_pack_payload_into(input.reshape(-1), output, group_size=group_size,
+                                           residual=None if residual is None else residual.reshape(-1))
 
     # ---- dequantize -----------------------------------------------------------------------------
     def dequantize(self, input, group_size, topk, bit, reduce_op, quant_type, dtype, compact):
@@ -142,40 +142,57 @@ class HipNativeModule:
     def inplace_dequantize(self, input, output, group_size, topk, bit, reduce_op, quant_type, compact) -> None:
         _require_policy(group_size, topk, False, bit, quant_type)
         _check_payload(input, "input")
-        codes, scales = _views(input, group_size)
+        padded = _padded_numel_of(input, group_size)
         flat = output.reshape(-1)
-        numel = min(flat.numel(), codes.numel())
-        if not ops.dequant_into(codes, scales, flat, numel=numel, group_size=group_size,
-                                reduce_op=_OP_NAME[ReduceOP(int(reduce_op))]):
+        if flat.numel() >= padded:        # the payload's own size decides; the usual workspace is padded
+            done = ops.dequant_payload_into(input, flat, numel=padded, group_size=group_size,
+                                            reduce_op=_OP_NAME[ReduceOP(int(reduce_op))])
+        else:                             # a trimmed output: codes and scales sit at offsets the payload size fixes
+            codes, scales = _views(input, group_size)
+            done = ops.dequant_into(codes, scales, flat, numel=flat.numel(), group_size=group_size,
+                                    reduce_op=_OP_NAME[ReduceOP(int(reduce_op))])
+        if not done:
             raise RuntimeError(f"no HIP dequantize kernel for output dtype {output.dtype}")
 
     # ---- dequantize + reduce ------------------------------------------------------------------
-    def _pairs(self, inputs: Sequence[torch.Tensor], group_size: int):
+    def _entries(self, inputs: Sequence[torch.Tensor], numel: int, group_size: int):
+        """The payloads as the ops layer takes them: the packed tensors themselves when they cover exactly ``numel``
+        elements' worth of groups (addresses are then computed without tensor views), (codes, scales) views when the
+        caller decodes fewer groups than the payloads hold."""
         if len(inputs) == 0:
             raise RuntimeError("inputs must not be empty")
         for i, buffer in enumerate(inputs):
             _check_payload(buffer, f"inputs[{i}]" if i else "input")
+        if all(buffer.numel() == ops.payload_nbytes(numel, group_size) for buffer in inputs):
+            return [buffer.reshape(-1) for buffer in inputs]
         return [_views(buffer, group_size) for buffer in inputs]
 
     def dequantize_reduce(self, inputs, group_size, topk, bit, quant_type, dtype, compact):
         _require_policy(group_size, topk, False, bit, quant_type)
-        pairs = self._pairs(inputs, group_size)
-        output = torch.empty(pairs[0][0].numel(), dtype=_TORCH_OF[DType(int(dtype))], device=inputs[0].device)
+        if len(inputs) == 0:
+            raise RuntimeError("inputs must not be empty")
+        _check_payload(inputs[0], "input")
+        output = torch.empty(_padded_numel_of(inputs[0], group_size), dtype=_TORCH_OF[DType(int(dtype))],
+                             device=inputs[0].device)
         self.inplace_dequantize_reduce(inputs, output, group_size, topk, bit, quant_type, compact)
         return output
 
     def inplace_dequantize_reduce(self, inputs, output, group_size, topk, bit, quant_type, compact) -> None:
         """Sum of all payloads into ``output`` in list order; any number of payloads (8 per fused launch)."""
         _require_policy(group_size, topk, False, bit, quant_type)
-        pairs = self._pairs(inputs, group_size)
+        if len(inputs) == 0:
+            raise RuntimeError("inputs must not be empty")
+        _check_payload(inputs[0], "input")
         flat = output.reshape(-1)
-        numel = min(flat.numel(), pairs[0][0].numel())
-        if len(pairs) <= ops.MAX_PAYLOADS:
-            if not ops.dequant_reduce_into(pairs, flat, numel=numel, group_size=group_size):
+        numel = min(flat.numel(), _padded_numel_of(inputs[0], group_size))
+        entries = self._entries(inputs, numel, group_size)
+        if len(entries) <= ops.MAX_PAYLOADS:
+            if not ops.dequant_reduce_into(entries, flat, numel=numel, group_size=group_size):
                 raise RuntimeError(f"no HIP dequantize-reduce kernel for output dtype {output.dtype}")
             return
         # More than 8 payloads: keep the left fold exact by chaining decode-and-add one payload at a time.
-        for r, (codes, scales) in enumerate(pairs):
+        for r, buffer in enumerate(inputs):
+            codes, scales = _views(buffer, group_size)
             if not ops.dequant_into(codes, scales, flat, numel=numel, group_size=group_size,
                                     reduce_op="none" if r == 0 else "sum"):
                 raise RuntimeError(f"no HIP dequantize kernel for output dtype {output.dtype}")
@@ -203,8 +220,7 @@ class HipNativeModule:
             raise RuntimeError("divisor must be > 0")
         if not self._fused_eligible(inputs, output, group_size, topk, bit, quant_type):
             return False
-        pairs = [_views(buffer, group_size) for buffer in inputs]
-        return ops.dequant_reduce_into(pairs, output.reshape(-1), group_size=group_size, divisor=float(divisor))
+        return ops.dequant_reduce_into(list(inputs), output.reshape(-1), group_size=group_size, divisor=float(divisor))
 
     # ---- error feedback -------------------------------------------------------------------------
     def inplace_error_feedback_update(self, prepared, restored, residual) -> None:
@@ -262,7 +278,6 @@ class HipNativeModule:
             if (not isinstance(buffer, torch.Tensor) or buffer.dtype != torch.uint8 or not buffer.is_cuda
                     or not buffer.is_contiguous() or buffer.device != prepared.device or buffer.numel() != expected):
                 return False
-        pairs = [_views(buffer, group_size) for buffer in inputs]
-        return ops.dequant_reduce_into(pairs, restored.reshape(-1), numel=numel, group_size=group_size,
+        return ops.dequant_reduce_into(list(inputs), restored.reshape(-1), numel=numel, group_size=group_size,
                                        divisor=float(divisor), prepared=prepared.reshape(-1),
                                        new_residual=residual.reshape(-1))

@@ -44,6 +44,26 @@ def split_payload(payload: torch.Tensor, numel: int, group_size: int = 64):
     return payload[:code_bytes].view(torch.int8), payload[code_bytes:].view(torch.float32)
 
 
+def payload_addresses(payload: torch.Tensor, numel: int, group_size: int = 64, *, name: str = "payload",
+                      device: torch.device | None = None) -> tuple[int, int]:
+    """Device addresses ``(codes, scales)`` inside a packed uint8 payload, without creating tensor views (a view
+    costs a few microseconds of host time; the hot callers hand over up to nine payloads per bucket)."""
+    groups = num_groups(numel, group_size)
+    code_bytes = groups * group_size
+    if not isinstance(payload, torch.Tensor) or payload.dtype != torch.uint8:
+        raise RuntimeError(f"{name} must be uint8")
+    if not payload.is_cuda:
+        raise RuntimeError(f"{name} must be a GPU tensor")
+    if not payload.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if device is not None and payload.device != device:
+        raise RuntimeError(f"{name} must be on {device}")
+    if payload.numel() != code_bytes + 4 * groups:
+        raise RuntimeError(f"{name} has an invalid quantized payload size")
+    base = payload.data_ptr()
+    return base, base + code_bytes
+
+
 def promote(a: torch.dtype, b: torch.dtype) -> torch.dtype:
     return a if a == b else torch.float32
 
@@ -192,10 +212,23 @@ def bind_quant_pack(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, 
     return BoundLaunch(lib.lbc_quant_pack, args, device, lib, (x, codes, scales, residual, new_residual, restored))
 
 
+def bind_quant_pack_payload(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64,
+                            residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
+                            restored: torch.Tensor | None = None,
+                            restored_dtype: torch.dtype | None = None) -> BoundLaunch:
+    """:func:`bind_quant_pack` writing the packed ``uint8[codes || scales]`` wire layout into ``payload``."""
+    lib = load_library()
+    x_code = _float_tensor(x, "input")
+    codes_at, scales_at = payload_addresses(payload, x.numel(), group_size, name="output", device=x.device)
+    r_code, n_code, d_code = _side_tensors(x, residual, new_residual, restored, restored_dtype)
+    args = (_ptr(x), x_code, _ptr(residual), r_code, x.numel(), group_size, ctypes.c_void_p(codes_at),
+            ctypes.c_void_p(scales_at), _ptr(new_residual), n_code, _ptr(restored), d_code)
+    return BoundLaunch(lib.lbc_quant_pack, args, x.device, lib, (x, payload, residual, new_residual, restored))
+
+
 def quant_pack_payload_into(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64, **kwargs) -> bool:
     """Same as :func:`quant_pack_into`, writing the packed ``uint8[codes || scales]`` wire layout."""
-    codes, scales = split_payload(payload, x.numel(), group_size)
-    return quant_pack_into(x, codes, scales, group_size=group_size, **kwargs)
+    return bind_quant_pack_payload(x, payload, group_size=group_size, **kwargs)()
 
 
 def quant_pack(x: torch.Tensor, *, group_size: int = 64, residual: torch.Tensor | None = None):
@@ -265,6 +298,20 @@ def bind_dequant(codes: torch.Tensor, scales: torch.Tensor, out: torch.Tensor, *
     return BoundLaunch(lib.lbc_dequant, args, device, lib, (codes, scales, out))
 
 
+def dequant_payload_into(payload: torch.Tensor, out: torch.Tensor, *, numel: int | None = None, group_size: int = 64,
+                         reduce_op: str = "none") -> bool:
+    """:func:`dequant_into` reading a packed ``uint8[codes || scales]`` payload that covers ``numel`` elements."""
+    lib = load_library()
+    o_code = _float_tensor(out, "output")
+    n = out.numel() if numel is None else int(numel)
+    _require(0 <= n <= out.numel(), "numel exceeds the output size")
+    _require(reduce_op in REDUCE_OPS, f"unsupported reduce op {reduce_op!r}")
+    codes_at, scales_at = payload_addresses(payload, n, group_size, name="input", device=out.device)
+    args = (ctypes.c_void_p(codes_at), ctypes.c_void_p(scales_at), n, group_size, _ptr(out), o_code,
+            REDUCE_OPS[reduce_op])
+    return BoundLaunch(lib.lbc_dequant, args, out.device, lib, (payload, out))()
+
+
 def dequant(codes: torch.Tensor, scales: torch.Tensor, numel: int, *, group_size: int = 64,
             dtype: torch.dtype = torch.float32) -> torch.Tensor:
     out = torch.empty(numel, dtype=dtype, device=codes.device)
@@ -295,7 +342,8 @@ def dequant_reduce_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], o
                         prepared: torch.Tensor | None = None, new_residual: torch.Tensor | None = None) -> bool:
     """``out[:numel] = (sum_r decode(payload_r)) / divisor`` in list order; optional ``new_residual = prepared - out``.
 
-    ``payloads`` is a sequence of ``(codes, scales)`` pairs.  More than 8 payloads returns ``False``.
+    ``payloads`` is a sequence of ``(codes, scales)`` pairs or of packed ``uint8[codes || scales]`` tensors covering
+    exactly ``numel`` elements.  More than 8 payloads returns ``False``.
     """
     bound = bind_dequant_reduce(payloads, out, numel=numel, group_size=group_size, divisor=divisor,
                                 prepared=prepared, new_residual=new_residual)
@@ -320,7 +368,11 @@ def bind_dequant_reduce(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], o
     world = len(payloads)
     code_ptrs = (ctypes.c_void_p * world)()
     scale_ptrs = (ctypes.c_void_p * world)()
-    for r, (codes, scales) in enumerate(payloads):
+    for r, entry in enumerate(payloads):
+        if isinstance(entry, torch.Tensor):          # a packed uint8[codes || scales] payload
+            code_ptrs[r], scale_ptrs[r] = payload_addresses(entry, n, group_size, name=f"inputs[{r}]", device=device)
+            continue
+        codes, scales = entry
         _device_tensor(codes, f"codes[{r}]", device)
         _device_tensor(scales, f"scales[{r}]", device)
         _require(codes.dtype in (torch.int8, torch.uint8), f"codes[{r}] must have int8 or uint8 dtype")
