@@ -185,7 +185,7 @@ def _f64_to_bf16(values: np.ndarray) -> np.ndarray:
     """float64 -> bf16 with a single rounding: round to odd into float32, then nearest-even to bf16."""
     with np.errstate(over="ignore", invalid="ignore"):
         near = values.astype(np.float32)
-    err = values - near.astype(np.float64)
+        err = values - near.astype(np.float64)
     bits = near.view(np.uint32).copy()
     inexact = (err != 0) & np.isfinite(near)
     even = (bits & np.uint32(1)) == 0
