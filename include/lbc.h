@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define LBC_ABI_VERSION 3
+#define LBC_ABI_VERSION 4
 
 enum { LBC_OK = 0, LBC_UNSUPPORTED = 1, LBC_EINVAL = -1, LBC_ELAUNCH = -2 };
 
@@ -42,6 +42,8 @@ enum { LBC_F32 = 0, LBC_F16 = 1, LBC_BF16 = 2, LBC_NONE = -1 };
 
 /* ccdl_comm/csrc/pybind.cpp:148-165 (ReduceOP) */
 enum { LBC_REDUCE_NONE = 0, LBC_REDUCE_SUM = 1, LBC_REDUCE_MAX = 2, LBC_REDUCE_MIN = 3 };
+/* QuantType of the reference (ccdl_comm/csrc/quantization/enum.cuh; code books: inner.cuh:9-35). */
+enum { LBC_QUANT_LINEAR = 0, LBC_QUANT_NORMAL = 1, LBC_QUANT_UNIFORM = 2, LBC_QUANT_E3M0 = 3, LBC_QUANT_E2M1 = 4 };
 
 #define LBC_MAX_PAYLOADS 8 /* ccdl_comm/csrc/quantization/dequant_reduce_kernel.cu:73-80,251 */
 
@@ -239,6 +241,31 @@ int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int
 int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t numel, int group_size,
                             int compact, float inv_divisor, int fused_multiply_add, void *out, int dtype,
                             const void *prepared, void *new_residual, void *stream);
+
+/*
+ * The remaining policies of the CUDA extension's format: non-linear 4-bit code books
+ * (quant_type != LINEAR needs bit == 4), stochastic rounding and the top-k side channel
+ * (topk 0, 1, 2), in any combination.  numel must be a multiple of group_size, as in the reference
+ * (gen_code_quant.py:164).  A group's bytes are [codes][scale][indices][top1][top2] in words of the
+ * tensor's item size, the metadata behind each group (compact) or behind all codes; the group
+ * maximum is the reference's running `(m > a) ? m : a`, which a NaN resets.
+ */
+int64_t lbc_wire_general_payload_nbytes(int64_t numel, int group_size, int dtype, int bit, int topk);
+
+/*
+ * Replaces native quantize / inplace_quantize (gen_code_quant.py:162-277 dispatching to
+ * quant_kernel_fp32.cuh:211-455 and quant_kernel.cuh:155-399).  With stochastic != 0, seed and offset are
+ * the Philox key and offset the reference takes from torch's CUDA generator
+ * (gen_code_quant.py:27-36: philox_engine_inputs(numel)); group s draws from subsequence s.
+ */
+int lbc_wire_quant_general(const void *x, int dtype, int64_t numel, int group_size, int bit, int quant_type,
+                           int topk, int stochastic, uint64_t seed, uint64_t offset, int compact,
+                           uint8_t *payload, void *stream);
+
+/* Replaces native dequantize / inplace_dequantize for those policies (dequant_kernel_fp32.cuh:122-353,
+ * dequant_kernel.cuh:62-291); reduce_op as in lbc_wire_dequant. */
+int lbc_wire_dequant_general(const uint8_t *payload, int64_t numel, int group_size, int bit, int quant_type,
+                             int topk, int compact, void *out, int dtype, int reduce_op, void *stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,428 @@
+// The policies of the reference's CUDA extension beyond plain linear codes, in its payload format:
+// non-linear 4-bit code books, stochastic rounding, the top-k side channel and the group maximum that
+// a NaN resets (ccdl_comm/csrc/quantization/quant_kernel_fp32.cuh, quant_kernel.cuh, inner.cuh,
+// dequant_kernel_fp32.cuh, dequant_kernel.cuh).  ccdl_cuda_ops.quantize / dequantize run these
+// kernels for every policy; inputs are whole groups (gen_code_quant.py:164).
+//
+// Payload of a group, in words of the tensor's item size (quant_kernel_fp32.cuh:283-331,390-417):
+//   [code words][scale]                                   top-k 0
+//   [code words][scale][index][top1]                      top-k 1
+//   [code words][scale][index1 | index2 << 8][top1][top2] top-k 2
+// with the metadata behind each group's codes (compact) or behind all codes.  The top-k elements are
+// stored as they are, encoded as zero, and the scale is the next largest magnitude.
+//
+// The reference walks a group with one thread, element by element: fp32 groups from element 0,
+// fp16/bf16 groups from element 4 * ((group & 31) / (32 / (G / 4))) with wrap-around.  That order
+// decides (a) which elements a NaN hides from the running maximum `(m > a) ? m : a`, (b) ties of the
+// top-k search (fp32 compares with >=: the later element wins and zeros qualify; 16-bit compares
+// with >: the earlier element of the scan wins and zeros do not), (c) which draw of the group's
+// Philox stream an element receives.  Here a group lies across G/VEC lanes of a DPP row as in the
+// other kernels, and each of the three is restated in an order-free form: (a) the maximum over the
+// scan positions behind the last NaN, (b) the three largest keys (magnitude bits, tie-break rank),
+// merged across the row, (c) Philox in counter mode - draw j of group s is word (offset + j) % 4
+// of block (offset + j) / 4 of subsequence s, so a lane computes the blocks of its own elements.
+#include "device_utils.h"
+#include "launch.h"
+#include "wire_common.h"
+
+namespace lbc {
+namespace {
+
+// inner.cuh:9-35 (entry 15 is never produced by the encoder)
+__constant__ float kCodeBooks[4][16] = {
+    {-1.0f, -0.815410147f, -0.655160150f, -0.510228027f, -0.375324982f, -0.246951370f, -0.122538030f, 0.0f,
+     0.122538030f, 0.246951370f, 0.375324982f, 0.510228027f, 0.655160150f, 0.815410147f, 1.0f, __builtin_inff()},
+    {-1.0f, -0.85714286f, -0.71428571f, -0.57142857f, -0.42857143f, -0.28571429f, -0.14285714f, 0.0f,
+     0.14285714f, 0.28571429f, 0.42857143f, 0.57142857f, 0.71428571f, 0.85714286f, 1.0f, __builtin_inff()},
+    {-1.0f, -0.5f, -0.25f, -0.125f, -0.0625f, -0.03125f, -0.015625f, 0.0f,
+     0.015625f, 0.03125f, 0.0625f, 0.125f, 0.25f, 0.5f, 1.0f, __builtin_inff()},
+    {-1.0f, -0.6666666666666666f, -0.5f, -0.3333333333333333f, -0.25f, -0.16666666666666666f, -0.125f, 0.0f,
+     0.125f, 0.16666666666666666f, 0.25f, 0.3333333333333333f, 0.5f, 0.6666666666666666f, 1.0f, __builtin_inff()},
+};
+
+template <typename T> struct raw_bits;
+template <> struct raw_bits<float> { using type = uint32_t; static constexpr uint32_t ABS = 0x7FFFFFFFu, INF = 0x7F800000u; };
+template <> struct raw_bits<f16> { using type = uint16_t; static constexpr uint32_t ABS = 0x7FFFu, INF = 0x7C00u; };
+template <> struct raw_bits<bf16> { using type = uint16_t; static constexpr uint32_t ABS = 0x7FFFu, INF = 0x7F80u; };
+
+template <typename T> __device__ __forceinline__ float value_of(uint32_t raw) {
+    return widen(__builtin_bit_cast(T, static_cast<typename raw_bits<T>::type>(raw)));
+}
+template <typename T> __device__ __forceinline__ uint32_t raw_from(float v) {
+    return __builtin_bit_cast(typename raw_bits<T>::type, narrow<T>(v));
+}
+
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_other(uint32_t v) {
+    return static_cast<uint32_t>(
+        __builtin_amdgcn_update_dpp(static_cast<int>(v), static_cast<int>(v), CTRL, 0xF, 0xF, false));
+}
+template <int CTRL> __device__ __forceinline__ uint64_t dpp_other(uint64_t v) {
+    const uint64_t lo = dpp_other<CTRL>(static_cast<uint32_t>(v));
+    const uint64_t hi = dpp_other<CTRL>(static_cast<uint32_t>(v >> 32));
+    return lo | (hi << 32);
+}
+
+// The three largest keys seen so far, a >= b >= c; 0 stands for "none".
+template <typename K> struct top3 {
+    K a, b, c;
+    __device__ __forceinline__ void insert(K k) {
+        K lo = a < k ? a : k;
+        a = a < k ? k : a;
+        k = lo;
+        lo = b < k ? b : k;
+        b = b < k ? k : b;
+        c = c < lo ? lo : c;
+    }
+    template <int CTRL> __device__ __forceinline__ void merge_with_partner() {
+        const K oa = dpp_other<CTRL>(a), ob = dpp_other<CTRL>(b), oc = dpp_other<CTRL>(c);
+        insert(oa);
+        insert(ob);
+        insert(oc);
+    }
+    template <int LANES> __device__ __forceinline__ void merge_group() {
+        if constexpr (LANES >= 2) merge_with_partner<0xB1>();    // quad_perm [1,0,3,2]
+        if constexpr (LANES >= 4) merge_with_partner<0x4E>();    // quad_perm [2,3,0,1]
+        if constexpr (LANES >= 8) merge_with_partner<0x141>();   // row_half_mirror
+        if constexpr (LANES >= 16) merge_with_partner<0x140>();  // row_mirror
+    }
+};
+
+// Philox4x32-10: one block of four 32-bit words.
+__device__ __forceinline__ void philox_block(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
+                                             uint32_t (&out)[4]) {
+#pragma unroll
+    for (int round = 0; round < 10; ++round) {
+        if (round) {
+            k0 += 0x9E3779B9u;
+            k1 += 0xBB67AE85u;
+        }
+        const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+        c0 = n0;
+        c1 = lo1;
+        c2 = n2;
+        c3 = lo0;
+    }
+    out[0] = c0;
+    out[1] = c1;
+    out[2] = c2;
+    out[3] = c3;
+}
+
+template <typename T, int G> __device__ __forceinline__ int scan_start(int64_t group) {
+    if constexpr (sizeof(T) == 4) return 0;
+    else return 4 * static_cast<int>((group & 31) / (32 / (G / 4)));
+}
+
+__device__ __forceinline__ int meta_words_of(int topk) { return topk == 0 ? 1 : topk + 2; }
+
+// ---------------------------------------------------------------------------------------------
+// quantize: one wavefront per tile of 64 * VEC elements
+// ---------------------------------------------------------------------------------------------
+template <typename T, int G, int BIT>
+__global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGeneralQuantArgs a) {
+    using W = wire<T, BIT>;
+    using RB = raw_bits<T>;
+    using Raw = typename RB::type;
+    constexpr int VEC = W::VEC, LPG = G / VEC, ITEM = sizeof(T), CB = G * BIT / 8;
+    constexpr bool WIDE = ITEM == 4;
+    static_assert(LPG >= 2 && LPG <= 16, "a group must span 2..16 lanes of one DPP row");
+
+    __shared__ float book[16];
+    if (a.kind != 0) {   // uniform over the grid
+        if (threadIdx.x < 16) book[threadIdx.x] = kCodeBooks[a.kind - 1][threadIdx.x];
+        __syncthreads();
+    }
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t tile_first = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * W::TILE;
+    if (tile_first >= a.numel) return;   // wavefront-uniform
+    const int64_t e0 = tile_first + lane * VEC;
+    const bool live = e0 < a.numel;      // numel is a multiple of G: dead lanes form whole dead groups
+    const int64_t group = e0 / G;
+    const int k0 = static_cast<int>(e0 - group * G);
+    const int start = scan_start<T, G>(group);
+
+    Raw raw[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) raw[i] = 0;
+    if (live) load_elems<Raw, VEC, kPlain>(static_cast<const Raw *>(a.x) + e0, raw);
+    float v[VEC];
+    uint32_t mag[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        v[i] = value_of<T>(raw[i]);
+        mag[i] = raw[i] & RB::ABS;
+    }
+
+    const int meta_bytes = meta_words_of(a.topk) * ITEM;
+    const int64_t groups = a.numel / G;
+    uint8_t *group_codes = a.payload + (a.compact ? group * (CB + meta_bytes) : group * CB);
+    uint8_t *group_meta = a.compact ? group_codes + CB : a.payload + groups * CB + group * meta_bytes;
+
+    uint32_t scale_raw;
+    if (a.topk == 0) {
+        // (m > a) ? m : a over the scan: the maximum of what follows the last NaN, the NaN itself when it is last.
+        uint32_t m = 0;
+        bool has_nan = false;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const bool nan = mag[i] > RB::INF;
+            has_nan |= nan;
+            m = (!nan && mag[i] > m) ? mag[i] : m;
+        }
+        if (__ballot(has_nan) != 0) {   // wavefront-uniform, rare
+            uint32_t last = 0;          // 1 + scan position of the group's last NaN
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                const uint32_t pos = static_cast<uint32_t>(k0 + i - start) & (G - 1);
+                if (mag[i] > RB::INF && pos + 1 > last) last = pos + 1;
+            }
+            last = group_max_bits<LPG>(last);
+            const uint32_t from = last == G ? G - 1 : last;
+            m = 0;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                const uint32_t pos = static_cast<uint32_t>(k0 + i - start) & (G - 1);
+                if (pos >= from && mag[i] > m) m = mag[i];
+            }
+        }
+        scale_raw = group_max_bits<LPG>(m);
+    } else {
+        using K = typename pick_t<WIDE, uint64_t, uint32_t>::type;
+        top3<K> best{0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const int pos = (k0 + i - start) & (G - 1);
+            const bool candidate = WIDE ? mag[i] <= RB::INF : (mag[i] != 0 && mag[i] <= RB::INF);
+            const K rank = static_cast<K>(WIDE ? k0 + i + 1 : G - pos);   // 1..G, larger wins a tie
+            best.insert(candidate ? ((static_cast<K>(mag[i]) << 8) | rank) : K(0));
+        }
+        best.template merge_group<LPG>();
+        auto index_of = [&](K key) {
+            const int rank = static_cast<int>(key & 0xFF);
+            return WIDE ? rank - 1 : ((G - rank) + start) & (G - 1);
+        };
+        const bool none = best.a == 0;
+        const int index1 = none ? 0 : index_of(best.a);
+        int index2 = -1;
+        if (a.topk == 1) {
+            // nothing comparable: the reference falls back to element 1 (as stored for fp32, its magnitude otherwise)
+            const uint32_t element1 = WIDE ? static_cast<uint32_t>(raw[1]) : mag[1];
+            const uint32_t fallback = static_cast<uint32_t>(__shfl(static_cast<int>(element1), lane & ~(LPG - 1)));
+            scale_raw = none ? fallback : static_cast<uint32_t>(best.b >> 8);
+        } else {
+            const bool lonely = !none && best.b == 0;
+            index2 = none ? 1 : (lonely ? ((index1 + 1) & (G - 1)) : index_of(best.b));
+            scale_raw = (none || lonely) ? 0u : static_cast<uint32_t>(best.c >> 8);
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const bool first = k0 + i == index1, second = k0 + i == index2;
+            if (live && first) *reinterpret_cast<Raw *>(group_meta + 2 * ITEM) = raw[i];
+            if (live && second) *reinterpret_cast<Raw *>(group_meta + 3 * ITEM) = raw[i];
+            if (first || second) v[i] = 0.0f;
+        }
+        if (live && k0 == 0)
+            *reinterpret_cast<Raw *>(group_meta + ITEM) =
+                static_cast<Raw>(a.topk == 1 ? index1 : (index1 | (index2 << 8)));
+    }
+    if (live && k0 == 0) *reinterpret_cast<Raw *>(group_meta) = static_cast<Raw>(scale_raw);
+
+    float scale = value_of<T>(scale_raw);
+    scale = scale < 1.0e-6f ? 1.0e-6f : scale;   // a NaN scale stays NaN and encodes every element as 0
+
+    float uniform[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) uniform[i] = 0.0f;
+    if (a.stochastic) {
+        const uint32_t key0 = static_cast<uint32_t>(a.seed), key1 = static_cast<uint32_t>(a.seed >> 32);
+        const uint32_t sub0 = static_cast<uint32_t>(group), sub1 = static_cast<uint32_t>(static_cast<uint64_t>(group) >> 32);
+        const int phase = static_cast<int>(a.offset & 3);
+#pragma unroll
+        for (int q = 0; q < VEC / 4; ++q) {
+            const uint64_t position = static_cast<uint64_t>((k0 + 4 * q - start) & (G - 1));   // a multiple of 4
+            const uint64_t block = (a.offset + position) >> 2;
+            uint32_t lo[4], hi[4] = {0, 0, 0, 0};
+            philox_block(static_cast<uint32_t>(block), static_cast<uint32_t>(block >> 32), sub0, sub1, key0, key1, lo);
+            if (phase != 0)
+                philox_block(static_cast<uint32_t>(block + 1), static_cast<uint32_t>((block + 1) >> 32), sub0, sub1, key0,
+                             key1, hi);
+            const uint32_t w[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t x = phase == 0 ? w[e] : (phase == 1 ? w[e + 1] : (phase == 2 ? w[e + 2] : w[e + 3]));
+                uniform[4 * q + e] = static_cast<float>(x) * 0x1p-32f + 0x1p-33f;   // curand_uniform: (0, 1]
+            }
+        }
+    }
+
+    int c[VEC];
+    if (a.kind == 0) {
+        const float multiplier = W::LEVELS / scale;
+        constexpr int L = static_cast<int>(W::LEVELS);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            // nvcc contracts v * m + noise into one FMA; without noise the product is rounded alone
+            const float t = a.stochastic ? __builtin_fmaf(v[i], multiplier, uniform[i] - 0.5f) : v[i] * multiplier;
+            const int r = cvt_i32(__builtin_rintf(t));
+            c[i] = r < -L ? -L : (r > L ? L : r);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const float t = v[i] / scale;
+            int lower = 0;   // the largest entry in [0, 14] with not (t < book[entry]); NaN ends at 14
+#pragma unroll
+            for (int step = 8; step >= 1; step >>= 1) {
+                const int mid = lower + step;
+                if (mid < 15 && !(t < book[mid])) lower = mid;
+            }
+            const float low = book[lower], gap = book[lower + 1] - low, excess = t - low;
+            const bool up = a.stochastic ? uniform[i] < excess / gap : excess > gap * 0.5f;
+            c[i] = lower + (up ? 1 : 0);
+        }
+    }
+    if (live) {
+        uint32_t words[W::WORDS];
+        pack_codes<T, BIT, VEC, W::WORDS>(c, words);
+        store_piece<T, BIT, kPlain, W::WORDS>(group_codes + piece_offset<T, BIT>(k0), words);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dequantize (optionally combined into `out`)
+// ---------------------------------------------------------------------------------------------
+template <typename T, int G, int BIT>
+__global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireGeneralDecodeArgs a) {
+    using W = wire<T, BIT>;
+    using Raw = typename raw_bits<T>::type;
+    constexpr int VEC = W::VEC, ITEM = sizeof(T), CB = G * BIT / 8;
+
+    __shared__ float book[16];
+    if (a.kind != 0) {
+        if (threadIdx.x < 16) book[threadIdx.x] = kCodeBooks[a.kind - 1][threadIdx.x];
+        __syncthreads();
+    }
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t e0 = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * W::TILE + lane * VEC;
+    if (e0 >= a.numel) return;
+    const int64_t group = e0 / G;
+    const int k0 = static_cast<int>(e0 - group * G);
+    const int meta_bytes = meta_words_of(a.topk) * ITEM;
+    const int64_t groups = a.numel / G;
+    const uint8_t *group_codes = a.payload + (a.compact ? group * (CB + meta_bytes) : group * CB);
+    const uint8_t *group_meta = a.compact ? group_codes + CB : a.payload + groups * CB + group * meta_bytes;
+
+    uint32_t words[W::WORDS];
+    load_piece<T, BIT, kPlain, W::WORDS>(group_codes + piece_offset<T, BIT>(k0), words);
+    const float scale = value_of<T>(*reinterpret_cast<const Raw *>(group_meta));
+    const float step = a.kind == 0 ? step_of<BIT>(scale) : scale;
+
+    Raw decoded[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        const float code = unpack_code<T, BIT, W::WORDS>(words, i);
+        float value = code * step;
+        if (a.kind != 0) value = book[static_cast<int>(code) & 15] * step;
+        decoded[i] = static_cast<Raw>(raw_from<T>(value));
+    }
+    if (a.topk >= 1) {
+        const uint32_t indices = *reinterpret_cast<const Raw *>(group_meta + ITEM);
+        const Raw top1 = *reinterpret_cast<const Raw *>(group_meta + 2 * ITEM);
+        const int index1 = static_cast<int>(indices & 0xFFu);
+        int index2 = -1;
+        Raw top2 = 0;
+        if (a.topk == 2) {
+            index2 = static_cast<int>((indices >> 8) & 0xFFu);
+            top2 = *reinterpret_cast<const Raw *>(group_meta + 3 * ITEM);
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            if (k0 + i == index1) decoded[i] = top1;
+            if (k0 + i == index2) decoded[i] = top2;   // written second, as in the reference
+        }
+    }
+    Raw *out = static_cast<Raw *>(a.out) + e0;
+    if (a.op != 0) {
+        Raw old[VEC];
+        load_elems<Raw, VEC, kPlain>(out, old);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const float o = value_of<T>(old[i]), d = value_of<T>(decoded[i]);
+            if (a.op == 1) decoded[i] = static_cast<Raw>(raw_from<T>(add_rounded_once<T>(o, d)));
+            else if (a.op == 2) decoded[i] = o > d ? old[i] : decoded[i];
+            else decoded[i] = o > d ? decoded[i] : old[i];
+        }
+    }
+    store_elems<Raw, VEC, kPlain>(out, decoded);
+}
+
+template <typename T, int G>
+hipError_t launch_general_quant_g(int bit, const WireGeneralQuantArgs &a, hipStream_t stream) {
+    const int64_t tile = wire<T, 8>::TILE * kWavesPerBlock;
+    const int64_t blocks = (a.numel + tile - 1) / tile;
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks));
+    if (bit == 8) hipLaunchKernelGGL((wire_general_quant_kernel<T, G, 8>), grid, dim3(kBlock), 0, stream, a);
+    else if (bit == 4) hipLaunchKernelGGL((wire_general_quant_kernel<T, G, 4>), grid, dim3(kBlock), 0, stream, a);
+    else return hipErrorNotSupported;
+    return hipGetLastError();
+}
+
+template <typename T> hipError_t launch_general_quant_t(int g, int bit, const WireGeneralQuantArgs &a, hipStream_t s) {
+    switch (g) {
+        case 64: return launch_general_quant_g<T, 64>(bit, a, s);
+        case 32: return launch_general_quant_g<T, 32>(bit, a, s);
+        case 16: return launch_general_quant_g<T, 16>(bit, a, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
+template <typename T, int G>
+hipError_t launch_general_decode_g(int bit, const WireGeneralDecodeArgs &a, hipStream_t stream) {
+    const int64_t tile = wire<T, 8>::TILE * kWavesPerBlock;
+    const int64_t blocks = (a.numel + tile - 1) / tile;
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks));
+    if (bit == 8) hipLaunchKernelGGL((wire_general_decode_kernel<T, G, 8>), grid, dim3(kBlock), 0, stream, a);
+    else if (bit == 4) hipLaunchKernelGGL((wire_general_decode_kernel<T, G, 4>), grid, dim3(kBlock), 0, stream, a);
+    else return hipErrorNotSupported;
+    return hipGetLastError();
+}
+
+template <typename T> hipError_t launch_general_decode_t(int g, int bit, const WireGeneralDecodeArgs &a, hipStream_t s) {
+    switch (g) {
+        case 64: return launch_general_decode_g<T, 64>(bit, a, s);
+        case 32: return launch_general_decode_g<T, 32>(bit, a, s);
+        case 16: return launch_general_decode_g<T, 16>(bit, a, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_wire_general_quant(int dtype, int group_size, int bit, const WireGeneralQuantArgs &args,
+                                     hipStream_t stream) {
+    switch (dtype) {
+        case kF32: return launch_general_quant_t<float>(group_size, bit, args, stream);
+        case kF16: return launch_general_quant_t<f16>(group_size, bit, args, stream);
+        case kBF16: return launch_general_quant_t<bf16>(group_size, bit, args, stream);
+        default: return hipErrorNotSupported;
+    }
+}
+
+hipError_t launch_wire_general_decode(int dtype, int group_size, int bit, const WireGeneralDecodeArgs &args,
+                                      hipStream_t stream) {
+    switch (dtype) {
+        case kF32: return launch_general_decode_t<float>(group_size, bit, args, stream);
+        case kF16: return launch_general_decode_t<f16>(group_size, bit, args, stream);
+        case kBF16: return launch_general_decode_t<bf16>(group_size, bit, args, stream);
+        default: return hipErrorNotSupported;
+    }
+}
+
+}  // namespace lbc

@@ -44,6 +44,9 @@ using vec_t = T __attribute__((ext_vector_type(N)));
 template <typename T> struct is_void_t { static constexpr bool value = false; };
 template <> struct is_void_t<void> { static constexpr bool value = true; };
 
+template <bool PICK_FIRST, typename A, typename B> struct pick_t { using type = A; };
+template <typename A, typename B> struct pick_t<false, A, B> { using type = B; };
+
 template <typename A, typename B> struct same_t { static constexpr bool value = false; };
 template <typename A> struct same_t<A, A> { static constexpr bool value = true; };
 

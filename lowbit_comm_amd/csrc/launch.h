@@ -89,6 +89,29 @@ struct WireDecodeArgs {
     int compact;
 };
 
+// The general policies of the CUDA extension's format (code books, stochastic rounding, top-k).
+struct WireGeneralQuantArgs {
+    const void *x;
+    uint8_t *payload;
+    int64_t numel;       // a multiple of the group size
+    int kind;            // 0 linear, 1 normal, 2 uniform, 3 e3m0, 4 e2m1
+    int topk;            // 0, 1, 2
+    int stochastic;
+    int compact;
+    uint64_t seed;       // Philox key
+    uint64_t offset;     // Philox offset (draws skipped in every group's stream)
+};
+
+struct WireGeneralDecodeArgs {
+    const uint8_t *payload;
+    void *out;
+    int64_t numel;
+    int kind;
+    int topk;
+    int compact;
+    int op;              // 0 none, 1 sum, 2 max, 3 min
+};
+
 // Each returns hipSuccess/last launch error, or hipErrorNotSupported when no
 // instantiation exists for the type combination.
 // `mode` is an lbc::AccessMode: 0 element-wise (any alignment), 1 vector, 2 vector + non-temporal.
@@ -115,5 +138,10 @@ hipError_t launch_wire_reduce(int dtype, int group_size, int world, bool fused_m
                               const WireReduceArgs &args, hipStream_t stream);
 hipError_t launch_wire_decode(int dtype, int group_size, int bit, int reduce_op, int mode, const WireDecodeArgs &args,
                               int world, hipStream_t stream);
+
+hipError_t launch_wire_general_quant(int dtype, int group_size, int bit, const WireGeneralQuantArgs &args,
+                                     hipStream_t stream);
+hipError_t launch_wire_general_decode(int dtype, int group_size, int bit, const WireGeneralDecodeArgs &args,
+                                      hipStream_t stream);
 
 }  // namespace lbc

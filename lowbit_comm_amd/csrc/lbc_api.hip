@@ -436,4 +436,67 @@ int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t n
                   "lbc_wire_dequant_reduce");
 }
 
+// ---- general policies of that format: code books, stochastic rounding, top-k ------------------
+static bool valid_general(int group_size, int bit, int quant_type, int topk) {
+    if (!valid_group(group_size) || (bit != 8 && bit != 4) || topk < 0 || topk > 2) return false;
+    if (quant_type < LBC_QUANT_LINEAR || quant_type > LBC_QUANT_E2M1) return false;
+    return quant_type == LBC_QUANT_LINEAR || bit == 4;
+}
+
+int64_t lbc_wire_general_payload_nbytes(int64_t numel, int group_size, int dtype, int bit, int topk) {
+    if (numel < 0 || !valid_dtype(dtype) || !valid_general(group_size, bit, LBC_QUANT_LINEAR, topk)) return -1;
+    const int64_t groups = numel == 0 ? 0 : (numel + group_size - 1) / group_size;
+    return groups * (group_size * bit / 8 + dtype_size(dtype) * (topk == 0 ? 1 : topk + 2));
+}
+
+int lbc_wire_quant_general(const void *x, int dtype, int64_t numel, int group_size, int bit, int quant_type, int topk,
+                           int stochastic, uint64_t seed, uint64_t offset, int compact, uint8_t *payload, void *stream) {
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported dtype %d", dtype);
+    if (!valid_general(group_size, bit, quant_type, topk)) return LBC_UNSUPPORTED;
+    if (numel % group_size != 0) return fail(LBC_EINVAL, "input numel should be multiple of group_size");
+    if (numel == 0) return LBC_OK;
+    const int item = dtype_size(dtype);
+    if (x == nullptr || payload == nullptr) return fail(LBC_EINVAL, "input and payload must not be null");
+    if (!aligned_to(x, item) || !aligned_to(payload, item))
+        return fail(LBC_EINVAL, "input/payload must be aligned to the element size");
+    lbc::WireGeneralQuantArgs a{};
+    a.x = x;
+    a.payload = payload;
+    a.numel = numel;
+    a.kind = quant_type;
+    a.topk = topk;
+    a.stochastic = stochastic != 0;
+    a.compact = compact != 0;
+    a.seed = seed;
+    a.offset = offset;
+    return finish(lbc::launch_wire_general_quant(dtype, group_size, bit, a, static_cast<hipStream_t>(stream)),
+                  "lbc_wire_quant_general");
+}
+
+int lbc_wire_dequant_general(const uint8_t *payload, int64_t numel, int group_size, int bit, int quant_type, int topk,
+                             int compact, void *out, int dtype, int reduce_op, void *stream) {
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported dtype %d", dtype);
+    if (reduce_op < LBC_REDUCE_NONE || reduce_op > LBC_REDUCE_MIN)
+        return fail(LBC_EINVAL, "unsupported reduce op %d", reduce_op);
+    if (!valid_general(group_size, bit, quant_type, topk)) return LBC_UNSUPPORTED;
+    if (numel % group_size != 0) return fail(LBC_EINVAL, "numel should be multiple of group_size");
+    if (numel == 0) return LBC_OK;
+    const int item = dtype_size(dtype);
+    if (payload == nullptr || out == nullptr) return fail(LBC_EINVAL, "payload and out must not be null");
+    if (!aligned_to(payload, item) || !aligned_to(out, item))
+        return fail(LBC_EINVAL, "payload/out must be aligned to the element size");
+    lbc::WireGeneralDecodeArgs a{};
+    a.payload = payload;
+    a.out = out;
+    a.numel = numel;
+    a.kind = quant_type;
+    a.topk = topk;
+    a.compact = compact != 0;
+    a.op = reduce_op;
+    return finish(lbc::launch_wire_general_decode(dtype, group_size, bit, a, static_cast<hipStream_t>(stream)),
+                  "lbc_wire_dequant_general");
+}
+
 }  // extern "C"

@@ -1,0 +1,191 @@
+// Byte layout and small arithmetic helpers shared by the kernels that read and write the payload
+// format of the reference's CUDA extension (cuda_wire.hip, cuda_wire_general.hip).
+#pragma once
+#include "device_utils.h"
+
+namespace lbc {
+
+constexpr int kPlain = 0, kNonTemporal = 1;
+
+// N 32-bit words at an address aligned to ALIGN bytes.
+template <int N, int ALIGN> struct words_at {
+    typedef vec_t<uint32_t, N> type __attribute__((aligned(ALIGN)));
+};
+
+template <int N, int ALIGN, int NT>
+__device__ __forceinline__ void load_words(const uint8_t *p, uint32_t (&w)[N]) {
+    using V = typename words_at<N, ALIGN>::type;
+    vec_t<uint32_t, N> v;
+    if constexpr (NT == kNonTemporal) v = __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+    else v = *reinterpret_cast<const V *>(p);
+#pragma unroll
+    for (int i = 0; i < N; ++i) w[i] = v[i];
+}
+
+template <int N, int ALIGN, int NT>
+__device__ __forceinline__ void store_words(uint8_t *p, const uint32_t (&w)[N]) {
+    using V = typename words_at<N, ALIGN>::type;
+    vec_t<uint32_t, N> v;
+#pragma unroll
+    for (int i = 0; i < N; ++i) v[i] = w[i];
+    if constexpr (NT == kNonTemporal) __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
+    else *reinterpret_cast<V *>(p) = v;
+}
+
+// VEC elements of T at an address aligned to sizeof(T) only.
+template <typename T, int VEC, int NT>
+__device__ __forceinline__ void load_elems(const T *p, T (&dst)[VEC]) {
+    typedef vec_t<T, VEC> V __attribute__((aligned(sizeof(T))));
+    vec_t<T, VEC> v;
+    if constexpr (NT == kNonTemporal) v = __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+    else v = *reinterpret_cast<const V *>(p);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) dst[i] = v[i];
+}
+
+template <typename T, int VEC, int NT>
+__device__ __forceinline__ void store_elems(T *p, const T (&src)[VEC]) {
+    typedef vec_t<T, VEC> V __attribute__((aligned(sizeof(T))));
+    vec_t<T, VEC> v;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = src[i];
+    if constexpr (NT == kNonTemporal) __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
+    else *reinterpret_cast<V *>(p) = v;
+}
+
+template <typename T, int BIT = 8> struct wire {
+    static constexpr int ITEM = sizeof(T);
+    static constexpr int VEC = 16 / ITEM;                  // elements per lane: 16 bytes of the tensor
+    static constexpr int CODE_BYTES = VEC * BIT / 8;        // 8, 4 or (4-bit codes of an fp32 tensor) 2
+    static constexpr int WORDS = CODE_BYTES >= 4 ? CODE_BYTES / 4 : 1;   // 32-bit registers holding them
+    static constexpr int TILE = kWave * VEC;
+    static constexpr float LEVELS = BIT == 8 ? 127.0f : 7.0f;
+};
+
+// Byte position of element k (0..3) inside its 32-bit word: fp32 payloads reverse all four
+// bytes, 16-bit payloads swap byte pairs.
+template <typename T> __device__ __forceinline__ constexpr int byte_in_word(int k) {
+    return sizeof(T) == 4 ? 3 - k : (k ^ 1);
+}
+// Byte position of element k of a group inside the group's code bytes.
+template <typename T> __device__ __forceinline__ int byte_in_group(int k) {
+    constexpr int ITEM = sizeof(T);
+    return (k / ITEM) * ITEM + (ITEM - 1 - k % ITEM);
+}
+
+// COMPACT payloads interleave [G code bytes][scale] per group, so a 128-byte line is shared by
+// neighbouring wavefront instructions and payload accesses must stay cacheable even when the tensors
+// stream with the non-temporal hint (the hint would drop the line between its two uses).  Otherwise
+// the policy measured for the portable format applies: code stores follow the tensors' hint, code
+// loads are non-temporal only from four payloads on.
+template <typename T, int G, bool COMPACT, int BIT = 8> struct group_layout {
+    static constexpr int ITEM = sizeof(T);
+    static constexpr int CB = G * BIT / 8;      // code bytes per group
+    const int64_t groups;
+    __device__ __forceinline__ int64_t codes(int64_t group) const { return COMPACT ? group * (CB + ITEM) : group * CB; }
+    __device__ __forceinline__ int64_t scale(int64_t group) const {
+        return COMPACT ? group * (CB + ITEM) + CB : groups * CB + group * ITEM;
+    }
+};
+
+// The VEC codes of one lane -> its 32-bit words, in the byte / nibble order of the format.
+template <typename T, int BIT, int VEC, int WORDS>
+__device__ __forceinline__ void pack_codes(const int (&c)[VEC], uint32_t (&words)[WORDS]) {
+    if constexpr (BIT == 8) {
+#pragma unroll
+        for (int k = 0; k < WORDS; ++k) {
+            if constexpr (sizeof(T) == 4) words[k] = pack4(c[4 * k + 3], c[4 * k + 2], c[4 * k + 1], c[4 * k]);
+            else words[k] = pack4(c[4 * k + 1], c[4 * k], c[4 * k + 3], c[4 * k + 2]);
+        }
+    } else {
+        // Four codes make one 16-bit unit with the first code on top.  A 16-bit tensor's lane holds two
+        // such units, low half first; an fp32 tensor's lane holds one (half of a 32-bit payload word).
+        static_assert(WORDS == 1 && (VEC == 8 || VEC == 4), "a 4-bit lane owns at most one register");
+        uint32_t word = 0;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+            word |= (static_cast<uint32_t>(c[i]) & 0xFu) << (16 * (i / 4) + 12 - 4 * (i % 4));
+        words[0] = word;
+    }
+}
+
+// Byte offset, inside a group's code bytes, of the piece owned by the lane whose first element is k0.
+// An fp32 payload word holds eight 4-bit codes, elements 0-3 in its upper half: the two lanes sharing a
+// word write its halves swapped, which keeps a wavefront's 2-byte accesses one contiguous run.
+template <typename T, int BIT> __device__ __forceinline__ int piece_offset(int k0) {
+    if constexpr (BIT == 4 && sizeof(T) == 4) return (k0 / 8) * 4 + ((k0 & 4) ? 0 : 2);
+    else return k0 * BIT / 8;
+}
+
+template <typename T, int BIT, int PNT, int WORDS>
+__device__ __forceinline__ void store_piece(uint8_t *p, const uint32_t (&words)[WORDS]) {
+    if constexpr (wire<T, BIT>::CODE_BYTES == 2) *reinterpret_cast<uint16_t *>(p) = static_cast<uint16_t>(words[0]);
+    else store_words<WORDS, sizeof(T), PNT>(p, words);
+}
+
+template <typename T, int BIT, int PNT, int WORDS>
+__device__ __forceinline__ void load_piece(const uint8_t *p, uint32_t (&words)[WORDS]) {
+    if constexpr (wire<T, BIT>::CODE_BYTES == 2) words[0] = *reinterpret_cast<const uint16_t *>(p);
+    else load_words<WORDS, sizeof(T), PNT>(p, words);
+}
+
+// Code i of the lane's words as a float.
+template <typename T, int BIT, int WORDS>
+__device__ __forceinline__ float unpack_code(const uint32_t (&words)[WORDS], int i) {
+    if constexpr (BIT == 8) {
+        return code_to_float(words[i / 4], byte_in_word<T>(i % 4));
+    } else {
+        const int top = 16 - 16 * (i / 4) + 4 * (i % 4);   // left shift that puts the nibble on top
+        return static_cast<float>(static_cast<int32_t>(words[0] << top) >> 28);
+    }
+}
+
+// Code of element k of a group read from the group's code bytes (ragged-edge path).
+template <typename T, int BIT> __device__ __forceinline__ float code_at(const uint8_t *group_codes, int k) {
+    if constexpr (BIT == 8) {
+        return static_cast<float>(static_cast<int8_t>(group_codes[byte_in_group<T>(k)]));
+    } else {
+        constexpr int ITEM = sizeof(T), PER_WORD = 2 * ITEM;
+        const int in_word = k % PER_WORD;
+        const uint32_t byte = group_codes[(k / PER_WORD) * ITEM + (ITEM - 1 - in_word / 2)];
+        const uint32_t nibble = (in_word & 1) ? (byte & 0xFu) : (byte >> 4);
+        return static_cast<float>(static_cast<int32_t>(nibble << 28) >> 28);
+    }
+}
+
+// float(scale) / levels with IEEE rounding.
+template <int BIT> __device__ __forceinline__ float step_of(float stored);
+
+template <bool COMPACT, int NT, int WORLD> constexpr int payload_load_hint() { return COMPACT || WORLD < 4 ? kPlain : NT; }
+
+// float(scale) / 127 with IEEE rounding: the three-operation form proven exhaustively for
+// every finite float (tests/native/check_scale127.c); an infinite scale passes through.
+static __device__ __forceinline__ float div127(float a) {
+    const float c = as_f32(0x3C010204u);
+    const float q0 = a * c;
+    const float r = __builtin_fmaf(-q0, 127.0f, a);
+    const float q = __builtin_fmaf(r, c, q0);
+    return (as_u32(a) & 0x7FFFFFFFu) == 0x7F800000u ? a : q;
+}
+
+template <> __device__ __forceinline__ float step_of<8>(float stored) { return div127(stored); }
+template <> __device__ __forceinline__ float step_of<4>(float stored) { return stored / 7.0f; }
+
+// a + b rounded once to T (what a native half / bfloat16 add returns): the float sum is turned
+// into a round-to-odd result with the exact error term, then rounded to T.
+template <typename T> __device__ __forceinline__ float add_rounded_once(float a, float b) {
+    float s = a + b;
+    if constexpr (same_t<T, float>::value) return s;
+    const float bb = s - a;
+    const float err = (a - (s - bb)) + (b - bb);
+    uint32_t u = as_u32(s);
+    const bool finite = (u & 0x7F800000u) != 0x7F800000u;
+    if (err != 0.0f && finite && (u & 1u) == 0) {
+        const bool larger_magnitude = (err > 0.0f) == (s > 0.0f);
+        u = larger_magnitude ? u + 1u : u - 1u;
+        s = as_f32(u);
+    }
+    return round_through<T>(s);
+}
+
+}  // namespace lbc

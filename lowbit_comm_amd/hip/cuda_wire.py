@@ -149,3 +149,63 @@ def dequant_reduce_into(payloads: Sequence[torch.Tensor], out: torch.Tensor, **k
     ``inplace_dequantize_reduce_mean_update_error_feedback``."""
     bound = bind_dequant_reduce(payloads, out, **kwargs)
     return False if bound is None else bound()
+
+
+# ---------------------------------------------------------------------------------------------------------
+# the extension's remaining policies: non-linear 4-bit code books, stochastic rounding, top-k side channel
+# ---------------------------------------------------------------------------------------------------------
+QUANT_TYPES = {"linear": 0, "normal": 1, "uniform": 2, "e3m0": 3, "e2m1": 4}
+_META_WORDS = {0: 1, 1: 3, 2: 4}
+
+
+def general_payload_nbytes(numel: int, dtype: torch.dtype, group_size: int = 64, bit: int = 8, topk: int = 0) -> int:
+    """``G * (g*bit/8 + element size * (1 | 3 | 4))`` (ccdl_comm/csrc/quantization/gen_code_quant.py:167-178)."""
+    _require(topk in _META_WORDS, f"topk must be 0, 1 or 2, got {topk}")
+    item = torch.empty((), dtype=dtype).element_size()
+    return num_groups(numel, group_size) * (group_size * bit // 8 + item * _META_WORDS[topk])
+
+
+def _policy(quant_type: str, bit: int, topk: int) -> int:
+    _require(quant_type in QUANT_TYPES, f"unsupported quant_type {quant_type!r}")
+    _require(topk in _META_WORDS, f"topk must be 0, 1 or 2, got {topk}")
+    _require(quant_type == "linear" or bit == 4, f"quant_type {quant_type!r} only supports 4-bit codes")
+    return QUANT_TYPES[quant_type]
+
+
+def bind_quant_general(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64, bit: int = 8,
+                       quant_type: str = "linear", topk: int = 0, stochastic: tuple[int, int] | None = None,
+                       compact: bool = False) -> BoundLaunch:
+    """``stochastic`` is the (seed, offset) pair of the Philox stream, ``None`` for round-to-nearest."""
+    lib = load_library()
+    code = _float_tensor(x, "input")
+    kind = _policy(quant_type, bit, topk)
+    _require(x.numel() % group_size == 0, "input numel should be multiple of group_size")
+    _payload(payload, "output", x.device, general_payload_nbytes(x.numel(), x.dtype, group_size, bit, topk))
+    seed, offset = (0, 0) if stochastic is None else (int(stochastic[0]), int(stochastic[1]))
+    args = (_ptr(x), code, x.numel(), group_size, int(bit), kind, int(topk), int(stochastic is not None),
+            seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF, int(compact), _ptr(payload))
+    return BoundLaunch(lib.lbc_wire_quant_general, args, x.device, lib, (x, payload))
+
+
+def quant_general_into(x: torch.Tensor, payload: torch.Tensor, **policy) -> bool:
+    """Replaces native ``inplace_quantize`` for every policy of the reference's extension."""
+    return bind_quant_general(x, payload, **policy)()
+
+
+def bind_dequant_general(payload: torch.Tensor, out: torch.Tensor, *, group_size: int = 64, bit: int = 8,
+                         quant_type: str = "linear", topk: int = 0, compact: bool = False,
+                         reduce_op: str = "none") -> BoundLaunch:
+    lib = load_library()
+    code = _float_tensor(out, "output")
+    kind = _policy(quant_type, bit, topk)
+    _require(reduce_op in REDUCE_OPS, f"unsupported reduce op {reduce_op!r}")
+    _require(out.numel() % group_size == 0, "output numel should be multiple of group_size")
+    _payload(payload, "input", out.device, general_payload_nbytes(out.numel(), out.dtype, group_size, bit, topk))
+    args = (_ptr(payload), out.numel(), group_size, int(bit), kind, int(topk), int(compact), _ptr(out), code,
+            REDUCE_OPS[reduce_op])
+    return BoundLaunch(lib.lbc_wire_dequant_general, args, out.device, lib, (payload, out))
+
+
+def dequant_general_into(payload: torch.Tensor, out: torch.Tensor, **policy) -> bool:
+    """Replaces native ``inplace_dequantize`` for every policy of the reference's extension."""
+    return bind_dequant_general(payload, out, **policy)()

@@ -11,7 +11,7 @@ from pathlib import Path
 from lowbit_comm_amd.exceptions import CCDLUnavailableError
 
 LIBRARY_PATH = Path(__file__).resolve().parent.parent / "liblbc_hip.so"
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 LBC_OK = 0
 LBC_UNSUPPORTED = 1
@@ -45,6 +45,11 @@ SIGNATURES = {
                                          _c_int, _c_int, _c_ptr]),
     "lbc_wire_dequant_reduce": (_c_int, [_c_ptr, _c_int, _c_i64, _c_int, _c_int, ctypes.c_float, _c_int, _c_ptr,
                                          _c_int, _c_ptr, _c_ptr, _c_ptr]),
+    "lbc_wire_general_payload_nbytes": (_c_i64, [_c_i64, _c_int, _c_int, _c_int, _c_int]),
+    "lbc_wire_quant_general": (_c_int, [_c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.c_uint64,
+                                        ctypes.c_uint64, _c_int, _c_ptr, _c_ptr]),
+    "lbc_wire_dequant_general": (_c_int, [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int,
+                                          _c_int, _c_ptr]),
 }
 
 _library: ctypes.CDLL | None = None

@@ -1,0 +1,176 @@
+"""GPU parity of the general CUDA-format kernels (code books, stochastic rounding, top-k side channel,
+NaN-resetting maximum) against the CPU oracle (oracle/cuda_wire_general_np.py): payload bytes and decoded
+values, bit-exact; size-independent properties at the full bucket size."""
+from __future__ import annotations
+
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cuda_wire_general_np as general
+from oracle import cuda_wire_np as wire
+
+from tests.test_cuda_wire_parity import NAMES, from_numpy, same, to_numpy
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip(hip_device):
+    from lowbit_comm_amd.hip import cuda_wire
+
+    return cuda_wire
+
+
+def policies():
+    for bit, topk, stochastic in itertools.product((4, 8), (0, 1, 2), (None, (42, 8), (7, 3))):
+        for quant_type in (general.QUANT_TYPES if bit == 4 else ("linear",)):
+            yield bit, quant_type, topk, stochastic
+
+
+def awkward_values(rng, n, g, case):
+    values = (rng.standard_normal(n) * rng.choice([1e-7, 1e-3, 1.0, 100.0])).astype(np.float32)
+    values[rng.integers(0, n, max(1, n // 40))] = 0.0
+    values[rng.integers(0, n, max(1, n // 500))] *= 50.0
+    if case % 2 == 0 and n >= 8 * g:
+        values[rng.integers(0, n, 1 + n // 300)] = np.nan
+        values[rng.integers(0, n, 3)] = np.inf
+        values[g:2 * g] = np.nan                      # nothing comparable
+        values[2 * g:3 * g] = 0.0                     # nothing non-zero
+        values[3 * g:4 * g] = -2.5                    # all equal
+        values[4 * g:5 * g] = 0.0
+        values[4 * g + 5] = 3.0                       # a single non-zero
+        values[5 * g + g - 1] = np.nan                # a NaN that ends an fp32 scan
+        values[6 * g:7 * g] = np.nan
+        values[6 * g + 1] = 4.0                       # one comparable element among NaNs
+    return values
+
+
+@pytest.mark.parametrize("name", list(NAMES))
+@pytest.mark.parametrize("g", (16, 32, 64))
+@pytest.mark.parametrize("compact", (False, True))
+def test_quantize_and_decode_bytes(hip, hip_device, name, g, compact):
+    rng = np.random.default_rng(g + 7 * compact)
+    for case, (bit, quant_type, topk, stochastic) in enumerate(policies()):
+        n = g * int(rng.choice([1, 7, 70, 1031]))      # 1031 groups: tiles end inside the last block
+        x_np = wire.from_f32(awkward_values(rng, n, g, case), name)
+        x = from_numpy(x_np, name, hip_device)
+        policy = dict(group_size=g, bit=bit, quant_type=quant_type, topk=topk, compact=compact)
+        what = f"{name} g={g} {policy} stochastic={stochastic} n={n}"
+        payload = torch.full((hip.general_payload_nbytes(n, x.dtype, g, bit, topk),), 0xA5, dtype=torch.uint8,
+                             device=hip_device)
+        assert hip.quant_general_into(x, payload, stochastic=stochastic, **policy), what
+        want = general.quantize(x_np, name, g, bit, quant_type, topk, stochastic, compact)
+        same(payload, want, "quantize " + what)
+        old_np = wire.from_f32((rng.standard_normal(n) * 0.5).astype(np.float32), name)
+        for op in ("none", "sum", "max", "min"):
+            out = from_numpy(old_np, name, hip_device)
+            assert hip.dequant_general_into(payload, out, reduce_op=op, **policy), what
+            same(out, general.dequantize(want, n, name, g, bit, quant_type, topk, compact, op, old_np),
+                 f"decode {op} " + what)
+
+
+@pytest.mark.parametrize("name", list(NAMES))
+def test_plain_policy_equals_the_pack_kernel_on_finite_input(hip, hip_device, name):
+    n = 64 * 4000
+    x = from_numpy(wire.from_f32((np.random.default_rng(3).standard_normal(n) * 0.02).astype(np.float32), name), name,
+                   hip_device)
+    for bit, compact in itertools.product((4, 8), (False, True)):
+        fast = hip.quant_pack(x, group_size=64, compact=compact, bit=bit)
+        payload = torch.empty_like(fast)
+        assert hip.quant_general_into(x, payload, group_size=64, bit=bit, compact=compact)
+        assert torch.equal(fast, payload)
+        a, b = torch.empty_like(x), torch.empty_like(x)
+        assert hip.dequant_into(fast, a, group_size=64, compact=compact, bit=bit)
+        assert hip.dequant_general_into(fast, b, group_size=64, bit=bit, compact=compact)
+        assert torch.equal(a.view(torch.int16 if name != "fp32" else torch.int32),
+                           b.view(torch.int16 if name != "fp32" else torch.int32))
+
+
+def test_contract_violations(hip, hip_device):
+    x = torch.zeros(64 * 3, device=hip_device)
+    payload = torch.empty(hip.general_payload_nbytes(x.numel(), x.dtype, 64, 8, 1), dtype=torch.uint8, device=hip_device)
+    with pytest.raises(RuntimeError, match="multiple of group_size"):
+        hip.quant_general_into(x[:100], payload, topk=1)
+    with pytest.raises(RuntimeError, match="invalid quantized payload size"):
+        hip.quant_general_into(x, payload[:-4], topk=1)
+    with pytest.raises(RuntimeError, match="only supports 4-bit"):
+        hip.quant_general_into(x, payload, quant_type="normal", bit=8)
+    with pytest.raises(RuntimeError, match="topk must be"):
+        hip.quant_general_into(x, payload, topk=3)
+    empty = torch.empty(0, device=hip_device)
+    assert hip.quant_general_into(empty, torch.empty(0, dtype=torch.uint8, device=hip_device), topk=2)
+
+
+# --------------------------------------------------------------------------- #
+# the 100 MiB bucket: properties that need no oracle pass over the whole tensor
+# --------------------------------------------------------------------------- #
+FULL = 26_214_400
+
+
+@pytest.mark.parametrize("name", ("fp32", "bf16"))
+def test_full_bucket_top2_restores_outliers_and_bounds_the_rest(hip, hip_device, name):
+    gen = torch.Generator(device=hip_device).manual_seed(1234)
+    x = (torch.randn(FULL, generator=gen, device=hip_device) * 1e-3).to(NAMES[name])
+    g = 64
+    payload = torch.empty(hip.general_payload_nbytes(FULL, x.dtype, g, 8, 2), dtype=torch.uint8, device=hip_device)
+    assert hip.quant_general_into(x, payload, group_size=g, topk=2, compact=True)
+    out = torch.empty_like(x)
+    assert hip.dequant_general_into(payload, out, group_size=g, topk=2, compact=True)
+    rows, got = x.float().view(-1, g), out.float().view(-1, g)
+    order = rows.abs().argsort(dim=1, descending=True)
+    top = order[:, :2]
+    assert torch.equal(rows.gather(1, top), got.gather(1, top))                 # outliers travel verbatim
+    third = rows.abs().gather(1, order[:, 2:3])
+    error = (rows - got).abs()
+    slack = 2.0 ** (-8 if name == "bf16" else -23)
+    assert bool((error <= third / 254 * 1.0001 + got.abs() * slack).all())
+    # the oracle on the first and last 64 Ki elements
+    for block in (slice(0, 65536), slice(FULL - 65536, FULL)):
+        part = torch.empty(hip.general_payload_nbytes(65536, x.dtype, g, 8, 2), dtype=torch.uint8, device=hip_device)
+        assert hip.quant_general_into(x[block].clone(), part, group_size=g, topk=2, compact=True)
+        if block.start == 0:       # group indices (which fix the 16-bit scan start) match the full run only here
+            same(payload[:part.numel()], to_numpy(part), "prefix of the full payload")
+        same(part, general.quantize(to_numpy(x[block]), name, g, 8, "linear", 2, None, True), "block against the oracle")
+
+
+def test_full_bucket_stochastic_rounding_is_unbiased_and_repeatable(hip, hip_device):
+    gen = torch.Generator(device=hip_device).manual_seed(99)
+    x = torch.randn(FULL, generator=gen, device=hip_device) * 1e-3
+    g = 64
+    payload = torch.empty(hip.general_payload_nbytes(FULL, x.dtype, g, 8, 0), dtype=torch.uint8, device=hip_device)
+    again = torch.empty_like(payload)
+    out = torch.empty_like(x)
+    assert hip.quant_general_into(x, payload, group_size=g, stochastic=(2024, 1 << 20))
+    assert hip.quant_general_into(x, again, group_size=g, stochastic=(2024, 1 << 20))
+    assert torch.equal(payload, again)
+    assert hip.quant_general_into(x, again, group_size=g, stochastic=(2024, (1 << 20) + 4 * FULL))
+    assert not torch.equal(payload, again)
+    assert hip.dequant_general_into(payload, out, group_size=g)
+    step = x.view(-1, g).abs().amax(dim=1, keepdim=True) / 127
+    error = ((out - x).view(-1, g) / step).double()
+    assert float(error.abs().max()) <= 1.0 + 1e-3                               # one of the two neighbouring codes
+    assert abs(float(error.mean())) < 5 * (1 / 6 / FULL) ** 0.5                 # variance of u(1-u) averaged is 1/6
+    # nearest rounding on the same data has a smaller error but is no closer on average
+    assert 0.15 < float((error ** 2).mean()) < 0.18
+    same(payload[:64 * 1024], general.quantize(to_numpy(x[:65536]), "fp32", g, 8, "linear", 0, (2024, 1 << 20), False)[:64 * 1024],
+         "codes of the first 1024 groups")
+
+
+@pytest.mark.parametrize("quant_type", ("normal", "e2m1"))
+def test_full_bucket_code_book_decode_is_the_nearest_entry(hip, hip_device, quant_type):
+    gen = torch.Generator(device=hip_device).manual_seed(5)
+    x = torch.randn(FULL, generator=gen, device=hip_device)
+    g = 64
+    payload = torch.empty(hip.general_payload_nbytes(FULL, x.dtype, g, 4, 0), dtype=torch.uint8, device=hip_device)
+    out = torch.empty_like(x)
+    assert hip.quant_general_into(x, payload, group_size=g, bit=4, quant_type=quant_type, compact=True)
+    assert hip.dequant_general_into(payload, out, group_size=g, bit=4, quant_type=quant_type, compact=True)
+    book = torch.from_numpy(general.CODE_BOOKS[quant_type][:15].copy()).to(hip_device)
+    scale = x.view(-1, g).abs().amax(dim=1, keepdim=True)
+    t = (x.view(-1, g) / scale)
+    nearest = (t.unsqueeze(-1) - book).abs().amin(dim=-1)
+    achieved = (out.view(-1, g) / scale - t).abs()
+    assert bool((achieved <= nearest + 1e-6).all())
