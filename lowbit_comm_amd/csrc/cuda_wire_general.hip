@@ -52,41 +52,6 @@ template <typename T> __device__ __forceinline__ uint32_t raw_from(float v) {
     return __builtin_bit_cast(typename raw_bits<T>::type, narrow<T>(v));
 }
 
-template <int CTRL> __device__ __forceinline__ uint32_t dpp_other(uint32_t v) {
-    return static_cast<uint32_t>(
-        __builtin_amdgcn_update_dpp(static_cast<int>(v), static_cast<int>(v), CTRL, 0xF, 0xF, false));
-}
-template <int CTRL> __device__ __forceinline__ uint64_t dpp_other(uint64_t v) {
-    const uint64_t lo = dpp_other<CTRL>(static_cast<uint32_t>(v));
-    const uint64_t hi = dpp_other<CTRL>(static_cast<uint32_t>(v >> 32));
-    return lo | (hi << 32);
-}
-
-// The three largest keys seen so far, a >= b >= c; 0 stands for "none".
-template <typename K> struct top3 {
-    K a, b, c;
-    __device__ __forceinline__ void insert(K k) {
-        K lo = a < k ? a : k;
-        a = a < k ? k : a;
-        k = lo;
-        lo = b < k ? b : k;
-        b = b < k ? k : b;
-        c = c < lo ? lo : c;
-    }
-    template <int CTRL> __device__ __forceinline__ void merge_with_partner() {
-        const K oa = dpp_other<CTRL>(a), ob = dpp_other<CTRL>(b), oc = dpp_other<CTRL>(c);
-        insert(oa);
-        insert(ob);
-        insert(oc);
-    }
-    template <int LANES> __device__ __forceinline__ void merge_group() {
-        if constexpr (LANES >= 2) merge_with_partner<0xB1>();    // quad_perm [1,0,3,2]
-        if constexpr (LANES >= 4) merge_with_partner<0x4E>();    // quad_perm [2,3,0,1]
-        if constexpr (LANES >= 8) merge_with_partner<0x141>();   // row_half_mirror
-        if constexpr (LANES >= 16) merge_with_partner<0x140>();  // row_mirror
-    }
-};
-
 // Philox4x32-10: one block of four 32-bit words.
 __device__ __forceinline__ void philox_block(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
                                              uint32_t (&out)[4]) {
@@ -96,13 +61,12 @@ __device__ __forceinline__ void philox_block(uint32_t c0, uint32_t c1, uint32_t 
             k0 += 0x9E3779B9u;
             k1 += 0xBB67AE85u;
         }
-        const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
-        const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+        const uint64_t p0 = static_cast<uint64_t>(0xD2511F53u) * c0, p1 = static_cast<uint64_t>(0xCD9E8D57u) * c2;
+        const uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c1 ^ k0, n2 = static_cast<uint32_t>(p0 >> 32) ^ c3 ^ k1;
         c0 = n0;
-        c1 = lo1;
+        c1 = static_cast<uint32_t>(p1);
         c2 = n2;
-        c3 = lo0;
+        c3 = static_cast<uint32_t>(p0);
     }
     out[0] = c0;
     out[1] = c1;
@@ -113,6 +77,20 @@ __device__ __forceinline__ void philox_block(uint32_t c0, uint32_t c1, uint32_t 
 template <typename T, int G> __device__ __forceinline__ int scan_start(int64_t group) {
     if constexpr (sizeof(T) == 4) return 0;
     else return 4 * static_cast<int>((group & 31) / (32 / (G / 4)));
+}
+
+// Each wavefront keeps its own copy of the code book in LDS: written and read by the same wavefront, whose LDS
+// operations execute in order, so no workgroup barrier stands between the first loads and the arithmetic.
+__device__ __forceinline__ const float *wave_code_book(int kind, int lane) {
+    __shared__ float books[kWavesPerBlock][16];
+    float *book = books[threadIdx.x >> 6];
+    if (kind != 0) {
+        if (lane < 16) book[lane] = kCodeBooks[kind - 1][lane];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    return book;
 }
 
 __device__ __forceinline__ int meta_words_of(int topk) { return topk == 0 ? 1 : topk + 2; }
@@ -129,13 +107,9 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     constexpr bool WIDE = ITEM == 4;
     static_assert(LPG >= 2 && LPG <= 16, "a group must span 2..16 lanes of one DPP row");
 
-    __shared__ float book[16];
-    if (a.kind != 0) {   // uniform over the grid
-        if (threadIdx.x < 16) book[threadIdx.x] = kCodeBooks[a.kind - 1][threadIdx.x];
-        __syncthreads();
-    }
-
     const int lane = threadIdx.x & (kWave - 1);
+    const int meta_bytes = meta_words_of(a.topk) * ITEM;
+    const int64_t groups = a.numel / G;
     const int64_t tile_first = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * W::TILE;
     if (tile_first >= a.numel) return;   // wavefront-uniform
     const int64_t e0 = tile_first + lane * VEC;
@@ -148,6 +122,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
 #pragma unroll
     for (int i = 0; i < VEC; ++i) raw[i] = 0;
     if (live) load_elems<Raw, VEC, kPlain>(static_cast<const Raw *>(a.x) + e0, raw);
+    const float *book = wave_code_book(a.kind, lane);   // after the loads were issued: its wait covers theirs
     float v[VEC];
     uint32_t mag[VEC];
 #pragma unroll
@@ -156,8 +131,6 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
         mag[i] = raw[i] & RB::ABS;
     }
 
-    const int meta_bytes = meta_words_of(a.topk) * ITEM;
-    const int64_t groups = a.numel / G;
     uint8_t *group_codes = a.payload + (a.compact ? group * (CB + meta_bytes) : group * CB);
     uint8_t *group_meta = a.compact ? group_codes + CB : a.payload + groups * CB + group * meta_bytes;
 
@@ -190,32 +163,60 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
         }
         scale_raw = group_max_bits<LPG>(m);
     } else {
-        using K = typename pick_t<WIDE, uint64_t, uint32_t>::type;
-        top3<K> best{0, 0, 0};
+        // Three rounds of "largest remaining candidate": the group maximum of the magnitude keys, then, among
+        // the elements that hold it, the maximum of the tie-break ranks (1..G, unique inside a group).
+        // A 16-bit magnitude and its rank share one 32-bit key, so a round is a single reduction there.
+        uint32_t key[VEC], rank[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const int pos = (k0 + i - start) & (G - 1);
             const bool candidate = WIDE ? mag[i] <= RB::INF : (mag[i] != 0 && mag[i] <= RB::INF);
-            const K rank = static_cast<K>(WIDE ? k0 + i + 1 : G - pos);   // 1..G, larger wins a tie
-            best.insert(candidate ? ((static_cast<K>(mag[i]) << 8) | rank) : K(0));
+            rank[i] = static_cast<uint32_t>(WIDE ? k0 + i + 1 : G - pos);     // the larger rank wins a tie
+            const uint32_t joined = WIDE ? mag[i] : ((mag[i] << 7) | (rank[i] - 1));
+            key[i] = candidate ? joined + 1 : 0;                              // 0 stands for "none"
         }
-        best.template merge_group<LPG>();
-        auto index_of = [&](K key) {
-            const int rank = static_cast<int>(key & 0xFF);
-            return WIDE ? rank - 1 : ((G - rank) + start) & (G - 1);
+        uint32_t best_key[3] = {0, 0, 0}, best_rank[2] = {0, 0};              // magnitude + 1, rank
+#pragma unroll
+        for (int round = 0; round < 3; ++round) {
+            if (round == 2 && a.topk == 1) break;                             // uniform
+            uint32_t m = 0;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) m = key[i] > m ? key[i] : m;
+            m = group_max_bits<LPG>(m);
+            if constexpr (WIDE) {
+                best_key[round] = m;
+                if (round == 2) break;
+                uint32_t r = 0;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) r = (key[i] == m && rank[i] > r) ? rank[i] : r;
+                r = group_max_bits<LPG>(r);
+                r = m == 0 ? 0 : r;
+                best_rank[round] = r;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) key[i] = (key[i] == m && rank[i] == r) ? 0 : key[i];   // taken
+            } else {
+                best_key[round] = m == 0 ? 0 : ((m - 1) >> 7) + 1;
+                if (round == 2) break;
+                best_rank[round] = m == 0 ? 0 : ((m - 1) & 0x7Fu) + 1;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) key[i] = (key[i] == m && m != 0) ? 0 : key[i];          // taken
+            }
+        }
+        auto index_of = [&](uint32_t r) {
+            return WIDE ? static_cast<int>(r) - 1 : ((G - static_cast<int>(r)) + start) & (G - 1);
         };
-        const bool none = best.a == 0;
-        const int index1 = none ? 0 : index_of(best.a);
+        const bool none = best_key[0] == 0;
+        const int index1 = none ? 0 : index_of(best_rank[0]);
         int index2 = -1;
         if (a.topk == 1) {
             // nothing comparable: the reference falls back to element 1 (as stored for fp32, its magnitude otherwise)
             const uint32_t element1 = WIDE ? static_cast<uint32_t>(raw[1]) : mag[1];
             const uint32_t fallback = static_cast<uint32_t>(__shfl(static_cast<int>(element1), lane & ~(LPG - 1)));
-            scale_raw = none ? fallback : static_cast<uint32_t>(best.b >> 8);
+            scale_raw = none ? fallback : (best_key[1] == 0 ? 0u : best_key[1] - 1);
         } else {
-            const bool lonely = !none && best.b == 0;
-            index2 = none ? 1 : (lonely ? ((index1 + 1) & (G - 1)) : index_of(best.b));
-            scale_raw = (none || lonely) ? 0u : static_cast<uint32_t>(best.c >> 8);
+            const bool lonely = !none && best_key[1] == 0;
+            index2 = none ? 1 : (lonely ? ((index1 + 1) & (G - 1)) : index_of(best_rank[1]));
+            scale_raw = (none || lonely || best_key[2] == 0) ? 0u : best_key[2] - 1;
         }
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
@@ -277,7 +278,8 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
 #pragma unroll
             for (int step = 8; step >= 1; step >>= 1) {
                 const int mid = lower + step;
-                if (mid < 15 && !(t < book[mid])) lower = mid;
+                const float entry = book[mid];
+                if (mid < 15 && !(t < entry)) lower = mid;
             }
             const float low = book[lower], gap = book[lower + 1] - low, excess = t - low;
             const bool up = a.stochastic ? uniform[i] < excess / gap : excess > gap * 0.5f;
@@ -300,24 +302,22 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
     using Raw = typename raw_bits<T>::type;
     constexpr int VEC = W::VEC, ITEM = sizeof(T), CB = G * BIT / 8;
 
-    __shared__ float book[16];
-    if (a.kind != 0) {
-        if (threadIdx.x < 16) book[threadIdx.x] = kCodeBooks[a.kind - 1][threadIdx.x];
-        __syncthreads();
-    }
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t e0 = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * W::TILE + lane * VEC;
-    if (e0 >= a.numel) return;
-    const int64_t group = e0 / G;
-    const int k0 = static_cast<int>(e0 - group * G);
     const int meta_bytes = meta_words_of(a.topk) * ITEM;
     const int64_t groups = a.numel / G;
+    const int64_t tile_first = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * W::TILE;
+    if (tile_first >= a.numel) return;   // wavefront-uniform
+    const int64_t e0 = tile_first + lane * VEC;
+    const bool live = e0 < a.numel;      // dead lanes read group 0 and store nothing
+    const int64_t group = live ? e0 / G : 0;
+    const int k0 = live ? static_cast<int>(e0 - group * G) : 0;
     const uint8_t *group_codes = a.payload + (a.compact ? group * (CB + meta_bytes) : group * CB);
     const uint8_t *group_meta = a.compact ? group_codes + CB : a.payload + groups * CB + group * meta_bytes;
 
     uint32_t words[W::WORDS];
     load_piece<T, BIT, kPlain, W::WORDS>(group_codes + piece_offset<T, BIT>(k0), words);
     const float scale = value_of<T>(*reinterpret_cast<const Raw *>(group_meta));
+    const float *book = wave_code_book(a.kind, lane);   // after the loads were issued: its wait covers theirs
     const float step = a.kind == 0 ? step_of<BIT>(scale) : scale;
 
     Raw decoded[VEC];
@@ -344,6 +344,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
             if (k0 + i == index2) decoded[i] = top2;   // written second, as in the reference
         }
     }
+    if (!live) return;
     Raw *out = static_cast<Raw *>(a.out) + e0;
     if (a.op != 0) {
         Raw old[VEC];
