@@ -48,6 +48,10 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
     const int64_t groups = (a.shard_numel + G - 1) / G;
     const int64_t padded = groups * G;
     const group_layout<T, G, COMPACT, BIT> at{groups};
+    // The reference sends a chunk of whole groups without a residual to its general kernels, whose running
+    // maximum a NaN resets, and everything else to the fused pack kernel, whose fmaxf skips NaNs
+    // (quant_pack_kernel.cu:231,259-262).
+    const bool resets = !HAS_R && a.nan_resets != 0 && valid % G == 0;
 
     const T *__restrict__ x = static_cast<const T *>(a.x) + chunk_start;
     const T *__restrict__ r = HAS_R ? static_cast<const T *>(a.residual) + chunk_start : nullptr;
@@ -56,10 +60,26 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
     const int64_t block_first = static_cast<int64_t>(blockIdx.x) * BLOCK_ELEMS;
     if (block_first >= padded) return;
 
-    auto group_multiplier = [](uint32_t absmax_bits, float &absmax) {
-        absmax = as_f32(group_max_bits<LPG>(absmax_bits));
-        const float scale = absmax < 1.0e-6f ? 1.0e-6f : absmax;
+    using Raw = typename raw_bits<T>::type;
+    auto multiplier_of = [&](float absmax) {
+        const float scale = absmax < 1.0e-6f ? 1.0e-6f : absmax;   // a NaN stays and zeroes every code
         return W::LEVELS / scale;
+    };
+    auto group_multiplier = [&](uint32_t absmax_bits, float &absmax) {
+        absmax = as_f32(group_max_bits<LPG>(absmax_bits));
+        return multiplier_of(absmax);
+    };
+    // The scale of the lane's group as the reference's general kernels compute it, from the elements as stored.
+    auto scan_scale = [&](const T (&elements)[VEC], int64_t group, int k0) {
+        uint32_t mag[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) mag[i] = __builtin_bit_cast(Raw, elements[i]) & raw_bits<T>::ABS;
+        return running_max_raw<T, G, VEC>(mag, k0, scan_start<T, G>(group));
+    };
+    auto clamp_codes = [&](int (&c)[VEC]) {
+        constexpr int L = static_cast<int>(W::LEVELS);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) c[i] = c[i] < -L ? -L : (c[i] > L ? L : c[i]);
     };
 
     if (block_first + BLOCK_ELEMS <= valid) {
@@ -76,26 +96,39 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
         for (int u = 0; u < UNROLL; ++u) {
             float p[VEC];
             uint32_t m = 0;
+            bool has_nan = false;
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
                 float v = widen(xv[u][i]);
                 if constexpr (HAS_R) v = round_through<T>(v + widen(rv[u][i]));
                 p[i] = v;
                 uint32_t bits = as_u32(v) & 0x7FFFFFFFu;
+                has_nan |= bits > 0x7F800000u;
                 bits = bits > 0x7F800000u ? 0u : bits;   // fmaxf skips NaN
                 m = bits > m ? bits : m;
             }
+            const int64_t group = e0[u] / G;
+            const int k0 = static_cast<int>(e0[u] - group * G);
             float absmax;
-            const float multiplier = group_multiplier(m, absmax);
+            float multiplier = group_multiplier(m, absmax);
+            Raw stored = __builtin_bit_cast(Raw, narrow<T>(absmax));
+            bool wide_codes = false;   // wavefront-uniform: codes may leave [-LEVELS, LEVELS]
+            if constexpr (!HAS_R) {
+                if (resets && __ballot(has_nan) != 0) {
+                    const uint32_t scale_raw = scan_scale(xv[u], group, k0);
+                    multiplier = multiplier_of(value_of<T>(scale_raw));
+                    stored = static_cast<Raw>(scale_raw);
+                    wide_codes = true;
+                }
+            }
             int c[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) c[i] = cvt_i32(__builtin_rintf(p[i] * multiplier));
+            if (wide_codes) clamp_codes(c);
             uint32_t words[W::WORDS];
             pack_codes<T, BIT, VEC, W::WORDS>(c, words);
-            const int64_t group = e0[u] / G;
-            const int k0 = static_cast<int>(e0[u] - group * G);
             store_piece<T, BIT, PNT, W::WORDS>(payload + at.codes(group) + piece_offset<T, BIT>(k0), words);
-            if ((lane & (LPG - 1)) == 0) *reinterpret_cast<T *>(payload + at.scale(group)) = narrow<T>(absmax);
+            if ((lane & (LPG - 1)) == 0) *reinterpret_cast<Raw *>(payload + at.scale(group)) = stored;
         }
         return;
     }
@@ -105,32 +138,48 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
         const int64_t e0 = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
         if (e0 - lane * VEC >= padded) break;  // wavefront-uniform
         float p[VEC];
+        T held[VEC];
         uint32_t m = 0;
+        bool has_nan = false;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const int64_t e = e0 + i;
             float v = 0.0f;
+            held[i] = narrow<T>(0.0f);
             if (e < valid) {
+                held[i] = x[e];
                 v = widen(x[e]);
                 if constexpr (HAS_R) v = round_through<T>(v + widen(r[e]));
             }
             p[i] = v;
             uint32_t bits = as_u32(v) & 0x7FFFFFFFu;
+            has_nan |= bits > 0x7F800000u;
             bits = bits > 0x7F800000u ? 0u : bits;
             m = bits > m ? bits : m;
         }
+        const int64_t group = e0 / G;
+        const int k0 = static_cast<int>(e0 - group * G);
         float absmax;
-        const float multiplier = group_multiplier(m, absmax);   // every lane of the row takes part
+        float multiplier = group_multiplier(m, absmax);   // every lane of the row takes part
+        Raw stored = __builtin_bit_cast(Raw, narrow<T>(absmax));
+        bool wide_codes = false;
+        if constexpr (!HAS_R) {
+            if (resets && __ballot(has_nan) != 0) {
+                const uint32_t scale_raw = scan_scale(held, group, k0);
+                multiplier = multiplier_of(value_of<T>(scale_raw));
+                stored = static_cast<Raw>(scale_raw);
+                wide_codes = true;
+            }
+        }
         if (e0 < padded) {   // the lane's VEC elements lie inside the padded range together: whole words again
-            const int64_t group = e0 / G;
-            const int k0 = static_cast<int>(e0 - group * G);
             int c[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) c[i] = cvt_i32(__builtin_rintf(p[i] * multiplier));
+            if (wide_codes) clamp_codes(c);
             uint32_t words[W::WORDS];
             pack_codes<T, BIT, VEC, W::WORDS>(c, words);
             store_piece<T, BIT, kPlain, W::WORDS>(payload + at.codes(group) + piece_offset<T, BIT>(k0), words);
-            if ((lane & (LPG - 1)) == 0) *reinterpret_cast<T *>(payload + at.scale(group)) = narrow<T>(absmax);
+            if ((lane & (LPG - 1)) == 0) *reinterpret_cast<Raw *>(payload + at.scale(group)) = stored;
         }
     }
 }

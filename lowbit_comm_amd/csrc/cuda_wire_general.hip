@@ -40,18 +40,6 @@ __constant__ float kCodeBooks[4][16] = {
      0.125f, 0.16666666666666666f, 0.25f, 0.3333333333333333f, 0.5f, 0.6666666666666666f, 1.0f, __builtin_inff()},
 };
 
-template <typename T> struct raw_bits;
-template <> struct raw_bits<float> { using type = uint32_t; static constexpr uint32_t ABS = 0x7FFFFFFFu, INF = 0x7F800000u; };
-template <> struct raw_bits<f16> { using type = uint16_t; static constexpr uint32_t ABS = 0x7FFFu, INF = 0x7C00u; };
-template <> struct raw_bits<bf16> { using type = uint16_t; static constexpr uint32_t ABS = 0x7FFFu, INF = 0x7F80u; };
-
-template <typename T> __device__ __forceinline__ float value_of(uint32_t raw) {
-    return widen(__builtin_bit_cast(T, static_cast<typename raw_bits<T>::type>(raw)));
-}
-template <typename T> __device__ __forceinline__ uint32_t raw_from(float v) {
-    return __builtin_bit_cast(typename raw_bits<T>::type, narrow<T>(v));
-}
-
 // Philox4x32-10: one block of four 32-bit words.
 __device__ __forceinline__ void philox_block(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
                                              uint32_t (&out)[4]) {
@@ -72,11 +60,6 @@ __device__ __forceinline__ void philox_block(uint32_t c0, uint32_t c1, uint32_t 
     out[1] = c1;
     out[2] = c2;
     out[3] = c3;
-}
-
-template <typename T, int G> __device__ __forceinline__ int scan_start(int64_t group) {
-    if constexpr (sizeof(T) == 4) return 0;
-    else return 4 * static_cast<int>((group & 31) / (32 / (G / 4)));
 }
 
 // Each wavefront keeps its own copy of the code book in LDS: written and read by the same wavefront, whose LDS
@@ -136,32 +119,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
 
     uint32_t scale_raw;
     if (a.topk == 0) {
-        // (m > a) ? m : a over the scan: the maximum of what follows the last NaN, the NaN itself when it is last.
-        uint32_t m = 0;
-        bool has_nan = false;
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            const bool nan = mag[i] > RB::INF;
-            has_nan |= nan;
-            m = (!nan && mag[i] > m) ? mag[i] : m;
-        }
-        if (__ballot(has_nan) != 0) {   // wavefront-uniform, rare
-            uint32_t last = 0;          // 1 + scan position of the group's last NaN
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                const uint32_t pos = static_cast<uint32_t>(k0 + i - start) & (G - 1);
-                if (mag[i] > RB::INF && pos + 1 > last) last = pos + 1;
-            }
-            last = group_max_bits<LPG>(last);
-            const uint32_t from = last == G ? G - 1 : last;
-            m = 0;
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                const uint32_t pos = static_cast<uint32_t>(k0 + i - start) & (G - 1);
-                if (pos >= from && mag[i] > m) m = mag[i];
-            }
-        }
-        scale_raw = group_max_bits<LPG>(m);
+        scale_raw = running_max_raw<T, G, VEC>(mag, k0, start);
     } else {
         // Three rounds of "largest remaining candidate": the group maximum of the magnitude keys, then, among
         // the elements that hold it, the maximum of the tie-break ranks (1..G, unique inside a group).

@@ -68,6 +68,8 @@ struct WireQuantArgs {
     int64_t shard_numel;     // elements per chunk (== numel for a single payload)
     int64_t payload_stride;  // bytes
     int compact;             // scales interleaved after each group's codes
+    int nan_resets;          // group maximum as the reference's general kernels take it (a NaN resets it); needs
+                             // residual == null and whole groups
 };
 
 struct WireReduceArgs {

@@ -354,6 +354,7 @@ int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, i
     a.shard_numel = shard;
     a.payload_stride = world > 1 ? payload_stride : 0;
     a.compact = compact != 0;
+    a.nan_resets = residual == nullptr;
     const int64_t moved = numel * (item * (residual ? 2 : 1) + 1);
     return finish(lbc::launch_wire_quant(dtype, group_size, bit, pick_mode(true, moved), a, world,
                                          static_cast<hipStream_t>(stream)),

@@ -188,4 +188,61 @@ template <typename T> __device__ __forceinline__ float add_rounded_once(float a,
     return round_through<T>(s);
 }
 
+// ---- elements as stored (bit patterns), for the kernels that must keep NaN payloads and compare magnitudes ----
+template <typename T> struct raw_bits;
+template <> struct raw_bits<float> { using type = uint32_t; static constexpr uint32_t ABS = 0x7FFFFFFFu, INF = 0x7F800000u; };
+template <> struct raw_bits<f16> { using type = uint16_t; static constexpr uint32_t ABS = 0x7FFFu, INF = 0x7C00u; };
+template <> struct raw_bits<bf16> { using type = uint16_t; static constexpr uint32_t ABS = 0x7FFFu, INF = 0x7F80u; };
+
+template <typename T> __device__ __forceinline__ float value_of(uint32_t raw) {
+    return widen(__builtin_bit_cast(T, static_cast<typename raw_bits<T>::type>(raw)));
+}
+template <typename T> __device__ __forceinline__ uint32_t raw_from(float v) {
+    return __builtin_bit_cast(typename raw_bits<T>::type, narrow<T>(v));
+}
+
+// First element of a group's scan in the reference's one-thread-per-group kernels: 0 for fp32 tensors,
+// rotated by shared-memory bank for 16-bit ones (quant_kernel.cuh:30-32).
+template <typename T, int G> __device__ __forceinline__ int scan_start(int64_t group) {
+    if constexpr (sizeof(T) == 4) return 0;
+    else return 4 * static_cast<int>((group & 31) / (32 / (G / 4)));
+}
+
+
+// The reference's general kernels take a group's maximum as a running `(m > a) ? m : a` over the group's
+// scan (utils.cuh:11-14, quant_kernel_fp32.cuh:93-97, quant_kernel.cuh:33-38): a NaN replaces the maximum and
+// the next element replaces the NaN, so the result is the maximum of what follows the group's last NaN, or that
+// NaN when it ends the scan.  `mag` are the magnitude bits of the lane's elements as stored, `k0` the lane's
+// first element inside its group, `start` the element the scan begins at.  Returns the scale as stored.
+template <typename T, int G, int VEC>
+__device__ __forceinline__ uint32_t running_max_raw(const uint32_t (&mag)[VEC], int k0, int start) {
+    constexpr int LPG = G / VEC;
+    using RB = raw_bits<T>;
+    uint32_t m = 0;
+    bool has_nan = false;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        const bool nan = mag[i] > RB::INF;
+        has_nan |= nan;
+        m = (!nan && mag[i] > m) ? mag[i] : m;
+    }
+    if (__ballot(has_nan) != 0) {   // wavefront-uniform, rare
+        uint32_t last = 0;          // 1 + scan position of the group's last NaN
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const uint32_t pos = static_cast<uint32_t>(k0 + i - start) & (G - 1);
+            if (mag[i] > RB::INF && pos + 1 > last) last = pos + 1;
+        }
+        last = group_max_bits<LPG>(last);
+        const uint32_t from = last == G ? G - 1 : last;
+        m = 0;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const uint32_t pos = static_cast<uint32_t>(k0 + i - start) & (G - 1);
+            if (pos >= from && mag[i] > m) m = mag[i];
+        }
+    }
+    return group_max_bits<LPG>(m);
+}
+
 }  // namespace lbc

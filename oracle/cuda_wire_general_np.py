@@ -266,6 +266,19 @@ def quantize(x: np.ndarray, dtype: str, group_size: int = 64, bit: int = 8, quan
     return np.concatenate([code_bytes.reshape(-1), meta_bytes.reshape(-1)])
 
 
+def quantize_pack(x: np.ndarray, dtype: str, group_size: int = 64, compact: bool = True,
+                  residual: np.ndarray | None = None, bit: int = 8) -> np.ndarray:
+    """What ``inplace_quantize_pack`` writes for a plain linear policy (quant_pack_kernel.cu:231,259-275): whole
+    groups without a residual go to the general kernels (running maximum, a NaN resets it), everything else to
+    the fused pack kernel (``fmaxf``, NaNs skipped).  The two differ only on groups that hold a NaN."""
+    from .cuda_wire_np import quantize as pack_kernel
+
+    n = np.asarray(x).size
+    if residual is None and n % group_size == 0:
+        return quantize(x, dtype, group_size, bit, "linear", 0, None, compact)
+    return pack_kernel(x, dtype, group_size, compact, residual, bit)
+
+
 # ---------------------------------------------------------------------------------------------------------
 # dequantize
 # ---------------------------------------------------------------------------------------------------------

@@ -89,6 +89,42 @@ def test_plain_policy_equals_the_pack_kernel_on_finite_input(hip, hip_device, na
                            b.view(torch.int16 if name != "fp32" else torch.int32))
 
 
+@pytest.mark.parametrize("name", list(NAMES))
+@pytest.mark.parametrize("g", (16, 64))
+def test_pack_entry_point_takes_the_maximum_as_the_reference_dispatch_does(hip, hip_device, name, g):
+    """Whole groups without a residual: a NaN resets the running maximum (general kernels); with a residual or a
+    ragged tail: NaNs are skipped (fused pack kernel).  Interior blocks and the edge block both see NaNs."""
+    rng = np.random.default_rng(g)
+    n = g * 3000
+    values = awkward_values(rng, n, g, 0)
+    values[rng.integers(0, n, 400)] = np.nan
+    values[n - 3] = np.nan
+    x_np = wire.from_f32(values, name)
+    x = from_numpy(x_np, name, hip_device)
+    r_np = wire.from_f32((rng.standard_normal(n) * 1e-3).astype(np.float32), name)
+    r = from_numpy(r_np, name, hip_device)
+    for bit, compact in itertools.product((8, 4), (True, False)):
+        same(hip.quant_pack(x, group_size=g, compact=compact, bit=bit),
+             general.quantize_pack(x_np, name, g, compact, None, bit), f"whole groups {bit} {compact}")
+        assert not np.array_equal(general.quantize_pack(x_np, name, g, compact, None, bit),
+                                  wire.quantize(x_np, name, g, compact, None, bit))
+        same(hip.quant_pack(x, group_size=g, compact=compact, bit=bit, residual=r),
+             wire.quantize(x_np, name, g, compact, r_np, bit), f"residual {bit} {compact}")
+        same(hip.quant_pack(x[:n - 5], group_size=g, compact=compact, bit=bit),
+             wire.quantize(x_np[:n - 5], name, g, compact, None, bit), f"ragged {bit} {compact}")
+    # chunks: a chunk of whole groups follows the general kernels, the ragged last chunk the pack kernel
+    world, total = 4, g * 1000 - 3
+    shard = -(-total // world)
+    assert shard == g * 250
+    stride = hip.payload_nbytes(shard, x.dtype, g) + 8
+    rows = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+    assert hip.bind_quant_pack_chunks(x[:total], rows, world, group_size=g)()
+    for d in range(world):
+        piece = x_np[d * shard:min(total, (d + 1) * shard)]
+        want = general.quantize_pack(piece, name, g, True, None, 8)
+        same(rows[d, :want.size], want, f"chunk {d}")
+
+
 def test_contract_violations(hip, hip_device):
     x = torch.zeros(64 * 3, device=hip_device)
     payload = torch.empty(hip.general_payload_nbytes(x.numel(), x.dtype, 64, 8, 1), dtype=torch.uint8, device=hip_device)
