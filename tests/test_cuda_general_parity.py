@@ -141,6 +141,76 @@ def test_contract_violations(hip, hip_device):
 
 
 # --------------------------------------------------------------------------- #
+# the extension module and the codec facade
+# --------------------------------------------------------------------------- #
+@pytest.fixture(scope="module")
+def wire_status(hip_device):
+    from lowbit_comm_amd.hip.loader import load_hip_extension
+
+    status = load_hip_extension(wire_format="native")
+    assert status.available, status.reason
+    return status
+
+
+@pytest.mark.parametrize("name", list(NAMES))
+def test_module_runs_every_policy(wire_status, hip_device, name):
+    module = wire_status.module
+    kinds = {"linear": module.QuantType.Linear, "normal": module.QuantType.Normal, "uniform": module.QuantType.Uniform,
+             "e3m0": module.QuantType.E3M0, "e2m1": module.QuantType.E2M1}
+    dtype_member = {"fp32": module.DType.FP32, "fp16": module.DType.FP16, "bf16": module.DType.BF16}[name]
+    rng = np.random.default_rng(17)
+    n, g = 64 * 300, 64
+    x_np = wire.from_f32(awkward_values(rng, n, g, 0), name)
+    x = from_numpy(x_np, name, hip_device)
+    for bit, quant_type, topk, stochastic in policies():
+        for compact in (False, True):
+            seeds = None
+            if stochastic is not None:
+                torch.cuda.manual_seed(stochastic[0])
+                generator = torch.cuda.default_generators[hip_device.index or 0]
+                generator.set_offset(4 * stochastic[1])
+                seeds = (stochastic[0], 4 * stochastic[1])
+            payload = module.quantize(x, g, topk, stochastic is not None, bit, kinds[quant_type], compact)
+            same(payload, general.quantize(x_np, name, g, bit, quant_type, topk, seeds, compact),
+                 f"{bit} {quant_type} {topk} {stochastic} {compact}")
+            if seeds is not None:       # the generator moved on by numel draws, as philox_engine_inputs does
+                assert torch.cuda.default_generators[hip_device.index or 0].get_offset() == seeds[1] + n
+            out = module.dequantize(payload, g, topk, bit, module.ReduceOP.NONE, kinds[quant_type], dtype_member, compact)
+            same(out, general.dequantize(to_numpy(payload), n, name, g, bit, quant_type, topk, compact))
+            if topk or quant_type != "linear":
+                assert module.inplace_quantize_pack(x, payload, None, g, topk, False, bit, kinds[quant_type], True) is False
+    # the decode-and-add chain of two payloads with outliers
+    pair = [module.quantize(x, g, 2, False, 8, kinds["linear"], True) for _ in range(2)]
+    total = module.dequantize_reduce(pair, g, 2, 8, kinds["linear"], dtype_member, True)
+    once = general.dequantize(to_numpy(pair[0]), n, name, g, 8, "linear", 2, True)
+    same(total, general.dequantize(to_numpy(pair[1]), n, name, g, 8, "linear", 2, True, "sum", once))
+    with pytest.raises(RuntimeError, match="multiple of group_size"):
+        module.quantize(x[:100], g, 1, False, 8, kinds["linear"], True)
+    with pytest.raises(RuntimeError, match="supports group_size"):
+        module.quantize(x, g, 0, False, 8, kinds["normal"], True)
+
+
+def test_facade_round_trip_with_outliers_and_code_book(wire_status, hip_device):
+    from lowbit_comm_amd.config import CompressionConfig
+    from lowbit_comm_amd.quantization import codec
+
+    gen = torch.Generator(device=hip_device).manual_seed(8)
+    x = torch.randn(64 * 500, generator=gen, device=hip_device, dtype=torch.float16)
+    x[::97] *= 40
+    for config in (CompressionConfig(topk=2), CompressionConfig(topk=1, compact=True),
+                   CompressionConfig(bit=4, quant_type="normal", allow_experimental=True),
+                   CompressionConfig(bit=4, quant_type="e2m1", topk=2, compact=True, allow_experimental=True)):
+        payload = codec.quantize_tensor(x, config, extension_status=wire_status)
+        restored = codec.dequantize_tensor(payload, tuple(x.shape), config, dtype="fp16", extension_status=wire_status)
+        kind = config.quant_type
+        want_bytes = general.quantize(to_numpy(x), "fp16", 64, config.bit, kind, config.topk, None, config.compact)
+        buffer = payload.buffer if hasattr(payload, "buffer") else payload
+        same(buffer, want_bytes, str(config))
+        same(restored.reshape(-1), general.dequantize(want_bytes, x.numel(), "fp16", 64, config.bit, kind, config.topk,
+                                                      config.compact), str(config))
+
+
+# --------------------------------------------------------------------------- #
 # the 100 MiB bucket: properties that need no oracle pass over the whole tensor
 # --------------------------------------------------------------------------- #
 FULL = 26_214_400

@@ -354,7 +354,7 @@ def test_module_error_feedback_paths(wire_status, hip_device):
         module.inplace_dequantize_reduce_mean_update_error_feedback(payloads, prepared, restored, residual, 64, 0, 8,
                                                                     linear, True, 0)
     with pytest.raises(RuntimeError):
-        module.quantize(prepared, 64, 2, False, 8, linear, True)          # top-k side channels have no kernel
+        module.quantize(prepared, 64, 2, False, 8, linear, True)          # the general policies need whole groups
     assert module.inplace_quantize_pack(prepared, payloads[0], None, 64, 1, False, 8, linear, True) is False
 
 
