@@ -489,6 +489,41 @@ def main() -> int:
             emit(6, f"4-bit decode 26.2M {name}, interleaved scales", n * item + p4,
                  timed(lambda i: decode[i % 4](), args.iters), p4, check)
             del xs, outs, back, quant, decode
+            # the extension's other policies (general kernels): top-k side channel, stochastic rounding, code books
+            if parity:
+                from oracle import cuda_wire_general_scalar as general_c
+            xs = [gen(SEED + 1100 + s, n, 1e-3, dtype) for s in range(4)]
+            back = [torch.empty(n, dtype=dtype, device=dev) for _ in range(4)]
+            for label, policy, seeds in (
+                    ("top-2 outliers, 8-bit linear", dict(bit=8, quant_type="linear", topk=2), None),
+                    ("stochastic rounding, 8-bit linear", dict(bit=8, quant_type="linear", topk=0), (SEED, 0)),
+                    ("4-bit normal code book", dict(bit=4, quant_type="normal", topk=0), None)):
+                pb = cuda_wire.general_payload_nbytes(n, dtype, 64, policy["bit"], policy["topk"])
+                outs = [torch.empty(pb, dtype=torch.uint8, device=dev) for _ in range(4)]
+                quant = [cuda_wire.bind_quant_general(xs[s], outs[s], compact=True, stochastic=seeds, **policy) for s in range(4)]
+                decode = [cuda_wire.bind_dequant_general(outs[s], back[s], compact=True, **policy) for s in range(4)]
+                check = None
+                if parity:          # the scalar restatement on the first 1 Mi elements (group indices coincide there)
+                    m = 1 << 20
+                    part = torch.empty(cuda_wire.general_payload_nbytes(m, dtype, 64, policy["bit"], policy["topk"]),
+                                       dtype=torch.uint8, device=dev)
+                    cuda_wire.quant_general_into(xs[0][:m], part, compact=True, stochastic=seeds, **policy)
+                    want = general_c.quantize(host(xs[0][:m]), name, 64, policy["bit"], policy["quant_type"],
+                                              policy["topk"], seeds, True)
+                    ok = host(part).tobytes() == want.tobytes()
+                    got = torch.empty(m, dtype=dtype, device=dev)
+                    cuda_wire.dequant_general_into(part, got, compact=True, **policy)
+                    ok = ok and host(got).tobytes() == general_c.dequantize(
+                        want, m, name, 64, policy["bit"], policy["quant_type"], policy["topk"], True).tobytes()
+                    check = "bit-exact (first 1Mi elements)" if ok else "MISMATCH"
+                for s in range(4):
+                    quant[s]()
+                emit(6, f"quantize, {label}, 26.2M {name}", n * item + pb, timed(lambda i: quant[i % 4](), args.iters),
+                     n * item, check)
+                emit(6, f"decode, {label}, 26.2M {name}", n * item + pb, timed(lambda i: decode[i % 4](), args.iters),
+                     pb, check)
+                del outs, quant, decode
+            del xs, back
 
     print(f"\n{'cfg':>3} {'us':>10} {'GB/s alg.':>10} {'% of 8TB/s':>10} {'input GB/s':>10}  parity / op", file=sys.stderr)
     for r in rows_out:
