@@ -25,7 +25,8 @@ they add:
 Everything is vectorised over groups and walks the g scan positions in a Python loop, so the running
 comparisons are literally the reference's.  ``cuda_wire_general_scalar.c`` restates the same kernels one
 group at a time; the tests hold the two against each other, against exact rational arithmetic, against
-the Philox known-answer vectors of the Random123 distribution and against closed forms of the code books.
+the Philox known-answer vectors of the Random123 distribution and against closed forms of the code books; a GPU
+test holds ``curand_draws`` against rocRAND's Philox device generator (documented to reproduce cuRAND's sequence).
 
 Parity with an actual NVIDIA build is unpinned (the reference holds no payload bytes for these policies):
 in particular whether nvcc contracts ``v * m + noise`` into one FMA (its default, restated here).

@@ -140,6 +140,49 @@ def test_contract_violations(hip, hip_device):
     assert hip.quant_general_into(empty, torch.empty(0, dtype=torch.uint8, device=hip_device), topk=2)
 
 
+def test_philox_stream_matches_the_platform_library(hip, hip_device):
+    """rocRAND's Philox4x32-10 device generator yields cuRAND's sequence for a (seed, subsequence, offset); the
+    oracle's counter-mode stream, which the quantize kernel was checked against above, must yield the same words,
+    and so must the stochastic codes of a payload rebuilt from the library's draws."""
+    import ctypes
+    from pathlib import Path
+
+    path = Path(__file__).resolve().parent / "native" / "_build" / "librocrand_draws.so"
+    assert path.exists(), "run __graft_entry__.build() first: it compiles tests/native/rocrand_draws.hip"
+    helper = ctypes.CDLL(str(path))
+    helper.rocrand_philox_draws.restype = ctypes.c_int
+    helper.rocrand_philox_draws.argtypes = [ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64, ctypes.c_int,
+                                            ctypes.c_void_p, ctypes.c_void_p]
+    subsequences = np.array([0, 1, 2, 77, 2 ** 20 + 3, 2 ** 32 + 5, 2 ** 40], dtype=np.uint64)
+    device_subsequences = torch.from_numpy(subsequences.view(np.int64)).to(hip_device)
+    for seed, offset in ((0, 0), (42, 8), (7, 3), (0x0123456789ABCDEF, 2 ** 33 + 1), (2 ** 63 + 11, 6)):
+        out = torch.zeros(len(subsequences) * 70, dtype=torch.int32, device=hip_device)
+        stream = torch.cuda.current_stream(hip_device).cuda_stream
+        assert helper.rocrand_philox_draws(seed, device_subsequences.data_ptr(), len(subsequences), offset, 70,
+                                           out.data_ptr(), stream) == 0
+        torch.cuda.synchronize()
+        library = out.cpu().numpy().view(np.uint32).reshape(len(subsequences), 70)
+        assert np.array_equal(library, general.curand_draws(seed, subsequences, offset, 70)), (seed, offset)
+    # end to end: the codes of group s are rint(fma(v, m, u - 0.5)) with u from the library's draws of subsequence s
+    g, groups, seed, offset = 64, 96, 1234, 12
+    x = torch.randn(g * groups, generator=torch.Generator(device=hip_device).manual_seed(1), device=hip_device)
+    payload = torch.empty(hip.general_payload_nbytes(x.numel(), x.dtype, g, 8, 0), dtype=torch.uint8, device=hip_device)
+    assert hip.quant_general_into(x, payload, group_size=g, stochastic=(seed, offset))
+    rows = torch.arange(groups, dtype=torch.int64, device=hip_device)
+    out = torch.zeros(groups * g, dtype=torch.int32, device=hip_device)
+    assert helper.rocrand_philox_draws(seed, rows.data_ptr(), groups, offset, g, out.data_ptr(),
+                                       torch.cuda.current_stream(hip_device).cuda_stream) == 0
+    torch.cuda.synchronize()
+    draws = out.cpu().numpy().view(np.uint32).reshape(groups, g)
+    uniform = general.curand_uniform(draws)
+    values = x.cpu().numpy().reshape(groups, g)
+    multiplier = (np.float64(127.0) / np.abs(values).max(axis=1).astype(np.float64)).astype(np.float32)[:, None]
+    noise = (uniform.astype(np.float64) - 0.5).astype(np.float32)
+    want = np.clip(np.rint(wire.fma_f32(values, np.broadcast_to(multiplier, values.shape), noise)), -127, 127)
+    codes, _ = general.split(to_numpy(payload), x.numel(), "fp32", g, 8, 0, False)
+    assert np.array_equal(codes, want.astype(np.int8))
+
+
 # --------------------------------------------------------------------------- #
 # the extension module and the codec facade
 # --------------------------------------------------------------------------- #
