@@ -50,6 +50,12 @@ def payload_addresses(payload: torch.Tensor, numel: int, group_size: int = 64, *
     costs a few microseconds of host time; the hot callers hand over up to nine payloads per bucket)."""
     groups = num_groups(numel, group_size)
     code_bytes = groups * group_size
+    # one combined test on the hot path; the separate tests below only run to name what is wrong
+    if (isinstance(payload, torch.Tensor) and payload.dtype is torch.uint8 and payload.is_cuda
+            and payload.numel() == code_bytes + 4 * groups and payload.is_contiguous()
+            and (device is None or payload.device == device)):
+        base = payload.data_ptr()
+        return base, base + code_bytes
     if not isinstance(payload, torch.Tensor) or payload.dtype != torch.uint8:
         raise RuntimeError(f"{name} must be uint8")
     if not payload.is_cuda:
@@ -58,10 +64,7 @@ def payload_addresses(payload: torch.Tensor, numel: int, group_size: int = 64, *
         raise RuntimeError(f"{name} must be contiguous")
     if device is not None and payload.device != device:
         raise RuntimeError(f"{name} must be on {device}")
-    if payload.numel() != code_bytes + 4 * groups:
-        raise RuntimeError(f"{name} has an invalid quantized payload size")
-    base = payload.data_ptr()
-    return base, base + code_bytes
+    raise RuntimeError(f"{name} has an invalid quantized payload size")
 
 
 def promote(a: torch.dtype, b: torch.dtype) -> torch.dtype:
@@ -101,6 +104,17 @@ def _ptr(t: torch.Tensor | None):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
+_raw_stream_of = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def current_stream_handle(device: torch.device) -> int:
+    """Raw ``hipStream_t`` of torch's current stream on ``device`` (the direct binding when this torch has it: it
+    skips building a ``torch.cuda.Stream`` object, a few microseconds per launch)."""
+    if _raw_stream_of is not None:
+        return _raw_stream_of(device.index if device.index is not None else torch.cuda.current_device())
+    return torch.cuda.current_stream(device).cuda_stream
+
+
 class _Launch:
     """Device guard + current stream of ``device`` for one ABI call."""
 
@@ -111,7 +125,7 @@ class _Launch:
     def __enter__(self):
         if self._guard is not None:
             self._guard.__enter__()
-        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        return ctypes.c_void_p(current_stream_handle(self.device))
 
     def __exit__(self, *exc):
         if self._guard is not None:
@@ -144,7 +158,7 @@ class BoundLaunch:
             if self._device.index not in (None, torch.cuda.current_device()):
                 with _Launch(self._device) as guarded:
                     return _finish(self._fn(*self._args, guarded), self._lib)
-            stream = torch.cuda.current_stream(self._device).cuda_stream
+            stream = current_stream_handle(self._device)
         rc = self._fn(*self._args, stream)
         return True if rc == LBC_OK else _finish(rc, self._lib)
 
@@ -370,7 +384,10 @@ def bind_dequant_reduce(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], o
     scale_ptrs = (ctypes.c_void_p * world)()
     for r, entry in enumerate(payloads):
         if isinstance(entry, torch.Tensor):          # a packed uint8[codes || scales] payload
-            code_ptrs[r], scale_ptrs[r] = payload_addresses(entry, n, group_size, name=f"inputs[{r}]", device=device)
+            try:
+                code_ptrs[r], scale_ptrs[r] = payload_addresses(entry, n, group_size, name="inputs", device=device)
+            except RuntimeError as error:            # name the entry only when something is wrong with it
+                raise RuntimeError(str(error).replace("inputs", f"inputs[{r}]", 1)) from None
             continue
         codes, scales = entry
         _device_tensor(codes, f"codes[{r}]", device)
