@@ -205,6 +205,11 @@ int64_t lbc_wire_payload_nbytes(int64_t numel, int group_size, int dtype, int bi
  * Quantize x (+ residual, added in fp32 and rounded to dtype first) into one payload.
  * Replaces native inplace_quantize_pack and inplace_quantize for linear 8- and 4-bit codes
  * (quant_pack_kernel.cu:220-275, ccdl_comm/csrc/pybind.cpp:36-63).  Ragged numel is zero padded.
+ * NaN elements: the reference sends a call without a residual whose numel is a multiple of
+ * group_size to its general kernels, whose running group maximum `(m > a) ? m : a` a NaN resets
+ * (utils.cuh:11, quant_kernel_fp32.cuh:93-97), and every other call to its pack kernel, whose
+ * fmaxf skips NaNs (quant_pack_kernel.cu:259-262,94-99); this entry point makes the same choice
+ * per call (per chunk in the chunked form).
  */
 int lbc_wire_quant_pack(const void *x, const void *residual, int dtype, int64_t numel, int group_size,
                         int bit, int compact, uint8_t *payload, void *stream);
