@@ -480,6 +480,51 @@ def test_pool_reuses_buffers_across_streams_without_host_sync(dev):
     assert torch.cuda.memory_allocated() == before and pool.stats.misses == 1
 
 
+def test_bucket_stream_captured_in_a_hip_graph_replays_like_eager(dev):
+    """The per-bucket launches allocate nothing and clear nothing, so a pass over many buckets can be captured in
+    a HIP graph.  Four replays, with eager work and a synchronisation between them, must leave the same residuals,
+    payload bytes and reduced shard as four eager passes from the same state (the residual update is in place, so
+    every pass differs from the one before)."""
+    from lowbit_comm_amd.hip import ops
+
+    world, g, buckets, n = 8, 64, 6, 64 * 4096 + 64 * 8 * 5          # not a multiple of the block size
+    shard = n // world
+    stride = -(-ops.payload_nbytes(shard, g) // 256) * 256
+    grads = grad(buckets * n, torch.bfloat16, 1, dev)
+    start = grad(buckets * n, torch.float32, 2, dev, sigma=1e-5)
+    residuals = start.clone()
+    rows = torch.empty(world, stride, dtype=torch.uint8, device=dev)
+    peers = [ops.quant_pack(grad(shard, torch.float32, 10 + r, dev), group_size=g) for r in range(world)]
+    out = torch.empty(shard, device=dev)
+    launches = []
+    for i in range(buckets):
+        piece = slice(i * n, (i + 1) * n)
+        launches.append(ops.bind_quant_pack_chunks(grads[piece], rows, world, residual=residuals[piece],
+                                                   new_residual=residuals[piece]))
+        launches.append(ops.bind_dequant_reduce(peers, out, numel=shard))
+
+    def one_pass():
+        for launch in launches:
+            assert launch()
+
+    eager = []
+    for _ in range(4):
+        one_pass()
+        torch.cuda.synchronize()
+        eager.append((residuals.clone(), rows.clone(), out.clone()))
+    residuals.copy_(start)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+        one_pass()
+    torch.cuda.synchronize()
+    residuals.copy_(start)                                            # capture enqueued nothing
+    for want_residuals, want_rows, want_out in eager:
+        graph.replay()
+        torch.cuda.synchronize()
+        assert same_bits(residuals, want_residuals) and torch.equal(rows, want_rows) and same_bits(out, want_out)
+        assert float((torch.randn(1 << 16, device=dev) * 2).sum().item()) == pytest.approx(0.0, abs=1e4)   # eager work
+
+
 def test_llama_shaped_bucket_stream_through_the_pool(dev):
     """Config 5 structure at 1/64 scale: bf16 parameter tensors of a Llama-3-8B-shaped layer stack, flattened in
     reverse registration order into fixed-size buckets with a ragged tail; per bucket EF quant-pack and a W=8
