@@ -274,7 +274,20 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
 
     uint32_t words[W::WORDS];
     load_piece<T, BIT, kPlain, W::WORDS>(group_codes + piece_offset<T, BIT>(k0), words);
-    const float scale = value_of<T>(*reinterpret_cast<const Raw *>(group_meta));
+    // the group's metadata words [scale][indices][top1][top2], fetched together with the codes
+    Raw meta[4] = {0, 0, 0, 0};
+    if (a.topk == 2) {
+        load_elems<Raw, 4, kPlain>(reinterpret_cast<const Raw *>(group_meta), meta);
+    } else if (a.topk == 1) {
+        Raw pair[2];
+        load_elems<Raw, 2, kPlain>(reinterpret_cast<const Raw *>(group_meta), pair);
+        meta[0] = pair[0];
+        meta[1] = pair[1];
+        meta[2] = *reinterpret_cast<const Raw *>(group_meta + 2 * ITEM);
+    } else {
+        meta[0] = *reinterpret_cast<const Raw *>(group_meta);
+    }
+    const float scale = value_of<T>(meta[0]);
     const float *book = wave_code_book(a.kind, lane);   // after the loads were issued: its wait covers theirs
     const float step = a.kind == 0 ? step_of<BIT>(scale) : scale;
 
@@ -287,19 +300,13 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
         decoded[i] = static_cast<Raw>(raw_from<T>(value));
     }
     if (a.topk >= 1) {
-        const uint32_t indices = *reinterpret_cast<const Raw *>(group_meta + ITEM);
-        const Raw top1 = *reinterpret_cast<const Raw *>(group_meta + 2 * ITEM);
+        const uint32_t indices = meta[1];
         const int index1 = static_cast<int>(indices & 0xFFu);
-        int index2 = -1;
-        Raw top2 = 0;
-        if (a.topk == 2) {
-            index2 = static_cast<int>((indices >> 8) & 0xFFu);
-            top2 = *reinterpret_cast<const Raw *>(group_meta + 3 * ITEM);
-        }
+        const int index2 = a.topk == 2 ? static_cast<int>((indices >> 8) & 0xFFu) : -1;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
-            if (k0 + i == index1) decoded[i] = top1;
-            if (k0 + i == index2) decoded[i] = top2;   // written second, as in the reference
+            if (k0 + i == index1) decoded[i] = meta[2];
+            if (k0 + i == index2) decoded[i] = meta[3];   // written second, as in the reference
         }
     }
     if (!live) return;
