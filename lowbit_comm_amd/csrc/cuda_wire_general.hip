@@ -176,13 +176,19 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
             index2 = none ? 1 : (lonely ? ((index1 + 1) & (G - 1)) : index_of(best_rank[1]));
             scale_raw = (none || lonely || best_key[2] == 0) ? 0u : best_key[2] - 1;
         }
+        Raw top1_raw = 0, top2_raw = 0;
+        bool own1 = false, own2 = false;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const bool first = k0 + i == index1, second = k0 + i == index2;
-            if (live && first) *reinterpret_cast<Raw *>(group_meta + 2 * ITEM) = raw[i];
-            if (live && second) *reinterpret_cast<Raw *>(group_meta + 3 * ITEM) = raw[i];
+            top1_raw = first ? raw[i] : top1_raw;
+            top2_raw = second ? raw[i] : top2_raw;
+            own1 |= first;
+            own2 |= second;
             if (first || second) v[i] = 0.0f;
         }
+        if (live && own1) *reinterpret_cast<Raw *>(group_meta + 2 * ITEM) = top1_raw;   // the owner lanes store
+        if (live && own2) *reinterpret_cast<Raw *>(group_meta + 3 * ITEM) = top2_raw;   // the outliers as they are
         if (live && k0 == 0)
             *reinterpret_cast<Raw *>(group_meta + ITEM) =
                 static_cast<Raw>(a.topk == 1 ? index1 : (index1 | (index2 << 8)));
