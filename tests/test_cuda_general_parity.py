@@ -72,6 +72,41 @@ def test_quantize_and_decode_bytes(hip, hip_device, name, g, compact):
                  f"decode {op} " + what)
 
 
+def test_randomized_policies_sizes_and_contents(hip, hip_device):
+    """400 seeded draws over dtype, group, bit, code book, top-k, rounding seed, layout, size (1 to 30,000 groups)
+    and content (scales 1e-8..1e3, NaN/Inf, many ties, many zeros): quantize bytes and one decode op each."""
+    rng = np.random.default_rng(2718)
+    for case in range(400):
+        name = str(rng.choice(list(NAMES)))
+        g, bit, topk = int(rng.choice([16, 32, 64])), int(rng.choice([4, 8])), int(rng.choice([0, 1, 2]))
+        quant_type = "linear" if bit == 8 else str(rng.choice(general.QUANT_TYPES))
+        stochastic = None if rng.random() < 0.4 else (int(rng.integers(0, 2 ** 63)), int(rng.integers(0, 2 ** 40)))
+        compact = bool(rng.integers(0, 2))
+        n = g * int(rng.choice([1, 3, 17, 64, 65, 255, 1024, 4097, 30000]))
+        values = (rng.standard_normal(n) * 10.0 ** rng.integers(-8, 4)).astype(np.float32)
+        content = int(rng.integers(0, 4))
+        if content == 1:
+            values[rng.integers(0, n, max(1, n // 50))] = np.nan
+            values[rng.integers(0, n, 2)] = np.inf
+        elif content == 2:
+            values = np.round(values * 4) / 4
+        elif content == 3:
+            values[rng.integers(0, n, max(1, n // 3))] = 0
+        x_np = wire.from_f32(values, name)
+        x = from_numpy(x_np, name, hip_device)
+        policy = dict(group_size=g, bit=bit, quant_type=quant_type, topk=topk, compact=compact)
+        what = f"case {case}: {name} {policy} stochastic={stochastic} n={n} content={content}"
+        payload = torch.empty(hip.general_payload_nbytes(n, x.dtype, g, bit, topk), dtype=torch.uint8, device=hip_device)
+        assert hip.quant_general_into(x, payload, stochastic=stochastic, **policy), what
+        want = general.quantize(x_np, name, g, bit, quant_type, topk, stochastic, compact)
+        same(payload, want, "quantize " + what)
+        op = str(rng.choice(["none", "sum", "max", "min"]))
+        old_np = wire.from_f32(rng.standard_normal(n).astype(np.float32), name)
+        out = from_numpy(old_np, name, hip_device)
+        assert hip.dequant_general_into(payload, out, reduce_op=op, **policy), what
+        same(out, general.dequantize(want, n, name, g, bit, quant_type, topk, compact, op, old_np), f"decode {op} " + what)
+
+
 @pytest.mark.parametrize("name", list(NAMES))
 def test_plain_policy_equals_the_pack_kernel_on_finite_input(hip, hip_device, name):
     n = 64 * 4000
