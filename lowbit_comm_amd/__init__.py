@@ -10,10 +10,11 @@ from .config import CompressionConfig
 from .exceptions import CCDLError, CCDLUnavailableError, UnsupportedCollective
 from .execution_info import ExecutionCounters, ExecutionCounterSnapshot, ExecutionInfo
 from .shard import ReducedShard
+from .work import CollectiveWork, CompletionWork, ImmediateWork
 
 __all__ = [
-    "CCDLError", "CCDLUnavailableError", "CompressionConfig", "ExecutionCounterSnapshot", "ExecutionCounters",
-    "ExecutionInfo", "Quantizer", "ReducedShard", "UnsupportedCollective", "dequantize_tensor",
+    "CCDLError", "CCDLUnavailableError", "CollectiveWork", "CompletionWork", "CompressionConfig",
+    "ExecutionCounterSnapshot", "ExecutionCounters", "ExecutionInfo", "ImmediateWork", "Quantizer", "ReducedShard", "UnsupportedCollective", "dequantize_tensor",
     "estimate_quantized_size", "quantize_tensor",
 ]
 

@@ -1,4 +1,5 @@
 """HIP (gfx950) backend: C-ABI binding, tensor-level ops, native-module shim, codec callables, workspace pool."""
+from .completion import HipCompletionManager, HipStreamWork
 from .loader import CudaExtensionStatus, HipExtensionStatus, load_cuda_extension, load_hip_extension
 from .workspace import (
     CudaOutputLease,
@@ -19,7 +20,8 @@ from .workspace import (
 
 __all__ = [
     "CudaExtensionStatus", "CudaOutputLease", "CudaShardWorkspaceProvider", "CudaShardWorkspaceSession",
-    "CudaWorkspacePool", "EventCompletion", "EventCompletionManager", "HipExtensionStatus", "HipOutputLease",
+    "CudaWorkspacePool", "EventCompletion", "EventCompletionManager", "HipCompletionManager", "HipExtensionStatus",
+    "HipOutputLease", "HipStreamWork",
     "HipWorkspacePool", "ShardWorkspaceProvider", "ShardWorkspaceSession", "WorkspaceKey", "WorkspaceLease",
     "WorkspaceStats", "create_torch_workspace_pool", "load_cuda_extension", "load_hip_extension",
 ]

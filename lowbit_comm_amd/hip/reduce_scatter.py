@@ -232,3 +232,31 @@ def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: Co
 
 __all__ = ["ReduceScatterPlan", "compressed_all_reduce_via_reduce_scatter", "compressed_reduce_scatter_shard",
            "ccdl_dtype", "torch_dtype"]
+
+
+def compressed_all_reduce_async(tensor: torch.Tensor, *, config: CompressionConfig, world_size: int, rank: int,
+                                all_to_all: Callable[[torch.Tensor, torch.Tensor], None],
+                                all_gather: Callable[[torch.Tensor, torch.Tensor], None], op: str = "sum",
+                                plan: ReduceScatterPlan | None = None, out: torch.Tensor | None = None,
+                                manager: Any | None = None) -> Any:
+    """:func:`compressed_all_reduce_via_reduce_scatter` on the communication stream: returns a work object at once.
+
+    All four launches and the two exchanges are enqueued on a side stream ordered after the caller's current
+    stream; ``work.wait()`` orders the caller's current stream after them (no host wait) and returns the reduced
+    tensor.  The plan's workspaces and the input stay referenced by the work while it is in flight."""
+    from lowbit_comm_amd.hip.completion import HipCompletionManager
+
+    manager = manager if manager is not None else HipCompletionManager()
+    if plan is None:
+        plan = ReduceScatterPlan(tensor.numel(), tensor.dtype, world_size=world_size, rank=rank, config=config,
+                                 device=tensor.device, shape=tuple(tensor.shape))
+    stream_work = manager.create_stream_work(async_op=True)
+    with stream_work:
+        result = compressed_all_reduce_via_reduce_scatter(tensor, config=config, world_size=world_size, rank=rank,
+                                                          all_to_all=all_to_all, all_gather=all_gather, op=op,
+                                                          plan=plan, out=out)
+        stream = getattr(stream_work, "stream", None)
+        if stream is not None:            # the caching allocator must not reuse these before the side stream is done
+            for held in (tensor, result):
+                held.record_stream(stream)
+    return manager.create_work(result=result, completion=stream_work, resources=(tensor, plan, result))

@@ -428,6 +428,60 @@ def test_reduce_scatter_plan_fused_requantize_matches_the_two_steps(hip_device):
     assert float((full_fused - exact).norm() / exact.norm()) < 0.02
 
 
+def test_asynchronous_plan_runs_on_the_communication_stream_and_completes_by_stream_wait(hip_device):
+    """The whole plan enqueued behind a work object: same bits as the synchronous call; the launches land on the
+    device's side stream (busy main stream: a long torch job is enqueued first and the work is handed back before
+    it finished); ``wait()`` orders the current stream after the plan without blocking the host on it; the work
+    keeps the plan and tensors referenced until released."""
+    from lowbit_comm_amd.hip.completion import HipCompletionManager, communication_stream
+    from lowbit_comm_amd.hip.reduce_scatter import (ReduceScatterPlan, compressed_all_reduce_async,
+                                                    compressed_all_reduce_via_reduce_scatter)
+    from lowbit_comm_amd.work import CompletionWork
+
+    world, n = 4, 64 * 4 * 3000 + 77
+    config = CompressionConfig(error_feedback=False)
+    buckets = [torch.randn(n, device=hip_device) * 1e-3 for _ in range(world)]
+    plans = [ReduceScatterPlan(n, torch.float32, world_size=world, rank=r, config=config, device=hip_device)
+             for r in range(world)]
+    for r in range(1, world):
+        plans[r].quantize_chunks(buckets[r])
+
+    def all_to_all(received, send):
+        received[0].copy_(send[0])
+        for r in range(1, world):
+            received[r].copy_(plans[r].send[0])
+
+    def all_gather(gathered, mine):
+        for r in range(1, world):
+            for src in range(world):
+                plans[r].received[src].copy_(plans[0].send[r] if src == 0 else plans[src].send[r])
+            gathered[r, :plans[r].payload_bytes].copy_(plans[r].reduce_and_requantize(op="mean"))
+
+    want = compressed_all_reduce_via_reduce_scatter(buckets[0], config=config, world_size=world, rank=0,
+                                                    all_to_all=all_to_all, all_gather=all_gather, op="mean",
+                                                    plan=plans[0]).clone()
+    torch.cuda.synchronize()
+    manager = HipCompletionManager()
+    big = torch.randn(4096, 4096, device=hip_device)
+    for _ in range(20):
+        big = big @ big * 1e-3                                   # keeps the main stream busy for a while
+    out = torch.empty(n, device=hip_device)
+    work = compressed_all_reduce_async(buckets[0], config=config, world_size=world, rank=0, all_to_all=all_to_all,
+                                       all_gather=all_gather, op="mean", plan=plans[0], out=out, manager=manager)
+    assert isinstance(work, CompletionWork)
+    assert work.query() is False                                 # handed back while the device still works
+    assert plans[0] in work.resources and buckets[0] is work.resources[0]
+    side = communication_stream(torch.cuda)
+    assert side != torch.cuda.current_stream(hip_device)
+    result = work.wait()                                         # a device-side wait on the current stream
+    doubled = result * 2                                         # ordered after the plan by that wait
+    torch.cuda.synchronize()
+    assert work.query() is True and result.data_ptr() == out.data_ptr()
+    assert same_bits(result, want) and same_bits(doubled, want * 2)
+    work.release_resources()
+    assert work.resources == () and work.wait() is result
+
+
 def test_reduce_scatter_plan_beyond_eight_ranks_chains_exactly(dev):
     from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
 
