@@ -90,3 +90,17 @@ def test_device_code_has_no_instruction_that_changes_the_rounding_contract(tmp_p
         assert "gfx950" in text
         for forbidden in ("v_fma_mix", "v_mad_mix", "v_pk_mul_f32", "v_pk_add_f32", "v_pk_fma_f32"):
             assert forbidden not in text, (out.name, forbidden)
+
+
+def test_product_code_never_reaches_into_the_oracle_or_the_working_folder():
+    """The oracle is a checker: only tests, the smoke check and the benchmark's CPU-baseline leg may load it."""
+    offenders = []
+    for path in sorted((ROOT / "lowbit_comm_amd").rglob("*")):
+        if path.suffix not in (".py", ".hip", ".h") or "_build" in path.parts:
+            continue
+        text = path.read_text(errors="ignore")
+        if re.search(r"^\s*(from|import)\s+oracle\b|oracle/|_work/|\b_work\b", text, flags=re.M):
+            offenders.append(str(path.relative_to(ROOT)))
+    assert offenders == []
+    bench = (ROOT / "bench.py").read_text()
+    assert "_work/" not in bench and "_work/" not in (ROOT / "__graft_entry__.py").read_text()
