@@ -235,6 +235,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
             c[i] = r < -L ? -L : (r > L ? L : r);
         }
     } else {
+        float excess[VEC], gap[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const float t = v[i] / scale;
@@ -245,9 +246,17 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
                 const float entry = book[mid];
                 if (mid < 15 && !(t < entry)) lower = mid;
             }
-            const float low = book[lower], gap = book[lower + 1] - low, excess = t - low;
-            const bool up = a.stochastic ? uniform[i] < excess / gap : excess > gap * 0.5f;
-            c[i] = lower + (up ? 1 : 0);
+            const float low = book[lower];
+            gap[i] = book[lower + 1] - low;
+            excess[i] = t - low;
+            c[i] = lower;
+        }
+        if (a.stochastic) {   // uniform: the second division only runs when it is needed
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) c[i] += uniform[i] < excess[i] / gap[i] ? 1 : 0;
+        } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) c[i] += excess[i] > gap[i] * 0.5f ? 1 : 0;
         }
     }
     if (live) {
