@@ -19,3 +19,12 @@ def hip_device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="session")
+def golden_vectors():
+    """The reference's literal test vectors and published known answers (tests/golden/reference_vectors.json)."""
+    import json
+    from pathlib import Path
+
+    return json.loads((Path(__file__).resolve().parent / "golden" / "reference_vectors.json").read_text())

@@ -36,19 +36,17 @@ def same_bits(a, b):
 # --------------------------------------------------------------------------- #
 # Philox4x32-10 and the cuRAND stream
 # --------------------------------------------------------------------------- #
-KNOWN_ANSWERS = [   # counter, key, output: kat_vectors of the Random123 distribution, philox4x32 with 10 rounds
-    ((0, 0, 0, 0), (0, 0), (0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8)),
-    ((0xFFFFFFFF,) * 4, (0xFFFFFFFF,) * 2, (0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD)),
-    ((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0),
-     (0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1)),
-]
-
-
-@pytest.mark.parametrize("counter,key,expected", KNOWN_ANSWERS)
-def test_philox_known_answers(counter, key, expected):
-    got = general.philox4x32_10([np.array([c]) for c in counter], [np.array([k]) for k in key])
-    assert tuple(int(word[0]) for word in got) == expected
-    assert tuple(int(word) for word in general_c.philox_block(counter, key)) == expected
+def test_philox_known_answers(golden_vectors):
+    """kat_vectors of the Random123 distribution, philox4x32 with 10 rounds (tests/golden/reference_vectors.json)."""
+    vectors = golden_vectors["philox4x32_10"]["vectors"]
+    assert len(vectors) == 3
+    for vector in vectors:
+        counter = tuple(int(word, 16) for word in vector["counter"])
+        key = tuple(int(word, 16) for word in vector["key"])
+        expected = tuple(int(word, 16) for word in vector["output"])
+        got = general.philox4x32_10([np.array([c]) for c in counter], [np.array([k]) for k in key])
+        assert tuple(int(word[0]) for word in got) == expected
+        assert tuple(int(word) for word in general_c.philox_block(counter, key)) == expected
 
 
 @pytest.mark.parametrize("offset", (0, 1, 2, 3, 4, 4099, 2 ** 34 + 6))

@@ -56,6 +56,14 @@ def test_config_defaults_and_validation():
 # --------------------------------------------------------------------------- #
 # sizing (reference tests/test_quantization_sizing.py:7-51)
 # --------------------------------------------------------------------------- #
+def test_native_sizing_matches_the_reference_fixture(golden_vectors):
+    for case in golden_vectors["sizing"]["cases"]:
+        estimate = estimate_quantized_size(case["numel"], dtype=case["dtype"], config=CompressionConfig(**case["config"]))
+        for field, want in case.items():
+            if field not in ("numel", "dtype", "config"):
+                assert getattr(estimate, field) == want, (case, field)
+
+
 def test_native_sizing_matches_the_reference_numbers():
     cfg = CompressionConfig()
     e = estimate_quantized_size(128, dtype="fp16", config=cfg)

@@ -322,12 +322,13 @@ def test_empty_payload_list_and_bad_mode_are_rejected():
 # --------------------------------------------------------------------------- #
 # wire format: literal vectors from the reference's packer test
 # --------------------------------------------------------------------------- #
-def test_pack_layout_literal_bytes():
-    codes = np.array([-2, 3, 7, 11], dtype=np.int8)
-    scales = np.array([0.25, 1.0], dtype=np.float32)
+def test_pack_layout_literal_bytes(golden_vectors):
+    vector = golden_vectors["packer"]
+    codes = np.array(vector["codes"], dtype=np.int8)
+    scales = np.array(vector["scales"], dtype=np.float32)
     packed = codec_np.pack(codes, scales)
     assert packed.dtype == np.uint8
-    assert packed.tolist() == [254, 3, 7, 11, 0, 0, 128, 62, 0, 0, 128, 63]
+    assert packed.tolist() == vector["packed_bytes"]
     assert codec_torch.pack(torch.from_numpy(codes), torch.from_numpy(scales)).tolist() == packed.tolist()
 
 
@@ -346,14 +347,16 @@ def test_pack_unpack_round_trip_and_size():
 # --------------------------------------------------------------------------- #
 # error feedback: literal vectors from the reference's tests
 # --------------------------------------------------------------------------- #
-def test_error_feedback_literal_cycle():
-    residual = codec_np.ef_residual(np.float32([1.0, 2.0]), np.float32([0.75, 1.5]), "fp32")
-    assert residual.tolist() == [0.25, 0.5]
-    assert codec_np.ef_compensate(np.float32([10.0, 20.0]), "fp32", residual).tolist() == [10.25, 20.5]
-    r = codec_np.ef_residual(np.float32([4.0]), np.float32([3.0]), "fp32")
-    p = codec_np.ef_compensate(np.float32([10.0]), "fp32", r)
-    assert p.tolist() == [11.0]
-    assert codec_np.ef_residual(p, np.float32([10.25]), "fp32").tolist() == [0.75]
+def test_error_feedback_literal_cycle(golden_vectors):
+    first = golden_vectors["error_feedback"]["update_then_compensate"]
+    residual = codec_np.ef_residual(np.float32(first["original"]), np.float32(first["transmitted"]), "fp32")
+    assert residual.tolist() == first["residual"]
+    assert codec_np.ef_compensate(np.float32(first["next_gradient"]), "fp32", residual).tolist() == first["compensated"]
+    cycle = golden_vectors["error_feedback"]["cycle"]
+    r = codec_np.ef_residual(np.float32(cycle["original"]), np.float32(cycle["transmitted"]), "fp32")
+    p = codec_np.ef_compensate(np.float32(cycle["gradient"]), "fp32", r)
+    assert p.tolist() == cycle["compensated"]
+    assert codec_np.ef_residual(p, np.float32(cycle["transmitted_next"]), "fp32").tolist() == cycle["residual_next"]
 
 
 @pytest.mark.parametrize("restored_dtype", ["fp32", "bf16"])
