@@ -230,8 +230,8 @@ def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: Co
     return plan.decode_gathered(out=out)
 
 
-__all__ = ["ReduceScatterPlan", "compressed_all_reduce_via_reduce_scatter", "compressed_reduce_scatter_shard",
-           "ccdl_dtype", "torch_dtype"]
+__all__ = ["ReduceScatterPlan", "compressed_all_reduce_async", "compressed_all_reduce_via_reduce_scatter",
+           "compressed_reduce_scatter_shard", "make_reduce_scatter_transport", "ccdl_dtype", "torch_dtype"]
 
 
 def compressed_all_reduce_async(tensor: torch.Tensor, *, config: CompressionConfig, world_size: int, rank: int,
@@ -260,3 +260,53 @@ def compressed_all_reduce_async(tensor: torch.Tensor, *, config: CompressionConf
             for held in (tensor, result):
                 held.record_stream(stream)
     return manager.create_work(result=result, completion=stream_work, resources=(tensor, plan, result))
+
+
+def make_reduce_scatter_transport(*, world_size: int, rank: int,
+                                  all_to_all: Callable[[torch.Tensor, torch.Tensor], None],
+                                  all_gather: Callable[[torch.Tensor, torch.Tensor], None],
+                                  max_plans: int = 64, manager: Any | None = None,
+                                  inplace: bool = True) -> Callable[..., Any]:
+    """The callable ``create_ddp_comm_hook(reduce_scatter_all_gather=...)`` expects, over pre-bound plans.
+
+    ``transport(tensor, *, config, op, async_op=False, dtype=None, extension_status=None)`` runs the compressed
+    reduce-scatter + all-gather of ``tensor`` and returns the reduced tensor (``async_op``: a work object whose
+    ``wait()`` returns it).  One :class:`ReduceScatterPlan` is kept per (element count, dtype, device, codec policy),
+    so a bucket costs three pre-bound launches and the two injected exchanges from its second step on; the least
+    recently used plan is dropped beyond ``max_plans``.  With ``inplace`` the decoded result overwrites ``tensor``
+    (a DDP bucket is consumed by the quantize launch before the decode launch writes it), so nothing is allocated.  Counterpart of ``compressed_reduce_scatter_all_gather``
+    (``ccdl_comm/communication/reduce_scatter_transport.py:186-377``) with the exchanges injected."""
+    from collections import OrderedDict
+
+    plans: OrderedDict = OrderedDict()
+
+    def plan_for(tensor: torch.Tensor, config: CompressionConfig) -> ReduceScatterPlan:
+        key = (tensor.numel(), tensor.dtype, tensor.device, config.bit, config.group_size, config.topk,
+               config.quant_type, config.stochastic)
+        plan = plans.get(key)
+        if plan is None:
+            plan = plans[key] = ReduceScatterPlan(tensor.numel(), tensor.dtype, world_size=world_size, rank=rank,
+                                                  config=config, device=tensor.device, shape=tuple(tensor.shape))
+            while len(plans) > max_plans:
+                plans.popitem(last=False)
+        else:
+            plans.move_to_end(key)
+        return plan
+
+    def transport(tensor: torch.Tensor, *, config: CompressionConfig, op: str = "sum", async_op: bool = False,
+                  dtype: str | None = None, extension_status: Any | None = None) -> Any:
+        del extension_status                      # the plan calls the C ABI directly
+        if dtype is not None and torch_dtype(dtype) != tensor.dtype:
+            raise ValueError(f"the reduce-scatter plan reduces in the bucket's dtype; got dtype={dtype!r} for {tensor.dtype}")
+        plan = plan_for(tensor, config)
+        out = tensor.reshape(-1) if inplace and tensor.is_contiguous() else None
+        if async_op:
+            return compressed_all_reduce_async(tensor, config=config, world_size=world_size, rank=rank,
+                                               all_to_all=all_to_all, all_gather=all_gather, op=op, plan=plan,
+                                               out=out, manager=manager)
+        return compressed_all_reduce_via_reduce_scatter(tensor, config=config, world_size=world_size, rank=rank,
+                                                        all_to_all=all_to_all, all_gather=all_gather, op=op, plan=plan,
+                                                        out=out)
+
+    transport.plans = plans
+    return transport

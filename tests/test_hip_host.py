@@ -482,6 +482,64 @@ def test_asynchronous_plan_runs_on_the_communication_stream_and_completes_by_str
     assert work.resources == () and work.wait() is result
 
 
+def test_hook_over_the_reduce_scatter_transport_reuses_one_plan_per_bucket_shape(hip_device):
+    """``create_ddp_comm_hook(strategy="reduce_scatter", reduce_scatter_all_gather=make_reduce_scatter_transport(...))``:
+    every bucket runs the pre-bound plan, results equal the plan called directly, the bucket is reduced in place
+    and steady-state steps allocate nothing."""
+    from lowbit_comm_amd.hip.reduce_scatter import (ReduceScatterPlan, compressed_all_reduce_via_reduce_scatter,
+                                                    make_reduce_scatter_transport)
+
+    world = 4
+    config = CompressionConfig(error_feedback=False)
+    sizes = [64 * 4 * 700 + 5, 64 * 4 * 300]
+    peers = {n: [ReduceScatterPlan(n, torch.float32, world_size=world, rank=r, config=config, device=hip_device)
+                 for r in range(world)] for n in sizes}
+    peer_data = {n: [torch.randn(n, device=hip_device) * 1e-3 for _ in range(world)] for n in sizes}
+    for n in sizes:
+        for r in range(1, world):
+            peers[n][r].quantize_chunks(peer_data[n][r])
+
+    def all_to_all(received, send):
+        n = next(k for k in sizes if peers[k][0].row_stride == send.shape[1])
+        received[0].copy_(send[0])
+        for r in range(1, world):
+            received[r].copy_(peers[n][r].send[0])
+
+    def all_gather(gathered, mine):
+        n = next(k for k in sizes if peers[k][0].row_stride == gathered.shape[1])
+        for r in range(1, world):
+            for src in range(world):
+                peers[n][r].received[src].copy_(mine_send[n][r] if src == 0 else peers[n][src].send[r])
+            gathered[r, :peers[n][r].payload_bytes].copy_(peers[n][r].reduce_and_requantize(op="mean"))
+
+    mine_send = {}
+    want = {}
+    for n in sizes:                                     # the expected result, through the plan called directly
+        probe = ReduceScatterPlan(n, torch.float32, world_size=world, rank=0, config=config, device=hip_device)
+        mine_send[n] = probe.quantize_chunks(peer_data[n][0]).clone()
+        want[n] = compressed_all_reduce_via_reduce_scatter(peer_data[n][0].clone(), config=config, world_size=world,
+                                                           rank=0, all_to_all=all_to_all, all_gather=all_gather,
+                                                           op="mean", plan=probe).clone()
+    transport = make_reduce_scatter_transport(world_size=world, rank=0, all_to_all=all_to_all, all_gather=all_gather)
+    hook = create_ddp_comm_hook(config, strategy="reduce_scatter", reduce="mean",
+                                reduce_scatter_all_gather=transport)
+    assert hook._ccdl_effective_strategy == "reduce_scatter"
+    buckets = {n: Bucket(peer_data[n][0].clone(), i) for i, n in enumerate(sizes)}
+    for n in sizes:
+        result = hook(None, buckets[n]).wait()
+        assert result.data_ptr() == buckets[n].buffer().data_ptr()          # reduced in place
+        assert same_bits(result, want[n])
+    assert len(transport.plans) == 2
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    for _ in range(3):
+        for n in sizes:
+            buckets[n].buffer().copy_(peer_data[n][0])
+            assert same_bits(hook(None, buckets[n]).wait(), want[n])
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before and len(transport.plans) == 2
+
+
 def test_reduce_scatter_plan_beyond_eight_ranks_chains_exactly(dev):
     from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
 
