@@ -218,6 +218,8 @@ def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: Co
     if plan is None:
         plan = ReduceScatterPlan(tensor.numel(), tensor.dtype, world_size=world_size, rank=rank, config=config,
                                  device=tensor.device, shape=tuple(tensor.shape))
+    if plan.numel == 0:       # nothing to exchange on any rank (reduce_scatter_transport.py:213-246 returns at once)
+        return out.reshape(plan.shape) if out is not None else tensor
     if keep_shard:
         compressed_reduce_scatter_shard(tensor, config=config, world_size=world_size, rank=rank,
                                         all_to_all=all_to_all, op=op, plan=plan)

@@ -538,6 +538,10 @@ def test_hook_over_the_reduce_scatter_transport_reuses_one_plan_per_bucket_shape
             assert same_bits(hook(None, buckets[n]).wait(), want[n])
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before and len(transport.plans) == 2
+    empty = hook(None, Bucket(torch.empty(0, device=hip_device), 9)).wait()         # an empty bucket is a no-op
+    assert empty.numel() == 0
+    with pytest.raises(ValueError, match="reduces in the bucket's dtype"):
+        transport(buckets[sizes[0]].buffer(), config=config, op="mean", dtype="bf16")
 
 
 def test_reduce_scatter_plan_beyond_eight_ranks_chains_exactly(dev):
