@@ -515,9 +515,12 @@ def test_full_plan_config4_scaled(ops, hip_device):
 # randomized sweep over shapes, dtypes, groups, alignments and payload counts
 # --------------------------------------------------------------------------- #
 def test_randomized_parity_sweep(ops, hip_device):
-    rng = np.random.default_rng(20261125)
+    """60 seeded cases by default; LBC_SWEEP_CASES / LBC_SWEEP_SEED lengthen or reseed the sweep."""
+    import os
+
+    rng = np.random.default_rng(int(os.environ.get("LBC_SWEEP_SEED", "20261125")))
     names = ["fp32", "fp16", "bf16"]
-    for case in range(60):
+    for case in range(int(os.environ.get("LBC_SWEEP_CASES", "60"))):
         g = int(rng.choice([16, 32, 64]))
         n = int(rng.integers(1, 200_000))
         x_name = names[int(rng.integers(0, 3))]
