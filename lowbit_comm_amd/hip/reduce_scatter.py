@@ -206,8 +206,12 @@ def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: Co
                                              rank: int, all_to_all: Callable[[torch.Tensor, torch.Tensor], None],
                                              all_gather: Callable[[torch.Tensor, torch.Tensor], None],
                                              op: str = "sum", plan: ReduceScatterPlan | None = None,
-                                             out: torch.Tensor | None = None, keep_shard: bool = False) -> torch.Tensor:
+                                             out: torch.Tensor | None = None, keep_shard: bool = False,
+                                             residual: torch.Tensor | None = None) -> torch.Tensor:
     """Full plan: reduce-scatter leg, requantize, all-gather leg, decode every shard.
+
+    ``residual`` (fp32 or the bucket's dtype, updated in place) turns on local error feedback in the quantize
+    launch: the chunks encode ``tensor + residual`` and the residual becomes what that encoding dropped.
 
     Reduce and requantize run as one launch unless ``keep_shard`` asks for the full-precision shard in
     ``plan.shard`` as well.
@@ -221,11 +225,13 @@ def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: Co
     if plan.numel == 0:       # nothing to exchange on any rank (reduce_scatter_transport.py:213-246 returns at once)
         return out.reshape(plan.shape) if out is not None else tensor
     if keep_shard:
+        if residual is not None:
+            raise ValueError("keep_shard and residual cannot be combined")
         compressed_reduce_scatter_shard(tensor, config=config, world_size=world_size, rank=rank,
                                         all_to_all=all_to_all, op=op, plan=plan)
         mine = plan.requantize_shard()
     else:
-        send = plan.quantize_chunks(tensor)
+        send = plan.quantize_chunks(tensor, residual=residual, new_residual=residual)
         all_to_all(plan.received, send)
         mine = plan.reduce_and_requantize(op=op)
     all_gather(plan.gathered, mine)
@@ -240,7 +246,7 @@ def compressed_all_reduce_async(tensor: torch.Tensor, *, config: CompressionConf
                                 all_to_all: Callable[[torch.Tensor, torch.Tensor], None],
                                 all_gather: Callable[[torch.Tensor, torch.Tensor], None], op: str = "sum",
                                 plan: ReduceScatterPlan | None = None, out: torch.Tensor | None = None,
-                                manager: Any | None = None) -> Any:
+                                manager: Any | None = None, residual: torch.Tensor | None = None) -> Any:
     """:func:`compressed_all_reduce_via_reduce_scatter` on the communication stream: returns a work object at once.
 
     All four launches and the two exchanges are enqueued on a side stream ordered after the caller's current
@@ -256,19 +262,19 @@ def compressed_all_reduce_async(tensor: torch.Tensor, *, config: CompressionConf
     with stream_work:
         result = compressed_all_reduce_via_reduce_scatter(tensor, config=config, world_size=world_size, rank=rank,
                                                           all_to_all=all_to_all, all_gather=all_gather, op=op,
-                                                          plan=plan, out=out)
+                                                          plan=plan, out=out, residual=residual)
         stream = getattr(stream_work, "stream", None)
         if stream is not None:            # the caching allocator must not reuse these before the side stream is done
-            for held in (tensor, result):
+            for held in (tensor, result) + (() if residual is None else (residual,)):
                 held.record_stream(stream)
-    return manager.create_work(result=result, completion=stream_work, resources=(tensor, plan, result))
+    return manager.create_work(result=result, completion=stream_work, resources=(tensor, plan, result, residual))
 
 
 def make_reduce_scatter_transport(*, world_size: int, rank: int,
                                   all_to_all: Callable[[torch.Tensor, torch.Tensor], None],
                                   all_gather: Callable[[torch.Tensor, torch.Tensor], None],
                                   max_plans: int = 64, manager: Any | None = None,
-                                  inplace: bool = True) -> Callable[..., Any]:
+                                  inplace: bool = True, error_feedback: bool = False) -> Callable[..., Any]:
     """The callable ``create_ddp_comm_hook(reduce_scatter_all_gather=...)`` expects, over pre-bound plans.
 
     ``transport(tensor, *, config, op, async_op=False, dtype=None, extension_status=None)`` runs the compressed
@@ -276,11 +282,25 @@ def make_reduce_scatter_transport(*, world_size: int, rank: int,
     ``wait()`` returns it).  One :class:`ReduceScatterPlan` is kept per (element count, dtype, device, codec policy),
     so a bucket costs three pre-bound launches and the two injected exchanges from its second step on; the least
     recently used plan is dropped beyond ``max_plans``.  With ``inplace`` the decoded result overwrites ``tensor``
-    (a DDP bucket is consumed by the quantize launch before the decode launch writes it), so nothing is allocated.  Counterpart of ``compressed_reduce_scatter_all_gather``
+    (a DDP bucket is consumed by the quantize launch before the decode launch writes it), so nothing is allocated.
+    With ``error_feedback`` every bucket (keyed by its storage address and size) keeps an fp32 residual that the
+    quantize launch adds before encoding and refreshes with what the encoding dropped, in the same launch - the
+    local error feedback of ``DDPBucketProcessor`` (``ccdl_comm/communication/ddp.py:69-97``); ``transport.residuals``
+    exposes them, ``transport.reset()`` drops them.  Counterpart of ``compressed_reduce_scatter_all_gather``
     (``ccdl_comm/communication/reduce_scatter_transport.py:186-377``) with the exchanges injected."""
     from collections import OrderedDict
 
     plans: OrderedDict = OrderedDict()
+    residuals: dict = {}
+
+    def residual_for(tensor: torch.Tensor) -> torch.Tensor | None:
+        if not error_feedback or tensor.numel() == 0:
+            return None
+        key = (tensor.data_ptr(), tensor.numel(), tensor.dtype)
+        residual = residuals.get(key)
+        if residual is None:
+            residual = residuals[key] = torch.zeros(tensor.numel(), dtype=torch.float32, device=tensor.device)
+        return residual
 
     def plan_for(tensor: torch.Tensor, config: CompressionConfig) -> ReduceScatterPlan:
         key = (tensor.numel(), tensor.dtype, tensor.device, config.bit, config.group_size, config.topk,
@@ -302,13 +322,16 @@ def make_reduce_scatter_transport(*, world_size: int, rank: int,
             raise ValueError(f"the reduce-scatter plan reduces in the bucket's dtype; got dtype={dtype!r} for {tensor.dtype}")
         plan = plan_for(tensor, config)
         out = tensor.reshape(-1) if inplace and tensor.is_contiguous() else None
+        residual = residual_for(tensor)
         if async_op:
             return compressed_all_reduce_async(tensor, config=config, world_size=world_size, rank=rank,
                                                all_to_all=all_to_all, all_gather=all_gather, op=op, plan=plan,
-                                               out=out, manager=manager)
+                                               out=out, manager=manager, residual=residual)
         return compressed_all_reduce_via_reduce_scatter(tensor, config=config, world_size=world_size, rank=rank,
                                                         all_to_all=all_to_all, all_gather=all_gather, op=op, plan=plan,
-                                                        out=out)
+                                                        out=out, residual=residual)
 
     transport.plans = plans
+    transport.residuals = residuals
+    transport.reset = residuals.clear
     return transport

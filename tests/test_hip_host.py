@@ -544,6 +544,51 @@ def test_hook_over_the_reduce_scatter_transport_reuses_one_plan_per_bucket_shape
         transport(buckets[sizes[0]].buffer(), config=config, op="mean", dtype="bf16")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_reduce_scatter_transport_with_local_error_feedback(hip_device, dtype):
+    """Three steps of one bucket through the transport with error feedback: what is sent and the residual it keeps
+    equal the oracle's compensate -> quantize -> residual cycle per destination chunk, step after step."""
+    from lowbit_comm_amd.hip.reduce_scatter import make_reduce_scatter_transport
+
+    world, g, n = 4, 64, 64 * 4 * 50 + 37
+    config = CompressionConfig()
+    sent = []
+
+    def all_to_all(received, send):
+        sent.append(send.clone())
+        for r in range(world):
+            received[r].copy_(send[0])
+
+    def all_gather(gathered, mine):
+        for r in range(world):
+            gathered[r, :mine.numel()].copy_(mine)
+
+    transport = make_reduce_scatter_transport(world_size=world, rank=0, all_to_all=all_to_all, all_gather=all_gather,
+                                              error_feedback=True)
+    bucket = torch.empty(n, dtype=dtype, device=hip_device)
+    shard = -(-n // world)
+    want_residual = torch.zeros(n)
+    for step in range(3):
+        x = grad(n, dtype, 40 + step, hip_device)
+        bucket.copy_(x)
+        result = transport(bucket, config=config, op="mean")
+        assert result.data_ptr() == bucket.data_ptr()
+        residual = next(iter(transport.residuals.values()))
+        assert len(transport.residuals) == 1 and residual.dtype == torch.float32
+        for d in range(world):
+            piece = slice(d * shard, min(n, (d + 1) * shard))
+            codes, scales, _restored, new_r = codec_torch.ef_round_trip(x[piece].cpu(), want_residual[piece], g, "fp32")
+            row = sent[-1][d].cpu()
+            padded = -(-shard // g) * g
+            assert torch.equal(row[:codes.numel()].view(torch.int8), codes), (step, d)
+            assert torch.equal(row[padded:padded + 4 * scales.numel()].view(torch.float32).view(torch.int32),
+                               scales.view(torch.int32)), (step, d)
+            want_residual[piece] = new_r
+        assert same_bits(residual, want_residual), step
+    transport.reset()
+    assert not transport.residuals
+
+
 def test_reduce_scatter_plan_beyond_eight_ranks_chains_exactly(dev):
     from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
 
