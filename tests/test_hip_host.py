@@ -795,7 +795,7 @@ def test_bucket_step_replays_from_a_hip_graph(dev):
         assert same_bits(plan.shard, codec_torch.reduce_payloads(received, shard, 64, "fp32", "mean")), step
 
 
-@pytest.mark.parametrize("wire_format", ["portable", "native"])
+@pytest.mark.parametrize("wire_format", ["portable", "native", "reduce_scatter"])
 def test_hook_on_a_real_distributed_data_parallel_model(hip_device, wire_format):
     """register_comm_hook on torch's own DDP (one rank, RCCL): real GradBucket objects and futures, gradients within
     the quantization error of the uncompressed model.  Runs in a child process under a time limit so that trouble in

@@ -1,7 +1,9 @@
 """Worker for tests/test_hip_host.py: the compressed hook registered on a real DistributedDataParallel model.
 
-One process, one GPU, a one-rank RCCL process group (the all-gather of a one-rank world is the identity, injected
-as such).  Prints one JSON line with the gradient errors against an unwrapped copy of the model.
+One process, one GPU, a one-rank RCCL process group.  Modes "portable" / "native": the all_gather strategy in that
+wire format (the all-gather of a one-rank world is the identity, injected as such).  Mode "reduce_scatter": the
+pre-bound reduce-scatter plan with its two exchanges as real RCCL calls (all_to_all_single, all_gather_into_tensor)
+and local error feedback.  Prints one JSON line with the gradient errors against an unwrapped copy of the model.
 """
 from __future__ import annotations
 
@@ -44,7 +46,7 @@ def main() -> int:
         model, plain = make(), make()
         plain.load_state_dict(model.state_dict())
         wrapped = DistributedDataParallel(model, device_ids=[0], bucket_cap_mb=1)
-        status = load_hip_extension(wire_format=wire_format)
+        status = load_hip_extension(wire_format="portable" if wire_format == "reduce_scatter" else wire_format)
         assert status.available, status.reason
         seen = []
 
@@ -52,8 +54,23 @@ def main() -> int:
             seen.append(int(payload.buffer.numel()))
             return GatheredPayloads(payloads=[payload], world_size=1)
 
-        hook = create_ddp_comm_hook(CompressionConfig(error_feedback=True), strategy="all_gather", reduce="mean",
-                                    all_gather=gather, extension_status=status)
+        if wire_format == "reduce_scatter":
+            from lowbit_comm_amd.hip.reduce_scatter import make_reduce_scatter_transport
+
+            def all_to_all(received, send):
+                seen.append(int(send.shape[1]))
+                dist.all_to_all_single(received, send)
+
+            def all_gather(gathered, mine):
+                dist.all_gather_into_tensor(gathered, gathered[0])
+
+            transport = make_reduce_scatter_transport(world_size=1, rank=0, all_to_all=all_to_all,
+                                                      all_gather=all_gather, error_feedback=True)
+            hook = create_ddp_comm_hook(CompressionConfig(error_feedback=False), strategy="reduce_scatter",
+                                        reduce="mean", reduce_scatter_all_gather=transport)
+        else:
+            hook = create_ddp_comm_hook(CompressionConfig(error_feedback=True), strategy="all_gather", reduce="mean",
+                                        all_gather=gather, extension_status=status)
         wrapped.register_comm_hook(None, hook)
         x = torch.randn(64, 512, device=device)
         errors = []
