@@ -13,10 +13,13 @@ object per configuration plus a summary table on stderr:
      bucket through the workspace pool
   6  the same bucket shapes in the byte format of the reference's CUDA extension (scales in the tensor
      dtype, interleaved or appended): quantize+pack, W=8 fused reduce, mean + error-feedback reduce
+  7  the host side: the DDP communication hook per bucket (all_gather strategy through the codec facade; reduce-scatter
+     strategy over pre-bound plans, without and with error feedback), a pre-bound launch, and the config-5 launch
+     sequence eager against one HIP-graph replay.  Rows report host microseconds per bucket next to wall time.
 
 "~N(0, s)" is read as standard deviation s.  Times are HIP-event averages over back-to-back launches.
 
-    python bench_configs.py [--configs 1,2,3,4,5,6] [--no-parity] [--llama-layers 32]
+    python bench_configs.py [--configs 1,2,3,4,5,6,7] [--no-parity] [--llama-layers 32]
 """
 from __future__ import annotations
 
@@ -37,7 +40,7 @@ G = 64
 
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--configs", default="1,2,3,4,5,6")
+    ap.add_argument("--configs", default="1,2,3,4,5,6,7")
     ap.add_argument("--no-parity", action="store_true", help="skip the CPU oracle comparisons")
     ap.add_argument("--llama-layers", type=int, default=32, help="config 5: number of transformer layers (32 = full model)")
     ap.add_argument("--iters", type=int, default=50)
@@ -525,8 +528,131 @@ def main() -> int:
                 del outs, quant, decode
             del xs, back
 
+
+    # ------------------------------------------------------------------------------------------ 7
+    if 7 in wanted:
+        from lowbit_comm_amd.communication import CompressedPayload, GatheredPayloads
+        from lowbit_comm_amd.communication.ddp_hook import create_ddp_comm_hook
+        from lowbit_comm_amd.hip.loader import load_hip_extension
+        from lowbit_comm_amd.hip.reduce_scatter import make_reduce_scatter_transport
+
+        class Bucket:
+            def __init__(self, tensor, index):
+                self._tensor, self._index = tensor, index
+
+            def buffer(self):
+                return self._tensor
+
+            def index(self):
+                return self._index
+
+        class Slot:
+            def set_result(self, value):
+                self.value = value
+
+        def host_and_wall(fn, count):
+            for i in range(8):
+                fn(i)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(count):
+                fn(i)
+            host = (time.perf_counter() - t0) / count
+            torch.cuda.synchronize()
+            return host, (time.perf_counter() - t0) / count
+
+        def host_row(op, host, wall, **extra):
+            row = {"config": 7, "op": op, "host_us": host * 1e6, "us": wall * 1e6, "algorithmic_bytes": 0,
+                   "achieved_GBps": 0.0, "frac_of_hbm_peak": 0.0, "input_GBps": 0.0, "parity": None}
+            row.update(extra)
+            rows_out.append(row)
+            print(json.dumps(row), flush=True)
+
+        world, n = 8, 13_107_200                                   # a 25 MiB bf16 bucket
+        status = load_hip_extension()
+        buckets = [Bucket(gen(SEED + 7000 + i, n, 1e-3, torch.bfloat16), i) for i in range(4)]
+        # all_gather strategy through the facade: W - 1 stand-in peers resident in HBM
+        peers = {}
+
+        def gather(payload):
+            key = payload.buffer.numel()
+            if key not in peers:
+                peers[key] = [payload.buffer.clone() for _ in range(world - 1)]
+            others = [CompressedPayload(buffer=b, shape=payload.shape, dtype=payload.dtype) for b in peers[key]]
+            return GatheredPayloads(payloads=[payload] + others, world_size=world)
+
+        for feedback in (False, True):
+            hook = create_ddp_comm_hook(CompressionConfig(error_feedback=feedback), strategy="all_gather", reduce="mean",
+                                        all_gather=gather, extension_status=status, future_factory=Slot,
+                                        workspace_cache_max_entries=8)
+            host, wall = host_and_wall(lambda i: hook(None, buckets[i % 4]), 40)
+            host_row(f"hook, all_gather strategy through the facade, 25 MiB bf16 bucket, W=8, error feedback {feedback}",
+                     host, wall)
+        # reduce-scatter strategy over pre-bound plans; the exchanges are stand-ins that fill the rows once
+        for feedback in (False, True):
+            filled = set()
+
+            def all_to_all(received, send):
+                if received.data_ptr() not in filled:
+                    for r in range(world):
+                        received[r].copy_(send[0])
+                    filled.add(received.data_ptr())
+
+            def all_gather(gathered, mine):
+                if gathered.data_ptr() not in filled:
+                    for r in range(world):
+                        gathered[r, :mine.numel()].copy_(mine)
+                    filled.add(gathered.data_ptr())
+
+            transport = make_reduce_scatter_transport(world_size=world, rank=0, all_to_all=all_to_all,
+                                                      all_gather=all_gather, error_feedback=feedback)
+            hook = create_ddp_comm_hook(CompressionConfig(error_feedback=False), strategy="reduce_scatter", reduce="mean",
+                                        reduce_scatter_all_gather=transport, future_factory=Slot)
+            host, wall = host_and_wall(lambda i: hook(None, buckets[i % 4]), 60)
+            host_row(f"hook, reduce_scatter strategy over pre-bound plans, 25 MiB bf16 bucket, W=8, error feedback {feedback}",
+                     host, wall)
+        # one pre-bound launch
+        x = gen(SEED + 7100, n, 1e-3, torch.bfloat16)
+        payload = torch.empty(ops.payload_nbytes(n, G), dtype=torch.uint8, device=dev)
+        codes, scales = ops.split_payload(payload, n, G)
+        bound = ops.bind_quant_pack(x, codes, scales)
+        host, wall = host_and_wall(lambda i: bound(), 300)
+        host_row("one pre-bound launch (quantize+pack of the bucket)", host, wall)
+        # the config-5 launch sequence (64 buckets): eager pre-bound launches against one graph replay
+        count = 64
+        shard = n // world
+        stride = -(-ops.payload_nbytes(shard, G) // 256) * 256
+        grads = gen(SEED + 7200, count * n, 1e-3, torch.bfloat16)
+        residuals = gen(SEED + 7300, count * n, 1e-5)
+        rows = torch.empty(world, stride, dtype=torch.uint8, device=dev)
+        received = [ops.quant_pack(gen(SEED + 7400 + r, shard, 1e-3), group_size=G) for r in range(world)]
+        out = torch.empty(shard, device=dev)
+        launches = []
+        for i in range(count):
+            piece = slice(i * n, (i + 1) * n)
+            launches.append(ops.bind_quant_pack_chunks(grads[piece], rows, world, residual=residuals[piece],
+                                                       new_residual=residuals[piece]))
+            launches.append(ops.bind_dequant_reduce(received, out, numel=shard))
+
+        def eager(_i=0):
+            for launch in launches:
+                launch()
+
+        host, wall = host_and_wall(eager, 5)
+        host_row("64 buckets x (EF quant-pack 8 chunks + W=8 shard reduce), eager pre-bound launches, per bucket",
+                 host / count, wall / count)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+            eager()
+        host, wall = host_and_wall(lambda i: graph.replay(), 5)
+        host_row("the same sequence as one HIP-graph replay, per bucket", host / count, wall / count)
+        del grads, residuals, launches, graph
+
     print(f"\n{'cfg':>3} {'us':>10} {'GB/s alg.':>10} {'% of 8TB/s':>10} {'input GB/s':>10}  parity / op", file=sys.stderr)
     for r in rows_out:
+        if "host_us" in r:
+            print(f"{r['config']:>3} {r['us']:10.2f} {'host us':>10} {r['host_us']:10.2f} {'':>10}  {r['op']}", file=sys.stderr)
+            continue
         print(f"{r['config']:>3} {r['us']:10.2f} {r['achieved_GBps']:10.1f} {r['frac_of_hbm_peak'] * 100:10.1f} "
               f"{r['input_GBps']:10.1f}  [{r['parity']}] {r['op']}", file=sys.stderr)
     return 0
