@@ -200,8 +200,11 @@ def _stored_bits(x: np.ndarray, dtype: str) -> np.ndarray:
 
 
 def quantize(x: np.ndarray, dtype: str, group_size: int = 64, bit: int = 8, quant_type: str = "linear",
-             topk: int = 0, stochastic: tuple[int, int] | None = None, compact: bool = False) -> np.ndarray:
-    """``stochastic`` is the generator's (seed, offset) pair, None for round-to-nearest."""
+             topk: int = 0, stochastic: tuple[int, int] | None = None, compact: bool = False,
+             first_group: int = 0) -> np.ndarray:
+    """``stochastic`` is the generator's (seed, offset) pair, None for round-to-nearest.  ``first_group`` restates a
+    window of a larger tensor: the index of the window's first group there (it fixes the 16-bit scan start and the
+    Philox subsequence of every group; the appended layout of a window is the window's own)."""
     if quant_type not in QUANT_TYPES or bit not in (4, 8) or (quant_type != "linear" and bit != 4):
         raise ValueError((quant_type, bit))
     item = _ITEMSIZE[dtype]
@@ -213,7 +216,7 @@ def quantize(x: np.ndarray, dtype: str, group_size: int = 64, bit: int = 8, quan
         return np.empty(0, dtype=np.uint8)
     rows_bits = bits.reshape(groups, group_size)
     rows = _bits_to_f32(bits, dtype).reshape(groups, group_size).copy()
-    group_index = np.arange(groups, dtype=np.int64)
+    group_index = np.arange(groups, dtype=np.int64) + int(first_group)
     start = scan_start(group_index, group_size, dtype)
     scale_bits, index1, index2, top1_bits, top2_bits = _scale_and_topk(rows_bits, rows, start, dtype, topk)
 

@@ -343,6 +343,53 @@ def test_full_bucket_stochastic_rounding_is_unbiased_and_repeatable(hip, hip_dev
          "codes of the first 1024 groups")
 
 
+def test_more_than_2_to_the_31_elements_in_the_cuda_byte_format(hip, hip_device):
+    """64-bit indexing in the pack, decode and general kernels: a 4.3 GB bf16 tensor of whole groups; windows at the
+    start, across the 2^31 boundary and at the end are compared with the oracle.  Payload offsets pass 2^31 bytes
+    too (2.2 GB interleaved, and the appended metadata of the general layout sits behind 2.1 GB of codes)."""
+    g = 64
+    n = (1 << 31) + g * 1024
+    x = torch.empty(n, dtype=torch.bfloat16, device=hip_device)
+    step = 1 << 28
+    for i, a in enumerate(range(0, n, step)):
+        b = min(a + step, n)
+        gen = torch.Generator(device=hip_device).manual_seed(777 + i)
+        x[a:b] = (torch.randn(b - a, generator=gen, device=hip_device) * 1e-3).to(torch.bfloat16)
+    windows = [(0, 1 << 18), ((1 << 31) - g * 2048, (1 << 31) + g * 512), (n - g * 1024, n)]
+    restored = torch.empty_like(x)
+
+    def check(payload, per_group_bytes, make_window_payload, decode_window, what):
+        for a, b in windows:
+            first, groups = a // g, (b - a) // g
+            # 16-bit scans start at an element that depends on the group index modulo 32: keep windows aligned to it
+            assert first % 32 == 0
+            piece = to_numpy(x[a:b])
+            want = make_window_payload(piece)
+            got = payload[first * per_group_bytes:(first + groups) * per_group_bytes]
+            same(got, want, f"{what} payload window {a}")
+            same(restored[a:b], decode_window(want, b - a), f"{what} decoded window {a}")
+
+    # plain linear 8-bit, interleaved scales: the dedicated pack and decode kernels
+    payload = hip.quant_pack(x, group_size=g, compact=True)
+    assert hip.dequant_into(payload, restored, group_size=g, compact=True)
+    check(payload, g + 2, lambda piece: general.quantize_pack(piece, "bf16", g, True, None, 8),
+          lambda want, count: wire.dequantize(want, count, "bf16", g, True), "pack kernel")
+    del payload
+    # top-2 outliers with stochastic rounding, interleaved metadata: the general kernels
+    policy = dict(group_size=g, bit=8, quant_type="linear", topk=2, compact=True)
+    payload = torch.empty(hip.general_payload_nbytes(n, x.dtype, g, 8, 2), dtype=torch.uint8, device=hip_device)
+    seeds = (99, 1 << 33)
+    assert hip.quant_general_into(x, payload, stochastic=seeds, **policy)
+    assert hip.dequant_general_into(payload, restored, **policy)
+
+    per_group = g + 4 * 2
+    for a, b in windows:
+        first, groups = a // g, (b - a) // g
+        want = general.quantize(to_numpy(x[a:b]), "bf16", g, 8, "linear", 2, seeds, True, first_group=first)
+        same(payload[first * per_group:(first + groups) * per_group], want, f"general payload window {a}")
+        same(restored[a:b], general.dequantize(want, b - a, "bf16", g, 8, "linear", 2, True), f"general decoded window {a}")
+
+
 @pytest.mark.parametrize("quant_type", ("normal", "e2m1"))
 def test_full_bucket_code_book_decode_is_the_nearest_entry(hip, hip_device, quant_type):
     gen = torch.Generator(device=hip_device).manual_seed(5)
