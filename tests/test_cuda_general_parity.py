@@ -374,7 +374,12 @@ def test_more_than_2_to_the_31_elements_in_the_cuda_byte_format(hip, hip_device)
     assert hip.dequant_into(payload, restored, group_size=g, compact=True)
     check(payload, g + 2, lambda piece: general.quantize_pack(piece, "bf16", g, True, None, 8),
           lambda want, count: wire.dequantize(want, count, "bf16", g, True), "pack kernel")
-    del payload
+    # the fused reduce of the payload with itself is exactly twice the single decode (a power-of-two scaling)
+    doubled = torch.empty_like(x)
+    assert hip.dequant_reduce_into([payload, payload], doubled, group_size=g, compact=True)
+    for a, b in windows:
+        assert torch.equal(doubled[a:b], restored[a:b] * 2), f"reduce window {a}"
+    del payload, doubled
     # top-2 outliers with stochastic rounding, interleaved metadata: the general kernels
     policy = dict(group_size=g, bit=8, quant_type="linear", topk=2, compact=True)
     payload = torch.empty(hip.general_payload_nbytes(n, x.dtype, g, 8, 2), dtype=torch.uint8, device=hip_device)
