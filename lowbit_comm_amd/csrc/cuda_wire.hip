@@ -57,7 +57,7 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
     const T *__restrict__ r = HAS_R ? static_cast<const T *>(a.residual) + chunk_start : nullptr;
     uint8_t *__restrict__ payload = a.payloads + chunk * a.payload_stride;
 
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block()) * BLOCK_ELEMS;
+    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(BLOCK_ELEMS)) * BLOCK_ELEMS;
     if (block_first >= padded) return;
 
     using Raw = typename raw_bits<T>::type;
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(kBlock) void wire_reduce_kernel(const WireReduceArg
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block()) * BLOCK_ELEMS;
+    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(BLOCK_ELEMS)) * BLOCK_ELEMS;
     const int64_t groups = (a.numel + G - 1) / G;
     const group_layout<T, G, COMPACT> at{groups};
     T *__restrict__ out = static_cast<T *>(a.out);
@@ -383,7 +383,7 @@ __global__ __launch_bounds__(kBlock) void wire_decode_kernel(const WireDecodeArg
     const group_layout<T, G, COMPACT, BIT> at{groups};
     const uint8_t *__restrict__ payload = a.payloads + chunk * a.payload_stride;
     T *__restrict__ out = static_cast<T *>(a.out) + chunk_start;
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block()) * BLOCK_ELEMS;
+    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(BLOCK_ELEMS)) * BLOCK_ELEMS;
     if (block_first >= valid) return;
 
     if (block_first + BLOCK_ELEMS <= valid) {

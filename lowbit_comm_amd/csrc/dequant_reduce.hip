@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block()) * T::BLOCK_ELEMS;
+    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(T::BLOCK_ELEMS)) * T::BLOCK_ELEMS;
     OT *__restrict__ out = static_cast<OT *>(a.out);
     const OT *prepared = static_cast<const OT *>(a.prepared);  // may alias new_r
     OT *new_r = static_cast<OT *>(a.new_residual);
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_quant_kernel(const Redu
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int64_t padded = (a.numel + G - 1) / G * G;
-    const int64_t e0 = static_cast<int64_t>(xcd_contiguous_block()) * BLOCK_ELEMS + static_cast<int64_t>(wave) * TILE + lane * VEC;
+    const int64_t e0 = static_cast<int64_t>(xcd_contiguous_block(BLOCK_ELEMS)) * BLOCK_ELEMS + static_cast<int64_t>(wave) * TILE + lane * VEC;
     const bool live = e0 < padded;     // whole lanes: padded and e0 are multiples of VEC
     const bool mean = a.divisor != 1.0f;
 
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
     const int8_t *__restrict__ codes = reinterpret_cast<const int8_t *>(a.codes_base + chunk * a.payload_stride);
     const float *__restrict__ scales = reinterpret_cast<const float *>(a.scales_base + chunk * a.payload_stride);
     OT *__restrict__ out = static_cast<OT *>(a.out) + chunk_start;
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block()) * T::BLOCK_ELEMS;
+    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(T::BLOCK_ELEMS)) * T::BLOCK_ELEMS;
     if (block_first >= valid) return;
 
     if (MODE != kScalar && block_first + T::BLOCK_ELEMS <= valid) {
@@ -416,7 +416,7 @@ __global__ __launch_bounds__(kBlock) void ef_update_kernel(const EfArgs a) {
     const PT *__restrict__ prepared = static_cast<const PT *>(a.prepared);
     const TT *__restrict__ restored = static_cast<const TT *>(a.restored);
     RT *__restrict__ residual = static_cast<RT *>(a.residual);
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block()) * BLOCK_ELEMS;
+    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(BLOCK_ELEMS)) * BLOCK_ELEMS;
     if (MODE != kScalar && block_first + BLOCK_ELEMS <= a.numel) {
         PT pv[UNROLL][VEC];
         TT tv[UNROLL][VEC];

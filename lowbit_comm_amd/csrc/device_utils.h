@@ -27,17 +27,18 @@ constexpr int kWavesPerBlock = kBlock / kWave;
 template <int UNROLL> __device__ __forceinline__ int tile_in_block(int u, int wave) {
     return LBC_TILE_ORDER == 0 ? u * kWavesPerBlock + wave : wave * UNROLL + u;
 }
-// Workgroups of a grid are dealt round-robin to the chip's 8 XCDs.  For grids of up to a few thousand workgroups
-// (shard-sized reduces, per-chunk rows of the chunked quantize) it measured 3-7 % faster to let every XCD walk one
-// contiguous eighth of the x range; for larger grids the round-robin order, which keeps all XCDs on one moving
-// front of addresses, measured 5-12 % faster, so those keep it.  The remainder of a grid that is not a multiple of
-// 8 keeps its place.
-#ifndef LBC_XCD_REMAP_MAX_BLOCKS
-#define LBC_XCD_REMAP_MAX_BLOCKS 4096
+// Workgroups of a grid are dealt round-robin to the chip's 8 XCDs.  When the x range of a launch covers at most
+// LBC_XCD_SPAN_ELEMS elements (shard-sized reduces, per-chunk rows of the chunked quantize: an eighth of the range
+// is then no more than a 2 MiB page of the widest tensor), letting every XCD walk one contiguous eighth measured
+// up to 7 % faster and never slower; for larger ranges the round-robin order, which keeps all XCDs on one moving front of addresses and
+// pages, measured 5-12 % faster, so those keep it.  The remainder of a grid that is not a multiple of 8 keeps its
+// place.
+#ifndef LBC_XCD_SPAN_ELEMS
+#define LBC_XCD_SPAN_ELEMS (1 << 22)
 #endif
-__device__ __forceinline__ unsigned xcd_contiguous_block() {
+__device__ __forceinline__ unsigned xcd_contiguous_block(int block_elems) {
     const unsigned per_xcd = gridDim.x >> 3;
-    const bool remap = gridDim.x <= LBC_XCD_REMAP_MAX_BLOCKS && blockIdx.x < (per_xcd << 3);
+    const bool remap = static_cast<int64_t>(gridDim.x) * block_elems <= LBC_XCD_SPAN_ELEMS && blockIdx.x < (per_xcd << 3);
     return remap ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
 }
 constexpr uint32_t kEpsBits = 0x34000000u;  // 2^-23, torch.finfo(float32).eps

@@ -66,7 +66,7 @@ __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
     NT *new_r = a.new_residual ? static_cast<NT *>(a.new_residual) + chunk_start : nullptr;
     DT *__restrict__ restored = a.restored ? static_cast<DT *>(a.restored) + chunk_start : nullptr;
 
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block()) * T::BLOCK_ELEMS;
+    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(T::BLOCK_ELEMS)) * T::BLOCK_ELEMS;
     if (block_first >= padded) return;
 
     if (MODE != kScalar && block_first + T::BLOCK_ELEMS <= valid) {
