@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define LBC_ABI_VERSION 4
+#define LBC_ABI_VERSION 5
 
 enum { LBC_OK = 0, LBC_UNSUPPORTED = 1, LBC_EINVAL = -1, LBC_ELAUNCH = -2 };
 
@@ -167,6 +167,26 @@ int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int worl
 int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *scales, int world,
                              int64_t numel, int group_size, float divisor, int mid_dtype,
                              int8_t *out_codes, float *out_scales, void *stream);
+
+/*
+ * One compute step of the quantized ring all-reduce on one chunk of the bucket, in place:
+ *   chunk[i] = decode(received)[i]                      reduce_op LBC_REDUCE_NONE
+ *   chunk[i] = chunk[i] + decode(received)[i]           reduce_op LBC_REDUCE_SUM (in `dtype` arithmetic)
+ *   chunk[i] = chunk[i] / divisor                       when divisor != 1 (true division)
+ * and, when send_codes and send_scales are given, quantize+pack of the updated chunk exactly as
+ * lbc_quant_pack would, without reading it back from memory.  Replaces, in one launch,
+ * TorchPipelinedRingRuntime.fused_reduce / apply_broadcast (ccdl_comm/cuda/transports/
+ * torch_topology.py:262-316: dequantize with reduce_op sum / none, div_ by the world size at the
+ * last reduce step) followed by the quant_pack of the same chunk that the ring schedule issues
+ * next (ccdl_comm/cuda/transports/pipelined_ring.py:221-225,250-254; the chunk a step receives
+ * into is the chunk the next step sends, :304-311,325-330).  Results are bit-identical to
+ * lbc_dequant + division + lbc_quant_pack.  recv_codes holds ceil(numel/g)*g codes, recv_scales
+ * ceil(numel/g) floats; the send buffers have the same sizes and may not alias the received
+ * ones.  Other reduce ops: LBC_UNSUPPORTED.
+ */
+int lbc_ring_step(const int8_t *recv_codes, const float *recv_scales, void *chunk, int dtype,
+                  int64_t numel, int group_size, int reduce_op, float divisor, int8_t *send_codes,
+                  float *send_scales, void *stream);
 
 /*
  * residual = prepared - restored, element-wise, subtraction in fp32, rounded to

@@ -59,6 +59,16 @@ struct EfArgs {
     int64_t numel;
 };
 
+struct RingStepArgs {
+    const int8_t *recv_codes;   // padded: ceil(numel/g)*g codes of the payload that arrived
+    const float *recv_scales;
+    void *chunk;                // numel elements, updated in place
+    int8_t *send_codes;         // null together with send_scales: no payload is produced
+    float *send_scales;
+    int64_t numel;
+    float divisor;              // 1 = no division
+};
+
 // ---- payload format of the reference's CUDA extension (cuda_wire.hip) ----------
 struct WireQuantArgs {
     const void *x;
@@ -128,6 +138,9 @@ hipError_t launch_dequant_reduce_quant(int mid_dtype, int group_size, int world,
                                        const ReduceQuantArgs &args, hipStream_t stream);
 hipError_t launch_decode(int out_dtype, int group_size, int reduce_op, int mode,
                          const DecodeArgs &args, int world, hipStream_t stream);
+// chunk (op)= decode(received) [/ divisor], then quantize+pack of the updated chunk.
+hipError_t launch_ring_step(int dtype, int group_size, bool accumulate, int mode, const RingStepArgs &args,
+                            hipStream_t stream);
 hipError_t launch_ef_update(int p_dtype, int t_dtype, int r_dtype, int mode, const EfArgs &args,
                             hipStream_t stream);
 

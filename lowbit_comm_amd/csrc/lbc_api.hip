@@ -303,6 +303,34 @@ int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *sca
                   "lbc_dequant_reduce_quant");
 }
 
+int lbc_ring_step(const int8_t *recv_codes, const float *recv_scales, void *chunk, int dtype, int64_t numel,
+                  int group_size, int reduce_op, float divisor, int8_t *send_codes, float *send_scales, void *stream) {
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported chunk dtype %d", dtype);
+    if (reduce_op < LBC_REDUCE_NONE || reduce_op > LBC_REDUCE_MIN) return fail(LBC_EINVAL, "unknown reduce op %d", reduce_op);
+    if (!(divisor > 0.0f)) return fail(LBC_EINVAL, "divisor must be > 0");
+    if ((send_codes == nullptr) != (send_scales == nullptr))
+        return fail(LBC_EINVAL, "send codes and send scales must be given together");
+    if (!valid_group(group_size)) return LBC_UNSUPPORTED;
+    if (reduce_op != LBC_REDUCE_NONE && reduce_op != LBC_REDUCE_SUM) return LBC_UNSUPPORTED;
+    if (numel == 0) return LBC_OK;
+    if (recv_codes == nullptr || recv_scales == nullptr) return fail(LBC_EINVAL, "received codes and scales must not be null");
+    if (chunk == nullptr) return fail(LBC_EINVAL, "chunk must not be null");
+    if (!aligned_to(chunk, dtype_size(dtype))) return fail(LBC_EINVAL, "chunk is not aligned to its element size");
+    if (!aligned_to(recv_scales, 4) || (send_scales != nullptr && !aligned_to(send_scales, 4)))
+        return fail(LBC_EINVAL, "scales must be 4-byte aligned");
+    if (send_codes == recv_codes || send_scales == recv_scales)
+        return fail(LBC_EINVAL, "the payload to send must not alias the received one");
+    const int vec = 16 / dtype_size(dtype);   // elements, and code bytes, one lane owns
+    const bool aligned = aligned_to(chunk, 16) && aligned_to(recv_codes, vec) &&
+                         (send_codes == nullptr || aligned_to(send_codes, vec));
+    const int64_t moved = numel * ((reduce_op == LBC_REDUCE_SUM ? 2 : 1) * dtype_size(dtype) + (send_codes ? 2 : 1));
+    lbc::RingStepArgs a{recv_codes, recv_scales, chunk, send_codes, send_scales, numel, divisor};
+    return finish(lbc::launch_ring_step(dtype, group_size, reduce_op == LBC_REDUCE_SUM, pick_mode(aligned, moved), a,
+                                        static_cast<hipStream_t>(stream)),
+                  "lbc_ring_step");
+}
+
 int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored, int restored_dtype,
                   void *residual, int residual_dtype, int64_t numel, void *stream) {
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");

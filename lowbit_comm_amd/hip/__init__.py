@@ -1,6 +1,17 @@
 """HIP (gfx950) backend: C-ABI binding, tensor-level ops, native-module shim, codec callables, workspace pool."""
 from .completion import HipCompletionManager, HipStreamWork
 from .loader import CudaExtensionStatus, HipExtensionStatus, load_cuda_extension, load_hip_extension
+from .ring import (
+    HipPipelinedRingRuntime,
+    JoinedCompletion,
+    LoopbackRing,
+    PipelinedRingExecutor,
+    PipelinedRingSchedule,
+    RingAllGatherStep,
+    RingReduceScatterStep,
+    compile_pipelined_ring_schedule,
+    make_pipelined_ring_executor,
+)
 from .workspace import (
     CudaOutputLease,
     CudaShardWorkspaceProvider,
@@ -21,7 +32,9 @@ from .workspace import (
 __all__ = [
     "CudaExtensionStatus", "CudaOutputLease", "CudaShardWorkspaceProvider", "CudaShardWorkspaceSession",
     "CudaWorkspacePool", "EventCompletion", "EventCompletionManager", "HipCompletionManager", "HipExtensionStatus",
-    "HipOutputLease", "HipStreamWork",
+    "HipOutputLease", "HipPipelinedRingRuntime", "HipStreamWork", "JoinedCompletion", "LoopbackRing",
+    "PipelinedRingExecutor", "PipelinedRingSchedule", "RingAllGatherStep", "RingReduceScatterStep",
+    "compile_pipelined_ring_schedule", "make_pipelined_ring_executor",
     "HipWorkspacePool", "ShardWorkspaceProvider", "ShardWorkspaceSession", "WorkspaceKey", "WorkspaceLease",
     "WorkspaceStats", "create_torch_workspace_pool", "load_cuda_extension", "load_hip_extension",
 ]

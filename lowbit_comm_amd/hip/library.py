@@ -11,7 +11,7 @@ from pathlib import Path
 from lowbit_comm_amd.exceptions import CCDLUnavailableError
 
 LIBRARY_PATH = Path(__file__).resolve().parent.parent / "liblbc_hip.so"
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 LBC_OK = 0
 LBC_UNSUPPORTED = 1
@@ -35,6 +35,8 @@ SIGNATURES = {
                                     _c_ptr, _c_ptr, _c_ptr]),
     "lbc_dequant_reduce_quant": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_int, _c_ptr,
                                           _c_ptr, _c_ptr]),
+    "lbc_ring_step": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, ctypes.c_float, _c_ptr, _c_ptr,
+                               _c_ptr]),
     "lbc_ef_update": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr]),
     "lbc_wire_payload_nbytes": (_c_i64, [_c_i64, _c_int, _c_int, _c_int]),
     "lbc_wire_quant_pack": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),

@@ -456,6 +456,35 @@ def dequant_reduce_quant_into(payloads: Sequence[tuple[torch.Tensor, torch.Tenso
     return False if bound is None else bound()
 
 
+# --------------------------------------------------------------------------- #
+# ring step: chunk (op)= decode(received) [/ divisor], then quantize+pack of the updated chunk
+# --------------------------------------------------------------------------- #
+def bind_ring_step(received: torch.Tensor, chunk: torch.Tensor, send: torch.Tensor | None = None, *,
+                   group_size: int = 64, reduce_op: str = "sum", divisor: float = 1.0) -> BoundLaunch:
+    """``received`` and ``send`` are packed ``uint8[codes || scales]`` payloads covering ``chunk.numel()``
+    elements; ``chunk`` is updated in place and, when ``send`` is given, quantized into it in the same launch."""
+    lib = load_library()
+    code = _float_tensor(chunk, "chunk")
+    device = chunk.device
+    n = chunk.numel()
+    _require(reduce_op in REDUCE_OPS, f"unsupported reduce op {reduce_op!r}")
+    _require(float(divisor) > 0.0, "divisor must be > 0")
+    recv_codes, recv_scales = payload_addresses(received, n, group_size, name="received payload", device=device)
+    send_codes = send_scales = None
+    if send is not None:
+        send_codes, send_scales = payload_addresses(send, n, group_size, name="send payload", device=device)
+        _require(n == 0 or send.data_ptr() != received.data_ptr(), "the payload to send must not alias the received one")
+    args = (ctypes.c_void_p(recv_codes), ctypes.c_void_p(recv_scales), _ptr(chunk), code, n, group_size,
+            REDUCE_OPS[reduce_op], float(divisor),
+            None if send is None else ctypes.c_void_p(send_codes), None if send is None else ctypes.c_void_p(send_scales))
+    return BoundLaunch(lib.lbc_ring_step, args, device, lib, (received, chunk, send))
+
+
+def ring_step_into(received: torch.Tensor, chunk: torch.Tensor, send: torch.Tensor | None = None, *,
+                   group_size: int = 64, reduce_op: str = "sum", divisor: float = 1.0) -> bool:
+    return bind_ring_step(received, chunk, send, group_size=group_size, reduce_op=reduce_op, divisor=divisor)()
+
+
 def ef_update_into(prepared: torch.Tensor, restored: torch.Tensor, residual: torch.Tensor) -> bool:
     """``residual = prepared - restored`` (fp32 subtraction, rounded to the residual's dtype)."""
     lib = load_library()

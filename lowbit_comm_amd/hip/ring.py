@@ -1,0 +1,636 @@
+"""Quantized ring all-reduce: compiled per-rank schedule, executor and the gfx950 runtime of its compute steps.
+
+Counterparts in the reference: the schedule types and ``compile_pipelined_ring_schedule``
+(``ccdl_comm/cuda/transports/pipelined_ring.py:19-110,285-331``), ``PipelinedRingExecutor`` (``:174-282``) with the
+ownership rules of ``ccdl_comm/cuda/transports/_executor_support.py``, and ``TorchPipelinedRingRuntime``
+(``ccdl_comm/cuda/transports/torch_topology.py:67-316``).
+
+A ring over W ranks moves every chunk of the bucket W-1 hops while it is summed (reduce-scatter) and W-1 hops while
+the mean is handed round (all-gather).  One rule generates the whole schedule: a rank always sends the chunk it has
+just received into, starting with its predecessor's chunk index, so that after W-1 steps rank r holds the complete
+chunk r.  The reference runs "decode into the chunk" and "quantize the chunk for the next hop" as separate kernels;
+the runtime here issues them as one launch of the ring-step kernel (``lbc_ring_step``), which quantizes the updated
+chunk while it is still in registers, and hands the staged payload to the next ``quant_pack`` call.  The point-to-point
+exchange itself is injected: ``exchange(payload, received, send_peer=, recv_peer=, stream=) -> handle``.
+"""
+from __future__ import annotations
+
+import threading
+from dataclasses import dataclass, field
+from typing import Any, Callable
+
+from lowbit_comm_amd.config import CompressionConfig
+from lowbit_comm_amd.hip.chunk_plan import ChunkPlan, ChunkRange, compile_chunk_plan
+
+# --------------------------------------------------------------------------- #
+# schedule
+# --------------------------------------------------------------------------- #
+_STEP_INTEGERS = ("step_index", "send_peer", "recv_peer", "send_chunk_owner", "recv_chunk_owner")
+
+
+def _natural(value: object, name: str) -> None:
+    if isinstance(value, bool) or not isinstance(value, int):
+        raise TypeError(f"{name} must be an integer")
+    if value < 0:
+        raise ValueError(f"{name} must be >= 0")
+
+
+def _rank_of(value: object, world_size: int, name: str) -> None:
+    _natural(value, name)
+    if value >= world_size:
+        raise ValueError(f"{name} must be in [0, {world_size})")
+
+
+def _check_step(step: Any) -> None:
+    for name in _STEP_INTEGERS:
+        _natural(getattr(step, name), name)
+    for name in ("send_chunk", "recv_chunk"):
+        if not isinstance(getattr(step, name), ChunkRange):
+            raise TypeError(f"{name} must be a ChunkRange")
+
+
+@dataclass(frozen=True)
+class RingReduceScatterStep:
+    """One hop of the summing phase.  ``received_contributors``: the ranks whose data the arriving payload already
+    sums, oldest first; its length is ``step_index + 1``."""
+
+    step_index: int
+    send_peer: int
+    recv_peer: int
+    send_chunk_owner: int
+    recv_chunk_owner: int
+    received_contributors: tuple[int, ...]
+    send_chunk: ChunkRange
+    recv_chunk: ChunkRange
+
+    def __post_init__(self) -> None:
+        _check_step(self)
+        ranks = self.received_contributors
+        if not isinstance(ranks, tuple):
+            raise TypeError("received_contributors must be a tuple")
+        if not ranks:
+            raise ValueError("received_contributors must not be empty")
+        for entry in ranks:
+            _natural(entry, "received_contributors entry")
+        if len(set(ranks)) != len(ranks):
+            raise ValueError("received_contributors must not contain duplicates")
+        if len(ranks) != self.step_index + 1:
+            raise ValueError("received_contributors length must equal step_index + 1")
+
+
+@dataclass(frozen=True)
+class RingAllGatherStep:
+    """One hop of the phase that hands the reduced chunks round."""
+
+    step_index: int
+    send_peer: int
+    recv_peer: int
+    send_chunk_owner: int
+    recv_chunk_owner: int
+    send_chunk: ChunkRange
+    recv_chunk: ChunkRange
+
+    def __post_init__(self) -> None:
+        _check_step(self)
+
+
+def _hops(world_size: int, first_sent: int):
+    """``(step, sent chunk, received chunk)``: what is received is what the predecessor sent, one index lower,
+    and it is what goes out next."""
+    sent = first_sent
+    for step in range(world_size - 1):
+        received = (sent - 1) % world_size
+        yield step, sent, received
+        sent = received
+
+
+def _reduce_steps(plan: ChunkPlan, rank: int) -> tuple[RingReduceScatterStep, ...]:
+    world = plan.world_size
+    after, before = (rank + 1) % world, (rank - 1) % world
+    return tuple(
+        RingReduceScatterStep(step_index=step, send_peer=after, recv_peer=before, send_chunk_owner=sent,
+                              recv_chunk_owner=received,
+                              received_contributors=tuple((before - back) % world for back in range(step, -1, -1)),
+                              send_chunk=plan.chunk_for_rank(sent), recv_chunk=plan.chunk_for_rank(received))
+        for step, sent, received in _hops(world, before))
+
+
+def _gather_steps(plan: ChunkPlan, rank: int) -> tuple[RingAllGatherStep, ...]:
+    world = plan.world_size
+    after, before = (rank + 1) % world, (rank - 1) % world
+    return tuple(
+        RingAllGatherStep(step_index=step, send_peer=after, recv_peer=before, send_chunk_owner=sent,
+                          recv_chunk_owner=received, send_chunk=plan.chunk_for_rank(sent),
+                          recv_chunk=plan.chunk_for_rank(received))
+        for step, sent, received in _hops(world, rank))
+
+
+@dataclass(frozen=True)
+class PipelinedRingSchedule:
+    """The steps of one rank, bound to an immutable chunk plan; only the deterministic schedule is accepted."""
+
+    chunk_plan: ChunkPlan
+    rank: int
+    steps: tuple[RingReduceScatterStep, ...]
+    gather_steps: tuple[RingAllGatherStep, ...]
+
+    def __post_init__(self) -> None:
+        if not isinstance(self.chunk_plan, ChunkPlan):
+            raise TypeError("chunk_plan must be a ChunkPlan")
+        _rank_of(self.rank, self.chunk_plan.world_size, "rank")
+        if self.steps != _reduce_steps(self.chunk_plan, self.rank):
+            raise ValueError("steps must match the deterministic ring schedule")
+        if self.gather_steps != _gather_steps(self.chunk_plan, self.rank):
+            raise ValueError("gather_steps must match the deterministic ring schedule")
+
+    @property
+    def local_chunk(self) -> ChunkRange:
+        """The chunk this rank holds completely reduced after the first phase."""
+        return self.chunk_plan.chunk_for_rank(self.rank)
+
+
+def compile_pipelined_ring_schedule(*, chunk_plan: ChunkPlan, rank: int) -> PipelinedRingSchedule:
+    if not isinstance(chunk_plan, ChunkPlan):
+        raise TypeError("chunk_plan must be a ChunkPlan")
+    _rank_of(rank, chunk_plan.world_size, "rank")
+    return PipelinedRingSchedule(chunk_plan=chunk_plan, rank=rank, steps=_reduce_steps(chunk_plan, rank),
+                                 gather_steps=_gather_steps(chunk_plan, rank))
+
+
+# --------------------------------------------------------------------------- #
+# completion plumbing shared by the executor
+# --------------------------------------------------------------------------- #
+def _probe(value: Any) -> Callable[[], Any] | None:
+    for name in ("query", "is_completed"):
+        method = getattr(value, name, None)
+        if callable(method):
+            return method
+    return None
+
+
+def _require_endpoint(value: Any, name: str) -> None:
+    if _probe(value) is None:
+        raise TypeError(f"{name} must provide nonblocking query() or is_completed()")
+    for method in ("wait", "wait_stream"):
+        if not callable(getattr(value, method, None)):
+            raise TypeError(f"{name} must provide {method}()")
+
+
+@dataclass(frozen=True)
+class JoinedCompletion:
+    """Ready when the submission context (the producer of the tensor) and the runtime's recorded end both are."""
+
+    context: Any
+    runtime_completion: Any
+
+    def __post_init__(self) -> None:
+        _require_endpoint(self.context, "submission context")
+        _require_endpoint(self.runtime_completion, "runtime completion")
+
+    def query(self) -> bool:
+        return bool(_probe(self.context)()) and bool(_probe(self.runtime_completion)())
+
+    def is_completed(self) -> bool:
+        return self.query()
+
+    def wait(self) -> None:
+        self.context.wait()
+        self.runtime_completion.wait()
+
+    def wait_stream(self, stream: Any) -> None:
+        self.context.wait_stream(stream)
+        self.runtime_completion.wait_stream(stream)
+
+
+@dataclass(eq=False)
+class _Submission:
+    """Everything one ``run()`` holds on to until the device has finished with it."""
+
+    tensor: Any
+    workspace: Any
+    context: Any
+    resources: list = field(default_factory=list)
+    dependencies: list = field(default_factory=list)
+    completion: Any = None
+    record_attempted: bool = False
+    failed: bool = False
+    settled: bool = False          # workspace released or aborted
+
+    def __post_init__(self) -> None:
+        self.resources += [self.tensor, self.workspace, self.context]
+
+    def keep(self, *values: Any) -> None:
+        self.resources += [v for v in values if v is not None]
+
+    def after(self, value: Any) -> None:
+        if value is not None:
+            self.dependencies.append(value)
+            self.keep(value)
+
+    def after_p2p(self, value: Any) -> None:
+        self.keep(value)
+        if _probe(value) is None:
+            raise TypeError("P2P dependency must provide nonblocking query() or is_completed()")
+        self.dependencies.append(value)
+
+    def keep_workspace_buffers(self) -> None:
+        leases = getattr(self.workspace, "leases", ())
+        if isinstance(leases, tuple):
+            self.keep(*leases)
+
+
+class PipelinedRingExecutor:
+    """Enqueues the whole schedule of one rank without waiting on the host and returns completion-backed work.
+
+    ``runtime`` provides ``create_submission_context``, ``wait_for_producer``, ``quant_pack``, ``send_recv``,
+    ``fused_reduce``, ``apply_broadcast`` and ``record_completion`` (the protocol of pipelined_ring.py:113-171);
+    ``workspace_session_factory(tensor)`` a session with ``release(completion=)`` and optionally ``abort()``;
+    ``completion_manager.create_work(result=, completion=, resources=)`` the work object.  A submission that fails
+    after device work was enqueued keeps its buffers until that work has drained (``reap_pending``), then aborts
+    the session instead of releasing it."""
+
+    def __init__(self, *, schedule: PipelinedRingSchedule, runtime: Any,
+                 workspace_session_factory: Callable[[Any], Any], completion_manager: Any) -> None:
+        if not isinstance(schedule, PipelinedRingSchedule):
+            raise TypeError("schedule must be a PipelinedRingSchedule")
+        if not callable(workspace_session_factory):
+            raise TypeError("workspace_session_factory must be callable")
+        self.schedule = schedule
+        self._runtime = runtime
+        self._sessions = workspace_session_factory
+        self._works = completion_manager
+        self._pending: list[_Submission] = []
+        self._busy = threading.Lock()
+
+    @property
+    def pending_submission_count(self) -> int:
+        return len(self._pending)
+
+    def reap_pending(self) -> None:
+        if not self._busy.acquire(blocking=False):
+            raise RuntimeError("cannot reap while topology submission is in progress")
+        try:
+            self._reap()
+        finally:
+            self._busy.release()
+
+    def run(self, tensor: Any) -> Any:
+        if not self._busy.acquire(blocking=False):
+            raise RuntimeError("concurrent run() on one topology executor is unsupported")
+        try:
+            return self._submit(tensor)
+        finally:
+            self._busy.release()
+
+    # ---- one submission ---------------------------------------------------- #
+    def _submit(self, tensor: Any) -> Any:
+        self._reap()
+        runtime = self._runtime
+        context = runtime.create_submission_context(tensor)
+        _require_endpoint(context, "submission context")
+        submission = _Submission(tensor=tensor, workspace=self._sessions(tensor), context=context)
+        try:
+            workspace = submission.workspace
+            runtime.wait_for_producer(tensor, context=context)
+            for step in self.schedule.steps:
+                received, handle = self._exchange(submission, step)
+                submission.after(runtime.fused_reduce(tensor, received, step.recv_chunk, step.received_contributors,
+                                                      workspace, context=context, dependency=handle))
+            for step in self.schedule.gather_steps:
+                received, handle = self._exchange(submission, step)
+                submission.after(runtime.apply_broadcast(tensor, received, step.recv_chunk, workspace,
+                                                         context=context, dependency=handle))
+            self._record(submission)
+            return self._finish(submission)
+        except BaseException:
+            self._fail(submission)
+            raise
+
+    def _exchange(self, submission: _Submission, step: Any) -> tuple[Any, Any]:
+        runtime, context, workspace = self._runtime, submission.context, submission.workspace
+        payload = runtime.quant_pack(submission.tensor, step.send_chunk, workspace, context=context)
+        submission.keep(payload)
+        received, handle = runtime.send_recv(payload, send_peer=step.send_peer, recv_peer=step.recv_peer,
+                                             recv_chunk=step.recv_chunk, workspace=workspace, context=context)
+        submission.keep(received)
+        submission.after_p2p(handle)
+        return received, handle
+
+    def _record(self, submission: _Submission) -> None:
+        submission.record_attempted = True
+        ended = self._runtime.record_completion(context=submission.context,
+                                                dependencies=tuple(submission.dependencies))
+        submission.keep(ended)
+        submission.completion = JoinedCompletion(submission.context, ended)
+        submission.keep(submission.completion)
+
+    def _finish(self, submission: _Submission) -> Any:
+        submission.keep_workspace_buffers()
+        self._hold(submission)
+        work = self._works.create_work(result=submission.tensor, completion=submission.completion,
+                                       resources=tuple(submission.resources))
+        submission.keep(work)
+        self._release(submission, submission.completion)
+        self._pending.remove(submission)
+        return work
+
+    def _fail(self, submission: _Submission) -> None:
+        submission.failed = True
+        submission.keep_workspace_buffers()
+        self._hold(submission)
+        if not submission.record_attempted:
+            try:
+                self._record(submission)      # so that there is something to wait for before the buffers go back
+            except BaseException:
+                pass
+
+    def _hold(self, submission: _Submission) -> None:
+        if submission not in self._pending:
+            self._pending.append(submission)
+
+    @staticmethod
+    def _release(submission: _Submission, completion: Any) -> None:
+        release = getattr(submission.workspace, "release", None)
+        if not callable(release):
+            raise TypeError("workspace session must provide release(completion=...)")
+        release(completion=completion)
+        submission.settled = True
+
+    def _reap(self) -> None:
+        for submission in tuple(self._pending):
+            readiness = submission.completion if submission.completion is not None else submission.context
+            probe = _probe(readiness)
+            try:
+                if probe is None or not probe():
+                    continue
+            except BaseException:
+                continue
+            if not submission.settled:
+                abort = getattr(submission.workspace, "abort", None)
+                try:
+                    if submission.failed and callable(abort):
+                        abort()
+                        submission.settled = True
+                    else:
+                        self._release(submission, readiness)
+                except BaseException:
+                    continue
+            self._pending.remove(submission)
+
+
+# --------------------------------------------------------------------------- #
+# gfx950 runtime of the compute steps
+# --------------------------------------------------------------------------- #
+@dataclass
+class RingSubmissionContext:
+    """Per-submission state; nothing mutable is shared between runs."""
+
+    tensor: Any
+    stream: Any
+    producer_completion: Any
+    quant_index: int = 0
+    recv_index: int = 0
+    mean_applied: bool = False
+    steps_done: int = 0
+    staged: tuple | None = None        # ((start, stop), payload) quantized by the previous step's launch
+
+    def query(self) -> bool:
+        return bool(self.producer_completion.query())
+
+    def wait(self) -> None:
+        self.producer_completion.wait()
+
+    def wait_stream(self, stream: Any) -> None:
+        self.producer_completion.wait_stream(stream)
+
+
+def _view(tensor: Any, chunk: ChunkRange) -> Any:
+    return tensor.reshape((-1,))[chunk.start:chunk.stop]
+
+
+class HipPipelinedRingRuntime:
+    """The coarse operations of the ring on one gfx950 device, for the portable INT8 payload
+    ``uint8[codes || fp32 scales]``.
+
+    ``fuse_steps=True`` (default): ``fused_reduce`` / ``apply_broadcast`` run the ring-step kernel, which also
+    quantizes the updated chunk into the send buffer of the next step; the following ``quant_pack`` of that chunk
+    returns the staged payload without a launch.  ``fuse_steps=False`` issues the reference's sequence (decode with
+    reduce op, in-place division, quantize) as separate launches; both give the same bits.  Unlike the reference's
+    native path, chunks need not be multiples of the group size."""
+
+    def __init__(self, *, config: CompressionConfig, dtype: str, world_size: int, rank: int,
+                 exchange: Callable[..., Any], completion_manager: Any | None = None, stream: Any | None = None,
+                 fuse_steps: bool = True) -> None:
+        from lowbit_comm_amd.hip.executors import fused_dequant_fallback_reason
+
+        reason = fused_dequant_fallback_reason(config)
+        if reason is not None:
+            raise ValueError(reason.replace("fused dequant", "the ring runtime"))
+        if dtype not in ("fp32", "fp16", "bf16"):
+            raise ValueError(f"unsupported dtype {dtype!r}")
+        if isinstance(world_size, bool) or not isinstance(world_size, int) or world_size <= 0:
+            raise ValueError("world_size must be a positive integer")
+        _rank_of(rank, world_size, "rank")
+        if not callable(exchange):
+            raise TypeError("exchange must be callable")
+        self.config = config
+        self.dtype = dtype
+        self.world_size = world_size
+        self.rank = rank
+        self.fuse_steps = bool(fuse_steps)
+        self._exchange = exchange
+        self._completions = completion_manager
+        self.stream = stream
+
+    # ---- context ----------------------------------------------------------- #
+    def _ready(self) -> None:
+        import torch
+
+        if self._completions is None:
+            from lowbit_comm_amd.hip.completion import HipCompletionManager
+
+            self._completions = HipCompletionManager()
+        if self.stream is None:
+            self.stream = torch.cuda.Stream()       # default priority
+
+    def create_submission_context(self, tensor: Any) -> RingSubmissionContext:
+        import torch
+
+        from lowbit_comm_amd.hip import ops
+
+        self._ready()
+        if not isinstance(tensor, torch.Tensor) or not tensor.is_cuda or not tensor.is_contiguous():
+            raise RuntimeError("the ring runs in place on a contiguous GPU tensor")
+        if ops.DTYPE_NAMES.get(tensor.dtype) != self.dtype:
+            raise RuntimeError(f"tensor dtype {tensor.dtype} does not match the runtime's {self.dtype}")
+        produced = self._completions.record_for(tensor, stream=torch.cuda.current_stream(tensor.device))
+        return RingSubmissionContext(tensor=tensor, stream=self.stream, producer_completion=produced)
+
+    def wait_for_producer(self, tensor: Any, *, context: RingSubmissionContext) -> None:
+        context.wait_stream(context.stream)
+        tensor.record_stream(context.stream)
+
+    def record_completion(self, *, context: RingSubmissionContext, dependencies: tuple[Any, ...]) -> Any:
+        for dependency in dependencies:
+            wait_stream = getattr(dependency, "wait_stream", None)
+            if callable(wait_stream):
+                wait_stream(context.stream)
+        return self._completions.record_for(context.tensor, stream=context.stream)
+
+    # ---- steps ------------------------------------------------------------- #
+    def _send_buffer(self, view: Any, workspace: Any, context: RingSubmissionContext) -> Any:
+        buffer = workspace.get_quantized_chunk(id(context.tensor), context.quant_index, view, self.config,
+                                               dtype=self.dtype, world_size=self.world_size)
+        context.quant_index += 1
+        return buffer
+
+    def quant_pack(self, tensor: Any, chunk: ChunkRange, workspace: Any, *, context: RingSubmissionContext) -> Any:
+        from lowbit_comm_amd.hip import ops
+
+        staged, context.staged = context.staged, None
+        if staged is not None and staged[0] == (chunk.start, chunk.stop):
+            return staged[1]
+        view = _view(tensor, chunk)
+        payload = self._send_buffer(view, workspace, context)
+        if not ops.bind_quant_pack_payload(view, payload, group_size=self.config.group_size)(context.stream.cuda_stream):
+            raise RuntimeError("quantize+pack has no kernel for this configuration")
+        return payload
+
+    def send_recv(self, payload: Any, *, send_peer: int, recv_peer: int, recv_chunk: ChunkRange, workspace: Any,
+                  context: RingSubmissionContext) -> tuple[Any, Any]:
+        for peer in (send_peer, recv_peer):
+            _rank_of(peer, self.world_size, "P2P peer")
+        # sized for the chunk that arrives, which is shorter than the one sent when it is the ragged last chunk
+        received = workspace.get_received_tensor_payload(id(context.tensor), context.recv_index,
+                                                         _view(context.tensor, recv_chunk), self.config,
+                                                         dtype=self.dtype, world_size=self.world_size)
+        context.recv_index += 1
+        handle = self._exchange(payload, received, send_peer=send_peer, recv_peer=recv_peer, stream=context.stream)
+        return received, handle
+
+    def _step(self, tensor: Any, received: Any, chunk: ChunkRange, workspace: Any, context: RingSubmissionContext,
+              dependency: Any, *, reduce_op: str, divisor: float) -> Any:
+        import torch
+
+        from lowbit_comm_amd.hip import ops
+
+        dependency.wait_stream(context.stream)
+        view = _view(tensor, chunk)
+        context.steps_done += 1
+        g = self.config.group_size
+        raw_stream = context.stream.cuda_stream
+        another_hop = context.steps_done < 2 * (self.world_size - 1)
+        if self.fuse_steps:
+            send = self._send_buffer(view, workspace, context) if another_hop else None
+            if not ops.bind_ring_step(received, view, send, group_size=g, reduce_op=reduce_op,
+                                      divisor=divisor)(raw_stream):
+                raise RuntimeError("the ring step has no kernel for this configuration")
+            context.staged = ((chunk.start, chunk.stop), send) if another_hop else None
+            return view
+        with torch.cuda.stream(context.stream):
+            if not ops.dequant_payload_into(received, view, group_size=g, reduce_op=reduce_op):
+                raise RuntimeError("decode has no kernel for this configuration")
+            if divisor != 1.0:
+                ops.true_divide_(view, divisor)
+        return view
+
+    def fused_reduce(self, tensor: Any, received: Any, chunk: ChunkRange, contributors: tuple[int, ...],
+                     workspace: Any, *, context: RingSubmissionContext, dependency: Any) -> Any:
+        last = len(contributors) == self.world_size - 1
+        out = self._step(tensor, received, chunk, workspace, context, dependency, reduce_op="sum",
+                         divisor=float(self.world_size) if last else 1.0)
+        if last:
+            context.mean_applied = True
+        return out
+
+    def apply_broadcast(self, tensor: Any, received: Any, chunk: ChunkRange, workspace: Any, *,
+                        context: RingSubmissionContext, dependency: Any) -> Any:
+        return self._step(tensor, received, chunk, workspace, context, dependency, reduce_op="none", divisor=1.0)
+
+
+# --------------------------------------------------------------------------- #
+# every rank of a ring on one device
+# --------------------------------------------------------------------------- #
+class _EventHandle:
+    def __init__(self, event: Any) -> None:
+        self._event = event
+
+    def query(self) -> bool:
+        return bool(self._event.query())
+
+    def is_completed(self) -> bool:
+        return self.query()
+
+    def wait(self) -> None:
+        self._event.wait()
+
+    def wait_stream(self, stream: Any) -> None:
+        stream.wait_event(self._event)
+
+
+class LoopbackRing:
+    """All W ranks of a ring in one process on one device, one host thread per rank: the exchange is a
+    device-to-device copy ordered by events, standing in for the links between GPUs (tests, single-GPU
+    measurements).  ``exchange_for(rank)`` is the callable a rank's runtime takes; every rank must reach every
+    step, as with a real collective.  A rank that fails calls :meth:`abort` so the others do not wait for it."""
+
+    def __init__(self, world_size: int, *, timeout: float = 120.0) -> None:
+        self.world_size = world_size
+        self._meet = threading.Barrier(world_size, timeout=timeout)
+        self._posted: list = [None] * world_size
+        self._taken: list = [None] * world_size
+
+    def abort(self) -> None:
+        self._meet.abort()
+
+    def exchange_for(self, rank: int) -> Callable[..., Any]:
+        import torch
+
+        def exchange(payload: Any, received: Any, *, send_peer: int, recv_peer: int, stream: Any) -> Any:
+            ready = torch.cuda.Event()
+            ready.record(stream)
+            self._posted[rank] = (payload, ready, send_peer)
+            self._meet.wait()
+            source, source_ready, addressed_to = self._posted[recv_peer]
+            if addressed_to != rank:
+                self._meet.abort()
+                raise RuntimeError(f"rank {recv_peer} sent to {addressed_to}, rank {rank} expected its payload")
+            if source.numel() != received.numel():
+                self._meet.abort()
+                raise RuntimeError("payload sizes of sender and receiver differ")
+            stream.wait_event(source_ready)
+            with torch.cuda.stream(stream):
+                received.copy_(source, non_blocking=True)
+            copied = torch.cuda.Event()
+            copied.record(stream)
+            self._taken[rank] = copied
+            self._meet.wait()
+            stream.wait_event(self._taken[send_peer])     # the send is over once the receiver has its copy
+            return _EventHandle(copied)
+
+        return exchange
+
+
+def make_pipelined_ring_executor(*, config: CompressionConfig, dtype: str, numel: int, world_size: int, rank: int,
+                                 exchange: Callable[..., Any], pool: Any | None = None,
+                                 completion_manager: Any | None = None, device: str = "cuda:0",
+                                 fuse_steps: bool = True) -> PipelinedRingExecutor:
+    """Plan, schedule, runtime, pooled workspaces and executor of one rank for buckets of ``numel`` elements."""
+    from lowbit_comm_amd.hip.completion import HipCompletionManager
+    from lowbit_comm_amd.hip.workspace import ShardWorkspaceProvider, create_torch_workspace_pool
+
+    manager = completion_manager if completion_manager is not None else HipCompletionManager()
+    plan = compile_chunk_plan(original_numel=numel, world_size=world_size)
+    schedule = compile_pipelined_ring_schedule(chunk_plan=plan, rank=rank)
+    runtime = HipPipelinedRingRuntime(config=config, dtype=dtype, world_size=world_size, rank=rank, exchange=exchange,
+                                      completion_manager=manager, fuse_steps=fuse_steps)
+    provider = ShardWorkspaceProvider(pool if pool is not None else create_torch_workspace_pool(), backend="hip",
+                                      collective="all_reduce", strategy="pipelined_ring", device=device)
+
+    def session_for(tensor: Any) -> Any:
+        del tensor
+        runtime._ready()
+        return provider.begin(stream=runtime.stream)
+
+    return PipelinedRingExecutor(schedule=schedule, runtime=runtime, workspace_session_factory=session_for,
+                                 completion_manager=manager)

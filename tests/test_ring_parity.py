@@ -1,0 +1,257 @@
+"""GPU parity of the ring-step kernel and of the ring all-reduce built on it, through the C ABI, against the CPU
+oracle (oracle/ring_np.py) on the same seeded inputs.  Bar: chunk values, int8 codes and fp32 scales bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import codec_np, ring_np
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module", params=["vector", "stream"])
+def ops(request, hip_device):
+    from lowbit_comm_amd.hip import ops as hip_ops
+    from lowbit_comm_amd.hip.library import load_library
+
+    lib = load_library()
+    previous = lib.lbc_set_stream_min_bytes({"vector": 1 << 62, "stream": 0}[request.param])
+    yield hip_ops
+    lib.lbc_set_stream_min_bytes(previous)
+
+
+def to_np(t: torch.Tensor, dtype: str) -> np.ndarray:
+    t = t.detach().cpu().contiguous()
+    if dtype == "bf16":
+        return t.view(torch.int16).numpy().view(np.uint16).copy()
+    return t.numpy().copy()
+
+
+def raw(a: np.ndarray) -> np.ndarray:
+    return a.view({2: np.uint16, 4: np.uint32}[a.dtype.itemsize])
+
+
+def tensor_like(n, dtype, seed, device, sigma=1e-3):
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    x = torch.randn(n, generator=gen) * sigma
+    if n:
+        mask = torch.rand(n, generator=gen) < 2e-3
+        x = torch.where(mask, torch.randn(n, generator=gen) * 1e-1, x)
+    return x.to(DTYPES[dtype]).to(device)
+
+
+def check_step(ops, device, dtype, g, n, reduce_op, divisor, emit, seed, offset=0):
+    incoming = tensor_like(n, "fp32", seed, device)
+    received = torch.empty(ops.payload_nbytes(n, g), dtype=torch.uint8, device=device)
+    assert ops.quant_pack_payload_into(incoming, received, group_size=g)
+    backing = tensor_like(n + offset, dtype, seed + 1, device, sigma=3e-3)
+    chunk = backing[offset:]
+    before = to_np(chunk, dtype)
+    send = torch.full((ops.payload_nbytes(n, g),), 0xAB, dtype=torch.uint8, device=device) if emit else None
+    assert ops.ring_step_into(received, chunk, send, group_size=g, reduce_op=reduce_op, divisor=divisor)
+    groups = ops.num_groups(n, g)
+    r = received.cpu().numpy()
+    codes, scales = r[:groups * g].view(np.int8), r[groups * g:].view(np.float32)
+    want_chunk, want_payload = ring_np.ring_step((codes, scales), before, dtype, g, reduce_op=reduce_op,
+                                                 divisor=divisor, emit=emit)
+    what = (dtype, g, n, reduce_op, divisor, emit, offset)
+    got = to_np(chunk, dtype)
+    assert np.array_equal(raw(got), raw(want_chunk)), what
+    if offset:
+        assert torch.equal(backing[:offset].cpu(), tensor_like(n + offset, dtype, seed + 1, "cpu", sigma=3e-3)[:offset])
+    if emit:
+        s = send.cpu().numpy()
+        assert np.array_equal(s[:groups * g].view(np.int8), want_payload[0]), what
+        assert np.array_equal(s[groups * g:].view(np.uint32), want_payload[1].view(np.uint32)), what
+    return chunk, send
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("g", [64, 32, 16])
+def test_ring_step_bit_exact(ops, hip_device, dtype, g):
+    seed = 100
+    for n in (1, g - 1, g, 1000, 4096 * 3, 65_536 + 7, 300_001):
+        for reduce_op, divisor in (("sum", 1.0), ("sum", 8.0), ("sum", 3.0), ("none", 1.0)):
+            for emit in (True, False):
+                seed += 2
+                check_step(ops, hip_device, dtype, g, n, reduce_op, divisor, emit, seed)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_ring_step_on_unaligned_chunk_views(ops, hip_device, dtype):
+    for offset in (1, 3):
+        for n in (4096 * 2 + 5, 64 * 100):
+            check_step(ops, hip_device, dtype, 64, n, "sum", 8.0, True, 900 + offset, offset=offset)
+
+
+def test_ring_step_equals_the_three_separate_launches(ops, hip_device):
+    g, n = 64, 1_000_003
+    for dtype in ("fp32", "bf16"):
+        incoming = tensor_like(n, "fp32", 5, hip_device)
+        codes, scales = ops.quant_pack(incoming, group_size=g)
+        received = torch.cat([codes.view(torch.uint8), scales.view(torch.uint8)])
+        start = tensor_like(n, dtype, 6, hip_device, sigma=2e-3)
+        fused_chunk = start.clone()
+        send = torch.empty_like(received)
+        assert ops.ring_step_into(received, fused_chunk, send, group_size=g, reduce_op="sum", divisor=3.0)
+        plain = start.clone()
+        assert ops.dequant_into(codes, scales, plain, group_size=g, reduce_op="sum")
+        ops.true_divide_(plain, 3.0)
+        two_codes, two_scales = ops.quant_pack(plain, group_size=g)
+        assert torch.equal(fused_chunk.view(torch.int16 if dtype == "bf16" else torch.int32),
+                           plain.view(torch.int16 if dtype == "bf16" else torch.int32))
+        groups = ops.num_groups(n, g)
+        assert torch.equal(send[:groups * g].view(torch.int8), two_codes)
+        assert torch.equal(send[groups * g:].view(torch.int32), two_scales.view(torch.int32))
+
+
+def test_ring_step_special_values(ops, hip_device):
+    """NaN and Inf travel as they do through decode, add and quantize: the scale keeps them, codes follow the
+    oracle's policy for non-finite quotients."""
+    g, n = 64, 64 * 6
+    incoming = torch.zeros(n, device=hip_device)
+    incoming[5] = 3.0
+    received = torch.empty(ops.payload_nbytes(n, g), dtype=torch.uint8, device=hip_device)
+    assert ops.quant_pack_payload_into(incoming, received, group_size=g)
+    chunk = torch.zeros(n, device=hip_device)
+    chunk[70] = float("nan")
+    chunk[130] = float("inf")
+    chunk[200] = -float("inf")
+    chunk[201] = 1.0
+    chunk[64 * 4:64 * 5] = 0.0                 # an all-zero group keeps the eps scale
+    before = chunk.cpu().numpy().copy()
+    send = torch.empty_like(received)
+    assert ops.ring_step_into(received, chunk, send, group_size=g, reduce_op="sum")
+    r = received.cpu().numpy()
+    want_chunk, (want_codes, want_scales) = ring_np.ring_step((r[:n].view(np.int8), r[n:].view(np.float32)), before,
+                                                              "fp32", g)
+    assert np.array_equal(chunk.cpu().numpy().view(np.uint32), want_chunk.view(np.uint32))
+    s = send.cpu().numpy()
+    assert np.array_equal(s[n:].view(np.uint32), want_scales.view(np.uint32))
+    finite_groups = np.isfinite(want_scales)
+    mask = np.repeat(finite_groups, g)
+    assert np.array_equal(s[:n].view(np.int8)[mask], want_codes[mask])
+
+
+def test_ring_step_contract(ops, hip_device):
+    g, n = 64, 640
+    x = tensor_like(n, "fp32", 1, hip_device)
+    received = torch.empty(ops.payload_nbytes(n, g), dtype=torch.uint8, device=hip_device)
+    assert ops.quant_pack_payload_into(x, received)
+    chunk = torch.zeros(n, device=hip_device)
+    assert ops.ring_step_into(received, chunk, None, reduce_op="max") is False            # unsupported, not an error
+    odd = torch.zeros(ops.payload_nbytes(n, 48), dtype=torch.uint8, device=hip_device)
+    assert ops.ring_step_into(odd, chunk, None, group_size=48) is False
+    with pytest.raises(RuntimeError, match="divisor must be > 0"):
+        ops.ring_step_into(received, chunk, None, divisor=0.0)
+    with pytest.raises(RuntimeError, match="invalid quantized payload size"):
+        ops.ring_step_into(received[:-4], chunk, None)
+    with pytest.raises(RuntimeError, match="must not alias"):
+        ops.ring_step_into(received, chunk, received)
+    with pytest.raises(RuntimeError, match="must be a GPU tensor"):
+        ops.ring_step_into(received.cpu(), chunk, None)
+    with pytest.raises(RuntimeError, match="fp16, bf16 or fp32"):
+        ops.ring_step_into(received, chunk.double(), None)
+    empty = torch.zeros(0, device=hip_device)
+    nothing = torch.zeros(0, dtype=torch.uint8, device=hip_device)
+    assert ops.ring_step_into(nothing, empty, nothing.clone())
+
+
+def test_ring_step_at_the_config4_chunk_size_keeps_the_sum_property(ops, hip_device):
+    """6,553,600-element chunk (one eighth of a 200 MiB fp32 bucket): too large for the oracle in seconds, so
+    check what must hold at any size: the updated chunk equals the separate decode-accumulate, and the payload
+    decodes to within half a scale of it."""
+    g, n = 64, 6_553_600
+    incoming = tensor_like(n, "fp32", 77, hip_device)
+    codes, scales = ops.quant_pack(incoming, group_size=g)
+    received = torch.cat([codes.view(torch.uint8), scales.view(torch.uint8)])
+    start = tensor_like(n, "fp32", 78, hip_device)
+    chunk = start.clone()
+    send = torch.empty_like(received)
+    assert ops.ring_step_into(received, chunk, send, group_size=g, reduce_op="sum", divisor=8.0)
+    plain = start.clone()
+    assert ops.dequant_into(codes, scales, plain, group_size=g, reduce_op="sum")
+    plain /= 8.0
+    assert torch.equal(chunk.view(torch.int32), plain.view(torch.int32))
+    out_codes, out_scales = send[:n].view(torch.int8), send[n:].view(torch.float32)
+    decoded = out_codes.float().view(-1, g) * out_scales[:, None]
+    assert bool(((decoded - chunk.view(-1, g)).abs() <= out_scales[:, None] * 0.5001).all())
+    assert int(out_codes.abs().view(-1, g).amax(dim=1).min()) == 127
+
+
+# --------------------------------------------------------------------------- #
+# the whole ring: every rank on one device, one host thread per rank
+# --------------------------------------------------------------------------- #
+def run_ring(device, buckets, dtype, g, fuse_steps, pools=None):
+    import threading
+
+    from lowbit_comm_amd.config import CompressionConfig
+    from lowbit_comm_amd.hip.ring import LoopbackRing, make_pipelined_ring_executor
+
+    world = len(buckets)
+    fabric = LoopbackRing(world, timeout=60.0)
+    config = CompressionConfig(group_size=g)
+    executors = [make_pipelined_ring_executor(config=config, dtype=dtype, numel=buckets[0].numel(), world_size=world,
+                                              rank=r, exchange=fabric.exchange_for(r), fuse_steps=fuse_steps,
+                                              pool=None if pools is None else pools[r], device=str(device))
+                 for r in range(world)]
+    errors = [None] * world
+    works = [None] * world
+
+    def body(rank):
+        try:
+            torch.cuda.set_device(device)
+            works[rank] = executors[rank].run(buckets[rank])
+            assert works[rank].wait() is buckets[rank]
+        except BaseException as error:      # noqa: BLE001 - reported by the caller
+            errors[rank] = error
+            fabric.abort()
+
+    threads = [threading.Thread(target=body, args=(r,)) for r in range(world)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    assert not any(t.is_alive() for t in threads)
+    first = next((e for e in errors if e is not None), None)
+    if first is not None:
+        raise first
+    torch.cuda.synchronize()
+    return executors, works
+
+
+@pytest.mark.parametrize("fuse_steps", [True, False])
+@pytest.mark.parametrize("dtype, world, n, g", [("fp32", 2, 64 * 9, 64), ("fp32", 3, 10_007, 64), ("fp32", 8, 8 * 64 * 40 + 13, 64),
+                                               ("bf16", 4, 33_333, 32), ("fp16", 5, 20_000, 16), ("fp32", 8, 5, 16),
+                                               ("bf16", 8, 200_003, 64), ("fp32", 1, 1000, 64)])
+def test_ring_all_reduce_matches_the_oracle_on_every_rank(ops, hip_device, fuse_steps, dtype, world, n, g):
+    buckets = [tensor_like(n, dtype, 4000 + 17 * r, hip_device, sigma=10.0 ** (r % 3 - 3)) for r in range(world)]
+    before = [to_np(b, dtype) for b in buckets]
+    run_ring(hip_device, buckets, dtype, g, fuse_steps)
+    want = ring_np.ring_all_reduce(before, dtype, g)
+    for rank in range(world):
+        got = to_np(buckets[rank], dtype)
+        assert np.array_equal(raw(got), raw(want[rank])), (rank, dtype, world, n, g, fuse_steps)
+
+
+def test_ring_reuses_pooled_workspaces_and_launches_one_kernel_per_hop(ops, hip_device):
+    from lowbit_comm_amd.hip.workspace import create_torch_workspace_pool
+
+    world, n, g = 4, 64 * 1000, 64
+    pools = [create_torch_workspace_pool() for _ in range(world)]
+    results = []
+    for repeat in range(3):
+        buckets = [tensor_like(n, "fp32", 70 + r, hip_device) for r in range(world)]
+        before = [to_np(b, "fp32") for b in buckets]
+        executors, _ = run_ring(hip_device, buckets, "fp32", g, True, pools=pools)
+        want = ring_np.ring_all_reduce(before, "fp32", g)
+        assert all(np.array_equal(raw(to_np(buckets[r], "fp32")), raw(want[r])) for r in range(world))
+        results.append([p.stats for p in pools])
+    # 2(W-1) send and 2(W-1) receive buffers per rank, all allocated by the first run
+    first, last = results[0], results[-1]
+    for rank in range(world):
+        assert first[rank].misses == 4 * (world - 1)
+        assert last[rank].misses == first[rank].misses
+        assert last[rank].hits == 2 * first[rank].misses
