@@ -17,9 +17,13 @@ object per configuration plus a summary table on stderr:
      strategy over pre-bound plans, without and with error feedback), a pre-bound launch, and the config-5 launch
      sequence eager against one HIP-graph replay.  Rows report host microseconds per bucket next to wall time.
 
+  8  the compute steps of the quantized ring all-reduce on one chunk (an eighth of the config-4 and config-5
+     buckets): the fused ring step (decode + accumulate [+ mean] + requantize in one launch) against the separate
+     decode-accumulate and quantize launches, and one rank's whole W=8 schedule through the executor
+
 "~N(0, s)" is read as standard deviation s.  Times are HIP-event averages over back-to-back launches.
 
-    python bench_configs.py [--configs 1,2,3,4,5,6,7] [--no-parity] [--llama-layers 32]
+    python bench_configs.py [--configs 1,2,3,4,5,6,7,8] [--no-parity] [--llama-layers 32]
 """
 from __future__ import annotations
 
@@ -40,7 +44,7 @@ G = 64
 
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--configs", default="1,2,3,4,5,6,7")
+    ap.add_argument("--configs", default="1,2,3,4,5,6,7,8")
     ap.add_argument("--no-parity", action="store_true", help="skip the CPU oracle comparisons")
     ap.add_argument("--llama-layers", type=int, default=32, help="config 5: number of transformer layers (32 = full model)")
     ap.add_argument("--iters", type=int, default=50)
@@ -647,6 +651,131 @@ def main() -> int:
         host, wall = host_and_wall(lambda i: graph.replay(), 5)
         host_row("the same sequence as one HIP-graph replay, per bucket", host / count, wall / count)
         del grads, residuals, launches, graph
+
+    # ------------------------------------------------------------------------------------------ 8
+    if 8 in wanted:
+        from lowbit_comm_amd.hip.ring import make_pipelined_ring_executor
+
+        for label, n, dtype, sets_n in (("fp32 chunk of 6,553,600 (200 MiB bucket / 8)", 6_553_600, torch.float32, 8),
+                                        ("bf16 chunk of 1,638,400 (25 MiB bucket / 8)", 1_638_400, torch.bfloat16, 24)):
+            eb = 4 if dtype == torch.float32 else 2
+            pb = ops.payload_nbytes(n, G)
+            sets = []
+            for k in range(sets_n):
+                received = torch.empty(pb, dtype=torch.uint8, device=dev)
+                ops.quant_pack_payload_into(gen(SEED + 8000 + k, n, 1e-3), received)
+                chunk = gen(SEED + 8100 + k, n, 1e-3, dtype)
+                send = torch.empty(pb, dtype=torch.uint8, device=dev)
+                codes, scales = ops.split_payload(send, n, G)
+                sets.append({
+                    "chunk": chunk, "send": send, "received": received,
+                    "sum": ops.bind_ring_step(received, chunk, send, reduce_op="sum"),
+                    "mean": ops.bind_ring_step(received, chunk, send, reduce_op="sum", divisor=8.0),
+                    "copy": ops.bind_ring_step(received, chunk, send, reduce_op="none"),
+                    "last": ops.bind_ring_step(received, chunk, None, reduce_op="none"),
+                    "decode_sum": ops.bind_dequant(*ops.split_payload(received, n, G), chunk, reduce_op="sum"),
+                    "quant": ops.bind_quant_pack(chunk, codes, scales),
+                })
+            check = None
+            if parity:
+                from oracle import codec_np, ring_np
+
+                small = 64 * 1000 + 7
+                incoming = torch.empty(ops.payload_nbytes(small, G), dtype=torch.uint8, device=dev)
+                ops.quant_pack_payload_into(gen(SEED + 8200, small, 1e-3), incoming)
+                piece = gen(SEED + 8201, small, 1e-3, dtype)
+                before = piece.cpu()
+                before = before.view(torch.int16).numpy().view("uint16") if dtype == torch.bfloat16 else before.numpy()
+                out_payload = torch.empty_like(incoming)
+                ops.ring_step_into(incoming, piece, out_payload, reduce_op="sum", divisor=8.0)
+                raw_in = incoming.cpu().numpy()
+                groups = ops.num_groups(small, G)
+                want, (w_codes, w_scales) = ring_np.ring_step(
+                    (raw_in[:groups * G].view("int8"), raw_in[groups * G:].view("float32")), before,
+                    "bf16" if dtype == torch.bfloat16 else "fp32", G, reduce_op="sum", divisor=8.0)
+                got = piece.cpu()
+                got = got.view(torch.int16).numpy().view("uint16") if dtype == torch.bfloat16 else got.numpy().view("uint32")
+                ok = bool((got == (want if dtype == torch.bfloat16 else want.view("uint32"))).all())
+                raw_out = out_payload.cpu().numpy()
+                ok = ok and bool((raw_out[:groups * G].view("int8") == w_codes).all())
+                ok = ok and bool((raw_out[groups * G:].view("uint32") == w_scales.view("uint32")).all())
+                # full size: the fused launch against the separate ones
+                a, b = sets[0], sets[1]
+                b["chunk"].copy_(a["chunk"]); b["received"].copy_(a["received"])
+                a["sum"](); b["decode_sum"](); b["quant"]()
+                ok = ok and bits_equal(a["chunk"], b["chunk"]) and torch.equal(a["send"], b["send"])
+                check = "bit-exact" if ok else "MISMATCH"
+            payload_bytes = pb
+            fused_bytes = 2 * payload_bytes + 2 * n * eb
+            emit(8, f"ring step, {label}: decode + accumulate + requantize, one launch", fused_bytes,
+                 timed(lambda i: sets[i % sets_n]["sum"](), args.iters * 2), n * eb, check)
+            emit(8, f"ring step, {label}: the same with the mean (last reduce hop)", fused_bytes,
+                 timed(lambda i: sets[i % sets_n]["mean"](), args.iters * 2), n * eb, check)
+            emit(8, f"ring step, {label}: decode + requantize (gather hop)", 2 * payload_bytes + n * eb,
+                 timed(lambda i: sets[i % sets_n]["copy"](), args.iters * 2), n * eb, check)
+            emit(8, f"ring step, {label}: decode only (last gather hop)", payload_bytes + n * eb,
+                 timed(lambda i: sets[i % sets_n]["last"](), args.iters * 2), n * eb, check)
+
+            def separate(i):
+                sets[i % sets_n]["decode_sum"]()
+                sets[i % sets_n]["quant"]()
+
+            emit(8, f"ring step, {label}: separate decode-accumulate and quantize launches (the reference's sequence)",
+                 (payload_bytes + 2 * n * eb) + (n * eb + payload_bytes), timed(separate, args.iters * 2), n * eb, check)
+            del sets
+
+        # one rank's whole schedule (W=8, 200 MiB fp32 bucket) through the executor, replaying the bucket's plan
+        world, n = 8, 52_428_800
+        peer_payload = torch.empty(ops.payload_nbytes(n // world, G), dtype=torch.uint8, device=dev)
+        ops.quant_pack_payload_into(gen(SEED + 8300, n // world, 1e-3), peer_payload)
+
+        class Arrived:
+            def query(self):
+                return True
+
+            def wait_stream(self, s):
+                return None
+
+        placed = set()
+
+        def exchange(payload, received, *, send_peer, recv_peer, stream):
+            # The link is not part of this measurement: a peer's payload is placed in every receive buffer once.
+            if received.data_ptr() not in placed:
+                with torch.cuda.stream(stream):
+                    received.copy_(peer_payload, non_blocking=True)
+                placed.add(received.data_ptr())
+            return Arrived()
+
+        buckets = [gen(SEED + 8400 + k, n, 1e-3) for k in range(3)]
+        for fused in (True, False):
+            executor = make_pipelined_ring_executor(config=cfg, dtype="fp32", numel=n, world_size=world, rank=3,
+                                                    exchange=exchange, fuse_steps=fused)
+
+            def whole(i, executor=executor):
+                executor.run(buckets[i % 3]).wait()
+
+            for i in range(3):
+                whole(i)
+            torch.cuda.synchronize()
+            count = 12
+            t0 = time.perf_counter()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            for i in range(count):
+                whole(i)
+            b.record(stream)
+            host = (time.perf_counter() - t0) / count
+            torch.cuda.synchronize()
+            seconds = a.elapsed_time(b) * 1e-3 / count
+            chunk_bytes, pay = n // world * 4, ops.payload_nbytes(n // world, G)
+            if fused:   # first quantize, 6 sum hops, 1 mean hop, 6 gather hops with payload, 1 without; 14 arrivals
+                nbytes = (chunk_bytes + pay) + 7 * (2 * pay + 2 * chunk_bytes) + 6 * (2 * pay + chunk_bytes) + (pay + chunk_bytes)
+            else:       # 14 quantize, 7 decode-accumulate, 1 division, 7 decode
+                nbytes = 14 * (chunk_bytes + pay) + 7 * (pay + 2 * chunk_bytes) + 2 * chunk_bytes + 7 * (pay + chunk_bytes)
+            emit(8, f"one rank's ring schedule, W=8, 200 MiB fp32 bucket, {'fused ring steps' if fused else 'separate launches'}"
+                    f" (14 hops through the executor, payloads of a peer already in the receive buffers; host "
+                    f"{host * 1e6:.0f} us per bucket)", nbytes, seconds, n * 4, None)
+        del buckets
 
     print(f"\n{'cfg':>3} {'us':>10} {'GB/s alg.':>10} {'% of 8TB/s':>10} {'input GB/s':>10}  parity / op", file=sys.stderr)
     for r in rows_out:

@@ -393,6 +393,8 @@ class RingSubmissionContext:
     mean_applied: bool = False
     steps_done: int = 0
     staged: tuple | None = None        # ((start, stop), payload) quantized by the previous step's launch
+    plan: dict | None = None           # buffers and bound launches of this tensor, when the runtime keeps plans
+    raw_stream: int = 0
 
     def query(self) -> bool:
         return bool(self.producer_completion.query())
@@ -416,11 +418,19 @@ class HipPipelinedRingRuntime:
     quantizes the updated chunk into the send buffer of the next step; the following ``quant_pack`` of that chunk
     returns the staged payload without a launch.  ``fuse_steps=False`` issues the reference's sequence (decode with
     reduce op, in-place division, quantize) as separate launches; both give the same bits.  Unlike the reference's
-    native path, chunks need not be multiples of the group size."""
+    native path, chunks need not be multiples of the group size.
+
+    ``max_plans > 0`` (default 16): the send and receive buffers of a bucket and its validated, marshalled launches
+    are kept per ``(address, numel)`` of the tensor and replayed on later runs, least recently used plans dropped
+    first; the workspace session is then not asked for buffers.  One plan holds ``4 (W - 1)`` payload buffers.  All of
+    a runtime's work is enqueued on its one stream, which orders the reuse of those buffers between runs.
+    ``max_plans=0``: every run leases its buffers from the workspace session."""
 
     def __init__(self, *, config: CompressionConfig, dtype: str, world_size: int, rank: int,
                  exchange: Callable[..., Any], completion_manager: Any | None = None, stream: Any | None = None,
-                 fuse_steps: bool = True) -> None:
+                 fuse_steps: bool = True, max_plans: int = 16) -> None:
+        from collections import OrderedDict
+
         from lowbit_comm_amd.hip.executors import fused_dequant_fallback_reason
 
         reason = fused_dequant_fallback_reason(config)
@@ -433,11 +443,15 @@ class HipPipelinedRingRuntime:
         _rank_of(rank, world_size, "rank")
         if not callable(exchange):
             raise TypeError("exchange must be callable")
+        if isinstance(max_plans, bool) or not isinstance(max_plans, int) or max_plans < 0:
+            raise ValueError("max_plans must be an integer >= 0")
         self.config = config
         self.dtype = dtype
         self.world_size = world_size
         self.rank = rank
         self.fuse_steps = bool(fuse_steps)
+        self.max_plans = max_plans
+        self.plans: "OrderedDict[tuple[int, int], dict]" = OrderedDict()
         self._exchange = exchange
         self._completions = completion_manager
         self.stream = stream
@@ -453,6 +467,19 @@ class HipPipelinedRingRuntime:
         if self.stream is None:
             self.stream = torch.cuda.Stream()       # default priority
 
+    def _plan_of(self, tensor: Any) -> dict | None:
+        if self.max_plans == 0:
+            return None
+        key = (tensor.data_ptr(), tensor.numel())
+        plan = self.plans.get(key)
+        if plan is None:
+            while len(self.plans) >= self.max_plans:
+                self.plans.popitem(last=False)
+            plan = self.plans[key] = {}
+        else:
+            self.plans.move_to_end(key)
+        return plan
+
     def create_submission_context(self, tensor: Any) -> RingSubmissionContext:
         import torch
 
@@ -464,7 +491,8 @@ class HipPipelinedRingRuntime:
         if ops.DTYPE_NAMES.get(tensor.dtype) != self.dtype:
             raise RuntimeError(f"tensor dtype {tensor.dtype} does not match the runtime's {self.dtype}")
         produced = self._completions.record_for(tensor, stream=torch.cuda.current_stream(tensor.device))
-        return RingSubmissionContext(tensor=tensor, stream=self.stream, producer_completion=produced)
+        return RingSubmissionContext(tensor=tensor, stream=self.stream, producer_completion=produced,
+                                     plan=self._plan_of(tensor), raw_stream=self.stream.cuda_stream)
 
     def wait_for_producer(self, tensor: Any, *, context: RingSubmissionContext) -> None:
         context.wait_stream(context.stream)
@@ -477,61 +505,103 @@ class HipPipelinedRingRuntime:
                 wait_stream(context.stream)
         return self._completions.record_for(context.tensor, stream=context.stream)
 
-    # ---- steps ------------------------------------------------------------- #
+    # ---- buffers ----------------------------------------------------------- #
+    def _payload_buffer(self, kind: str, index: int, view: Any, workspace: Any, context: RingSubmissionContext) -> Any:
+        """Send or receive buffer number ``index`` of this submission, sized for ``view``'s chunk."""
+        plan = context.plan
+        if plan is not None:
+            buffer = plan.get((kind, index))
+            if buffer is None:
+                import torch
+
+                from lowbit_comm_amd.hip import ops
+
+                with torch.cuda.stream(context.stream):
+                    buffer = torch.empty(ops.payload_nbytes(view.numel(), self.config.group_size), dtype=torch.uint8,
+                                         device=view.device)
+                plan[(kind, index)] = buffer
+            return buffer
+        if kind == "send":
+            return workspace.get_quantized_chunk(id(context.tensor), index, view, self.config, dtype=self.dtype,
+                                                 world_size=self.world_size)
+        return workspace.get_received_tensor_payload(id(context.tensor), index, view, self.config, dtype=self.dtype,
+                                                     world_size=self.world_size)
+
     def _send_buffer(self, view: Any, workspace: Any, context: RingSubmissionContext) -> Any:
-        buffer = workspace.get_quantized_chunk(id(context.tensor), context.quant_index, view, self.config,
-                                               dtype=self.dtype, world_size=self.world_size)
+        buffer = self._payload_buffer("send", context.quant_index, view, workspace, context)
         context.quant_index += 1
         return buffer
 
+    # ---- steps ------------------------------------------------------------- #
     def quant_pack(self, tensor: Any, chunk: ChunkRange, workspace: Any, *, context: RingSubmissionContext) -> Any:
         from lowbit_comm_amd.hip import ops
 
         staged, context.staged = context.staged, None
         if staged is not None and staged[0] == (chunk.start, chunk.stop):
             return staged[1]
-        view = _view(tensor, chunk)
-        payload = self._send_buffer(view, workspace, context)
-        if not ops.bind_quant_pack_payload(view, payload, group_size=self.config.group_size)(context.stream.cuda_stream):
+        plan, key = context.plan, ("quantize", context.quant_index, chunk.start, chunk.stop)
+        bound = None if plan is None else plan.get(key)
+        if bound is None:
+            view = _view(tensor, chunk)
+            payload = self._send_buffer(view, workspace, context)
+            bound = (ops.bind_quant_pack_payload(view, payload, group_size=self.config.group_size), payload)
+            if plan is not None:
+                plan[key] = bound
+        else:
+            context.quant_index += 1
+        if not bound[0](context.raw_stream):
             raise RuntimeError("quantize+pack has no kernel for this configuration")
-        return payload
+        return bound[1]
 
     def send_recv(self, payload: Any, *, send_peer: int, recv_peer: int, recv_chunk: ChunkRange, workspace: Any,
                   context: RingSubmissionContext) -> tuple[Any, Any]:
-        for peer in (send_peer, recv_peer):
-            _rank_of(peer, self.world_size, "P2P peer")
-        # sized for the chunk that arrives, which is shorter than the one sent when it is the ragged last chunk
-        received = workspace.get_received_tensor_payload(id(context.tensor), context.recv_index,
-                                                         _view(context.tensor, recv_chunk), self.config,
-                                                         dtype=self.dtype, world_size=self.world_size)
-        context.recv_index += 1
+        world = self.world_size
+        if not (0 <= send_peer < world and 0 <= recv_peer < world):
+            raise ValueError("P2P peer must be a valid group-local rank")
+        index = context.recv_index
+        context.recv_index = index + 1
+        received = None if context.plan is None else context.plan.get(("recv", index))
+        if received is None:
+            # sized for the chunk that arrives, which is shorter than the one sent when it is the ragged last chunk
+            received = self._payload_buffer("recv", index, _view(context.tensor, recv_chunk), workspace, context)
         handle = self._exchange(payload, received, send_peer=send_peer, recv_peer=recv_peer, stream=context.stream)
         return received, handle
 
     def _step(self, tensor: Any, received: Any, chunk: ChunkRange, workspace: Any, context: RingSubmissionContext,
               dependency: Any, *, reduce_op: str, divisor: float) -> Any:
-        import torch
-
         from lowbit_comm_amd.hip import ops
 
         dependency.wait_stream(context.stream)
-        view = _view(tensor, chunk)
         context.steps_done += 1
-        g = self.config.group_size
-        raw_stream = context.stream.cuda_stream
         another_hop = context.steps_done < 2 * (self.world_size - 1)
-        if self.fuse_steps:
-            send = self._send_buffer(view, workspace, context) if another_hop else None
-            if not ops.bind_ring_step(received, view, send, group_size=g, reduce_op=reduce_op,
-                                      divisor=divisor)(raw_stream):
+        plan, key = context.plan, ("step", context.steps_done, chunk.start, chunk.stop, received.data_ptr())
+        bound = None if plan is None else plan.get(key)
+        if bound is None:
+            view = _view(tensor, chunk)
+            g = self.config.group_size
+            if self.fuse_steps:
+                send = self._send_buffer(view, workspace, context) if another_hop else None
+                launches = (ops.bind_ring_step(received, view, send, group_size=g, reduce_op=reduce_op,
+                                               divisor=divisor),)
+            else:
+                send = None
+                launches = (ops.bind_dequant(*ops.split_payload(received, view.numel(), g), view, group_size=g,
+                                             reduce_op=reduce_op),)
+            bound = (launches, view, send)
+            if plan is not None:
+                plan[key] = bound
+        elif bound[2] is not None:
+            context.quant_index += 1
+        launches, view, send = bound
+        for launch in launches:
+            if not launch(context.raw_stream):
                 raise RuntimeError("the ring step has no kernel for this configuration")
-            context.staged = ((chunk.start, chunk.stop), send) if another_hop else None
-            return view
-        with torch.cuda.stream(context.stream):
-            if not ops.dequant_payload_into(received, view, group_size=g, reduce_op=reduce_op):
-                raise RuntimeError("decode has no kernel for this configuration")
-            if divisor != 1.0:
+        if not self.fuse_steps and divisor != 1.0:
+            import torch
+
+            with torch.cuda.stream(context.stream):
                 ops.true_divide_(view, divisor)
+        context.staged = ((chunk.start, chunk.stop), send) if send is not None else None
         return view
 
     def fused_reduce(self, tensor: Any, received: Any, chunk: ChunkRange, contributors: tuple[int, ...],
@@ -614,7 +684,7 @@ class LoopbackRing:
 def make_pipelined_ring_executor(*, config: CompressionConfig, dtype: str, numel: int, world_size: int, rank: int,
                                  exchange: Callable[..., Any], pool: Any | None = None,
                                  completion_manager: Any | None = None, device: str = "cuda:0",
-                                 fuse_steps: bool = True) -> PipelinedRingExecutor:
+                                 fuse_steps: bool = True, max_plans: int = 16) -> PipelinedRingExecutor:
     """Plan, schedule, runtime, pooled workspaces and executor of one rank for buckets of ``numel`` elements."""
     from lowbit_comm_amd.hip.completion import HipCompletionManager
     from lowbit_comm_amd.hip.workspace import ShardWorkspaceProvider, create_torch_workspace_pool
@@ -623,7 +693,7 @@ def make_pipelined_ring_executor(*, config: CompressionConfig, dtype: str, numel
     plan = compile_chunk_plan(original_numel=numel, world_size=world_size)
     schedule = compile_pipelined_ring_schedule(chunk_plan=plan, rank=rank)
     runtime = HipPipelinedRingRuntime(config=config, dtype=dtype, world_size=world_size, rank=rank, exchange=exchange,
-                                      completion_manager=manager, fuse_steps=fuse_steps)
+                                      completion_manager=manager, fuse_steps=fuse_steps, max_plans=max_plans)
     provider = ShardWorkspaceProvider(pool if pool is not None else create_torch_workspace_pool(), backend="hip",
                                       collective="all_reduce", strategy="pipelined_ring", device=device)
 

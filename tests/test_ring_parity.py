@@ -184,19 +184,25 @@ def test_ring_step_at_the_config4_chunk_size_keeps_the_sum_property(ops, hip_dev
 # --------------------------------------------------------------------------- #
 # the whole ring: every rank on one device, one host thread per rank
 # --------------------------------------------------------------------------- #
-def run_ring(device, buckets, dtype, g, fuse_steps, pools=None):
-    import threading
-
+def build_ring(device, world, n, dtype, g, fuse_steps, pools=None, max_plans=16):
     from lowbit_comm_amd.config import CompressionConfig
     from lowbit_comm_amd.hip.ring import LoopbackRing, make_pipelined_ring_executor
 
-    world = len(buckets)
     fabric = LoopbackRing(world, timeout=60.0)
     config = CompressionConfig(group_size=g)
-    executors = [make_pipelined_ring_executor(config=config, dtype=dtype, numel=buckets[0].numel(), world_size=world,
-                                              rank=r, exchange=fabric.exchange_for(r), fuse_steps=fuse_steps,
-                                              pool=None if pools is None else pools[r], device=str(device))
+    executors = [make_pipelined_ring_executor(config=config, dtype=dtype, numel=n, world_size=world, rank=r,
+                                              exchange=fabric.exchange_for(r), fuse_steps=fuse_steps,
+                                              pool=None if pools is None else pools[r], device=str(device),
+                                              max_plans=max_plans)
                  for r in range(world)]
+    return fabric, executors
+
+
+def run_ring(device, buckets, dtype, g, fuse_steps, pools=None, max_plans=16, ring=None):
+    import threading
+
+    world = len(buckets)
+    fabric, executors = ring or build_ring(device, world, buckets[0].numel(), dtype, g, fuse_steps, pools, max_plans)
     errors = [None] * world
     works = [None] * world
 
@@ -226,10 +232,11 @@ def run_ring(device, buckets, dtype, g, fuse_steps, pools=None):
 @pytest.mark.parametrize("dtype, world, n, g", [("fp32", 2, 64 * 9, 64), ("fp32", 3, 10_007, 64), ("fp32", 8, 8 * 64 * 40 + 13, 64),
                                                ("bf16", 4, 33_333, 32), ("fp16", 5, 20_000, 16), ("fp32", 8, 5, 16),
                                                ("bf16", 8, 200_003, 64), ("fp32", 1, 1000, 64)])
-def test_ring_all_reduce_matches_the_oracle_on_every_rank(ops, hip_device, fuse_steps, dtype, world, n, g):
+@pytest.mark.parametrize("max_plans", [16, 0])
+def test_ring_all_reduce_matches_the_oracle_on_every_rank(ops, hip_device, fuse_steps, max_plans, dtype, world, n, g):
     buckets = [tensor_like(n, dtype, 4000 + 17 * r, hip_device, sigma=10.0 ** (r % 3 - 3)) for r in range(world)]
     before = [to_np(b, dtype) for b in buckets]
-    run_ring(hip_device, buckets, dtype, g, fuse_steps)
+    run_ring(hip_device, buckets, dtype, g, fuse_steps, max_plans=max_plans)
     want = ring_np.ring_all_reduce(before, dtype, g)
     for rank in range(world):
         got = to_np(buckets[rank], dtype)
@@ -245,7 +252,7 @@ def test_ring_reuses_pooled_workspaces_and_launches_one_kernel_per_hop(ops, hip_
     for repeat in range(3):
         buckets = [tensor_like(n, "fp32", 70 + r, hip_device) for r in range(world)]
         before = [to_np(b, "fp32") for b in buckets]
-        executors, _ = run_ring(hip_device, buckets, "fp32", g, True, pools=pools)
+        executors, _ = run_ring(hip_device, buckets, "fp32", g, True, pools=pools, max_plans=0)
         want = ring_np.ring_all_reduce(before, "fp32", g)
         assert all(np.array_equal(raw(to_np(buckets[r], "fp32")), raw(want[r])) for r in range(world))
         results.append([p.stats for p in pools])
@@ -255,3 +262,46 @@ def test_ring_reuses_pooled_workspaces_and_launches_one_kernel_per_hop(ops, hip_
         assert first[rank].misses == 4 * (world - 1)
         assert last[rank].misses == first[rank].misses
         assert last[rank].hits == 2 * first[rank].misses
+
+
+@pytest.mark.parametrize("fuse_steps", [True, False])
+def test_ring_replays_a_buckets_plan_without_allocating(ops, hip_device, fuse_steps):
+    world, n, g = 4, 64 * 777 + 5, 64
+    ring = build_ring(hip_device, world, n, "bf16", g, fuse_steps)
+    buckets = [torch.empty(n, dtype=torch.bfloat16, device=hip_device) for _ in range(world)]
+    other = [torch.empty(n // 2, dtype=torch.bfloat16, device=hip_device) for _ in range(world)]
+    allocated = None
+    for repeat in range(4):
+        fresh = [tensor_like(n, "bf16", 300 + 10 * repeat + r, hip_device) for r in range(world)]
+        for bucket, values in zip(buckets, fresh):
+            bucket.copy_(values)
+        before = [to_np(b, "bf16") for b in buckets]
+        del fresh
+        torch.cuda.synchronize()
+        if repeat >= 1:
+            allocated = torch.cuda.memory_allocated(hip_device)
+        executors, _ = run_ring(hip_device, buckets, "bf16", g, fuse_steps, ring=ring)
+        if repeat >= 1:
+            assert torch.cuda.memory_allocated(hip_device) == allocated
+        want = ring_np.ring_all_reduce(before, "bf16", g)
+        for rank in range(world):
+            assert np.array_equal(to_np(buckets[rank], "bf16"), want[rank]), (repeat, rank)
+    assert all(len(e._runtime.plans) == 1 for e in ring[1])
+    # a second bucket shape gets its own plan; the oldest plan goes when the limit is reached
+    for e in ring[1]:
+        e._runtime.max_plans = 1
+    for bucket in other:
+        bucket.normal_(std=1e-3)
+    before = [to_np(b, "bf16") for b in other]
+    from lowbit_comm_amd.hip.chunk_plan import compile_chunk_plan
+    from lowbit_comm_amd.hip.ring import PipelinedRingExecutor, compile_pipelined_ring_schedule
+
+    half_plan = compile_chunk_plan(original_numel=n // 2, world_size=world)
+    ring2 = (ring[0], [PipelinedRingExecutor(schedule=compile_pipelined_ring_schedule(chunk_plan=half_plan, rank=r),
+                                             runtime=ring[1][r]._runtime, workspace_session_factory=ring[1][r]._sessions,
+                                             completion_manager=ring[1][r]._works) for r in range(world)])
+    run_ring(hip_device, other, "bf16", g, fuse_steps, ring=ring2)
+    want = ring_np.ring_all_reduce(before, "bf16", g)
+    for rank in range(world):
+        assert np.array_equal(to_np(other[rank], "bf16"), want[rank])
+    assert all(list(e._runtime.plans) == [(other[r].data_ptr(), n // 2)] for r, e in enumerate(ring2[1]))
