@@ -657,7 +657,9 @@ def main() -> int:
         from lowbit_comm_amd.hip.ring import make_pipelined_ring_executor
 
         for label, n, dtype, sets_n in (("fp32 chunk of 6,553,600 (200 MiB bucket / 8)", 6_553_600, torch.float32, 8),
-                                        ("bf16 chunk of 1,638,400 (25 MiB bucket / 8)", 1_638_400, torch.bfloat16, 24)):
+                                        ("bf16 chunk of 1,638,400 (25 MiB bucket / 8)", 1_638_400, torch.bfloat16, 24),
+                                        ("fp32 chunk of 26,214,400 (a size past the launch ramp-up)", 26_214_400,
+                                         torch.float32, 4)):
             eb = 4 if dtype == torch.float32 else 2
             pb = ops.payload_nbytes(n, G)
             sets = []
