@@ -704,3 +704,47 @@ def make_pipelined_ring_executor(*, config: CompressionConfig, dtype: str, numel
 
     return PipelinedRingExecutor(schedule=schedule, runtime=runtime, workspace_session_factory=session_for,
                                  completion_manager=manager)
+
+
+def make_pipelined_ring_transport(*, world_size: int, rank: int, exchange: Callable[..., Any],
+                                  max_executors: int = 16, fuse_steps: bool = True, max_plans: int = 16,
+                                  completion_manager: Any | None = None, pool: Any | None = None) -> Callable[..., Any]:
+    """The callable ``create_ddp_comm_hook(strategy="topology", topology_all_reduce=...)`` expects, over the ring.
+
+    ``transport(tensor, *, config, op, async_op=False, dtype=None, extension_status=None)`` averages ``tensor`` over
+    the ring in place and returns it, ordered on the caller's current stream (``async_op``: the executor's work
+    object, whose ``wait()`` returns the tensor).  The ring computes the mean, as the reference's executor does
+    (the division sits on the hop that completes the sum, ``ccdl_comm/cuda/transports/torch_topology.py:287-289``);
+    any other ``op`` is refused.  One executor is kept per (element count, dtype, device, group size)."""
+    from collections import OrderedDict
+
+    from lowbit_comm_amd.exceptions import UnsupportedCollective
+
+    executors: OrderedDict = OrderedDict()
+
+    def transport(tensor: Any, *, config: CompressionConfig, op: str = "mean", async_op: bool = False,
+                  dtype: str | None = None, extension_status: Any | None = None) -> Any:
+        del extension_status                      # the runtime calls the C ABI directly
+        from lowbit_comm_amd.hip import ops
+
+        if op != "mean":
+            raise UnsupportedCollective(f"pipelined_ring:{op}", reason="the quantized ring computes the mean")
+        name = ops.DTYPE_NAMES.get(tensor.dtype)
+        if name is None or (dtype is not None and dtype != name):
+            raise ValueError(f"the ring reduces in the bucket's dtype; got dtype={dtype!r} for {tensor.dtype}")
+        key = (tensor.numel(), name, str(tensor.device), config.group_size)
+        executor = executors.get(key)
+        if executor is None:
+            executor = executors[key] = make_pipelined_ring_executor(
+                config=config, dtype=name, numel=tensor.numel(), world_size=world_size, rank=rank, exchange=exchange,
+                pool=pool, completion_manager=completion_manager, device=str(tensor.device), fuse_steps=fuse_steps,
+                max_plans=max_plans)
+            while len(executors) > max_executors:
+                executors.popitem(last=False)
+        else:
+            executors.move_to_end(key)
+        work = executor.run(tensor)
+        return work if async_op else work.wait()
+
+    transport.executors = executors
+    return transport

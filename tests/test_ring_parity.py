@@ -305,3 +305,65 @@ def test_ring_replays_a_buckets_plan_without_allocating(ops, hip_device, fuse_st
     for rank in range(world):
         assert np.array_equal(to_np(other[rank], "bf16"), want[rank])
     assert all(list(e._runtime.plans) == [(other[r].data_ptr(), n // 2)] for r, e in enumerate(ring2[1]))
+
+
+def test_ddp_hook_over_the_ring_transport(ops, hip_device):
+    """``create_ddp_comm_hook(strategy="topology", topology_all_reduce=make_pipelined_ring_transport(...))`` on
+    every rank of a loopback ring: each rank's bucket ends as the oracle's result for that rank, in place, and a
+    second step replays the same executor and plan."""
+    import threading
+
+    from lowbit_comm_amd.communication.ddp_hook import create_ddp_comm_hook
+    from lowbit_comm_amd.config import CompressionConfig
+    from lowbit_comm_amd.exceptions import UnsupportedCollective
+    from lowbit_comm_amd.hip.ring import LoopbackRing, make_pipelined_ring_transport
+
+    class Bucket:
+        def __init__(self, tensor, index=0):
+            self._tensor, self._index = tensor, index
+
+        def buffer(self):
+            return self._tensor
+
+        def index(self):
+            return self._index
+
+    world, n, g = 4, 64 * 500 + 9, 64
+    config = CompressionConfig(group_size=g, error_feedback=False)
+    fabric = LoopbackRing(world, timeout=60.0)
+    transports = [make_pipelined_ring_transport(world_size=world, rank=r, exchange=fabric.exchange_for(r))
+                  for r in range(world)]
+    hooks = [create_ddp_comm_hook(config, dtype="auto", strategy="topology", reduce="mean",
+                                  topology_all_reduce=transports[r]) for r in range(world)]
+    assert hooks[0]._ccdl_effective_strategy == "topology"
+    buckets = [torch.empty(n, device=hip_device) for _ in range(world)]
+    for step in range(2):
+        for r, bucket in enumerate(buckets):
+            bucket.copy_(tensor_like(n, "fp32", 600 + 10 * step + r, hip_device))
+        before = [to_np(b, "fp32") for b in buckets]
+        results, errors = [None] * world, [None] * world
+
+        def body(rank):
+            try:
+                torch.cuda.set_device(hip_device)
+                results[rank] = hooks[rank](None, Bucket(buckets[rank], index=3)).wait()
+            except BaseException as error:      # noqa: BLE001
+                errors[rank] = error
+                fabric.abort()
+
+        threads = [threading.Thread(target=body, args=(r,)) for r in range(world)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(120)
+        assert not any(t.is_alive() for t in threads)
+        assert errors == [None] * world, errors
+        torch.cuda.synchronize()
+        want = ring_np.ring_all_reduce(before, "fp32", g)
+        for r in range(world):
+            value = results[r][0] if isinstance(results[r], (list, tuple)) else results[r]
+            assert value.data_ptr() == buckets[r].data_ptr()
+            assert np.array_equal(raw(to_np(buckets[r], "fp32")), raw(want[r])), (step, r)
+    assert all(len(t.executors) == 1 for t in transports)
+    with pytest.raises(UnsupportedCollective, match="computes the mean"):
+        transports[0](buckets[0], config=config, op="sum")
