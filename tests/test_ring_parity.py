@@ -367,3 +367,39 @@ def test_ddp_hook_over_the_ring_transport(ops, hip_device):
     assert all(len(t.executors) == 1 for t in transports)
     with pytest.raises(UnsupportedCollective, match="computes the mean"):
         transports[0](buckets[0], config=config, op="sum")
+
+
+def test_ring_step_on_more_than_2_to_the_31_elements(hip_device):
+    """Indexing is 64-bit: a 4.3 GB bf16 chunk with a ragged tail; group-aligned windows at the start, across the
+    2^31 boundary and at the tail are compared with the oracle (a ring step is local to a group)."""
+    from lowbit_comm_amd.hip import ops
+
+    g = 64
+    n = (1 << 31) + g * 1000 + 5
+    chunk = torch.empty(n, dtype=torch.bfloat16, device=hip_device)
+    incoming = torch.empty(n, dtype=torch.bfloat16, device=hip_device)
+    step = 1 << 28
+    for i, a in enumerate(range(0, n, step)):
+        b = min(a + step, n)
+        gen = torch.Generator(device=hip_device).manual_seed(777 + i)
+        chunk[a:b] = (torch.randn(b - a, generator=gen, device=hip_device) * 2e-3).to(torch.bfloat16)
+        incoming[a:b] = (torch.randn(b - a, generator=gen, device=hip_device) * 1e-3).to(torch.bfloat16)
+    groups = ops.num_groups(n, g)
+    received = torch.empty(ops.payload_nbytes(n, g), dtype=torch.uint8, device=hip_device)
+    assert ops.quant_pack_payload_into(incoming, received, group_size=g)
+    del incoming
+    windows = [(0, 1 << 20), ((1 << 31) - g * 2000, (1 << 31) + g * 500), (n - g * 3000 - 5, n)]
+    before = [to_np(chunk[a:b], "bf16") for a, b in windows]
+    send = torch.empty_like(received)
+    assert ops.ring_step_into(received, chunk, send, group_size=g, reduce_op="sum", divisor=3.0)
+    torch.cuda.synchronize()
+    for (a, b), old in zip(windows, before):
+        assert a % g == 0
+        first, count = a // g, ops.num_groups(b - a, g)
+        codes = received[a:a + count * g].cpu().numpy().view(np.int8)
+        scales = received[groups * g + 4 * first:groups * g + 4 * (first + count)].cpu().numpy().view(np.float32)
+        want, (w_codes, w_scales) = ring_np.ring_step((codes, scales), old, "bf16", g, reduce_op="sum", divisor=3.0)
+        assert np.array_equal(to_np(chunk[a:b], "bf16"), want), (a, b)
+        assert np.array_equal(send[a:a + count * g].cpu().numpy().view(np.int8), w_codes), (a, b)
+        got_scales = send[groups * g + 4 * first:groups * g + 4 * (first + count)].cpu().numpy().view(np.uint32)
+        assert np.array_equal(got_scales, w_scales.view(np.uint32)), (a, b)
