@@ -424,16 +424,22 @@ class HipPipelinedRingRuntime:
     are kept per ``(address, numel)`` of the tensor and replayed on later runs, least recently used plans dropped
     first; the workspace session is then not asked for buffers.  One plan holds ``4 (W - 1)`` payload buffers.  All of
     a runtime's work is enqueued on its one stream, which orders the reuse of those buffers between runs.
-    ``max_plans=0``: every run leases its buffers from the workspace session."""
+    ``max_plans=0``: every run leases its buffers from the workspace session.
+
+    ``extension_status``: run the steps through the codec facade of that native module instead
+    (``quantize_tensor(view, output=...)``, ``dequantize_tensor(received, output=view, reduce_op=...)``,
+    ``view.div_(W)``), exactly the calls of the reference's runtime.  This serves every policy and payload format
+    the module does - in particular the CUDA extension's byte format, for rings that mix ranks running that
+    extension with gfx950 ranks - at the reference's launch count; chunks must then be whole groups, as there."""
 
     def __init__(self, *, config: CompressionConfig, dtype: str, world_size: int, rank: int,
                  exchange: Callable[..., Any], completion_manager: Any | None = None, stream: Any | None = None,
-                 fuse_steps: bool = True, max_plans: int = 16) -> None:
+                 fuse_steps: bool = True, max_plans: int = 16, extension_status: Any | None = None) -> None:
         from collections import OrderedDict
 
         from lowbit_comm_amd.hip.executors import fused_dequant_fallback_reason
 
-        reason = fused_dequant_fallback_reason(config)
+        reason = None if extension_status is not None else fused_dequant_fallback_reason(config)
         if reason is not None:
             raise ValueError(reason.replace("fused dequant", "the ring runtime"))
         if dtype not in ("fp32", "fp16", "bf16"):
@@ -449,7 +455,8 @@ class HipPipelinedRingRuntime:
         self.dtype = dtype
         self.world_size = world_size
         self.rank = rank
-        self.fuse_steps = bool(fuse_steps)
+        self.fuse_steps = bool(fuse_steps) and extension_status is None
+        self.extension_status = extension_status
         self.max_plans = max_plans
         self.plans: "OrderedDict[tuple[int, int], dict]" = OrderedDict()
         self._exchange = exchange
@@ -506,20 +513,26 @@ class HipPipelinedRingRuntime:
         return self._completions.record_for(context.tensor, stream=context.stream)
 
     # ---- buffers ----------------------------------------------------------- #
+    def _payload_nbytes(self, numel: int) -> int:
+        from lowbit_comm_amd.quantization.sizing import estimate_quantized_size
+
+        wire = "portable"
+        if self.extension_status is not None:
+            wire = getattr(getattr(self.extension_status, "module", None), "NATIVE_WIRE_FORMAT", "native")
+        return estimate_quantized_size(numel, dtype=self.dtype, config=self.config, wire_format=wire).quantized_bytes
+
     def _payload_buffer(self, kind: str, index: int, view: Any, workspace: Any, context: RingSubmissionContext) -> Any:
         """Send or receive buffer number ``index`` of this submission, sized for ``view``'s chunk."""
         plan = context.plan
-        if plan is not None:
-            buffer = plan.get((kind, index))
+        if plan is not None or self.extension_status is not None:      # the pool sizes portable payloads only
+            buffer = None if plan is None else plan.get((kind, index))
             if buffer is None:
                 import torch
 
-                from lowbit_comm_amd.hip import ops
-
                 with torch.cuda.stream(context.stream):
-                    buffer = torch.empty(ops.payload_nbytes(view.numel(), self.config.group_size), dtype=torch.uint8,
-                                         device=view.device)
-                plan[(kind, index)] = buffer
+                    buffer = torch.empty(self._payload_nbytes(view.numel()), dtype=torch.uint8, device=view.device)
+                if plan is not None:
+                    plan[(kind, index)] = buffer
             return buffer
         if kind == "send":
             return workspace.get_quantized_chunk(id(context.tensor), index, view, self.config, dtype=self.dtype,
@@ -539,6 +552,8 @@ class HipPipelinedRingRuntime:
         staged, context.staged = context.staged, None
         if staged is not None and staged[0] == (chunk.start, chunk.stop):
             return staged[1]
+        if self.extension_status is not None:
+            return self._facade_quantize(tensor, chunk, workspace, context)
         plan, key = context.plan, ("quantize", context.quant_index, chunk.start, chunk.stop)
         bound = None if plan is None else plan.get(key)
         if bound is None:
@@ -573,6 +588,8 @@ class HipPipelinedRingRuntime:
 
         dependency.wait_stream(context.stream)
         context.steps_done += 1
+        if self.extension_status is not None:
+            return self._facade_step(tensor, received, chunk, context, reduce_op=reduce_op, divisor=divisor)
         another_hop = context.steps_done < 2 * (self.world_size - 1)
         plan, key = context.plan, ("step", context.steps_done, chunk.start, chunk.stop, received.data_ptr())
         bound = None if plan is None else plan.get(key)
@@ -602,6 +619,49 @@ class HipPipelinedRingRuntime:
             with torch.cuda.stream(context.stream):
                 ops.true_divide_(view, divisor)
         context.staged = ((chunk.start, chunk.stop), send) if send is not None else None
+        return view
+
+    # ---- the same steps through the codec facade of a native module -------- #
+    def _whole_groups(self, view: Any) -> None:
+        from lowbit_comm_amd.exceptions import UnsupportedCollective
+
+        if view.numel() % self.config.group_size != 0:
+            raise UnsupportedCollective(
+                "topology_all_reduce",
+                reason=f"the module's in-place decode needs group-aligned chunks; numel={view.numel()}, "
+                       f"group_size={self.config.group_size}")
+
+    def _facade_quantize(self, tensor: Any, chunk: ChunkRange, workspace: Any, context: RingSubmissionContext) -> Any:
+        import torch
+
+        from lowbit_comm_amd.quantization.codec import quantize_tensor
+
+        view = _view(tensor, chunk)
+        self._whole_groups(view)
+        payload = self._send_buffer(view, workspace, context)
+        with torch.cuda.stream(context.stream):
+            quantize_tensor(view, self.config, extension_status=self.extension_status, output=payload)
+        return payload
+
+    def _facade_step(self, tensor: Any, received: Any, chunk: ChunkRange, context: RingSubmissionContext, *,
+                     reduce_op: str, divisor: float) -> Any:
+        import torch
+
+        from lowbit_comm_amd.quantization.codec import dequantize_tensor
+
+        view = _view(tensor, chunk)
+        self._whole_groups(view)
+        portable = getattr(getattr(self.extension_status, "module", None), "NATIVE_WIRE_FORMAT", "native") == "portable"
+        with torch.cuda.stream(context.stream):
+            dequantize_tensor(received, (view.numel(),), self.config, dtype=self.dtype,
+                              extension_status=self.extension_status, output=view, reduce_op=reduce_op)
+            if divisor != 1.0:
+                if portable:
+                    from lowbit_comm_amd.hip.ops import true_divide_
+
+                    true_divide_(view, divisor)      # the CPU codec's true division
+                else:
+                    view.div_(int(divisor))          # what a rank on the CUDA extension computes on its device
         return view
 
     def fused_reduce(self, tensor: Any, received: Any, chunk: ChunkRange, contributors: tuple[int, ...],
@@ -684,7 +744,8 @@ class LoopbackRing:
 def make_pipelined_ring_executor(*, config: CompressionConfig, dtype: str, numel: int, world_size: int, rank: int,
                                  exchange: Callable[..., Any], pool: Any | None = None,
                                  completion_manager: Any | None = None, device: str = "cuda:0",
-                                 fuse_steps: bool = True, max_plans: int = 16) -> PipelinedRingExecutor:
+                                 fuse_steps: bool = True, max_plans: int = 16,
+                                 extension_status: Any | None = None) -> PipelinedRingExecutor:
     """Plan, schedule, runtime, pooled workspaces and executor of one rank for buckets of ``numel`` elements."""
     from lowbit_comm_amd.hip.completion import HipCompletionManager
     from lowbit_comm_amd.hip.workspace import ShardWorkspaceProvider, create_torch_workspace_pool
@@ -693,7 +754,8 @@ def make_pipelined_ring_executor(*, config: CompressionConfig, dtype: str, numel
     plan = compile_chunk_plan(original_numel=numel, world_size=world_size)
     schedule = compile_pipelined_ring_schedule(chunk_plan=plan, rank=rank)
     runtime = HipPipelinedRingRuntime(config=config, dtype=dtype, world_size=world_size, rank=rank, exchange=exchange,
-                                      completion_manager=manager, fuse_steps=fuse_steps, max_plans=max_plans)
+                                      completion_manager=manager, fuse_steps=fuse_steps, max_plans=max_plans,
+                                      extension_status=extension_status)
     provider = ShardWorkspaceProvider(pool if pool is not None else create_torch_workspace_pool(), backend="hip",
                                       collective="all_reduce", strategy="pipelined_ring", device=device)
 

@@ -10,6 +10,9 @@ Reference lines each function follows (paths under the upstream repository):
                        contributed; ``apply_broadcast``: dequantize with reduce_op "none") followed by
                        ``quant_pack`` of the same view (:236-240, the codec of
                        ccdl_comm/quantization/torch_fallback.py:24-36)
+* ``PortableCodec`` / ``CudaWireCodec``
+                       what ``quantize_tensor`` / ``dequantize_tensor`` compute in the two payload formats (the
+                       restatements of oracle/codec_np.py and oracle/cuda_wire_general_np.py)
 * ``ring_all_reduce``  ccdl_comm/cuda/transports/pipelined_ring.py:216-275 (the order of quantize, exchange and
                        reduce on every rank) with chunk views ``tensor.reshape(-1)[start:stop]``
                        (torch_topology.py:418-419) of the plan of
@@ -33,30 +36,76 @@ import numpy as np
 from oracle import codec_np
 
 
+class PortableCodec:
+    """The portable payload ``(int8 codes, fp32 scales)`` and the CPU codec's arithmetic: decode rounded to the
+    chunk's type, sum in that type, true division (ccdl_comm/quantization/torch_fallback.py:24-53)."""
+
+    def __init__(self, group_size: int = 64) -> None:
+        self.group_size = group_size
+
+    def quantize(self, chunk: np.ndarray, dtype: str):
+        return codec_np.quantize(codec_np.widen(chunk, dtype), self.group_size)
+
+    def decode_into(self, payload, chunk: np.ndarray, dtype: str, reduce_op: str) -> np.ndarray:
+        decoded = codec_np.widen(codec_np.dequantize(payload[0], payload[1], int(chunk.size), self.group_size, dtype),
+                                 dtype)
+        if reduce_op == "none":
+            return codec_np.narrow(decoded, dtype)
+        with np.errstate(invalid="ignore", over="ignore"):
+            return codec_np.narrow(codec_np.widen(chunk, dtype) + decoded, dtype)
+
+    def divide(self, chunk: np.ndarray, dtype: str, divisor: float) -> np.ndarray:
+        with np.errstate(invalid="ignore", over="ignore"):
+            return codec_np.narrow(codec_np.widen(chunk, dtype) / np.float32(divisor), dtype)
+
+
+class CudaWireCodec:
+    """The byte format and arithmetic of the reference's CUDA extension for any of its policies
+    (oracle/cuda_wire_general_np.py); the in-place division is the one ``tensor.div_(int)`` performs on a GPU
+    tensor, a multiplication by the float32 reciprocal (torch_topology.py:287-289 runs it on the device)."""
+
+    def __init__(self, group_size: int = 64, *, bit: int = 8, quant_type: str = "linear", topk: int = 0,
+                 compact: bool = False) -> None:
+        self.group_size, self.bit, self.quant_type, self.topk, self.compact = group_size, bit, quant_type, topk, compact
+
+    def quantize(self, chunk: np.ndarray, dtype: str):
+        from oracle import cuda_wire_general_np as general
+
+        return general.quantize(chunk, dtype, self.group_size, self.bit, self.quant_type, self.topk, None,
+                                self.compact)
+
+    def decode_into(self, payload, chunk: np.ndarray, dtype: str, reduce_op: str) -> np.ndarray:
+        from oracle import cuda_wire_general_np as general
+
+        return general.dequantize(payload, int(chunk.size), dtype, self.group_size, self.bit, self.quant_type,
+                                  self.topk, self.compact, reduce_op=reduce_op, out=chunk)
+
+    def divide(self, chunk: np.ndarray, dtype: str, divisor: float) -> np.ndarray:
+        reciprocal = np.float32(1.0) / np.float32(divisor)
+        with np.errstate(invalid="ignore", over="ignore"):
+            return codec_np.narrow(codec_np.widen(chunk, dtype) * reciprocal, dtype)
+
+
 def ring_step(received, chunk: np.ndarray, dtype: str, group_size: int = 64, *, reduce_op: str = "sum",
-              divisor: float = 1.0, emit: bool = True):
-    """One compute step on one chunk.  ``received`` = ``(codes, scales)`` covering ``chunk.size`` elements;
-    ``chunk`` holds values of ``dtype`` (bf16 as uint16 bit patterns).  Returns ``(new_chunk, payload | None)``."""
+              divisor: float = 1.0, emit: bool = True, codec=None):
+    """One compute step on one chunk.  ``received`` is a payload of ``codec`` (portable: ``(codes, scales)``)
+    covering ``chunk.size`` elements; ``chunk`` holds values of ``dtype`` (bf16 as uint16 bit patterns).
+    Returns ``(new_chunk, payload | None)``."""
     if reduce_op not in ("sum", "none"):
         raise ValueError(f"unsupported reduce op {reduce_op!r}")
-    n = int(chunk.size)
-    decoded = codec_np.widen(codec_np.dequantize(received[0], received[1], n, group_size, dtype), dtype)
-    with np.errstate(invalid="ignore", over="ignore"):
-        if reduce_op == "sum":
-            value = codec_np._round_through(codec_np.widen(chunk, dtype) + decoded, dtype)
-        else:
-            value = decoded
-        if divisor != 1.0:
-            value = codec_np._round_through(value / np.float32(divisor), dtype)
-    payload = codec_np.quantize(value, group_size) if emit else None
-    return codec_np.narrow(value, dtype), payload
+    codec = codec or PortableCodec(group_size)
+    value = codec.decode_into(received, chunk, dtype, reduce_op)
+    if divisor != 1.0:
+        value = codec.divide(value, dtype, divisor)
+    return value, (codec.quantize(value, dtype) if emit else None)
 
 
-def ring_all_reduce(buckets, dtype: str, group_size: int = 64, trace: list | None = None):
+def ring_all_reduce(buckets, dtype: str, group_size: int = 64, trace: list | None = None, codec=None):
     """Mean all-reduce of ``W = len(buckets)`` equally sized flat buckets of ``dtype`` over a ring, every rank
     simulated on the host.  Returns the W result buckets (they differ between ranks: a rank keeps the unquantized
     mean of its own chunk and the decoded payloads of the others).  ``trace``, when given, receives one
     ``(phase, step, rank, sent_chunk, received_from, received_chunk)`` tuple per rank and step."""
+    codec = codec or PortableCodec(group_size)
     world = len(buckets)
     tensors = [np.array(b, copy=True).reshape(-1) for b in buckets]
     n = int(tensors[0].size)
@@ -65,7 +114,7 @@ def ring_all_reduce(buckets, dtype: str, group_size: int = 64, trace: list | Non
 
     def quantize_chunk(rank: int, index: int):
         a, b = views[index]
-        return codec_np.quantize(codec_np.widen(tensors[rank][a:b], dtype), group_size)
+        return codec.quantize(tensors[rank][a:b], dtype)
 
     carried = [(rank - 1) % world for rank in range(world)]       # chunk each rank sends next
     for phase in ("reduce", "gather"):
@@ -78,7 +127,7 @@ def ring_all_reduce(buckets, dtype: str, group_size: int = 64, trace: list | Non
                 last_reduce = phase == "reduce" and step == world - 2
                 new_chunk, _ = ring_step(payload, tensors[rank][a:b], dtype, group_size,
                                          reduce_op="sum" if phase == "reduce" else "none",
-                                         divisor=float(world) if last_reduce else 1.0, emit=False)
+                                         divisor=float(world) if last_reduce else 1.0, emit=False, codec=codec)
                 tensors[rank][a:b] = new_chunk
                 if trace is not None:
                     trace.append((phase, step, rank, sent[rank][0], source, index))

@@ -196,3 +196,29 @@ def test_the_owner_keeps_the_unquantized_mean_and_its_successor_the_quantized_on
         nxt = results[(owner + 1) % world][a:b]
         assert np.array_equal(nxt, codec_np.dequantize(codes, scales, 64, g, "fp32"))
         assert not np.array_equal(nxt, own)
+
+
+@pytest.mark.parametrize("compact", [False, True])
+@pytest.mark.parametrize("world, n, g", [(2, 64 * 6, 64), (4, 4 * 32 * 5, 32), (8, 8 * 16 * 3, 16)])
+def test_ring_in_the_cuda_byte_format_returns_the_exact_mean_on_lossless_inputs(world, n, g, compact):
+    """Same construction in the other payload format: a group maximum of 127 * 2^j * K is stored exactly, the
+    extreme codes are +-127 and decode by (scale / 127) = 2^j * K exactly."""
+    rng = np.random.default_rng(world * 77 + n)
+    buckets, exact_sum = lossless_buckets(world, n, g, rng)
+    codec = ring_np.CudaWireCodec(g, compact=compact)
+    results = ring_np.ring_all_reduce(buckets, "fp32", g, codec=codec)
+    want = (exact_sum / world).astype(np.float32)
+    for rank in range(world):
+        assert np.array_equal(results[rank], want), rank
+
+
+def test_the_two_codecs_divide_differently_where_the_reference_does():
+    """True division on the CPU codec's path, multiplication by the float32 reciprocal where the division runs
+    on the device: they differ in the last bit for some inputs when W is not a power of two."""
+    x = np.arange(1, 4001, dtype=np.float32)
+    exact = ring_np.PortableCodec().divide(x, "fp32", 3.0)
+    device = ring_np.CudaWireCodec().divide(x, "fp32", 3.0)
+    assert np.array_equal(exact, (x / np.float32(3.0)).astype(np.float32))
+    assert np.array_equal(device, (x * (np.float32(1.0) / np.float32(3.0))).astype(np.float32))
+    assert 0 < np.count_nonzero(exact != device) < x.size
+    assert np.array_equal(ring_np.PortableCodec().divide(x, "fp32", 8.0), ring_np.CudaWireCodec().divide(x, "fp32", 8.0))

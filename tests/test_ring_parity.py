@@ -184,16 +184,16 @@ def test_ring_step_at_the_config4_chunk_size_keeps_the_sum_property(ops, hip_dev
 # --------------------------------------------------------------------------- #
 # the whole ring: every rank on one device, one host thread per rank
 # --------------------------------------------------------------------------- #
-def build_ring(device, world, n, dtype, g, fuse_steps, pools=None, max_plans=16):
+def build_ring(device, world, n, dtype, g, fuse_steps, pools=None, max_plans=16, config=None, extension_status=None):
     from lowbit_comm_amd.config import CompressionConfig
     from lowbit_comm_amd.hip.ring import LoopbackRing, make_pipelined_ring_executor
 
     fabric = LoopbackRing(world, timeout=60.0)
-    config = CompressionConfig(group_size=g)
+    config = config or CompressionConfig(group_size=g)
     executors = [make_pipelined_ring_executor(config=config, dtype=dtype, numel=n, world_size=world, rank=r,
                                               exchange=fabric.exchange_for(r), fuse_steps=fuse_steps,
                                               pool=None if pools is None else pools[r], device=str(device),
-                                              max_plans=max_plans)
+                                              max_plans=max_plans, extension_status=extension_status)
                  for r in range(world)]
     return fabric, executors
 
@@ -403,3 +403,53 @@ def test_ring_step_on_more_than_2_to_the_31_elements(hip_device):
         assert np.array_equal(send[a:a + count * g].cpu().numpy().view(np.int8), w_codes), (a, b)
         got_scales = send[groups * g + 4 * first:groups * g + 4 * (first + count)].cpu().numpy().view(np.uint32)
         assert np.array_equal(got_scales, w_scales.view(np.uint32)), (a, b)
+
+
+POLICIES = [dict(), dict(compact=True), dict(bit=4, allow_experimental=True), dict(topk=2),
+            dict(bit=4, quant_type="normal", allow_experimental=True)]
+
+
+@pytest.mark.parametrize("policy", POLICIES, ids=lambda p: "-".join(f"{k}={v}" for k, v in p.items()) or "linear8")
+@pytest.mark.parametrize("dtype, world, g", [("fp32", 4, 64), ("bf16", 3, 32), ("fp16", 8, 16)])
+def test_ring_through_the_codec_facade_in_the_cuda_byte_format(hip_device, policy, dtype, world, g):
+    """The runtime's facade mode over the module that speaks the CUDA extension's bytes: every hop is the
+    reference's own sequence of calls, for policies the ring-step kernel does not serve; every rank's bucket
+    equals the oracle's ring over the CUDA-format codec, bit for bit."""
+    from lowbit_comm_amd.config import CompressionConfig
+    from lowbit_comm_amd.hip.loader import load_hip_extension
+
+    status = load_hip_extension(wire_format="native")
+    assert status.available, status.reason
+    config = CompressionConfig(group_size=g, error_feedback=False, **policy)
+    n = world * g * 37
+    buckets = [tensor_like(n, dtype, 9100 + 3 * r, hip_device, sigma=10.0 ** (r % 2 - 3)) for r in range(world)]
+    before = [to_np(b, dtype) for b in buckets]
+    ring = build_ring(hip_device, world, n, dtype, g, True, config=config, extension_status=status)
+    assert all(e._runtime.fuse_steps is False for e in ring[1])
+    run_ring(hip_device, buckets, dtype, g, True, ring=ring)
+    codec = ring_np.CudaWireCodec(g, bit=config.bit, quant_type=config.quant_type, topk=config.topk,
+                                  compact=config.compact)
+    want = ring_np.ring_all_reduce(before, dtype, g, codec=codec)
+    for rank in range(world):
+        assert np.array_equal(raw(to_np(buckets[rank], dtype)), raw(want[rank])), (rank, policy, dtype)
+
+
+def test_ring_through_the_facade_of_the_portable_module_equals_the_fused_ring(hip_device):
+    from lowbit_comm_amd.exceptions import UnsupportedCollective
+    from lowbit_comm_amd.hip.loader import load_hip_extension
+
+    status = load_hip_extension(wire_format="portable")
+    world, g = 3, 64
+    n = world * g * 50
+    start = [tensor_like(n, "fp32", 9300 + r, hip_device) for r in range(world)]
+    fused = [b.clone() for b in start]
+    facade = [b.clone() for b in start]
+    run_ring(hip_device, fused, "fp32", g, True)
+    run_ring(hip_device, facade, "fp32", g, True, ring=build_ring(hip_device, world, n, "fp32", g, True,
+                                                                 extension_status=status))
+    for a, b in zip(fused, facade):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    ragged = [tensor_like(n + 5, "fp32", 9400 + r, hip_device) for r in range(world)]
+    with pytest.raises(UnsupportedCollective, match="group-aligned chunks"):
+        run_ring(hip_device, ragged, "fp32", g, True, ring=build_ring(hip_device, world, n + 5, "fp32", g, True,
+                                                                      extension_status=status))
