@@ -187,19 +187,41 @@ class ReduceScatterPlan:
 
 
 def compressed_reduce_scatter_shard(tensor: torch.Tensor, *, config: CompressionConfig, world_size: int, rank: int,
-                                    all_to_all: Callable[[torch.Tensor, torch.Tensor], None], op: str = "sum",
-                                    plan: ReduceScatterPlan | None = None) -> ReducedShard:
+                                    all_to_all: Callable[[torch.Tensor, torch.Tensor], Any], op: str = "sum",
+                                    plan: ReduceScatterPlan | None = None, async_op: bool = False,
+                                    future_factory: Callable[[], Any] | None = None,
+                                    completion_manager: Any | None = None,
+                                    update_feedback: Callable[[ReducedShard], None] | None = None,
+                                    advance_policy: Callable[[], None] | None = None) -> Any:
     """Quantize per-destination chunks, exchange, reduce: returns this rank's :class:`ReducedShard`.
 
     ``all_to_all(received_rows, send_rows)`` must fill row ``r`` of ``received_rows`` with rank ``r``'s
     payload for this rank (row ``rank`` of ``send_rows`` of that rank) - the one collective of the leg.
+
+    ``async_op``: ``all_to_all`` starts the exchange and returns its work object (``wait()``, optionally
+    ``get_future()``), e.g. ``dist.all_to_all_single(received, send, async_op=True)``; the call returns an
+    :class:`~lowbit_comm_amd.communication.AsyncShardPipeline` that reduces the shard when the exchange is over
+    and completes a future (``future_factory``, default ``torch.futures.Future``) with it
+    (``ccdl_comm/communication/reduce_scatter_transport.py:286-333``).
     """
     if plan is None:
         plan = ReduceScatterPlan(tensor.numel(), tensor.dtype, world_size=world_size, rank=rank, config=config,
                                  device=tensor.device, shape=tuple(tensor.shape))
     send = plan.quantize_chunks(tensor)
-    all_to_all(plan.received, send)
-    return plan.reduce_received(op=op)
+    if not async_op:
+        all_to_all(plan.received, send)
+        return plan.reduce_received(op=op)
+    from lowbit_comm_amd.communication.async_shard_pipeline import AsyncShardPipeline
+
+    exchange = all_to_all(plan.received, send)
+    if not callable(getattr(exchange, "wait", None)):
+        raise TypeError("with async_op the exchange must return a work object with wait()")
+    future = future_factory() if future_factory is not None else torch.futures.Future()
+    return AsyncShardPipeline(communication_work=exchange, future=future,
+                              reduce_shard=lambda _received: plan.reduce_received(op=op),
+                              update_feedback=update_feedback or (lambda _shard: None),
+                              advance_policy=advance_policy or (lambda: None),
+                              completion_manager=completion_manager, resources=(tensor, plan, send)).run()
 
 
 def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: CompressionConfig, world_size: int,

@@ -383,6 +383,63 @@ def test_reduce_scatter_all_gather_plan_matches_the_oracle(dev, n, world):
     assert np.array_equal(out.cpu().numpy().view(np.uint32), want_full.view(np.uint32))
 
 
+def test_asynchronous_shard_exchange_completes_through_the_pipeline(dev):
+    """``compressed_reduce_scatter_shard(async_op=True)``: the exchange returns a work object, the shard is reduced
+    when its future fires and arrives through a torch future, bit-identical to the synchronous call."""
+    from lowbit_comm_amd.communication import AsyncShardPipeline
+    from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan, compressed_reduce_scatter_shard
+
+    world, n = 4, 64 * 4 * 300 + 11
+    buckets = [grad(n, torch.float32, 950 + r, dev) for r in range(world)]
+    plans = [ReduceScatterPlan(n, torch.float32, world_size=world, rank=r, config=CFG, device=dev) for r in range(world)]
+    for plan, bucket in zip(plans[1:], buckets[1:]):
+        plan.quantize_chunks(bucket)
+
+    def copy_rows(received, send):
+        received[0].copy_(send[0])
+        for src in range(1, world):
+            received[src].copy_(plans[src].send[0])
+
+    class StartedExchange:
+        """Stands in for the work of ``all_to_all_single(..., async_op=True)``: the copies are enqueued when the
+        exchange starts; the future fires when the test lets it."""
+
+        def __init__(self):
+            self.future = torch.futures.Future()
+            self.waited = 0
+
+        def get_future(self):
+            return self.future
+
+        def wait(self):
+            self.waited += 1
+
+    started = []
+
+    def start(received, send):
+        copy_rows(received, send)
+        started.append(StartedExchange())
+        return started[-1]
+
+    want = compressed_reduce_scatter_shard(buckets[0], config=CFG, world_size=world, rank=0, all_to_all=copy_rows)
+    want_bits = want.shard.clone()
+    advanced, fed = [], []
+    work = compressed_reduce_scatter_shard(buckets[0], config=CFG, world_size=world, rank=0, all_to_all=start,
+                                           plan=plans[0], async_op=True, update_feedback=fed.append,
+                                           advance_policy=lambda: advanced.append(True))
+    assert isinstance(work, AsyncShardPipeline) and work.query() is False and not fed
+    assert buckets[0] in work.resources
+    started[0].future.set_result(None)                          # the exchange is over
+    assert work.query() is True and started[0].waited == 1 and advanced == [True]
+    shard = work.wait()
+    assert shard is fed[0] and shard.metadata["async_completion"] is True and shard.shard_index == 0
+    torch.cuda.synchronize()
+    assert same_bits(shard.shard, want_bits.cpu())
+    with pytest.raises(TypeError, match="must return a work object"):
+        compressed_reduce_scatter_shard(buckets[0], config=CFG, world_size=world, rank=0, all_to_all=copy_rows,
+                                        plan=plans[0], async_op=True)
+
+
 def test_reduce_scatter_plan_fused_requantize_matches_the_two_steps(hip_device):
     from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan, compressed_all_reduce_via_reduce_scatter
 
