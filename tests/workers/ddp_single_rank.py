@@ -1,7 +1,7 @@
 """Worker for tests/test_hip_host.py: the compressed hook registered on a real DistributedDataParallel model.
 
 One process, one GPU, a one-rank RCCL process group.  Modes "portable" / "native": the all_gather strategy in that
-wire format (the all-gather of a one-rank world is the identity, injected as such).  Mode "reduce_scatter": the
+wire format, the packed payload bytes moved by a real RCCL ``all_gather_into_tensor``.  Mode "reduce_scatter": the
 pre-bound reduce-scatter plan with its two exchanges as real RCCL calls (all_to_all_single, all_gather_into_tensor)
 and local error feedback.  Prints one JSON line with the gradient errors against an unwrapped copy of the model.
 """
@@ -51,8 +51,15 @@ def main() -> int:
         seen = []
 
         def gather(payload):
-            seen.append(int(payload.buffer.numel()))
-            return GatheredPayloads(payloads=[payload], world_size=1)
+            """The packed payload bytes through a real RCCL all-gather; row r is rank r's payload."""
+            from dataclasses import replace
+
+            mine = payload.buffer.reshape(-1)
+            seen.append(int(mine.numel()))
+            world = dist.get_world_size()
+            rows = torch.empty((world, mine.numel()), dtype=mine.dtype, device=mine.device)
+            dist.all_gather_into_tensor(rows, mine)
+            return GatheredPayloads(payloads=[replace(payload, buffer=rows[r]) for r in range(world)], world_size=world)
 
         if wire_format == "reduce_scatter":
             from lowbit_comm_amd.hip.reduce_scatter import make_reduce_scatter_transport
