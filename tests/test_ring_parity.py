@@ -453,3 +453,24 @@ def test_ring_through_the_facade_of_the_portable_module_equals_the_fused_ring(hi
     with pytest.raises(UnsupportedCollective, match="group-aligned chunks"):
         run_ring(hip_device, ragged, "fp32", g, True, ring=build_ring(hip_device, world, n + 5, "fp32", g, True,
                                                                       extension_status=status))
+
+
+def test_ring_step_randomized_sweep(ops, hip_device):
+    """Random sizes (ragged, tiny, block-boundary), groups, dtypes, ops, divisors, view offsets; every case
+    bit-exact against the oracle.  ``LBC_SWEEP_CASES`` / ``LBC_SWEEP_SEED`` widen or reseed the sweep."""
+    import os
+    import random
+
+    cases = int(os.environ.get("LBC_SWEEP_CASES", "150"))
+    rng = random.Random(int(os.environ.get("LBC_SWEEP_SEED", "2024")))
+    edges = [1, 63, 64, 65, 1023, 1024, 4095, 4096, 4097, 8192, 16384, 16385, 65536]
+    for case in range(cases):
+        dtype = rng.choice(["fp32", "fp16", "bf16"])
+        g = rng.choice([16, 32, 64])
+        n = rng.choice(edges) + rng.choice([0, 0, 1, -1, 7, 100]) if rng.random() < 0.5 else rng.randint(1, 200_000)
+        n = max(1, n)
+        reduce_op = rng.choice(["sum", "sum", "none"])
+        divisor = rng.choice([1.0, 1.0, 2.0, 3.0, 8.0, 7.0])
+        emit = rng.random() < 0.7
+        offset = rng.choice([0, 0, 0, 1, 2, 5])
+        check_step(ops, hip_device, dtype, g, n, reduce_op, divisor, emit, 50_000 + 3 * case, offset=offset)
