@@ -12,6 +12,7 @@ from .ring import (
     compile_pipelined_ring_schedule,
     make_pipelined_ring_executor,
 )
+from .tree import HipTreeRuntime, LoopbackMesh, TreeEdge, TreeExecutor, TreeSchedule, compile_tree_schedule, make_tree_executor
 from .workspace import (
     CudaOutputLease,
     CudaShardWorkspaceProvider,
@@ -34,7 +35,8 @@ __all__ = [
     "CudaWorkspacePool", "EventCompletion", "EventCompletionManager", "HipCompletionManager", "HipExtensionStatus",
     "HipOutputLease", "HipPipelinedRingRuntime", "HipStreamWork", "JoinedCompletion", "LoopbackRing",
     "PipelinedRingExecutor", "PipelinedRingSchedule", "RingAllGatherStep", "RingReduceScatterStep",
-    "compile_pipelined_ring_schedule", "make_pipelined_ring_executor",
+    "compile_pipelined_ring_schedule", "make_pipelined_ring_executor", "HipTreeRuntime", "LoopbackMesh", "TreeEdge",
+    "TreeExecutor", "TreeSchedule", "compile_tree_schedule", "make_tree_executor",
     "HipWorkspacePool", "ShardWorkspaceProvider", "ShardWorkspaceSession", "WorkspaceKey", "WorkspaceLease",
     "WorkspaceStats", "create_torch_workspace_pool", "load_cuda_extension", "load_hip_extension",
 ]

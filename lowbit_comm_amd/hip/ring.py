@@ -239,20 +239,22 @@ class _Submission:
             self.keep(*leases)
 
 
-class PipelinedRingExecutor:
+class TopologyExecutor:
     """Enqueues the whole schedule of one rank without waiting on the host and returns completion-backed work.
 
-    ``runtime`` provides ``create_submission_context``, ``wait_for_producer``, ``quant_pack``, ``send_recv``,
-    ``fused_reduce``, ``apply_broadcast`` and ``record_completion`` (the protocol of pipelined_ring.py:113-171);
-    ``workspace_session_factory(tensor)`` a session with ``release(completion=)`` and optionally ``abort()``;
+    ``workspace_session_factory(tensor)`` gives a session with ``release(completion=)`` and optionally ``abort()``;
     ``completion_manager.create_work(result=, completion=, resources=)`` the work object.  A submission that fails
     after device work was enqueued keeps its buffers until that work has drained (``reap_pending``), then aborts
-    the session instead of releasing it."""
+    the session instead of releasing it (the ownership rules of
+    ``ccdl_comm/cuda/transports/_executor_support.py:121-257``).  Subclasses say what a schedule is and enqueue its
+    steps in :meth:`_enqueue`."""
 
-    def __init__(self, *, schedule: PipelinedRingSchedule, runtime: Any,
-                 workspace_session_factory: Callable[[Any], Any], completion_manager: Any) -> None:
-        if not isinstance(schedule, PipelinedRingSchedule):
-            raise TypeError("schedule must be a PipelinedRingSchedule")
+    schedule_type: type = object
+
+    def __init__(self, *, schedule: Any, runtime: Any, workspace_session_factory: Callable[[Any], Any],
+                 completion_manager: Any) -> None:
+        if not isinstance(schedule, self.schedule_type):
+            raise TypeError(f"schedule must be a {self.schedule_type.__name__}")
         if not callable(workspace_session_factory):
             raise TypeError("workspace_session_factory must be callable")
         self.schedule = schedule
@@ -290,31 +292,16 @@ class PipelinedRingExecutor:
         _require_endpoint(context, "submission context")
         submission = _Submission(tensor=tensor, workspace=self._sessions(tensor), context=context)
         try:
-            workspace = submission.workspace
             runtime.wait_for_producer(tensor, context=context)
-            for step in self.schedule.steps:
-                received, handle = self._exchange(submission, step)
-                submission.after(runtime.fused_reduce(tensor, received, step.recv_chunk, step.received_contributors,
-                                                      workspace, context=context, dependency=handle))
-            for step in self.schedule.gather_steps:
-                received, handle = self._exchange(submission, step)
-                submission.after(runtime.apply_broadcast(tensor, received, step.recv_chunk, workspace,
-                                                         context=context, dependency=handle))
+            self._enqueue(submission)
             self._record(submission)
             return self._finish(submission)
         except BaseException:
             self._fail(submission)
             raise
 
-    def _exchange(self, submission: _Submission, step: Any) -> tuple[Any, Any]:
-        runtime, context, workspace = self._runtime, submission.context, submission.workspace
-        payload = runtime.quant_pack(submission.tensor, step.send_chunk, workspace, context=context)
-        submission.keep(payload)
-        received, handle = runtime.send_recv(payload, send_peer=step.send_peer, recv_peer=step.recv_peer,
-                                             recv_chunk=step.recv_chunk, workspace=workspace, context=context)
-        submission.keep(received)
-        submission.after_p2p(handle)
-        return received, handle
+    def _enqueue(self, submission: _Submission) -> None:
+        raise NotImplementedError
 
     def _record(self, submission: _Submission) -> None:
         submission.record_attempted = True
@@ -376,6 +363,34 @@ class PipelinedRingExecutor:
                 except BaseException:
                     continue
             self._pending.remove(submission)
+
+
+class PipelinedRingExecutor(TopologyExecutor):
+    """The ring: per hop ``quant_pack``, ``send_recv``, then ``fused_reduce`` (first phase) or ``apply_broadcast``
+    (second phase) - the runtime protocol and call order of ``ccdl_comm/cuda/transports/pipelined_ring.py:113-275``."""
+
+    schedule_type = PipelinedRingSchedule
+
+    def _enqueue(self, submission: _Submission) -> None:
+        runtime, tensor, context, workspace = self._runtime, submission.tensor, submission.context, submission.workspace
+        for step in self.schedule.steps:
+            received, handle = self._exchange(submission, step)
+            submission.after(runtime.fused_reduce(tensor, received, step.recv_chunk, step.received_contributors,
+                                                  workspace, context=context, dependency=handle))
+        for step in self.schedule.gather_steps:
+            received, handle = self._exchange(submission, step)
+            submission.after(runtime.apply_broadcast(tensor, received, step.recv_chunk, workspace,
+                                                     context=context, dependency=handle))
+
+    def _exchange(self, submission: _Submission, step: Any) -> tuple[Any, Any]:
+        runtime, context, workspace = self._runtime, submission.context, submission.workspace
+        payload = runtime.quant_pack(submission.tensor, step.send_chunk, workspace, context=context)
+        submission.keep(payload)
+        received, handle = runtime.send_recv(payload, send_peer=step.send_peer, recv_peer=step.recv_peer,
+                                             recv_chunk=step.recv_chunk, workspace=workspace, context=context)
+        submission.keep(received)
+        submission.after_p2p(handle)
+        return received, handle
 
 
 # --------------------------------------------------------------------------- #
@@ -583,14 +598,17 @@ class HipPipelinedRingRuntime:
         return received, handle
 
     def _step(self, tensor: Any, received: Any, chunk: ChunkRange, workspace: Any, context: RingSubmissionContext,
-              dependency: Any, *, reduce_op: str, divisor: float) -> Any:
+              dependency: Any, *, reduce_op: str, divisor: float, another_hop: bool | None = None) -> Any:
+        """``another_hop``: the updated chunk is sent on before anything else changes it, so its payload is worth
+        producing in the same launch (default: every hop of a ring but the last)."""
         from lowbit_comm_amd.hip import ops
 
         dependency.wait_stream(context.stream)
         context.steps_done += 1
         if self.extension_status is not None:
             return self._facade_step(tensor, received, chunk, context, reduce_op=reduce_op, divisor=divisor)
-        another_hop = context.steps_done < 2 * (self.world_size - 1)
+        if another_hop is None:
+            another_hop = context.steps_done < 2 * (self.world_size - 1)
         plan, key = context.plan, ("step", context.steps_done, chunk.start, chunk.stop, received.data_ptr())
         bound = None if plan is None else plan.get(key)
         if bound is None:

@@ -1,4 +1,4 @@
-"""CPU oracle (numpy) for the quantized ring all-reduce.  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle (numpy) for the quantized ring and tree all-reduce.  TEST INFRASTRUCTURE ONLY.
 
 Only tests, the smoke check and the CPU-baseline leg of the benchmark may import this module; the product never
 routes through it.
@@ -18,6 +18,9 @@ Reference lines each function follows (paths under the upstream repository):
                        (torch_topology.py:418-419) of the plan of
                        ccdl_comm/cuda/transports/compressed_reduce_scatter.py:72-94
 
+* ``tree_edges`` / ``tree_all_reduce``
+                       ccdl_comm/cuda/transports/tree.py:196-306 and torch_topology.py:319-415
+
 ``ring_all_reduce`` does not restate the schedule compiler's index formulas (pipelined_ring.py:298-331).  It
 passes messages: every rank sends to its successor the chunk it has just received into, starting with the
 chunk of its predecessor's index, which is the one rule under which rank r ends the first W-1 steps holding the
@@ -27,7 +30,10 @@ Pinning (tests/test_ring_oracle.py): ``ring_step`` against Python-float brute fo
 the composition of the separately pinned ``dequantize`` / ``quantize``; ``ring_all_reduce`` on inputs built so
 that every quantization on the way is lossless, where the result must equal the exact mean on every rank (a
 wrong peer, chunk, contributor count or a second division fails it), on world sizes 1 to 8 with ragged and
-empty chunks, and against the error bound of W-1 successive quantizations on random inputs.
+empty chunks, and against the error bound of W-1 successive quantizations on random inputs; ``tree_edges`` against
+the edge list the reference's test spells out for five ranks and the properties it states for every root (each
+rank once, connected, acyclic), ``tree_all_reduce`` on the same lossless construction and by following the mean
+down the levels.
 """
 from __future__ import annotations
 
@@ -132,4 +138,31 @@ def ring_all_reduce(buckets, dtype: str, group_size: int = 64, trace: list | Non
                 if trace is not None:
                     trace.append((phase, step, rank, sent[rank][0], source, index))
                 carried[rank] = index
+    return tensors
+
+
+def tree_edges(world: int, root: int = 0):
+    """``(child, parent)`` pairs of the reference's tree (ccdl_comm/cuda/transports/tree.py:297-306): the ranks
+    form a binary heap counted from the root, and the edges are listed from the last heap position up to the
+    root's first child, so a rank's own children come before its edge to its parent."""
+    at = [(root + position) % world for position in range(world)]
+    return [(at[position], at[(position - 1) // 2]) for position in range(world - 1, 0, -1)]
+
+
+def tree_all_reduce(buckets, dtype: str, group_size: int = 64, codec=None, root: int = 0):
+    """Mean all-reduce over that tree, every rank simulated on the host (TreeExecutor,
+    ccdl_comm/cuda/transports/tree.py:196-281, with TorchTreeRuntime, torch_topology.py:319-415): each edge carries
+    the child's whole bucket, quantized, to the parent, which adds it in the bucket's type; the root divides by W
+    before its first send down; the mean descends the edges in reverse order, quantized again at every level.
+    The root keeps the unquantized mean."""
+    codec = codec or PortableCodec(group_size)
+    world = len(buckets)
+    tensors = [np.array(b, copy=True).reshape(-1) for b in buckets]
+    edges = tree_edges(world, root)
+    for child, parent in edges:
+        tensors[parent] = codec.decode_into(codec.quantize(tensors[child], dtype), tensors[parent], dtype, "sum")
+    if edges:
+        tensors[root] = codec.divide(tensors[root], dtype, float(world))
+    for child, parent in reversed(edges):
+        tensors[child] = codec.decode_into(codec.quantize(tensors[parent], dtype), tensors[child], dtype, "none")
     return tensors

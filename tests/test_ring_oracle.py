@@ -222,3 +222,77 @@ def test_the_two_codecs_divide_differently_where_the_reference_does():
     assert np.array_equal(device, (x * (np.float32(1.0) / np.float32(3.0))).astype(np.float32))
     assert 0 < np.count_nonzero(exact != device) < x.size
     assert np.array_equal(ring_np.PortableCodec().divide(x, "fp32", 8.0), ring_np.CudaWireCodec().divide(x, "fp32", 8.0))
+
+
+# --------------------------------------------------------------------------- #
+# tree
+# --------------------------------------------------------------------------- #
+def test_tree_edges_of_five_ranks_are_the_ones_the_reference_test_spells_out():
+    """tests/cuda/test_topology_executors.py:1711-1745 names, for five ranks and root 0, the reduce edges in
+    order: 4->1, 3->1, 2->0, 1->0."""
+    assert ring_np.tree_edges(5, 0) == [(4, 1), (3, 1), (2, 0), (1, 0)]
+    assert ring_np.tree_edges(1, 0) == []
+    assert ring_np.tree_edges(2, 1) == [(0, 1)]
+
+
+@pytest.mark.parametrize("world", [2, 3, 5, 8, 13])
+def test_tree_reaches_every_rank_once_without_cycles_for_every_root(world):
+    for root in range(world):
+        edges = ring_np.tree_edges(world, root)
+        parents = dict(edges)
+        assert len(edges) == world - 1 and set(parents) == set(range(world)) - {root}
+        for child in parents:
+            seen, at = set(), child
+            while at != root:
+                assert at not in seen
+                seen.add(at)
+                at = parents[at]
+        position = {rank: k for k, rank in enumerate([child for child, _ in edges])}
+        for child, parent in edges:                      # a rank's children are listed before its own edge up
+            if parent != root:
+                assert position[child] < position[parent]
+        assert all(sum(1 for _, p in edges if p == rank) <= 2 for rank in range(world))
+
+
+def whole_bucket_lossless(world, n, g, rng):
+    signs = rng.choice(np.array([-1.0, 1.0], dtype=np.float32), size=n)
+    local = np.arange(n) // g
+    groups = int(local[-1]) + 1
+    base = signs * np.float32(127.0) * np.exp2(rng.integers(-12, 4, size=groups)[local]).astype(np.float32)
+    factors = np.stack([rng.integers(1, 6, size=groups)[local] for _ in range(world)])
+    buckets = [(base * factors[r].astype(np.float32)).astype(np.float32) for r in range(world)]
+    return buckets, base.astype(np.float64) * factors.sum(axis=0)
+
+
+@pytest.mark.parametrize("codec", ["portable", "cuda"])
+@pytest.mark.parametrize("world, n, g, root", [(2, 64 * 3, 64, 0), (4, 32 * 9, 32, 3), (8, 16 * 21, 16, 5)])
+def test_tree_all_reduce_returns_the_exact_mean_when_every_quantization_is_lossless(world, n, g, root, codec):
+    rng = np.random.default_rng(world * 31 + root)
+    buckets, exact_sum = whole_bucket_lossless(world, n, g, rng)
+    active = ring_np.PortableCodec(g) if codec == "portable" else ring_np.CudaWireCodec(g, compact=True)
+    results = ring_np.tree_all_reduce(buckets, "fp32", g, codec=active, root=root)
+    want = (exact_sum / world).astype(np.float32)
+    assert np.array_equal(want.astype(np.float64), exact_sum / world)
+    for rank in range(world):
+        assert np.array_equal(results[rank], want), rank
+
+
+def test_tree_keeps_the_unquantized_mean_at_the_root_and_quantizes_once_per_level():
+    world, n, g, root = 5, 16 * 40 + 3, 16, 2
+    rng = np.random.default_rng(9)
+    buckets = [rng.standard_normal(n).astype(np.float32) for _ in range(world)]
+    results = ring_np.tree_all_reduce(buckets, "fp32", g, root=root)
+    parents = dict(ring_np.tree_edges(world, root))
+    for rank in range(world):
+        if rank == root:
+            continue
+        above = results[parents[rank]]
+        codes, scales = codec_np.quantize(above, g)
+        assert np.array_equal(results[rank], codec_np.dequantize(codes, scales, n, g, "fp32")), rank
+    first_child = next(child for child, parent in parents.items() if parent == root)
+    assert not np.array_equal(results[root], results[first_child])
+    exact = np.mean([b.astype(np.float64) for b in buckets], axis=0)
+    peak = sum(float(np.max(np.abs(b))) for b in buckets)
+    assert np.max(np.abs(results[root].astype(np.float64) - exact)) <= 3 * peak / 254 / world * world
+    single = ring_np.tree_all_reduce([buckets[0]], "fp32", g)
+    assert np.array_equal(single[0], buckets[0])
