@@ -1,0 +1,160 @@
+// A host program with no Python and no torch in it: allocates with the HIP runtime, calls the codec through the
+// C ABI of include/lbc.h on a stream of its own, and compares every byte with the scalar C oracle
+// (oracle/codec_scalar.c, linked from oracle/_build).  Built by __graft_entry__.build(), run by
+// tests/test_abi_client.py on the GPU box.  Prints "OK <checks>" or the first mismatch.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <vector>
+
+#include "../../include/lbc.h"
+
+extern "C" {
+void lbo_quantize_f32(const float *x, int64_t n, int group_size, int8_t *codes, float *scales);
+void lbo_reduce_f32(const int8_t *const *codes, const float *const *scales, int world, int64_t n, int group_size,
+                    float divisor, float *out);
+}
+
+#define HIP_OK(call)                                                                       \
+    do {                                                                                   \
+        hipError_t status_ = (call);                                                       \
+        if (status_ != hipSuccess) {                                                       \
+            printf("FAIL %s: %s\n", #call, hipGetErrorString(status_));                    \
+            return 2;                                                                      \
+        }                                                                                  \
+    } while (0)
+
+#define LBC_OK_OR_FAIL(call)                                                               \
+    do {                                                                                   \
+        int status_ = (call);                                                              \
+        if (status_ != LBC_OK) {                                                           \
+            printf("FAIL %s -> %d: %s\n", #call, status_, lbc_last_error());               \
+            return 3;                                                                      \
+        }                                                                                  \
+    } while (0)
+
+static uint32_t lcg(uint32_t &state) {
+    state = state * 1664525u + 1013904223u;
+    return state;
+}
+
+// roughly normal values of standard deviation `sigma` (sum of four uniforms), with a few large outliers
+static void fill(std::vector<float> &x, uint32_t seed, float sigma) {
+    uint32_t s = seed;
+    for (size_t i = 0; i < x.size(); ++i) {
+        float u = 0.0f;
+        for (int k = 0; k < 4; ++k) u += static_cast<float>(lcg(s) >> 8) * (1.0f / 16777216.0f) - 0.5f;
+        x[i] = u * 1.7320508f * sigma;
+        if ((lcg(s) & 1023u) == 0u) x[i] *= 100.0f;
+    }
+}
+
+int main() {
+    if (lbc_abi_version() != LBC_ABI_VERSION) {
+        printf("FAIL abi version %d, header %d\n", lbc_abi_version(), LBC_ABI_VERSION);
+        return 1;
+    }
+    const int world = 4, g = 64;
+    const int64_t n = 64 * 3000 + 37;   // ragged tail
+    const int64_t groups = (n + g - 1) / g, padded = groups * g;
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+
+    std::vector<std::vector<float>> x(world, std::vector<float>(n));
+    std::vector<std::vector<int8_t>> want_codes(world, std::vector<int8_t>(padded));
+    std::vector<std::vector<float>> want_scales(world, std::vector<float>(groups));
+    float *d_x = nullptr, *d_out = nullptr;
+    std::vector<int8_t *> d_codes(world, nullptr);
+    std::vector<float *> d_scales(world, nullptr);
+    HIP_OK(hipMalloc(&d_x, n * sizeof(float)));
+    HIP_OK(hipMalloc(&d_out, n * sizeof(float)));
+    long checks = 0;
+    for (int r = 0; r < world; ++r) {
+        fill(x[r], 1234u + 17u * r, 1e-3f * (r + 1));
+        lbo_quantize_f32(x[r].data(), n, g, want_codes[r].data(), want_scales[r].data());
+        HIP_OK(hipMalloc(&d_codes[r], padded));
+        HIP_OK(hipMalloc(&d_scales[r], groups * sizeof(float)));
+        HIP_OK(hipMemcpyAsync(d_x, x[r].data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
+        LBC_OK_OR_FAIL(lbc_quant_pack(d_x, LBC_F32, nullptr, LBC_NONE, n, g, d_codes[r], d_scales[r], nullptr, LBC_NONE,
+                                      nullptr, LBC_NONE, stream));
+        std::vector<int8_t> codes(padded);
+        std::vector<float> scales(groups);
+        HIP_OK(hipMemcpyAsync(codes.data(), d_codes[r], padded, hipMemcpyDeviceToHost, stream));
+        HIP_OK(hipMemcpyAsync(scales.data(), d_scales[r], groups * sizeof(float), hipMemcpyDeviceToHost, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        if (memcmp(codes.data(), want_codes[r].data(), padded) != 0) {
+            printf("FAIL codes of payload %d differ from the oracle\n", r);
+            return 4;
+        }
+        if (memcmp(scales.data(), want_scales[r].data(), groups * sizeof(float)) != 0) {
+            printf("FAIL scales of payload %d differ from the oracle\n", r);
+            return 4;
+        }
+        checks += 2;
+    }
+
+    // fused dequant-reduce (mean) of the four payloads, fixed rank order
+    std::vector<const int8_t *> code_ptrs(d_codes.begin(), d_codes.end());
+    std::vector<const float *> scale_ptrs(d_scales.begin(), d_scales.end());
+    LBC_OK_OR_FAIL(lbc_dequant_reduce(code_ptrs.data(), scale_ptrs.data(), world, n, g, static_cast<float>(world), d_out,
+                                      LBC_F32, nullptr, nullptr, stream));
+    std::vector<float> got(n), want(n);
+    HIP_OK(hipMemcpyAsync(got.data(), d_out, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<const int8_t *> host_codes(world);
+    std::vector<const float *> host_scales(world);
+    for (int r = 0; r < world; ++r) {
+        host_codes[r] = want_codes[r].data();
+        host_scales[r] = want_scales[r].data();
+    }
+    lbo_reduce_f32(host_codes.data(), host_scales.data(), world, n, g, static_cast<float>(world), want.data());
+    if (memcmp(got.data(), want.data(), n * sizeof(float)) != 0) {
+        printf("FAIL reduced mean differs from the oracle\n");
+        return 5;
+    }
+    ++checks;
+
+    // one ring step: out += decode(payload 1), then quantize the sum; against decode + add + quantize on the host
+    std::vector<float> chunk(x[0]);
+    HIP_OK(hipMemcpyAsync(d_out, chunk.data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
+    int8_t *d_send_codes = nullptr;
+    float *d_send_scales = nullptr;
+    HIP_OK(hipMalloc(&d_send_codes, padded));
+    HIP_OK(hipMalloc(&d_send_scales, groups * sizeof(float)));
+    LBC_OK_OR_FAIL(lbc_ring_step(d_codes[1], d_scales[1], d_out, LBC_F32, n, g, LBC_REDUCE_SUM, 1.0f, d_send_codes,
+                                 d_send_scales, stream));
+    std::vector<int8_t> send_codes(padded), want_send_codes(padded);
+    std::vector<float> send_scales(groups), want_send_scales(groups);
+    HIP_OK(hipMemcpyAsync(got.data(), d_out, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(send_codes.data(), d_send_codes, padded, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(send_scales.data(), d_send_scales, groups * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    for (int64_t i = 0; i < n; ++i) {
+        volatile float decoded = static_cast<float>(want_codes[1][i]) * want_scales[1][i / g];
+        want[i] = chunk[i] + decoded;
+    }
+    lbo_quantize_f32(want.data(), n, g, want_send_codes.data(), want_send_scales.data());
+    if (memcmp(got.data(), want.data(), n * sizeof(float)) != 0 || memcmp(send_codes.data(), want_send_codes.data(), padded) != 0 ||
+        memcmp(send_scales.data(), want_send_scales.data(), groups * sizeof(float)) != 0) {
+        printf("FAIL ring step differs from the oracle\n");
+        return 6;
+    }
+    checks += 3;
+
+    // contract: a bad argument is refused with a message, an unsupported group size is "unsupported", not an error
+    if (lbc_quant_pack(d_x, LBC_F32, nullptr, LBC_NONE, -1, g, d_codes[0], d_scales[0], nullptr, LBC_NONE, nullptr, LBC_NONE,
+                       stream) != LBC_EINVAL || strstr(lbc_last_error(), "numel") == nullptr) {
+        printf("FAIL negative numel was not refused\n");
+        return 7;
+    }
+    if (lbc_quant_pack(d_x, LBC_F32, nullptr, LBC_NONE, n, 48, d_codes[0], d_scales[0], nullptr, LBC_NONE, nullptr, LBC_NONE,
+                       stream) != LBC_UNSUPPORTED) {
+        printf("FAIL group size 48 should be unsupported\n");
+        return 7;
+    }
+    checks += 2;
+    printf("OK %ld\n", checks);
+    return 0;
+}

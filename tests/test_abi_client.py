@@ -1,0 +1,26 @@
+"""The C ABI driven by a host program that has neither Python nor torch in it (tests/native/abi_client.cpp, built by
+``__graft_entry__.build()``): HIP runtime allocations, a stream of its own, results compared byte for byte with the
+scalar C oracle inside the program."""
+import subprocess
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+CLIENT = ROOT / "tests" / "native" / "_build" / "abi_client"
+
+
+def test_client_source_uses_only_the_header_and_the_hip_runtime():
+    text = (ROOT / "tests" / "native" / "abi_client.cpp").read_text()
+    includes = [line.split()[1] for line in text.splitlines() if line.startswith("#include")]
+    assert '"../../include/lbc.h"' in includes and "<hip/hip_runtime.h>" in includes
+    assert not any("torch" in name or "Python" in name or "pybind" in name for name in includes)
+    assert CLIENT.exists(), "run __graft_entry__.build() first"
+
+
+@pytest.mark.gpu
+def test_client_runs_quantize_reduce_and_ring_step_bit_exact_against_the_c_oracle(hip_device):
+    done = subprocess.run([str(CLIENT)], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0, (done.stdout, done.stderr[-2000:])
+    assert done.stdout.strip().startswith("OK "), done.stdout
+    assert int(done.stdout.split()[1]) == 14
