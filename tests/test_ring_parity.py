@@ -474,3 +474,42 @@ def test_ring_step_randomized_sweep(ops, hip_device):
         emit = rng.random() < 0.7
         offset = rng.choice([0, 0, 0, 1, 2, 5])
         check_step(ops, hip_device, dtype, g, n, reduce_op, divisor, emit, 50_000 + 3 * case, offset=offset)
+
+
+def test_ring_steps_captured_in_a_hip_graph_replay_like_eager(hip_device):
+    """A chain of ring steps (each hop's payload feeds the next) allocates and clears nothing, so it can be captured;
+    four replays with eager work and synchronisations in between equal four eager passes from the same state."""
+    from lowbit_comm_amd.hip import ops
+
+    g, n, hops = 64, 64 * 3000 + 21, 5
+    incoming = torch.empty(ops.payload_nbytes(n, g), dtype=torch.uint8, device=hip_device)
+    assert ops.quant_pack_payload_into(tensor_like(n, "fp32", 31, hip_device), incoming, group_size=g)
+    start = tensor_like(n, "fp32", 32, hip_device)
+    chunks = [start.clone() for _ in range(hops)]
+    payloads = [torch.empty_like(incoming) for _ in range(hops)]
+    launches = [ops.bind_ring_step(incoming if h == 0 else payloads[h - 1], chunks[h], payloads[h], group_size=g,
+                                   reduce_op="sum", divisor=2.0 if h == hops - 1 else 1.0) for h in range(hops)]
+
+    def one_pass():
+        for launch in launches:
+            assert launch()
+
+    eager = []
+    for _ in range(4):
+        one_pass()
+        torch.cuda.synchronize()
+        eager.append(([c.clone() for c in chunks], payloads[-1].clone()))
+    for c in chunks:
+        c.copy_(start)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+        one_pass()
+    torch.cuda.synchronize()
+    for c in chunks:
+        c.copy_(start)                                               # capture enqueued nothing
+    for want_chunks, want_payload in eager:
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a.view(torch.int32), b.view(torch.int32)) for a, b in zip(chunks, want_chunks))
+        assert torch.equal(payloads[-1], want_payload)
+        assert torch.isfinite((torch.randn(1 << 16, device=hip_device) * 2).sum())   # eager work between replays
