@@ -756,6 +756,40 @@ def main() -> int:
                  (payload_bytes + 2 * n * eb) + (n * eb + payload_bytes), timed(separate, args.iters * 2), n * eb, check)
             del sets
 
+        # the same hop in the CUDA extension's byte format (interleaved scales)
+        from lowbit_comm_amd.hip import cuda_wire as cw
+
+        for label, n, dtype, sets_n in (("fp32 chunk of 6,553,600", 6_553_600, torch.float32, 8),
+                                        ("fp32 chunk of 26,214,400", 26_214_400, torch.float32, 4),
+                                        ("bf16 chunk of 13,107,200", 13_107_200, torch.bfloat16, 8)):
+            eb = 4 if dtype == torch.float32 else 2
+            pb = cw.payload_nbytes(n, dtype)
+            sets = []
+            for k in range(sets_n):
+                received = cw.quant_pack(gen(SEED + 8500 + k, n, 1e-3, dtype))
+                chunk = gen(SEED + 8600 + k, n, 1e-3, dtype)
+                send = torch.empty(pb, dtype=torch.uint8, device=dev)
+                sets.append({"chunk": chunk, "send": send, "received": received,
+                             "sum": cw.bind_ring_step(received, chunk, send, reduce_op="sum"),
+                             "decode_sum": cw.bind_dequant(received, chunk, reduce_op="sum"),
+                             "quant": cw.bind_quant_pack(chunk, send)})
+            check = None
+            if parity:
+                a, b = sets[0], sets[1]
+                b["chunk"].copy_(a["chunk"]); b["received"].copy_(a["received"])
+                a["sum"](); b["decode_sum"](); b["quant"]()
+                check = "bit-exact vs separate launches" if bits_equal(a["chunk"], b["chunk"]) and torch.equal(a["send"], b["send"]) else "MISMATCH"
+            emit(8, f"ring step in the CUDA byte format, {label}: decode + accumulate + requantize, one launch",
+                 2 * pb + 2 * n * eb, timed(lambda i: sets[i % sets_n]["sum"](), args.iters * 2), n * eb, check)
+
+            def separate_wire(i):
+                sets[i % sets_n]["decode_sum"]()
+                sets[i % sets_n]["quant"]()
+
+            emit(8, f"ring step in the CUDA byte format, {label}: separate decode-accumulate and quantize launches",
+                 (pb + 2 * n * eb) + (n * eb + pb), timed(separate_wire, args.iters * 2), n * eb, check)
+            del sets
+
         # one rank's whole schedule (W=8, 200 MiB fp32 bucket) through the executor, replaying the bucket's plan
         world, n = 8, 52_428_800
         peer_payload = torch.empty(ops.payload_nbytes(n // world, G), dtype=torch.uint8, device=dev)

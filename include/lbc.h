@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define LBC_ABI_VERSION 5
+#define LBC_ABI_VERSION 6
 
 enum { LBC_OK = 0, LBC_UNSUPPORTED = 1, LBC_EINVAL = -1, LBC_ELAUNCH = -2 };
 
@@ -266,6 +266,23 @@ int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int
 int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t numel, int group_size,
                             int compact, float inv_divisor, int fused_multiply_add, void *out, int dtype,
                             const void *prepared, void *new_residual, void *stream);
+
+/*
+ * One hop of the quantized ring or tree in this format, in place on a chunk of whole groups:
+ *   chunk[i] = decode(received)[i]                   reduce_op LBC_REDUCE_NONE
+ *   chunk[i] = chunk[i] + decode(received)[i]        reduce_op LBC_REDUCE_SUM (one rounding to `dtype`)
+ *   chunk[i] = chunk[i] * (1 / divisor)              when divisor != 1: what `tensor.div_(W)` computes on a
+ *                                                    device tensor (float reciprocal, rounded to `dtype`)
+ * and, when `send` is given, the payload lbc_wire_quant_pack would write for the updated chunk (linear 8-bit
+ * codes), in the same launch.  Replaces TorchPipelinedRingRuntime / TorchTreeRuntime .fused_reduce and
+ * .apply_broadcast with the extension loaded (ccdl_comm/cuda/transports/torch_topology.py:262-316,367-415:
+ * inplace_dequantize with SUM / NONE, div_) plus the quant_pack of the same chunk that follows
+ * (pipelined_ring.py:221-225,250-254).  numel must be a multiple of group_size, as the reference's in-place
+ * decode demands (torch_topology.py:205-214); `send` must not alias `received`.  Other reduce ops:
+ * LBC_UNSUPPORTED.
+ */
+int lbc_wire_ring_step(const uint8_t *received, void *chunk, int dtype, int64_t numel, int group_size,
+                       int compact, int reduce_op, float divisor, uint8_t *send, void *stream);
 
 /*
  * The remaining policies of the CUDA extension's format: non-linear 4-bit code books

@@ -475,6 +475,144 @@ hipError_t launch_wire_decode_t(int g, int bit, int op, int mode, const WireDeco
     }
 }
 
+// ---------------------------------------------------------------------------
+// ring / tree step in this format: chunk (op)= decode(received) [* 1/W], then the quantize of the updated chunk
+// ---------------------------------------------------------------------------
+// What a rank running the reference does per hop with its extension loaded (torch_topology.py:262-316): decode the
+// arriving payload into the chunk with reduce op SUM or NONE, `div_` by the world size on the hop that completes
+// the sum (a multiplication by the float reciprocal, the way torch divides a device tensor by a number), then
+// quantize the chunk for the next hop - here in one launch, the updated chunk still in registers.  Linear 8-bit
+// codes, whole groups (the reference's in-place decode needs them).  The encode is the one a chunk of whole groups
+// without a residual gets in the reference: group maximum with NaNs skipped, and when a group holds a NaN the
+// running maximum of the general kernels, which a NaN resets (see wire_quant_kernel).
+template <typename T, int G, bool COMPACT, int NT, bool ACC>
+__global__ __launch_bounds__(kBlock) void wire_ring_step_kernel(const WireRingStepArgs a) {
+    constexpr int PNT_LOAD = payload_load_hint<COMPACT, NT, 1>();
+    constexpr int PNT_STORE = COMPACT ? kPlain : NT;
+    using W = wire<T, 8>;
+    using Raw = typename raw_bits<T>::type;
+    constexpr int VEC = W::VEC;
+    constexpr int LPG = G / VEC;
+    constexpr int UNROLL = ACC ? 1 : 2;
+    constexpr int BLOCK_ELEMS = W::TILE * kWavesPerBlock * UNROLL;
+    static_assert(LPG >= 1 && LPG <= 16, "a group must fit one DPP row");
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t groups = a.numel / G;               // whole groups only
+    const group_layout<T, G, COMPACT, 8> at{groups};
+    const uint8_t *__restrict__ received = a.received;
+    T *chunk = static_cast<T *>(a.chunk);
+    const bool scaled = a.inv_divisor != 1.0f;
+    const bool emit = a.send != nullptr;
+    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(BLOCK_ELEMS)) * BLOCK_ELEMS;
+    if (block_first >= a.numel) return;
+
+    uint32_t words[UNROLL][W::WORDS];
+    T stored[UNROLL];
+    T xv[UNROLL][VEC];
+    int64_t e0[UNROLL];
+    bool live[UNROLL];   // a lane's elements, and its whole group, lie inside the chunk or outside it together
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * W::TILE + lane * VEC;
+        live[u] = e0[u] < a.numel;
+        if (live[u]) {
+            const int64_t group = e0[u] / G;
+            const int k0 = static_cast<int>(e0[u] - group * G);
+            load_piece<T, 8, PNT_LOAD, W::WORDS>(received + at.codes(group) + piece_offset<T, 8>(k0), words[u]);
+            stored[u] = *reinterpret_cast<const T *>(received + at.scale(group));
+            if constexpr (ACC) load_elems<T, VEC, NT>(chunk + e0[u], xv[u]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        float p[VEC];
+        T held[VEC];
+        uint32_t m = 0;
+        bool has_nan = false;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            p[i] = 0.0f;
+            held[i] = narrow<T>(0.0f);
+        }
+        if (live[u]) {
+            const float step = step_of<8>(widen(stored[u]));
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                float v = round_through<T>(unpack_code<T, 8, W::WORDS>(words[u], i) * step);
+                if constexpr (ACC) v = add_rounded_once<T>(widen(xv[u][i]), v);
+                if (scaled) v = round_through<T>(v * a.inv_divisor);
+                held[i] = narrow<T>(v);
+                p[i] = v;
+                uint32_t bits = as_u32(v) & 0x7FFFFFFFu;
+                has_nan |= bits > 0x7F800000u;
+                bits = bits > 0x7F800000u ? 0u : bits;   // fmaxf skips NaN
+                m = bits > m ? bits : m;
+            }
+            store_elems<T, VEC, NT>(chunk + e0[u], held);
+        }
+        if (!emit) continue;    // uniform over the grid
+        // every lane of a row takes part in the group reductions; rows past the end carry zeros
+        const int64_t group = e0[u] / G;
+        const int k0 = static_cast<int>(e0[u] - group * G);
+        const float absmax = as_f32(group_max_bits<LPG>(m));
+        float scale = absmax < 1.0e-6f ? 1.0e-6f : absmax;    // a NaN stays and zeroes every code
+        Raw kept = __builtin_bit_cast(Raw, narrow<T>(absmax));
+        bool wide_codes = false;                               // wavefront-uniform
+        if (__ballot(has_nan) != 0) {
+            uint32_t mag[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) mag[i] = __builtin_bit_cast(Raw, held[i]) & raw_bits<T>::ABS;
+            const uint32_t scale_raw = running_max_raw<T, G, VEC>(mag, k0, scan_start<T, G>(group));
+            const float rescanned = value_of<T>(scale_raw);
+            scale = rescanned < 1.0e-6f ? 1.0e-6f : rescanned;
+            kept = static_cast<Raw>(scale_raw);
+            wide_codes = true;
+        }
+        if (!live[u]) continue;
+        const float multiplier = W::LEVELS / scale;
+        int c[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            c[i] = cvt_i32(__builtin_rintf(p[i] * multiplier));
+            if (wide_codes) c[i] = c[i] < -127 ? -127 : (c[i] > 127 ? 127 : c[i]);
+        }
+        uint32_t out_words[W::WORDS];
+        pack_codes<T, 8, VEC, W::WORDS>(c, out_words);
+        store_piece<T, 8, PNT_STORE, W::WORDS>(a.send + at.codes(group) + piece_offset<T, 8>(k0), out_words);
+        if ((lane & (LPG - 1)) == 0) *reinterpret_cast<Raw *>(a.send + at.scale(group)) = kept;
+    }
+}
+
+template <typename T, int G, bool COMPACT, bool ACC>
+hipError_t launch_wire_ring_c(int mode, const WireRingStepArgs &a, hipStream_t stream) {
+    constexpr int BLOCK_ELEMS = wire<T, 8>::TILE * kWavesPerBlock * (ACC ? 1 : 2);
+    const int64_t blocks = (a.numel + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    const dim3 grid(static_cast<unsigned>(blocks));
+    if (mode == kStream) hipLaunchKernelGGL((wire_ring_step_kernel<T, G, COMPACT, kNonTemporal, ACC>), grid, dim3(kBlock), 0, stream, a);
+    else hipLaunchKernelGGL((wire_ring_step_kernel<T, G, COMPACT, kPlain, ACC>), grid, dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+template <typename T, int G>
+hipError_t launch_wire_ring_g(bool accumulate, int mode, const WireRingStepArgs &a, hipStream_t s) {
+    if (a.compact) return accumulate ? launch_wire_ring_c<T, G, true, true>(mode, a, s) : launch_wire_ring_c<T, G, true, false>(mode, a, s);
+    return accumulate ? launch_wire_ring_c<T, G, false, true>(mode, a, s) : launch_wire_ring_c<T, G, false, false>(mode, a, s);
+}
+
+template <typename T>
+hipError_t launch_wire_ring_t(int g, bool accumulate, int mode, const WireRingStepArgs &a, hipStream_t s) {
+    switch (g) {
+        case 64: return launch_wire_ring_g<T, 64>(accumulate, mode, a, s);
+        case 32: return launch_wire_ring_g<T, 32>(accumulate, mode, a, s);
+        case 16: return launch_wire_ring_g<T, 16>(accumulate, mode, a, s);
+        default: return hipErrorNotSupported;
+    }
+}
+
 }  // namespace
 
 hipError_t launch_wire_quant(int dtype, int group_size, int bit, int mode, const WireQuantArgs &args, int world,
@@ -503,6 +641,16 @@ hipError_t launch_wire_decode(int dtype, int group_size, int bit, int reduce_op,
         case kF32: return launch_wire_decode_t<float>(group_size, bit, reduce_op, mode, args, world, stream);
         case kF16: return launch_wire_decode_t<f16>(group_size, bit, reduce_op, mode, args, world, stream);
         case kBF16: return launch_wire_decode_t<bf16>(group_size, bit, reduce_op, mode, args, world, stream);
+        default: return hipErrorNotSupported;
+    }
+}
+
+hipError_t launch_wire_ring_step(int dtype, int group_size, bool accumulate, int mode, const WireRingStepArgs &args,
+                                 hipStream_t stream) {
+    switch (dtype) {
+        case kF32: return launch_wire_ring_t<float>(group_size, accumulate, mode, args, stream);
+        case kF16: return launch_wire_ring_t<f16>(group_size, accumulate, mode, args, stream);
+        case kBF16: return launch_wire_ring_t<bf16>(group_size, accumulate, mode, args, stream);
         default: return hipErrorNotSupported;
     }
 }

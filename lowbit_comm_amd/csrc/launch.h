@@ -101,6 +101,15 @@ struct WireDecodeArgs {
     int compact;
 };
 
+struct WireRingStepArgs {
+    const uint8_t *received;   // payload covering numel elements
+    void *chunk;               // numel elements (a multiple of the group size), updated in place
+    uint8_t *send;             // null: no payload is produced
+    int64_t numel;
+    float inv_divisor;         // 1 = no division
+    int compact;
+};
+
 // The general policies of the CUDA extension's format (code books, stochastic rounding, top-k).
 struct WireGeneralQuantArgs {
     const void *x;
@@ -153,6 +162,9 @@ hipError_t launch_wire_reduce(int dtype, int group_size, int world, bool fused_m
                               const WireReduceArgs &args, hipStream_t stream);
 hipError_t launch_wire_decode(int dtype, int group_size, int bit, int reduce_op, int mode, const WireDecodeArgs &args,
                               int world, hipStream_t stream);
+
+hipError_t launch_wire_ring_step(int dtype, int group_size, bool accumulate, int mode, const WireRingStepArgs &args,
+                                 hipStream_t stream);
 
 hipError_t launch_wire_general_quant(int dtype, int group_size, int bit, const WireGeneralQuantArgs &args,
                                      hipStream_t stream);

@@ -465,6 +465,28 @@ int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t n
                   "lbc_wire_dequant_reduce");
 }
 
+int lbc_wire_ring_step(const uint8_t *received, void *chunk, int dtype, int64_t numel, int group_size, int compact,
+                       int reduce_op, float divisor, uint8_t *send, void *stream) {
+    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
+    if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported chunk dtype %d", dtype);
+    if (reduce_op < LBC_REDUCE_NONE || reduce_op > LBC_REDUCE_MIN) return fail(LBC_EINVAL, "unknown reduce op %d", reduce_op);
+    if (!(divisor > 0.0f)) return fail(LBC_EINVAL, "divisor must be > 0");
+    if (!valid_group(group_size)) return LBC_UNSUPPORTED;
+    if (reduce_op != LBC_REDUCE_NONE && reduce_op != LBC_REDUCE_SUM) return LBC_UNSUPPORTED;
+    if (numel % group_size != 0) return fail(LBC_EINVAL, "numel should be multiple of group_size");
+    if (numel == 0) return LBC_OK;
+    if (received == nullptr || chunk == nullptr) return fail(LBC_EINVAL, "received payload and chunk must not be null");
+    const int item = dtype_size(dtype);
+    if (!aligned_to(chunk, item) || !aligned_to(received, item) || !aligned_to(send, item))
+        return fail(LBC_EINVAL, "chunk and payloads must be aligned to the element size");
+    if (send == received) return fail(LBC_EINVAL, "the payload to send must not alias the received one");
+    lbc::WireRingStepArgs a{received, chunk, send, numel, divisor == 1.0f ? 1.0f : 1.0f / divisor, compact != 0};
+    const int64_t moved = numel * ((reduce_op == LBC_REDUCE_SUM ? 2 : 1) * item + (send ? 2 : 1));
+    return finish(lbc::launch_wire_ring_step(dtype, group_size, reduce_op == LBC_REDUCE_SUM, pick_mode(true, moved), a,
+                                             static_cast<hipStream_t>(stream)),
+                  "lbc_wire_ring_step");
+}
+
 // ---- general policies of that format: code books, stochastic rounding, top-k ------------------
 static bool valid_general(int group_size, int bit, int quant_type, int topk) {
     if (!valid_group(group_size) || (bit != 8 && bit != 4) || topk < 0 || topk > 2) return false;

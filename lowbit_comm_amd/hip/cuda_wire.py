@@ -158,6 +158,31 @@ QUANT_TYPES = {"linear": 0, "normal": 1, "uniform": 2, "e3m0": 3, "e2m1": 4}
 _META_WORDS = {0: 1, 1: 3, 2: 4}
 
 
+def bind_ring_step(received: torch.Tensor, chunk: torch.Tensor, send: torch.Tensor | None = None, *,
+                   group_size: int = 64, compact: bool = True, reduce_op: str = "sum",
+                   divisor: float = 1.0) -> BoundLaunch:
+    """One ring / tree hop in this format: ``chunk (op)= decode(received)``, ``chunk *= 1/divisor`` (torch's device
+    ``div_``), and - with ``send`` - the payload of the updated chunk, in one launch.  ``chunk`` holds whole groups."""
+    lib = load_library()
+    code = _float_tensor(chunk, "chunk")
+    n = chunk.numel()
+    _require(n % group_size == 0, "numel should be multiple of group_size")
+    _require(reduce_op in REDUCE_OPS, f"unsupported reduce op {reduce_op!r}")
+    _require(float(divisor) > 0.0, "divisor must be > 0")
+    nbytes = payload_nbytes(n, chunk.dtype, group_size)
+    _payload(received, "received payload", chunk.device, nbytes)
+    if send is not None:
+        _payload(send, "send payload", chunk.device, nbytes)
+        _require(n == 0 or send.data_ptr() != received.data_ptr(), "the payload to send must not alias the received one")
+    args = (_ptr(received), _ptr(chunk), code, n, group_size, int(compact), REDUCE_OPS[reduce_op], float(divisor),
+            _ptr(send))
+    return BoundLaunch(lib.lbc_wire_ring_step, args, chunk.device, lib, (received, chunk, send))
+
+
+def ring_step_into(received: torch.Tensor, chunk: torch.Tensor, send: torch.Tensor | None = None, **kwargs) -> bool:
+    return bind_ring_step(received, chunk, send, **kwargs)()
+
+
 def general_payload_nbytes(numel: int, dtype: torch.dtype, group_size: int = 64, bit: int = 8, topk: int = 0) -> int:
     """``G * (g*bit/8 + element size * (1 | 3 | 4))`` (ccdl_comm/csrc/quantization/gen_code_quant.py:167-178)."""
     _require(topk in _META_WORDS, f"topk must be 0, 1 or 2, got {topk}")

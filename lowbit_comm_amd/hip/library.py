@@ -11,7 +11,7 @@ from pathlib import Path
 from lowbit_comm_amd.exceptions import CCDLUnavailableError
 
 LIBRARY_PATH = Path(__file__).resolve().parent.parent / "liblbc_hip.so"
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 LBC_OK = 0
 LBC_UNSUPPORTED = 1
@@ -42,6 +42,7 @@ SIGNATURES = {
     "lbc_wire_quant_pack": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
     "lbc_wire_quant_pack_chunks": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_ptr,
                                             _c_i64, _c_ptr]),
+    "lbc_wire_ring_step": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, ctypes.c_float, _c_ptr, _c_ptr]),
     "lbc_wire_dequant": (_c_int, [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
     "lbc_wire_dequant_chunks": (_c_int, [_c_ptr, _c_i64, _c_int, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_ptr,
                                          _c_int, _c_int, _c_ptr]),

@@ -445,7 +445,9 @@ class HipPipelinedRingRuntime:
     (``quantize_tensor(view, output=...)``, ``dequantize_tensor(received, output=view, reduce_op=...)``,
     ``view.div_(W)``), exactly the calls of the reference's runtime.  This serves every policy and payload format
     the module does - in particular the CUDA extension's byte format, for rings that mix ranks running that
-    extension with gfx950 ranks - at the reference's launch count; chunks must then be whole groups, as there."""
+    extension with gfx950 ranks - at the reference's launch count; chunks must then be whole groups, as there.
+    Plain linear 8-bit codes in the CUDA byte format do not need the facade: with ``fuse_steps`` they take that
+    format's own fused step (``lbc_wire_ring_step``), one launch per hop as in the portable format."""
 
     def __init__(self, *, config: CompressionConfig, dtype: str, world_size: int, rank: int,
                  exchange: Callable[..., Any], completion_manager: Any | None = None, stream: Any | None = None,
@@ -470,7 +472,14 @@ class HipPipelinedRingRuntime:
         self.dtype = dtype
         self.world_size = world_size
         self.rank = rank
-        self.fuse_steps = bool(fuse_steps) and extension_status is None
+        module = getattr(extension_status, "module", None)
+        cuda_bytes = extension_status is not None and getattr(module, "NATIVE_WIRE_FORMAT", "native") == "native"
+        plain = config.bit == 8 and config.quant_type == "linear" and config.topk == 0 and not config.stochastic
+        # the CUDA byte format has a fused step of its own for plain linear 8-bit codes; everything else a module
+        # serves goes through its facade
+        self._wire_direct = bool(fuse_steps) and cuda_bytes and plain
+        self._facade = extension_status is not None and not self._wire_direct
+        self.fuse_steps = bool(fuse_steps) and not self._facade
         self.extension_status = extension_status
         self.max_plans = max_plans
         self.plans: "OrderedDict[tuple[int, int], dict]" = OrderedDict()
@@ -560,6 +569,30 @@ class HipPipelinedRingRuntime:
         context.quant_index += 1
         return buffer
 
+    # ---- launches in the active payload format ------------------------------ #
+    def _bind_quantize(self, view: Any, payload: Any) -> Any:
+        g = self.config.group_size
+        if self._wire_direct:
+            from lowbit_comm_amd.hip import cuda_wire
+
+            self._whole_groups(view)
+            return cuda_wire.bind_quant_pack(view, payload, group_size=g, compact=self.config.compact)
+        from lowbit_comm_amd.hip import ops
+
+        return ops.bind_quant_pack_payload(view, payload, group_size=g)
+
+    def _bind_step(self, received: Any, view: Any, send: Any, reduce_op: str, divisor: float) -> Any:
+        g = self.config.group_size
+        if self._wire_direct:
+            from lowbit_comm_amd.hip import cuda_wire
+
+            self._whole_groups(view)
+            return cuda_wire.bind_ring_step(received, view, send, group_size=g, compact=self.config.compact,
+                                            reduce_op=reduce_op, divisor=divisor)
+        from lowbit_comm_amd.hip import ops
+
+        return ops.bind_ring_step(received, view, send, group_size=g, reduce_op=reduce_op, divisor=divisor)
+
     # ---- steps ------------------------------------------------------------- #
     def quant_pack(self, tensor: Any, chunk: ChunkRange, workspace: Any, *, context: RingSubmissionContext) -> Any:
         from lowbit_comm_amd.hip import ops
@@ -567,14 +600,14 @@ class HipPipelinedRingRuntime:
         staged, context.staged = context.staged, None
         if staged is not None and staged[0] == (chunk.start, chunk.stop):
             return staged[1]
-        if self.extension_status is not None:
+        if self._facade:
             return self._facade_quantize(tensor, chunk, workspace, context)
         plan, key = context.plan, ("quantize", context.quant_index, chunk.start, chunk.stop)
         bound = None if plan is None else plan.get(key)
         if bound is None:
             view = _view(tensor, chunk)
             payload = self._send_buffer(view, workspace, context)
-            bound = (ops.bind_quant_pack_payload(view, payload, group_size=self.config.group_size), payload)
+            bound = (self._bind_quantize(view, payload), payload)
             if plan is not None:
                 plan[key] = bound
         else:
@@ -605,7 +638,7 @@ class HipPipelinedRingRuntime:
 
         dependency.wait_stream(context.stream)
         context.steps_done += 1
-        if self.extension_status is not None:
+        if self._facade:
             return self._facade_step(tensor, received, chunk, context, reduce_op=reduce_op, divisor=divisor)
         if another_hop is None:
             another_hop = context.steps_done < 2 * (self.world_size - 1)
@@ -616,8 +649,7 @@ class HipPipelinedRingRuntime:
             g = self.config.group_size
             if self.fuse_steps:
                 send = self._send_buffer(view, workspace, context) if another_hop else None
-                launches = (ops.bind_ring_step(received, view, send, group_size=g, reduce_op=reduce_op,
-                                               divisor=divisor),)
+                launches = (self._bind_step(received, view, send, reduce_op, divisor),)
             else:
                 send = None
                 launches = (ops.bind_dequant(*ops.split_payload(received, view.numel(), g), view, group_size=g,

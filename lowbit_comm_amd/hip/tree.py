@@ -170,7 +170,7 @@ class HipTreeRuntime(HipPipelinedRingRuntime):
         if edge.parent_rank == self.rank and not context.mean_applied:
             self._divide(tensor, context)             # only reached when the steps are not fused
         payload = super().quant_pack(tensor, self._whole, workspace, context=context)
-        if self.extension_status is None:
+        if not self._facade:
             context.staged = ((self._whole.start, self._whole.stop), payload)
         return payload
 

@@ -424,9 +424,19 @@ def test_ring_through_the_codec_facade_in_the_cuda_byte_format(hip_device, polic
     n = world * g * 37
     buckets = [tensor_like(n, dtype, 9100 + 3 * r, hip_device, sigma=10.0 ** (r % 2 - 3)) for r in range(world)]
     before = [to_np(b, dtype) for b in buckets]
+    plain = config.bit == 8 and config.topk == 0 and config.quant_type == "linear"
     ring = build_ring(hip_device, world, n, dtype, g, True, config=config, extension_status=status)
-    assert all(e._runtime.fuse_steps is False for e in ring[1])
+    # plain linear codes take the format's own fused step, everything else the module's facade
+    assert all(e._runtime._wire_direct is plain and e._runtime._facade is (not plain) for e in ring[1])
     run_ring(hip_device, buckets, dtype, g, True, ring=ring)
+    if plain:       # and the facade gives the same bits for them
+        again = [torch.from_numpy(b.view(np.int16) if dtype == "bf16" else b).to(hip_device) for b in before]
+        again = [a.view(torch.bfloat16) if dtype == "bf16" else a for a in again]
+        slow = build_ring(hip_device, world, n, dtype, g, False, config=config, extension_status=status)
+        assert all(e._runtime._facade for e in slow[1])
+        run_ring(hip_device, again, dtype, g, False, ring=slow)
+        for a, b in zip(again, buckets):
+            assert np.array_equal(raw(to_np(a, dtype)), raw(to_np(b, dtype)))
     codec = ring_np.CudaWireCodec(g, bit=config.bit, quant_type=config.quant_type, topk=config.topk,
                                   compact=config.compact)
     want = ring_np.ring_all_reduce(before, dtype, g, codec=codec)
@@ -513,3 +523,73 @@ def test_ring_steps_captured_in_a_hip_graph_replay_like_eager(hip_device):
         assert all(torch.equal(a.view(torch.int32), b.view(torch.int32)) for a, b in zip(chunks, want_chunks))
         assert torch.equal(payloads[-1], want_payload)
         assert torch.isfinite((torch.randn(1 << 16, device=hip_device) * 2).sum())   # eager work between replays
+
+
+# --------------------------------------------------------------------------- #
+# the same hop in the CUDA extension's byte format
+# --------------------------------------------------------------------------- #
+def check_wire_step(device, dtype, g, n, compact, reduce_op, divisor, emit, seed, poison=False):
+    from lowbit_comm_amd.hip import cuda_wire
+
+    tdtype = DTYPES[dtype]
+    incoming = tensor_like(n, dtype, seed, device)
+    received = cuda_wire.quant_pack(incoming, group_size=g, compact=compact)
+    chunk = tensor_like(n, dtype, seed + 1, device, sigma=3e-3)
+    if poison and n >= 4 * g:
+        chunk[g + 3] = float("nan")               # a NaN inside a group: the running maximum restarts after it
+        chunk[3 * g - 1] = float("nan")           # a NaN that ends a group's scan
+        chunk[5] = float("inf")
+    before = to_np(chunk, dtype)
+    send = torch.full((cuda_wire.payload_nbytes(n, tdtype, g),), 0xAB, dtype=torch.uint8, device=device) if emit else None
+    assert cuda_wire.ring_step_into(received, chunk, send, group_size=g, compact=compact, reduce_op=reduce_op,
+                                    divisor=divisor)
+    codec = ring_np.CudaWireCodec(g, compact=compact)
+    want_chunk, want_payload = ring_np.ring_step(received.cpu().numpy(), before, dtype, g, reduce_op=reduce_op,
+                                                 divisor=divisor, emit=emit, codec=codec)
+    what = (dtype, g, n, compact, reduce_op, divisor, emit, poison)
+    assert np.array_equal(raw(to_np(chunk, dtype)), raw(want_chunk)), what
+    if emit:
+        assert np.array_equal(send.cpu().numpy(), want_payload), what
+
+
+@pytest.mark.parametrize("compact", [True, False])
+@pytest.mark.parametrize("dtype", ["fp32", "fp16", "bf16"])
+def test_wire_ring_step_bit_exact(hip_device, dtype, compact):
+    seed = 70_000
+    for g in (64, 32, 16):
+        for n in (g, g * 17, g * 4096 // 16 + g, g * 5000):
+            for reduce_op, divisor in (("sum", 1.0), ("sum", 8.0), ("sum", 3.0), ("none", 1.0)):
+                for emit in (True, False):
+                    seed += 2
+                    check_wire_step(hip_device, dtype, g, n, compact, reduce_op, divisor, emit, seed)
+    check_wire_step(hip_device, dtype, 64, 64 * 40, compact, "sum", 1.0, True, 79_001, poison=True)
+    check_wire_step(hip_device, dtype, 16, 16 * 64, compact, "none", 1.0, True, 79_003, poison=False)
+
+
+def test_wire_ring_step_equals_the_separate_launches_and_checks_its_arguments(hip_device):
+    from lowbit_comm_amd.hip import cuda_wire
+
+    g, n = 64, 64 * 20_000
+    for dtype in (torch.float32, torch.bfloat16):
+        received = cuda_wire.quant_pack(tensor_like(n, "fp32", 5, hip_device).to(dtype))
+        start = tensor_like(n, "fp32", 6, hip_device).to(dtype)
+        fused = start.clone()
+        send = torch.empty_like(received)
+        assert cuda_wire.ring_step_into(received, fused, send, reduce_op="sum", divisor=3.0)
+        plain = start.clone()
+        assert cuda_wire.dequant_into(received, plain, reduce_op="sum")
+        plain.div_(3)
+        assert torch.equal(fused.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                           plain.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+        assert torch.equal(send, cuda_wire.quant_pack(plain))
+    chunk = torch.zeros(64 * 3, device=hip_device)
+    payload = cuda_wire.quant_pack(chunk)
+    assert cuda_wire.ring_step_into(payload, chunk, None, reduce_op="max") is False
+    with pytest.raises(RuntimeError, match="multiple of group_size"):
+        cuda_wire.ring_step_into(payload, chunk[:100], None)
+    with pytest.raises(RuntimeError, match="invalid quantized payload size"):
+        cuda_wire.ring_step_into(payload[:-4], chunk, None)
+    with pytest.raises(RuntimeError, match="must not alias"):
+        cuda_wire.ring_step_into(payload, chunk, payload)
+    with pytest.raises(RuntimeError, match="divisor must be > 0"):
+        cuda_wire.ring_step_into(payload, chunk, None, divisor=-1.0)

@@ -104,11 +104,11 @@ def test_tree_replays_its_plan_without_allocating_and_launches_once_per_changing
     assert not any(k[0] == "quantize" for k in plan)          # every payload came out of a fused step
 
 
-POLICIES = [dict(compact=True), dict(bit=4, allow_experimental=True), dict(topk=1)]
+POLICIES = [dict(), dict(compact=True), dict(bit=4, allow_experimental=True), dict(topk=1)]
 
 
-@pytest.mark.parametrize("policy", POLICIES, ids=lambda p: "-".join(f"{k}={v}" for k, v in p.items()))
-@pytest.mark.parametrize("dtype, world, g, root", [("fp32", 5, 64, 0), ("bf16", 6, 32, 4)])
+@pytest.mark.parametrize("policy", POLICIES, ids=lambda p: "-".join(f"{k}={v}" for k, v in p.items()) or "linear8")
+@pytest.mark.parametrize("dtype, world, g, root", [("fp32", 5, 64, 0), ("bf16", 6, 32, 4), ("fp16", 3, 16, 1)])
 def test_tree_through_the_codec_facade_in_the_cuda_byte_format(hip_device, policy, dtype, world, g, root):
     from lowbit_comm_amd.config import CompressionConfig
     from lowbit_comm_amd.hip.loader import load_hip_extension
