@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
                 NT diff_out[VEC];
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
-                    const float rest = round_through<DT>(static_cast<float>(c[i]) * scale);
+                    const float rest = round_through<DT>(code_value(c[i]) * scale);
                     rest_out[i] = narrow<DT>(rest);
                     diff_out[i] = narrow<NT>(p[i] - rest);
                 }
