@@ -1,0 +1,133 @@
+// What a trivial streaming kernel reaches on this part: read-only, write-only, copy and a 16-bytes-in / 4-bytes-out
+// kernel (the traffic shape of an fp32 quantize) over rotating buffers, one workgroup per tile or a grid-stride loop,
+// with and without the non-temporal hint.  The codec kernels are judged against these figures as well as against
+// the 8 TB/s on the data sheet.  Usage: stream_probe [MiB per buffer, default 100].  Not part of the product.
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+#define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("HIP error %s at %d\n", hipGetErrorString(e), __LINE__); exit(1);} } while (0)
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+template <int UNROLL, bool NT>
+__global__ __launch_bounds__(256) void read_kernel(const float4v* __restrict__ in, float* __restrict__ out, size_t n4) {
+    size_t base = (size_t)blockIdx.x * 256 * UNROLL + threadIdx.x;
+    float4v acc = {0, 0, 0, 0};
+    float4v v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        size_t i = base + (size_t)u * 256;
+        if (i < n4) v[u] = NT ? __builtin_nontemporal_load(in + i) : in[i]; else v[u] = acc;
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) acc += v[u];
+    if (acc.x + acc.y + acc.z + acc.w == 12345.678f) out[0] = 1.0f;
+}
+
+template <int UNROLL, bool NT>
+__global__ __launch_bounds__(256) void read_gs_kernel(const float4v* __restrict__ in, float* __restrict__ out, size_t n4) {
+    // grid-stride persistent
+    float4v acc = {0, 0, 0, 0};
+    size_t stride = (size_t)gridDim.x * 256 * UNROLL;
+    for (size_t base = (size_t)blockIdx.x * 256 * UNROLL + threadIdx.x; base < n4; base += stride) {
+        float4v v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            size_t i = base + (size_t)u * 256;
+            if (i < n4) v[u] = NT ? __builtin_nontemporal_load(in + i) : in[i]; else v[u] = float4v{0,0,0,0};
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) acc += v[u];
+    }
+    if (acc.x + acc.y + acc.z + acc.w == 12345.678f) out[0] = 1.0f;
+}
+
+template <int UNROLL, bool NT>
+__global__ __launch_bounds__(256) void write_kernel(float4v* __restrict__ out, size_t n4) {
+    size_t base = (size_t)blockIdx.x * 256 * UNROLL + threadIdx.x;
+    float4v v = {1.0f, 2.0f, 3.0f, (float)threadIdx.x};
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        size_t i = base + (size_t)u * 256;
+        if (i < n4) { if (NT) __builtin_nontemporal_store(v, out + i); else out[i] = v; }
+    }
+}
+
+template <int UNROLL, bool NT>
+__global__ __launch_bounds__(256) void copy_kernel(const float4v* __restrict__ in, float4v* __restrict__ out, size_t n4) {
+    size_t base = (size_t)blockIdx.x * 256 * UNROLL + threadIdx.x;
+    float4v v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        size_t i = base + (size_t)u * 256;
+        if (i < n4) v[u] = NT ? __builtin_nontemporal_load(in + i) : in[i];
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        size_t i = base + (size_t)u * 256;
+        if (i < n4) { if (NT) __builtin_nontemporal_store(v[u], out + i); else out[i] = v[u]; }
+    }
+}
+
+// 4:1 read:write like quantize (read 16B, write 4B per lane)
+template <int UNROLL>
+__global__ __launch_bounds__(256) void quantlike_kernel(const float4v* __restrict__ in, unsigned* __restrict__ out, size_t n4) {
+    size_t base = (size_t)blockIdx.x * 256 * UNROLL + threadIdx.x;
+    float4v v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) { size_t i = base + (size_t)u * 256; if (i < n4) v[u] = in[i]; }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) { size_t i = base + (size_t)u * 256; if (i < n4) out[i] = __builtin_bit_cast(unsigned, v[u].x + v[u].y + v[u].z + v[u].w); }
+}
+
+struct Timer {
+    hipEvent_t a, b;
+    Timer() { CK(hipEventCreate(&a)); CK(hipEventCreate(&b)); }
+};
+
+template <typename F>
+double run(F launch, int iters, int nbuf) {
+    Timer t;
+    for (int i = 0; i < 5; ++i) launch(i % nbuf);
+    CK(hipDeviceSynchronize());
+    CK(hipEventRecord(t.a));
+    for (int i = 0; i < iters; ++i) launch(i % nbuf);
+    CK(hipEventRecord(t.b));
+    CK(hipEventSynchronize(t.b));
+    float ms; CK(hipEventElapsedTime(&ms, t.a, t.b));
+    return ms * 1e-3 / iters;
+}
+
+int main(int argc, char** argv) {
+    size_t bytes = (argc > 1 ? atol(argv[1]) : 100) * (size_t)1048576;
+    int nbuf = 6;
+    std::vector<float4v*> in(nbuf), out(nbuf);
+    for (int i = 0; i < nbuf; ++i) { CK(hipMalloc(&in[i], bytes)); CK(hipMalloc(&out[i], bytes)); CK(hipMemset(in[i], 1, bytes)); CK(hipMemset(out[i], 0, bytes)); }
+    float* flag; CK(hipMalloc(&flag, 4));
+    size_t n4 = bytes / 16;
+    int iters = 50;
+    int cus = 256;
+    printf("buffer %zu MiB x %d rotating\n", bytes >> 20, nbuf);
+#define REPORT(name, nb, t) printf("%-44s %8.2f us  %8.1f GB/s (%4.1f%%)\n", name, (t)*1e6, (nb)/(t)/1e9, (nb)/(t)/8e12*100); fflush(stdout)
+#define GRID(U) (unsigned)((n4 + 256 * (U) - 1) / (256 * (U)))
+    { double t = run([&](int b){ read_kernel<1,false><<<GRID(1),256>>>(in[b], flag, n4); }, iters, nbuf); REPORT("read  U=1", bytes, t); }
+    { double t = run([&](int b){ read_kernel<2,false><<<GRID(2),256>>>(in[b], flag, n4); }, iters, nbuf); REPORT("read  U=2", bytes, t); }
+    { double t = run([&](int b){ read_kernel<4,false><<<GRID(4),256>>>(in[b], flag, n4); }, iters, nbuf); REPORT("read  U=4", bytes, t); }
+    { double t = run([&](int b){ read_kernel<8,false><<<GRID(8),256>>>(in[b], flag, n4); }, iters, nbuf); REPORT("read  U=8", bytes, t); }
+    { double t = run([&](int b){ read_kernel<4,true><<<GRID(4),256>>>(in[b], flag, n4); }, iters, nbuf); REPORT("read  U=4 nontemporal", bytes, t); }
+    for (int mult : {2, 4, 8, 16}) {
+        char name[64]; snprintf(name, 64, "read  grid-stride U=4 blocks=%d*CU", mult);
+        double t = run([&](int b){ read_gs_kernel<4,false><<<cus*mult,256>>>(in[b], flag, n4); }, iters, nbuf); REPORT(name, bytes, t);
+    }
+    { double t = run([&](int b){ write_kernel<1,false><<<GRID(1),256>>>(out[b], n4); }, iters, nbuf); REPORT("write U=1", bytes, t); }
+    { double t = run([&](int b){ write_kernel<4,false><<<GRID(4),256>>>(out[b], n4); }, iters, nbuf); REPORT("write U=4", bytes, t); }
+    { double t = run([&](int b){ write_kernel<4,true><<<GRID(4),256>>>(out[b], n4); }, iters, nbuf); REPORT("write U=4 nontemporal", bytes, t); }
+    { double t = run([&](int b){ copy_kernel<1,false><<<GRID(1),256>>>(in[b], out[b], n4); }, iters, nbuf); REPORT("copy  U=1", 2*bytes, t); }
+    { double t = run([&](int b){ copy_kernel<4,false><<<GRID(4),256>>>(in[b], out[b], n4); }, iters, nbuf); REPORT("copy  U=4", 2*bytes, t); }
+    { double t = run([&](int b){ copy_kernel<4,true><<<GRID(4),256>>>(in[b], out[b], n4); }, iters, nbuf); REPORT("copy  U=4 nontemporal", 2*bytes, t); }
+    { double t = run([&](int b){ copy_kernel<8,true><<<GRID(8),256>>>(in[b], out[b], n4); }, iters, nbuf); REPORT("copy  U=8 nontemporal", 2*bytes, t); }
+    { double t = run([&](int b){ quantlike_kernel<4><<<GRID(4),256>>>(in[b], (unsigned*)out[b], n4); }, iters, nbuf); REPORT("quant-like 16B in / 4B out U=4", bytes + bytes/4, t); }
+    { double t = run([&](int b){ quantlike_kernel<8><<<GRID(8),256>>>(in[b], (unsigned*)out[b], n4); }, iters, nbuf); REPORT("quant-like 16B in / 4B out U=8", bytes + bytes/4, t); }
+    { double t = run([&](int b){ CK(hipMemcpyAsync(out[b], in[b], bytes, hipMemcpyDeviceToDevice, 0)); }, iters, nbuf); REPORT("hipMemcpyAsync D2D", 2*bytes, t); }
+    return 0;
+}
