@@ -734,7 +734,7 @@ def main() -> int:
                 })
             check = None
             if parity:
-                from oracle import codec_np, ring_np
+                from oracle import ring_np
 
                 small = 64 * 1000 + 7
                 incoming = torch.empty(ops.payload_nbytes(small, G), dtype=torch.uint8, device=dev)

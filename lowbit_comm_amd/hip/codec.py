@@ -15,7 +15,7 @@ from typing import Any
 
 import torch
 
-from lowbit_comm_amd.communication.collectives import CompressedPayload, PackedPayload
+from lowbit_comm_amd.communication.collectives import PackedPayload
 from lowbit_comm_amd.config import CompressionConfig
 from lowbit_comm_amd.hip import ops
 from lowbit_comm_amd.quantization.error_feedback import ErrorFeedbackState

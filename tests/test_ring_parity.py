@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from oracle import codec_np, ring_np
+from oracle import ring_np
 
 pytestmark = pytest.mark.gpu
 
