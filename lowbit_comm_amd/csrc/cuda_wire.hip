@@ -23,6 +23,7 @@
 #include "launch.h"
 #include "wire_common.h"
 
+
 namespace lbc {
 namespace {
 
@@ -95,16 +96,13 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             float p[VEC];
-            uint32_t m = 0;
-            bool has_nan = false;
+            uint32_t m = 0;   // largest magnitude pattern; above the pattern of infinity when the lane holds a NaN
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
                 float v = widen(xv[u][i]);
                 if constexpr (HAS_R) v = round_through<T>(v + widen(rv[u][i]));
                 p[i] = v;
-                uint32_t bits = as_u32(v) & 0x7FFFFFFFu;
-                has_nan |= bits > 0x7F800000u;
-                bits = bits > 0x7F800000u ? 0u : bits;   // fmaxf skips NaN
+                const uint32_t bits = as_u32(v) & 0x7FFFFFFFu;
                 m = bits > m ? bits : m;
             }
             const int64_t group = e0[u] / G;
@@ -113,12 +111,21 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
             float multiplier = group_multiplier(m, absmax);
             Raw stored = __builtin_bit_cast(Raw, narrow<T>(absmax));
             bool wide_codes = false;   // wavefront-uniform: codes may leave [-LEVELS, LEVELS]
-            if constexpr (!HAS_R) {
-                if (resets && __ballot(has_nan) != 0) {
+            if (__ballot(m > 0x7F800000u) != 0) {   // a NaN somewhere in the wavefront: rare, and uniform
+                if (!HAS_R && resets) {
                     const uint32_t scale_raw = scan_scale(xv[u], group, k0);
                     multiplier = multiplier_of(value_of<T>(scale_raw));
                     stored = static_cast<Raw>(scale_raw);
                     wide_codes = true;
+                } else {                            // fmaxf skips NaNs
+                    uint32_t skipping = 0;
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) {
+                        const uint32_t bits = as_u32(p[i]) & 0x7FFFFFFFu;
+                        skipping = (bits <= 0x7F800000u && bits > skipping) ? bits : skipping;
+                    }
+                    multiplier = group_multiplier(skipping, absmax);
+                    stored = __builtin_bit_cast(Raw, narrow<T>(absmax));
                 }
             }
             int c[VEC];
@@ -359,7 +366,7 @@ hipError_t launch_wire_reduce_t(int g, int world, bool fma, int mode, const Wire
 // decode of one payload (optionally combined into `out`), or of `world` shard payloads
 // ---------------------------------------------------------------------------
 template <typename T, int OP> __device__ __forceinline__ float combine_in(float old, float v) {
-    if constexpr (OP == 1) return add_rounded_once<T>(old, v);
+    if constexpr (OP == 1) return add_in<T>(old, v);
     else if constexpr (OP == 2) return old > v ? old : v;
     else if constexpr (OP == 3) return old > v ? v : old;
     else return v;
@@ -485,6 +492,8 @@ hipError_t launch_wire_decode_t(int g, int bit, int op, int mode, const WireDeco
 // codes, whole groups (the reference's in-place decode needs them).  The encode is the one a chunk of whole groups
 // without a residual gets in the reference: group maximum with NaNs skipped, and when a group holds a NaN the
 // running maximum of the general kernels, which a NaN resets (see wire_quant_kernel).
+template <typename T, bool ACC> constexpr int wire_ring_unroll() { return ACC || sizeof(T) == 2 ? 1 : 4; }
+
 template <typename T, int G, bool COMPACT, int NT, bool ACC>
 __global__ __launch_bounds__(kBlock) void wire_ring_step_kernel(const WireRingStepArgs a) {
     constexpr int PNT_LOAD = payload_load_hint<COMPACT, NT, 1>();
@@ -493,7 +502,9 @@ __global__ __launch_bounds__(kBlock) void wire_ring_step_kernel(const WireRingSt
     using Raw = typename raw_bits<T>::type;
     constexpr int VEC = W::VEC;
     constexpr int LPG = G / VEC;
-    constexpr int UNROLL = ACC ? 1 : 2;
+    // Tiles in flight per wavefront, as measured on 6.5 M to 52 M element chunks: one for the accumulating step and
+    // for 16-bit chunks, four for the write-only steps on fp32 chunks.
+    constexpr int UNROLL = wire_ring_unroll<T, ACC>();
     constexpr int BLOCK_ELEMS = W::TILE * kWavesPerBlock * UNROLL;
     static_assert(LPG >= 1 && LPG <= 16, "a group must fit one DPP row");
 
@@ -529,8 +540,7 @@ __global__ __launch_bounds__(kBlock) void wire_ring_step_kernel(const WireRingSt
     for (int u = 0; u < UNROLL; ++u) {
         float p[VEC];
         T held[VEC];
-        uint32_t m = 0;
-        bool has_nan = false;
+        uint32_t m = 0;   // largest magnitude pattern; above the pattern of infinity when the lane holds a NaN
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             p[i] = 0.0f;
@@ -541,13 +551,11 @@ __global__ __launch_bounds__(kBlock) void wire_ring_step_kernel(const WireRingSt
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
                 float v = round_through<T>(unpack_code<T, 8, W::WORDS>(words[u], i) * step);
-                if constexpr (ACC) v = add_rounded_once<T>(widen(xv[u][i]), v);
+                if constexpr (ACC) v = add_in<T>(widen(xv[u][i]), v);
                 if (scaled) v = round_through<T>(v * a.inv_divisor);
                 held[i] = narrow<T>(v);
                 p[i] = v;
-                uint32_t bits = as_u32(v) & 0x7FFFFFFFu;
-                has_nan |= bits > 0x7F800000u;
-                bits = bits > 0x7F800000u ? 0u : bits;   // fmaxf skips NaN
+                const uint32_t bits = as_u32(v) & 0x7FFFFFFFu;
                 m = bits > m ? bits : m;
             }
             store_elems<T, VEC, NT>(chunk + e0[u], held);
@@ -556,11 +564,11 @@ __global__ __launch_bounds__(kBlock) void wire_ring_step_kernel(const WireRingSt
         // every lane of a row takes part in the group reductions; rows past the end carry zeros
         const int64_t group = e0[u] / G;
         const int k0 = static_cast<int>(e0[u] - group * G);
-        const float absmax = as_f32(group_max_bits<LPG>(m));
-        float scale = absmax < 1.0e-6f ? 1.0e-6f : absmax;    // a NaN stays and zeroes every code
+        const float absmax = as_f32(group_max_bits<LPG>(m));   // the group maximum when the wavefront holds no NaN
+        float scale = absmax < 1.0e-6f ? 1.0e-6f : absmax;
         Raw kept = __builtin_bit_cast(Raw, narrow<T>(absmax));
         bool wide_codes = false;                               // wavefront-uniform
-        if (__ballot(has_nan) != 0) {
+        if (__ballot(m > 0x7F800000u) != 0) {                  // a NaN somewhere: every group is scanned again
             uint32_t mag[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) mag[i] = __builtin_bit_cast(Raw, held[i]) & raw_bits<T>::ABS;
@@ -587,7 +595,7 @@ __global__ __launch_bounds__(kBlock) void wire_ring_step_kernel(const WireRingSt
 
 template <typename T, int G, bool COMPACT, bool ACC>
 hipError_t launch_wire_ring_c(int mode, const WireRingStepArgs &a, hipStream_t stream) {
-    constexpr int BLOCK_ELEMS = wire<T, 8>::TILE * kWavesPerBlock * (ACC ? 1 : 2);
+    constexpr int BLOCK_ELEMS = wire<T, 8>::TILE * kWavesPerBlock * wire_ring_unroll<T, ACC>();
     const int64_t blocks = (a.numel + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;

@@ -332,7 +332,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const float o = value_of<T>(old[i]), d = value_of<T>(decoded[i]);
-            if (a.op == 1) decoded[i] = static_cast<Raw>(raw_from<T>(add_rounded_once<T>(o, d)));
+            if (a.op == 1) decoded[i] = static_cast<Raw>(raw_from<T>(add_in<T>(o, d)));
             else if (a.op == 2) decoded[i] = o > d ? old[i] : decoded[i];
             else decoded[i] = o > d ? decoded[i] : old[i];
         }

@@ -90,6 +90,18 @@ def test_scale_formula_is_exact_for_every_finite_float(tmp_path):
     assert "0x3C010204" in done.stdout
 
 
+def test_sum_of_two_16_bit_values_through_fp32_is_the_native_sum(tmp_path):
+    """The CUDA-format kernels add two fp16 / bfloat16 values with one fp32 add and one conversion; for every pair
+    of finite values of either type that is the correctly rounded 16-bit sum (about half a minute on 8 cores)."""
+    binary = tmp_path / "check_half_sum"
+    subprocess.run(["gcc", "-O2", "-fopenmp", "-ffp-contract=off", "-o", str(binary),
+                    str(ROOT / "tests" / "native" / "check_half_sum.c"), "-lm"], check=True)
+    done = subprocess.run([str(binary)], capture_output=True, text=True, timeout=900)
+    assert done.returncode == 0, done.stdout
+    assert "fp16: 2015394816 pairs, 0 mismatches" in done.stdout
+    assert "bfloat16: 2130771840 pairs, 0 mismatches" in done.stdout
+
+
 def test_device_code_has_no_instruction_that_changes_the_rounding_contract(tmp_path):
     """The parity argument rests on build flags: products and sums round separately.  Compile the two kernel
     files to assembly with the Makefile's flags and check that no packed-fp32 arithmetic and no
