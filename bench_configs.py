@@ -713,7 +713,9 @@ def main() -> int:
         for label, n, dtype, sets_n in (("fp32 chunk of 6,553,600 (200 MiB bucket / 8)", 6_553_600, torch.float32, 8),
                                         ("bf16 chunk of 1,638,400 (25 MiB bucket / 8)", 1_638_400, torch.bfloat16, 24),
                                         ("fp32 chunk of 26,214,400 (a size past the launch ramp-up)", 26_214_400,
-                                         torch.float32, 4)):
+                                         torch.float32, 4),
+                                        ("bf16 chunk of 52,428,800 (a size past the launch ramp-up)", 52_428_800,
+                                         torch.bfloat16, 3)):
             eb = 4 if dtype == torch.float32 else 2
             pb = ops.payload_nbytes(n, G)
             sets = []
@@ -780,23 +782,27 @@ def main() -> int:
                  (payload_bytes + 2 * n * eb) + (n * eb + payload_bytes), timed(separate, args.iters * 2), n * eb, check)
             del sets
 
-        # the same hop in the CUDA extension's byte format (interleaved scales)
+        # the same hop in the CUDA extension's byte format (scales interleaved with the codes, or appended)
         from lowbit_comm_amd.hip import cuda_wire as cw
 
-        for label, n, dtype, sets_n in (("fp32 chunk of 6,553,600", 6_553_600, torch.float32, 8),
-                                        ("fp32 chunk of 26,214,400", 26_214_400, torch.float32, 4),
-                                        ("bf16 chunk of 13,107,200", 13_107_200, torch.bfloat16, 8)):
+        for label, n, dtype, sets_n, compact in (
+                ("fp32 chunk of 6,553,600", 6_553_600, torch.float32, 8, True),
+                ("fp32 chunk of 26,214,400", 26_214_400, torch.float32, 4, True),
+                ("bf16 chunk of 13,107,200", 13_107_200, torch.bfloat16, 8, True),
+                ("bf16 chunk of 52,428,800", 52_428_800, torch.bfloat16, 3, True),
+                ("bf16 chunk of 52,428,800, appended scales", 52_428_800, torch.bfloat16, 3, False)):
             eb = 4 if dtype == torch.float32 else 2
             pb = cw.payload_nbytes(n, dtype)
             sets = []
             for k in range(sets_n):
-                received = cw.quant_pack(gen(SEED + 8500 + k, n, 1e-3, dtype))
+                received = cw.quant_pack(gen(SEED + 8500 + k, n, 1e-3, dtype), compact=compact)
                 chunk = gen(SEED + 8600 + k, n, 1e-3, dtype)
                 send = torch.empty(pb, dtype=torch.uint8, device=dev)
                 sets.append({"chunk": chunk, "send": send, "received": received,
-                             "sum": cw.bind_ring_step(received, chunk, send, reduce_op="sum"),
-                             "decode_sum": cw.bind_dequant(received, chunk, reduce_op="sum"),
-                             "quant": cw.bind_quant_pack(chunk, send)})
+                             "sum": cw.bind_ring_step(received, chunk, send, reduce_op="sum", compact=compact),
+                             "copy": cw.bind_ring_step(received, chunk, send, reduce_op="none", compact=compact),
+                             "decode_sum": cw.bind_dequant(received, chunk, reduce_op="sum", compact=compact),
+                             "quant": cw.bind_quant_pack(chunk, send, compact=compact)})
             check = None
             if parity:
                 a, b = sets[0], sets[1]
@@ -805,6 +811,8 @@ def main() -> int:
                 check = "bit-exact vs separate launches" if bits_equal(a["chunk"], b["chunk"]) and torch.equal(a["send"], b["send"]) else "MISMATCH"
             emit(8, f"ring step in the CUDA byte format, {label}: decode + accumulate + requantize, one launch",
                  2 * pb + 2 * n * eb, timed(lambda i: sets[i % sets_n]["sum"](), args.iters * 2), n * eb, check)
+            emit(8, f"ring step in the CUDA byte format, {label}: decode + requantize (gather hop)",
+                 2 * pb + n * eb, timed(lambda i: sets[i % sets_n]["copy"](), args.iters * 2), pb, check)
 
             def separate_wire(i):
                 sets[i % sets_n]["decode_sum"]()

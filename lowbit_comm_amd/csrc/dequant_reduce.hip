@@ -104,10 +104,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
                     acc[i] = round_through<OT>(acc[i] + t);
                 }
             }
-            if (mean) {
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) acc[i] = round_through<OT>(acc[i] / a.divisor);
-            }
+            if (mean) divide_all<OT, VEC>(acc, a.divisor);
             OT o[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) o[i] = narrow<OT>(acc[i]);
@@ -227,10 +224,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_quant_kernel(const Redu
                 p[i] = round_through<MT>(p[i] + t);
             }
         }
-        if (mean) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) p[i] = round_through<MT>(p[i] / a.divisor);
-        }
+        if (mean) divide_all<MT, VEC>(p, a.divisor);
         if (e0 + VEC > a.numel) {
 #pragma unroll
             for (int i = 0; i < VEC; ++i) p[i] = e0 + i < a.numel ? p[i] : 0.0f;

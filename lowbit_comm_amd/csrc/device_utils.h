@@ -196,6 +196,23 @@ __device__ __forceinline__ int cvt_i32(float v) {  // NaN -> 0, saturating
     return c;
 }
 
+// v[i] = T(v[i] / divisor) for a divisor that is the same for the whole grid (the mean of a reduction).  When the
+// divisor is a power of two whose reciprocal is a normal float - the usual world sizes - the product with that
+// reciprocal is taken instead: both are the correctly rounded value of the same real number, so the bits agree for
+// every input, and the division's ten-odd instructions per element become one.
+template <typename T, int N> __device__ __forceinline__ void divide_all(float (&v)[N], float divisor) {
+    const uint32_t bits = as_u32(divisor);
+    const uint32_t exponent = bits >> 23;                  // the sign bit is part of it: positive divisors only
+    if ((bits & 0x007FFFFFu) == 0 && exponent >= 2 && exponent <= 252) {
+        const float reciprocal = as_f32((254u - exponent) << 23);
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = round_through<T>(v[i] * reciprocal);
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = round_through<T>(v[i] / divisor);
+    }
+}
+
 // codes[i] = rint(p[i] / scale) as the reference computes it (IEEE division, then round-half-even), a NaN
 // quotient -> 0.  A code comes back as the bit pattern of (code + 1.5 * 2^23): its low byte is the int8 code that
 // goes into the payload (pack4 takes low bytes), and code_value() gives the integer back as a float.

@@ -76,10 +76,11 @@ __global__ __launch_bounds__(kBlock) void ring_step_kernel(const RingStepArgs a)
             for (int i = 0; i < VEC; ++i) {
                 float v = round_through<T>(code_to_float(words[u][i / 4], i % 4) * rscale[u]);
                 if constexpr (ACC) v = round_through<T>(widen(xv[u][i]) + v);
-                if (mean) v = round_through<T>(v / a.divisor);
                 p[i] = v;
-                out[i] = narrow<T>(v);
             }
+            if (mean) divide_all<T, VEC>(p, a.divisor);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) out[i] = narrow<T>(p[i]);
             store_wide<T, VEC, MODE>(chunk + e0[u], out);
             if (emit) {
                 const float scale = group_scale<VEC, LPG>(p);
