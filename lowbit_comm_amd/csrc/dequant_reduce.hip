@@ -14,7 +14,8 @@
 // Semantics follow the reference's portable path: decode each payload with one
 // rounding (ccdl_comm/quantization/torch_fallback.py:48-53) and add them left to
 // right in list order (ccdl_comm/communication/gather_reduce.py:39-45) in the
-// output dtype; "mean" is a true division.  The translation unit is compiled
+// output dtype; "mean" is a true division (divide_all: by the bit-identical
+// product with the reciprocal when the divisor is a power of two).  The translation unit is compiled
 // with -ffp-contract=off so that no product/sum pair is fused into an FMA.
 #include "device_utils.h"
 #include "launch.h"

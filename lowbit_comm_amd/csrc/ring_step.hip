@@ -11,7 +11,7 @@
 // Per element, in the order the two-kernel sequence rounds:
 //   d = T(float(code) * scale)                  decode, rounded to the chunk's type T
 //   v = T(float(chunk) + d)      (ACC only)     the in-place sum in T arithmetic
-//   v = T(v / divisor)           (divisor != 1) the in-place mean
+//   v = T(v / divisor)           (divisor != 1) the in-place mean (divide_all)
 //   chunk = v;  payload = quantize(v)           same group maximum, scale and rounding as quant_pack_kernel
 //
 // Mapping: one lane owns 16 bytes of the chunk (4 fp32 or 8 16-bit elements), a group sits in adjacent lanes of
