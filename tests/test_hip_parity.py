@@ -306,6 +306,31 @@ def test_dequant_reduce_mean_and_16bit_accumulation(ops, hip_device, world, out_
     assert_same_bits(out, want, "mean")
 
 
+@pytest.mark.parametrize("out_dtype", ["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("divisor", [8.0, 2.0, 0.5, 1024.0, 2.0 ** -20, 2.0 ** 125, 2.0 ** 126, 2.0 ** -125, 3.0, 7.0, 1.5])
+def test_mean_divides_exactly_for_every_kind_of_divisor(ops, hip_device, out_dtype, divisor):
+    """Power-of-two divisors take a product with the reciprocal inside the kernel, the others a division: either
+    way the result is the true quotient, also where it is subnormal, overflows or starts from an infinity."""
+    n, g = 64 * 257, 64
+    rng = np.random.default_rng(int(abs(np.log2(divisor)) * 10) + 3)
+    # every decoded value stays finite in the output type, so no sum is inf - inf (the sign of a generated NaN is
+    # the one thing a CPU and a GPU may differ in); sums still overflow to infinity and quotients go subnormal
+    if out_dtype == "fp16":
+        scale_pool = np.array([1e-9, 1e-7, 6e-5, 1e-3, 1.0, 100.0, 500.0], dtype=np.float32)
+    else:
+        scale_pool = np.array([2.0 ** -140, 1e-38, 2.0 ** -126, 3e-30, 1e-3, 1.0, 1e30, 2e36], dtype=np.float32)
+    payloads = []
+    for _ in range(2):
+        codes = torch.from_numpy(rng.integers(-127, 128, n, dtype=np.int8)).to(hip_device)
+        scales = torch.from_numpy(rng.choice(scale_pool, n // g)).to(hip_device)
+        payloads.append((codes, scales))
+    out = torch.empty(n, dtype=DTYPES[out_dtype], device=hip_device)
+    assert ops.dequant_reduce_into(payloads, out, divisor=divisor)
+    total = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in payloads], n, g, out_dtype, "sum")
+    want = (total.float() / torch.tensor(divisor, dtype=torch.float32)).to(DTYPES[out_dtype])
+    assert_same_bits(out, want, f"mean by {divisor}")
+
+
 def test_dequant_reduce_order_follows_the_list(ops, hip_device):
     n = 64 * 2000
     payloads = make_payloads(ops, 8, n, hip_device, 700)
