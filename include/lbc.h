@@ -5,8 +5,8 @@
  * current HIP device unless stated otherwise, every launch is asynchronous on
  * the `stream` argument (a hipStream_t passed as void*; NULL = the null
  * stream), nothing here allocates, frees or synchronises, and the only state is a
- * per-thread error string and one process-wide tuning threshold
- * (lbc_set_stream_min_bytes).  Inputs are never written.
+ * per-thread error string: what a call does depends on its arguments alone.
+ * Inputs are never written.
  *
  * Wire format ("format A", the reference's portable codec,
  * ccdl_comm/quantization/torch_fallback.py:24-36): for a flat tensor of n
@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define LBC_ABI_VERSION 6
+#define LBC_ABI_VERSION 7
 
 enum { LBC_OK = 0, LBC_UNSUPPORTED = 1, LBC_EINVAL = -1, LBC_ELAUNCH = -2 };
 
@@ -53,13 +53,20 @@ int lbc_abi_version(void);
 const char *lbc_last_error(void);
 
 /*
- * Tuning knob with no counterpart in the reference: calls that move at least
- * `min_bytes` use non-temporal (streaming) loads and stores, smaller ones plain
- * vector access.  Process-wide; the initial value is 96 MiB or the environment
- * variable LBC_STREAM_MIN_BYTES.  Returns the previous threshold.  Results do not
- * depend on it.
+ * Access mode, the `access` argument of every launching entry point (no counterpart in the
+ * reference).  It selects cache hints only; results never depend on it.
+ *   LBC_ACCESS_AUTO    the library's rule, which looks at the call's arguments and nothing else:
+ *                      today the same as LBC_ACCESS_STREAM.
+ *   LBC_ACCESS_CACHED  plain cached loads and stores.  For a caller that knows the operands were
+ *                      produced on this GPU a moment ago and still sit in its caches (measured ~5 %
+ *                      faster than streaming then, 10-25 % slower when they do not).
+ *   LBC_ACCESS_STREAM  non-temporal loads (each operand is read once); stores plain, non-temporal or
+ *                      written through, as measured best per kernel and output size.
+ * Operands without the alignment the vector kernels need (16 bytes for tensors, the lane's code
+ * width for codes) are processed element by element under every mode.  Any other value:
+ * LBC_EINVAL.
  */
-int64_t lbc_set_stream_min_bytes(int64_t min_bytes);
+enum { LBC_ACCESS_AUTO = 0, LBC_ACCESS_CACHED = 1, LBC_ACCESS_STREAM = 2 };
 
 /*
  * Quantize + pack, optionally fused with error feedback.
@@ -85,7 +92,7 @@ int64_t lbc_set_stream_min_bytes(int64_t min_bytes);
 int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residual_dtype,
                    int64_t numel, int group_size, int8_t *codes, float *scales,
                    void *new_residual, int new_residual_dtype, void *restored, int restored_dtype,
-                   void *stream);
+                   int access, void *stream);
 
 /*
  * Quantize `world` equal destination chunks of one flat bucket in a single
@@ -105,7 +112,7 @@ int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residua
 int lbc_quant_pack_chunks(const void *x, int x_dtype, const void *residual, int residual_dtype,
                           int64_t numel, int world, int group_size, uint8_t *payloads,
                           int64_t payload_stride, void *new_residual, int new_residual_dtype,
-                          void *restored, int restored_dtype, void *stream);
+                          void *restored, int restored_dtype, int access, void *stream);
 
 /*
  * Decode one payload: out[i] (op)= float(code[i]) * scale[i/g], rounded to out_dtype.
@@ -116,7 +123,7 @@ int lbc_quant_pack_chunks(const void *x, int x_dtype, const void *residual, int 
  * multiple of group_size; exactly numel elements are written.
  */
 int lbc_dequant(const int8_t *codes, const float *scales, int64_t numel, int group_size,
-                void *out, int out_dtype, int reduce_op, void *stream);
+                void *out, int out_dtype, int reduce_op, int access, void *stream);
 
 /*
  * Fused dequant-reduce of `world` payloads (1..8) into one tensor, in the
@@ -139,7 +146,7 @@ int lbc_dequant(const int8_t *codes, const float *scales, int64_t numel, int gro
  */
 int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, int world,
                        int64_t numel, int group_size, float divisor, void *out, int out_dtype,
-                       const void *prepared, void *new_residual, void *stream);
+                       const void *prepared, void *new_residual, int access, void *stream);
 
 /*
  * Decode `world` payloads into `world` consecutive shards of one flat tensor in a
@@ -151,7 +158,7 @@ int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, i
  */
 int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world,
                        int64_t shard_numel, int64_t total_numel, int group_size, void *out,
-                       int out_dtype, void *stream);
+                       int out_dtype, int access, void *stream);
 
 /*
  * Fused reduce + requantize for the reduce-scatter -> all-gather hand-over: the payload of
@@ -166,7 +173,7 @@ int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int worl
  */
 int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *scales, int world,
                              int64_t numel, int group_size, float divisor, int mid_dtype,
-                             int8_t *out_codes, float *out_scales, void *stream);
+                             int8_t *out_codes, float *out_scales, int access, void *stream);
 
 /*
  * One compute step of the quantized ring all-reduce on one chunk of the bucket, in place:
@@ -186,7 +193,7 @@ int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *sca
  */
 int lbc_ring_step(const int8_t *recv_codes, const float *recv_scales, void *chunk, int dtype,
                   int64_t numel, int group_size, int reduce_op, float divisor, int8_t *send_codes,
-                  float *send_scales, void *stream);
+                  float *send_scales, int access, void *stream);
 
 /*
  * residual = prepared - restored, element-wise, subtraction in fp32, rounded to
@@ -196,7 +203,7 @@ int lbc_ring_step(const int8_t *recv_codes, const float *recv_scales, void *chun
  * ErrorFeedbackState.update (ccdl_comm/quantization/error_feedback.py:38-41).
  */
 int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored, int restored_dtype,
-                  void *residual, int residual_dtype, int64_t numel, void *stream);
+                  void *residual, int residual_dtype, int64_t numel, int access, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Payload format of the reference's CUDA extension ("format B", the bytes ccdl_cuda_ops
@@ -232,13 +239,13 @@ int64_t lbc_wire_payload_nbytes(int64_t numel, int group_size, int dtype, int bi
  * per call (per chunk in the chunked form).
  */
 int lbc_wire_quant_pack(const void *x, const void *residual, int dtype, int64_t numel, int group_size,
-                        int bit, int compact, uint8_t *payload, void *stream);
+                        int bit, int compact, uint8_t *payload, int access, void *stream);
 
 /* As lbc_quant_pack_chunks, in this format: chunk d of ceil(numel/world) elements becomes the
  * payload at payloads + d*payload_stride (ccdl_comm/cuda/transports/compressed_reduce_scatter.py:72-94). */
 int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, int64_t numel, int world,
                                int group_size, int bit, int compact, uint8_t *payloads,
-                               int64_t payload_stride, void *stream);
+                               int64_t payload_stride, int access, void *stream);
 
 /*
  * Decode one payload into out (reduce_op NONE) or combine it with the values already in out:
@@ -247,12 +254,12 @@ int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, i
  * dequant_kernel.cuh:46-60, pybind.cpp:64-90).
  */
 int lbc_wire_dequant(const uint8_t *payload, int64_t numel, int group_size, int bit, int compact, void *out,
-                     int dtype, int reduce_op, void *stream);
+                     int dtype, int reduce_op, int access, void *stream);
 
 /* As lbc_dequant_chunks, in this format (ccdl_comm/communication/topology_transport.py:866-894). */
 int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world, int64_t shard_numel,
                             int64_t total_numel, int group_size, int bit, int compact, void *out, int dtype,
-                            int reduce_op, void *stream);
+                            int reduce_op, int access, void *stream);
 
 /*
  * out = dtype(sum_r float(code_r) * (scale_r / 127) * inv_divisor), payloads added in list order in
@@ -265,7 +272,7 @@ int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int
  */
 int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t numel, int group_size,
                             int compact, float inv_divisor, int fused_multiply_add, void *out, int dtype,
-                            const void *prepared, void *new_residual, void *stream);
+                            const void *prepared, void *new_residual, int access, void *stream);
 
 /*
  * One hop of the quantized ring or tree in this format, in place on a chunk of whole groups:
@@ -282,7 +289,7 @@ int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t n
  * LBC_UNSUPPORTED.
  */
 int lbc_wire_ring_step(const uint8_t *received, void *chunk, int dtype, int64_t numel, int group_size,
-                       int compact, int reduce_op, float divisor, uint8_t *send, void *stream);
+                       int compact, int reduce_op, float divisor, uint8_t *send, int access, void *stream);
 
 /*
  * The remaining policies of the CUDA extension's format: non-linear 4-bit code books

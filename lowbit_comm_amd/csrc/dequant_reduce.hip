@@ -45,6 +45,31 @@ template <typename OT, int W = 8> struct decode_tiling {
 template <int W> __device__ __forceinline__ constexpr int code_load_mode(int mode) {
     return mode == kStream && W < 4 ? kVector : mode;
 }
+// Cache policy of the fused reduce under the streaming modes, from sweeps of every load/store policy pair at
+// W = 1, 2, 4, 8 on 3.3 M, 6.6 M and 26 M fp32 elements with buffers rotating through 650 MB.  The non-temporal
+// hint pays on the direction that carries most of the bytes and costs when both directions carry it:
+//   reads/writes < 0.8  (W = 1, 2 for fp32)  plain code loads, non-temporal stores       (26 M, W = 1: 19.0 us; with
+//                                             non-temporal loads as well 24.8 us)
+//   up to 1.6           (W = 4)               non-temporal loads; stores non-temporal, or written through for
+//                                             outputs beyond the L2s
+//   above               (W = 8)               non-temporal loads; plain stores while the output fits the L2s
+//                                             (3.3 M: 7.9 us against 8.1 written through, 8.4 non-temporal - the
+//                                             write-back then overlaps the next kernel's ramp), written through
+//                                             beyond (26 M: 47.3 us against 50.2 plain, 53.6 non-temporal)
+// The host picks kStream or kStreamThrough by the size of the output.
+template <typename OT, int W> constexpr int read_write_class() {
+    constexpr int reads16 = W * 17, writes16 = static_cast<int>(sizeof(OT)) * 16;   // bytes per element, x16
+    return reads16 * 10 < writes16 * 8 ? 0 : (reads16 * 10 < writes16 * 16 ? 1 : 2);
+}
+template <typename OT, int W, int MODE> constexpr int code_policy() {
+    return MODE >= kStream && read_write_class<OT, W>() >= 1 ? kNtBit : kCached;
+}
+template <typename OT, int W, int MODE> constexpr int reduce_store_policy() {
+    if (MODE < kStream) return kCached;
+    if (read_write_class<OT, W>() == 0) return kNtBit;
+    if (MODE == kStreamThrough) return kSc1Bit;
+    return read_write_class<OT, W>() == 1 ? kNtBit : kCached;
+}
 
 template <int VEC, int MODE>
 __device__ __forceinline__ void load_codes(const int8_t *__restrict__ p, uint32_t (&w)[VEC / 4]) {
@@ -71,27 +96,37 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(T::BLOCK_ELEMS)) * T::BLOCK_ELEMS;
+    // every XCD walks one contiguous eighth of the shard at any size: with the policies above that measured
+    // 6-15 % faster than the round-robin order from 3 M to 26 M elements (W = 8), and no slower at W = 1, 2, 4
+    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block<true>(T::BLOCK_ELEMS)) * T::BLOCK_ELEMS;
     OT *__restrict__ out = static_cast<OT *>(a.out);
     const OT *prepared = static_cast<const OT *>(a.prepared);  // may alias new_r
     OT *new_r = static_cast<OT *>(a.new_residual);
     const bool mean = a.divisor != 1.0f;
 
     if (MODE != kScalar && block_first + T::BLOCK_ELEMS <= a.numel) {
-        // ---- interior block ---------------------------------------------------
+        // ---- interior block: one descriptor per stream over the block's span, 32-bit offsets per lane ----
+        constexpr int kCodes = code_policy<OT, W, MODE>();
+        constexpr int kLoad = policy_of<MODE>();
+        constexpr int kStore = reduce_store_policy<OT, W, MODE>();
         uint32_t words[UNROLL][W][VEC / 4];
         float scale[UNROLL][W];
-        int64_t e0[UNROLL];
+        uint32_t at[UNROLL];   // element offset inside the block
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
-            const int64_t g = e0[u] / G;
+        for (int u = 0; u < UNROLL; ++u) at[u] = static_cast<uint32_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
 #pragma unroll
-            for (int r = 0; r < W; ++r) {
-                load_codes<VEC, code_load_mode<W>(MODE)>(a.codes[r] + e0[u], words[u][r]);
-                scale[u][r] = a.scales[r][g];
+        for (int r = 0; r < W; ++r) {
+            const buffer_t codes = buffer_over(a.codes[r] + block_first, T::BLOCK_ELEMS);
+            const buffer_t scales = buffer_over(a.scales[r] + block_first / G, T::BLOCK_ELEMS / G * 4);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                buffer_load<uint32_t, VEC / 4, kCodes>(codes, at[u], words[u][r]);
+                float one[1];
+                buffer_load<float, 1, kCached>(scales, at[u] / G * 4, one);
+                scale[u][r] = one[0];
             }
         }
+        const buffer_t out_b = buffer_over(out + block_first, T::BLOCK_ELEMS * sizeof(OT));
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             float acc[VEC];
@@ -109,13 +144,13 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs
             OT o[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) o[i] = narrow<OT>(acc[i]);
-            store_vec<OT, VEC, MODE>(out + e0[u], o);
+            buffer_store<OT, VEC, kStore>(out_b, at[u] * sizeof(OT), o);
             if (new_r != nullptr) {
                 OT pv[VEC], d[VEC];
-                load_vec<OT, VEC, MODE>(prepared + e0[u], pv);
+                buffer_load<OT, VEC, kLoad>(buffer_over(prepared + block_first, T::BLOCK_ELEMS * sizeof(OT)), at[u] * sizeof(OT), pv);
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) d[i] = narrow<OT>(widen(pv[i]) - acc[i]);
-                store_vec<OT, VEC, MODE>(new_r + e0[u], d);
+                buffer_store<OT, VEC, kStore>(buffer_over(new_r + block_first, T::BLOCK_ELEMS * sizeof(OT)), at[u] * sizeof(OT), d);
             }
         }
         return;
@@ -148,6 +183,7 @@ hipError_t launch_reduce_w(int mode, const ReduceArgs &a, hipStream_t stream) {
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
     switch (mode) {
+        case kStreamThrough: hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, kStreamThrough>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a); break;
         case kStream: hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, kStream>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a); break;
         case kVector: hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, kVector>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a); break;
         default: hipLaunchKernelGGL((dequant_reduce_kernel<OT, G, W, kScalar>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, stream, a); break;
@@ -199,7 +235,7 @@ __global__ __launch_bounds__(kBlock) void dequant_reduce_quant_kernel(const Redu
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
     const int64_t padded = (a.numel + G - 1) / G * G;
-    const int64_t e0 = static_cast<int64_t>(xcd_contiguous_block(BLOCK_ELEMS)) * BLOCK_ELEMS + static_cast<int64_t>(wave) * TILE + lane * VEC;
+    const int64_t e0 = static_cast<int64_t>(xcd_contiguous_block<true>(BLOCK_ELEMS)) * BLOCK_ELEMS + static_cast<int64_t>(wave) * TILE + lane * VEC;
     const bool live = e0 < padded;     // whole lanes: padded and e0 are multiples of VEC
     const bool mean = a.divisor != 1.0f;
 

@@ -36,21 +36,26 @@ template <int UNROLL> __device__ __forceinline__ int tile_in_block(int u, int wa
 #ifndef LBC_XCD_SPAN_ELEMS
 #define LBC_XCD_SPAN_ELEMS (1 << 22)
 #endif
+template <bool ALWAYS = false>
 __device__ __forceinline__ unsigned xcd_contiguous_block(int block_elems) {
     const unsigned per_xcd = gridDim.x >> 3;
-    const bool remap = static_cast<int64_t>(gridDim.x) * block_elems <= LBC_XCD_SPAN_ELEMS && blockIdx.x < (per_xcd << 3);
+    const bool in_span = ALWAYS || static_cast<int64_t>(gridDim.x) * block_elems <= LBC_XCD_SPAN_ELEMS;
+    const bool remap = in_span && blockIdx.x < (per_xcd << 3);
     return remap ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
 }
 constexpr uint32_t kEpsBits = 0x34000000u;  // 2^-23, torch.finfo(float32).eps
 
 // Access modes of the bulk loads and stores.  kScalar: element by element (any
 // alignment).  kVector: one vector instruction per lane (the caller guarantees
-// N*sizeof(T) alignment).  kStream: vector instructions carrying the
-// non-temporal hint - every tensor here is read once and written once, and on
-// working sets well beyond the last-level cache the hint raises achieved
-// bandwidth; small working sets do better without it because the producer's
-// lines are still cached.
-enum AccessMode { kScalar = 0, kVector = 1, kStream = 2 };
+// N*sizeof(T) alignment), plain cached accesses - for operands that are known to
+// sit in the last-level cache.  kStream: vector instructions with the
+// non-temporal hint on the loads - every tensor here is read once, and when it is
+// not already cached the hint measured 10-25 % more bandwidth at every size from
+// 16 MB to 600 MB of traffic (with it the time no longer depends on what the
+// 256 MiB memory-side cache holds; cached loads are ~5 % faster only when
+// everything is resident).  Stores under kStream are chosen per kernel.
+// kStreamThrough (fused reduce only): kStream with write-through stores.
+enum AccessMode { kScalar = 0, kVector = 1, kStream = 2, kStreamThrough = 3 };
 
 template <typename T, int N>
 using vec_t = T __attribute__((ext_vector_type(N)));
@@ -137,6 +142,81 @@ __device__ __forceinline__ void store_wide(T *__restrict__ p, const T (&src)[N])
 #pragma unroll
             for (int i = 0; i < PER; ++i) piece[i] = src[k * PER + i];
             store_vec<T, PER, MODE>(p + k * PER, piece);
+        }
+    }
+}
+
+// ---- buffer addressing ---------------------------------------------------------
+// A descriptor over [base, base + bytes) held in scalar registers.  Loads and stores through it take a 32-bit
+// byte offset per lane, so a wavefront spends no vector instructions on 64-bit addresses before its first load
+// is out (on shard-sized launches, which are all ramp, that measured 6-9 % of the kernel), and an access past
+// `bytes` is dropped by the hardware instead of faulting.  The interior blocks of the kernels build one
+// descriptor per stream over the block's own span.
+using buffer_t = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ buffer_t buffer_over(const void *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+// Cache policy operand of the buffer instructions: plain, the non-temporal bit, or (stores) the sc1 bit, which
+// makes a store write through the XCD's L2 instead of leaving a dirty line for a later eviction.
+constexpr int kCached = 0, kNtBit = 2, kSc1Bit = 16;
+template <int MODE> constexpr int policy_of() { return MODE >= kStream ? kNtBit : kCached; }
+
+using u32x2 = vec_t<uint32_t, 2>;
+using u32x4 = vec_t<uint32_t, 4>;
+
+// N elements of T (4, 8 or 16 bytes, or a multiple of 16) at byte offset `at`.
+template <typename T, int N, int POLICY>
+__device__ __forceinline__ void buffer_load(buffer_t b, uint32_t at, T (&dst)[N]) {
+    constexpr int BYTES = N * sizeof(T);
+    static_assert(BYTES == 4 || BYTES == 8 || BYTES % 16 == 0, "whole dwords");
+    using V = vec_t<T, N>;
+    if constexpr (BYTES == 4) {
+        const uint32_t w = __builtin_amdgcn_raw_buffer_load_b32(b, at, 0, POLICY);
+        const V v = __builtin_bit_cast(V, w);
+#pragma unroll
+        for (int i = 0; i < N; ++i) dst[i] = v[i];
+    } else if constexpr (BYTES == 8) {
+        const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(b, at, 0, POLICY);
+        const V v = __builtin_bit_cast(V, w);
+#pragma unroll
+        for (int i = 0; i < N; ++i) dst[i] = v[i];
+    } else {
+        constexpr int PER = 16 / sizeof(T);
+        using P = vec_t<T, PER>;
+#pragma unroll
+        for (int k = 0; k < BYTES / 16; ++k) {
+            const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(b, at + 16 * k, 0, POLICY);
+            const P v = __builtin_bit_cast(P, w);
+#pragma unroll
+            for (int i = 0; i < PER; ++i) dst[k * PER + i] = v[i];
+        }
+    }
+}
+
+template <typename T, int N, int POLICY>
+__device__ __forceinline__ void buffer_store(buffer_t b, uint32_t at, const T (&src)[N]) {
+    constexpr int BYTES = N * sizeof(T);
+    static_assert(BYTES == 4 || BYTES == 8 || BYTES % 16 == 0, "whole dwords");
+    using V = vec_t<T, N>;
+    if constexpr (BYTES == 4) {
+        V v;
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = src[i];
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), b, at, 0, POLICY);
+    } else if constexpr (BYTES == 8) {
+        V v;
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = src[i];
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), b, at, 0, POLICY);
+    } else {
+        constexpr int PER = 16 / sizeof(T);
+        using P = vec_t<T, PER>;
+#pragma unroll
+        for (int k = 0; k < BYTES / 16; ++k) {
+            P v;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) v[i] = src[k * PER + i];
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), b, at + 16 * k, 0, POLICY);
         }
     }
 }

@@ -1,14 +1,12 @@
 // C ABI of the codec library (declared in include/lbc.h): argument validation,
 // alignment probing and dispatch.  No allocation, no synchronisation, no state
-// besides a per-thread error string.
+// besides a per-thread error string: what a call does is a function of its arguments.
 #include "../../include/lbc.h"
 
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
-
-#include <atomic>
 
 #include "launch.h"
 
@@ -33,26 +31,13 @@ bool aligned_to(const void *p, uintptr_t bytes) { return (reinterpret_cast<uintp
 // torch promotion of two of {f32, f16, bf16}
 int promote(int a, int b) { return a == b ? a : LBC_F32; }
 
-// Streaming (non-temporal) access pays off once a call moves far more bytes than
-// the last-level cache holds; below that the producer's lines are still cached and
-// plain vector access is faster.  The threshold is a process-wide tuning knob:
-// LBC_STREAM_MIN_BYTES at first use, or lbc_set_stream_min_bytes().
-std::atomic<int64_t> g_stream_min{-1};
+// Access mode of a call (LBC_ACCESS_*): a function of the arguments only, no process state.  Operands that lack
+// the alignment of the vector paths take the element-wise kernels whatever the caller asked for.
+bool valid_access(int access) { return access >= LBC_ACCESS_AUTO && access <= LBC_ACCESS_STREAM; }
 
-int64_t stream_threshold() {
-    int64_t value = g_stream_min.load(std::memory_order_relaxed);
-    if (value < 0) {
-        const char *env = getenv("LBC_STREAM_MIN_BYTES");
-        value = env != nullptr ? atoll(env) : (int64_t{96} << 20);
-        if (value < 0) value = 0;
-        g_stream_min.store(value, std::memory_order_relaxed);
-    }
-    return value;
-}
-
-int pick_mode(bool aligned, int64_t bytes_moved) {
+int pick_mode(bool aligned, int access) {
     if (!aligned) return 0;
-    return bytes_moved >= stream_threshold() ? 2 : 1;
+    return access == LBC_ACCESS_CACHED ? 1 : 2;
 }
 
 int finish(hipError_t err, const char *what) {
@@ -70,7 +55,7 @@ namespace {
 int quant_pack_common(const char *what, const void *x, int x_dtype, const void *residual, int residual_dtype,
                       int64_t numel, int world, int group_size, uint8_t *codes_base, uint8_t *scales_base,
                       int64_t payload_stride, int64_t shard_numel, void *new_residual, int new_residual_dtype,
-                      void *restored, int restored_dtype, bool rows_aligned, void *stream) {
+                      void *restored, int restored_dtype, bool rows_aligned, int access, void *stream) {
     const int r_dtype = residual ? residual_dtype : LBC_NONE;
     const int p_dtype = residual ? promote(x_dtype, r_dtype) : x_dtype;
     const bool wants_outputs = new_residual != nullptr || restored != nullptr;
@@ -90,11 +75,9 @@ int quant_pack_common(const char *what, const void *x, int x_dtype, const void *
 
     const int vec = lbc::quant_pack_vec(x_dtype, r_dtype, d_dtype, wants_outputs);
     bool aligned = rows_aligned && aligned_to(x, 16) && aligned_to(codes_base, vec) && payload_stride % vec == 0;
-    int64_t moved = numel * (dtype_size(x_dtype) + 1);
     auto side = [&](const void *p, int dtype) {
         if (p == nullptr) return;
         aligned = aligned && aligned_to(p, 16) && (world == 1 || (shard_numel * dtype_size(dtype)) % 16 == 0);
-        moved += numel * dtype_size(dtype);
     };
     if (world > 1) aligned = aligned && (shard_numel * dtype_size(x_dtype)) % 16 == 0;
     side(residual, r_dtype);
@@ -112,7 +95,7 @@ int quant_pack_common(const char *what, const void *x, int x_dtype, const void *
     a.shard_numel = shard_numel;
     a.payload_stride = payload_stride;
     return finish(lbc::launch_quant_pack(x_dtype, r_dtype, d_dtype, wants_outputs, group_size,
-                                         pick_mode(aligned, moved), a, world, static_cast<hipStream_t>(stream)),
+                                         pick_mode(aligned, access), a, world, static_cast<hipStream_t>(stream)),
                   what);
 }
 
@@ -124,15 +107,10 @@ int lbc_abi_version(void) { return LBC_ABI_VERSION; }
 
 const char *lbc_last_error(void) { return g_error; }
 
-int64_t lbc_set_stream_min_bytes(int64_t min_bytes) {
-    const int64_t previous = stream_threshold();
-    g_stream_min.store(min_bytes < 0 ? 0 : min_bytes, std::memory_order_relaxed);
-    return previous;
-}
-
 int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel,
                    int group_size, int8_t *codes, float *scales, void *new_residual, int new_residual_dtype,
-                   void *restored, int restored_dtype, void *stream) {
+                   void *restored, int restored_dtype, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (!valid_dtype(x_dtype)) return fail(LBC_EINVAL, "unsupported input dtype %d", x_dtype);
     if (residual != nullptr && !valid_dtype(residual_dtype))
@@ -145,12 +123,13 @@ int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residua
     if (!aligned_to(x, dtype_size(x_dtype))) return fail(LBC_EINVAL, "input is not aligned to its element size");
     return quant_pack_common("lbc_quant_pack", x, x_dtype, residual, residual_dtype, numel, 1, group_size,
                              reinterpret_cast<uint8_t *>(codes), reinterpret_cast<uint8_t *>(scales), 0, numel,
-                             new_residual, new_residual_dtype, restored, restored_dtype, true, stream);
+                             new_residual, new_residual_dtype, restored, restored_dtype, true, access, stream);
 }
 
 int lbc_quant_pack_chunks(const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel,
                           int world, int group_size, uint8_t *payloads, int64_t payload_stride, void *new_residual,
-                          int new_residual_dtype, void *restored, int restored_dtype, void *stream) {
+                          int new_residual_dtype, void *restored, int restored_dtype, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
     if (!valid_dtype(x_dtype)) return fail(LBC_EINVAL, "unsupported input dtype %d", x_dtype);
@@ -169,11 +148,12 @@ int lbc_quant_pack_chunks(const void *x, int x_dtype, const void *residual, int 
     if (!aligned_to(x, dtype_size(x_dtype))) return fail(LBC_EINVAL, "input is not aligned to its element size");
     return quant_pack_common("lbc_quant_pack_chunks", x, x_dtype, residual, residual_dtype, numel, world, group_size,
                              payloads, payloads + groups * group_size, payload_stride, shard, new_residual,
-                             new_residual_dtype, restored, restored_dtype, true, stream);
+                             new_residual_dtype, restored, restored_dtype, true, access, stream);
 }
 
 int lbc_dequant(const int8_t *codes, const float *scales, int64_t numel, int group_size, void *out,
-                int out_dtype, int reduce_op, void *stream) {
+                int out_dtype, int reduce_op, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (!valid_dtype(out_dtype)) return fail(LBC_EINVAL, "unsupported output dtype %d", out_dtype);
     if (reduce_op < LBC_REDUCE_NONE || reduce_op > LBC_REDUCE_MIN)
@@ -193,13 +173,14 @@ int lbc_dequant(const int8_t *codes, const float *scales, int64_t numel, int gro
     a.shard_numel = numel;
     a.total_numel = numel;
     a.payload_stride = 0;
-    return finish(lbc::launch_decode(out_dtype, group_size, reduce_op, pick_mode(aligned, numel * (dtype_size(out_dtype) + 1)),
+    return finish(lbc::launch_decode(out_dtype, group_size, reduce_op, pick_mode(aligned, access),
                                      a, 1, static_cast<hipStream_t>(stream)),
                   "lbc_dequant");
 }
 
 int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world, int64_t shard_numel,
-                       int64_t total_numel, int group_size, void *out, int out_dtype, void *stream) {
+                       int64_t total_numel, int group_size, void *out, int out_dtype, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (shard_numel < 0 || total_numel < 0) return fail(LBC_EINVAL, "element counts must be >= 0");
     if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
     if (total_numel > shard_numel * world) return fail(LBC_EINVAL, "total_numel exceeds world * shard_numel");
@@ -225,14 +206,15 @@ int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int worl
     a.total_numel = total_numel;
     a.payload_stride = payload_stride;
     return finish(lbc::launch_decode(out_dtype, group_size, LBC_REDUCE_NONE,
-                                     pick_mode(aligned, total_numel * (dtype_size(out_dtype) + 1)), a, world,
+                                     pick_mode(aligned, access), a, world,
                                      static_cast<hipStream_t>(stream)),
                   "lbc_dequant_chunks");
 }
 
 int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, int world, int64_t numel,
                        int group_size, float divisor, void *out, int out_dtype, const void *prepared,
-                       void *new_residual, void *stream) {
+                       void *new_residual, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (world <= 0) return fail(LBC_EINVAL, "inputs must not be empty");
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (!(divisor > 0.0f)) return fail(LBC_EINVAL, "divisor must be > 0");
@@ -264,16 +246,18 @@ int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, i
     a.new_residual = new_residual;
     a.numel = numel;
     a.divisor = divisor;
-    int64_t moved = numel * (world + dtype_size(out_dtype));
-    if (prepared != nullptr) moved += 2 * numel * dtype_size(out_dtype);
-    return finish(lbc::launch_dequant_reduce(out_dtype, group_size, world, pick_mode(aligned, moved), a,
+    // Streaming calls whose output is well beyond the 32 MiB of L2 write it through; smaller outputs stay plain
+    // cached stores, which leave the write-back to overlap with whatever runs next.
+    int mode = pick_mode(aligned, access);
+    if (mode == 2 && numel * dtype_size(out_dtype) >= (int64_t{24} << 20)) mode = 3;
+    return finish(lbc::launch_dequant_reduce(out_dtype, group_size, world, mode, a,
                                              static_cast<hipStream_t>(stream)),
                   "lbc_dequant_reduce");
 }
 
 int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *scales, int world, int64_t numel,
-                             int group_size, float divisor, int mid_dtype, int8_t *out_codes, float *out_scales,
-                             void *stream) {
+                             int group_size, float divisor, int mid_dtype, int8_t *out_codes, float *out_scales, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (world <= 0) return fail(LBC_EINVAL, "inputs must not be empty");
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (!(divisor > 0.0f)) return fail(LBC_EINVAL, "divisor must be > 0");
@@ -298,13 +282,14 @@ int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *sca
     a.out_scales = out_scales;
     a.numel = numel;
     a.divisor = divisor;
-    return finish(lbc::launch_dequant_reduce_quant(mid_dtype, group_size, world, pick_mode(aligned, numel * (world + 1)),
+    return finish(lbc::launch_dequant_reduce_quant(mid_dtype, group_size, world, pick_mode(aligned, access),
                                                    a, static_cast<hipStream_t>(stream)),
                   "lbc_dequant_reduce_quant");
 }
 
 int lbc_ring_step(const int8_t *recv_codes, const float *recv_scales, void *chunk, int dtype, int64_t numel,
-                  int group_size, int reduce_op, float divisor, int8_t *send_codes, float *send_scales, void *stream) {
+                  int group_size, int reduce_op, float divisor, int8_t *send_codes, float *send_scales, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported chunk dtype %d", dtype);
     if (reduce_op < LBC_REDUCE_NONE || reduce_op > LBC_REDUCE_MIN) return fail(LBC_EINVAL, "unknown reduce op %d", reduce_op);
@@ -324,15 +309,15 @@ int lbc_ring_step(const int8_t *recv_codes, const float *recv_scales, void *chun
     const int vec = 16 / dtype_size(dtype);   // elements, and code bytes, one lane owns
     const bool aligned = aligned_to(chunk, 16) && aligned_to(recv_codes, vec) &&
                          (send_codes == nullptr || aligned_to(send_codes, vec));
-    const int64_t moved = numel * ((reduce_op == LBC_REDUCE_SUM ? 2 : 1) * dtype_size(dtype) + (send_codes ? 2 : 1));
     lbc::RingStepArgs a{recv_codes, recv_scales, chunk, send_codes, send_scales, numel, divisor};
-    return finish(lbc::launch_ring_step(dtype, group_size, reduce_op == LBC_REDUCE_SUM, pick_mode(aligned, moved), a,
+    return finish(lbc::launch_ring_step(dtype, group_size, reduce_op == LBC_REDUCE_SUM, pick_mode(aligned, access), a,
                                         static_cast<hipStream_t>(stream)),
                   "lbc_ring_step");
 }
 
 int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored, int restored_dtype,
-                  void *residual, int residual_dtype, int64_t numel, void *stream) {
+                  void *residual, int residual_dtype, int64_t numel, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (!valid_dtype(prepared_dtype) || !valid_dtype(restored_dtype) || !valid_dtype(residual_dtype))
         return fail(LBC_EINVAL, "unsupported dtype");
@@ -344,8 +329,7 @@ int lbc_ef_update(const void *prepared, int prepared_dtype, const void *restored
         return fail(LBC_EINVAL, "a tensor is not aligned to its element size");
     const bool aligned = aligned_to(prepared, 16) && aligned_to(restored, 16) && aligned_to(residual, 16);
     lbc::EfArgs a{prepared, restored, residual, numel};
-    const int64_t moved = numel * (dtype_size(prepared_dtype) + dtype_size(restored_dtype) + dtype_size(residual_dtype));
-    return finish(lbc::launch_ef_update(prepared_dtype, restored_dtype, residual_dtype, pick_mode(aligned, moved), a,
+    return finish(lbc::launch_ef_update(prepared_dtype, restored_dtype, residual_dtype, pick_mode(aligned, access), a,
                                         static_cast<hipStream_t>(stream)),
                   "lbc_ef_update");
 }
@@ -358,8 +342,8 @@ int64_t lbc_wire_payload_nbytes(int64_t numel, int group_size, int dtype, int bi
 }
 
 int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, int64_t numel, int world,
-                               int group_size, int bit, int compact, uint8_t *payloads, int64_t payload_stride,
-                               void *stream) {
+                               int group_size, int bit, int compact, uint8_t *payloads, int64_t payload_stride, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
     if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported dtype %d", dtype);
@@ -383,20 +367,20 @@ int lbc_wire_quant_pack_chunks(const void *x, const void *residual, int dtype, i
     a.payload_stride = world > 1 ? payload_stride : 0;
     a.compact = compact != 0;
     a.nan_resets = residual == nullptr;
-    const int64_t moved = numel * (item * (residual ? 2 : 1) + 1);
-    return finish(lbc::launch_wire_quant(dtype, group_size, bit, pick_mode(true, moved), a, world,
+    return finish(lbc::launch_wire_quant(dtype, group_size, bit, pick_mode(true, access), a, world,
                                          static_cast<hipStream_t>(stream)),
                   "lbc_wire_quant_pack");
 }
 
 int lbc_wire_quant_pack(const void *x, const void *residual, int dtype, int64_t numel, int group_size, int bit,
-                        int compact, uint8_t *payload, void *stream) {
-    return lbc_wire_quant_pack_chunks(x, residual, dtype, numel, 1, group_size, bit, compact, payload, 0, stream);
+                        int compact, uint8_t *payload, int access, void *stream) {
+    return lbc_wire_quant_pack_chunks(x, residual, dtype, numel, 1, group_size, bit, compact, payload, 0, access, stream);
 }
 
 int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world, int64_t shard_numel,
                             int64_t total_numel, int group_size, int bit, int compact, void *out, int dtype,
-                            int reduce_op, void *stream) {
+                            int reduce_op, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (shard_numel < 0 || total_numel < 0) return fail(LBC_EINVAL, "element counts must be >= 0");
     if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
     if (total_numel > shard_numel * world) return fail(LBC_EINVAL, "total_numel exceeds world * shard_numel");
@@ -419,21 +403,21 @@ int lbc_wire_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int
     a.total_numel = total_numel;
     a.payload_stride = world > 1 ? payload_stride : 0;
     a.compact = compact != 0;
-    const int64_t moved = total_numel * (item * (reduce_op == LBC_REDUCE_NONE ? 1 : 2) + 1);
-    return finish(lbc::launch_wire_decode(dtype, group_size, bit, reduce_op, pick_mode(true, moved), a, world,
+    return finish(lbc::launch_wire_decode(dtype, group_size, bit, reduce_op, pick_mode(true, access), a, world,
                                           static_cast<hipStream_t>(stream)),
                   "lbc_wire_dequant");
 }
 
 int lbc_wire_dequant(const uint8_t *payload, int64_t numel, int group_size, int bit, int compact, void *out,
-                     int dtype, int reduce_op, void *stream) {
+                     int dtype, int reduce_op, int access, void *stream) {
     return lbc_wire_dequant_chunks(payload, 0, 1, numel, numel, group_size, bit, compact, out, dtype, reduce_op,
-                                   stream);
+                                   access, stream);
 }
 
 int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t numel, int group_size, int compact,
                             float inv_divisor, int fused_multiply_add, void *out, int dtype, const void *prepared,
-                            void *new_residual, void *stream) {
+                            void *new_residual, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (world <= 0) return fail(LBC_EINVAL, "inputs must not be empty");
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (!(inv_divisor > 0.0f)) return fail(LBC_EINVAL, "inv_divisor must be > 0");
@@ -458,15 +442,14 @@ int lbc_wire_dequant_reduce(const uint8_t *const *payloads, int world, int64_t n
     a.numel = numel;
     a.inv_divisor = inv_divisor;
     a.compact = compact != 0;
-    int64_t moved = numel * (world + item);
-    if (prepared != nullptr) moved += 2 * numel * item;
-    return finish(lbc::launch_wire_reduce(dtype, group_size, world, fused_multiply_add != 0, pick_mode(true, moved), a,
+    return finish(lbc::launch_wire_reduce(dtype, group_size, world, fused_multiply_add != 0, pick_mode(true, access), a,
                                           static_cast<hipStream_t>(stream)),
                   "lbc_wire_dequant_reduce");
 }
 
 int lbc_wire_ring_step(const uint8_t *received, void *chunk, int dtype, int64_t numel, int group_size, int compact,
-                       int reduce_op, float divisor, uint8_t *send, void *stream) {
+                       int reduce_op, float divisor, uint8_t *send, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (!valid_dtype(dtype)) return fail(LBC_EINVAL, "unsupported chunk dtype %d", dtype);
     if (reduce_op < LBC_REDUCE_NONE || reduce_op > LBC_REDUCE_MIN) return fail(LBC_EINVAL, "unknown reduce op %d", reduce_op);
@@ -481,8 +464,7 @@ int lbc_wire_ring_step(const uint8_t *received, void *chunk, int dtype, int64_t 
         return fail(LBC_EINVAL, "chunk and payloads must be aligned to the element size");
     if (send == received) return fail(LBC_EINVAL, "the payload to send must not alias the received one");
     lbc::WireRingStepArgs a{received, chunk, send, numel, divisor == 1.0f ? 1.0f : 1.0f / divisor, compact != 0};
-    const int64_t moved = numel * ((reduce_op == LBC_REDUCE_SUM ? 2 : 1) * item + (send ? 2 : 1));
-    return finish(lbc::launch_wire_ring_step(dtype, group_size, reduce_op == LBC_REDUCE_SUM, pick_mode(true, moved), a,
+    return finish(lbc::launch_wire_ring_step(dtype, group_size, reduce_op == LBC_REDUCE_SUM, pick_mode(true, access), a,
                                              static_cast<hipStream_t>(stream)),
                   "lbc_wire_ring_step");
 }

@@ -16,7 +16,7 @@ import torch
 
 from lowbit_comm_amd.hip.library import load_library
 from lowbit_comm_amd.hip.ops import (MAX_PAYLOADS, REDUCE_OPS, BoundLaunch, _device_tensor, _float_tensor, _ptr,
-                                     _require, num_groups)
+                                     _require, access_code, num_groups)
 
 
 def payload_nbytes(numel: int, dtype: torch.dtype, group_size: int = 64, bit: int = 8) -> int:
@@ -37,7 +37,8 @@ def _payload(t: torch.Tensor, name: str, device: torch.device, nbytes: int) -> N
 
 
 def bind_quant_pack(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64, compact: bool = True,
-                    residual: torch.Tensor | None = None, bit: int = 8) -> BoundLaunch:
+                    residual: torch.Tensor | None = None, bit: int = 8,
+                    access: str | None = None) -> BoundLaunch:
     lib = load_library()
     code = _float_tensor(x, "input")
     _payload(payload, "output", x.device, payload_nbytes(x.numel(), x.dtype, group_size, bit))
@@ -46,25 +47,29 @@ def bind_quant_pack(x: torch.Tensor, payload: torch.Tensor, *, group_size: int =
         _require(residual.dtype == x.dtype, "input and residual must have the same dtype")
         _require(residual.numel() == x.numel(), "input and residual must have the same number of elements")
     args = (_ptr(x), _ptr(residual), code, x.numel(), group_size, int(bit), int(compact), _ptr(payload))
-    return BoundLaunch(lib.lbc_wire_quant_pack, args, x.device, lib, (x, residual, payload))
+    return BoundLaunch(lib.lbc_wire_quant_pack, args + (access_code(access),), x.device, lib, (x, residual, payload))
 
 
 def quant_pack_into(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64, compact: bool = True,
-                    residual: torch.Tensor | None = None, bit: int = 8) -> bool:
+                    residual: torch.Tensor | None = None, bit: int = 8,
+                    access: str | None = None) -> bool:
     """``payload = encode(x [+ residual])``; replaces native ``inplace_quantize_pack`` / ``inplace_quantize``."""
-    return bind_quant_pack(x, payload, group_size=group_size, compact=compact, residual=residual, bit=bit)()
+    return bind_quant_pack(x, payload, group_size=group_size, compact=compact, residual=residual, bit=bit,
+                           access=access)()
 
 
 def quant_pack(x: torch.Tensor, *, group_size: int = 64, compact: bool = True,
-               residual: torch.Tensor | None = None, bit: int = 8) -> torch.Tensor:
+               residual: torch.Tensor | None = None, bit: int = 8, access: str | None = None) -> torch.Tensor:
     payload = torch.empty(payload_nbytes(x.numel(), x.dtype, group_size, bit), dtype=torch.uint8, device=x.device)
-    if not quant_pack_into(x, payload, group_size=group_size, compact=compact, residual=residual, bit=bit):
+    if not quant_pack_into(x, payload, group_size=group_size, compact=compact, residual=residual, bit=bit,
+                           access=access):
         raise RuntimeError(f"no kernel for group_size={group_size}, bit={bit}")
     return payload
 
 
 def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64,
-                           compact: bool = True, residual: torch.Tensor | None = None, bit: int = 8) -> BoundLaunch:
+                           compact: bool = True, residual: torch.Tensor | None = None, bit: int = 8,
+                           access: str | None = None) -> BoundLaunch:
     """``payloads`` is a ``(world, stride)`` uint8 tensor; row d receives chunk d of ``ceil(numel/world)`` elements."""
     lib = load_library()
     code = _float_tensor(x, "input")
@@ -78,11 +83,13 @@ def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, 
                  "input and residual must have the same dtype and number of elements")
     args = (_ptr(x), _ptr(residual), code, x.numel(), world, group_size, int(bit), int(compact), _ptr(payloads),
             payloads.stride(0))
-    return BoundLaunch(lib.lbc_wire_quant_pack_chunks, args, x.device, lib, (x, residual, payloads))
+    return BoundLaunch(lib.lbc_wire_quant_pack_chunks, args + (access_code(access),), x.device, lib,
+                       (x, residual, payloads))
 
 
 def bind_dequant(payload: torch.Tensor, out: torch.Tensor, *, numel: int | None = None, group_size: int = 64,
-                 compact: bool = True, reduce_op: str = "none", bit: int = 8) -> BoundLaunch:
+                 compact: bool = True, reduce_op: str = "none", bit: int = 8,
+                 access: str | None = None) -> BoundLaunch:
     lib = load_library()
     code = _float_tensor(out, "output")
     n = out.numel() if numel is None else int(numel)
@@ -90,18 +97,19 @@ def bind_dequant(payload: torch.Tensor, out: torch.Tensor, *, numel: int | None 
     _require(reduce_op in REDUCE_OPS, f"unsupported reduce op {reduce_op!r}")
     _payload(payload, "input", out.device, payload_nbytes(n, out.dtype, group_size, bit))
     args = (_ptr(payload), n, group_size, int(bit), int(compact), _ptr(out), code, REDUCE_OPS[reduce_op])
-    return BoundLaunch(lib.lbc_wire_dequant, args, out.device, lib, (payload, out))
+    return BoundLaunch(lib.lbc_wire_dequant, args + (access_code(access),), out.device, lib, (payload, out))
 
 
 def dequant_into(payload: torch.Tensor, out: torch.Tensor, *, numel: int | None = None, group_size: int = 64,
-                 compact: bool = True, reduce_op: str = "none", bit: int = 8) -> bool:
+                 compact: bool = True, reduce_op: str = "none", bit: int = 8,
+                 access: str | None = None) -> bool:
     """Decode into ``out`` or combine with it (``sum``/``max``/``min``); replaces native ``inplace_dequantize``."""
     return bind_dequant(payload, out, numel=numel, group_size=group_size, compact=compact, reduce_op=reduce_op,
-                        bit=bit)()
+                        bit=bit, access=access)()
 
 
 def bind_dequant_chunks(payloads: torch.Tensor, out: torch.Tensor, shard_numel: int, *, group_size: int = 64,
-                        compact: bool = True, bit: int = 8) -> BoundLaunch:
+                        compact: bool = True, bit: int = 8, access: str | None = None) -> BoundLaunch:
     lib = load_library()
     code = _float_tensor(out, "output")
     _payload_rows(payloads, out.device)
@@ -110,13 +118,13 @@ def bind_dequant_chunks(payloads: torch.Tensor, out: torch.Tensor, shard_numel: 
     _require(payloads.shape[1] >= payload_nbytes(shard_numel, out.dtype, group_size, bit), "payload rows are too small")
     args = (_ptr(payloads), payloads.stride(0), world, shard_numel, out.numel(), group_size, int(bit), int(compact),
             _ptr(out), code, REDUCE_OPS["none"])
-    return BoundLaunch(lib.lbc_wire_dequant_chunks, args, out.device, lib, (payloads, out))
+    return BoundLaunch(lib.lbc_wire_dequant_chunks, args + (access_code(access),), out.device, lib, (payloads, out))
 
 
 def bind_dequant_reduce(payloads: Sequence[torch.Tensor], out: torch.Tensor, *, numel: int | None = None,
                         group_size: int = 64, compact: bool = True, inv_divisor: float = 1.0,
                         fused_multiply_add: bool = True, prepared: torch.Tensor | None = None,
-                        new_residual: torch.Tensor | None = None) -> BoundLaunch | None:
+                        new_residual: torch.Tensor | None = None, access: str | None = None) -> BoundLaunch | None:
     """``None`` when the request has no kernel (more than 8 payloads, group size other than 64)."""
     lib = load_library()
     _require(len(payloads) > 0, "inputs must not be empty")
@@ -140,7 +148,8 @@ def bind_dequant_reduce(payloads: Sequence[torch.Tensor], out: torch.Tensor, *, 
             _require(t.numel() == n, f"{name} must have numel elements")
     args = (pointers, len(payloads), n, group_size, int(compact), float(inv_divisor), int(fused_multiply_add),
             _ptr(out), code, _ptr(prepared), _ptr(new_residual))
-    return BoundLaunch(lib.lbc_wire_dequant_reduce, args, device, lib, (tuple(payloads), out, prepared, new_residual))
+    return BoundLaunch(lib.lbc_wire_dequant_reduce, args + (access_code(access),), device, lib,
+                       (tuple(payloads), out, prepared, new_residual))
 
 
 def dequant_reduce_into(payloads: Sequence[torch.Tensor], out: torch.Tensor, **kwargs) -> bool:
@@ -160,7 +169,7 @@ _META_WORDS = {0: 1, 1: 3, 2: 4}
 
 def bind_ring_step(received: torch.Tensor, chunk: torch.Tensor, send: torch.Tensor | None = None, *,
                    group_size: int = 64, compact: bool = True, reduce_op: str = "sum",
-                   divisor: float = 1.0) -> BoundLaunch:
+                   divisor: float = 1.0, access: str | None = None) -> BoundLaunch:
     """One ring / tree hop in this format: ``chunk (op)= decode(received)``, ``chunk *= 1/divisor`` (torch's device
     ``div_``), and - with ``send`` - the payload of the updated chunk, in one launch.  ``chunk`` holds whole groups."""
     lib = load_library()
@@ -176,7 +185,8 @@ def bind_ring_step(received: torch.Tensor, chunk: torch.Tensor, send: torch.Tens
         _require(n == 0 or send.data_ptr() != received.data_ptr(), "the payload to send must not alias the received one")
     args = (_ptr(received), _ptr(chunk), code, n, group_size, int(compact), REDUCE_OPS[reduce_op], float(divisor),
             _ptr(send))
-    return BoundLaunch(lib.lbc_wire_ring_step, args, chunk.device, lib, (received, chunk, send))
+    return BoundLaunch(lib.lbc_wire_ring_step, args + (access_code(access),), chunk.device, lib,
+                       (received, chunk, send))
 
 
 def ring_step_into(received: torch.Tensor, chunk: torch.Tensor, send: torch.Tensor | None = None, **kwargs) -> bool:

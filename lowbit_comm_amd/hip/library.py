@@ -11,7 +11,7 @@ from pathlib import Path
 from lowbit_comm_amd.exceptions import CCDLUnavailableError
 
 LIBRARY_PATH = Path(__file__).resolve().parent.parent / "liblbc_hip.so"
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 LBC_OK = 0
 LBC_UNSUPPORTED = 1
@@ -24,30 +24,29 @@ _c_int = ctypes.c_int
 SIGNATURES = {
     "lbc_abi_version": (_c_int, []),
     "lbc_last_error": (ctypes.c_char_p, []),
-    "lbc_set_stream_min_bytes": (_c_i64, [_c_i64]),
     "lbc_quant_pack": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_ptr, _c_ptr,
-                                _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr]),
+                                _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
     "lbc_quant_pack_chunks": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_ptr, _c_i64,
-                                       _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr]),
-    "lbc_dequant": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
-    "lbc_dequant_chunks": (_c_int, [_c_ptr, _c_i64, _c_int, _c_i64, _c_i64, _c_int, _c_ptr, _c_int, _c_ptr]),
+                                       _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
+    "lbc_dequant": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]),
+    "lbc_dequant_chunks": (_c_int, [_c_ptr, _c_i64, _c_int, _c_i64, _c_i64, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
     "lbc_dequant_reduce": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_ptr, _c_int,
-                                    _c_ptr, _c_ptr, _c_ptr]),
+                                    _c_ptr, _c_ptr, _c_int, _c_ptr]),
     "lbc_dequant_reduce_quant": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_int, _c_ptr,
-                                          _c_ptr, _c_ptr]),
+                                          _c_ptr, _c_int, _c_ptr]),
     "lbc_ring_step": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, ctypes.c_float, _c_ptr, _c_ptr,
-                               _c_ptr]),
-    "lbc_ef_update": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_ptr]),
+                               _c_int, _c_ptr]),
+    "lbc_ef_update": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_ptr]),
     "lbc_wire_payload_nbytes": (_c_i64, [_c_i64, _c_int, _c_int, _c_int]),
-    "lbc_wire_quant_pack": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
+    "lbc_wire_quant_pack": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_ptr]),
     "lbc_wire_quant_pack_chunks": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_ptr,
-                                            _c_i64, _c_ptr]),
-    "lbc_wire_ring_step": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, ctypes.c_float, _c_ptr, _c_ptr]),
-    "lbc_wire_dequant": (_c_int, [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
+                                            _c_i64, _c_int, _c_ptr]),
+    "lbc_wire_ring_step": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, ctypes.c_float, _c_ptr, _c_int, _c_ptr]),
+    "lbc_wire_dequant": (_c_int, [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]),
     "lbc_wire_dequant_chunks": (_c_int, [_c_ptr, _c_i64, _c_int, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_ptr,
-                                         _c_int, _c_int, _c_ptr]),
+                                         _c_int, _c_int, _c_int, _c_ptr]),
     "lbc_wire_dequant_reduce": (_c_int, [_c_ptr, _c_int, _c_i64, _c_int, _c_int, ctypes.c_float, _c_int, _c_ptr,
-                                         _c_int, _c_ptr, _c_ptr, _c_ptr]),
+                                         _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr]),
     "lbc_wire_general_payload_nbytes": (_c_i64, [_c_i64, _c_int, _c_int, _c_int, _c_int]),
     "lbc_wire_quant_general": (_c_int, [_c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.c_uint64,
                                         ctypes.c_uint64, _c_int, _c_ptr, _c_ptr]),

@@ -22,6 +22,39 @@ TORCH_DTYPES = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bflo
 REDUCE_OPS = {"none": 0, "sum": 1, "max": 2, "min": 3}
 MAX_PAYLOADS = 8
 _NONE = -1
+ACCESS_MODES = {"auto": 0, "cached": 1, "stream": 2}
+_default_access = "auto"
+
+
+def access_code(access: str | None) -> int:
+    """ABI code of an access mode; ``None`` means the module default (see :func:`access_mode`)."""
+    name = _default_access if access is None else access
+    if name not in ACCESS_MODES:
+        raise RuntimeError(f"access must be one of {sorted(ACCESS_MODES)}; got {access!r}")
+    return ACCESS_MODES[name]
+
+
+class access_mode:
+    """``with access_mode("cached"):`` - launches *bound* inside the block without an explicit ``access=`` use
+    that mode ("auto": the library's rule, "cached": plain cached accesses for operands that are still in cache,
+    "stream": non-temporal loads).  The mode is fixed when a launch is bound; replaying a :class:`BoundLaunch`
+    later does not consult this default again.  Results never depend on the mode."""
+
+    def __init__(self, mode: str) -> None:
+        if mode not in ACCESS_MODES:
+            raise RuntimeError(f"access must be one of {sorted(ACCESS_MODES)}; got {mode!r}")
+        self._mode = mode
+        self._previous = None
+
+    def __enter__(self):
+        global _default_access
+        self._previous, _default_access = _default_access, self._mode
+        return self
+
+    def __exit__(self, *exc):
+        global _default_access
+        _default_access = self._previous
+        return False
 
 
 def num_groups(numel: int, group_size: int) -> int:
@@ -199,15 +232,17 @@ def _side_tensors(x: torch.Tensor, residual, new_residual, restored, restored_dt
 # --------------------------------------------------------------------------- #
 def quant_pack_into(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, *, group_size: int = 64,
                     residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
-                    restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None) -> bool:
+                    restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None,
+                    access: str | None = None) -> bool:
     """``codes, scales <- quant(x + residual)``; optionally ``restored`` and ``new_residual = p - restored``."""
     return bind_quant_pack(x, codes, scales, group_size=group_size, residual=residual, new_residual=new_residual,
-                           restored=restored, restored_dtype=restored_dtype)()
+                           restored=restored, restored_dtype=restored_dtype, access=access)()
 
 
 def bind_quant_pack(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, *, group_size: int = 64,
                     residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
-                    restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None) -> BoundLaunch:
+                    restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None,
+                    access: str | None = None) -> BoundLaunch:
     """Validate once; the returned :class:`BoundLaunch` replays :func:`quant_pack_into` on the same tensors."""
     lib = load_library()
     x_code = _float_tensor(x, "input")
@@ -223,13 +258,14 @@ def bind_quant_pack(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, 
     r_code, n_code, d_code = _side_tensors(x, residual, new_residual, restored, restored_dtype)
     args = (_ptr(x), x_code, _ptr(residual), r_code, n, group_size, _ptr(codes), _ptr(scales),
             _ptr(new_residual), n_code, _ptr(restored), d_code)
-    return BoundLaunch(lib.lbc_quant_pack, args, device, lib, (x, codes, scales, residual, new_residual, restored))
+    return BoundLaunch(lib.lbc_quant_pack, args + (access_code(access),), device, lib,
+                       (x, codes, scales, residual, new_residual, restored))
 
 
 def bind_quant_pack_payload(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64,
                             residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
                             restored: torch.Tensor | None = None,
-                            restored_dtype: torch.dtype | None = None) -> BoundLaunch:
+                            restored_dtype: torch.dtype | None = None, access: str | None = None) -> BoundLaunch:
     """:func:`bind_quant_pack` writing the packed ``uint8[codes || scales]`` wire layout into ``payload``."""
     lib = load_library()
     x_code = _float_tensor(x, "input")
@@ -237,7 +273,8 @@ def bind_quant_pack_payload(x: torch.Tensor, payload: torch.Tensor, *, group_siz
     r_code, n_code, d_code = _side_tensors(x, residual, new_residual, restored, restored_dtype)
     args = (_ptr(x), x_code, _ptr(residual), r_code, x.numel(), group_size, ctypes.c_void_p(codes_at),
             ctypes.c_void_p(scales_at), _ptr(new_residual), n_code, _ptr(restored), d_code)
-    return BoundLaunch(lib.lbc_quant_pack, args, x.device, lib, (x, payload, residual, new_residual, restored))
+    return BoundLaunch(lib.lbc_quant_pack, args + (access_code(access),), x.device, lib,
+                       (x, payload, residual, new_residual, restored))
 
 
 def quant_pack_payload_into(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64, **kwargs) -> bool:
@@ -257,18 +294,20 @@ def quant_pack(x: torch.Tensor, *, group_size: int = 64, residual: torch.Tensor 
 
 def quant_pack_chunks_into(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64,
                            residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
-                           restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None) -> bool:
+                           restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None,
+                           access: str | None = None) -> bool:
     """Quantize the ``world`` destination chunks of ``x`` (+ ``residual``) into the rows of ``payloads``
     (uint8 ``[world, stride]``) in one launch; optional fused error-feedback outputs as in
     :func:`quant_pack_into`."""
     return bind_quant_pack_chunks(x, payloads, world, group_size=group_size, residual=residual,
-                                  new_residual=new_residual, restored=restored, restored_dtype=restored_dtype)()
+                                  new_residual=new_residual, restored=restored, restored_dtype=restored_dtype,
+                                  access=access)()
 
 
 def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64,
                            residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
                            restored: torch.Tensor | None = None,
-                           restored_dtype: torch.dtype | None = None) -> BoundLaunch:
+                           restored_dtype: torch.dtype | None = None, access: str | None = None) -> BoundLaunch:
     lib = load_library()
     x_code = _float_tensor(x, "input")
     device = x.device
@@ -281,20 +320,21 @@ def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, 
     r_code, n_code, d_code = _side_tensors(x, residual, new_residual, restored, restored_dtype)
     args = (_ptr(x), x_code, _ptr(residual), r_code, n, world, group_size, _ptr(payloads), payloads.stride(0),
             _ptr(new_residual), n_code, _ptr(restored), d_code)
-    return BoundLaunch(lib.lbc_quant_pack_chunks, args, device, lib, (x, payloads, residual, new_residual, restored))
+    return BoundLaunch(lib.lbc_quant_pack_chunks, args + (access_code(access),), device, lib,
+                       (x, payloads, residual, new_residual, restored))
 
 
 # --------------------------------------------------------------------------- #
 # decode
 # --------------------------------------------------------------------------- #
 def dequant_into(codes: torch.Tensor, scales: torch.Tensor, out: torch.Tensor, *, numel: int | None = None,
-                 group_size: int = 64, reduce_op: str = "none") -> bool:
+                 group_size: int = 64, reduce_op: str = "none", access: str | None = None) -> bool:
     """``out[:numel] (op)= float(code) * scale``."""
-    return bind_dequant(codes, scales, out, numel=numel, group_size=group_size, reduce_op=reduce_op)()
+    return bind_dequant(codes, scales, out, numel=numel, group_size=group_size, reduce_op=reduce_op, access=access)()
 
 
 def bind_dequant(codes: torch.Tensor, scales: torch.Tensor, out: torch.Tensor, *, numel: int | None = None,
-                 group_size: int = 64, reduce_op: str = "none") -> BoundLaunch:
+                 group_size: int = 64, reduce_op: str = "none", access: str | None = None) -> BoundLaunch:
     lib = load_library()
     o_code = _float_tensor(out, "output")
     device = out.device
@@ -309,11 +349,11 @@ def bind_dequant(codes: torch.Tensor, scales: torch.Tensor, out: torch.Tensor, *
     _require(scales.numel() >= groups, "scales is smaller than the group count")
     _require(reduce_op in REDUCE_OPS, f"unsupported reduce op {reduce_op!r}")
     args = (_ptr(codes), _ptr(scales), n, group_size, _ptr(out), o_code, REDUCE_OPS[reduce_op])
-    return BoundLaunch(lib.lbc_dequant, args, device, lib, (codes, scales, out))
+    return BoundLaunch(lib.lbc_dequant, args + (access_code(access),), device, lib, (codes, scales, out))
 
 
 def dequant_payload_into(payload: torch.Tensor, out: torch.Tensor, *, numel: int | None = None, group_size: int = 64,
-                         reduce_op: str = "none") -> bool:
+                         reduce_op: str = "none", access: str | None = None) -> bool:
     """:func:`dequant_into` reading a packed ``uint8[codes || scales]`` payload that covers ``numel`` elements."""
     lib = load_library()
     o_code = _float_tensor(out, "output")
@@ -323,7 +363,7 @@ def dequant_payload_into(payload: torch.Tensor, out: torch.Tensor, *, numel: int
     codes_at, scales_at = payload_addresses(payload, n, group_size, name="input", device=out.device)
     args = (ctypes.c_void_p(codes_at), ctypes.c_void_p(scales_at), n, group_size, _ptr(out), o_code,
             REDUCE_OPS[reduce_op])
-    return BoundLaunch(lib.lbc_dequant, args, out.device, lib, (payload, out))()
+    return BoundLaunch(lib.lbc_dequant, args + (access_code(access),), out.device, lib, (payload, out))()
 
 
 def dequant(codes: torch.Tensor, scales: torch.Tensor, numel: int, *, group_size: int = 64,
@@ -334,12 +374,14 @@ def dequant(codes: torch.Tensor, scales: torch.Tensor, numel: int, *, group_size
     return out
 
 
-def dequant_chunks_into(payloads: torch.Tensor, out: torch.Tensor, shard_numel: int, *, group_size: int = 64) -> bool:
+def dequant_chunks_into(payloads: torch.Tensor, out: torch.Tensor, shard_numel: int, *, group_size: int = 64,
+                        access: str | None = None) -> bool:
     """Decode row ``d`` of ``payloads`` into ``out[d*shard : (d+1)*shard]`` (clipped to ``out.numel()``)."""
-    return bind_dequant_chunks(payloads, out, shard_numel, group_size=group_size)()
+    return bind_dequant_chunks(payloads, out, shard_numel, group_size=group_size, access=access)()
 
 
-def bind_dequant_chunks(payloads: torch.Tensor, out: torch.Tensor, shard_numel: int, *, group_size: int = 64) -> BoundLaunch:
+def bind_dequant_chunks(payloads: torch.Tensor, out: torch.Tensor, shard_numel: int, *, group_size: int = 64,
+                        access: str | None = None) -> BoundLaunch:
     lib = load_library()
     o_code = _float_tensor(out, "output")
     _device_tensor(payloads, "payloads", out.device)
@@ -348,26 +390,27 @@ def bind_dequant_chunks(payloads: torch.Tensor, out: torch.Tensor, shard_numel: 
     _require(payloads.shape[1] >= payload_nbytes(shard_numel, group_size), "payload rows are too small")
     _require(out.numel() <= world * shard_numel, "output is larger than world * shard_numel")
     args = (_ptr(payloads), payloads.stride(0), world, shard_numel, out.numel(), group_size, _ptr(out), o_code)
-    return BoundLaunch(lib.lbc_dequant_chunks, args, out.device, lib, (payloads, out))
+    return BoundLaunch(lib.lbc_dequant_chunks, args + (access_code(access),), out.device, lib, (payloads, out))
 
 
 def dequant_reduce_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out: torch.Tensor, *,
                         numel: int | None = None, group_size: int = 64, divisor: float = 1.0,
-                        prepared: torch.Tensor | None = None, new_residual: torch.Tensor | None = None) -> bool:
+                        prepared: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
+                        access: str | None = None) -> bool:
     """``out[:numel] = (sum_r decode(payload_r)) / divisor`` in list order; optional ``new_residual = prepared - out``.
 
     ``payloads`` is a sequence of ``(codes, scales)`` pairs or of packed ``uint8[codes || scales]`` tensors covering
     exactly ``numel`` elements.  More than 8 payloads returns ``False``.
     """
     bound = bind_dequant_reduce(payloads, out, numel=numel, group_size=group_size, divisor=divisor,
-                                prepared=prepared, new_residual=new_residual)
+                                prepared=prepared, new_residual=new_residual, access=access)
     return False if bound is None else bound()
 
 
 def bind_dequant_reduce(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out: torch.Tensor, *,
                         numel: int | None = None, group_size: int = 64, divisor: float = 1.0,
                         prepared: torch.Tensor | None = None,
-                        new_residual: torch.Tensor | None = None) -> BoundLaunch | None:
+                        new_residual: torch.Tensor | None = None, access: str | None = None) -> BoundLaunch | None:
     """Bound form of :func:`dequant_reduce_into`; ``None`` when there are more than 8 payloads."""
     lib = load_library()
     _require(len(payloads) > 0, "inputs must not be empty")
@@ -409,12 +452,13 @@ def bind_dequant_reduce(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], o
     args = (code_ptrs, scale_ptrs, world, n, group_size, float(divisor), _ptr(out), o_code,
             _ptr(prepared), _ptr(new_residual))
     keep = (tuple(payloads), out, prepared, new_residual)
-    return BoundLaunch(lib.lbc_dequant_reduce, args, device, lib, keep)
+    return BoundLaunch(lib.lbc_dequant_reduce, args + (access_code(access),), device, lib, keep)
 
 
 def bind_dequant_reduce_quant(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out_codes: torch.Tensor,
                               out_scales: torch.Tensor, numel: int, *, group_size: int = 64, divisor: float = 1.0,
-                              mid_dtype: torch.dtype = torch.float32) -> BoundLaunch | None:
+                              mid_dtype: torch.dtype = torch.float32,
+                              access: str | None = None) -> BoundLaunch | None:
     """Bound form of :func:`dequant_reduce_quant_into`; ``None`` when there are more than 8 payloads."""
     lib = load_library()
     _require(len(payloads) > 0, "inputs must not be empty")
@@ -445,7 +489,8 @@ def bind_dequant_reduce_quant(payloads: Sequence[tuple[torch.Tensor, torch.Tenso
         scale_ptrs[r] = scales.data_ptr()
     args = (code_ptrs, scale_ptrs, world, n, group_size, float(divisor), DTYPE_CODES[mid_dtype], _ptr(out_codes),
             _ptr(out_scales))
-    return BoundLaunch(lib.lbc_dequant_reduce_quant, args, device, lib, (tuple(payloads), out_codes, out_scales))
+    return BoundLaunch(lib.lbc_dequant_reduce_quant, args + (access_code(access),), device, lib,
+                       (tuple(payloads), out_codes, out_scales))
 
 
 def dequant_reduce_quant_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out_codes: torch.Tensor,
@@ -460,7 +505,8 @@ def dequant_reduce_quant_into(payloads: Sequence[tuple[torch.Tensor, torch.Tenso
 # ring step: chunk (op)= decode(received) [/ divisor], then quantize+pack of the updated chunk
 # --------------------------------------------------------------------------- #
 def bind_ring_step(received: torch.Tensor, chunk: torch.Tensor, send: torch.Tensor | None = None, *,
-                   group_size: int = 64, reduce_op: str = "sum", divisor: float = 1.0) -> BoundLaunch:
+                   group_size: int = 64, reduce_op: str = "sum", divisor: float = 1.0,
+                   access: str | None = None) -> BoundLaunch:
     """``received`` and ``send`` are packed ``uint8[codes || scales]`` payloads covering ``chunk.numel()``
     elements; ``chunk`` is updated in place and, when ``send`` is given, quantized into it in the same launch."""
     lib = load_library()
@@ -477,15 +523,18 @@ def bind_ring_step(received: torch.Tensor, chunk: torch.Tensor, send: torch.Tens
     args = (ctypes.c_void_p(recv_codes), ctypes.c_void_p(recv_scales), _ptr(chunk), code, n, group_size,
             REDUCE_OPS[reduce_op], float(divisor),
             None if send is None else ctypes.c_void_p(send_codes), None if send is None else ctypes.c_void_p(send_scales))
-    return BoundLaunch(lib.lbc_ring_step, args, device, lib, (received, chunk, send))
+    return BoundLaunch(lib.lbc_ring_step, args + (access_code(access),), device, lib, (received, chunk, send))
 
 
 def ring_step_into(received: torch.Tensor, chunk: torch.Tensor, send: torch.Tensor | None = None, *,
-                   group_size: int = 64, reduce_op: str = "sum", divisor: float = 1.0) -> bool:
-    return bind_ring_step(received, chunk, send, group_size=group_size, reduce_op=reduce_op, divisor=divisor)()
+                   group_size: int = 64, reduce_op: str = "sum", divisor: float = 1.0,
+                   access: str | None = None) -> bool:
+    return bind_ring_step(received, chunk, send, group_size=group_size, reduce_op=reduce_op, divisor=divisor,
+    access=access)()
 
 
-def ef_update_into(prepared: torch.Tensor, restored: torch.Tensor, residual: torch.Tensor) -> bool:
+def ef_update_into(prepared: torch.Tensor, restored: torch.Tensor, residual: torch.Tensor, *,
+                   access: str | None = None) -> bool:
     """``residual = prepared - restored`` (fp32 subtraction, rounded to the residual's dtype)."""
     lib = load_library()
     p_code = _float_tensor(prepared, "prepared")
@@ -494,4 +543,5 @@ def ef_update_into(prepared: torch.Tensor, restored: torch.Tensor, residual: tor
     _require(prepared.numel() == restored.numel(), "prepared and restored must have the same number of elements")
     _require(prepared.numel() == residual.numel(), "prepared and residual must have the same number of elements")
     args = (_ptr(prepared), p_code, _ptr(restored), t_code, _ptr(residual), r_code, prepared.numel())
-    return BoundLaunch(lib.lbc_ef_update, args, prepared.device, lib, (prepared, restored, residual))()
+    return BoundLaunch(lib.lbc_ef_update, args + (access_code(access),), prepared.device, lib,
+                       (prepared, restored, residual))()

@@ -78,7 +78,7 @@ int main() {
         HIP_OK(hipMalloc(&d_scales[r], groups * sizeof(float)));
         HIP_OK(hipMemcpyAsync(d_x, x[r].data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
         LBC_OK_OR_FAIL(lbc_quant_pack(d_x, LBC_F32, nullptr, LBC_NONE, n, g, d_codes[r], d_scales[r], nullptr, LBC_NONE,
-                                      nullptr, LBC_NONE, stream));
+                                      nullptr, LBC_NONE, LBC_ACCESS_AUTO, stream));
         std::vector<int8_t> codes(padded);
         std::vector<float> scales(groups);
         HIP_OK(hipMemcpyAsync(codes.data(), d_codes[r], padded, hipMemcpyDeviceToHost, stream));
@@ -99,7 +99,7 @@ int main() {
     std::vector<const int8_t *> code_ptrs(d_codes.begin(), d_codes.end());
     std::vector<const float *> scale_ptrs(d_scales.begin(), d_scales.end());
     LBC_OK_OR_FAIL(lbc_dequant_reduce(code_ptrs.data(), scale_ptrs.data(), world, n, g, static_cast<float>(world), d_out,
-                                      LBC_F32, nullptr, nullptr, stream));
+                                      LBC_F32, nullptr, nullptr, LBC_ACCESS_CACHED, stream));
     std::vector<float> got(n), want(n);
     HIP_OK(hipMemcpyAsync(got.data(), d_out, n * sizeof(float), hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
@@ -124,7 +124,7 @@ int main() {
     HIP_OK(hipMalloc(&d_send_codes, padded));
     HIP_OK(hipMalloc(&d_send_scales, groups * sizeof(float)));
     LBC_OK_OR_FAIL(lbc_ring_step(d_codes[1], d_scales[1], d_out, LBC_F32, n, g, LBC_REDUCE_SUM, 1.0f, d_send_codes,
-                                 d_send_scales, stream));
+                                 d_send_scales, LBC_ACCESS_STREAM, stream));
     std::vector<int8_t> send_codes(padded), want_send_codes(padded);
     std::vector<float> send_scales(groups), want_send_scales(groups);
     HIP_OK(hipMemcpyAsync(got.data(), d_out, n * sizeof(float), hipMemcpyDeviceToHost, stream));
@@ -145,12 +145,12 @@ int main() {
 
     // contract: a bad argument is refused with a message, an unsupported group size is "unsupported", not an error
     if (lbc_quant_pack(d_x, LBC_F32, nullptr, LBC_NONE, -1, g, d_codes[0], d_scales[0], nullptr, LBC_NONE, nullptr, LBC_NONE,
-                       stream) != LBC_EINVAL || strstr(lbc_last_error(), "numel") == nullptr) {
+                       LBC_ACCESS_AUTO, stream) != LBC_EINVAL || strstr(lbc_last_error(), "numel") == nullptr) {
         printf("FAIL negative numel was not refused\n");
         return 7;
     }
     if (lbc_quant_pack(d_x, LBC_F32, nullptr, LBC_NONE, n, 48, d_codes[0], d_scales[0], nullptr, LBC_NONE, nullptr, LBC_NONE,
-                       stream) != LBC_UNSUPPORTED) {
+                       LBC_ACCESS_AUTO, stream) != LBC_UNSUPPORTED) {
         printf("FAIL group size 48 should be unsupported\n");
         return 7;
     }

@@ -21,14 +21,12 @@ def hip(hip_device):
     return cuda_wire
 
 
-@pytest.fixture(params=["plain", "stream"])
+@pytest.fixture(params=["cached", "stream"])
 def access(request):
-    from lowbit_comm_amd.hip.library import load_library
+    from lowbit_comm_amd.hip import ops as hip_ops
 
-    lib = load_library()
-    previous = lib.lbc_set_stream_min_bytes(0 if request.param == "stream" else 1 << 62)
-    yield request.param
-    lib.lbc_set_stream_min_bytes(previous)
+    with hip_ops.access_mode(request.param):
+        yield request.param
 
 
 def to_numpy(t: torch.Tensor) -> np.ndarray:

@@ -15,18 +15,14 @@ pytestmark = pytest.mark.gpu
 DTYPES = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
 
 
-@pytest.fixture(scope="module", params=["vector", "stream", "default"])
+@pytest.fixture(scope="module", params=["cached", "stream", "auto"])
 def ops(request, hip_device):
-    """The tensor-level ops with the bulk access mode forced to plain vector, to non-temporal, or left to
-    the size threshold - results must not depend on it."""
+    """The tensor-level ops with every launch bound under one access mode (plain cached accesses, non-temporal
+    loads, or the library's own rule) - results must not depend on it."""
     from lowbit_comm_amd.hip import ops as hip_ops
-    from lowbit_comm_amd.hip.library import load_library
 
-    lib = load_library()
-    wanted = {"vector": 1 << 62, "stream": 0, "default": 96 << 20}[request.param]
-    previous = lib.lbc_set_stream_min_bytes(wanted)
-    yield hip_ops
-    lib.lbc_set_stream_min_bytes(previous)
+    with hip_ops.access_mode(request.param):
+        yield hip_ops
 
 
 def gradient_like(n, dtype, seed, device, sigma=1e-3, outliers=True):

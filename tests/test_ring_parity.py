@@ -11,15 +11,12 @@ pytestmark = pytest.mark.gpu
 DTYPES = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
 
 
-@pytest.fixture(scope="module", params=["vector", "stream"])
+@pytest.fixture(scope="module", params=["cached", "stream"])
 def ops(request, hip_device):
     from lowbit_comm_amd.hip import ops as hip_ops
-    from lowbit_comm_amd.hip.library import load_library
 
-    lib = load_library()
-    previous = lib.lbc_set_stream_min_bytes({"vector": 1 << 62, "stream": 0}[request.param])
-    yield hip_ops
-    lib.lbc_set_stream_min_bytes(previous)
+    with hip_ops.access_mode(request.param):
+        yield hip_ops
 
 
 def to_np(t: torch.Tensor, dtype: str) -> np.ndarray:
