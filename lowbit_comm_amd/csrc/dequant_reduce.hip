@@ -56,7 +56,9 @@ template <int W> __device__ __forceinline__ constexpr int code_load_mode(int mod
 //                                             (3.3 M: 7.9 us against 8.1 written through, 8.4 non-temporal - the
 //                                             write-back then overlaps the next kernel's ramp), written through
 //                                             beyond (26 M: 47.3 us against 50.2 plain, 53.6 non-temporal)
-// The host picks kStream or kStreamThrough by the size of the output.
+// The host picks kStream or kStreamThrough by the size of the output.  The choice holds inside a pipeline as well:
+// a quantize -> shard-reduce step measured 31.7 us with these stores against 32.2-32.5 us with any other pair, and
+// a 613-bucket stream of (error-feedback quantize, shard reduce) 20.69 ms against 20.8-21.2 ms.
 template <typename OT, int W> constexpr int read_write_class() {
     constexpr int reads16 = W * 17, writes16 = static_cast<int>(sizeof(OT)) * 16;   // bytes per element, x16
     return reads16 * 10 < writes16 * 8 ? 0 : (reads16 * 10 < writes16 * 16 ? 1 : 2);

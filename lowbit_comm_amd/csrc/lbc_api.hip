@@ -40,6 +40,13 @@ int pick_mode(bool aligned, int access) {
     return access == LBC_ACCESS_CACHED ? 1 : 2;
 }
 
+// The fused reduce writes through once a streaming call's output is well beyond the 32 MiB of L2; smaller outputs
+// stay in plain cached stores, whose write-back then overlaps with whatever runs next.
+int pick_mode(bool aligned, int access, int64_t written_bytes) {
+    const int mode = pick_mode(aligned, access);
+    return mode == 2 && written_bytes >= (int64_t{24} << 20) ? 3 : mode;
+}
+
 int finish(hipError_t err, const char *what) {
     if (err == hipSuccess) return LBC_OK;
     if (err == hipErrorNotSupported) return LBC_UNSUPPORTED;
@@ -246,11 +253,8 @@ int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, i
     a.new_residual = new_residual;
     a.numel = numel;
     a.divisor = divisor;
-    // Streaming calls whose output is well beyond the 32 MiB of L2 write it through; smaller outputs stay plain
-    // cached stores, which leave the write-back to overlap with whatever runs next.
-    int mode = pick_mode(aligned, access);
-    if (mode == 2 && numel * dtype_size(out_dtype) >= (int64_t{24} << 20)) mode = 3;
-    return finish(lbc::launch_dequant_reduce(out_dtype, group_size, world, mode, a,
+    return finish(lbc::launch_dequant_reduce(out_dtype, group_size, world,
+                                             pick_mode(aligned, access, numel * dtype_size(out_dtype)), a,
                                              static_cast<hipStream_t>(stream)),
                   "lbc_dequant_reduce");
 }

@@ -32,6 +32,11 @@ template <typename A> struct promote<A, void> { using type = A; };
 template <typename T> struct or_float { using type = T; };
 template <> struct or_float<void> { using type = float; };
 
+// Stores of the interior blocks carry the non-temporal hint under the streaming mode, like the loads.  Plain or
+// written-through code stores make this kernel 3-4 % faster when it is timed alone (26 M fp32 elements: 21.3 us
+// written through, 21.4 plain, 21.9 non-temporal), but the lines they leave behind are paid for by the kernel
+// that follows: a quantize -> shard-reduce step measured 32.0 us with non-temporal code stores against 32.6
+// written through and 33.0 plain, and the four-launch reduce-scatter plan 99.1 against 101.8 and 103.3 us.
 template <int VEC> struct quant_tiling {
     static constexpr int TILE = kWave * VEC;        // elements per wavefront step
     static constexpr int UNROLL = LBC_QUANT_UNROLL; // tiles in flight per wavefront
@@ -70,16 +75,22 @@ __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
     if (block_first >= padded) return;
 
     if (MODE != kScalar && block_first + T::BLOCK_ELEMS <= valid) {
-        // ---- interior block: every tile is full, vector loads and stores -----
+        // ---- interior block: every tile is full; one descriptor per stream over the block's span ----
+        constexpr int kLoad = policy_of<MODE>();
+        constexpr int kStore = policy_of<MODE>();
         XT xv[UNROLL][VEC];
         RLoad rv[UNROLL][VEC];
-        int64_t e0[UNROLL];
+        uint32_t at[UNROLL];   // element offset inside the block
+        const buffer_t x_b = buffer_over(x + block_first, T::BLOCK_ELEMS * sizeof(XT));
+        const buffer_t r_b = buffer_over(HAS_R ? r + block_first : nullptr, T::BLOCK_ELEMS * sizeof(RLoad));
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
-            load_wide<XT, VEC, MODE>(x + e0[u], xv[u]);
-            if constexpr (HAS_R) load_wide<RLoad, VEC, MODE>(r + e0[u], rv[u]);
+            at[u] = static_cast<uint32_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
+            buffer_load<XT, VEC, kLoad>(x_b, at[u] * sizeof(XT), xv[u]);
+            if constexpr (HAS_R) buffer_load<RLoad, VEC, kLoad>(r_b, at[u] * sizeof(RLoad), rv[u]);
         }
+        const buffer_t codes_b = buffer_over(codes + block_first, T::BLOCK_ELEMS);
+        const buffer_t scales_b = buffer_over(scales + block_first / G, T::BLOCK_ELEMS / G * 4);
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             float p[VEC];
@@ -96,11 +107,11 @@ __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
             uint32_t words[VEC / 4];
 #pragma unroll
             for (int k = 0; k < VEC / 4; ++k) words[k] = pack4(c[4 * k], c[4 * k + 1], c[4 * k + 2], c[4 * k + 3]);
-            // Codes stream out with the same hint as the tensors.  Leaving them cacheable makes this
-            // kernel look 4-7 % faster in isolation, but the dirty lines are written back under the
-            // next kernel and a quantize -> reduce sequence as a whole measures 2-3 us slower.
-            store_vec<uint32_t, VEC / 4, MODE>(reinterpret_cast<uint32_t *>(codes + e0[u]), words);
-            if ((lane & (LPG - 1)) == 0) scales[e0[u] / G] = scale;
+            buffer_store<uint32_t, VEC / 4, kStore>(codes_b, at[u], words);
+            if ((lane & (LPG - 1)) == 0) {
+                const float one[1] = {scale};
+                buffer_store<float, 1, kCached>(scales_b, at[u] / G * 4, one);
+            }
 
             if (new_r != nullptr || restored != nullptr) {
                 DT rest_out[VEC];
@@ -111,8 +122,10 @@ __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
                     rest_out[i] = narrow<DT>(rest);
                     diff_out[i] = narrow<NT>(p[i] - rest);
                 }
-                if (restored != nullptr) store_wide<DT, VEC, MODE>(restored + e0[u], rest_out);
-                if (new_r != nullptr) store_wide<NT, VEC, MODE>(new_r + e0[u], diff_out);
+                if (restored != nullptr)
+                    buffer_store<DT, VEC, kStore>(buffer_over(restored + block_first, T::BLOCK_ELEMS * sizeof(DT)), at[u] * sizeof(DT), rest_out);
+                if (new_r != nullptr)
+                    buffer_store<NT, VEC, kStore>(buffer_over(new_r + block_first, T::BLOCK_ELEMS * sizeof(NT)), at[u] * sizeof(NT), diff_out);
             }
         }
         return;
