@@ -11,9 +11,18 @@ The line also carries, for the dominant kernel (quantize+pack of the 100 MiB buc
 roofline: algorithmic bytes per launch / average launch duration measured with HIP events around
 back-to-back launches on the launch stream; and a CPU baseline: the torch-op restatement of the
 reference codec timed on this host for the same step.  `kernels` adds the same roofline figures for
-the other kernels of the path (shard reduce, full-bucket all-gather-reduce shape, EF quantize).
+the other kernels of the path (shard reduce, full-bucket all-gather-reduce shape, EF quantize); every
+leg rotates through more than 600 MB of buffers, so none of them is served by the 256 MiB memory-side
+cache.
+
+`roofline.traffic` (HBM bytes per launch of the dominant kernel) is not measured by this run: it comes
+from profiles/hbm_traffic.json, which `--record-traffic` writes from two rocprofv3 counter runs
+(FETCH_SIZE, WRITE_SIZE) of `bench.py --only quant_pack_chunks,copy_calibration`, each counter scaled by
+what it reads for the plain 100 MiB device copy of the same run.  The file remembers a hash of the kernel
+sources it was measured on; when they have changed since, `traffic` is null rather than stale.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py --record-traffic FETCH_SIZE.db WRITE_SIZE.db     (rocprofv3 rocpd databases; no GPU needed)
 """
 from __future__ import annotations
 
@@ -32,8 +41,80 @@ BUCKET_NUMEL = 26_214_400  # 100 MiB of fp32
 WORLD = 8
 GROUP = 64
 SEED = 1234
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), or None
-MEASURED_TRAFFIC = {"quant_pack_chunks": 132_750_000}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+KERNEL_SOURCES = ("quant_pack.hip", "device_utils.h", "launch.h", "lbc_api.hip")   # what the dominant kernel is built from
+SHARD_SETS = 16            # payload sets of the shard-reduce leg: 16 x 41 MB
+
+
+def kernel_sources_hash() -> str:
+    import hashlib
+
+    digest = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "lowbit_comm_amd", "csrc", name), "rb") as handle:
+            digest.update(handle.read())
+    return digest.hexdigest()[:16]
+
+
+def recorded_traffic():
+    """(bytes per launch of the dominant kernel, where it comes from) or (None, why not)."""
+    try:
+        with open(TRAFFIC_FILE) as handle:
+            record = json.load(handle)
+    except (OSError, ValueError):
+        return None, "profiles/hbm_traffic.json is missing"
+    if record.get("kernel_sources_sha256_16") != kernel_sources_hash():
+        return None, "profiles/hbm_traffic.json was measured on other kernel sources; record it again"
+    return record["quant_pack_chunks"]["traffic_bytes"], "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated)"
+
+
+def record_traffic(fetch_db: str, write_db: str) -> int:
+    """Write profiles/hbm_traffic.json from the rocpd databases of the two counter runs."""
+    import sqlite3
+
+    def per_kernel(path, counter):
+        """Median counter value per dispatch (KiB) of every kernel, over its dispatches with the largest grid (the
+        set-up phase launches the same quantize kernel on single chunks)."""
+        cur = sqlite3.connect(path).cursor()
+        tables = [r[0] for r in cur.execute("select name from sqlite_master where type='table'")]
+        pick = lambda part: next(t for t in tables if part in t)
+        rows = cur.execute(
+            f"select s.kernel_name, d.grid_size_x * d.grid_size_y, p.value from {pick('pmc_event')} p "
+            f"join {pick('info_pmc')} i on p.pmc_id = i.id join {pick('kernel_dispatch')} d on p.event_id = d.event_id "
+            f"join {pick('kernel_symbol')} s on d.kernel_id = s.id where i.name = ?", (counter,)).fetchall()
+        largest = {}
+        for name, grid, _ in rows:
+            largest[name] = max(largest.get(name, 0), grid)
+        out = {}
+        for name, grid, value in rows:
+            if grid == largest[name]:
+                out.setdefault(name, []).append(value)
+        return {name: sorted(values)[len(values) // 2] for name, values in out.items()}
+
+    fetch, write = per_kernel(fetch_db, "FETCH_SIZE"), per_kernel(write_db, "WRITE_SIZE")
+    find = lambda table, part: next(v for k, v in table.items() if part in k)
+    copy_kib = BUCKET_NUMEL * 4 / 1024
+    fetch_factor, write_factor = copy_kib / find(fetch, "copyBuffer.kd"), copy_kib / find(write, "copyBuffer.kd")
+    quant = "quant_pack_kernelIfvfLi64ELi4ELi2E"      # mangled <float, void, float, 64, 4, streaming>
+    quant_fetch, quant_write = find(fetch, quant), find(write, quant)
+    traffic = (quant_fetch * fetch_factor + quant_write * write_factor) * 1024
+    record = {
+        "kernel_sources_sha256_16": kernel_sources_hash(), "kernel_sources": list(KERNEL_SOURCES),
+        "commands": ["rocprofv3 --pmc FETCH_SIZE -d <dir> -o f -- python3 bench.py --steps 20 --warmup 2 --only quant_pack_chunks,copy_calibration",
+                     "rocprofv3 --pmc WRITE_SIZE -d <dir> -o w -- python3 bench.py --steps 20 --warmup 2 --only quant_pack_chunks,copy_calibration",
+                     "python3 bench.py --record-traffic <dir>/f_results.db <dir>/w_results.db"],
+        "calibration": {"kernel": "__amd_rocclr_copyBuffer of 100 MiB (102400 KiB read, 102400 KiB written)",
+                        "FETCH_SIZE_factor": fetch_factor, "WRITE_SIZE_factor": write_factor},
+        "quant_pack_chunks": {"kernel": "quant_pack_kernel<float, void, float, 64, 4, 2>, 100 MiB fp32 bucket as 8 chunks",
+                              "FETCH_SIZE_KiB_median": quant_fetch, "WRITE_SIZE_KiB_median": quant_write,
+                              "traffic_bytes": round(traffic),
+                              "algorithmic_bytes": BUCKET_NUMEL * 4 + BUCKET_NUMEL // GROUP * (GROUP + 4)},
+    }
+    with open(TRAFFIC_FILE, "w") as handle:
+        json.dump(record, handle, indent=1)
+        handle.write("\n")
+    print(json.dumps(record["quant_pack_chunks"]))
+    return 0
 
 
 def parse_args():
@@ -44,11 +125,15 @@ def parse_args():
     ap.add_argument("--sets", type=int, default=6, help="distinct buffer sets rotated through (defeats the LLC)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma list of kernel legs to time (for profiling one kernel)")
+    ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_DB", "WRITE_DB"),
+                    help="write profiles/hbm_traffic.json from two rocprofv3 counter databases and exit")
     return ap.parse_args()
 
 
 def main() -> int:
     args = parse_args()
+    if args.record_traffic:
+        return record_traffic(*args.record_traffic)
     if args.gpus != 1:
         print(f"bench.py measures one GPU's share of the path; --gpus {args.gpus} is not supported "
               "(this build has no collectives or multi-GPU sharding)", file=sys.stderr)
@@ -133,7 +218,18 @@ def main() -> int:
 
     quant_bytes = n * 4 + world * payload_bytes
     leg("quant_pack_chunks", lambda i: sets[i % len(sets)]["quant"](), quant_bytes)
-    leg("dequant_reduce_shard", lambda i: sets[i % len(sets)]["reduce"](), world * payload_bytes + shard * 4)
+    if not only or "dequant_reduce_shard" in only:
+        # the shard reduce alone moves 41 MB a launch: it gets payload sets of its own, enough of them (656 MB) that
+        # no launch finds its operands in the memory-side cache
+        shard_sets = []
+        for s in range(SHARD_SETS):
+            rows = sets[s % len(sets)]["received"].clone()
+            out = torch.empty(shard, dtype=torch.float32, device=dev)
+            pairs = [ops.split_payload(rows[r, :payload_bytes], shard, g) for r in range(world)]
+            shard_sets.append(ops.bind_dequant_reduce(pairs, out, group_size=g))
+        leg("dequant_reduce_shard", lambda i: shard_sets[i % SHARD_SETS](), world * payload_bytes + shard * 4)
+        del shard_sets
+        torch.cuda.empty_cache()
 
     if not only or "copy_calibration" in only:
         # a plain device copy of known size (100 MiB read + 100 MiB written): scales the HBM counters, and shows
@@ -236,6 +332,7 @@ def main() -> int:
         }
 
     dominant = kernels.get("quant_pack_chunks")
+    traffic, traffic_source = recorded_traffic()
     line = {
         "metric": "quant-pack & fused dequant-reduce GB/s on 1 MI355X; % of HBM roofline",
         "value": result.get("value"),
@@ -258,7 +355,7 @@ def main() -> int:
         "roofline": None if dominant is None else {
             "bound": "hbm", "kernel": "quant_pack_kernel (100 MiB fp32 bucket, 8 chunks, one launch)",
             "achieved": dominant["achieved_GBps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-            "frac": dominant["frac_of_hbm_peak"], "traffic": MEASURED_TRAFFIC["quant_pack_chunks"],
+            "frac": dominant["frac_of_hbm_peak"], "traffic": traffic, "traffic_source": traffic_source,
             "algorithmic_bytes": dominant["algorithmic_bytes"], "us_per_launch": dominant["us_per_launch"],
         },
         "cpu_baseline": cpu_baseline,
