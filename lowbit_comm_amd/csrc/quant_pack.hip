@@ -32,11 +32,20 @@ template <typename A> struct promote<A, void> { using type = A; };
 template <typename T> struct or_float { using type = T; };
 template <> struct or_float<void> { using type = float; };
 
-// Stores of the interior blocks carry the non-temporal hint under the streaming mode, like the loads.  Plain or
-// written-through code stores make this kernel 3-4 % faster when it is timed alone (26 M fp32 elements: 21.3 us
-// written through, 21.4 plain, 21.9 non-temporal), but the lines they leave behind are paid for by the kernel
-// that follows: a quantize -> shard-reduce step measured 32.0 us with non-temporal code stores against 32.6
-// written through and 33.0 plain, and the four-launch reduce-scatter plan 99.1 against 101.8 and 103.3 us.
+// Stores of the interior blocks under the streaming mode, settled at the level of a pipeline, not of this kernel
+// alone.  Without error feedback the codes are the only output and carry the non-temporal hint like the loads:
+// plain or written-through code stores make the kernel 3-4 % faster when it is timed alone (26 M fp32 elements:
+// 21.3 us written through, 21.4 plain, 21.9 non-temporal), but the lines they leave behind are paid for by the
+// kernel that follows (a quantize -> shard-reduce step: 32.0 us non-temporal, 32.6 written through, 33.0 plain;
+// the four-launch reduce-scatter plan 99.1 / 101.8 / 103.3 us).  With error feedback the residual is the large
+// output and keeps the hint, and the codes are written through: a 613-bucket stream of (error-feedback quantize,
+// shard reduce) measured 20.17 ms that way against 20.74 ms with both non-temporal, 20.75 both written through,
+// 21.57 both plain and 21.97 the other way round; the 52 M-element bucket alone 89.9 against 93.2 us.
+template <bool HAS_RESIDUAL, int MODE> constexpr int quant_code_store_policy() {
+    if (MODE < kStream) return kCached;
+    return HAS_RESIDUAL ? kSc1Bit : kNtBit;
+}
+
 template <int VEC> struct quant_tiling {
     static constexpr int TILE = kWave * VEC;        // elements per wavefront step
     static constexpr int UNROLL = LBC_QUANT_UNROLL; // tiles in flight per wavefront
@@ -77,7 +86,8 @@ __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
     if (MODE != kScalar && block_first + T::BLOCK_ELEMS <= valid) {
         // ---- interior block: every tile is full; one descriptor per stream over the block's span ----
         constexpr int kLoad = policy_of<MODE>();
-        constexpr int kStore = policy_of<MODE>();
+        constexpr int kSideStore = policy_of<MODE>();
+        constexpr int kCodeStore = quant_code_store_policy<HAS_R, MODE>();
         XT xv[UNROLL][VEC];
         RLoad rv[UNROLL][VEC];
         uint32_t at[UNROLL];   // element offset inside the block
@@ -107,7 +117,7 @@ __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
             uint32_t words[VEC / 4];
 #pragma unroll
             for (int k = 0; k < VEC / 4; ++k) words[k] = pack4(c[4 * k], c[4 * k + 1], c[4 * k + 2], c[4 * k + 3]);
-            buffer_store<uint32_t, VEC / 4, kStore>(codes_b, at[u], words);
+            buffer_store<uint32_t, VEC / 4, kCodeStore>(codes_b, at[u], words);
             if ((lane & (LPG - 1)) == 0) {
                 const float one[1] = {scale};
                 buffer_store<float, 1, kCached>(scales_b, at[u] / G * 4, one);
@@ -123,9 +133,9 @@ __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
                     diff_out[i] = narrow<NT>(p[i] - rest);
                 }
                 if (restored != nullptr)
-                    buffer_store<DT, VEC, kStore>(buffer_over(restored + block_first, T::BLOCK_ELEMS * sizeof(DT)), at[u] * sizeof(DT), rest_out);
+                    buffer_store<DT, VEC, kSideStore>(buffer_over(restored + block_first, T::BLOCK_ELEMS * sizeof(DT)), at[u] * sizeof(DT), rest_out);
                 if (new_r != nullptr)
-                    buffer_store<NT, VEC, kStore>(buffer_over(new_r + block_first, T::BLOCK_ELEMS * sizeof(NT)), at[u] * sizeof(NT), diff_out);
+                    buffer_store<NT, VEC, kSideStore>(buffer_over(new_r + block_first, T::BLOCK_ELEMS * sizeof(NT)), at[u] * sizeof(NT), diff_out);
             }
         }
         return;
