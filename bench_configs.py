@@ -55,7 +55,7 @@ def main() -> int:
     import torch
 
     from lowbit_comm_amd import CompressionConfig
-    from lowbit_comm_amd.hip import EventCompletion, ShardWorkspaceProvider, create_torch_workspace_pool, ops
+    from lowbit_comm_amd.hip import ShardWorkspaceProvider, StreamOrderedCompletion, create_torch_workspace_pool, ops
     from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
 
     if not torch.cuda.is_available():
@@ -401,7 +401,7 @@ def main() -> int:
                 if index in check_indices:
                     torch.cuda.synchronize()
                     results[index] += (rows.cpu(), residuals[a:b].cpu(), out[:shard].cpu(), cached[3])
-                session.release(completion=EventCompletion(stream))
+                session.release(completion=StreamOrderedCompletion(stream))
             return results
 
         check = None
@@ -448,6 +448,66 @@ def main() -> int:
              host_enqueue_s=host1 - host0, pool_misses=stats.misses, pool_misses_after_first_pass=misses_after_first,
              pool_hits=stats.hits, steady_state_allocation_bytes=torch.cuda.memory_allocated() - allocated,
              distinct_workspace_keys=2 * 2)
+
+        # the same stream as a pipeline: the quantize of bucket k shares its grid with the reduce of what arrived for
+        # bucket k-1 (one launch per bucket, the last reduce on its own)
+        shared = {}
+
+        def one_pass_shared():
+            previous = None
+            for index, (a, b) in enumerate(bounds):
+                size = b - a
+                shard = -(-size // world)
+                session = provider.begin(stream=stream)
+                rows = send_matrix(session, size, shard)
+                out = session.get_reduced_shard(index, residuals[:0], (shard,), cfg, dtype="fp32", world_size=world, rank=0)
+                cached = bound_cache[index]
+                assert cached[2] == (rows.data_ptr(), out.data_ptr())
+                if previous is None:
+                    cached[0](raw_stream)
+                else:
+                    both = shared.get(index)
+                    if both is None:
+                        both = shared[index] = ops.bind_quant_chunks_and_reduce(cached[0], previous[1])
+                    if not both(raw_stream):
+                        cached[0](raw_stream)
+                        previous[1](raw_stream)
+                previous = cached
+                session.release(completion=StreamOrderedCompletion(stream))
+            previous[1](raw_stream)
+
+        shared_check = None
+        if parity:
+            # both schedules from the same residual state must leave the same residuals and the same last shard
+            start_state = residuals.clone()
+            one_pass()
+            torch.cuda.synchronize()
+            want_residuals = residuals.clone()
+            last_size = bounds[-1][1] - bounds[-1][0]
+            want_last = bound_cache[len(bounds) - 1][1]._keep[1][:-(-last_size // world)].clone()
+            residuals.copy_(start_state)
+            one_pass_shared()
+            torch.cuda.synchronize()
+            got_last = bound_cache[len(bounds) - 1][1]._keep[1][:-(-last_size // world)]
+            same = torch.equal(residuals.view(torch.int32), want_residuals.view(torch.int32)) and \
+                torch.equal(got_last.view(torch.int32), want_last.view(torch.int32))
+            shared_check = "bit-exact against the two-launch schedule (all residuals, last shard)" if same else "MISMATCH"
+            del start_state, want_residuals
+            torch.cuda.empty_cache()
+        one_pass_shared()
+        torch.cuda.synchronize()
+        host0 = time.perf_counter()
+        a_ev.record(stream)
+        one_pass_shared()
+        b_ev.record(stream)
+        host1 = time.perf_counter()
+        torch.cuda.synchronize()
+        seconds = a_ev.elapsed_time(b_ev) * 1e-3
+        emit(5, f"same stream, one launch per bucket: EF quant-pack of bucket k + shard reduce of bucket k-1 in one grid",
+             nbytes, seconds, total * 2, shared_check, buckets=len(bounds), us_per_bucket=seconds / len(bounds) * 1e6,
+             host_enqueue_s=host1 - host0)
+        del grads, residuals
+        torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------------------------------ 6
     if 6 in wanted:

@@ -149,6 +149,27 @@ int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, i
                        const void *prepared, void *new_residual, int access, void *stream);
 
 /*
+ * One launch for two independent pieces of work of a bucket stream: lbc_quant_pack_chunks of one bucket
+ * (arguments x ... new_residual_dtype; `restored` is not offered) and lbc_dequant_reduce of the
+ * `reduce_world` payloads that arrived for another bucket's shard (arguments codes ... reduce_new_residual),
+ * both with `group_size`.  In the reference's reduce-scatter pipeline the exchange of bucket k-1 is in flight
+ * while bucket k is quantized (ccdl_comm/communication/reduce_scatter_transport.py:262-347), so the two are
+ * ready together; a shard-sized reduce is mostly launch ramp, and sharing the quantize's grid hides it
+ * (25 MiB bf16 bucket with fp32 residual + W=8 reduce of its 1.6 M-element shard: 27.5 us against 29.7 us).
+ * Results are bit-identical to the two separate calls in either order.  The reduce must not read what the
+ * quantize writes: nothing orders the two inside the launch.
+ * One side with nothing to do (numel == 0) launches the other alone.  LBC_UNSUPPORTED - issue the two calls
+ * yourself - unless: group_size 64; every operand aligned for the vector kernels and numel/world * element
+ * size a multiple of 16; residual absent (fp32 input only) or fp32; out_dtype fp32 or x_dtype; reduce_world
+ * 2, 4 or 8.  Argument errors are reported as by the two calls.
+ */
+int lbc_quant_pack_chunks_and_dequant_reduce(
+    const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel, int world, int group_size,
+    uint8_t *payloads, int64_t payload_stride, void *new_residual, int new_residual_dtype,
+    const int8_t *const *codes, const float *const *scales, int reduce_world, int64_t reduce_numel, float divisor,
+    void *out, int out_dtype, const void *prepared, void *reduce_new_residual, int access, void *stream);
+
+/*
  * Decode `world` payloads into `world` consecutive shards of one flat tensor in a
  * single launch (the all-gather leg: ccdl_comm/communication/topology_transport.py:
  * 866-894 decodes every gathered shard payload into its slot).  Payload d is

@@ -17,165 +17,20 @@
 // output dtype; "mean" is a true division (divide_all: by the bit-identical
 // product with the reciprocal when the divisor is a power of two).  The translation unit is compiled
 // with -ffp-contract=off so that no product/sum pair is fused into an FMA.
-#include "device_utils.h"
-#include "launch.h"
+#include "dequant_reduce_block.h"
 
 namespace lbc {
 namespace {
+
+using namespace reduce;
 
 // Elements per lane of the fused reduce + requantize: 4 (one dword of codes per payload, 16 lanes per group
 // of 64) measured 3-4 % faster on a full bucket than 8 and the same on shards.
 constexpr int kReduceQuantVec = 4;
 
-#ifndef LBC_DECODE_UNROLL
-#define LBC_DECODE_UNROLL 1
-#endif
-// W payloads give 2*W loads per tile; with one or two payloads a second tile in
-// flight per wavefront is needed to cover the memory latency.
-template <typename OT, int W = 8> struct decode_tiling {
-    static constexpr int VEC = sizeof(OT) == 4 ? 4 : 8;
-    static constexpr int TILE = kWave * VEC;
-    static constexpr int UNROLL = W <= 2 ? 2 * LBC_DECODE_UNROLL : LBC_DECODE_UNROLL;
-    static constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock * UNROLL;
-};
-
-// Cache policy of the code loads in streaming mode, from measurement on 100 MiB buckets: with one to
-// three payloads the output dominates the traffic and cacheable code loads are ~13 % faster; from
-// four payloads on the codes dominate and the non-temporal hint wins by ~9 %.
-template <int W> __device__ __forceinline__ constexpr int code_load_mode(int mode) {
-    return mode == kStream && W < 4 ? kVector : mode;
-}
-// Cache policy of the fused reduce under the streaming modes, from sweeps of every load/store policy pair at
-// W = 1, 2, 4, 8 on 3.3 M, 6.6 M and 26 M fp32 elements with buffers rotating through 650 MB.  The non-temporal
-// hint pays on the direction that carries most of the bytes and costs when both directions carry it:
-//   reads/writes < 0.8  (W = 1, 2 for fp32)  plain code loads, non-temporal stores       (26 M, W = 1: 19.0 us; with
-//                                             non-temporal loads as well 24.8 us)
-//   up to 1.6           (W = 4)               non-temporal loads; stores non-temporal, or written through for
-//                                             outputs beyond the L2s
-//   above               (W = 8)               non-temporal loads; plain stores while the output fits the L2s
-//                                             (3.3 M: 7.9 us against 8.1 written through, 8.4 non-temporal - the
-//                                             write-back then overlaps the next kernel's ramp), written through
-//                                             beyond (26 M: 47.3 us against 50.2 plain, 53.6 non-temporal)
-// The host picks kStream or kStreamThrough by the size of the output.  The choice holds inside a pipeline as well:
-// a quantize -> shard-reduce step measured 31.7 us with these stores against 32.2-32.5 us with any other pair, and
-// a 613-bucket stream of (error-feedback quantize, shard reduce) 20.69 ms against 20.8-21.2 ms.
-template <typename OT, int W> constexpr int read_write_class() {
-    constexpr int reads16 = W * 17, writes16 = static_cast<int>(sizeof(OT)) * 16;   // bytes per element, x16
-    return reads16 * 10 < writes16 * 8 ? 0 : (reads16 * 10 < writes16 * 16 ? 1 : 2);
-}
-template <typename OT, int W, int MODE> constexpr int code_policy() {
-    return MODE >= kStream && read_write_class<OT, W>() >= 1 ? kNtBit : kCached;
-}
-template <typename OT, int W, int MODE> constexpr int reduce_store_policy() {
-    if (MODE < kStream) return kCached;
-    if (read_write_class<OT, W>() == 0) return kNtBit;
-    if (MODE == kStreamThrough) return kSc1Bit;
-    return read_write_class<OT, W>() == 1 ? kNtBit : kCached;
-}
-
-template <int VEC, int MODE>
-__device__ __forceinline__ void load_codes(const int8_t *__restrict__ p, uint32_t (&w)[VEC / 4]) {
-    if constexpr (MODE != kScalar) {
-        load_vec<uint32_t, VEC / 4, MODE>(reinterpret_cast<const uint32_t *>(p), w);
-    } else {
-#pragma unroll
-        for (int k = 0; k < VEC / 4; ++k) {
-            const uint8_t *b = reinterpret_cast<const uint8_t *>(p) + 4 * k;
-            w[k] = static_cast<uint32_t>(b[0]) | (static_cast<uint32_t>(b[1]) << 8) |
-                   (static_cast<uint32_t>(b[2]) << 16) | (static_cast<uint32_t>(b[3]) << 24);
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// fused dequant-reduce
-// ---------------------------------------------------------------------------
 template <typename OT, int G, int W, int MODE>
 __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs a) {
-    using T = decode_tiling<OT, W>;
-    constexpr int VEC = T::VEC;
-    constexpr int UNROLL = T::UNROLL;
-
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x >> 6;
-    // every XCD walks one contiguous eighth of the shard at any size: with the policies above that measured
-    // 6-15 % faster than the round-robin order from 3 M to 26 M elements (W = 8), and no slower at W = 1, 2, 4
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block<true>(T::BLOCK_ELEMS)) * T::BLOCK_ELEMS;
-    OT *__restrict__ out = static_cast<OT *>(a.out);
-    const OT *prepared = static_cast<const OT *>(a.prepared);  // may alias new_r
-    OT *new_r = static_cast<OT *>(a.new_residual);
-    const bool mean = a.divisor != 1.0f;
-
-    if (MODE != kScalar && block_first + T::BLOCK_ELEMS <= a.numel) {
-        // ---- interior block: one descriptor per stream over the block's span, 32-bit offsets per lane ----
-        constexpr int kCodes = code_policy<OT, W, MODE>();
-        constexpr int kLoad = policy_of<MODE>();
-        constexpr int kStore = reduce_store_policy<OT, W, MODE>();
-        uint32_t words[UNROLL][W][VEC / 4];
-        float scale[UNROLL][W];
-        uint32_t at[UNROLL];   // element offset inside the block
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) at[u] = static_cast<uint32_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
-#pragma unroll
-        for (int r = 0; r < W; ++r) {
-            const buffer_t codes = buffer_over(a.codes[r] + block_first, T::BLOCK_ELEMS);
-            const buffer_t scales = buffer_over(a.scales[r] + block_first / G, T::BLOCK_ELEMS / G * 4);
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                buffer_load<uint32_t, VEC / 4, kCodes>(codes, at[u], words[u][r]);
-                float one[1];
-                buffer_load<float, 1, kCached>(scales, at[u] / G * 4, one);
-                scale[u][r] = one[0];
-            }
-        }
-        const buffer_t out_b = buffer_over(out + block_first, T::BLOCK_ELEMS * sizeof(OT));
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            float acc[VEC];
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[i] = round_through<OT>(code_to_float(words[u][0][i / 4], i % 4) * scale[u][0]);
-#pragma unroll
-            for (int r = 1; r < W; ++r) {
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) {
-                    const float t = round_through<OT>(code_to_float(words[u][r][i / 4], i % 4) * scale[u][r]);
-                    acc[i] = round_through<OT>(acc[i] + t);
-                }
-            }
-            if (mean) divide_all<OT, VEC>(acc, a.divisor);
-            OT o[VEC];
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) o[i] = narrow<OT>(acc[i]);
-            buffer_store<OT, VEC, kStore>(out_b, at[u] * sizeof(OT), o);
-            if (new_r != nullptr) {
-                OT pv[VEC], d[VEC];
-                buffer_load<OT, VEC, kLoad>(buffer_over(prepared + block_first, T::BLOCK_ELEMS * sizeof(OT)), at[u] * sizeof(OT), pv);
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) d[i] = narrow<OT>(widen(pv[i]) - acc[i]);
-                buffer_store<OT, VEC, kStore>(buffer_over(new_r + block_first, T::BLOCK_ELEMS * sizeof(OT)), at[u] * sizeof(OT), d);
-            }
-        }
-        return;
-    }
-
-    // ---- edge block: element-wise, stores guarded by numel ----------------------
-    for (int u = 0; u < UNROLL; ++u) {
-        const int64_t e0 = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
-        for (int i = 0; i < VEC; ++i) {
-            const int64_t e = e0 + i;
-            if (e >= a.numel) break;
-            const int64_t g = e / G;
-            float acc = 0.0f;
-#pragma unroll
-            for (int r = 0; r < W; ++r) {
-                const float t = round_through<OT>(static_cast<float>(a.codes[r][e]) * a.scales[r][g]);
-                acc = r == 0 ? t : round_through<OT>(acc + t);
-            }
-            if (mean) acc = round_through<OT>(acc / a.divisor);
-            out[e] = narrow<OT>(acc);
-            if (new_r != nullptr) new_r[e] = narrow<OT>(widen(prepared[e]) - acc);
-        }
-    }
+    dequant_reduce_block<OT, G, W, MODE>(a, blockIdx.x, gridDim.x);
 }
 
 template <typename OT, int G, int W>

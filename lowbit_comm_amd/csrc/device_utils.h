@@ -37,11 +37,15 @@ template <int UNROLL> __device__ __forceinline__ int tile_in_block(int u, int wa
 #define LBC_XCD_SPAN_ELEMS (1 << 22)
 #endif
 template <bool ALWAYS = false>
+__device__ __forceinline__ unsigned xcd_contiguous_block(unsigned block, unsigned grid, int block_elems) {
+    const unsigned per_xcd = grid >> 3;
+    const bool in_span = ALWAYS || static_cast<int64_t>(grid) * block_elems <= LBC_XCD_SPAN_ELEMS;
+    const bool remap = in_span && block < (per_xcd << 3);
+    return remap ? (block & 7u) * per_xcd + (block >> 3) : block;
+}
+template <bool ALWAYS = false>
 __device__ __forceinline__ unsigned xcd_contiguous_block(int block_elems) {
-    const unsigned per_xcd = gridDim.x >> 3;
-    const bool in_span = ALWAYS || static_cast<int64_t>(gridDim.x) * block_elems <= LBC_XCD_SPAN_ELEMS;
-    const bool remap = in_span && blockIdx.x < (per_xcd << 3);
-    return remap ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
+    return xcd_contiguous_block<ALWAYS>(blockIdx.x, gridDim.x, block_elems);
 }
 constexpr uint32_t kEpsBits = 0x34000000u;  // 2^-23, torch.finfo(float32).eps
 

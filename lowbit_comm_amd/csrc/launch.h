@@ -142,6 +142,10 @@ hipError_t launch_quant_pack(int x_dtype, int r_dtype, int d_dtype, bool outputs
 int quant_pack_vec(int x_dtype, int r_dtype, int d_dtype, bool outputs);
 hipError_t launch_dequant_reduce(int out_dtype, int group_size, int world, int mode,
                                  const ReduceArgs &args, hipStream_t stream);
+// Both of the above in one grid (group size 64; restored rounded to fp32; residual none or fp32; output fp32 or the
+// input's type; 2, 4 or 8 payloads; vector or streaming mode).  hipErrorNotSupported for anything else.
+hipError_t launch_bucket_step(int x_dtype, int r_dtype, int out_dtype, int reduce_world, int mode, const QuantArgs &quant,
+                              int quant_world, const ReduceArgs &reduce, hipStream_t stream);
 // Reduce of `world` payloads in `mid_dtype` arithmetic, requantized without leaving the chip.
 hipError_t launch_dequant_reduce_quant(int mid_dtype, int group_size, int world, int mode,
                                        const ReduceQuantArgs &args, hipStream_t stream);

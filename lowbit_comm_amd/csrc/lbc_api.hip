@@ -57,31 +57,51 @@ int finish(hipError_t err, const char *what) {
 
 namespace {
 
+// A validated call, ready to launch.  status != LBC_OK: return it (nothing to launch); `empty`: LBC_OK with no work.
+struct QuantCall {
+    int status = LBC_OK;
+    bool empty = false;
+    lbc::QuantArgs args{};
+    int x_dtype = LBC_F32, r_dtype = LBC_NONE, d_dtype = LBC_F32, world = 1, group_size = 64;
+    bool outputs = false, aligned = false;
+};
+
+struct ReduceCall {
+    int status = LBC_OK;
+    bool empty = false;
+    lbc::ReduceArgs args{};
+    int out_dtype = LBC_F32, world = 0, group_size = 64;
+    bool aligned = false;
+};
+
+QuantCall refuse_quant(int status) { QuantCall c; c.status = status; return c; }
+ReduceCall refuse_reduce(int status) { ReduceCall c; c.status = status; return c; }
+
 // Shared body of lbc_quant_pack (world == 1, separate codes/scales pointers) and
-// lbc_quant_pack_chunks (world >= 1, packed rows).
-int quant_pack_common(const char *what, const void *x, int x_dtype, const void *residual, int residual_dtype,
-                      int64_t numel, int world, int group_size, uint8_t *codes_base, uint8_t *scales_base,
-                      int64_t payload_stride, int64_t shard_numel, void *new_residual, int new_residual_dtype,
-                      void *restored, int restored_dtype, bool rows_aligned, int access, void *stream) {
+// lbc_quant_pack_chunks (world >= 1, packed rows): dtype rules and alignment.
+QuantCall quant_pack_common(const void *x, int x_dtype, const void *residual, int residual_dtype,
+                            int64_t numel, int world, int group_size, uint8_t *codes_base, uint8_t *scales_base,
+                            int64_t payload_stride, int64_t shard_numel, void *new_residual, int new_residual_dtype,
+                            void *restored, int restored_dtype) {
     const int r_dtype = residual ? residual_dtype : LBC_NONE;
     const int p_dtype = residual ? promote(x_dtype, r_dtype) : x_dtype;
     const bool wants_outputs = new_residual != nullptr || restored != nullptr;
     int d_dtype = LBC_F32;
     if (wants_outputs) {
-        if (!valid_dtype(restored_dtype)) return fail(LBC_EINVAL, "unsupported restored dtype %d", restored_dtype);
+        if (!valid_dtype(restored_dtype)) return refuse_quant(fail(LBC_EINVAL, "unsupported restored dtype %d", restored_dtype));
         d_dtype = restored_dtype;
         if (new_residual != nullptr) {
             if (!valid_dtype(new_residual_dtype))
-                return fail(LBC_EINVAL, "unsupported new-residual dtype %d", new_residual_dtype);
+                return refuse_quant(fail(LBC_EINVAL, "unsupported new-residual dtype %d", new_residual_dtype));
             if (new_residual_dtype != promote(p_dtype, d_dtype))
-                return fail(LBC_EINVAL, "new residual must have the promoted dtype of (input+residual) and restored");
+                return refuse_quant(fail(LBC_EINVAL, "new residual must have the promoted dtype of (input+residual) and restored"));
         }
     }
-    if (r_dtype != LBC_NONE && r_dtype != LBC_F32 && r_dtype != x_dtype) return LBC_UNSUPPORTED;
-    if (d_dtype != LBC_F32 && d_dtype != x_dtype) return LBC_UNSUPPORTED;
+    if (r_dtype != LBC_NONE && r_dtype != LBC_F32 && r_dtype != x_dtype) return refuse_quant(LBC_UNSUPPORTED);
+    if (d_dtype != LBC_F32 && d_dtype != x_dtype) return refuse_quant(LBC_UNSUPPORTED);
 
     const int vec = lbc::quant_pack_vec(x_dtype, r_dtype, d_dtype, wants_outputs);
-    bool aligned = rows_aligned && aligned_to(x, 16) && aligned_to(codes_base, vec) && payload_stride % vec == 0;
+    bool aligned = aligned_to(x, 16) && aligned_to(codes_base, vec) && payload_stride % vec == 0;
     auto side = [&](const void *p, int dtype) {
         if (p == nullptr) return;
         aligned = aligned && aligned_to(p, 16) && (world == 1 || (shard_numel * dtype_size(dtype)) % 16 == 0);
@@ -91,19 +111,113 @@ int quant_pack_common(const char *what, const void *x, int x_dtype, const void *
     side(new_residual, new_residual_dtype);
     side(restored, d_dtype);
 
-    lbc::QuantArgs a{};
-    a.x = x;
-    a.residual = residual;
-    a.codes_base = codes_base;
-    a.scales_base = scales_base;
-    a.new_residual = new_residual;
-    a.restored = restored;
-    a.numel = numel;
-    a.shard_numel = shard_numel;
-    a.payload_stride = payload_stride;
-    return finish(lbc::launch_quant_pack(x_dtype, r_dtype, d_dtype, wants_outputs, group_size,
-                                         pick_mode(aligned, access), a, world, static_cast<hipStream_t>(stream)),
+    QuantCall c;
+    c.args.x = x;
+    c.args.residual = residual;
+    c.args.codes_base = codes_base;
+    c.args.scales_base = scales_base;
+    c.args.new_residual = new_residual;
+    c.args.restored = restored;
+    c.args.numel = numel;
+    c.args.shard_numel = shard_numel;
+    c.args.payload_stride = payload_stride;
+    c.x_dtype = x_dtype;
+    c.r_dtype = r_dtype;
+    c.d_dtype = d_dtype;
+    c.world = world;
+    c.group_size = group_size;
+    c.outputs = wants_outputs;
+    c.aligned = aligned;
+    return c;
+}
+
+int launch_quant(const QuantCall &c, const char *what, int access, void *stream) {
+    if (c.status != LBC_OK || c.empty) return c.status;
+    return finish(lbc::launch_quant_pack(c.x_dtype, c.r_dtype, c.d_dtype, c.outputs, c.group_size,
+                                         pick_mode(c.aligned, access), c.args, c.world, static_cast<hipStream_t>(stream)),
                   what);
+}
+
+// Validation of lbc_quant_pack_chunks, shared with the entry point that carries a reduce in the same launch.
+QuantCall prepare_quant_chunks(const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel,
+                               int world, int group_size, uint8_t *payloads, int64_t payload_stride, void *new_residual,
+                               int new_residual_dtype, void *restored, int restored_dtype) {
+    if (numel < 0) return refuse_quant(fail(LBC_EINVAL, "numel must be >= 0"));
+    if (world <= 0) return refuse_quant(fail(LBC_EINVAL, "world must be > 0"));
+    if (!valid_dtype(x_dtype)) return refuse_quant(fail(LBC_EINVAL, "unsupported input dtype %d", x_dtype));
+    if (residual != nullptr && !valid_dtype(residual_dtype))
+        return refuse_quant(fail(LBC_EINVAL, "unsupported residual dtype %d", residual_dtype));
+    if (!valid_group(group_size)) return refuse_quant(LBC_UNSUPPORTED);
+    if (world > 65535) return refuse_quant(LBC_UNSUPPORTED);
+    const int64_t shard = (numel + world - 1) / world;
+    if (shard == 0) {
+        QuantCall c;
+        c.empty = true;
+        return c;
+    }
+    const int64_t groups = (shard + group_size - 1) / group_size;
+    const int64_t payload_bytes = groups * (group_size + 4);
+    if (x == nullptr || payloads == nullptr) return refuse_quant(fail(LBC_EINVAL, "input and payloads must not be null"));
+    if (payload_stride < payload_bytes || (payload_stride & 3) != 0)
+        return refuse_quant(fail(LBC_EINVAL, "payload_stride must be a multiple of 4 and >= %lld", (long long)payload_bytes));
+    if (!aligned_to(payloads, 4)) return refuse_quant(fail(LBC_EINVAL, "payloads must be 4-byte aligned"));
+    if (!aligned_to(x, dtype_size(x_dtype))) return refuse_quant(fail(LBC_EINVAL, "input is not aligned to its element size"));
+    return quant_pack_common(x, x_dtype, residual, residual_dtype, numel, world, group_size, payloads,
+                             payloads + groups * group_size, payload_stride, shard, new_residual, new_residual_dtype,
+                             restored, restored_dtype);
+}
+
+// Validation of lbc_dequant_reduce, shared in the same way.
+ReduceCall prepare_reduce(const int8_t *const *codes, const float *const *scales, int world, int64_t numel,
+                          int group_size, float divisor, void *out, int out_dtype, const void *prepared,
+                          void *new_residual) {
+    if (world <= 0) return refuse_reduce(fail(LBC_EINVAL, "inputs must not be empty"));
+    if (numel < 0) return refuse_reduce(fail(LBC_EINVAL, "numel must be >= 0"));
+    if (!(divisor > 0.0f)) return refuse_reduce(fail(LBC_EINVAL, "divisor must be > 0"));
+    if (!valid_dtype(out_dtype)) return refuse_reduce(fail(LBC_EINVAL, "unsupported output dtype %d", out_dtype));
+    if ((prepared == nullptr) != (new_residual == nullptr))
+        return refuse_reduce(fail(LBC_EINVAL, "prepared and new_residual must be given together"));
+    if (world > LBC_MAX_PAYLOADS || !valid_group(group_size)) return refuse_reduce(LBC_UNSUPPORTED);
+    ReduceCall c;
+    if (numel == 0) {
+        c.empty = true;
+        return c;
+    }
+    if (codes == nullptr || scales == nullptr || out == nullptr)
+        return refuse_reduce(fail(LBC_EINVAL, "codes, scales and out must not be null"));
+    const int vec = out_dtype == LBC_F32 ? 4 : 8;
+    bool aligned = aligned_to(out, 16);
+    if (!aligned_to(out, dtype_size(out_dtype))) return refuse_reduce(fail(LBC_EINVAL, "out is not aligned to its element size"));
+    for (int r = 0; r < world; ++r) {
+        if (codes[r] == nullptr || scales[r] == nullptr) return refuse_reduce(fail(LBC_EINVAL, "payload %d has a null pointer", r));
+        if (!aligned_to(scales[r], 4)) return refuse_reduce(fail(LBC_EINVAL, "scales of payload %d must be 4-byte aligned", r));
+        aligned = aligned && aligned_to(codes[r], vec);
+        c.args.codes[r] = codes[r];
+        c.args.scales[r] = scales[r];
+    }
+    if (prepared != nullptr) {
+        if (!aligned_to(prepared, dtype_size(out_dtype)) || !aligned_to(new_residual, dtype_size(out_dtype)))
+            return refuse_reduce(fail(LBC_EINVAL, "prepared/new_residual are not aligned to their element size"));
+        aligned = aligned && aligned_to(prepared, 16) && aligned_to(new_residual, 16);
+    }
+    c.args.out = out;
+    c.args.prepared = prepared;
+    c.args.new_residual = new_residual;
+    c.args.numel = numel;
+    c.args.divisor = divisor;
+    c.out_dtype = out_dtype;
+    c.world = world;
+    c.group_size = group_size;
+    c.aligned = aligned;
+    return c;
+}
+
+int launch_reduce(const ReduceCall &c, int access, void *stream) {
+    if (c.status != LBC_OK || c.empty) return c.status;
+    return finish(lbc::launch_dequant_reduce(c.out_dtype, c.group_size, c.world,
+                                             pick_mode(c.aligned, access, c.args.numel * dtype_size(c.out_dtype)), c.args,
+                                             static_cast<hipStream_t>(stream)),
+                  "lbc_dequant_reduce");
 }
 
 }  // namespace
@@ -128,34 +242,19 @@ int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residua
     if (codes == nullptr || scales == nullptr) return fail(LBC_EINVAL, "codes and scales must not be null");
     if (!aligned_to(scales, 4)) return fail(LBC_EINVAL, "scales must be 4-byte aligned");
     if (!aligned_to(x, dtype_size(x_dtype))) return fail(LBC_EINVAL, "input is not aligned to its element size");
-    return quant_pack_common("lbc_quant_pack", x, x_dtype, residual, residual_dtype, numel, 1, group_size,
-                             reinterpret_cast<uint8_t *>(codes), reinterpret_cast<uint8_t *>(scales), 0, numel,
-                             new_residual, new_residual_dtype, restored, restored_dtype, true, access, stream);
+    return launch_quant(quant_pack_common(x, x_dtype, residual, residual_dtype, numel, 1, group_size,
+                                          reinterpret_cast<uint8_t *>(codes), reinterpret_cast<uint8_t *>(scales), 0, numel,
+                                          new_residual, new_residual_dtype, restored, restored_dtype),
+                        "lbc_quant_pack", access, stream);
 }
 
 int lbc_quant_pack_chunks(const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel,
                           int world, int group_size, uint8_t *payloads, int64_t payload_stride, void *new_residual,
                           int new_residual_dtype, void *restored, int restored_dtype, int access, void *stream) {
     if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
-    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
-    if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
-    if (!valid_dtype(x_dtype)) return fail(LBC_EINVAL, "unsupported input dtype %d", x_dtype);
-    if (residual != nullptr && !valid_dtype(residual_dtype))
-        return fail(LBC_EINVAL, "unsupported residual dtype %d", residual_dtype);
-    if (!valid_group(group_size)) return LBC_UNSUPPORTED;
-    if (world > 65535) return LBC_UNSUPPORTED;
-    const int64_t shard = (numel + world - 1) / world;
-    if (shard == 0) return LBC_OK;
-    const int64_t groups = (shard + group_size - 1) / group_size;
-    const int64_t payload_bytes = groups * (group_size + 4);
-    if (x == nullptr || payloads == nullptr) return fail(LBC_EINVAL, "input and payloads must not be null");
-    if (payload_stride < payload_bytes || (payload_stride & 3) != 0)
-        return fail(LBC_EINVAL, "payload_stride must be a multiple of 4 and >= %lld", (long long)payload_bytes);
-    if (!aligned_to(payloads, 4)) return fail(LBC_EINVAL, "payloads must be 4-byte aligned");
-    if (!aligned_to(x, dtype_size(x_dtype))) return fail(LBC_EINVAL, "input is not aligned to its element size");
-    return quant_pack_common("lbc_quant_pack_chunks", x, x_dtype, residual, residual_dtype, numel, world, group_size,
-                             payloads, payloads + groups * group_size, payload_stride, shard, new_residual,
-                             new_residual_dtype, restored, restored_dtype, true, access, stream);
+    return launch_quant(prepare_quant_chunks(x, x_dtype, residual, residual_dtype, numel, world, group_size, payloads,
+                                             payload_stride, new_residual, new_residual_dtype, restored, restored_dtype),
+                        "lbc_quant_pack_chunks", access, stream);
 }
 
 int lbc_dequant(const int8_t *codes, const float *scales, int64_t numel, int group_size, void *out,
@@ -222,41 +321,32 @@ int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, i
                        int group_size, float divisor, void *out, int out_dtype, const void *prepared,
                        void *new_residual, int access, void *stream) {
     if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
-    if (world <= 0) return fail(LBC_EINVAL, "inputs must not be empty");
-    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
-    if (!(divisor > 0.0f)) return fail(LBC_EINVAL, "divisor must be > 0");
-    if (!valid_dtype(out_dtype)) return fail(LBC_EINVAL, "unsupported output dtype %d", out_dtype);
-    if ((prepared == nullptr) != (new_residual == nullptr))
-        return fail(LBC_EINVAL, "prepared and new_residual must be given together");
-    if (world > LBC_MAX_PAYLOADS || !valid_group(group_size)) return LBC_UNSUPPORTED;
-    if (numel == 0) return LBC_OK;
-    if (codes == nullptr || scales == nullptr || out == nullptr)
-        return fail(LBC_EINVAL, "codes, scales and out must not be null");
-    const int vec = out_dtype == LBC_F32 ? 4 : 8;
-    bool aligned = aligned_to(out, 16);
-    if (!aligned_to(out, dtype_size(out_dtype))) return fail(LBC_EINVAL, "out is not aligned to its element size");
-    lbc::ReduceArgs a{};
-    for (int r = 0; r < world; ++r) {
-        if (codes[r] == nullptr || scales[r] == nullptr) return fail(LBC_EINVAL, "payload %d has a null pointer", r);
-        if (!aligned_to(scales[r], 4)) return fail(LBC_EINVAL, "scales of payload %d must be 4-byte aligned", r);
-        aligned = aligned && aligned_to(codes[r], vec);
-        a.codes[r] = codes[r];
-        a.scales[r] = scales[r];
-    }
-    if (prepared != nullptr) {
-        if (!aligned_to(prepared, dtype_size(out_dtype)) || !aligned_to(new_residual, dtype_size(out_dtype)))
-            return fail(LBC_EINVAL, "prepared/new_residual are not aligned to their element size");
-        aligned = aligned && aligned_to(prepared, 16) && aligned_to(new_residual, 16);
-    }
-    a.out = out;
-    a.prepared = prepared;
-    a.new_residual = new_residual;
-    a.numel = numel;
-    a.divisor = divisor;
-    return finish(lbc::launch_dequant_reduce(out_dtype, group_size, world,
-                                             pick_mode(aligned, access, numel * dtype_size(out_dtype)), a,
-                                             static_cast<hipStream_t>(stream)),
-                  "lbc_dequant_reduce");
+    return launch_reduce(prepare_reduce(codes, scales, world, numel, group_size, divisor, out, out_dtype, prepared,
+                                        new_residual),
+                         access, stream);
+}
+
+int lbc_quant_pack_chunks_and_dequant_reduce(
+    const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel, int world, int group_size,
+    uint8_t *payloads, int64_t payload_stride, void *new_residual, int new_residual_dtype,
+    const int8_t *const *codes, const float *const *scales, int reduce_world, int64_t reduce_numel, float divisor,
+    void *out, int out_dtype, const void *prepared, void *reduce_new_residual, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
+    const QuantCall q = prepare_quant_chunks(x, x_dtype, residual, residual_dtype, numel, world, group_size, payloads,
+                                             payload_stride, new_residual, new_residual_dtype, nullptr, LBC_F32);
+    if (q.status != LBC_OK) return q.status;
+    const ReduceCall r = prepare_reduce(codes, scales, reduce_world, reduce_numel, group_size, divisor, out, out_dtype,
+                                        prepared, reduce_new_residual);
+    if (r.status != LBC_OK) return r.status;
+    if (q.empty) return launch_reduce(r, access, stream);
+    if (r.empty) return launch_quant(q, "lbc_quant_pack_chunks_and_dequant_reduce", access, stream);
+    // one grid exists for aligned operands, whole 16-byte chunks, group 64, a residual that is absent or fp32 and
+    // 2, 4 or 8 payloads; everything else is for the caller to issue as the two separate calls
+    if (!q.aligned || !r.aligned || group_size != 64 || lbc::quant_pack_vec(q.x_dtype, q.r_dtype, q.d_dtype, q.outputs) != 4)
+        return LBC_UNSUPPORTED;
+    return finish(lbc::launch_bucket_step(q.x_dtype, q.r_dtype, r.out_dtype, r.world, pick_mode(true, access), q.args,
+                                          q.world, r.args, static_cast<hipStream_t>(stream)),
+                  "lbc_quant_pack_chunks_and_dequant_reduce");
 }
 
 int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *scales, int world, int64_t numel,

@@ -14,164 +14,16 @@
 // Semantics follow the reference's portable codec
 // (ccdl_comm/quantization/torch_fallback.py:24-36): fp32 arithmetic, IEEE
 // division for absmax/127 and p/scale, round-half-even, eps clamp on the scale.
-#include "device_utils.h"
-#include "launch.h"
-
-#ifndef LBC_QUANT_UNROLL
-#define LBC_QUANT_UNROLL 4
-#endif
+#include "quant_pack_block.h"
 
 namespace lbc {
 namespace {
 
-// torch type promotion for "a (op) b" restricted to {float, f16, bf16}.
-template <typename A, typename B> struct promote { using type = float; };
-template <typename A> struct promote<A, A> { using type = A; };
-template <typename A> struct promote<A, void> { using type = A; };
+using namespace quant;
 
-template <typename T> struct or_float { using type = T; };
-template <> struct or_float<void> { using type = float; };
-
-// Stores of the interior blocks under the streaming mode, settled at the level of a pipeline, not of this kernel
-// alone.  Without error feedback the codes are the only output and carry the non-temporal hint like the loads:
-// plain or written-through code stores make the kernel 3-4 % faster when it is timed alone (26 M fp32 elements:
-// 21.3 us written through, 21.4 plain, 21.9 non-temporal), but the lines they leave behind are paid for by the
-// kernel that follows (a quantize -> shard-reduce step: 32.0 us non-temporal, 32.6 written through, 33.0 plain;
-// the four-launch reduce-scatter plan 99.1 / 101.8 / 103.3 us).  With error feedback the residual is the large
-// output and keeps the hint, and the codes are written through: a 613-bucket stream of (error-feedback quantize,
-// shard reduce) measured 20.17 ms that way against 20.74 ms with both non-temporal, 20.75 both written through,
-// 21.57 both plain and 21.97 the other way round; the 52 M-element bucket alone 89.9 against 93.2 us.
-template <bool HAS_RESIDUAL, int MODE> constexpr int quant_code_store_policy() {
-    if (MODE < kStream) return kCached;
-    return HAS_RESIDUAL ? kSc1Bit : kNtBit;
-}
-
-template <int VEC> struct quant_tiling {
-    static constexpr int TILE = kWave * VEC;        // elements per wavefront step
-    static constexpr int UNROLL = LBC_QUANT_UNROLL; // tiles in flight per wavefront
-    static constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock * UNROLL;
-};
-
-// XT input, RT residual (void = none), DT type `restored` is rounded to.
 template <typename XT, typename RT, typename DT, int G, int VEC, int MODE>
 __global__ __launch_bounds__(kBlock) void quant_pack_kernel(const QuantArgs a) {
-    using T = quant_tiling<VEC>;
-    using PT = typename promote<XT, RT>::type;  // type of p = x + r
-    using NT = typename promote<PT, DT>::type;  // type of p - restored
-    using RLoad = typename or_float<RT>::type;  // placeholder when there is no residual
-    constexpr bool HAS_R = !is_void_t<RT>::value;
-    constexpr int LPG = G / VEC;                // lanes per group
-    constexpr int UNROLL = T::UNROLL;
-    static_assert(LPG >= 1 && LPG <= 16, "a group must fit one DPP row");
-
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x >> 6;
-    const int64_t chunk = blockIdx.y;
-    const int64_t chunk_start = chunk * a.shard_numel;
-    int64_t valid = a.numel - chunk_start;  // live elements of this chunk
-    valid = valid < 0 ? 0 : (valid > a.shard_numel ? a.shard_numel : valid);
-    const int64_t groups = (a.shard_numel + G - 1) / G;
-    const int64_t padded = groups * G;
-
-    const XT *__restrict__ x = static_cast<const XT *>(a.x) + chunk_start;
-    const RLoad *r = HAS_R ? static_cast<const RLoad *>(a.residual) + chunk_start : nullptr;  // may alias new_r
-    int8_t *__restrict__ codes = reinterpret_cast<int8_t *>(a.codes_base + chunk * a.payload_stride);
-    float *__restrict__ scales = reinterpret_cast<float *>(a.scales_base + chunk * a.payload_stride);
-    NT *new_r = a.new_residual ? static_cast<NT *>(a.new_residual) + chunk_start : nullptr;
-    DT *__restrict__ restored = a.restored ? static_cast<DT *>(a.restored) + chunk_start : nullptr;
-
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(T::BLOCK_ELEMS)) * T::BLOCK_ELEMS;
-    if (block_first >= padded) return;
-
-    if (MODE != kScalar && block_first + T::BLOCK_ELEMS <= valid) {
-        // ---- interior block: every tile is full; one descriptor per stream over the block's span ----
-        constexpr int kLoad = policy_of<MODE>();
-        constexpr int kSideStore = policy_of<MODE>();
-        constexpr int kCodeStore = quant_code_store_policy<HAS_R, MODE>();
-        XT xv[UNROLL][VEC];
-        RLoad rv[UNROLL][VEC];
-        uint32_t at[UNROLL];   // element offset inside the block
-        const buffer_t x_b = buffer_over(x + block_first, T::BLOCK_ELEMS * sizeof(XT));
-        const buffer_t r_b = buffer_over(HAS_R ? r + block_first : nullptr, T::BLOCK_ELEMS * sizeof(RLoad));
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            at[u] = static_cast<uint32_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
-            buffer_load<XT, VEC, kLoad>(x_b, at[u] * sizeof(XT), xv[u]);
-            if constexpr (HAS_R) buffer_load<RLoad, VEC, kLoad>(r_b, at[u] * sizeof(RLoad), rv[u]);
-        }
-        const buffer_t codes_b = buffer_over(codes + block_first, T::BLOCK_ELEMS);
-        const buffer_t scales_b = buffer_over(scales + block_first / G, T::BLOCK_ELEMS / G * 4);
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            float p[VEC];
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                float v = widen(xv[u][i]);
-                if constexpr (HAS_R) v = round_through<PT>(v + widen(rv[u][i]));
-                p[i] = v;
-            }
-            const float scale = group_scale<VEC, LPG>(p);
-            int c[VEC];
-            encode_group<VEC>(p, scale, c);
-
-            uint32_t words[VEC / 4];
-#pragma unroll
-            for (int k = 0; k < VEC / 4; ++k) words[k] = pack4(c[4 * k], c[4 * k + 1], c[4 * k + 2], c[4 * k + 3]);
-            buffer_store<uint32_t, VEC / 4, kCodeStore>(codes_b, at[u], words);
-            if ((lane & (LPG - 1)) == 0) {
-                const float one[1] = {scale};
-                buffer_store<float, 1, kCached>(scales_b, at[u] / G * 4, one);
-            }
-
-            if (new_r != nullptr || restored != nullptr) {
-                DT rest_out[VEC];
-                NT diff_out[VEC];
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) {
-                    const float rest = round_through<DT>(code_value(c[i]) * scale);
-                    rest_out[i] = narrow<DT>(rest);
-                    diff_out[i] = narrow<NT>(p[i] - rest);
-                }
-                if (restored != nullptr)
-                    buffer_store<DT, VEC, kSideStore>(buffer_over(restored + block_first, T::BLOCK_ELEMS * sizeof(DT)), at[u] * sizeof(DT), rest_out);
-                if (new_r != nullptr)
-                    buffer_store<NT, VEC, kSideStore>(buffer_over(new_r + block_first, T::BLOCK_ELEMS * sizeof(NT)), at[u] * sizeof(NT), diff_out);
-            }
-        }
-        return;
-    }
-
-    // ---- edge block: ragged tail and zero padding, element-wise and guarded ----
-    for (int u = 0; u < UNROLL; ++u) {
-        const int64_t e0 = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
-        if (e0 - lane * VEC >= padded) break;  // wavefront-uniform
-        float p[VEC];
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            const int64_t e = e0 + i;
-            float v = 0.0f;
-            if (e < valid) {
-                v = widen(x[e]);
-                if constexpr (HAS_R) v = round_through<PT>(v + widen(r[e]));
-            }
-            p[i] = v;
-        }
-        // Every lane of the row takes part in the DPP butterfly, also lanes past
-        // the padded end (they contribute zeros), so no lane reads a disabled one.
-        const float scale = group_scale<VEC, LPG>(p);
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            const int64_t e = e0 + i;
-            const int c = encode(p[i], scale);
-            if (e < padded) codes[e] = static_cast<int8_t>(c);
-            if (e < valid) {
-                const float rest = round_through<DT>(static_cast<float>(c) * scale);
-                if (restored != nullptr) restored[e] = narrow<DT>(rest);
-                if (new_r != nullptr) new_r[e] = narrow<NT>(p[i] - rest);
-            }
-        }
-        if ((lane & (LPG - 1)) == 0 && e0 < padded) scales[e0 / G] = scale;
-    }
+    quant_pack_block<XT, RT, DT, G, VEC, MODE>(a, blockIdx.x, gridDim.x, blockIdx.y);
 }
 
 template <typename XT, typename RT, typename DT, int G, int VEC>

@@ -24,6 +24,7 @@ from .workspace import (
     HipWorkspacePool,
     ShardWorkspaceProvider,
     ShardWorkspaceSession,
+    StreamOrderedCompletion,
     WorkspaceKey,
     WorkspaceLease,
     WorkspaceStats,
@@ -37,6 +38,6 @@ __all__ = [
     "PipelinedRingExecutor", "PipelinedRingSchedule", "RingAllGatherStep", "RingReduceScatterStep",
     "compile_pipelined_ring_schedule", "make_pipelined_ring_executor", "HipTreeRuntime", "LoopbackMesh", "TreeEdge",
     "TreeExecutor", "TreeSchedule", "compile_tree_schedule", "make_tree_executor",
-    "HipWorkspacePool", "ShardWorkspaceProvider", "ShardWorkspaceSession", "WorkspaceKey", "WorkspaceLease",
-    "WorkspaceStats", "create_torch_workspace_pool", "load_cuda_extension", "load_hip_extension",
+    "HipWorkspacePool", "ShardWorkspaceProvider", "ShardWorkspaceSession", "StreamOrderedCompletion", "WorkspaceKey",
+    "WorkspaceLease", "WorkspaceStats", "create_torch_workspace_pool", "load_cuda_extension", "load_hip_extension",
 ]

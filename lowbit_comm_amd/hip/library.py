@@ -32,6 +32,9 @@ SIGNATURES = {
     "lbc_dequant_chunks": (_c_int, [_c_ptr, _c_i64, _c_int, _c_i64, _c_i64, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
     "lbc_dequant_reduce": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_ptr, _c_int,
                                     _c_ptr, _c_ptr, _c_int, _c_ptr]),
+    "lbc_quant_pack_chunks_and_dequant_reduce": (_c_int, [
+        _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int,
+        _c_ptr, _c_ptr, _c_int, _c_i64, ctypes.c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr]),
     "lbc_dequant_reduce_quant": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_int, _c_ptr,
                                           _c_ptr, _c_int, _c_ptr]),
     "lbc_ring_step": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, ctypes.c_float, _c_ptr, _c_ptr,

@@ -175,14 +175,15 @@ class BoundLaunch:
     the per-bucket fast path: a DDP hook binds once per bucket shape and replays every step.
     """
 
-    __slots__ = ("_fn", "_args", "_device", "_lib", "_keep")
+    __slots__ = ("_fn", "_args", "_device", "_lib", "_keep", "_kind")
 
-    def __init__(self, fn, args: tuple, device: torch.device, lib, keep: tuple) -> None:
+    def __init__(self, fn, args: tuple, device: torch.device, lib, keep: tuple, kind: str | None = None) -> None:
         self._fn = fn
         self._args = args
         self._device = device
         self._lib = lib
         self._keep = keep
+        self._kind = kind      # which entry point the arguments belong to, for launches that can share a grid
 
     def __call__(self, stream: int | None = None) -> bool:
         """Enqueue.  ``stream``: raw ``hipStream_t`` handle (``torch.cuda.Stream.cuda_stream``) of a stream on
@@ -321,7 +322,7 @@ def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, 
     args = (_ptr(x), x_code, _ptr(residual), r_code, n, world, group_size, _ptr(payloads), payloads.stride(0),
             _ptr(new_residual), n_code, _ptr(restored), d_code)
     return BoundLaunch(lib.lbc_quant_pack_chunks, args + (access_code(access),), device, lib,
-                       (x, payloads, residual, new_residual, restored))
+                       (x, payloads, residual, new_residual, restored), kind="quant_pack_chunks")
 
 
 # --------------------------------------------------------------------------- #
@@ -452,7 +453,29 @@ def bind_dequant_reduce(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], o
     args = (code_ptrs, scale_ptrs, world, n, group_size, float(divisor), _ptr(out), o_code,
             _ptr(prepared), _ptr(new_residual))
     keep = (tuple(payloads), out, prepared, new_residual)
-    return BoundLaunch(lib.lbc_dequant_reduce, args + (access_code(access),), device, lib, keep)
+    return BoundLaunch(lib.lbc_dequant_reduce, args + (access_code(access),), device, lib, keep, kind="dequant_reduce")
+
+
+def bind_quant_chunks_and_reduce(quant: BoundLaunch, reduce: BoundLaunch) -> BoundLaunch:
+    """One launch for the chunked quantize of one bucket and the fused reduce of the payloads that arrived for another
+    bucket's shard (``lbc_quant_pack_chunks_and_dequant_reduce``).  ``quant`` comes from :func:`bind_quant_pack_chunks`
+    (without ``restored``), ``reduce`` from :func:`bind_dequant_reduce`; the two must not touch the same memory, and
+    the access mode is the quantize's.  Calling the result returns ``False`` when the combination has no shared grid
+    (then call ``quant`` and ``reduce`` themselves); the results are bit-identical either way."""
+    _require(isinstance(quant, BoundLaunch) and quant._kind == "quant_pack_chunks",
+             "quant must come from bind_quant_pack_chunks")
+    _require(isinstance(reduce, BoundLaunch) and reduce._kind == "dequant_reduce",
+             "reduce must come from bind_dequant_reduce")
+    _require(quant._device == reduce._device, "both launches must be on the same device")
+    (x, x_code, residual, r_code, n, world, group_size, payloads, stride, new_residual, n_code, restored, _d_code,
+     access) = quant._args
+    _require(restored is None, "the shared launch does not write `restored`")
+    code_ptrs, scale_ptrs, r_world, r_n, r_group, divisor, out, o_code, prepared, r_new_residual, _r_access = reduce._args
+    _require(group_size == r_group, "both launches must use the same group size")
+    args = (x, x_code, residual, r_code, n, world, group_size, payloads, stride, new_residual, n_code,
+            code_ptrs, scale_ptrs, r_world, r_n, divisor, out, o_code, prepared, r_new_residual, access)
+    return BoundLaunch(quant._lib.lbc_quant_pack_chunks_and_dequant_reduce, args, quant._device, quant._lib,
+                       (quant._keep, reduce._keep), kind="bucket_step")
 
 
 def bind_dequant_reduce_quant(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out_codes: torch.Tensor,

@@ -121,7 +121,7 @@ def test_config4_reduce_scatter_all_gather_plan_of_a_200_mib_bucket(ops, hip_dev
 
 def test_config5_llama_3_8b_shaped_stream_through_the_workspace_pool(ops, hip_device):
     from lowbit_comm_amd import CompressionConfig
-    from lowbit_comm_amd.hip import EventCompletion, ShardWorkspaceProvider, WorkspaceKey, create_torch_workspace_pool
+    from lowbit_comm_amd.hip import ShardWorkspaceProvider, StreamOrderedCompletion, WorkspaceKey, create_torch_workspace_pool
 
     dev = hip_device
     cfg = CompressionConfig(bit=8, group_size=G)
@@ -193,7 +193,7 @@ def test_config5_llama_3_8b_shaped_stream_through_the_workspace_pool(ops, hip_de
             if index in check:
                 torch.cuda.synchronize()
                 seen[index] += (rows.cpu(), residuals[a:b].cpu(), out[:shard].cpu(), entry[3])
-            session.release(completion=EventCompletion(stream))
+            session.release(completion=StreamOrderedCompletion(stream))
         return seen
 
     first = one_pass(check=(0, 306, 612))
@@ -220,3 +220,47 @@ def test_config5_llama_3_8b_shaped_stream_through_the_workspace_pool(ops, hip_de
     torch.cuda.synchronize()
     assert pool.stats.misses == misses
     assert torch.cuda.memory_allocated() == allocated
+
+    # the same stream as a pipeline, one launch per bucket: the quantize of bucket k shares its grid with the reduce
+    # of what arrived for bucket k-1.  From the same residual state it must leave the same residuals and shards.
+    def shared_pass(keep=()):
+        kept, previous = {}, None
+        for index, (a, b) in enumerate(bounds):
+            session = provider.begin(stream=stream)
+            size = b - a
+            shard = -(-size // world)
+            rows = send_matrix(session, size, shard)
+            out = session.get_reduced_shard(index, residuals[:0], (shard,), cfg, dtype="fp32", world_size=world, rank=0)
+            entry = bound[index]
+            assert entry[2] == (rows.data_ptr(), out.data_ptr())
+            if previous is None:
+                entry[0]()
+            else:
+                assert ops.bind_quant_chunks_and_reduce(entry[0], previous[1][1])() is True
+                if previous[0] in keep:
+                    kept[previous[0]] = previous[3][:previous[2]].clone()
+            previous = (index, entry, shard, out)          # the shard buffer this bucket's reduce is bound to
+            session.release(completion=StreamOrderedCompletion(stream))
+        previous[1][1]()
+        if previous[0] in keep:
+            kept[previous[0]] = previous[3][:previous[2]].clone()
+        return kept
+
+    sample = (0, 306, 611, 612)
+    start_state = residuals.clone()
+    one_pass()
+    want_residuals = residuals.clone()
+    want_shards = {}
+    for index in sample:                                 # the two-launch schedule overwrites the pooled shard: redo these
+        size = bounds[index][1] - bounds[index][0]
+        shard = -(-size // world)
+        piece = torch.empty(shard, device=dev)
+        assert ops.dequant_reduce_into(bound[index][3], piece)
+        want_shards[index] = piece
+    residuals.copy_(start_state)
+    got_shards = shared_pass(keep=sample)
+    torch.cuda.synchronize()
+    assert torch.equal(residuals.view(torch.int32), want_residuals.view(torch.int32))
+    for index in sample:
+        assert torch.equal(got_shards[index].view(torch.int32), want_shards[index].view(torch.int32)), f"shard of bucket {index}"
+    assert pool.stats.misses == misses

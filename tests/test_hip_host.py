@@ -743,6 +743,42 @@ def test_bucket_stream_captured_in_a_hip_graph_replays_like_eager(dev):
         assert float((torch.randn(1 << 16, device=dev) * 2).sum().item()) == pytest.approx(0.0, abs=1e4)   # eager work
 
 
+def test_stream_ordered_completion_records_nothing_while_a_buffer_stays_on_one_stream(dev):
+    from lowbit_comm_amd.hip import StreamOrderedCompletion, WorkspaceKey, create_torch_workspace_pool
+
+    pool = create_torch_workspace_pool()
+    key = WorkspaceKey(backend="hip", collective="reduce_scatter", strategy="compressed", shape_class=(1 << 20,),
+                       dtype="float32", world_size=8, bit=8, group_size=64, chunk_config=(0,), workspace_kind="reduced",
+                       device=str(dev))
+    main, other = torch.cuda.current_stream(), torch.cuda.Stream()
+    completions = []
+    first = None
+    for step in range(5):                              # the same stream again and again: one buffer, no event, no wait
+        lease = pool.acquire(key, main)
+        first = first if first is not None else lease.buffer.data_ptr()
+        assert lease.buffer.data_ptr() == first
+        lease.buffer.fill_(float(step))
+        completions.append(StreamOrderedCompletion(main))
+        lease.release(completion=completions[-1])
+    assert all(c._event is None for c in completions)
+    assert pool.stats.misses == 1 and pool.stats.hits == 4
+    assert completions[-1].covers(main) and not completions[-1].covers(other) and not completions[-1].peek()
+    # another stream takes the buffer over: now the event exists, and the consumer is ordered after the fill
+    with torch.cuda.stream(other):
+        taken = pool.acquire(key, other)
+        assert taken.buffer.data_ptr() == first
+        total = taken.buffer.sum()
+        taken.release(completion=StreamOrderedCompletion(other))
+    assert completions[-1]._event is not None
+    torch.cuda.synchronize()
+    assert float(total) == 4.0 * (1 << 20)
+    # query() answers for the host: it records (once) and becomes true when the stream has drained
+    done = StreamOrderedCompletion(main)
+    assert done.peek() is False
+    done.synchronize()
+    assert done.query() is True and done.peek() is True
+
+
 def test_llama_shaped_bucket_stream_through_the_pool(dev):
     """Config 5 structure at 1/64 scale: bf16 parameter tensors of a Llama-3-8B-shaped layer stack, flattened in
     reverse registration order into fixed-size buckets with a ragged tail; per bucket EF quant-pack and a W=8

@@ -639,3 +639,83 @@ def test_reduce_requantize_contract(ops, hip_device):
     want_codes, want_scales = codec_torch.quantize(reduced, 64)
     assert torch.equal(c2.cpu(), want_codes) and torch.equal(c2[n:].cpu(), torch.zeros(128 - n, dtype=torch.int8))
     assert_same_bits(s2, want_scales, "non-finite tail")
+
+
+# --------------------------------------------------------------------------- #
+# quantize of one bucket and reduce of another bucket's shard in one launch
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("grad_dtype,with_residual,out_dtype", [
+    ("bf16", True, "fp32"), ("bf16", True, "bf16"), ("fp16", True, "fp32"), ("fp32", True, "fp32"), ("fp32", False, "fp32"),
+])
+@pytest.mark.parametrize("world,payloads", [(8, 8), (4, 2), (2, 4)])
+@pytest.mark.parametrize("n,reduce_n", [(64 * 8 * 640, 64 * 640), (64 * 8 * 64 * 3 + 64 * 8, 50_048), (64 * 8 * 30, 4096 * 3)])
+def test_shared_launch_of_quantize_and_reduce_equals_the_two_launches_and_the_oracle(
+        ops, hip_device, grad_dtype, with_residual, out_dtype, world, payloads, n, reduce_n):
+    grad = gradient_like(n, DTYPES[grad_dtype], 3100 + n, hip_device)
+    residual = gradient_like(n, torch.float32, 3101, hip_device, sigma=1e-5, outliers=False) if with_residual else None
+    keep = None if residual is None else residual.clone()
+    shard = -(-n // world)
+    stride = (ops.payload_nbytes(shard) + 255) // 256 * 256
+    rows = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+    peers = [ops.quant_pack(gradient_like(reduce_n, torch.float32, 3200 + r, hip_device)) for r in range(payloads)]
+    out = torch.empty(reduce_n, dtype=DTYPES[out_dtype], device=hip_device)
+    quant = ops.bind_quant_pack_chunks(grad, rows, world, residual=residual, new_residual=residual)
+    reduce = ops.bind_dequant_reduce(peers, out, divisor=float(payloads))
+    both = ops.bind_quant_chunks_and_reduce(quant, reduce)
+    assert both() is True
+    got_rows, got_out = rows.clone(), out.clone()
+    got_residual = None if residual is None else residual.clone()
+    # the two launches on the same inputs
+    rows.zero_(); out.zero_()
+    if residual is not None:
+        residual.copy_(keep)
+    assert quant() and reduce()
+    assert torch.equal(got_rows, rows)
+    assert_same_bits(got_out, out.cpu(), "reduced shard")
+    if residual is not None:
+        assert_same_bits(got_residual, residual.cpu(), "residual")
+    # and the oracle
+    prepared = grad.cpu() if keep is None else grad.cpu() + keep.cpu()
+    nbytes = ops.payload_nbytes(shard)
+    for d in range(world):
+        chunk = prepared[d * shard:(d + 1) * shard]
+        if chunk.numel() < shard:
+            chunk = torch.cat([chunk, torch.zeros(shard - chunk.numel(), dtype=chunk.dtype)])
+        assert torch.equal(got_rows[d, :nbytes].cpu(), codec_torch.pack(*codec_torch.quantize(chunk, 64))), f"chunk {d}"
+    want = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in peers], reduce_n, 64, out_dtype, "mean")
+    assert_same_bits(got_out, want, "reduced shard against the oracle")
+
+
+def test_shared_launch_reports_what_it_has_no_grid_for(ops, hip_device):
+    n, world = 64 * 8 * 64, 8
+    shard = n // world
+    rows = torch.zeros(world, (ops.payload_nbytes(shard) + 255) // 256 * 256, dtype=torch.uint8, device=hip_device)
+    peers8 = [ops.quant_pack(gradient_like(4096, torch.float32, 3300 + r, hip_device)) for r in range(8)]
+    out = torch.empty(4096, device=hip_device)
+    reduce8 = ops.bind_dequant_reduce(peers8, out)
+    reduce3 = ops.bind_dequant_reduce(peers8[:3], out)
+    bf16 = gradient_like(n, torch.bfloat16, 3301, hip_device)
+    fp32 = gradient_like(n, torch.float32, 3302, hip_device)
+    # 16-bit input without a residual, three payloads, another group size: valid requests, no shared grid
+    assert ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(bf16, rows, world), reduce8)() is False
+    assert ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(fp32, rows, world), reduce3)() is False
+    rows32 = torch.zeros(world, (ops.payload_nbytes(shard, 32) + 255) // 256 * 256, dtype=torch.uint8, device=hip_device)
+    peers32 = [ops.quant_pack(gradient_like(4096, torch.float32, 3310 + r, hip_device), group_size=32) for r in range(8)]
+    assert ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(fp32, rows32, world, group_size=32),
+                                            ops.bind_dequant_reduce(peers32, out, group_size=32))() is False
+    # an unaligned view: element-wise kernels only
+    odd = gradient_like(n + 1, torch.float32, 3303, hip_device)[1:]
+    assert ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(odd, rows, world), reduce8)() is False
+    # one side empty: the other runs alone
+    empty = torch.empty(0, dtype=torch.float32, device=hip_device)
+    no_rows = torch.zeros(world, 0, dtype=torch.uint8, device=hip_device)
+    out.zero_()
+    assert ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(empty, no_rows, world), reduce8)() is True
+    want = torch.empty_like(out)
+    assert ops.dequant_reduce_into(peers8, want)
+    assert torch.equal(out.view(torch.int32), want.view(torch.int32))
+    with pytest.raises(RuntimeError, match="bind_quant_pack_chunks"):
+        ops.bind_quant_chunks_and_reduce(reduce8, reduce8)
+    restored = torch.empty(n, device=hip_device)
+    with pytest.raises(RuntimeError, match="restored"):
+        ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(fp32, rows, world, restored=restored), reduce8)
