@@ -43,13 +43,157 @@ SEED = 1234
 G = 64
 
 
+MANIFEST = os.path.join(ROOT, "profiles", "baseline_manifest.json")
+
+
+def gate_rows(quads: int = 3, only=None):
+    """The five hot-path launches a later change is held to, each timed against a plain 100 MiB device copy in
+    A-B-B-A order (copy, kernel, kernel, copy; the reference's gate alternates baseline and candidate the same way,
+    tests/benchmarks/fused_dequant_executor_gate.py:16-33) so that clock and thermal drift cancel in the ratio.
+    Returns ``{name: {"us", "copy_us", "ratio", "algorithmic_bytes", "frac_of_hbm_peak"}}``; ``ratio`` is the smallest
+    kernel/copy ratio over ``quads`` A-B-B-A rounds.  Buffers rotate through more than 600 MB per row.  ``only``: a
+    collection of row names to measure instead of all five."""
+    import torch
+
+    from lowbit_comm_amd.hip import ops
+
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream(dev)
+
+    def gen(seed, numel, sigma, dtype=torch.float32):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        return (torch.randn(numel, generator=g, device=dev) * sigma).to(dtype)
+
+    def batch(launches, repeats):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        for _ in range(repeats):
+            for launch in launches:
+                launch()
+        stop.record(stream)
+        stop.synchronize()
+        return start.elapsed_time(stop) * 1e3 / (repeats * len(launches))          # us per launch
+
+    copy_numel = 26_214_400
+    sources = [gen(900 + i, copy_numel, 1.0) for i in range(4)]
+    sinks = [torch.empty(copy_numel, device=dev) for _ in range(4)]
+    copies = [lambda a=a, b=b: b.copy_(a) for a, b in zip(sources, sinks)]
+
+    def payload_rows(shard, world, seed):
+        rows = torch.empty(world, ops.payload_nbytes(shard, G), dtype=torch.uint8, device=dev)
+        for r in range(world):
+            assert ops.quant_pack_payload_into(gen(seed + r, shard, 1e-3), rows[r])
+        return rows
+
+    def build(name):
+        world = 8
+        if name == "quant_pack_chunks_100MiB_fp32_W8":
+            n, shard = 26_214_400, 3_276_800
+            stride = -(-ops.payload_nbytes(shard, G) // 256) * 256
+            return [ops.bind_quant_pack_chunks(gen(10 + s, n, 1e-3), torch.empty(world, stride, dtype=torch.uint8, device=dev), world)
+                    for s in range(6)], n * 4 + world * ops.payload_nbytes(shard, G)
+        if name == "dequant_reduce_shard_3276800_W8":
+            shard = 3_276_800
+            sets = []
+            for s in range(16):
+                rows = payload_rows(shard, world, 100 + 8 * s) if s < 4 else sets_rows[s % 4].clone()
+                if s < 4:
+                    sets_rows.append(rows)
+                sets.append(ops.bind_dequant_reduce([rows[r] for r in range(world)], torch.empty(shard, device=dev)))
+            return sets, world * ops.payload_nbytes(shard, G) + shard * 4
+        if name == "dequant_reduce_full_26214400_W8":
+            n = 26_214_400
+            sets = []
+            for s in range(2):
+                rows = payload_rows(n, world, 300 + 8 * s)
+                sets.append(ops.bind_dequant_reduce([rows[r] for r in range(world)], torch.empty(n, device=dev)))
+            return sets, world * ops.payload_nbytes(n, G) + n * 4
+        if name == "ef_quant_pack_100MiB_bf16_fp32_residual":
+            n = 52_428_800
+            groups = ops.num_groups(n, G)
+            sets = []
+            for s in range(2):
+                residual = gen(500 + s, n, 1e-5)
+                sets.append(ops.bind_quant_pack(gen(510 + s, n, 1e-3, torch.bfloat16), torch.empty(groups * G, dtype=torch.int8, device=dev),
+                                                torch.empty(groups, device=dev), residual=residual, new_residual=residual))
+            return sets, n * 10 + groups * (G + 4)
+        if name == "bucket_step_25MiB_bf16_ef_plus_shard_reduce_W8":
+            n, shard = 13_107_200, 1_638_400
+            stride = -(-ops.payload_nbytes(shard, G) // 256) * 256
+            sets = []
+            for s in range(5):
+                residual = gen(700 + s, n, 1e-5)
+                quant = ops.bind_quant_pack_chunks(gen(710 + s, n, 1e-3, torch.bfloat16), torch.empty(world, stride, dtype=torch.uint8, device=dev),
+                                                   world, residual=residual, new_residual=residual)
+                rows = payload_rows(shard, world, 720 + 8 * s)
+                reduce = ops.bind_dequant_reduce([rows[r] for r in range(world)], torch.empty(shard, device=dev))
+                both = ops.bind_quant_chunks_and_reduce(quant, reduce)
+                assert both() is True
+                sets.append(both)
+            return sets, n * 10 + 2 * world * ops.payload_nbytes(shard, G) + shard * 4
+        raise KeyError(name)
+
+    names = ["quant_pack_chunks_100MiB_fp32_W8", "dequant_reduce_shard_3276800_W8", "dequant_reduce_full_26214400_W8",
+             "ef_quant_pack_100MiB_bf16_fp32_residual", "bucket_step_25MiB_bf16_ef_plus_shard_reduce_W8"]
+    rows = {}
+    for name in names:
+        if only is not None and name not in only:
+            continue
+        sets_rows = []
+        launches, nbytes = build(name)
+        repeats = max(2, 96 // len(launches))
+        batch(launches, 1)
+        batch(copies, 2)
+        best = None
+        for _ in range(quads):
+            a1 = batch(copies, 6)
+            b1 = batch(launches, repeats)
+            b2 = batch(launches, repeats)
+            a2 = batch(copies, 6)
+            entry = ((b1 + b2) / (a1 + a2), min(b1, b2), (a1 + a2) / 2)
+            best = entry if best is None or entry[0] < best[0] else best
+        rows[name] = {"us": best[1], "copy_us": best[2], "ratio": best[0], "algorithmic_bytes": nbytes,
+                      "frac_of_hbm_peak": nbytes / (best[1] * 1e-6) / HBM_PEAK}
+        del launches, sets_rows
+        torch.cuda.empty_cache()
+    return rows
+
+
+def write_manifest(path: str = MANIFEST) -> int:
+    import subprocess
+
+    rows = gate_rows(quads=5)
+    try:
+        commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
+    except OSError:
+        commit = ""
+    record = {
+        "what": "frozen performance baseline of the hot-path launches on one MI355X: microseconds per launch and the ratio "
+                "to a plain 100 MiB device copy timed in A-B-B-A order in the same run (gate_rows in bench_configs.py)",
+        "written_by": "python3 bench_configs.py --write-manifest", "commit": commit or None,
+        "copy": "torch copy_ of 26,214,400 fp32 elements (104,857,600 bytes read, as many written), four rotating pairs",
+        "regression_budget": 0.05, "rows": rows,
+    }
+    with open(path, "w") as handle:
+        json.dump(record, handle, indent=1)
+        handle.write("\n")
+    for name, row in rows.items():
+        print(f"{name:52s} {row['us']:8.2f} us  {row['frac_of_hbm_peak'] * 100:5.1f} % of 8 TB/s  ratio to copy {row['ratio']:.4f}",
+              file=sys.stderr)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--configs", default="1,2,3,4,5,6,7,8")
     ap.add_argument("--no-parity", action="store_true", help="skip the CPU oracle comparisons")
     ap.add_argument("--llama-layers", type=int, default=32, help="config 5: number of transformer layers (32 = full model)")
     ap.add_argument("--iters", type=int, default=50)
+    ap.add_argument("--write-manifest", nargs="?", const=MANIFEST, default=None, metavar="PATH",
+                    help="measure the gate rows and freeze them (default: profiles/baseline_manifest.json), then exit")
     args = ap.parse_args()
+    if args.write_manifest:
+        return write_manifest(args.write_manifest)
     wanted = {int(c) for c in args.configs.split(",") if c}
 
     import torch
