@@ -233,8 +233,10 @@ __device__ __forceinline__ void buffer_store(buffer_t b, uint32_t at, const T (&
 // order equals float order and a NaN pattern exceeds +Inf, so a NaN anywhere in
 // the group wins the reduction - the behaviour of torch.amax.
 template <int CTRL> __device__ __forceinline__ uint32_t dpp_max_step(uint32_t v) {
-    uint32_t other = static_cast<uint32_t>(
-        __builtin_amdgcn_update_dpp(static_cast<int>(v), static_cast<int>(v), CTRL, 0xF, 0xF, false));
+    // old value 0 with bound_ctrl set: 0 is the identity of an unsigned maximum, which lets the compiler fold the
+    // lane permutation into the maximum itself (one v_max_u32 with a DPP operand per step instead of a copy, a
+    // permuting move, two wait states and the maximum).  Every lane has a valid source under these permutations.
+    uint32_t other = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xF, 0xF, true));
     return other > v ? other : v;
 }
 
@@ -262,16 +264,27 @@ __device__ __forceinline__ float scale_from_absmax(float absmax) {
     return s < as_f32(kEpsBits) ? as_f32(kEpsBits) : s;
 }
 
-// Scale of the group that the VEC values of LPG adjacent lanes form; every lane gets it.
+// Bit pattern of the largest magnitude in the group that the VEC values of LPG adjacent lanes form; every lane gets it.
 template <int VEC, int LPG>
-__device__ __forceinline__ float group_scale(const float (&p)[VEC]) {
+__device__ __forceinline__ uint32_t group_absmax_bits(const float (&p)[VEC]) {
     uint32_t m = 0;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
         const uint32_t a = as_u32(p[i]) & 0x7FFFFFFFu;
         m = a > m ? a : m;
     }
-    return scale_from_absmax(as_f32(group_max_bits<LPG>(m)));
+    return group_max_bits<LPG>(m);
+}
+
+// Scale of that group.
+template <int VEC, int LPG>
+__device__ __forceinline__ float group_scale(const float (&p)[VEC]) {
+    return scale_from_absmax(as_f32(group_absmax_bits<VEC, LPG>(p)));
+}
+
+// Value of lane K of the caller's quad (four adjacent lanes), in every lane of the quad.
+template <int K> __device__ __forceinline__ float quad_broadcast(float v) {
+    return as_f32(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(as_u32(v)), K * 0x55, 0xF, 0xF, true)));
 }
 
 __device__ __forceinline__ int cvt_i32(float v) {  // NaN -> 0, saturating
@@ -320,23 +333,22 @@ constexpr float kCodeMagic = 12582912.0f;   // 1.5 * 2^23
 
 __device__ __forceinline__ float code_value(int code_bits) { return as_f32(static_cast<uint32_t>(code_bits)) - kCodeMagic; }
 
+// `y` is the correctly rounded reciprocal of `scale` (an IEEE division 1/scale).
 template <int N>
-__device__ __forceinline__ void encode_group(const float (&p)[N], float scale, int (&codes)[N]) {
-    const float y = 1.0f / scale;
-    float t[N];
+__device__ __forceinline__ void encode_group(const float (&p)[N], float scale, float y, int (&codes)[N]) {
+    const bool no_codes = (as_u32(scale) & 0x7F800000u) == 0x7F800000u;   // Inf or NaN scale: one compare per lane
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         const float q0 = p[i] * y;
         const float r = __builtin_fmaf(-q0, scale, p[i]);
-        t[i] = __builtin_fmaf(r, y, q0) + kCodeMagic;
+        const float t = __builtin_fmaf(r, y, q0) + kCodeMagic;
+        codes[i] = static_cast<int>(as_u32(no_codes ? kCodeMagic : t));
     }
-    const bool no_codes = (as_u32(scale) & 0x7F800000u) == 0x7F800000u;   // Inf or NaN scale
-    if (__ballot(no_codes) != 0) {   // wavefront-uniform, practically never taken
-#pragma unroll
-        for (int i = 0; i < N; ++i) t[i] = no_codes ? kCodeMagic : t[i];
-    }
-#pragma unroll
-    for (int i = 0; i < N; ++i) codes[i] = static_cast<int>(as_u32(t[i]));
+}
+
+template <int N>
+__device__ __forceinline__ void encode_group(const float (&p)[N], float scale, int (&codes)[N]) {
+    encode_group<N>(p, scale, 1.0f / scale, codes);
 }
 
 // Single-element form for the ragged edge.

@@ -91,36 +91,67 @@ __device__ __forceinline__ void quant_pack_block(const QuantArgs &a, unsigned bl
         }
         const buffer_t codes_b = buffer_over(codes + block_first, T::BLOCK_ELEMS);
         const buffer_t scales_b = buffer_over(scales + block_first / G, T::BLOCK_ELEMS / G * 4);
+        float p[UNROLL][VEC];
+        uint32_t absmax[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            float p[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
                 float v = widen(xv[u][i]);
                 if constexpr (HAS_R) v = round_through<PT>(v + widen(rv[u][i]));
-                p[i] = v;
+                p[u][i] = v;
             }
-            const float scale = group_scale<VEC, LPG>(p);
+            absmax[u] = group_absmax_bits<VEC, LPG>(p[u]);
+        }
+        // The scale of a group and its reciprocal cost ~18 instructions, and after the butterflies every lane of a
+        // group holds the maxima of all four tiles.  With four tiles and at least four lanes per group the lanes of
+        // a quad split the work: lane j of the quad takes tile j, and quad broadcasts hand the four results round.
+        // Same operations on the same values as one computation per tile; 43 instructions fewer per wavefront.
+        constexpr bool kSplit = UNROLL == 4 && LPG >= 4;
+        float scale[UNROLL], recip[UNROLL];
+        if constexpr (kSplit) {
+            const int j = lane & 3;
+            const uint32_t low = (j & 1) ? absmax[1] : absmax[0], high = (j & 1) ? absmax[3] : absmax[2];
+            const float mine = scale_from_absmax(as_f32((j & 2) ? high : low));
+            const float mine_recip = 1.0f / mine;
+            scale[0] = quad_broadcast<0>(mine); recip[0] = quad_broadcast<0>(mine_recip);
+            scale[1] = quad_broadcast<1>(mine); recip[1] = quad_broadcast<1>(mine_recip);
+            scale[2] = quad_broadcast<2>(mine); recip[2] = quad_broadcast<2>(mine_recip);
+            scale[3] = quad_broadcast<3>(mine); recip[3] = quad_broadcast<3>(mine_recip);
+            if ((lane & (LPG - 1)) < 4) {     // the first quad of every group writes the four scales in one store
+                const uint32_t mine_at = static_cast<uint32_t>(tile_in_block<UNROLL>(j, wave)) * T::TILE + lane * VEC;
+                const float one[1] = {mine};
+                buffer_store<float, 1, kCached>(scales_b, mine_at / G * 4, one);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                scale[u] = scale_from_absmax(as_f32(absmax[u]));
+                recip[u] = 1.0f / scale[u];
+                if ((lane & (LPG - 1)) == 0) {
+                    const float one[1] = {scale[u]};
+                    buffer_store<float, 1, kCached>(scales_b, at[u] / G * 4, one);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
             int c[VEC];
-            encode_group<VEC>(p, scale, c);
+            encode_group<VEC>(p[u], scale[u], recip[u], c);
 
             uint32_t words[VEC / 4];
 #pragma unroll
             for (int k = 0; k < VEC / 4; ++k) words[k] = pack4(c[4 * k], c[4 * k + 1], c[4 * k + 2], c[4 * k + 3]);
             buffer_store<uint32_t, VEC / 4, kCodeStore>(codes_b, at[u], words);
-            if ((lane & (LPG - 1)) == 0) {
-                const float one[1] = {scale};
-                buffer_store<float, 1, kCached>(scales_b, at[u] / G * 4, one);
-            }
 
             if (new_r != nullptr || restored != nullptr) {
                 DT rest_out[VEC];
                 NT diff_out[VEC];
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
-                    const float rest = round_through<DT>(code_value(c[i]) * scale);
+                    const float rest = round_through<DT>(code_value(c[i]) * scale[u]);
                     rest_out[i] = narrow<DT>(rest);
-                    diff_out[i] = narrow<NT>(p[i] - rest);
+                    diff_out[i] = narrow<NT>(p[u][i] - rest);
                 }
                 if (restored != nullptr)
                     buffer_store<DT, VEC, kSideStore>(buffer_over(restored + block_first, T::BLOCK_ELEMS * sizeof(DT)), at[u] * sizeof(DT), rest_out);

@@ -1,10 +1,17 @@
-// What a trivial streaming kernel reaches on this part: read-only, write-only, copy and a 16-bytes-in / 4-bytes-out
-// kernel (the traffic shape of an fp32 quantize) over rotating buffers, one workgroup per tile or a grid-stride loop,
-// with and without the non-temporal hint.  The codec kernels are judged against these figures as well as against
-// the 8 TB/s on the data sheet.  Usage: stream_probe [MiB per buffer, default 100].  Not part of the product.
+// What a trivial streaming kernel reaches on this part: read-only, write-only, copy, a 16-bytes-in / 4-bytes-out
+// kernel (the traffic shape of an fp32 quantize) and an 8 x 4-bytes-in (+ 8 scales) / 16-bytes-out kernel (the
+// traffic shape of the W=8 fused reduce) over rotating buffers, one workgroup per tile or a grid-stride loop, with
+// and without the non-temporal hint.  They do no arithmetic worth the name: the codec kernels are judged against
+// these figures as well as against the 8 TB/s on the data sheet, and tests/test_zx_streaming_ceiling.py holds the hot
+// kernels to 0.9 of the row with their traffic mix.
+// Usage: stream_probe [MiB per buffer, default 100]           the table
+//        stream_probe rows <elements of a W=8 reduce> <elements of an fp32 quantize>
+//                                                             two machine-readable rows: "ROW name microseconds bytes"
+// Not part of the product.
 #include <hip/hip_runtime.h>
 #include <cstdio>
 #include <cstdlib>
+#include <string>
 #include <vector>
 #define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("HIP error %s at %d\n", hipGetErrorString(e), __LINE__); exit(1);} } while (0)
 typedef float float4v __attribute__((ext_vector_type(4)));
@@ -80,6 +87,41 @@ __global__ __launch_bounds__(256) void quantlike_kernel(const float4v* __restric
     for (int u = 0; u < UNROLL; ++u) { size_t i = base + (size_t)u * 256; if (i < n4) out[i] = __builtin_bit_cast(unsigned, v[u].x + v[u].y + v[u].z + v[u].w); }
 }
 
+// 4:1 read:write with the hint on both directions
+template <int UNROLL>
+__global__ __launch_bounds__(256) void quantlike_nt_kernel(const float4v* __restrict__ in, unsigned* __restrict__ out, size_t n4) {
+    size_t base = (size_t)blockIdx.x * 256 * UNROLL + threadIdx.x;
+    float4v v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) { size_t i = base + (size_t)u * 256; if (i < n4) v[u] = __builtin_nontemporal_load(in + i); }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        size_t i = base + (size_t)u * 256;
+        if (i < n4) __builtin_nontemporal_store(__builtin_bit_cast(unsigned, v[u].x + v[u].y + v[u].z + v[u].w), out + i);
+    }
+}
+
+// The W=8 fused reduce's traffic: per lane eight dwords of codes (non-temporal), eight scales shared by 16 lanes, one
+// 16-byte store (STORE: cache policy operand, 0 plain, 16 written through); every XCD walks a contiguous eighth.
+typedef unsigned uint4v __attribute__((ext_vector_type(4)));
+struct ReduceLike { const unsigned* codes[8]; const float* scales[8]; float* out; unsigned n4; };
+template <int STORE>
+__global__ __launch_bounds__(256) void reducelike_kernel(const ReduceLike a) {
+    const unsigned per = gridDim.x >> 3;
+    const unsigned b = blockIdx.x < (per << 3) ? (blockIdx.x & 7u) * per + (blockIdx.x >> 3) : blockIdx.x;
+    const unsigned i = b * 256 + threadIdx.x;
+    if (i >= a.n4) return;
+    unsigned m = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const __amdgpu_buffer_rsrc_t codes = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned*>(a.codes[r]), 0, a.n4 * 4, 0x00020000);
+        const __amdgpu_buffer_rsrc_t scales = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.scales[r]), 0, a.n4 / 4, 0x00020000);
+        m |= __builtin_amdgcn_raw_buffer_load_b32(codes, i * 4, 0, 2) ^ __builtin_amdgcn_raw_buffer_load_b32(scales, (i >> 4) * 4, 0, 0);
+    }
+    const uint4v v = {m, m + 1, m + 2, m + 3};
+    __builtin_amdgcn_raw_buffer_store_b128(v, __builtin_amdgcn_make_buffer_rsrc(a.out, 0, a.n4 * 16, 0x00020000), i * 16, 0, STORE);
+}
+
 struct Timer {
     hipEvent_t a, b;
     Timer() { CK(hipEventCreate(&a)); CK(hipEventCreate(&b)); }
@@ -98,7 +140,42 @@ double run(F launch, int iters, int nbuf) {
     return ms * 1e-3 / iters;
 }
 
+// "rows" mode: the two traffic mixes the hot kernels are held to, at the caller's sizes, over > 600 MB of buffers
+static int rows_mode(size_t reduce_elems, size_t quant_elems) {
+    {
+        const size_t n4 = reduce_elems / 4, groups = reduce_elems / 64;
+        const size_t per_set = 8 * (reduce_elems + groups * 4) + reduce_elems * 4;
+        const int sets = (int)((size_t)640000000 / per_set) + 1;
+        std::vector<ReduceLike> args(sets);
+        for (auto& a : args) {
+            for (int r = 0; r < 8; ++r) {
+                unsigned* c; float* s;
+                CK(hipMalloc(&c, reduce_elems)); CK(hipMalloc(&s, groups * 4)); CK(hipMemset(c, 1, reduce_elems)); CK(hipMemset(s, 1, groups * 4));
+                a.codes[r] = c; a.scales[r] = s;
+            }
+            CK(hipMalloc(&a.out, reduce_elems * 4)); a.n4 = (unsigned)n4;
+        }
+        const unsigned grid = (unsigned)((n4 + 255) / 256);
+        const bool large = reduce_elems * 4 >= ((size_t)24 << 20);
+        double t = run([&](int b) { if (large) reducelike_kernel<16><<<grid, 256>>>(args[b]); else reducelike_kernel<0><<<grid, 256>>>(args[b]); },
+                       10 * sets, sets);
+        printf("ROW reduce_like_w8 %.3f %zu\n", t * 1e6, per_set);
+        for (auto& a : args) { for (int r = 0; r < 8; ++r) { CK(hipFree((void*)a.codes[r])); CK(hipFree((void*)a.scales[r])); } CK(hipFree(a.out)); }
+    }
+    {
+        const size_t n4 = quant_elems / 4, per_set = quant_elems * 4 + quant_elems;
+        const int sets = (int)((size_t)640000000 / per_set) + 1;
+        std::vector<float4v*> in(sets); std::vector<unsigned*> out(sets);
+        for (int i = 0; i < sets; ++i) { CK(hipMalloc(&in[i], quant_elems * 4)); CK(hipMalloc(&out[i], quant_elems)); CK(hipMemset(in[i], 1, quant_elems * 4)); }
+        const unsigned grid = (unsigned)((n4 + 1023) / 1024);
+        double t = run([&](int b) { quantlike_nt_kernel<4><<<grid, 256>>>(in[b], out[b], n4); }, 10 * sets, sets);
+        printf("ROW quant_like_fp32 %.3f %zu\n", t * 1e6, per_set);
+    }
+    return 0;
+}
+
 int main(int argc, char** argv) {
+    if (argc > 3 && std::string(argv[1]) == "rows") return rows_mode((size_t)atoll(argv[2]), (size_t)atoll(argv[3]));
     size_t bytes = (argc > 1 ? atol(argv[1]) : 100) * (size_t)1048576;
     int nbuf = 6;
     std::vector<float4v*> in(nbuf), out(nbuf);
@@ -128,6 +205,7 @@ int main(int argc, char** argv) {
     { double t = run([&](int b){ copy_kernel<8,true><<<GRID(8),256>>>(in[b], out[b], n4); }, iters, nbuf); REPORT("copy  U=8 nontemporal", 2*bytes, t); }
     { double t = run([&](int b){ quantlike_kernel<4><<<GRID(4),256>>>(in[b], (unsigned*)out[b], n4); }, iters, nbuf); REPORT("quant-like 16B in / 4B out U=4", bytes + bytes/4, t); }
     { double t = run([&](int b){ quantlike_kernel<8><<<GRID(8),256>>>(in[b], (unsigned*)out[b], n4); }, iters, nbuf); REPORT("quant-like 16B in / 4B out U=8", bytes + bytes/4, t); }
+    { double t = run([&](int b){ quantlike_nt_kernel<4><<<GRID(4),256>>>(in[b], (unsigned*)out[b], n4); }, iters, nbuf); REPORT("quant-like 16B in / 4B out U=4 nontemporal", bytes + bytes/4, t); }
     { double t = run([&](int b){ CK(hipMemcpyAsync(out[b], in[b], bytes, hipMemcpyDeviceToDevice, 0)); }, iters, nbuf); REPORT("hipMemcpyAsync D2D", 2*bytes, t); }
     return 0;
 }
