@@ -373,6 +373,13 @@ class PipelinedRingExecutor(TopologyExecutor):
 
     def _enqueue(self, submission: _Submission) -> None:
         runtime, tensor, context, workspace = self._runtime, submission.tensor, submission.context, submission.workspace
+        replay = getattr(runtime, "replay_program", None)
+        if callable(replay):
+            handles = replay(context)
+            if handles is not None:          # this tensor's launches and exchanges were recorded by an earlier run
+                for handle in handles:
+                    submission.after_p2p(handle)
+                return
         for step in self.schedule.steps:
             received, handle = self._exchange(submission, step)
             submission.after(runtime.fused_reduce(tensor, received, step.recv_chunk, step.received_contributors,
@@ -381,6 +388,9 @@ class PipelinedRingExecutor(TopologyExecutor):
             received, handle = self._exchange(submission, step)
             submission.after(runtime.apply_broadcast(tensor, received, step.recv_chunk, workspace,
                                                      context=context, dependency=handle))
+        finish = getattr(runtime, "finish_program", None)
+        if callable(finish):
+            finish(context)
 
     def _exchange(self, submission: _Submission, step: Any) -> tuple[Any, Any]:
         runtime, context, workspace = self._runtime, submission.context, submission.workspace
@@ -410,6 +420,7 @@ class RingSubmissionContext:
     staged: tuple | None = None        # ((start, stop), payload) quantized by the previous step's launch
     plan: dict | None = None           # buffers and bound launches of this tensor, when the runtime keeps plans
     raw_stream: int = 0
+    program: list | None = None        # the launches and exchanges of this run in order, while a plan is being made
 
     def query(self) -> bool:
         return bool(self.producer_completion.query())
@@ -441,6 +452,13 @@ class HipPipelinedRingRuntime:
     a runtime's work is enqueued on its one stream, which orders the reuse of those buffers between runs.
     ``max_plans=0``: every run leases its buffers from the workspace session.
 
+    With plans, the first run on a tensor also records its launches and exchanges in order, and later runs replay that
+    list without going through the per-hop protocol again (14 hops of a W=8 ring: 193 us of host time per bucket
+    through the protocol, which left the GPU waiting; the replay is a loop over pre-bound calls).
+    ``graph_replay=True``: the second run captures the list as one HIP graph - the injected ``exchange`` must then
+    be capturable on the stream it is given (enqueue-only, no host synchronisation, no allocation) - and later runs
+    replay the graph.  Results are the same bits either way.
+
     ``extension_status``: run the steps through the codec facade of that native module instead
     (``quantize_tensor(view, output=...)``, ``dequantize_tensor(received, output=view, reduce_op=...)``,
     ``view.div_(W)``), exactly the calls of the reference's runtime.  This serves every policy and payload format
@@ -451,7 +469,8 @@ class HipPipelinedRingRuntime:
 
     def __init__(self, *, config: CompressionConfig, dtype: str, world_size: int, rank: int,
                  exchange: Callable[..., Any], completion_manager: Any | None = None, stream: Any | None = None,
-                 fuse_steps: bool = True, max_plans: int = 16, extension_status: Any | None = None) -> None:
+                 fuse_steps: bool = True, max_plans: int = 16, extension_status: Any | None = None,
+                 graph_replay: bool = False) -> None:
         from collections import OrderedDict
 
         from lowbit_comm_amd.hip.executors import fused_dequant_fallback_reason
@@ -486,6 +505,7 @@ class HipPipelinedRingRuntime:
         self._exchange = exchange
         self._completions = completion_manager
         self.stream = stream
+        self.graph_replay = bool(graph_replay)
 
     # ---- context ----------------------------------------------------------- #
     def _ready(self) -> None:
@@ -522,8 +542,60 @@ class HipPipelinedRingRuntime:
         if ops.DTYPE_NAMES.get(tensor.dtype) != self.dtype:
             raise RuntimeError(f"tensor dtype {tensor.dtype} does not match the runtime's {self.dtype}")
         produced = self._completions.record_for(tensor, stream=torch.cuda.current_stream(tensor.device))
+        plan = self._plan_of(tensor)
+        recording = plan is not None and "program" not in plan and not self._facade
         return RingSubmissionContext(tensor=tensor, stream=self.stream, producer_completion=produced,
-                                     plan=self._plan_of(tensor), raw_stream=self.stream.cuda_stream)
+                                     plan=plan, raw_stream=self.stream.cuda_stream, program=[] if recording else None)
+
+    # ---- replay of a recorded run ------------------------------------------- #
+    def finish_program(self, context: RingSubmissionContext) -> None:
+        """The schedule has been enqueued once through the protocol: keep what it launched, in order."""
+        if context.plan is not None and context.program is not None:
+            context.plan["program"] = tuple(context.program)
+            context.program = None
+
+    def _run_program(self, program: tuple, stream: Any, raw_stream: int) -> list:
+        handles = []
+        for op in program:
+            kind = op[0]
+            if kind == "launch":
+                if not op[1](raw_stream):
+                    raise RuntimeError("a ring launch has no kernel for this configuration")
+            elif kind == "exchange":
+                handle = self._exchange(op[1], op[2], send_peer=op[3], recv_peer=op[4], stream=stream)
+                handle.wait_stream(stream)
+                handles.append(handle)
+            else:                                    # "divide": the unfused sequence's in-place mean
+                import torch
+
+                from lowbit_comm_amd.hip import ops
+
+                with torch.cuda.stream(stream):
+                    ops.true_divide_(op[1], op[2])
+        return handles
+
+    def replay_program(self, context: RingSubmissionContext) -> list | None:
+        """Enqueue the recorded launches and exchanges of this tensor's plan; ``None`` when there is no record yet."""
+        plan = context.plan
+        program = None if plan is None else plan.get("program")
+        if program is None:
+            return None
+        if not self.graph_replay:
+            return self._run_program(program, context.stream, context.raw_stream)
+        import torch
+
+        graph = plan.get("graph")
+        if graph is None:
+            graph = torch.cuda.CUDAGraph()
+            side = torch.cuda.Stream()               # default priority; capture needs a stream of its own
+            side.wait_stream(context.stream)
+            with torch.cuda.graph(graph, stream=side):
+                self._run_program(program, side, side.cuda_stream)
+            context.stream.wait_stream(side)
+            plan["graph"] = graph
+        with torch.cuda.stream(context.stream):
+            graph.replay()
+        return []
 
     def wait_for_producer(self, tensor: Any, *, context: RingSubmissionContext) -> None:
         context.wait_stream(context.stream)
@@ -614,6 +686,8 @@ class HipPipelinedRingRuntime:
             context.quant_index += 1
         if not bound[0](context.raw_stream):
             raise RuntimeError("quantize+pack has no kernel for this configuration")
+        if context.program is not None:
+            context.program.append(("launch", bound[0]))
         return bound[1]
 
     def send_recv(self, payload: Any, *, send_peer: int, recv_peer: int, recv_chunk: ChunkRange, workspace: Any,
@@ -628,6 +702,8 @@ class HipPipelinedRingRuntime:
             # sized for the chunk that arrives, which is shorter than the one sent when it is the ragged last chunk
             received = self._payload_buffer("recv", index, _view(context.tensor, recv_chunk), workspace, context)
         handle = self._exchange(payload, received, send_peer=send_peer, recv_peer=recv_peer, stream=context.stream)
+        if context.program is not None:
+            context.program.append(("exchange", payload, received, send_peer, recv_peer))
         return received, handle
 
     def _step(self, tensor: Any, received: Any, chunk: ChunkRange, workspace: Any, context: RingSubmissionContext,
@@ -663,11 +739,15 @@ class HipPipelinedRingRuntime:
         for launch in launches:
             if not launch(context.raw_stream):
                 raise RuntimeError("the ring step has no kernel for this configuration")
+            if context.program is not None:
+                context.program.append(("launch", launch))
         if not self.fuse_steps and divisor != 1.0:
             import torch
 
             with torch.cuda.stream(context.stream):
                 ops.true_divide_(view, divisor)
+            if context.program is not None:
+                context.program.append(("divide", view, divisor))
         context.staged = ((chunk.start, chunk.stop), send) if send is not None else None
         return view
 
@@ -795,7 +875,7 @@ def make_pipelined_ring_executor(*, config: CompressionConfig, dtype: str, numel
                                  exchange: Callable[..., Any], pool: Any | None = None,
                                  completion_manager: Any | None = None, device: str = "cuda:0",
                                  fuse_steps: bool = True, max_plans: int = 16,
-                                 extension_status: Any | None = None) -> PipelinedRingExecutor:
+                                 extension_status: Any | None = None, graph_replay: bool = False) -> PipelinedRingExecutor:
     """Plan, schedule, runtime, pooled workspaces and executor of one rank for buckets of ``numel`` elements."""
     from lowbit_comm_amd.hip.completion import HipCompletionManager
     from lowbit_comm_amd.hip.workspace import ShardWorkspaceProvider, create_torch_workspace_pool
@@ -805,7 +885,7 @@ def make_pipelined_ring_executor(*, config: CompressionConfig, dtype: str, numel
     schedule = compile_pipelined_ring_schedule(chunk_plan=plan, rank=rank)
     runtime = HipPipelinedRingRuntime(config=config, dtype=dtype, world_size=world_size, rank=rank, exchange=exchange,
                                       completion_manager=manager, fuse_steps=fuse_steps, max_plans=max_plans,
-                                      extension_status=extension_status)
+                                      extension_status=extension_status, graph_replay=graph_replay)
     provider = ShardWorkspaceProvider(pool if pool is not None else create_torch_workspace_pool(), backend="hip",
                                       collective="all_reduce", strategy="pipelined_ring", device=device)
 

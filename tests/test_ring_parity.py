@@ -284,6 +284,12 @@ def test_ring_replays_a_buckets_plan_without_allocating(ops, hip_device, fuse_st
         for rank in range(world):
             assert np.array_equal(to_np(buckets[rank], "bf16"), want[rank]), (repeat, rank)
     assert all(len(e._runtime.plans) == 1 for e in ring[1])
+    # runs two to four did not go through the per-hop protocol: they replayed the launches the first run recorded
+    for e in ring[1]:
+        (plan,) = e._runtime.plans.values()
+        kinds = [op[0] for op in plan["program"]]
+        assert kinds.count("exchange") == 2 * (world - 1)
+        assert kinds.count("launch") == (1 + 2 * (world - 1) if fuse_steps else 4 * (world - 1))
     # a second bucket shape gets its own plan; the oldest plan goes when the limit is reached
     for e in ring[1]:
         e._runtime.max_plans = 1
@@ -481,6 +487,52 @@ def test_ring_step_randomized_sweep(ops, hip_device):
         emit = rng.random() < 0.7
         offset = rng.choice([0, 0, 0, 1, 2, 5])
         check_step(ops, hip_device, dtype, g, n, reduce_op, divisor, emit, 50_000 + 3 * case, offset=offset)
+
+
+@pytest.mark.parametrize("dtype,n", [("fp32", 64 * 8 * 300), ("bf16", 64 * 8 * 101 + 40)])
+def test_one_ranks_schedule_replayed_as_a_hip_graph_gives_the_protocols_bits(hip_device, dtype, n):
+    """One rank of a W=8 ring with a stand-in for the link that a graph can capture (a device copy of a fixed peer
+    payload into the receive buffer).  Run one goes through the per-hop protocol and records, run two captures the
+    recorded launches as one graph, runs three and four replay it - with eager work and synchronisations in
+    between, and each compared with an executor that only ever uses the protocol."""
+    from lowbit_comm_amd.config import CompressionConfig
+    from lowbit_comm_amd.hip import ops
+    from lowbit_comm_amd.hip.ring import make_pipelined_ring_executor
+
+    world, rank, g = 8, 3, 64
+    config = CompressionConfig(group_size=g)
+    chunk = -(-n // world)
+    peer = torch.empty(ops.payload_nbytes(chunk, g), dtype=torch.uint8, device=hip_device)
+    assert ops.quant_pack_payload_into(tensor_like(chunk, "fp32", 9100, hip_device), peer)
+
+    class Arrived:
+        def query(self):
+            return True
+
+        def wait_stream(self, stream):
+            return None
+
+    def exchange(payload, received, *, send_peer, recv_peer, stream):
+        with torch.cuda.stream(stream):
+            received.copy_(peer[:received.numel()], non_blocking=True)
+        return Arrived()
+
+    protocol = make_pipelined_ring_executor(config=config, dtype=dtype, numel=n, world_size=world, rank=rank,
+                                            exchange=exchange, max_plans=0)
+    graphed = make_pipelined_ring_executor(config=config, dtype=dtype, numel=n, world_size=world, rank=rank,
+                                           exchange=exchange, graph_replay=True)
+    bucket = torch.empty(n, dtype=DTYPES[dtype], device=hip_device)
+    for run in range(4):
+        values = tensor_like(n, dtype, 9200 + run, hip_device)
+        want = values.clone()
+        assert protocol.run(want).wait() is want
+        bucket.copy_(values)
+        assert graphed.run(bucket).wait() is bucket
+        torch.cuda.synchronize()
+        assert np.array_equal(raw(to_np(bucket, dtype)), raw(to_np(want, dtype))), run
+        assert float((torch.randn(1 << 16, device=hip_device) * 2).sum().item()) == pytest.approx(0.0, abs=1e4)   # eager work
+    (plan,) = graphed._runtime.plans.values()
+    assert isinstance(plan["graph"], torch.cuda.CUDAGraph) and len(plan["program"]) == 1 + 4 * (world - 1)
 
 
 def test_ring_steps_captured_in_a_hip_graph_replay_like_eager(hip_device):
