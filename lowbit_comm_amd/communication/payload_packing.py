@@ -46,13 +46,24 @@ def _bytes_of(tensor: Any) -> Any:
 
 
 def _is_view_of_packed(payload: CompressedPayload, fields: tuple[TensorFieldSchema, ...]) -> Any | None:
-    """The packed tensor itself when buffer and metadata are already adjacent views of one allocation
-    (a :class:`~lowbit_comm_amd.communication.collectives.PackedPayload`)."""
+    """The packed tensor itself when buffer and metadata are adjacent views of that one allocation, each at its
+    offset in the schema (a :class:`~lowbit_comm_amd.communication.collectives.PackedPayload` as the quantizer made
+    it).  A payload whose buffer or metadata were replaced since (``dataclasses.replace``, an edited metadata
+    dict) no longer passes and is packed by copying."""
     packed = getattr(payload, "packed", None)
-    if packed is None:
+    if packed is None or int(packed.numel()) != sum(f.byte_count for f in fields):
         return None
-    total = sum(f.byte_count for f in fields)
-    return packed if int(packed.numel()) == total else None
+    base = packed.data_ptr()
+    for f in fields:
+        piece = payload.buffer if f.name == "buffer" else payload.metadata.get(f.name)
+        if not _looks_like_tensor(piece) or not callable(getattr(piece, "data_ptr", None)):
+            return None
+        contiguous = getattr(piece, "is_contiguous", None)
+        if callable(contiguous) and not contiguous():
+            return None
+        if piece.data_ptr() != base + f.offset or int(piece.numel()) * int(piece.element_size()) != f.byte_count:
+            return None
+    return packed
 
 
 @dataclass(frozen=True)

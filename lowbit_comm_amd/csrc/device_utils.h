@@ -314,14 +314,20 @@ template <typename T, int N> __device__ __forceinline__ void divide_all(float (&
 // quotient -> 0.  A code comes back as the bit pattern of (code + 1.5 * 2^23): its low byte is the int8 code that
 // goes into the payload (pack4 takes low bytes), and code_value() gives the integer back as a float.
 //
-// The quotient is exact and the path has no data-dependent branch.  y = 1/scale is one IEEE division per lane,
-// i.e. the correctly rounded reciprocal; per element q0 = p*y is within an ulp of p/scale, r = fma(-q0, scale, p)
-// is its exact remainder, and q1 = fma(r, y, q0) is then the correctly rounded quotient (Markstein's correction
-// step for division with a fused multiply-add; its premise is exactly a correctly rounded reciprocal).  The one
-// case outside the theorem, a remainder that underflows, needs |p/scale| < 2^-70, where the code is 0 whatever
-// the last bit of the quotient is.  tests/native/quotient_check.hip compares q1 with the division on the device
-// for 2*10^11 pairs from this domain, among them 7*10^10 quotients within four ulps of a half-integer and
-// dividends with 8 or 11 significant bits: no code differs.  (A reciprocal-multiply fast path with a fallback
+// The path has no division per element and no data-dependent branch.  y = 1/scale is one IEEE division per lane,
+// i.e. the correctly rounded reciprocal; per element q0 = p*y is within an ulp and a half of p/scale,
+// r = fma(-q0, scale, p) is its exact remainder, and q1 = fma(r, y, q0) is Markstein's correction step for division
+// with a fused multiply-add: RN(q + d) for the real quotient q and a |d| below 2^-23 ulp.  Markstein's theorem
+// promises q1 = RN(q) only for a q0 within one ulp, so the claim that matters here - rint(q1) is the code the
+// division gives - is checked, not inferred: q1 and RN(q) are equal or neighbouring floats and every half-integer
+// up to 127.5 is a float, so the codes can differ only for a p within a few ulps of (k + 0.5) * scale, and the
+// operations are invariant under a common power of two away from underflow.  tests/native/quotient_check.hip walks
+// all 2^23 scale mantissas x 256 half-integers x 13 neighbouring dividends at three exponents (8*10^10 pairs, every
+// such case) and 2.6*10^10 sampled pairs over the whole exponent range 2^-23 .. 2^120, among them dividends with 8
+// or 11 significant bits: no code and no quotient differs.  The one case outside, a remainder that underflows,
+// needs |p/scale| < 2^-64, where the code is 0 whatever the last bit of the quotient is.  The ragged edge uses
+// the same operations (encode below), so an element's code does not depend on the block it falls into.
+// (A reciprocal-multiply fast path with a fallback
 // for quotients next to a tie, which this replaces, took the fallback in most wavefronts of a 16-bit tensor -
 // 127*x/absmax hits exact ties all the time when x and absmax have 8-bit mantissas - and ran it 25 % slower.)
 // Adding 1.5 * 2^23 rounds q1 to an integer, half to even, and leaves it in the low mantissa bits.
@@ -351,8 +357,14 @@ __device__ __forceinline__ void encode_group(const float (&p)[N], float scale, i
     encode_group<N>(p, scale, 1.0f / scale, codes);
 }
 
-// Single-element form for the ragged edge.
-__device__ __forceinline__ int encode(float p, float scale) { return cvt_i32(__builtin_rintf(p / scale)); }
+// Single-element form for the ragged edge: the same operations as encode_group, so that an element gets the same
+// code whether it falls into an interior block or into the tail.
+__device__ __forceinline__ int encode(float p, float scale) {
+    const float one[1] = {p};
+    int bits[1];
+    encode_group<1>(one, scale, bits);
+    return static_cast<int>(code_value(bits[0]));   // an integer in [-127, 127]: the conversion is exact
+}
 
 // Low bytes of four ints -> one little-endian word (three v_perm_b32).
 __device__ __forceinline__ uint32_t pack4(int c0, int c1, int c2, int c3) {

@@ -12,10 +12,13 @@ injected (or synthesised by a test / benchmark) and every compute step is one la
     requantize shard    -> lbc_quant_pack            (into row ``rank`` of the gather buffer)
     decode W shards     -> lbc_dequant_chunks        (one launch for all W shards)
 
-Workspaces are allocated once per plan and reused, so a steady-state bucket allocates nothing.
+Workspaces are allocated once per plan and reused, so a steady-state bucket allocates nothing.  A plan serves one
+bucket at a time: uses on one stream are ordered by the stream, a use on another stream is ordered after the previous
+one by an event, and a plan whose asynchronous exchange has not been waited for refuses the next bucket.
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 from collections.abc import Callable
 from typing import Any
 
@@ -58,15 +61,37 @@ class ReduceScatterPlan:
         self.received = torch.empty(rows, dtype=torch.uint8, device=self.device)   # every rank's chunk for me
         self.gathered = torch.empty(rows, dtype=torch.uint8, device=self.device)   # every rank's requantized shard
         self.shard = torch.empty(shard, dtype=self.reduced_dtype, device=self.device)
-        self._bound: dict[Any, ops.BoundLaunch] = {}   # launches bound to tensor addresses seen so far
+        # Launches bound to the tensor addresses seen last.  A bound launch keeps its tensors alive, so the cache is
+        # small: one entry for each of the five steps of a bucket whose tensors stay put, and a few to spare.
+        self._bound: OrderedDict[Any, ops.BoundLaunch] = OrderedDict()
+        self._last_stream: torch.cuda.Stream | None = None
+        self.exchange_in_flight: Any | None = None     # work object of an exchange that nobody has waited for yet
+
+    _BOUND_LAUNCHES = 8
 
     def _remember(self, key: Any, make: Callable[[], ops.BoundLaunch]) -> ops.BoundLaunch:
         bound = self._bound.get(key)
         if bound is None:
-            if len(self._bound) >= 32:      # addresses keep changing: do not grow without bound
-                self._bound.clear()
             bound = self._bound[key] = make()
+            while len(self._bound) > self._BOUND_LAUNCHES:
+                self._bound.popitem(last=False)
+        else:
+            self._bound.move_to_end(key)
         return bound
+
+    def _order_after_previous_use(self) -> None:
+        """Called by every step before it touches the plan's buffers.  On the stream of the previous step nothing is
+        needed; on another stream an event recorded there now (it covers everything that stream was given so far,
+        the previous step included) is waited for by the current stream."""
+        if self.device.type != "cuda":
+            return
+        stream = torch.cuda.current_stream(self.device)
+        previous = self._last_stream
+        if previous is not None and previous != stream:
+            event = torch.cuda.Event()
+            event.record(previous)
+            stream.wait_event(event)
+        self._last_stream = stream
 
     # ---- payload views ---------------------------------------------------------------------------
     def payload(self, rows: torch.Tensor, index: int) -> torch.Tensor:
@@ -87,8 +112,12 @@ class ReduceScatterPlan:
         flat = tensor.reshape(-1)
         if flat.numel() != self.numel or flat.dtype != self.dtype:
             raise ValueError("tensor does not match the planned bucket")
-        key = ("q", flat.data_ptr(), None if residual is None else residual.data_ptr(),
-               None if new_residual is None else new_residual.data_ptr())
+        if self.exchange_in_flight is not None:
+            raise RuntimeError("this plan's send and receive buffers belong to an exchange that has not been waited for: "
+                               "wait for the previous bucket's work first, or give every bucket in flight its own plan")
+        self._order_after_previous_use()
+        key = ("q", flat.data_ptr(), None if residual is None else (residual.data_ptr(), residual.dtype),
+               None if new_residual is None else (new_residual.data_ptr(), new_residual.dtype))
         bound = self._remember(key, lambda: ops.bind_quant_pack_chunks(
             flat, self.send, self.world_size, group_size=self.config.group_size,
             residual=None if residual is None else residual.reshape(-1),
@@ -106,9 +135,10 @@ class ReduceScatterPlan:
         target = self.shard if out is None else out
         shard = self.chunks.shard_numel
         fused = self.world_size <= ops.MAX_PAYLOADS
+        self._order_after_previous_use()
         if shard:
             if fused:
-                bound = self._remember(("r", rows.data_ptr(), target.data_ptr(), op), lambda: ops.bind_dequant_reduce(
+                bound = self._remember(("r", rows.data_ptr(), target.data_ptr(), target.dtype, op), lambda: ops.bind_dequant_reduce(
                     self._pairs(rows), target, numel=shard, group_size=self.config.group_size,
                     divisor=float(self.world_size) if op == "mean" else 1.0))
                 fused = bool(bound())
@@ -142,7 +172,8 @@ class ReduceScatterPlan:
             codes, scales = ops.split_payload(row, self.chunks.shard_numel, self.config.group_size)
             return ops.bind_quant_pack(source, codes, scales, group_size=self.config.group_size)
 
-        bound = self._remember(("g", source.data_ptr()), make)
+        self._order_after_previous_use()
+        bound = self._remember(("g", source.data_ptr(), source.dtype), make)
         if self.chunks.shard_numel and not bound():
             raise ValueError(f"no HIP quantize kernel for dtype {source.dtype}")
         return row
@@ -162,6 +193,7 @@ class ReduceScatterPlan:
         if self.world_size > ops.MAX_PAYLOADS:
             self.reduce_received(rows, op=op)
             return self.requantize_shard()
+        self._order_after_previous_use()
 
         def make() -> ops.BoundLaunch:
             codes, scales = ops.split_payload(row, shard, self.config.group_size)
@@ -180,7 +212,8 @@ class ReduceScatterPlan:
         target = out if out is not None else torch.empty(self.numel, dtype=self.reduced_dtype, device=self.device)
         make = lambda: ops.bind_dequant_chunks(rows, target.reshape(-1), self.chunks.shard_numel,  # noqa: E731
                                                group_size=self.config.group_size)
-        bound = self._remember(("d", rows.data_ptr(), target.data_ptr()), make) if out is not None else make()
+        self._order_after_previous_use()
+        bound = self._remember(("d", rows.data_ptr(), target.data_ptr(), target.dtype), make) if out is not None else make()
         if self.numel and not bound():
             raise ValueError(f"no HIP decode kernel for dtype {target.dtype}")
         return target.reshape(self.shape)
@@ -217,8 +250,20 @@ def compressed_reduce_scatter_shard(tensor: torch.Tensor, *, config: Compression
     if not callable(getattr(exchange, "wait", None)):
         raise TypeError("with async_op the exchange must return a work object with wait()")
     future = future_factory() if future_factory is not None else torch.futures.Future()
-    return AsyncShardPipeline(communication_work=exchange, future=future,
-                              reduce_shard=lambda _received: plan.reduce_received(op=op),
+    plan.exchange_in_flight = exchange       # the exchange reads plan.send and writes plan.received on a stream of its own
+
+    def reduce_shard(_received: Any) -> ReducedShard:   # runs once the exchange has been waited for
+        plan.exchange_in_flight = None
+        return plan.reduce_received(op=op)
+
+    def release_plan(_done: Any) -> None:               # also when the exchange failed and the reduce never ran
+        if plan.exchange_in_flight is exchange:
+            plan.exchange_in_flight = None
+
+    if callable(getattr(future, "add_done_callback", None)):
+        future.add_done_callback(release_plan)
+
+    return AsyncShardPipeline(communication_work=exchange, future=future, reduce_shard=reduce_shard,
                               update_feedback=update_feedback or (lambda _shard: None),
                               advance_policy=advance_policy or (lambda: None),
                               completion_manager=completion_manager, resources=(tensor, plan, send)).run()

@@ -28,11 +28,13 @@ def test_client_runs_quantize_reduce_and_ring_step_bit_exact_against_the_c_oracl
 
 @pytest.mark.gpu
 def test_exact_quotient_without_a_division_matches_the_division_on_billions_of_pairs(hip_device):
-    """tests/native/quotient_check.hip: the encode's FMA-refined quotient against ``p / s`` on the device, 4.3e9
-    pairs in each of six modes (random, extreme scale mantissas, quotients next to ties, 16-bit dividends)."""
+    """tests/native/quotient_check.hip: the encode's FMA-refined quotient against ``p / s`` on the device.  4.3e9
+    pairs in each of six sampled modes (random, extreme scale mantissas, quotients next to ties, 16-bit dividends)
+    with scale exponents over the whole domain, and the exhaustive walk over every scale mantissa and every dividend
+    next to a half-integer multiple of the scale, the only pairs whose code the refinement could change."""
     checker = ROOT / "tests" / "native" / "_build" / "quotient_check"
     assert checker.exists(), "run __graft_entry__.build() first"
-    done = subprocess.run([str(checker), "1"], capture_output=True, text=True, timeout=300)
+    done = subprocess.run([str(checker), "1", "1"], capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stdout[-2000:]
-    assert "CODE MISMATCHES 0" in done.stdout
-    assert done.stdout.count("code mismatches 0") == 6
+    assert "MISMATCHES 0" in done.stdout.splitlines()[-1]
+    assert done.stdout.count("code mismatches 0") == 7 and done.stdout.count("quotient mismatches 0 ") == 7

@@ -429,6 +429,8 @@ def test_asynchronous_shard_exchange_completes_through_the_pipeline(dev):
                                            advance_policy=lambda: advanced.append(True))
     assert isinstance(work, AsyncShardPipeline) and work.query() is False and not fed
     assert buckets[0] in work.resources
+    with pytest.raises(RuntimeError, match="has not been waited for"):   # one bucket in flight per plan
+        plans[0].quantize_chunks(buckets[0])
     started[0].future.set_result(None)                          # the exchange is over
     assert work.query() is True and started[0].waited == 1 and advanced == [True]
     shard = work.wait()
@@ -438,6 +440,42 @@ def test_asynchronous_shard_exchange_completes_through_the_pipeline(dev):
     with pytest.raises(TypeError, match="must return a work object"):
         compressed_reduce_scatter_shard(buckets[0], config=CFG, world_size=world, rank=0, all_to_all=copy_rows,
                                         plan=plans[0], async_op=True)
+
+
+def test_reduce_scatter_plan_keeps_few_bound_launches_and_orders_uses_across_streams(hip_device):
+    """A caller whose tensors are new every step must not pin them through the plan's cache of bound launches, a
+    residual of another dtype at a recycled address must not reuse a stale binding, and a use of the plan on
+    another stream is ordered after the previous use."""
+    from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
+
+    world, n = 4, 64 * 4 * 200
+    config = CompressionConfig(error_feedback=False)
+    plan = ReduceScatterPlan(n, torch.float32, world_size=world, rank=1, config=config, device=hip_device)
+    kept = [torch.randn(n, device=hip_device) * 1e-3 for _ in range(20)]
+    for bucket in kept:
+        plan.quantize_chunks(bucket)
+    assert len(plan._bound) <= ReduceScatterPlan._BOUND_LAUNCHES
+    assert kept[-1].data_ptr() in [key[1] for key in plan._bound] and kept[0].data_ptr() not in [key[1] for key in plan._bound]
+
+    residual32 = torch.zeros(n, device=hip_device)
+    residual16 = residual32.view(torch.bfloat16)[:n]            # same address, another dtype
+    plan.quantize_chunks(kept[0], residual=residual32, new_residual=residual32)
+    keys = {key for key in plan._bound if key[0] == "q"}
+    plan.quantize_chunks(kept[0].bfloat16().float(), residual=residual32)
+    assert ("q", kept[0].data_ptr(), (residual32.data_ptr(), torch.float32), (residual32.data_ptr(), torch.float32)) in keys
+    assert residual16.data_ptr() == residual32.data_ptr()
+    assert ("q", kept[0].data_ptr(), (residual16.data_ptr(), torch.bfloat16), None) not in plan._bound
+
+    want = plan.quantize_chunks(kept[3]).clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        plan.quantize_chunks(kept[5])                           # the side stream now owns the plan's buffers
+    assert plan._last_stream == side
+    got = plan.quantize_chunks(kept[3])                         # back on the default stream: ordered after the side stream
+    assert plan._last_stream == torch.cuda.current_stream()
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
 
 
 def test_reduce_scatter_plan_fused_requantize_matches_the_two_steps(hip_device):

@@ -222,6 +222,23 @@ def test_packed_bytes_are_codes_then_little_endian_fp32_scales():
     assert back.buffer.dtype == torch.int8 and back.metadata["scales"].dtype == torch.float32
 
 
+def test_packed_payload_is_shipped_as_is_only_while_its_pieces_are_still_views_of_it():
+    from lowbit_comm_amd.communication import PackedPayload
+
+    packed = torch.tensor([254, 3, 7, 11, 0, 0, 128, 62, 0, 0, 128, 63], dtype=torch.uint8)
+    codes, scales = packed[:4].view(torch.int8), packed[4:].view(torch.float32)
+    payload = PackedPayload(buffer=codes, shape=(4,), dtype="fp32", metadata={"scales": scales, "original_numel": 4},
+                            packed=packed)
+    packer = FusedPayloadPacker.from_payload(payload)
+    assert packer.pack(payload) is packed                              # no copy
+    swapped = dataclasses.replace(payload, buffer=torch.tensor([1, 2, 3, 4], dtype=torch.int8))
+    assert packer.pack(swapped).tolist() == [1, 2, 3, 4, 0, 0, 128, 62, 0, 0, 128, 63]
+    edited = dataclasses.replace(payload, metadata={"scales": torch.tensor([2.0, 4.0]), "original_numel": 4})
+    assert packer.pack(edited).tolist() == [254, 3, 7, 11, 0, 0, 0, 64, 0, 0, 128, 64]
+    shifted = dataclasses.replace(payload, metadata={"scales": packed[0:8].view(torch.float32), "original_numel": 4})
+    assert packer.pack(shifted) is not packed                          # a view of the allocation, at the wrong offset
+
+
 def test_fused_packer_rejects_payloads_without_tensor_metadata():
     fused = make_fused_payload_all_gather(lambda packed: GatheredPayloads([packed], 1))
     bare = CompressedPayload(buffer=torch.tensor([1, 2, 3], dtype=torch.int8), shape=(3,), dtype="fp16",
