@@ -838,10 +838,10 @@ def main() -> int:
 
         def gather(payload):
             key = payload.buffer.numel()
-            if key not in peers:
-                peers[key] = [payload.buffer.clone() for _ in range(world - 1)]
-            others = [CompressedPayload(buffer=b, shape=payload.shape, dtype=payload.dtype) for b in peers[key]]
-            return GatheredPayloads(payloads=[payload] + others, world_size=world)
+            if key not in peers:       # the peers' payloads stay where they are, as in a reused gather buffer
+                peers[key] = [CompressedPayload(buffer=payload.buffer.clone(), shape=payload.shape, dtype=payload.dtype)
+                              for _ in range(world - 1)]
+            return GatheredPayloads(payloads=[payload] + peers[key], world_size=world)
 
         for feedback in (False, True):
             hook = create_ddp_comm_hook(CompressionConfig(error_feedback=feedback), strategy="all_gather", reduce="mean",

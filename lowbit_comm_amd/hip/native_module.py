@@ -15,6 +15,8 @@ and ignored: the portable format has a single layout.
 from __future__ import annotations
 
 import enum
+import operator
+from collections import OrderedDict
 from typing import Sequence
 
 import torch
@@ -44,6 +46,8 @@ class ReduceOP(enum.IntEnum):
     MIN = 3
 
 
+_IS_CUDA = operator.attrgetter("is_cuda")
+_DTYPE = operator.attrgetter("dtype")
 _TORCH_OF = {DType.FP16: torch.float16, DType.BF16: torch.bfloat16, DType.FP32: torch.float32}
 _OP_NAME = {ReduceOP.NONE: "none", ReduceOP.SUM: "sum", ReduceOP.MAX: "max", ReduceOP.MIN: "min"}
 
@@ -93,6 +97,56 @@ class HipNativeModule:
 
     def __init__(self) -> None:
         self._lib = load_library()
+        # Launches of the allocation-free entry points, bound to the addresses they were last called with.  A DDP
+        # hook presents the same bucket, payload and workspace addresses every step, so from the second step on a
+        # call is one key lookup and one ABI call.  The key holds everything a binding depends on (addresses,
+        # dtypes, element counts, policy), the entries do not keep the tensors alive, least recently used go first.
+        self._launches: OrderedDict = OrderedDict()
+
+    _LAUNCH_MEMO_ENTRIES = 256
+
+    def _memoized(self, key: tuple, bind):
+        """The launch remembered under ``key``, else ``bind()`` (which validates and may raise; nothing is then
+        stored).  ``bind`` may return ``None`` for a call that has no single launch."""
+        launches = self._launches
+        bound = launches.get(key)
+        if bound is not None:
+            launches.move_to_end(key)
+            return bound
+        bound = bind()
+        if bound is not None:
+            launches[key] = bound.forget_tensors()
+            while len(launches) > self._LAUNCH_MEMO_ENTRIES:
+                launches.popitem(last=False)
+        return bound
+
+    @staticmethod
+    def _spec(tensor):
+        """What a binding depends on, for a contiguous GPU tensor; ``None`` for anything else (the caller then takes
+        the validating path, which names what is wrong)."""
+        if tensor is None:
+            return ()
+        if not isinstance(tensor, torch.Tensor) or not tensor.is_cuda or not tensor.is_contiguous():
+            return None
+        return (tensor.data_ptr(), tensor.dtype, tensor.numel())
+
+    def _reduce_key(self, tag, inputs, tensors, policy):
+        """Memo key of a fused reduce: payload addresses and sizes, the other tensors' specs, the policy."""
+        if not isinstance(inputs, (list, tuple)) or not 1 <= len(inputs) <= ops.MAX_PAYLOADS:
+            return None
+        specs = []
+        for tensor in tensors:
+            spec = self._spec(tensor)
+            if spec is None:
+                return None
+            specs.append(spec)
+        try:        # loops that stay in C: this runs for every bucket
+            if not (all(map(_IS_CUDA, inputs)) and all(map(torch.Tensor.is_contiguous, inputs))):
+                return None
+            return (tag, tuple(map(torch.Tensor.data_ptr, inputs)), tuple(map(torch.Tensor.numel, inputs)),
+                    tuple(map(_DTYPE, inputs)), tuple(specs), policy)
+        except (TypeError, AttributeError):      # something in the list is not a tensor
+            return None
 
     # ---- quantize ------------------------------------------------------------------------------
     def quantize(self, input, group_size, topk, stochastic, bit, quant_type, compact):
@@ -125,8 +179,17 @@ class HipNativeModule:
                 raise RuntimeError("output has an invalid quantized payload size")
             return True
         # payload dtype / contiguity / size are checked where the addresses are taken
-        return ops.quant_pack_payload_into(input.reshape(-1), output, group_size=group_size,
-                                           residual=None if residual is None else residual.reshape(-1))
+        bind = lambda: ops.bind_quant_pack_payload(input.reshape(-1), output, group_size=group_size,  # noqa: E731
+                                                   residual=None if residual is None else residual.reshape(-1))
+        out_spec, r_spec = self._spec(output), self._spec(residual)
+        if out_spec is None or r_spec is None:
+            return bind()()
+        key = ("quant_pack", input.data_ptr(), input.dtype, input.numel(), out_spec, r_spec, group_size)
+        bound = self._launches.get(key)         # the steady state: same addresses as last step
+        if bound is not None:
+            self._launches.move_to_end(key)
+            return bound()
+        return self._memoized(key, bind)()
 
     # ---- dequantize -----------------------------------------------------------------------------
     def dequantize(self, input, group_size, topk, bit, reduce_op, quant_type, dtype, compact):
@@ -177,6 +240,20 @@ class HipNativeModule:
         self.inplace_dequantize_reduce(inputs, output, group_size, topk, bit, quant_type, compact)
         return output
 
+    def dequantize_reduce_mean(self, inputs, group_size, topk, bit, quant_type, dtype, compact, divisor):
+        """``dequantize_reduce`` with the division by ``divisor`` in the same launch (no counterpart in the
+        reference's module: its facade divides the sum afterwards, which costs a copy and a second pass; the bits
+        are the same).  ``None`` when the fused launch does not apply: the caller then sums and divides."""
+        _require_policy(group_size, topk, False, bit, quant_type)
+        if len(inputs) == 0:
+            raise RuntimeError("inputs must not be empty")
+        _check_payload(inputs[0], "input")
+        output = torch.empty(_padded_numel_of(inputs[0], group_size), dtype=_TORCH_OF[DType(int(dtype))],
+                             device=inputs[0].device)
+        if self.inplace_dequantize_reduce_mean(inputs, output, group_size, topk, bit, quant_type, compact, divisor):
+            return output
+        return None
+
     def inplace_dequantize_reduce(self, inputs, output, group_size, topk, bit, quant_type, compact) -> None:
         """Sum of all payloads into ``output`` in list order; any number of payloads (8 per fused launch)."""
         _require_policy(group_size, topk, False, bit, quant_type)
@@ -185,9 +262,17 @@ class HipNativeModule:
         _check_payload(inputs[0], "input")
         flat = output.reshape(-1)
         numel = min(flat.numel(), _padded_numel_of(inputs[0], group_size))
+        key = self._reduce_key("reduce", inputs, (flat,), (group_size, topk, bit, int(quant_type), numel))
+        bound = self._launches.get(key) if key is not None else None
+        if bound is not None:
+            self._launches.move_to_end(key)
+            if not bound():
+                raise RuntimeError(f"no HIP dequantize-reduce kernel for output dtype {output.dtype}")
+            return
         entries = self._entries(inputs, numel, group_size)
         if len(entries) <= ops.MAX_PAYLOADS:
-            if not ops.dequant_reduce_into(entries, flat, numel=numel, group_size=group_size):
+            bind = lambda: ops.bind_dequant_reduce(entries, flat, numel=numel, group_size=group_size)  # noqa: E731
+            if not (self._memoized(key, bind) if key is not None else bind())():
                 raise RuntimeError(f"no HIP dequantize-reduce kernel for output dtype {output.dtype}")
             return
         # More than 8 payloads: keep the left fold exact by chaining decode-and-add one payload at a time.
@@ -218,9 +303,16 @@ class HipNativeModule:
                                        divisor) -> bool:
         if divisor <= 0:
             raise RuntimeError("divisor must be > 0")
-        if not self._fused_eligible(inputs, output, group_size, topk, bit, quant_type):
-            return False
-        return ops.dequant_reduce_into(list(inputs), output.reshape(-1), group_size=group_size, divisor=float(divisor))
+        key = self._reduce_key("reduce_mean", inputs, (output,),
+                               (group_size, topk, bit, int(quant_type), float(divisor)))
+        bound = self._launches.get(key) if key is not None else None
+        if bound is None:
+            if not self._fused_eligible(inputs, output, group_size, topk, bit, quant_type):
+                return False
+            bind = lambda: ops.bind_dequant_reduce(list(inputs), output.reshape(-1), group_size=group_size,  # noqa: E731
+                                                   divisor=float(divisor))
+            bound = self._memoized(key, bind) if key is not None else bind()
+        return bound()
 
     # ---- error feedback -------------------------------------------------------------------------
     def inplace_error_feedback_update(self, prepared, restored, residual) -> None:
@@ -253,6 +345,12 @@ class HipNativeModule:
         """One launch: ``restored = mean/sum of payloads``, ``residual = prepared - restored``."""
         if divisor <= 0:
             raise RuntimeError("divisor must be > 0")
+        key = self._reduce_key("reduce_mean_feedback", inputs, (prepared, restored, residual),
+                               (group_size, topk, bit, int(quant_type), float(divisor)))
+        bound = self._launches.get(key) if key is not None else None
+        if bound is not None:
+            self._launches.move_to_end(key)
+            return bound()
         for name, t in (("prepared", prepared), ("restored", restored), ("residual", residual)):
             if not isinstance(t, torch.Tensor) or not t.is_cuda:
                 raise RuntimeError(f"{name} must be a GPU tensor")
@@ -278,6 +376,7 @@ class HipNativeModule:
             if (not isinstance(buffer, torch.Tensor) or buffer.dtype != torch.uint8 or not buffer.is_cuda
                     or not buffer.is_contiguous() or buffer.device != prepared.device or buffer.numel() != expected):
                 return False
-        return ops.dequant_reduce_into(list(inputs), restored.reshape(-1), numel=numel, group_size=group_size,
-                                       divisor=float(divisor), prepared=prepared.reshape(-1),
-                                       new_residual=residual.reshape(-1))
+        bind = lambda: ops.bind_dequant_reduce(list(inputs), restored.reshape(-1), numel=numel,  # noqa: E731
+                                               group_size=group_size, divisor=float(divisor),
+                                               prepared=prepared.reshape(-1), new_residual=residual.reshape(-1))
+        return (self._memoized(key, bind) if key is not None else bind())()

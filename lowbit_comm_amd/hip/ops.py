@@ -185,6 +185,13 @@ class BoundLaunch:
         self._keep = keep
         self._kind = kind      # which entry point the arguments belong to, for launches that can share a grid
 
+    def forget_tensors(self) -> "BoundLaunch":
+        """Stop keeping the bound tensors alive.  For a cache keyed by everything the binding depends on (addresses,
+        dtypes, element counts) whose user passes the live tensors at every call anyway: the launch stays valid for
+        any tensor that matches the key, and the cache pins no memory."""
+        self._keep = ()
+        return self
+
     def __call__(self, stream: int | None = None) -> bool:
         """Enqueue.  ``stream``: raw ``hipStream_t`` handle (``torch.cuda.Stream.cuda_stream``) of a stream on
         the tensors' device, which must be the current device; ``None`` looks up torch's current stream."""

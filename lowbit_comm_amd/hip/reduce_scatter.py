@@ -61,18 +61,20 @@ class ReduceScatterPlan:
         self.received = torch.empty(rows, dtype=torch.uint8, device=self.device)   # every rank's chunk for me
         self.gathered = torch.empty(rows, dtype=torch.uint8, device=self.device)   # every rank's requantized shard
         self.shard = torch.empty(shard, dtype=self.reduced_dtype, device=self.device)
-        # Launches bound to the tensor addresses seen last.  A bound launch keeps its tensors alive, so the cache is
-        # small: one entry for each of the five steps of a bucket whose tensors stay put, and a few to spare.
+        # Launches bound to the tensor addresses seen so far, least recently used dropped first.  Many buckets of one
+        # shape share a plan (the layers of a transformer), so the cache is sized for them; its entries do not keep
+        # the callers' tensors alive (the key holds everything a binding depends on, and every step is handed the
+        # live tensors), so it pins no memory beyond the plan's own buffers.
         self._bound: OrderedDict[Any, ops.BoundLaunch] = OrderedDict()
-        self._last_stream: torch.cuda.Stream | None = None
+        self._last_stream_handle: int | None = None
         self.exchange_in_flight: Any | None = None     # work object of an exchange that nobody has waited for yet
 
-    _BOUND_LAUNCHES = 8
+    _BOUND_LAUNCHES = 256
 
     def _remember(self, key: Any, make: Callable[[], ops.BoundLaunch]) -> ops.BoundLaunch:
         bound = self._bound.get(key)
         if bound is None:
-            bound = self._bound[key] = make()
+            bound = self._bound[key] = make().forget_tensors()
             while len(self._bound) > self._BOUND_LAUNCHES:
                 self._bound.popitem(last=False)
         else:
@@ -85,13 +87,13 @@ class ReduceScatterPlan:
         the previous step included) is waited for by the current stream."""
         if self.device.type != "cuda":
             return
-        stream = torch.cuda.current_stream(self.device)
-        previous = self._last_stream
-        if previous is not None and previous != stream:
+        handle = ops.current_stream_handle(self.device)
+        previous = self._last_stream_handle
+        if previous is not None and previous != handle:
             event = torch.cuda.Event()
-            event.record(previous)
-            stream.wait_event(event)
-        self._last_stream = stream
+            event.record(torch.cuda.ExternalStream(previous, device=self.device))
+            torch.cuda.current_stream(self.device).wait_event(event)
+        self._last_stream_handle = handle
 
     # ---- payload views ---------------------------------------------------------------------------
     def payload(self, rows: torch.Tensor, index: int) -> torch.Tensor:
@@ -116,8 +118,8 @@ class ReduceScatterPlan:
             raise RuntimeError("this plan's send and receive buffers belong to an exchange that has not been waited for: "
                                "wait for the previous bucket's work first, or give every bucket in flight its own plan")
         self._order_after_previous_use()
-        key = ("q", flat.data_ptr(), None if residual is None else (residual.data_ptr(), residual.dtype),
-               None if new_residual is None else (new_residual.data_ptr(), new_residual.dtype))
+        key = ("q", flat.data_ptr(), None if residual is None else (residual.data_ptr(), residual.dtype, residual.numel()),
+               None if new_residual is None else (new_residual.data_ptr(), new_residual.dtype, new_residual.numel()))
         bound = self._remember(key, lambda: ops.bind_quant_pack_chunks(
             flat, self.send, self.world_size, group_size=self.config.group_size,
             residual=None if residual is None else residual.reshape(-1),
@@ -138,7 +140,7 @@ class ReduceScatterPlan:
         self._order_after_previous_use()
         if shard:
             if fused:
-                bound = self._remember(("r", rows.data_ptr(), target.data_ptr(), target.dtype, op), lambda: ops.bind_dequant_reduce(
+                bound = self._remember(("r", rows.data_ptr(), rows.numel(), target.data_ptr(), target.dtype, target.numel(), op), lambda: ops.bind_dequant_reduce(
                     self._pairs(rows), target, numel=shard, group_size=self.config.group_size,
                     divisor=float(self.world_size) if op == "mean" else 1.0))
                 fused = bool(bound())
@@ -173,7 +175,7 @@ class ReduceScatterPlan:
             return ops.bind_quant_pack(source, codes, scales, group_size=self.config.group_size)
 
         self._order_after_previous_use()
-        bound = self._remember(("g", source.data_ptr(), source.dtype), make)
+        bound = self._remember(("g", source.data_ptr(), source.dtype, source.numel()), make)
         if self.chunks.shard_numel and not bound():
             raise ValueError(f"no HIP quantize kernel for dtype {source.dtype}")
         return row
@@ -202,7 +204,7 @@ class ReduceScatterPlan:
                                                  divisor=float(self.world_size) if op == "mean" else 1.0,
                                                  mid_dtype=self.reduced_dtype)
 
-        if not self._remember(("rq", rows.data_ptr(), op), make)():
+        if not self._remember(("rq", rows.data_ptr(), rows.numel(), op), make)():
             raise ValueError(f"no HIP reduce-requantize kernel for dtype {self.reduced_dtype}")
         return row
 
@@ -213,7 +215,7 @@ class ReduceScatterPlan:
         make = lambda: ops.bind_dequant_chunks(rows, target.reshape(-1), self.chunks.shard_numel,  # noqa: E731
                                                group_size=self.config.group_size)
         self._order_after_previous_use()
-        bound = self._remember(("d", rows.data_ptr(), target.data_ptr(), target.dtype), make) if out is not None else make()
+        bound = self._remember(("d", rows.data_ptr(), rows.numel(), target.data_ptr(), target.dtype, target.numel()), make) if out is not None else make()
         if self.numel and not bound():
             raise ValueError(f"no HIP decode kernel for dtype {target.dtype}")
         return target.reshape(self.shape)

@@ -99,6 +99,9 @@ def _divide(decoded: Any, count: int, *, in_place: bool, exact: bool = True) -> 
 def _trim_to_shape(decoded: Any, shape: tuple[int, ...]) -> Any:
     if not hasattr(decoded, "reshape"):
         return decoded
+    count = getattr(decoded, "numel", None)
+    if callable(count) and count() == prod(shape):          # nothing to trim: one view instead of three
+        return decoded.reshape(shape)
     flat = decoded.reshape((-1,))
     try:
         flat = flat[:prod(shape)]
@@ -204,8 +207,15 @@ def dequantize_reduce_tensors(buffers: list[object], shape: tuple[int, ...], con
     dtype_member = _dtype(module, dtype)
     fused = False
     if output is None:
-        decoded = _symbol(module, "dequantize_reduce")(buffers, config.group_size, config.topk, config.bit,
-                                                       quant_type, dtype_member, config.compact)
+        decoded = None
+        one_launch = getattr(module, "dequantize_reduce_mean", None) if reduce == "mean" else None
+        if one_launch is not None:      # an extension that divides in the reduce launch itself (same bits)
+            decoded = one_launch(buffers, config.group_size, config.topk, config.bit, quant_type, dtype_member,
+                                 config.compact, len(buffers))
+            fused = decoded is not None
+        if decoded is None:
+            decoded = _symbol(module, "dequantize_reduce")(buffers, config.group_size, config.topk, config.bit,
+                                                           quant_type, dtype_member, config.compact)
     else:
         if hasattr(module, "inplace_dequantize_reduce_mean"):
             fused = inplace_dequantize_reduce_mean(buffers, output, config, extension_status=extension_status,

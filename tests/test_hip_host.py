@@ -442,38 +442,53 @@ def test_asynchronous_shard_exchange_completes_through_the_pipeline(dev):
                                         plan=plans[0], async_op=True)
 
 
-def test_reduce_scatter_plan_keeps_few_bound_launches_and_orders_uses_across_streams(hip_device):
-    """A caller whose tensors are new every step must not pin them through the plan's cache of bound launches, a
+def test_reduce_scatter_plan_pins_no_caller_tensors_and_orders_uses_across_streams(hip_device):
+    """A caller whose tensors are new every step must not have them pinned by the plan's cache of bound launches, a
     residual of another dtype at a recycled address must not reuse a stale binding, and a use of the plan on
     another stream is ordered after the previous use."""
+    import weakref
+
+    from lowbit_comm_amd.hip import ops
     from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
 
     world, n = 4, 64 * 4 * 200
     config = CompressionConfig(error_feedback=False)
     plan = ReduceScatterPlan(n, torch.float32, world_size=world, rank=1, config=config, device=hip_device)
-    kept = [torch.randn(n, device=hip_device) * 1e-3 for _ in range(20)]
+    kept = [torch.randn(n, device=hip_device) * 1e-3 for _ in range(6)]
     for bucket in kept:
         plan.quantize_chunks(bucket)
-    assert len(plan._bound) <= ReduceScatterPlan._BOUND_LAUNCHES
-    assert kept[-1].data_ptr() in [key[1] for key in plan._bound] and kept[0].data_ptr() not in [key[1] for key in plan._bound]
+    assert len(plan._bound) == 6 <= ReduceScatterPlan._BOUND_LAUNCHES
+    again = plan._bound[next(iter(plan._bound))]
+    plan.quantize_chunks(kept[0])
+    assert plan._bound[("q", kept[0].data_ptr(), None, None)] is again and len(plan._bound) == 6   # bound once per address
+    fresh = torch.randn(n, device=hip_device)
+    alive = weakref.ref(fresh)
+    plan.quantize_chunks(fresh)
+    torch.cuda.synchronize()
+    del fresh
+    assert alive() is None                                      # the cache did not keep the caller's tensor
+    plan._BOUND_LAUNCHES = 4
+    recycled, elsewhere = torch.randn(n, device=hip_device), torch.randn(n, device=hip_device)
+    plan.quantize_chunks(recycled)                              # very likely the address `fresh` had: a hit
+    plan.quantize_chunks(elsewhere)                             # a new address for sure
+    assert len(plan._bound) == 4
 
     residual32 = torch.zeros(n, device=hip_device)
     residual16 = residual32.view(torch.bfloat16)[:n]            # same address, another dtype
     plan.quantize_chunks(kept[0], residual=residual32, new_residual=residual32)
-    keys = {key for key in plan._bound if key[0] == "q"}
-    plan.quantize_chunks(kept[0].bfloat16().float(), residual=residual32)
-    assert ("q", kept[0].data_ptr(), (residual32.data_ptr(), torch.float32), (residual32.data_ptr(), torch.float32)) in keys
-    assert residual16.data_ptr() == residual32.data_ptr()
-    assert ("q", kept[0].data_ptr(), (residual16.data_ptr(), torch.bfloat16), None) not in plan._bound
+    spec32 = (residual32.data_ptr(), torch.float32, n)
+    assert ("q", kept[0].data_ptr(), spec32, spec32) in plan._bound
+    with pytest.raises(RuntimeError):                           # no stale binding: bound anew, and refused (an fp32
+        plan.quantize_chunks(kept[0], residual=residual16, new_residual=residual16)   # sum needs an fp32 residual out)
 
     want = plan.quantize_chunks(kept[3]).clone()
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
         plan.quantize_chunks(kept[5])                           # the side stream now owns the plan's buffers
-    assert plan._last_stream == side
+    assert plan._last_stream_handle == side.cuda_stream
     got = plan.quantize_chunks(kept[3])                         # back on the default stream: ordered after the side stream
-    assert plan._last_stream == torch.cuda.current_stream()
+    assert plan._last_stream_handle == ops.current_stream_handle(hip_device)
     torch.cuda.synchronize()
     assert torch.equal(got, want)
 
