@@ -143,6 +143,57 @@ def test_facade_error_feedback_calls(status, dev):
             buffers, prepared, restored, residual[:-1], CFG, extension_status=status)
 
 
+def test_native_module_remembers_launches_by_address_without_pinning_or_going_stale(status, dev):
+    """From the second call with the same addresses on, an in-place entry point replays its bound launch.  The memo
+    must follow the data (same launch, new contents), must not keep tensors alive, and must not serve a call whose
+    tensors differ in anything the binding depends on."""
+    import weakref
+
+    module = status.module
+    linear = module.QuantType.Linear
+    n, world = 64 * 700, 4
+
+    def unpack(packed):
+        raw = packed.cpu()
+        return raw[:n].view(torch.int8), raw[n:].view(torch.float32)
+
+    x = grad(n, torch.float32, 31, dev)
+    payload = torch.empty(n // 64 * 68, dtype=torch.uint8, device=dev)
+    before = len(module._launches)
+    for seed in (32, 33, 34):                                   # same addresses, new contents every time
+        x.copy_(grad(n, torch.float32, seed, dev))
+        assert module.inplace_quantize_pack(x, payload, None, 64, 0, False, 8, linear, False)
+        assert torch.equal(payload.cpu(), oracle_packed(x.cpu()))
+    assert len(module._launches) == before + 1
+    peers = [codec.quantize_tensor(grad(n, torch.float32, 40 + r, dev), CFG, extension_status=status) for r in range(world)]
+    out = torch.empty(n, device=dev)
+    for _ in range(2):
+        assert module.inplace_dequantize_reduce_mean(peers, out, 64, 0, 8, linear, False, world)
+    want = codec_torch.reduce_payloads([unpack(p) for p in peers], n, 64, "fp32", "mean")
+    assert same_bits(out, want)
+    assert module.inplace_dequantize_reduce_mean(peers[::-1], out, 64, 0, 8, linear, False, world)   # another order: another key
+    want_reversed = codec_torch.reduce_payloads([unpack(p) for p in peers[::-1]], n, 64, "fp32", "mean")
+    assert same_bits(out, want_reversed)
+    assert module.inplace_dequantize_reduce_mean(peers, out, 64, 0, 8, linear, False, 1)             # another divisor
+    assert same_bits(out, codec_torch.reduce_payloads([unpack(p) for p in peers], n, 64, "fp32", "sum"))
+    # a tensor at a remembered address that is not what was bound: validated again, and refused
+    with pytest.raises(RuntimeError):
+        module.inplace_quantize_pack(x, payload.view(torch.int8), None, 64, 0, False, 8, linear, False)
+    strided = torch.empty(2 * payload.numel(), dtype=torch.uint8, device=dev)[::2]
+    with pytest.raises(RuntimeError):
+        module.inplace_quantize_pack(x, strided, None, 64, 0, False, 8, linear, False)
+    assert module.inplace_dequantize_reduce_mean([p[:-68] for p in peers], out, 64, 0, 8, linear, False, world) is False
+    # nothing is kept alive
+    fresh = grad(n, torch.float32, 50, dev)
+    alive = weakref.ref(fresh)
+    assert module.inplace_quantize_pack(fresh, payload, None, 64, 0, False, 8, linear, False)
+    torch.cuda.synchronize()
+    del fresh
+    assert alive() is None
+    limit = type(module)._LAUNCH_MEMO_ENTRIES
+    assert len(module._launches) <= limit
+
+
 def test_unsupported_policies_decline_instead_of_failing(status, dev):
     x = grad(1024, torch.float32, 3, dev)
     out = torch.empty(1024 // 64 * 68, dtype=torch.uint8, device=dev)
