@@ -276,6 +276,10 @@ __device__ __forceinline__ uint32_t group_absmax_bits(const float (&p)[VEC]) {
     return group_max_bits<LPG>(m);
 }
 
+// (For a pure 16-bit tensor the lane's maximum could be taken on pairs of 16-bit magnitudes before widening,
+// v_pk_max_u16, half the instructions of this loop.  Measured: 2 % slower at every size, 26 M bf16 elements 14.7
+// against 14.4 us - the kernel waits on memory, and the packed chain is longer.  Not used.)
+
 // Scale of that group.
 template <int VEC, int LPG>
 __device__ __forceinline__ float group_scale(const float (&p)[VEC]) {
@@ -339,17 +343,28 @@ constexpr float kCodeMagic = 12582912.0f;   // 1.5 * 2^23
 
 __device__ __forceinline__ float code_value(int code_bits) { return as_f32(static_cast<uint32_t>(code_bits)) - kCodeMagic; }
 
+// Inf or NaN scale: every code of the group is 0.
+__device__ __forceinline__ bool scale_not_finite(float scale) { return (as_u32(scale) & 0x7F800000u) == 0x7F800000u; }
+
+// The codes of a group whose scale is finite; for any other scale the caller must discard them (encode_group
+// does it per element; a caller that only packs them can zero whole words instead, one select per four codes).
 // `y` is the correctly rounded reciprocal of `scale` (an IEEE division 1/scale).
 template <int N>
-__device__ __forceinline__ void encode_group(const float (&p)[N], float scale, float y, int (&codes)[N]) {
-    const bool no_codes = (as_u32(scale) & 0x7F800000u) == 0x7F800000u;   // Inf or NaN scale: one compare per lane
+__device__ __forceinline__ void encode_group_finite(const float (&p)[N], float scale, float y, int (&codes)[N]) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         const float q0 = p[i] * y;
         const float r = __builtin_fmaf(-q0, scale, p[i]);
-        const float t = __builtin_fmaf(r, y, q0) + kCodeMagic;
-        codes[i] = static_cast<int>(as_u32(no_codes ? kCodeMagic : t));
+        codes[i] = static_cast<int>(as_u32(__builtin_fmaf(r, y, q0) + kCodeMagic));
     }
+}
+
+template <int N>
+__device__ __forceinline__ void encode_group(const float (&p)[N], float scale, float y, int (&codes)[N]) {
+    const bool no_codes = scale_not_finite(scale);   // one compare per lane
+    encode_group_finite<N>(p, scale, y, codes);
+#pragma unroll
+    for (int i = 0; i < N; ++i) codes[i] = no_codes ? static_cast<int>(as_u32(kCodeMagic)) : codes[i];
 }
 
 template <int N>

@@ -137,11 +137,15 @@ __device__ __forceinline__ void quant_pack_block(const QuantArgs &a, unsigned bl
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             int c[VEC];
-            encode_group<VEC>(p[u], scale[u], recip[u], c);
+            const bool no_codes = scale_not_finite(scale[u]);     // then every code of the group is 0
+            encode_group_finite<VEC>(p[u], scale[u], recip[u], c);
 
             uint32_t words[VEC / 4];
 #pragma unroll
-            for (int k = 0; k < VEC / 4; ++k) words[k] = pack4(c[4 * k], c[4 * k + 1], c[4 * k + 2], c[4 * k + 3]);
+            for (int k = 0; k < VEC / 4; ++k) {                   // one select per packed word, not per code
+                const uint32_t word = pack4(c[4 * k], c[4 * k + 1], c[4 * k + 2], c[4 * k + 3]);
+                words[k] = no_codes ? 0u : word;
+            }
             buffer_store<uint32_t, VEC / 4, kCodeStore>(codes_b, at[u], words);
 
             if (new_r != nullptr || restored != nullptr) {
@@ -149,7 +153,8 @@ __device__ __forceinline__ void quant_pack_block(const QuantArgs &a, unsigned bl
                 NT diff_out[VEC];
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
-                    const float rest = round_through<DT>(code_value(c[i]) * scale[u]);
+                    const float code = no_codes ? 0.0f : code_value(c[i]);
+                    const float rest = round_through<DT>(code * scale[u]);
                     rest_out[i] = narrow<DT>(rest);
                     diff_out[i] = narrow<NT>(p[u][i] - rest);
                 }

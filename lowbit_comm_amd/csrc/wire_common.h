@@ -53,6 +53,45 @@ __device__ __forceinline__ void store_elems(T *p, const T (&src)[VEC]) {
     else *reinterpret_cast<V *>(p) = v;
 }
 
+// Compact 16-bit payloads have a group pitch of 66 bytes (64 codes, a 2-byte scale), so a lane's 8 code bytes
+// start at an address that is only 2-byte aligned, and a misaligned 8-byte access runs at a fraction of the
+// aligned rate.  This reads the aligned 12-byte window that contains them instead and shifts the piece out:
+// at == 0 mod 4: window [at, at + 12); at == 2 mod 4: window [at - 2, at + 10).  `after` receives the two bytes
+// that follow the piece - for the lane that owns the last piece of a group, the group's scale - so the scales
+// need no loads of their own.  `b` covers the payload from a 4-byte aligned address on, up to window_span() of
+// its last byte, and `at` is relative to it.  The span is rounded up to whole dwords because the hardware drops a
+// dword that is only partly inside a buffer, and the last dword of an odd number of groups holds the last scale;
+// the two bytes read past the payload share an aligned dword, hence a page, with that scale.  Whole dwords past
+// the span read as zero (only ever the unused tail of a window).
+__device__ __forceinline__ uint32_t window_span(uint32_t bytes) { return (bytes + 3u) & ~3u; }
+
+template <int POLICY>
+__device__ __forceinline__ void load_piece16(buffer_t b, uint32_t at, uint32_t (&words)[2], uint32_t &after) {
+    const uint32_t odd = at & 2u;
+    const vec_t<uint32_t, 3> w = __builtin_amdgcn_raw_buffer_load_b96(b, at - odd, 0, POLICY);
+    const uint32_t shift = odd * 8u;
+    words[0] = __builtin_amdgcn_alignbit(w[1], w[0], shift);
+    words[1] = __builtin_amdgcn_alignbit(w[2], w[1], shift);
+    after = odd ? w[2] >> 16 : w[2] & 0xFFFFu;
+}
+
+// Cache policy of those windows.  Measured on the W=8 reduce of 26.2 M bf16 elements: windows 45.9 us with the
+// non-temporal hint, 47.6 us without, against 50.0 us for misaligned 8-byte loads plus a 2-byte load per scale
+// (and 55.9 us when the runs are staged through LDS with aligned 16-byte loads: the barrier costs more than the
+// misalignment).  Few payloads: the output dominates and cached payload loads are the faster ones, as in the
+// other layouts.
+template <int NT, int WORLD> constexpr int window_policy() { return NT == kNonTemporal && WORLD >= 4 ? kNtBit : kCached; }
+
+// (Stores to such positions stay misaligned 8-byte stores: splitting them into short, aligned dword, short
+// made the ring's gather hop 30 % slower, 56.5 against 43.0 us on 52 M bf16 elements.)
+
+// The value lane 7 (lanes 0-7) or lane 15 (lanes 8-15) of the caller's row holds: the last lane of an 8-lane group.
+__device__ __forceinline__ uint32_t from_last_lane_of_8(uint32_t v, bool upper_half) {
+    const uint32_t low = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x150 + 7, 0xF, 0xF, true));
+    const uint32_t high = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x150 + 15, 0xF, 0xF, true));
+    return upper_half ? high : low;
+}
+
 template <typename T, int BIT = 8> struct wire {
     static constexpr int ITEM = sizeof(T);
     static constexpr int VEC = 16 / ITEM;                  // elements per lane: 16 bytes of the tensor

@@ -174,6 +174,34 @@ def test_fused_reduce_and_error_feedback(hip, hip_device, access, name, compact,
         same(alias, want_residual, f"aliased residual n={n}")
 
 
+@pytest.mark.parametrize("name", ("fp16", "bf16"))
+@pytest.mark.parametrize("world", (2, 3, 8))
+def test_fused_reduce_of_interleaved_16_bit_payloads_at_any_2_byte_alignment(hip, hip_device, access, name, world):
+    """Payloads of 66-byte groups are read through aligned 12-byte windows with the scales taken out of the windows;
+    a payload may start at any 2-byte aligned address, and the blocks of the fast path reach the payload's last
+    group when the element count is a multiple of theirs."""
+    for n, lead in ((2048 * 5, 0), (2048 * 5, 2), (4096 * 3, 6), (2048 * 4 + 64 * 3, 2), (100_003, 10)):
+        grads = [make(n, name, 900 + 10 * world + r, hip_device, sigma=10.0 ** (r % 3 - 2)) for r in range(world)]
+        packed = [hip.quant_pack(g_, compact=True) for g_ in grads]
+        holders = [torch.zeros(p.numel() + 32, dtype=torch.uint8, device=hip_device) for p in packed]
+        payloads = []
+        for holder, p in zip(holders, packed):
+            holder[lead:lead + p.numel()].copy_(p)
+            holder[lead + p.numel():].fill_(0xA5)              # whatever follows a payload must not matter
+            payloads.append(holder[lead:lead + p.numel()])
+        host = [to_numpy(p) for p in packed]
+        inv = float(np.float32(1.0) / np.float32(world))
+        out = torch.empty(n, dtype=NAMES[name], device=hip_device)
+        assert hip.dequant_reduce_into(payloads, out, compact=True, inv_divisor=inv, fused_multiply_add=False)
+        same(out, wire.reduce_payloads(host, n, name, 64, True, inv, False), f"reduce n={n} lead={lead}")
+        prepared = make(n, name, 950 + world, hip_device)
+        residual = torch.empty_like(prepared)
+        assert hip.dequant_reduce_into(payloads, out, compact=True, inv_divisor=inv, prepared=prepared, new_residual=residual)
+        want_restored, want_residual = wire.reduce_mean_error_feedback(host, to_numpy(prepared), n, name, 64, True, world, True)
+        same(out, want_restored, f"restored n={n} lead={lead}")
+        same(residual, want_residual, f"residual n={n} lead={lead}")
+
+
 def test_reduce_rejections(hip, hip_device):
     x = make(640, "fp16", 1, hip_device)
     payload = hip.quant_pack(x)

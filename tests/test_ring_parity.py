@@ -577,12 +577,16 @@ def test_ring_steps_captured_in_a_hip_graph_replay_like_eager(hip_device):
 # --------------------------------------------------------------------------- #
 # the same hop in the CUDA extension's byte format
 # --------------------------------------------------------------------------- #
-def check_wire_step(device, dtype, g, n, compact, reduce_op, divisor, emit, seed, poison=False):
+def check_wire_step(device, dtype, g, n, compact, reduce_op, divisor, emit, seed, poison=False, lead=0):
     from lowbit_comm_amd.hip import cuda_wire
 
     tdtype = DTYPES[dtype]
     incoming = tensor_like(n, dtype, seed, device)
     received = cuda_wire.quant_pack(incoming, group_size=g, compact=compact)
+    if lead:                                      # the payload at a 2-byte aligned address, other bytes after it
+        holder = torch.full((received.numel() + lead + 16,), 0x5A, dtype=torch.uint8, device=device)
+        holder[lead:lead + received.numel()].copy_(received)
+        received = holder[lead:lead + received.numel()]
     chunk = tensor_like(n, dtype, seed + 1, device, sigma=3e-3)
     if poison and n >= 4 * g:
         chunk[g + 3] = float("nan")               # a NaN inside a group: the running maximum restarts after it
@@ -613,6 +617,12 @@ def test_wire_ring_step_bit_exact(hip_device, dtype, compact):
                     check_wire_step(hip_device, dtype, g, n, compact, reduce_op, divisor, emit, seed)
     check_wire_step(hip_device, dtype, 64, 64 * 40, compact, "sum", 1.0, True, 79_001, poison=True)
     check_wire_step(hip_device, dtype, 16, 16 * 64, compact, "none", 1.0, True, 79_003, poison=False)
+    if dtype != "fp32":                            # 66-byte groups: every parity of address and of group count
+        for n in (64, 64 * 2, 64 * 3, 64 * 33, 64 * 4096 // 16 + 64):
+            for lead in (2, 4, 6):
+                for reduce_op in ("none", "sum"):
+                    seed += 2
+                    check_wire_step(hip_device, dtype, 64, n, compact, reduce_op, 1.0, True, seed, lead=lead)
 
 
 def test_wire_ring_step_equals_the_separate_launches_and_checks_its_arguments(hip_device):
