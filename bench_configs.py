@@ -1049,9 +1049,10 @@ def main() -> int:
             return Arrived()
 
         buckets = [gen(SEED + 8400 + k, n, 1e-3) for k in range(3)]
-        for fused, graphed in ((True, False), (True, True), (False, False)):
+        for fused, graphed, inline in ((True, False, False), (True, False, True), (True, True, False), (False, False, False)):
             executor = make_pipelined_ring_executor(config=cfg, dtype="fp32", numel=n, world_size=world, rank=3,
-                                                    exchange=exchange, fuse_steps=fused, graph_replay=graphed)
+                                                    exchange=exchange, fuse_steps=fused, graph_replay=graphed,
+                                                    stream=stream if inline else None)
 
             def whole(i, executor=executor):
                 executor.run(buckets[i % 3]).wait()
@@ -1076,6 +1077,7 @@ def main() -> int:
                 nbytes = 14 * (chunk_bytes + pay) + 7 * (pay + 2 * chunk_bytes) + 2 * chunk_bytes + 7 * (pay + chunk_bytes)
             emit(8, f"one rank's ring schedule, W=8, 200 MiB fp32 bucket, {'fused ring steps' if fused else 'separate launches'}"
                     f"{', replayed as one HIP graph' if graphed else ''}"
+                    + (", on the caller's own stream" if inline else "") +
                     f" (14 hops through the executor, payloads of a peer already in the receive buffers; host "
                     f"{host * 1e6:.0f} us per bucket)", nbytes, seconds, n * 4, None)
         del buckets

@@ -541,7 +541,10 @@ class HipPipelinedRingRuntime:
             raise RuntimeError("the ring runs in place on a contiguous GPU tensor")
         if ops.DTYPE_NAMES.get(tensor.dtype) != self.dtype:
             raise RuntimeError(f"tensor dtype {tensor.dtype} does not match the runtime's {self.dtype}")
-        produced = self._completions.record_for(tensor, stream=torch.cuda.current_stream(tensor.device))
+        from lowbit_comm_amd.hip.workspace import StreamOrderedCompletion
+
+        # The producer's work so far: no event unless the ring runs on another stream than the producer.
+        produced = StreamOrderedCompletion(torch.cuda.current_stream(tensor.device))
         plan = self._plan_of(tensor)
         recording = plan is not None and "program" not in plan and not self._facade
         return RingSubmissionContext(tensor=tensor, stream=self.stream, producer_completion=produced,
@@ -606,6 +609,12 @@ class HipPipelinedRingRuntime:
             wait_stream = getattr(dependency, "wait_stream", None)
             if callable(wait_stream):
                 wait_stream(context.stream)
+        import torch
+
+        from lowbit_comm_amd.hip.workspace import StreamOrderedCompletion
+
+        if context.stream == torch.cuda.current_stream(context.tensor.device):
+            return StreamOrderedCompletion(context.stream)     # the caller's own stream: its order is the completion
         return self._completions.record_for(context.tensor, stream=context.stream)
 
     # ---- buffers ----------------------------------------------------------- #
@@ -875,8 +884,13 @@ def make_pipelined_ring_executor(*, config: CompressionConfig, dtype: str, numel
                                  exchange: Callable[..., Any], pool: Any | None = None,
                                  completion_manager: Any | None = None, device: str = "cuda:0",
                                  fuse_steps: bool = True, max_plans: int = 16,
-                                 extension_status: Any | None = None, graph_replay: bool = False) -> PipelinedRingExecutor:
-    """Plan, schedule, runtime, pooled workspaces and executor of one rank for buckets of ``numel`` elements."""
+                                 extension_status: Any | None = None, graph_replay: bool = False,
+                                 stream: Any | None = None) -> PipelinedRingExecutor:
+    """Plan, schedule, runtime, pooled workspaces and executor of one rank for buckets of ``numel`` elements.
+
+    ``stream``: the stream the ring's launches go to.  ``None`` gives the runtime a stream of its own, which lets
+    the ring overlap with the caller's compute at the price of an event hand-off in each direction per bucket;
+    the caller's own stream (``torch.cuda.current_stream()``) makes a bucket's ring plain stream-ordered work."""
     from lowbit_comm_amd.hip.completion import HipCompletionManager
     from lowbit_comm_amd.hip.workspace import ShardWorkspaceProvider, create_torch_workspace_pool
 
@@ -885,7 +899,7 @@ def make_pipelined_ring_executor(*, config: CompressionConfig, dtype: str, numel
     schedule = compile_pipelined_ring_schedule(chunk_plan=plan, rank=rank)
     runtime = HipPipelinedRingRuntime(config=config, dtype=dtype, world_size=world_size, rank=rank, exchange=exchange,
                                       completion_manager=manager, fuse_steps=fuse_steps, max_plans=max_plans,
-                                      extension_status=extension_status, graph_replay=graph_replay)
+                                      extension_status=extension_status, graph_replay=graph_replay, stream=stream)
     provider = ShardWorkspaceProvider(pool if pool is not None else create_torch_workspace_pool(), backend="hip",
                                       collective="all_reduce", strategy="pipelined_ring", device=device)
 
