@@ -42,7 +42,7 @@ WORLD = 8
 GROUP = 64
 SEED = 1234
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-KERNEL_SOURCES = ("quant_pack.hip", "device_utils.h", "launch.h", "lbc_api.hip")   # what the dominant kernel is built from
+KERNEL_SOURCES = ("quant_pack.hip", "quant_pack_block.h", "device_utils.h", "launch.h", "lbc_api.hip")   # what the dominant kernel is built from
 SHARD_SETS = 16            # payload sets of the shard-reduce leg: 16 x 41 MB
 
 
