@@ -104,7 +104,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     Raw raw[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) raw[i] = 0;
-    if (live) load_elems<Raw, VEC, kPlain>(static_cast<const Raw *>(a.x) + e0, raw);
+    if (live) load_elems<Raw, VEC, kPlain>(static_cast<const Raw *>(a.x) + e0, raw);   // instruction-bound: the hint only costs
     const float *book = wave_code_book(a.kind, lane);   // after the loads were issued: its wait covers theirs
     float v[VEC];
     uint32_t mag[VEC];
@@ -328,7 +328,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
     Raw *out = static_cast<Raw *>(a.out) + e0;
     if (a.op != 0) {
         Raw old[VEC];
-        load_elems<Raw, VEC, kPlain>(out, old);
+        load_elems<Raw, VEC, kNonTemporal>(out, old);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const float o = value_of<T>(old[i]), d = value_of<T>(decoded[i]);
@@ -337,7 +337,9 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
             else decoded[i] = o > d ? decoded[i] : old[i];
         }
     }
-    store_elems<Raw, VEC, kPlain>(out, decoded);
+    // The decoded tensor is the large stream of this kernel and nothing here reads it again: with the non-temporal
+    // hint the decode of 26.2 M fp32 elements takes 19.9 instead of 30.2 us (top-2), 18.0 instead of 31.1 us (code book).
+    store_elems<Raw, VEC, kNonTemporal>(out, decoded);
 }
 
 template <typename T, int G>

@@ -587,6 +587,11 @@ int lbc_wire_quant_general(const void *x, int dtype, int64_t numel, int group_si
     if (x == nullptr || payload == nullptr) return fail(LBC_EINVAL, "input and payload must not be null");
     if (!aligned_to(x, item) || !aligned_to(payload, item))
         return fail(LBC_EINVAL, "input/payload must be aligned to the element size");
+    // Plain linear codes without outliers or noise are what the dedicated pack kernel writes (with the NaN rule of
+    // the general kernels for a call without a residual): same bytes, a memory-bound kernel instead of this
+    // instruction-bound one.
+    if (quant_type == 0 && topk == 0 && stochastic == 0)
+        return lbc_wire_quant_pack(x, nullptr, dtype, numel, group_size, bit, compact, payload, LBC_ACCESS_AUTO, stream);
     lbc::WireGeneralQuantArgs a{};
     a.x = x;
     a.payload = payload;
@@ -614,6 +619,10 @@ int lbc_wire_dequant_general(const uint8_t *payload, int64_t numel, int group_si
     if (payload == nullptr || out == nullptr) return fail(LBC_EINVAL, "payload and out must not be null");
     if (!aligned_to(payload, item) || !aligned_to(out, item))
         return fail(LBC_EINVAL, "payload/out must be aligned to the element size");
+    // Linear codes without an outlier channel decode the same way however they were rounded: the dedicated decode
+    // kernel reads the same bytes at the memory-bound rate.
+    if (quant_type == 0 && topk == 0)
+        return lbc_wire_dequant(payload, numel, group_size, bit, compact, out, dtype, reduce_op, LBC_ACCESS_AUTO, stream);
     lbc::WireGeneralDecodeArgs a{};
     a.payload = payload;
     a.out = out;
