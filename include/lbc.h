@@ -327,13 +327,16 @@ int64_t lbc_wire_general_payload_nbytes(int64_t numel, int group_size, int dtype
  * quant_kernel_fp32.cuh:211-455 and quant_kernel.cuh:155-399).  With stochastic != 0, seed and offset are
  * the Philox key and offset the reference takes from torch's CUDA generator
  * (gen_code_quant.py:27-36: philox_engine_inputs(numel)); group s draws from subsequence s.
+ * A policy with nothing general about it (linear codes, topk 0, no stochastic rounding) is handed to the
+ * kernel of lbc_wire_quant_pack, which writes the same bytes at the memory-bound rate.
  */
 int lbc_wire_quant_general(const void *x, int dtype, int64_t numel, int group_size, int bit, int quant_type,
                            int topk, int stochastic, uint64_t seed, uint64_t offset, int compact,
                            uint8_t *payload, void *stream);
 
 /* Replaces native dequantize / inplace_dequantize for those policies (dequant_kernel_fp32.cuh:122-353,
- * dequant_kernel.cuh:62-291); reduce_op as in lbc_wire_dequant. */
+ * dequant_kernel.cuh:62-291); reduce_op as in lbc_wire_dequant.  Linear codes without an outlier channel
+ * (however they were rounded) are decoded by the kernel of lbc_wire_dequant. */
 int lbc_wire_dequant_general(const uint8_t *payload, int64_t numel, int group_size, int bit, int quant_type,
                              int topk, int compact, void *out, int dtype, int reduce_op, void *stream);
 
