@@ -235,21 +235,57 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
             c[i] = r < -L ? -L : (r > L ? L : r);
         }
     } else {
+        // t = v / scale, the IEEE quotient.  A lane's elements share the divisor, so the reciprocal part of the
+        // division is done once: v_rcp_f32 and one Newton step, then per element the product and two corrections.
+        // These are the very operations the compiler emits for `v / scale`, minus its operand scaling and
+        // special-case fix-up (v_div_scale / v_div_fmas / v_div_fixup), which change nothing while the divisor
+        // lies in [2^-60, 2^60], |v| <= scale, and the dividend is not so small (below 2^-103) that the division
+        // would rescale it.  The scale is at least 1e-6 here, so such a dividend means a quotient below 2^-80, and a
+        // quotient below 2^-30 encodes as the book's zero whatever its last bits are: it is closer to that entry
+        // than the rounding error of the comparisons with its neighbours.  A wavefront with any other divisor,
+        // or with an element above its scale (only a group that holds a NaN has one) or not a number, takes the
+        // division.  tests/native/quotient_check.hip compares the two forms on the device.
+        float t[VEC];
+        const uint32_t scale_exponent = (as_u32(scale) >> 23) & 0xFFu;
+        bool unusual = scale_exponent < 127u - 60u || scale_exponent > 127u + 60u;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) unusual |= !(__builtin_fabsf(v[i]) <= scale);
+        if (__ballot(unusual) == 0) {   // wavefront-uniform
+            float reciprocal = __builtin_amdgcn_rcpf(scale);
+            reciprocal = __builtin_fmaf(__builtin_fmaf(-scale, reciprocal, 1.0f), reciprocal, reciprocal);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                float q = v[i] * reciprocal;
+                q = __builtin_fmaf(__builtin_fmaf(-scale, q, v[i]), reciprocal, q);
+                t[i] = __builtin_fmaf(__builtin_fmaf(-scale, q, v[i]), reciprocal, q);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) t[i] = v[i] / scale;
+        }
+        // The largest entry in [0, 14] with not (t < book[entry]); a NaN ends at 14.  Four halving steps, each
+        // over all of the lane's elements so that their LDS reads are in flight together; positions are kept as
+        // byte offsets into the book.
+        const char *book_bytes = reinterpret_cast<const char *>(book);
+        int at[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) at[i] = 0;
+#pragma unroll
+        for (int step = 8 * 4; step >= 4; step >>= 1) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                const int mid = at[i] + step;
+                const float entry = *reinterpret_cast<const float *>(book_bytes + mid);
+                at[i] = (mid < 15 * 4 && !(t[i] < entry)) ? mid : at[i];
+            }
+        }
         float excess[VEC], gap[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
-            const float t = v[i] / scale;
-            int lower = 0;   // the largest entry in [0, 14] with not (t < book[entry]); NaN ends at 14
-#pragma unroll
-            for (int step = 8; step >= 1; step >>= 1) {
-                const int mid = lower + step;
-                const float entry = book[mid];
-                if (mid < 15 && !(t < entry)) lower = mid;
-            }
-            const float low = book[lower];
-            gap[i] = book[lower + 1] - low;
-            excess[i] = t - low;
-            c[i] = lower;
+            const float low = *reinterpret_cast<const float *>(book_bytes + at[i]);
+            gap[i] = *reinterpret_cast<const float *>(book_bytes + at[i] + 4) - low;
+            excess[i] = t[i] - low;
+            c[i] = at[i] >> 2;
         }
         if (a.stochastic) {   // uniform: the second division only runs when it is needed
 #pragma unroll

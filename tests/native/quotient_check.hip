@@ -15,6 +15,16 @@
 // half-integers k + 0.5 in (-128, 128) and the 13 dividends within six ulps of RN((k + 0.5) * s): every case in
 // which the refined quotient could change a code.
 //
+// Mode 7 is the other division-free quotient of the library (csrc/cuda_wire_general.hip, code-book quantizer):
+// the compiler's own expansion of v / s - v_rcp_f32, a Newton step, product, two corrections - with the reciprocal
+// part shared by the elements that have the same divisor and without the operand scaling and fix-up instructions,
+// for divisors in [2^-60, 2^60] and |v| <= s.  It must equal v / s bit for bit for every quotient of 2^-40 and
+// above.  Below that the caller does not look at the bits: such a quotient lies between the code book's zero and
+// its neighbours by less than their rounding error, so it encodes as the zero entry whatever its last bits are -
+// and that is where the two forms do differ, for dividends so small (below 2^-103) that the hardware division
+// rescales them first.  Sampled over random divisors and dividends of every magnitude down to the denormals,
+// 4.3e9 pairs a round.
+//
 // Usage: quotient_check [rounds per sampled mode, 4.3e9 pairs each; 0 skips them] [exhaustive 0|1, default 1].
 // Exit status 1 when a code differs or a quotient differs for |p/s| >= 2^-64; below that the exact remainder
 // fma(-q0, s, p) can underflow and lose its last bits, the code is 0 either way, and such pairs are only counted.
@@ -50,6 +60,34 @@ __global__ void check_all_ties(uint32_t sexp, unsigned long long *bad, float *ex
         for (int ulps = -6; ulps <= 6; ++ulps) {
             const float p = __uint_as_float(__float_as_uint(base) + ulps);
             if (fabsf(p) <= 127.5f * s) compare(p, s, t, ex);
+        }
+    }
+    publish(t, bad);
+}
+__global__ void check_shared_reciprocal(uint64_t seed, unsigned long long *bad, float *ex) {
+    uint64_t id = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    Tally t = {0, 0, 0};
+    for (int it = 0; it < 1024; ++it) {
+        uint64_t h = seed * 0x9E3779B97F4A7C15ULL + id * 1024 + it;
+        uint32_t a = mix(h), b = mix(h ^ 0xDEADBEEFCAFEULL);
+        const float s = __uint_as_float(((67u + a % 121u) << 23) | (b & 0x7FFFFF));      // 2^-60 .. 2^60
+        float r = __builtin_amdgcn_rcpf(s);
+        r = __builtin_fmaf(__builtin_fmaf(-s, r, 1.0f), r, r);
+        for (int e = 0; e < 4; ++e) {                                                    // four dividends a divisor
+            uint32_t c = mix(h + 0x1234567ULL * (e + 1));
+            float v;
+            if (e == 0) v = s * (((float)(c & 0xFFFFFF) / 16777216.0f) * 2.0f - 1.0f);   // anywhere in [-s, s]
+            else if (e == 1) v = __uint_as_float(__float_as_uint(s) - (c & 0xFFFF));      // just below s
+            else if (e == 2) v = __uint_as_float(c & 0x7FFFFFFF);                         // any exponent
+            else v = __uint_as_float((__float_as_uint(s) & 0x7F800000u) - ((c % 90) << 23) | (c & 0x7FFFFF)); // scaled down
+            if (!(fabsf(v) <= s)) continue;
+            float q = v * r;
+            q = __builtin_fmaf(__builtin_fmaf(-s, q, v), r, q);
+            q = __builtin_fmaf(__builtin_fmaf(-s, q, v), r, q);
+            const float want = v / s;
+            if (__float_as_uint(q) != __float_as_uint(want)) {
+                if (fabsf(want) < 0x1p-40f) ++t.tiny; else { ++t.quotient; ex[0] = v; ex[1] = s; }
+            }
         }
     }
     publish(t, bad);
@@ -94,12 +132,15 @@ int main(int argc, char **argv) {
     unsigned long long *bad; float *ex;
     if (hipMalloc(&bad, 24) != hipSuccess || hipMalloc(&ex, 8) != hipSuccess) return 2;
     unsigned long long failures = 0;
-    for (int mode = 0; mode <= 6; ++mode) {
-        if (mode < 6 ? rounds == 0 : !exhaustive) continue;
+    for (int mode = 0; mode <= 7; ++mode) {
+        if (mode == 6 ? !exhaustive : rounds == 0) continue;
         if (hipMemset(bad, 0, 24) != hipSuccess || hipMemset(ex, 0, 8) != hipSuccess) return 2;
         unsigned long long n;
         if (mode < 6) {
             for (int r = 0; r < rounds; ++r) hipLaunchKernelGGL(check, dim3(4096), dim3(256), 0, 0, (uint64_t)(mode * 1000 + r + 1), mode, bad, ex);
+            n = (unsigned long long)rounds * 4096ULL * 256ULL * 4096ULL;
+        } else if (mode == 7) {
+            for (int r = 0; r < rounds; ++r) hipLaunchKernelGGL(check_shared_reciprocal, dim3(4096), dim3(256), 0, 0, (uint64_t)(7000 + r), bad, ex);
             n = (unsigned long long)rounds * 4096ULL * 256ULL * 4096ULL;
         } else {
             const uint32_t exponents[3] = {127, 104, 247};      // 1, the smallest scale, the largest the domain holds
@@ -109,7 +150,7 @@ int main(int argc, char **argv) {
         unsigned long long h[3]; float he[2];
         if (hipDeviceSynchronize() != hipSuccess || hipMemcpy(h, bad, 24, hipMemcpyDeviceToHost) != hipSuccess ||
             hipMemcpy(he, ex, 8, hipMemcpyDeviceToHost) != hipSuccess) return 2;
-        printf("mode %d: %llu pairs, quotient mismatches %llu (and %llu below 2^-64), code mismatches %llu (example p=%a s=%a)\n",
+        printf("mode %d: %llu pairs, quotient mismatches %llu (and %llu too small to matter), code mismatches %llu (example p=%a s=%a)\n",
                mode, n, h[1], h[0], h[2], he[0], he[1]);
         failures += h[1] + h[2];
     }

@@ -31,10 +31,11 @@ def test_exact_quotient_without_a_division_matches_the_division_on_billions_of_p
     """tests/native/quotient_check.hip: the encode's FMA-refined quotient against ``p / s`` on the device.  4.3e9
     pairs in each of six sampled modes (random, extreme scale mantissas, quotients next to ties, 16-bit dividends)
     with scale exponents over the whole domain, and the exhaustive walk over every scale mantissa and every dividend
-    next to a half-integer multiple of the scale, the only pairs whose code the refinement could change."""
+    next to a half-integer multiple of the scale, the only pairs whose code the refinement could change; and the
+    code-book quantizer's division with a shared reciprocal against the division, bit for bit."""
     checker = ROOT / "tests" / "native" / "_build" / "quotient_check"
     assert checker.exists(), "run __graft_entry__.build() first"
     done = subprocess.run([str(checker), "1", "1"], capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stdout[-2000:]
     assert "MISMATCHES 0" in done.stdout.splitlines()[-1]
-    assert done.stdout.count("code mismatches 0") == 7 and done.stdout.count("quotient mismatches 0 ") == 7
+    assert done.stdout.count("code mismatches 0") == 8 and done.stdout.count("quotient mismatches 0 ") == 8
