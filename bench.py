@@ -3,21 +3,23 @@
 
 One "step" pushes one 100 MiB fp32 gradient bucket through the compressed reduce-scatter hot path
 of one rank at simulated world size 8 (the "config 2" workload): quantize+pack the bucket's 8 destination
-chunks (one launch), then the fused dequant-reduce of the 8 peer payloads of this rank's shard in
-fixed rank order (one launch).  Peer payloads are synthesised in HBM before the timed region; there
-are no collectives.  `value` is GB/s of gradient input consumed per step.
+chunks, and the fused dequant-reduce of the 8 peer payloads of this rank's shard in fixed rank order.
+In a stream of buckets the reduce that is ready when bucket k is quantized belongs to bucket k-1, and the
+library carries the two in one launch (lbc_quant_pack_chunks_and_dequant_reduce): that launch is the step,
+with the quantize on one buffer set and the reduce on the previous one.  `ms_per_step_two_launches` is the same
+work as two launches.  Peer payloads are synthesised in HBM before the timed region; there are no collectives.
+`value` is GB/s of gradient input consumed per step.
 
-The line also carries, for the dominant kernel (quantize+pack of the 100 MiB bucket), the HBM
-roofline: algorithmic bytes per launch / average launch duration measured with HIP events around
-back-to-back launches on the launch stream; and a CPU baseline: the torch-op restatement of the
-reference codec timed on this host for the same step.  `kernels` adds the same roofline figures for
-the other kernels of the path (shard reduce, full-bucket all-gather-reduce shape, EF quantize); every
-leg rotates through more than 600 MB of buffers, so none of them is served by the 256 MiB memory-side
-cache.
+The line also carries, for the kernel of the step, the HBM roofline: algorithmic bytes per launch / average
+launch duration measured with HIP events around back-to-back launches on the launch stream; and a CPU
+baseline: the torch-op restatement of the reference codec timed on this host for the same step.  `kernels`
+adds the same roofline figures for the kernels of the path launched on their own (quantize+pack of the bucket,
+shard reduce, full-bucket all-gather-reduce shape, EF quantize); every leg rotates through more than 600 MB of
+buffers, so none of them is served by the 256 MiB memory-side cache.
 
-`roofline.traffic` (HBM bytes per launch of the dominant kernel) is not measured by this run: it comes
+`roofline.traffic` (HBM bytes per launch of that kernel) is not measured by this run: it comes
 from profiles/hbm_traffic.json, which `--record-traffic` writes from two rocprofv3 counter runs
-(FETCH_SIZE, WRITE_SIZE) of `bench.py --only quant_pack_chunks,copy_calibration`, each counter scaled by
+(FETCH_SIZE, WRITE_SIZE) of `bench.py --only step,copy_calibration`, each counter scaled by
 what it reads for the plain 100 MiB device copy of the same run.  The file remembers a hash of the kernel
 sources it was measured on; when they have changed since, `traffic` is null rather than stale.
 
@@ -42,7 +44,8 @@ WORLD = 8
 GROUP = 64
 SEED = 1234
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-KERNEL_SOURCES = ("quant_pack.hip", "quant_pack_block.h", "device_utils.h", "launch.h", "lbc_api.hip")   # what the dominant kernel is built from
+# what the kernel of the step is built from
+KERNEL_SOURCES = ("bucket_step.hip", "quant_pack_block.h", "dequant_reduce_block.h", "device_utils.h", "launch.h", "lbc_api.hip")
 SHARD_SETS = 16            # payload sets of the shard-reduce leg: 16 x 41 MB
 
 
@@ -65,7 +68,7 @@ def recorded_traffic():
         return None, "profiles/hbm_traffic.json is missing"
     if record.get("kernel_sources_sha256_16") != kernel_sources_hash():
         return None, "profiles/hbm_traffic.json was measured on other kernel sources; record it again"
-    return record["quant_pack_chunks"]["traffic_bytes"], "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated)"
+    return record["bucket_step"]["traffic_bytes"], "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated)"
 
 
 def record_traffic(fetch_db: str, write_db: str) -> int:
@@ -95,25 +98,28 @@ def record_traffic(fetch_db: str, write_db: str) -> int:
     find = lambda table, part: next(v for k, v in table.items() if part in k)
     copy_kib = BUCKET_NUMEL * 4 / 1024
     fetch_factor, write_factor = copy_kib / find(fetch, "copyBuffer.kd"), copy_kib / find(write, "copyBuffer.kd")
-    quant = "quant_pack_kernelIfvfLi64ELi4ELi2E"      # mangled <float, void, float, 64, 4, streaming>
-    quant_fetch, quant_write = find(fetch, quant), find(write, quant)
-    traffic = (quant_fetch * fetch_factor + quant_write * write_factor) * 1024
+    step_kernel = "bucket_step_kernelIfvfLi8ELi2E"     # mangled <float, void, float, 8 payloads, streaming>
+    step_fetch, step_write = find(fetch, step_kernel), find(write, step_kernel)
+    traffic = (step_fetch * fetch_factor + step_write * write_factor) * 1024
+    shard = BUCKET_NUMEL // WORLD
+    payload = shard // GROUP * (GROUP + 4)
     record = {
         "kernel_sources_sha256_16": kernel_sources_hash(), "kernel_sources": list(KERNEL_SOURCES),
-        "commands": ["rocprofv3 --pmc FETCH_SIZE -d <dir> -o f -- python3 bench.py --steps 20 --warmup 2 --only quant_pack_chunks,copy_calibration",
-                     "rocprofv3 --pmc WRITE_SIZE -d <dir> -o w -- python3 bench.py --steps 20 --warmup 2 --only quant_pack_chunks,copy_calibration",
+        "commands": ["rocprofv3 --pmc FETCH_SIZE -d <dir> -o f -- python3 bench.py --steps 20 --warmup 2 --only step,copy_calibration",
+                     "rocprofv3 --pmc WRITE_SIZE -d <dir> -o w -- python3 bench.py --steps 20 --warmup 2 --only step,copy_calibration",
                      "python3 bench.py --record-traffic <dir>/f_results.db <dir>/w_results.db"],
         "calibration": {"kernel": "__amd_rocclr_copyBuffer of 100 MiB (102400 KiB read, 102400 KiB written)",
                         "FETCH_SIZE_factor": fetch_factor, "WRITE_SIZE_factor": write_factor},
-        "quant_pack_chunks": {"kernel": "quant_pack_kernel<float, void, float, 64, 4, 2>, 100 MiB fp32 bucket as 8 chunks",
-                              "FETCH_SIZE_KiB_median": quant_fetch, "WRITE_SIZE_KiB_median": quant_write,
-                              "traffic_bytes": round(traffic),
-                              "algorithmic_bytes": BUCKET_NUMEL * 4 + BUCKET_NUMEL // GROUP * (GROUP + 4)},
+        "bucket_step": {"kernel": "bucket_step_kernel<float, void, float, 8, 2>: quantize+pack of a 100 MiB fp32 bucket as 8 "
+                                  "chunks and the W=8 reduce of a 3,276,800-element shard in one launch",
+                        "FETCH_SIZE_KiB_median": step_fetch, "WRITE_SIZE_KiB_median": step_write,
+                        "traffic_bytes": round(traffic),
+                        "algorithmic_bytes": BUCKET_NUMEL * 4 + WORLD * payload + WORLD * payload + shard * 4},
     }
     with open(TRAFFIC_FILE, "w") as handle:
         json.dump(record, handle, indent=1)
         handle.write("\n")
-    print(json.dumps(record["quant_pack_chunks"]))
+    print(json.dumps(record["bucket_step"]))
     return 0
 
 
@@ -176,12 +182,18 @@ def main() -> int:
             "quant": ops.bind_quant_pack_chunks(bucket, sent, world, group_size=g),
             "reduce": ops.bind_dequant_reduce(pairs, out, group_size=g),
         })
+    # the step: the quantize of one set's bucket and the reduce of the previous set's payloads, one launch
+    for k, s in enumerate(sets):
+        s["step"] = ops.bind_quant_chunks_and_reduce(s["quant"], sets[k - 1]["reduce"])
     torch.cuda.synchronize()
 
     def step(i):
-        s = sets[i % len(sets)]
-        s["quant"]()
-        s["reduce"]()
+        if not sets[i % len(sets)]["step"]():
+            raise RuntimeError("the library has no shared launch for this quantize and reduce")
+
+    def step_two_launches(i):
+        sets[i % len(sets)]["quant"]()
+        sets[i % len(sets) - 1]["reduce"]()
 
     def timed(fn, count, warmup):
         for i in range(warmup):
@@ -202,6 +214,7 @@ def main() -> int:
         total = timed(step, args.steps, args.warmup)
         result["ms_per_step"] = total / args.steps * 1e3
         result["value"] = n * 4 * args.steps / total / 1e9
+        result["ms_per_step_two_launches"] = timed(step_two_launches, args.steps, args.warmup) / args.steps * 1e3
 
     # ---- per-kernel launch durations ---------------------------------------------------------------
     kernels = {}
@@ -217,6 +230,14 @@ def main() -> int:
         }
 
     quant_bytes = n * 4 + world * payload_bytes
+    reduce_bytes = world * payload_bytes + shard * 4
+    if "ms_per_step" in result:
+        seconds = result["ms_per_step"] * 1e-3
+        kernels["bucket_step"] = {
+            "us_per_launch": seconds * 1e6, "algorithmic_bytes": quant_bytes + reduce_bytes,
+            "achieved_GBps": (quant_bytes + reduce_bytes) / seconds / 1e9,
+            "frac_of_hbm_peak": (quant_bytes + reduce_bytes) / seconds / HBM_PEAK,
+        }
     leg("quant_pack_chunks", lambda i: sets[i % len(sets)]["quant"](), quant_bytes)
     if not only or "dequant_reduce_shard" in only:
         # the shard reduce alone moves 41 MB a launch: it gets payload sets of its own, enough of them (656 MB) that
@@ -227,7 +248,7 @@ def main() -> int:
             out = torch.empty(shard, dtype=torch.float32, device=dev)
             pairs = [ops.split_payload(rows[r, :payload_bytes], shard, g) for r in range(world)]
             shard_sets.append(ops.bind_dequant_reduce(pairs, out, group_size=g))
-        leg("dequant_reduce_shard", lambda i: shard_sets[i % SHARD_SETS](), world * payload_bytes + shard * 4)
+        leg("dequant_reduce_shard", lambda i: shard_sets[i % SHARD_SETS](), reduce_bytes)
         del shard_sets
         torch.cuda.empty_cache()
 
@@ -274,7 +295,8 @@ def main() -> int:
         from oracle import codec_torch
 
         s0 = sets[0]
-        s0["quant"](); s0["reduce"]()
+        if not ops.bind_quant_chunks_and_reduce(s0["quant"], s0["reduce"])():     # the step's launch, on one set
+            raise RuntimeError("the library has no shared launch for this quantize and reduce")
         torch.cuda.synchronize()
         bucket_cpu = s0["bucket"].cpu()
         received_cpu = s0["received"].cpu()
@@ -331,7 +353,7 @@ def main() -> int:
             "cpu_model": model,
         }
 
-    dominant = kernels.get("quant_pack_chunks")
+    dominant = kernels.get("bucket_step")
     traffic, traffic_source = recorded_traffic()
     line = {
         "metric": "quant-pack & fused dequant-reduce GB/s on 1 MI355X; % of HBM roofline",
@@ -341,6 +363,7 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": result.get("ms_per_step"),
+        "ms_per_step_two_launches": result.get("ms_per_step_two_launches"),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -348,12 +371,14 @@ def main() -> int:
         "data": "synthetic",
         "config": {
             "workload": "config 2: 100 MiB fp32 bucket ~N(0,1e-3 std), W=8, group 64: quant-pack of the 8 chunks + "
-                        "fused dequant-reduce of one rank's shard (8 payloads x 3,276,800 codes), fixed rank order",
+                        "fused dequant-reduce of one rank's shard (8 payloads x 3,276,800 codes), fixed rank order; "
+                        "one launch carries the quantize of a bucket and the shard reduce of the bucket before it",
             "bucket_numel": n, "world_size": world, "group_size": g, "buffer_sets": args.sets,
             "value_is": "bucket bytes (104,857,600) consumed per step / step time",
         },
         "roofline": None if dominant is None else {
-            "bound": "hbm", "kernel": "quant_pack_kernel (100 MiB fp32 bucket, 8 chunks, one launch)",
+            "bound": "hbm", "kernel": "bucket_step_kernel (quant-pack of the 100 MiB fp32 bucket as 8 chunks + W=8 reduce "
+                                      "of one shard, one launch)",
             "achieved": dominant["achieved_GBps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
             "frac": dominant["frac_of_hbm_peak"], "traffic": traffic, "traffic_source": traffic_source,
             "algorithmic_bytes": dominant["algorithmic_bytes"], "us_per_launch": dominant["us_per_launch"],
