@@ -284,14 +284,19 @@ def main() -> int:
             payload = torch.empty(ops.payload_nbytes(n, G), dtype=torch.uint8, device=dev)
             codes, scales = ops.split_payload(payload, n, G)
             out = torch.empty(n, device=dev)
-            sets.append((x, payload, ops.bind_quant_pack(x, codes, scales), ops.bind_dequant(codes, scales, out), out))
+            sets.append((x, payload, ops.bind_quant_pack(x, codes, scales), ops.bind_dequant(codes, scales, out), out,
+                         ops.bind_quant_pack(x, codes, scales, restored=out)))
         check = None
         cpu = {}
         if parity:
-            x, payload, q, d, out = sets[0]
+            x, payload, q, d, out, both = sets[0]
             q(); d()
             w_codes, w_scales = codec_torch.quantize(x.cpu(), G)
             ok = torch.equal(payload.cpu(), codec_torch.pack(w_codes, w_scales))
+            ok = ok and bits_equal(out, codec_torch.dequantize(w_codes, w_scales, n, G, "fp32"))
+            payload.zero_(); out.zero_()
+            both()                                  # the same two results from one launch
+            ok = ok and torch.equal(payload.cpu(), codec_torch.pack(w_codes, w_scales))
             ok = ok and bits_equal(out, codec_torch.dequantize(w_codes, w_scales, n, G, "fp32"))
             rel = float((x - out).norm() / x.norm())
             check = "bit-exact" if ok else "MISMATCH"
@@ -303,6 +308,8 @@ def main() -> int:
         emit(1, "quantize+pack 25 MiB fp32", nbytes, timed(lambda i: sets[i % 8][2](), args.iters), n * 4, check, **cpu)
         emit(1, "dequantize 25 MiB fp32", nbytes, timed(lambda i: sets[i % 8][3](), args.iters), ops.payload_nbytes(n, G), check)
         emit(1, "round trip (2 launches)", 2 * nbytes, timed(lambda i: (sets[i % 8][2](), sets[i % 8][3]()), args.iters), n * 4, check)
+        emit(1, "round trip, one launch (quantize+pack with the decoded tensor as a second output)", nbytes + n * 4,
+             timed(lambda i: sets[i % 8][5](), args.iters), n * 4, check)
         emit(1, "quantize+pack 25 MiB fp32, one buffer set (cache-warm, not an HBM figure)", nbytes,
              timed(lambda i: sets[0][2](), args.iters), n * 4, check)
         emit(1, "dequantize 25 MiB fp32, one buffer set (cache-warm, not an HBM figure)", nbytes,
