@@ -95,6 +95,20 @@ def test_scale_formula_is_exact_for_every_finite_float(tmp_path):
     assert "0x3C010204" in done.stdout
 
 
+def test_division_free_quotient_matches_the_division_next_to_every_tie(tmp_path):
+    """The encode's q1 = fma(fma(-q0, s, p), 1/s, q0) against p / s on the CPU, for dividends within 8 ulps of every
+    half-integer and integer multiple of the scale: every scale with at most 11 significant mantissa bits and the
+    (almost) all-ones mantissas at the ends and the middle of the scale's exponent range, and four million random
+    mantissas (3.6e10 pairs, about 15 s on 8 cores).  The GPU suite walks all 2^23 mantissas on the device."""
+    binary = tmp_path / "check_quotient"
+    subprocess.run(["gcc", "-O2", "-mfma", "-fopenmp", "-ffp-contract=off", "-o", str(binary),
+                    str(ROOT / "tests" / "native" / "check_quotient.c"), "-lm"], check=True)
+    done = subprocess.run([str(binary)], capture_output=True, text=True, timeout=900)
+    assert done.returncode == 0, done.stdout
+    assert "code mismatches 0, quotient mismatches 0" in done.stdout
+    assert int(done.stdout.split()[1].rstrip(",")) > 3 * 10 ** 10
+
+
 def test_sum_of_two_16_bit_values_through_fp32_is_the_native_sum(tmp_path):
     """The CUDA-format kernels add two fp16 / bfloat16 values with one fp32 add and one conversion; for every pair
     of finite values of either type that is the correctly rounded 16-bit sum (about half a minute on 8 cores)."""
