@@ -686,6 +686,56 @@ def test_shared_launch_of_quantize_and_reduce_equals_the_two_launches_and_the_or
     assert_same_bits(got_out, want, "reduced shard against the oracle")
 
 
+def test_bucket_steps_dealt_to_two_streams_in_turn_equal_the_one_stream_schedule(ops, hip_device):
+    """Consecutive buckets are independent: their launches (quantize of bucket k + reduce of bucket k-1) may alternate
+    between two streams, each with its own send matrix and shard output, and must leave the same residuals, payloads
+    and shards as the same launches on one stream."""
+    world, n, buckets = 8, 64 * 8 * 500, 9
+    shard = n // world
+    stride = (ops.payload_nbytes(shard) + 255) // 256 * 256
+    grads = [gradient_like(n, torch.bfloat16, 4000 + k, hip_device) for k in range(buckets)]
+    start = [gradient_like(n, torch.float32, 4100 + k, hip_device, sigma=1e-5, outliers=False) for k in range(buckets)]
+    peers = [[ops.quant_pack(gradient_like(shard, torch.float32, 4200 + 8 * k + r, hip_device)) for r in range(world)]
+             for k in range(buckets)]
+
+    def schedule(residuals, rows, outs):
+        launches, previous = [], None
+        for k in range(buckets):
+            quant = ops.bind_quant_pack_chunks(grads[k], rows[k], world, residual=residuals[k], new_residual=residuals[k])
+            reduce = ops.bind_dequant_reduce(peers[k], outs[k], divisor=float(world))
+            launches.append(quant if previous is None else ops.bind_quant_chunks_and_reduce(quant, previous))
+            previous = reduce
+        return launches, previous
+
+    def fresh():
+        return ([r.clone() for r in start],
+                [torch.zeros(world, stride, dtype=torch.uint8, device=hip_device) for _ in range(buckets)],
+                [torch.empty(shard, device=hip_device) for _ in range(buckets)])
+
+    want_residuals, want_rows, want_outs = fresh()
+    launches, last = schedule(want_residuals, want_rows, want_outs)
+    for launch in launches:
+        assert launch() is True
+    assert last() is True
+    torch.cuda.synchronize()
+
+    got_residuals, got_rows, got_outs = fresh()
+    launches, last = schedule(got_residuals, got_rows, got_outs)
+    lanes = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for lane in lanes:
+        lane.wait_stream(torch.cuda.current_stream())
+    for k, launch in enumerate(launches):
+        assert launch(lanes[k & 1].cuda_stream) is True
+    assert last(lanes[buckets & 1].cuda_stream) is True
+    for lane in lanes:
+        torch.cuda.current_stream().wait_stream(lane)
+    torch.cuda.synchronize()
+    for k in range(buckets):
+        assert torch.equal(got_rows[k], want_rows[k]), f"payloads of bucket {k}"
+        assert_same_bits(got_residuals[k], want_residuals[k].cpu(), f"residual of bucket {k}")
+        assert_same_bits(got_outs[k], want_outs[k].cpu(), f"shard of bucket {k}")
+
+
 def test_shared_launch_reports_what_it_has_no_grid_for(ops, hip_device):
     n, world = 64 * 8 * 64, 8
     shard = n // world
