@@ -220,16 +220,16 @@ def main() -> int:
             # Consecutive steps touch different buffer sets, so they may also be dealt to two streams in turn: the
             # ramp-up of one launch then overlaps the drain of the one before.  Reported next to the headline, which
             # stays on one stream so that a step is one kernel's duration.
-            lanes = [torch.cuda.Stream(), torch.cuda.Stream()]      # default priority
+            from lowbit_comm_amd.hip.lanes import StreamLanes
+
+            lanes = StreamLanes(2, dev)
 
             def run_lanes(count):
-                for lane in lanes:
-                    lane.wait_stream(stream)
+                lanes.fork()
                 for i in range(count):
-                    if not sets[i % len(sets)]["step"](lanes[i & 1].cuda_stream):
+                    if not sets[i % len(sets)]["step"](lanes.handle(i)):
                         raise RuntimeError("the library has no shared launch for this quantize and reduce")
-                for lane in lanes:
-                    stream.wait_stream(lane)
+                lanes.join()
 
             run_lanes(args.warmup)
             torch.cuda.synchronize()

@@ -660,7 +660,9 @@ def main() -> int:
         # The same launches dealt to two streams in turn.  Consecutive buckets are independent, so the ramp-up of one
         # bucket's launch overlaps the drain of the one before.  Each stream has its own send matrix and shard output
         # (a bucket's payloads must survive until they are exchanged), hence nothing crosses between the streams.
-        lanes = [torch.cuda.Stream(), torch.cuda.Stream()]      # default priority
+        from lowbit_comm_amd.hip.lanes import StreamLanes
+
+        lanes = StreamLanes(2, dev)
         lane_buffers = {}
         lane_launches = []
 
@@ -685,14 +687,12 @@ def main() -> int:
         last_reduce, last_out = previous, out
 
         def one_pass_two_streams():
+            lanes.fork()
             for index, launch in enumerate(lane_launches):
-                if not launch(lanes[index & 1].cuda_stream):
+                if not launch(lanes.handle(index)):
                     raise RuntimeError("no shared launch for this bucket")
-            last_reduce(lanes[len(lane_launches) & 1].cuda_stream)
-
-        def settle():
-            for lane in lanes:
-                stream.wait_stream(lane)
+            last_reduce(lanes.handle(len(lane_launches)))
+            lanes.join()
 
         lanes_check = None
         if parity:
@@ -715,10 +715,7 @@ def main() -> int:
         torch.cuda.synchronize()
         host0 = time.perf_counter()
         a_ev.record(stream)
-        for lane in lanes:
-            lane.wait_stream(stream)
         one_pass_two_streams()
-        settle()
         b_ev.record(stream)
         host1 = time.perf_counter()
         torch.cuda.synchronize()

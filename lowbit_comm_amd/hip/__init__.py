@@ -1,5 +1,6 @@
 """HIP (gfx950) backend: C-ABI binding, tensor-level ops, native-module shim, codec callables, workspace pool."""
 from .completion import HipCompletionManager, HipStreamWork
+from .lanes import StreamLanes
 from .loader import CudaExtensionStatus, HipExtensionStatus, load_cuda_extension, load_hip_extension
 from .ring import (
     HipPipelinedRingRuntime,
@@ -38,6 +39,7 @@ __all__ = [
     "PipelinedRingExecutor", "PipelinedRingSchedule", "RingAllGatherStep", "RingReduceScatterStep",
     "compile_pipelined_ring_schedule", "make_pipelined_ring_executor", "HipTreeRuntime", "LoopbackMesh", "TreeEdge",
     "TreeExecutor", "TreeSchedule", "compile_tree_schedule", "make_tree_executor",
-    "HipWorkspacePool", "ShardWorkspaceProvider", "ShardWorkspaceSession", "StreamOrderedCompletion", "WorkspaceKey",
+    "HipWorkspacePool", "ShardWorkspaceProvider", "ShardWorkspaceSession", "StreamLanes", "StreamOrderedCompletion",
+    "WorkspaceKey",
     "WorkspaceLease", "WorkspaceStats", "create_torch_workspace_pool", "load_cuda_extension", "load_hip_extension",
 ]

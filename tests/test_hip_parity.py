@@ -721,14 +721,16 @@ def test_bucket_steps_dealt_to_two_streams_in_turn_equal_the_one_stream_schedule
 
     got_residuals, got_rows, got_outs = fresh()
     launches, last = schedule(got_residuals, got_rows, got_outs)
-    lanes = [torch.cuda.Stream(), torch.cuda.Stream()]
-    for lane in lanes:
-        lane.wait_stream(torch.cuda.current_stream())
+    from lowbit_comm_amd.hip import StreamLanes
+
+    lanes = StreamLanes(2)
+    assert len(lanes) == 2 and lanes.handle(0) != lanes.handle(1) and lanes.handle(2) == lanes.handle(0)
+    assert lanes.stream(3).cuda_stream == lanes.handle(1)
+    lanes.fork()
     for k, launch in enumerate(launches):
-        assert launch(lanes[k & 1].cuda_stream) is True
-    assert last(lanes[buckets & 1].cuda_stream) is True
-    for lane in lanes:
-        torch.cuda.current_stream().wait_stream(lane)
+        assert launch(lanes.handle(k)) is True
+    assert last(lanes.handle(buckets)) is True
+    lanes.join()
     torch.cuda.synchronize()
     for k in range(buckets):
         assert torch.equal(got_rows[k], want_rows[k]), f"payloads of bucket {k}"
