@@ -66,6 +66,7 @@ class ReduceScatterPlan:
         # the callers' tensors alive (the key holds everything a binding depends on, and every step is handed the
         # live tensors), so it pins no memory beyond the plan's own buffers.
         self._bound: OrderedDict[Any, ops.BoundLaunch] = OrderedDict()
+        self._last_stream: Any | None = None
         self._last_stream_handle: int | None = None
         self.exchange_in_flight: Any | None = None     # work object of an exchange that nobody has waited for yet
 
@@ -87,13 +88,15 @@ class ReduceScatterPlan:
         the previous step included) is waited for by the current stream."""
         if self.device.type != "cuda":
             return
-        handle = ops.current_stream_handle(self.device)
-        previous = self._last_stream_handle
-        if previous is not None and previous != handle:
+        handle = ops.current_stream_handle(self.device)      # a raw handle: no stream object in the usual case
+        if handle == self._last_stream_handle:
+            return
+        stream = torch.cuda.current_stream(self.device)
+        if self._last_stream is not None:
             event = torch.cuda.Event()
-            event.record(torch.cuda.ExternalStream(previous, device=self.device))
-            torch.cuda.current_stream(self.device).wait_event(event)
-        self._last_stream_handle = handle
+            event.record(self._last_stream)                   # the stream object is kept, so its handle stays valid
+            stream.wait_event(event)
+        self._last_stream, self._last_stream_handle = stream, handle
 
     # ---- payload views ---------------------------------------------------------------------------
     def payload(self, rows: torch.Tensor, index: int) -> torch.Tensor:
