@@ -981,7 +981,37 @@ def main() -> int:
             eager()
         host, wall = host_and_wall(lambda i: graph.replay(), 5)
         host_row("the same sequence as one HIP-graph replay, per bucket", host / count, wall / count)
-        del grads, residuals, launches, graph
+        # one launch per bucket, the buckets dealt to two streams in turn (a send matrix and an output per lane)
+        from lowbit_comm_amd.hip.lanes import StreamLanes
+
+        lanes = StreamLanes(2, dev)
+        lane_rows = [rows, torch.empty_like(rows)]
+        lane_outs = [out, torch.empty_like(out)]
+        steps, previous = [], None
+        for i in range(count):
+            piece = slice(i * n, (i + 1) * n)
+            quant = ops.bind_quant_pack_chunks(grads[piece], lane_rows[i & 1], world, residual=residuals[piece],
+                                               new_residual=residuals[piece])
+            reduce = ops.bind_dequant_reduce(received, lane_outs[i & 1], numel=shard)
+            steps.append(quant if previous is None else ops.bind_quant_chunks_and_reduce(quant, previous))
+            previous = reduce
+
+        def two_lanes(_i=0):
+            lanes.fork()
+            for k, launch in enumerate(steps):
+                launch(lanes.handle(k))
+            previous(lanes.handle(count))
+            lanes.join()
+
+        host, wall = host_and_wall(two_lanes, 5)
+        host_row("64 buckets x one launch (EF quant-pack of bucket k + shard reduce of bucket k-1) on two streams in turn, "
+                 "eager, per bucket", host / count, wall / count)
+        lane_graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(lane_graph, stream=torch.cuda.Stream()):
+            two_lanes()
+        host, wall = host_and_wall(lambda i: lane_graph.replay(), 5)
+        host_row("the same two-stream sequence as one HIP-graph replay, per bucket", host / count, wall / count)
+        del grads, residuals, launches, graph, steps, lane_graph
 
     # ------------------------------------------------------------------------------------------ 8
     if 8 in wanted:

@@ -847,6 +847,62 @@ def test_bucket_stream_captured_in_a_hip_graph_replays_like_eager(dev):
         assert float((torch.randn(1 << 16, device=dev) * 2).sum().item()) == pytest.approx(0.0, abs=1e4)   # eager work
 
 
+def test_two_lane_bucket_stream_captured_in_a_hip_graph_replays_like_eager(dev):
+    """The one-launch bucket steps dealt to two streams (fork, alternate, join) captured as one graph with two
+    parallel branches: four replays with eager work between them against four eager one-stream passes."""
+    from lowbit_comm_amd.hip import StreamLanes, ops
+
+    world, g, buckets, n = 8, 64, 7, 64 * 8 * 520
+    shard = n // world
+    stride = -(-ops.payload_nbytes(shard, g) // 256) * 256
+    grads = grad(buckets * n, torch.bfloat16, 21, dev)
+    start = grad(buckets * n, torch.float32, 22, dev, sigma=1e-5)
+    residuals = start.clone()
+    rows = [torch.empty(world, stride, dtype=torch.uint8, device=dev) for _ in range(2)]       # one pair per lane
+    outs = [torch.empty(shard, device=dev) for _ in range(2)]
+    peers = [[ops.quant_pack(grad(shard, torch.float32, 30 + 8 * i + r, dev), group_size=g) for r in range(world)]
+             for i in range(buckets)]
+    launches, previous = [], None
+    for i in range(buckets):
+        piece = slice(i * n, (i + 1) * n)
+        quant = ops.bind_quant_pack_chunks(grads[piece], rows[i & 1], world, residual=residuals[piece],
+                                           new_residual=residuals[piece])
+        reduce = ops.bind_dequant_reduce(peers[i], outs[i & 1], numel=shard)
+        launches.append(quant if previous is None else ops.bind_quant_chunks_and_reduce(quant, previous))
+        previous = reduce
+    lanes = StreamLanes(2)
+
+    def one_stream():
+        for launch in launches:
+            assert launch()
+        assert previous()
+
+    def two_lanes():
+        lanes.fork()
+        for i, launch in enumerate(launches):
+            assert launch(lanes.handle(i))
+        assert previous(lanes.handle(buckets))
+        lanes.join()
+
+    eager = []
+    for _ in range(4):
+        one_stream()
+        torch.cuda.synchronize()
+        eager.append((residuals.clone(), rows[0].clone(), rows[1].clone(), outs[0].clone(), outs[1].clone()))
+    residuals.copy_(start)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+        two_lanes()
+    torch.cuda.synchronize()
+    residuals.copy_(start)                                            # capture enqueued nothing
+    for want in eager:
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (residuals, rows[0], rows[1], outs[0], outs[1])
+        assert all(torch.equal(a.view(torch.uint8), b.view(torch.uint8)) for a, b in zip(got, want))
+        assert float((torch.randn(1 << 16, device=dev) * 2).sum().item()) == pytest.approx(0.0, abs=1e4)   # eager work
+
+
 def test_stream_ordered_completion_records_nothing_while_a_buffer_stays_on_one_stream(dev):
     from lowbit_comm_amd.hip import StreamOrderedCompletion, WorkspaceKey, create_torch_workspace_pool
 
