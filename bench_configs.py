@@ -1152,7 +1152,8 @@ def main() -> int:
             return Arrived()
 
         buckets = [gen(SEED + 8400 + k, n, 1e-3) for k in range(3)]
-        for fused, graphed, inline in ((True, False, False), (True, False, True), (True, True, False), (False, False, False)):
+        for fused, graphed, inline in ((True, False, False), (True, False, True), (True, True, False), (True, True, True),
+                                       (False, False, False)):
             executor = make_pipelined_ring_executor(config=cfg, dtype="fp32", numel=n, world_size=world, rank=3,
                                                     exchange=exchange, fuse_steps=fused, graph_replay=graphed,
                                                     stream=stream if inline else None)
