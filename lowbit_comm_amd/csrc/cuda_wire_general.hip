@@ -21,6 +21,7 @@
 // scan positions behind the last NaN, (b) the three largest keys (magnitude bits, tie-break rank),
 // merged across the row, (c) Philox in counter mode - draw j of group s is word (offset + j) % 4
 // of block (offset + j) / 4 of subsequence s, so a lane computes the blocks of its own elements.
+#include "code_book_cells.h"
 #include "device_utils.h"
 #include "launch.h"
 #include "wire_common.h"
@@ -28,17 +29,10 @@
 namespace lbc {
 namespace {
 
-// inner.cuh:9-35 (entry 15 is never produced by the encoder)
-__constant__ float kCodeBooks[4][16] = {
-    {-1.0f, -0.815410147f, -0.655160150f, -0.510228027f, -0.375324982f, -0.246951370f, -0.122538030f, 0.0f,
-     0.122538030f, 0.246951370f, 0.375324982f, 0.510228027f, 0.655160150f, 0.815410147f, 1.0f, __builtin_inff()},
-    {-1.0f, -0.85714286f, -0.71428571f, -0.57142857f, -0.42857143f, -0.28571429f, -0.14285714f, 0.0f,
-     0.14285714f, 0.28571429f, 0.42857143f, 0.57142857f, 0.71428571f, 0.85714286f, 1.0f, __builtin_inff()},
-    {-1.0f, -0.5f, -0.25f, -0.125f, -0.0625f, -0.03125f, -0.015625f, 0.0f,
-     0.015625f, 0.03125f, 0.0625f, 0.125f, 0.25f, 0.5f, 1.0f, __builtin_inff()},
-    {-1.0f, -0.6666666666666666f, -0.5f, -0.3333333333333333f, -0.25f, -0.16666666666666666f, -0.125f, 0.0f,
-     0.125f, 0.16666666666666666f, 0.25f, 0.3333333333333333f, 0.5f, 0.6666666666666666f, 1.0f, __builtin_inff()},
-};
+// inner.cuh:9-35, and the one-lookup form of the encoder built from them at compile time
+__constant__ book_cells::Books kCodeBooks = book_cells::kBookSet;
+__constant__ book_cells::Tables kBookCells = book_cells::kTables;
+__constant__ book_cells::Steps kBookSteps = book_cells::kSteps;
 
 // Philox4x32-10: one block of four 32-bit words.
 __device__ __forceinline__ void philox_block(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
@@ -68,7 +62,7 @@ __device__ __forceinline__ const float *wave_code_book(int kind, int lane) {
     __shared__ float books[kWavesPerBlock][16];
     float *book = books[threadIdx.x >> 6];
     if (kind != 0) {
-        if (lane < 16) book[lane] = kCodeBooks[kind - 1][lane];
+        if (lane < 16) book[lane] = kCodeBooks.value[kind - 1][lane];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -76,13 +70,44 @@ __device__ __forceinline__ const float *wave_code_book(int kind, int lane) {
     return book;
 }
 
+// The same for the quantizer, with the book's table of steps (code_book_cells.h) behind the sixteen entries.
+__device__ __forceinline__ const float *wave_code_book_and_steps(int kind, int lane) {
+    __shared__ float tables[kWavesPerBlock][32];
+    float *table = tables[threadIdx.x >> 6];
+    if (kind != 0) {
+        if (lane < 32) table[lane] = lane < 16 ? kCodeBooks.value[kind - 1][lane] : kBookSteps.value[kind - 1][lane - 16];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    return table;
+}
+
+// The workgroup's copy of a book's cell table (code_book_cells.h) in LDS.  Every wavefront of the workgroup must
+// come here: the copy ends in a workgroup barrier.
+__device__ __forceinline__ const book_cells::Cell *block_book_cells(int kind) {
+    __shared__ book_cells::Cell cells[book_cells::kCells];
+    static_assert(book_cells::kCells <= kBlock + 1, "one table entry per thread, and one more");
+    const book_cells::Cell *table = kBookCells.book[kind - 1].cell;
+    cells[threadIdx.x] = table[threadIdx.x];
+    if (threadIdx.x == 0) cells[kBlock] = table[kBlock];
+    __syncthreads();
+    return cells;
+}
+
 __device__ __forceinline__ int meta_words_of(int topk) { return topk == 0 ? 1 : topk + 2; }
 
 // ---------------------------------------------------------------------------------------------
 // quantize: one wavefront per tile of 64 * VEC elements
 // ---------------------------------------------------------------------------------------------
-template <typename T, int G, int BIT>
+// FIXED names what the launch knows about the policy at compile time, so that the code of the other policies
+// is not part of the kernel: bit 0 "no outlier channel", bit 1 "round to nearest", bit 2 "linear codes".
+// 0 is the kernel for every policy.
+template <typename T, int G, int BIT, int FIXED>
 __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGeneralQuantArgs a) {
+    const int topk = (FIXED & 1) ? 0 : a.topk;
+    const bool stochastic = (FIXED & 2) ? false : a.stochastic != 0;
+    const int kind = (FIXED & 4) ? 0 : a.kind;
     using W = wire<T, BIT>;
     using RB = raw_bits<T>;
     using Raw = typename RB::type;
@@ -91,10 +116,9 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     static_assert(LPG >= 2 && LPG <= 16, "a group must span 2..16 lanes of one DPP row");
 
     const int lane = threadIdx.x & (kWave - 1);
-    const int meta_bytes = meta_words_of(a.topk) * ITEM;
+    const int meta_bytes = meta_words_of(topk) * ITEM;
     const int64_t groups = a.numel / G;
     const int64_t tile_first = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * W::TILE;
-    if (tile_first >= a.numel) return;   // wavefront-uniform
     const int64_t e0 = tile_first + lane * VEC;
     const bool live = e0 < a.numel;      // numel is a multiple of G: dead lanes form whole dead groups
     const int64_t group = e0 / G;
@@ -105,7 +129,15 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
 #pragma unroll
     for (int i = 0; i < VEC; ++i) raw[i] = 0;
     if (live) load_elems<Raw, VEC, kPlain>(static_cast<const Raw *>(a.x) + e0, raw);   // instruction-bound: the hint only costs
-    const float *book = wave_code_book(a.kind, lane);   // after the loads were issued: its wait covers theirs
+    // After the loads were issued: the waits of the tables cover theirs.  The cell table pays for its copy and its
+    // barrier with eight elements a lane (26.2 M bf16 elements: 20.1 us against 24.6 us with the search), not with
+    // the four of a 32-bit tensor (33.3 against 32.2 us, although a wavefront issues 125 vector instructions
+    // instead of 187); those search the table of steps, which needs no barrier.
+    constexpr bool CELLS = ITEM == 2;
+    const bool by_cells = CELLS && kind != 0 && !stochastic;   // uniform over the grid
+    const book_cells::Cell *cells = by_cells ? block_book_cells(kind) : nullptr;
+    if (tile_first >= a.numel) return;   // wavefront-uniform, behind the workgroup's barrier
+    const float *book = wave_code_book_and_steps(kind, lane);
     float v[VEC];
     uint32_t mag[VEC];
 #pragma unroll
@@ -118,7 +150,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     uint8_t *group_meta = a.compact ? group_codes + CB : a.payload + groups * CB + group * meta_bytes;
 
     uint32_t scale_raw;
-    if (a.topk == 0) {
+    if (topk == 0) {
         scale_raw = running_max_raw<T, G, VEC>(mag, k0, start);
     } else {
         // Three rounds of "largest remaining candidate": the group maximum of the magnitude keys, then, among
@@ -136,7 +168,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
         uint32_t best_key[3] = {0, 0, 0}, best_rank[2] = {0, 0};              // magnitude + 1, rank
 #pragma unroll
         for (int round = 0; round < 3; ++round) {
-            if (round == 2 && a.topk == 1) break;                             // uniform
+            if (round == 2 && topk == 1) break;                             // uniform
             uint32_t m = 0;
 #pragma unroll
             for (int i = 0; i < VEC; ++i) m = key[i] > m ? key[i] : m;
@@ -166,7 +198,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
         const bool none = best_key[0] == 0;
         const int index1 = none ? 0 : index_of(best_rank[0]);
         int index2 = -1;
-        if (a.topk == 1) {
+        if (topk == 1) {
             // nothing comparable: the reference falls back to element 1 (as stored for fp32, its magnitude otherwise)
             const uint32_t element1 = WIDE ? static_cast<uint32_t>(raw[1]) : mag[1];
             const uint32_t fallback = static_cast<uint32_t>(__shfl(static_cast<int>(element1), lane & ~(LPG - 1)));
@@ -191,7 +223,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
         if (live && own2) *reinterpret_cast<Raw *>(group_meta + 3 * ITEM) = top2_raw;   // the outliers as they are
         if (live && k0 == 0)
             *reinterpret_cast<Raw *>(group_meta + ITEM) =
-                static_cast<Raw>(a.topk == 1 ? index1 : (index1 | (index2 << 8)));
+                static_cast<Raw>(topk == 1 ? index1 : (index1 | (index2 << 8)));
     }
     if (live && k0 == 0) *reinterpret_cast<Raw *>(group_meta) = static_cast<Raw>(scale_raw);
 
@@ -201,7 +233,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     float uniform[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) uniform[i] = 0.0f;
-    if (a.stochastic) {
+    if (stochastic) {
         const uint32_t key0 = static_cast<uint32_t>(a.seed), key1 = static_cast<uint32_t>(a.seed >> 32);
         const uint32_t sub0 = static_cast<uint32_t>(group), sub1 = static_cast<uint32_t>(static_cast<uint64_t>(group) >> 32);
         const int phase = static_cast<int>(a.offset & 3);
@@ -224,13 +256,13 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     }
 
     int c[VEC];
-    if (a.kind == 0) {
+    if (kind == 0) {
         const float multiplier = W::LEVELS / scale;
         constexpr int L = static_cast<int>(W::LEVELS);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             // nvcc contracts v * m + noise into one FMA; without noise the product is rounded alone
-            const float t = a.stochastic ? __builtin_fmaf(v[i], multiplier, uniform[i] - 0.5f) : v[i] * multiplier;
+            const float t = stochastic ? __builtin_fmaf(v[i], multiplier, uniform[i] - 0.5f) : v[i] * multiplier;
             const int r = cvt_i32(__builtin_rintf(t));
             c[i] = r < -L ? -L : (r > L ? L : r);
         }
@@ -250,7 +282,8 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
         bool unusual = scale_exponent < 127u - 60u || scale_exponent > 127u + 60u;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) unusual |= !(__builtin_fabsf(v[i]) <= scale);
-        if (__ballot(unusual) == 0) {   // wavefront-uniform
+        const bool usual = __ballot(unusual) == 0;   // wavefront-uniform
+        if (usual) {
             float reciprocal = __builtin_amdgcn_rcpf(scale);
             reciprocal = __builtin_fmaf(__builtin_fmaf(-scale, reciprocal, 1.0f), reciprocal, reciprocal);
 #pragma unroll
@@ -263,6 +296,31 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
 #pragma unroll
             for (int i = 0; i < VEC; ++i) t[i] = v[i] / scale;
         }
+        if (usual && by_cells) {
+            // Every t is a number in [-1, 1]: search and rounding are one table lookup (code_book_cells.h).
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                const book_cells::Cell cell = cells[static_cast<uint32_t>(__builtin_fmaf(t[i], 128.0f, 128.0f))];
+                c[i] = static_cast<int>(cell.base) + (t[i] >= cell.threshold ? 1 : 0);
+            }
+        } else if (usual && !stochastic) {
+            // Every t is a number in [-1, 1]: the code is the number of the book's steps not above t, found by the
+            // halving search below run over the table of steps, with no rounding stage behind it.
+            const char *step_bytes = reinterpret_cast<const char *>(book + 16);
+            int at[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) at[i] = 0;
+#pragma unroll
+            for (int half = 8 * 4; half >= 4; half >>= 1) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const int mid = at[i] + half;
+                    at[i] = !(t[i] < *reinterpret_cast<const float *>(step_bytes + mid)) ? mid : at[i];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) c[i] = at[i] >> 2;
+        } else {
         // The largest entry in [0, 14] with not (t < book[entry]); a NaN ends at 14.  Four halving steps, each
         // over all of the lane's elements so that their LDS reads are in flight together; positions are kept as
         // byte offsets into the book.
@@ -287,12 +345,13 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
             excess[i] = t[i] - low;
             c[i] = at[i] >> 2;
         }
-        if (a.stochastic) {   // uniform: the second division only runs when it is needed
+        if (stochastic) {   // uniform: the second division only runs when it is needed
 #pragma unroll
             for (int i = 0; i < VEC; ++i) c[i] += uniform[i] < excess[i] / gap[i] ? 1 : 0;
         } else {
 #pragma unroll
             for (int i = 0; i < VEC; ++i) c[i] += excess[i] > gap[i] * 0.5f ? 1 : 0;
+        }
         }
     }
     if (live) {
@@ -385,9 +444,23 @@ hipError_t launch_general_quant_g(int bit, const WireGeneralQuantArgs &a, hipStr
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
     const dim3 grid(static_cast<unsigned>(blocks));
-    if (bit == 8) hipLaunchKernelGGL((wire_general_quant_kernel<T, G, 8>), grid, dim3(kBlock), 0, stream, a);
-    else if (bit == 4) hipLaunchKernelGGL((wire_general_quant_kernel<T, G, 4>), grid, dim3(kBlock), 0, stream, a);
-    else return hipErrorNotSupported;
+    // Policies that round to nearest run a kernel without the code of the others (26.2 M fp32 elements: top-2
+    // 30.8 instead of 32.3 us, a code book 30.0 instead of 31.7 us); stochastic rounding is faster in the kernel
+    // for every policy (37.4 against 38.6 us), whose Philox rounds leave the compiler less room to reorder.
+    const int fixed = a.stochastic ? 0 : ((a.topk == 0 ? 1 : 0) | 2 | (a.kind == 0 ? 4 : 0));
+    if (bit != 8 && bit != 4) return hipErrorNotSupported;
+    if (bit == 8 && a.kind != 0) return hipErrorNotSupported;   // eight bits: linear codes only
+#define LBC_GENERAL_QUANT(BIT, FIXED) \
+    hipLaunchKernelGGL((wire_general_quant_kernel<T, G, BIT, FIXED>), grid, dim3(kBlock), 0, stream, a)
+    if (bit == 8) {
+        if (fixed == 6) LBC_GENERAL_QUANT(8, 6);
+        else LBC_GENERAL_QUANT(8, 0);
+    } else {
+        if (fixed == 2 || fixed == 6) LBC_GENERAL_QUANT(4, 2);
+        else if (fixed == 3) LBC_GENERAL_QUANT(4, 3);
+        else LBC_GENERAL_QUANT(4, 0);
+    }
+#undef LBC_GENERAL_QUANT
     return hipGetLastError();
 }
 

@@ -109,6 +109,21 @@ def test_division_free_quotient_matches_the_division_next_to_every_tie(tmp_path)
     assert int(done.stdout.split()[1].rstrip(",")) > 3 * 10 ** 10
 
 
+def test_code_book_cell_lookup_is_the_search_and_rounding_on_every_float(tmp_path):
+    """The code-book quantizer of the CUDA byte format encodes a 16-bit tensor's quotients with one table lookup
+    (csrc/code_book_cells.h, tables built at compile time).  For each of the four books and every float in [-1, 1]
+    (8.5e9 values, about 15 s on 8 cores) the lookup gives the code of the reference's search and rounding step, and
+    every step of the table is checked on both sides whatever the stride."""
+    binary = tmp_path / "check_book_cells"
+    subprocess.run(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-fopenmp", "-o", str(binary),
+                    str(ROOT / "tests" / "native" / "check_book_cells.cpp")], check=True)
+    done = subprocess.run([str(binary)], capture_output=True, text=True, timeout=900)
+    assert done.returncode == 0, done.stdout
+    lines = done.stdout.splitlines()
+    assert lines[-1] == "MISMATCHES 0" and int(lines[-2].split()[1]) > 8 * 10 ** 9
+    assert sum(line.endswith(", 0 mismatches") for line in lines) == 4
+
+
 def test_sum_of_two_16_bit_values_through_fp32_is_the_native_sum(tmp_path):
     """The CUDA-format kernels add two fp16 / bfloat16 values with one fp32 add and one conversion; for every pair
     of finite values of either type that is the correctly rounded 16-bit sum (about half a minute on 8 cores)."""

@@ -39,3 +39,16 @@ def test_exact_quotient_without_a_division_matches_the_division_on_billions_of_p
     assert done.returncode == 0, done.stdout[-2000:]
     assert "MISMATCHES 0" in done.stdout.splitlines()[-1]
     assert done.stdout.count("code mismatches 0") == 8 and done.stdout.count("quotient mismatches 0 ") == 8
+
+
+@pytest.mark.gpu
+def test_code_book_cell_lookup_is_the_search_and_rounding_on_the_device(hip_device):
+    """tests/native/book_cells_check.hip: the one-lookup code-book encoder of the 16-bit quantize kernel (the cell of
+    fma(t, 128, 128), then ``base + (t >= threshold)``) against the search and rounding it stands for, both on the
+    device, for the four books and every float in [-1, 1]."""
+    checker = ROOT / "tests" / "native" / "_build" / "book_cells_check"
+    assert checker.exists(), "run __graft_entry__.build() first"
+    done = subprocess.run([str(checker)], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stdout[-2000:]
+    lines = done.stdout.splitlines()
+    assert lines[-1] == "MISMATCHES 0" and int(lines[-2].split()[1]) > 8 * 10 ** 9

@@ -410,3 +410,31 @@ def test_full_bucket_code_book_decode_is_the_nearest_entry(hip, hip_device, quan
     nearest = (t.unsqueeze(-1) - book).abs().amin(dim=-1)
     achieved = (out.view(-1, g) / scale - t).abs()
     assert bool((achieved <= nearest + 1e-6).all())
+
+
+@pytest.mark.parametrize("name", ("fp16", "bf16"))
+@pytest.mark.parametrize("quant_type", tuple(general.CODE_BOOKS))
+def test_code_books_on_every_16_bit_quotient(hip, hip_device, name, quant_type):
+    """Every finite 16-bit value v with |v| <= top, in groups whose first element is `top`, so that the scale is
+    `top` and the quotients v / top sweep [-1, 1] through every step of the book: with top = 1 the quotient is the
+    value itself, with top = 1.5 and 0.0791 it is a rounded division.  The 16-bit kernels encode these with a table
+    lookup; the bytes must be the oracle's."""
+    g = 64
+    bits = np.arange(0, 0x8000, dtype=np.uint16)
+    for top in (1.0, 1.5, 0.0791):
+        top_bits = wire.from_f32(np.array([top], dtype=np.float32), name)
+        magnitudes = wire.to_f32(bits.view(top_bits.dtype), name)
+        keep = bits[np.isfinite(magnitudes) & (magnitudes <= wire.to_f32(top_bits, name)[0])]
+        both = np.concatenate([keep, keep | 0x8000]).astype(np.uint16)
+        rows = -(-both.size // (g - 1))
+        padded = np.zeros(rows * (g - 1), dtype=np.uint16)
+        padded[:both.size] = both
+        x_bits = np.empty((rows, g), dtype=np.uint16)
+        x_bits[:, 0] = top_bits.view(np.uint16)[0]
+        x_bits[:, 1:] = padded.reshape(rows, g - 1)
+        x_np = x_bits.reshape(-1).view(top_bits.dtype)
+        x = from_numpy(x_np, name, hip_device)
+        n = x_np.size
+        payload = torch.empty(hip.general_payload_nbytes(n, x.dtype, g, 4, 0), dtype=torch.uint8, device=hip_device)
+        assert hip.quant_general_into(x, payload, group_size=g, bit=4, quant_type=quant_type, compact=True)
+        same(payload, general.quantize(x_np, name, g, 4, quant_type, 0, None, True), f"{name} {quant_type} top={top}")
