@@ -8,9 +8,7 @@
 // [-1, 1] is cut into 256 cells of width 1/128, none of which holds two steps.  A cell stores the code at its left
 // end and the step inside it, if any, so that on the device
 //     code(t) = cell.base + (t >= cell.threshold),   cell = cells[(unsigned)fma(t, 128, 128)]
-// for every finite t in [-1, 1].  The steps alone serve as a second table: the code is the number of steps not
-// above t, found by the reference's own halving search run over the steps instead of the entries, with no
-// rounding stage behind it.  tests/native/check_book_cells.cpp compares all forms on every such float.
+// for every finite t in [-1, 1].  tests/native/check_book_cells.cpp compares the two forms on every such float.
 // Plain C++17 (host and device): no HIP types.
 #pragma once
 #include <cstdint>
@@ -45,11 +43,6 @@ struct Table {
 };
 struct Tables {
     Table book[kBooks];
-};
-// value[k], k = 1..14: the smallest float whose code is k or more; value[0] = -inf and value[15] = +inf close the
-// search, so that "the largest k in [0, 15) with not (t < value[k])" is the code of t.
-struct Steps {
-    float value[kBooks][16];
 };
 
 // The reference's encoder for a number t (not NaN): search, then rounding.
@@ -101,16 +94,6 @@ constexpr Table make_table(const float (&book)[16]) {
     return table;
 }
 
-constexpr Steps make_steps() {
-    Steps steps{};
-    for (int b = 0; b < kBooks; ++b) {
-        steps.value[b][0] = -__builtin_inff();
-        for (int k = 1; k <= 14; ++k) steps.value[b][k] = step_after(kBookSet.value[b], k - 1);
-        steps.value[b][15] = __builtin_inff();
-    }
-    return steps;
-}
-
 // One step per cell at most, or the lookup would miss a step.
 constexpr bool steps_in_separate_cells(const float (&book)[16]) {
     int previous = -1;
@@ -127,16 +110,6 @@ constexpr Tables kTables = {{make_table(kBookSet.value[0]), make_table(kBookSet.
 static_assert(steps_in_separate_cells(kBookSet.value[0]) && steps_in_separate_cells(kBookSet.value[1]) &&
                   steps_in_separate_cells(kBookSet.value[2]) && steps_in_separate_cells(kBookSet.value[3]),
               "a cell of width 1/128 holds two steps of a code book");
-
-constexpr Steps kSteps = make_steps();
-
-// The code as the number of steps not above t, by the halving search.
-constexpr int stepped_code(const float (&steps)[16], float t) {
-    int at = 0;
-    for (int half = 8; half >= 1; half >>= 1)
-        if (!(t < steps[at + half])) at += half;
-    return at;
-}
 
 // The lookup, as the device does it.
 constexpr int cell_code(const Table &table, float t) {

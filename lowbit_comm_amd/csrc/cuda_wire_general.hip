@@ -32,7 +32,6 @@ namespace {
 // inner.cuh:9-35, and the one-lookup form of the encoder built from them at compile time
 __constant__ book_cells::Books kCodeBooks = book_cells::kBookSet;
 __constant__ book_cells::Tables kBookCells = book_cells::kTables;
-__constant__ book_cells::Steps kBookSteps = book_cells::kSteps;
 
 // Philox4x32-10: one block of four 32-bit words.
 __device__ __forceinline__ void philox_block(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
@@ -70,19 +69,6 @@ __device__ __forceinline__ const float *wave_code_book(int kind, int lane) {
     return book;
 }
 
-// The same for the quantizer, with the book's table of steps (code_book_cells.h) behind the sixteen entries.
-__device__ __forceinline__ const float *wave_code_book_and_steps(int kind, int lane) {
-    __shared__ float tables[kWavesPerBlock][32];
-    float *table = tables[threadIdx.x >> 6];
-    if (kind != 0) {
-        if (lane < 32) table[lane] = lane < 16 ? kCodeBooks.value[kind - 1][lane] : kBookSteps.value[kind - 1][lane - 16];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
-    return table;
-}
-
 // The workgroup's copy of a book's cell table (code_book_cells.h) in LDS.  Every wavefront of the workgroup must
 // come here: the copy ends in a workgroup barrier.
 __device__ __forceinline__ const book_cells::Cell *block_book_cells(int kind) {
@@ -98,8 +84,15 @@ __device__ __forceinline__ const book_cells::Cell *block_book_cells(int kind) {
 __device__ __forceinline__ int meta_words_of(int topk) { return topk == 0 ? 1 : topk + 2; }
 
 // ---------------------------------------------------------------------------------------------
-// quantize: one wavefront per tile of 64 * VEC elements
+// quantize: a wavefront works on tiles of 64 * VEC elements (64 lanes x 16 bytes of the tensor)
 // ---------------------------------------------------------------------------------------------
+// Tiles per wavefront: 32 bytes of the tensor per lane either way.  A 32-bit tensor's wavefront asks for both of
+// its tiles before it does anything else and encodes one while the other is on its way (26.2 M fp32 elements:
+// stochastic rounding 28.8 instead of 37.4 us, top-2 30.3 instead of 30.8, a code book 28.2 instead of 30.0);
+// four tiles are slower again (32.7 us top-2), and so are two tiles of eight 16-bit elements a lane (bf16 top-2
+// 25.9 instead of 23.2 us): the kernels are bound by instruction issue and need their eight wavefronts per SIMD.
+template <typename T> constexpr int general_quant_tiles() { return sizeof(T) == 4 ? 2 : 1; }
+
 // FIXED names what the launch knows about the policy at compile time, so that the code of the other policies
 // is not part of the kernel: bit 0 "no outlier channel", bit 1 "round to nearest", bit 2 "linear codes".
 // 0 is the kernel for every policy.
@@ -115,29 +108,75 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     constexpr bool WIDE = ITEM == 4;
     static_assert(LPG >= 2 && LPG <= 16, "a group must span 2..16 lanes of one DPP row");
 
+    constexpr int TILES = general_quant_tiles<T>();
     const int lane = threadIdx.x & (kWave - 1);
     const int meta_bytes = meta_words_of(topk) * ITEM;
     const int64_t groups = a.numel / G;
-    const int64_t tile_first = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * W::TILE;
+    const int64_t first = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * (TILES * W::TILE);
+
+    // all of the wavefront's elements are asked for before anything else
+    Raw raws[TILES][VEC];
+#pragma unroll
+    for (int tile = 0; tile < TILES; ++tile) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) raws[tile][i] = 0;
+        const int64_t e0 = first + tile * W::TILE + lane * VEC;
+        // numel is a multiple of G: dead lanes form whole dead groups.  Instruction-bound: a cache hint only costs.
+        if (e0 < a.numel) load_elems<Raw, VEC, kPlain>(static_cast<const Raw *>(a.x) + e0, raws[tile]);
+    }
+    // After the loads were issued: the waits of the tables cover theirs.  The cell table pays for its copy and its
+    // barrier with the eight elements a lane has here (26.2 M bf16 elements: 20.1 us against 24.6 us with the
+    // search and rounding; fp32, two tiles: 28.0 against 30.0 us); with four it did not (33.3 against 32.2 us).
+    const bool by_cells = kind != 0 && !stochastic;   // uniform over the grid
+    const book_cells::Cell *cells = by_cells ? block_book_cells(kind) : nullptr;
+    if (first >= a.numel) return;   // wavefront-uniform, behind the workgroup's barrier
+    const float *book = wave_code_book(kind, lane);
+
+    auto encode_tile = [&](const int64_t tile_first, const Raw (&raw)[VEC]) __attribute__((always_inline)) {
     const int64_t e0 = tile_first + lane * VEC;
-    const bool live = e0 < a.numel;      // numel is a multiple of G: dead lanes form whole dead groups
+    const bool live = e0 < a.numel;
     const int64_t group = e0 / G;
     const int k0 = static_cast<int>(e0 - group * G);
     const int start = scan_start<T, G>(group);
-
-    Raw raw[VEC];
+    // The draws depend on the element's place only.
+    float uniform[VEC];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) raw[i] = 0;
-    if (live) load_elems<Raw, VEC, kPlain>(static_cast<const Raw *>(a.x) + e0, raw);   // instruction-bound: the hint only costs
-    // After the loads were issued: the waits of the tables cover theirs.  The cell table pays for its copy and its
-    // barrier with eight elements a lane (26.2 M bf16 elements: 20.1 us against 24.6 us with the search), not with
-    // the four of a 32-bit tensor (33.3 against 32.2 us, although a wavefront issues 125 vector instructions
-    // instead of 187); those search the table of steps, which needs no barrier.
-    constexpr bool CELLS = ITEM == 2;
-    const bool by_cells = CELLS && kind != 0 && !stochastic;   // uniform over the grid
-    const book_cells::Cell *cells = by_cells ? block_book_cells(kind) : nullptr;
-    if (tile_first >= a.numel) return;   // wavefront-uniform, behind the workgroup's barrier
-    const float *book = wave_code_book_and_steps(kind, lane);
+    for (int i = 0; i < VEC; ++i) uniform[i] = 0.0f;
+    auto draw = [&]() __attribute__((always_inline)) {
+    if (stochastic) {
+        const uint32_t key0 = static_cast<uint32_t>(a.seed), key1 = static_cast<uint32_t>(a.seed >> 32);
+        const uint32_t sub0 = static_cast<uint32_t>(group), sub1 = static_cast<uint32_t>(static_cast<uint64_t>(group) >> 32);
+        const int phase = static_cast<int>(a.offset & 3);
+        auto to_uniform = [](uint32_t x) { return static_cast<float>(x) * 0x1p-32f + 0x1p-33f; };   // curand_uniform: (0, 1]
+        uint64_t block[VEC / 4];
+#pragma unroll
+        for (int q = 0; q < VEC / 4; ++q)
+            block[q] = (a.offset + static_cast<uint64_t>((k0 + 4 * q - start) & (G - 1))) >> 2;   // positions are multiples of 4
+        uint32_t lo[VEC / 4][4];
+#pragma unroll
+        for (int q = 0; q < VEC / 4; ++q)
+            philox_block(static_cast<uint32_t>(block[q]), static_cast<uint32_t>(block[q] >> 32), sub0, sub1, key0, key1, lo[q]);
+        if (phase == 0) {   // uniform; the offsets torch hands out are multiples of four: one block a quad
+#pragma unroll
+            for (int q = 0; q < VEC / 4; ++q)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) uniform[4 * q + e] = to_uniform(lo[q][e]);
+        } else {            // a quad's draws lie across two blocks
+#pragma unroll
+            for (int q = 0; q < VEC / 4; ++q) {
+                uint32_t hi[4];
+                philox_block(static_cast<uint32_t>(block[q] + 1), static_cast<uint32_t>((block[q] + 1) >> 32), sub0, sub1,
+                             key0, key1, hi);
+                const uint32_t w[8] = {lo[q][0], lo[q][1], lo[q][2], lo[q][3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    uniform[4 * q + e] = to_uniform(phase == 1 ? w[e + 1] : (phase == 2 ? w[e + 2] : w[e + 3]));
+            }
+        }
+    }
+    };
+    draw();   // while the element's value is still on its way
+
     float v[VEC];
     uint32_t mag[VEC];
 #pragma unroll
@@ -230,31 +269,6 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     float scale = value_of<T>(scale_raw);
     scale = scale < 1.0e-6f ? 1.0e-6f : scale;   // a NaN scale stays NaN and encodes every element as 0
 
-    float uniform[VEC];
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) uniform[i] = 0.0f;
-    if (stochastic) {
-        const uint32_t key0 = static_cast<uint32_t>(a.seed), key1 = static_cast<uint32_t>(a.seed >> 32);
-        const uint32_t sub0 = static_cast<uint32_t>(group), sub1 = static_cast<uint32_t>(static_cast<uint64_t>(group) >> 32);
-        const int phase = static_cast<int>(a.offset & 3);
-#pragma unroll
-        for (int q = 0; q < VEC / 4; ++q) {
-            const uint64_t position = static_cast<uint64_t>((k0 + 4 * q - start) & (G - 1));   // a multiple of 4
-            const uint64_t block = (a.offset + position) >> 2;
-            uint32_t lo[4], hi[4] = {0, 0, 0, 0};
-            philox_block(static_cast<uint32_t>(block), static_cast<uint32_t>(block >> 32), sub0, sub1, key0, key1, lo);
-            if (phase != 0)
-                philox_block(static_cast<uint32_t>(block + 1), static_cast<uint32_t>((block + 1) >> 32), sub0, sub1, key0,
-                             key1, hi);
-            const uint32_t w[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const uint32_t x = phase == 0 ? w[e] : (phase == 1 ? w[e + 1] : (phase == 2 ? w[e + 2] : w[e + 3]));
-                uniform[4 * q + e] = static_cast<float>(x) * 0x1p-32f + 0x1p-33f;   // curand_uniform: (0, 1]
-            }
-        }
-    }
-
     int c[VEC];
     if (kind == 0) {
         const float multiplier = W::LEVELS / scale;
@@ -303,23 +317,6 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
                 const book_cells::Cell cell = cells[static_cast<uint32_t>(__builtin_fmaf(t[i], 128.0f, 128.0f))];
                 c[i] = static_cast<int>(cell.base) + (t[i] >= cell.threshold ? 1 : 0);
             }
-        } else if (usual && !stochastic) {
-            // Every t is a number in [-1, 1]: the code is the number of the book's steps not above t, found by the
-            // halving search below run over the table of steps, with no rounding stage behind it.
-            const char *step_bytes = reinterpret_cast<const char *>(book + 16);
-            int at[VEC];
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) at[i] = 0;
-#pragma unroll
-            for (int half = 8 * 4; half >= 4; half >>= 1) {
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) {
-                    const int mid = at[i] + half;
-                    at[i] = !(t[i] < *reinterpret_cast<const float *>(step_bytes + mid)) ? mid : at[i];
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) c[i] = at[i] >> 2;
         } else {
         // The largest entry in [0, 14] with not (t < book[entry]); a NaN ends at 14.  Four halving steps, each
         // over all of the lane's elements so that their LDS reads are in flight together; positions are kept as
@@ -358,6 +355,13 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
         uint32_t words[W::WORDS];
         pack_codes<T, BIT, VEC, W::WORDS>(c, words);
         store_piece<T, BIT, kPlain, W::WORDS>(group_codes + piece_offset<T, BIT>(k0), words);
+    }
+    };
+#pragma unroll
+    for (int tile = 0; tile < TILES; ++tile) {
+        const int64_t tile_first = first + tile * W::TILE;
+        if (tile_first >= a.numel) return;   // wavefront-uniform
+        encode_tile(tile_first, raws[tile]);
     }
 }
 
@@ -439,7 +443,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
 
 template <typename T, int G>
 hipError_t launch_general_quant_g(int bit, const WireGeneralQuantArgs &a, hipStream_t stream) {
-    const int64_t tile = wire<T, 8>::TILE * kWavesPerBlock;
+    const int64_t tile = wire<T, 8>::TILE * kWavesPerBlock * general_quant_tiles<T>();
     const int64_t blocks = (a.numel + tile - 1) / tile;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;

@@ -1,7 +1,6 @@
 // Device check of the one-lookup code-book encoder (lowbit_comm_amd/csrc/code_book_cells.h): for each of the four
 // books and every float t in [-1, 1], the lookup as the quantize kernel does it - the cell of fma(t, 128, 128)
-// converted to an unsigned integer, then `base + (t >= threshold)` - and the halving search over the table of
-// steps that the 32-bit kernel runs, against the search and rounding step they stand
+// converted to an unsigned integer, then `base + (t >= threshold)` - against the search and rounding step it stands
 // for (ccdl_comm/csrc/quantization/inner.cuh:74-118), both evaluated on the device.  Prints "MISMATCHES n";
 // exit status 1 when n is not 0.
 #include <hip/hip_runtime.h>
@@ -14,7 +13,6 @@ namespace bc = lbc::book_cells;
 
 __constant__ bc::Books kBooks = bc::kBookSet;
 __constant__ bc::Tables kCells = bc::kTables;
-__constant__ bc::Steps kStepTable = bc::kSteps;
 
 __global__ void compare(int book_index, uint32_t first_key, uint64_t count, unsigned long long *bad) {
     const float *book = kBooks.value[book_index];
@@ -33,11 +31,6 @@ __global__ void compare(int book_index, uint32_t first_key, uint64_t count, unsi
         const bc::Cell cell = cells[static_cast<uint32_t>(__builtin_fmaf(t, 128.0f, 128.0f))];
         const int looked_up = static_cast<int>(cell.base) + (t >= cell.threshold ? 1 : 0);
         mine += searched != looked_up;
-        const float *steps = kStepTable.value[book_index];
-        int stepped = 0;
-        for (int half = 8; half >= 1; half >>= 1)
-            if (!(t < steps[stepped + half])) stepped += half;
-        mine += searched != stepped;
     }
     if (mine) atomicAdd(bad, mine);
 }

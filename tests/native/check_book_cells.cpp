@@ -1,6 +1,5 @@
 // Host check of the one-lookup code-book encoder (lowbit_comm_amd/csrc/code_book_cells.h): on every float in
-// [-1, 1], for each of the four books, the cell lookup and the search over the steps must give the code of the
-// search-and-round form
+// [-1, 1], for each of the four books, the cell lookup must give the code of the search-and-round form
 // (ccdl_comm/csrc/quantization/inner.cuh:74-118), evaluated here at run time with ordinary float arithmetic.
 // Build: g++ -O2 -std=c++17 -ffp-contract=off -fopenmp check_book_cells.cpp.  Prints "MISMATCHES n".
 #include <cstdint>
@@ -38,9 +37,7 @@ int main(int argc, char **argv) {
             const float u = __builtin_fmaf(t, 128.0f, 128.0f);
             const bc::Cell &cell = table.cell[static_cast<uint32_t>(u)];
             const int got = static_cast<int>(cell.base) + (t >= cell.threshold ? 1 : 0);
-            const int want = searched(book, t);
-            bad += got != want;
-            bad += bc::stepped_code(bc::kSteps.value[b], t) != want;
+            bad += got != searched(book, t);
             ++seen;
         }
         // every step itself and the float before it, whatever the stride

@@ -110,7 +110,7 @@ def test_division_free_quotient_matches_the_division_next_to_every_tie(tmp_path)
 
 
 def test_code_book_cell_lookup_is_the_search_and_rounding_on_every_float(tmp_path):
-    """The code-book quantizer of the CUDA byte format encodes a 16-bit tensor's quotients with one table lookup
+    """The code-book quantizer of the CUDA byte format encodes the quotients with one table lookup
     (csrc/code_book_cells.h, tables built at compile time).  For each of the four books and every float in [-1, 1]
     (8.5e9 values, about 15 s on 8 cores) the lookup gives the code of the reference's search and rounding step, and
     every step of the table is checked on both sides whatever the stride."""

@@ -43,7 +43,7 @@ def test_exact_quotient_without_a_division_matches_the_division_on_billions_of_p
 
 @pytest.mark.gpu
 def test_code_book_cell_lookup_is_the_search_and_rounding_on_the_device(hip_device):
-    """tests/native/book_cells_check.hip: the one-lookup code-book encoder of the 16-bit quantize kernel (the cell of
+    """tests/native/book_cells_check.hip: the one-lookup code-book encoder of the quantize kernel (the cell of
     fma(t, 128, 128), then ``base + (t >= threshold)``) against the search and rounding it stands for, both on the
     device, for the four books and every float in [-1, 1]."""
     checker = ROOT / "tests" / "native" / "_build" / "book_cells_check"

@@ -417,8 +417,8 @@ def test_full_bucket_code_book_decode_is_the_nearest_entry(hip, hip_device, quan
 def test_code_books_on_every_16_bit_quotient(hip, hip_device, name, quant_type):
     """Every finite 16-bit value v with |v| <= top, in groups whose first element is `top`, so that the scale is
     `top` and the quotients v / top sweep [-1, 1] through every step of the book: with top = 1 the quotient is the
-    value itself, with top = 1.5 and 0.0791 it is a rounded division.  The 16-bit kernels encode these with a table
-    lookup; the bytes must be the oracle's."""
+    value itself, with top = 1.5 and 0.0791 it is a rounded division.  The kernels encode these with a table lookup;
+    the bytes must be the oracle's."""
     g = 64
     bits = np.arange(0, 0x8000, dtype=np.uint16)
     for top in (1.0, 1.5, 0.0791):
