@@ -82,8 +82,36 @@ __device__ __forceinline__ void load_piece16(buffer_t b, uint32_t at, uint32_t (
 // other layouts.
 template <int NT, int WORLD> constexpr int window_policy() { return NT == kNonTemporal && WORLD >= 4 ? kNtBit : kCached; }
 
-// (Stores to such positions stay misaligned 8-byte stores: splitting them into short, aligned dword, short
-// made the ring's gather hop 30 % slower, 56.5 against 43.0 us on 52 M bf16 elements.)
+// Stores to such positions are misaligned 8-byte stores in most kernels.  Splitting one into short, aligned dword,
+// short made the ring's gather hop 30 % slower (56.5 against 43.0 us on 52 M bf16 elements).  What pays, on the
+// gather hop of large chunks and together with the non-temporal hint, is to shift the bytes across lanes instead: a DPP row holds two groups, lanes 0-7 the even one, whose codes start on a dword when the payload
+// does, and lanes 8-15 the odd one, whose 66 bytes start two bytes into a dword.  The pair is 33 dwords:
+//   D[0..15]  the even group's codes, two dwords a lane, as they are;
+//   D[16+j], j = 0..15: the odd group's code dwords moved up by two bytes, alignbit(in[j], in[j - 1], 16), where
+//             in[-1] is the even group's scale in its upper half - so D[16] carries that scale;
+//   D[32]     the odd group's last two code bytes and its scale.
+// in[j - 1] is the lane's own first dword or the second dword of the lane before it (row_shr:1).  Every lane of the
+// row must call this (live or not); `pair` points at the even group's codes and is 4-byte aligned; `scale` is the
+// group's 16-bit scale, the same in its eight lanes; when the odd group lies past the end, the even group's scale is
+// written by itself.
+template <int POLICY>
+__device__ __forceinline__ void store_group_pair16(uint8_t *pair, int lane, const uint32_t (&words)[2], uint32_t scale, bool live,
+                                                   bool odd_group_live) {
+    const int row_lane = lane & 15, l = row_lane & 7;
+    const bool odd = (row_lane & 8) != 0;
+    const uint32_t before = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(words[1]), 0x111, 0xF, 0xF, true));
+    const uint32_t even_scale = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(scale), 0x118, 0xF, 0xF, true));
+    const uint32_t previous = l == 0 ? even_scale << 16 : before;
+    uint32_t out[2] = {words[0], words[1]};
+    if (odd) {
+        out[0] = __builtin_amdgcn_alignbit(words[0], previous, 16);
+        out[1] = __builtin_amdgcn_alignbit(words[1], words[0], 16);
+    }
+    if (!live) return;
+    store_words<2, 4, POLICY>(pair + (odd ? 64 : 0) + 8 * l, out);
+    if (row_lane == 15) *reinterpret_cast<uint32_t *>(pair + 128) = (words[1] >> 16) | (scale << 16);
+    if (row_lane == 0 && !odd_group_live) *reinterpret_cast<uint16_t *>(pair + 64) = static_cast<uint16_t>(scale);
+}
 
 // The value lane 7 (lanes 0-7) or lane 15 (lanes 8-15) of the caller's row holds: the last lane of an 8-lane group.
 __device__ __forceinline__ uint32_t from_last_lane_of_8(uint32_t v, bool upper_half) {

@@ -577,7 +577,7 @@ def test_ring_steps_captured_in_a_hip_graph_replay_like_eager(hip_device):
 # --------------------------------------------------------------------------- #
 # the same hop in the CUDA extension's byte format
 # --------------------------------------------------------------------------- #
-def check_wire_step(device, dtype, g, n, compact, reduce_op, divisor, emit, seed, poison=False, lead=0):
+def check_wire_step(device, dtype, g, n, compact, reduce_op, divisor, emit, seed, poison=False, lead=0, send_lead=0):
     from lowbit_comm_amd.hip import cuda_wire
 
     tdtype = DTYPES[dtype]
@@ -593,7 +593,10 @@ def check_wire_step(device, dtype, g, n, compact, reduce_op, divisor, emit, seed
         chunk[3 * g - 1] = float("nan")           # a NaN that ends a group's scan
         chunk[5] = float("inf")
     before = to_np(chunk, dtype)
-    send = torch.full((cuda_wire.payload_nbytes(n, tdtype, g),), 0xAB, dtype=torch.uint8, device=device) if emit else None
+    send = None
+    if emit:                                      # send_lead: the outgoing payload at a 2-byte aligned address
+        room = torch.full((cuda_wire.payload_nbytes(n, tdtype, g) + send_lead + 16,), 0xAB, dtype=torch.uint8, device=device)
+        send = room[send_lead:send_lead + cuda_wire.payload_nbytes(n, tdtype, g)]
     assert cuda_wire.ring_step_into(received, chunk, send, group_size=g, compact=compact, reduce_op=reduce_op,
                                     divisor=divisor)
     codec = ring_np.CudaWireCodec(g, compact=compact)
@@ -603,6 +606,20 @@ def check_wire_step(device, dtype, g, n, compact, reduce_op, divisor, emit, seed
     assert np.array_equal(raw(to_np(chunk, dtype)), raw(want_chunk)), what
     if emit:
         assert np.array_equal(send.cpu().numpy(), want_payload), what
+        assert bool((room[:send_lead] == 0xAB).all()) and bool((room[send_lead + send.numel():] == 0xAB).all()), what
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_wire_gather_hop_of_a_large_chunk_bit_exact(hip_device, dtype):
+    """From 16 Mi elements on, the hop that only decodes and requantizes writes a 16-bit payload with interleaved
+    scales as whole dwords shifted across lanes.  An odd number of groups (the last group has no partner), an even
+    one with NaNs and an infinity in the chunk, and an outgoing payload at a 2-byte aligned address (the kernel's
+    other store path at this size); bytes around the payload stay untouched."""
+    groups = 1 << 18
+    check_wire_step(hip_device, dtype, 64, 64 * (groups + 1), True, "none", 1.0, True, 81_000)
+    check_wire_step(hip_device, dtype, 64, 64 * (groups + 2), True, "none", 1.0, True, 81_002, poison=True)
+    check_wire_step(hip_device, dtype, 64, 64 * (groups + 3), True, "none", 1.0, True, 81_004, lead=2, send_lead=2)
+    check_wire_step(hip_device, dtype, 64, 64 * (groups + 5), True, "sum", 8.0, True, 81_006)
 
 
 @pytest.mark.parametrize("compact", [True, False])
