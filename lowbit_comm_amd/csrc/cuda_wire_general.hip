@@ -133,229 +133,226 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     const float *book = wave_code_book(kind, lane);
 
     auto encode_tile = [&](const int64_t tile_first, const Raw (&raw)[VEC]) __attribute__((always_inline)) {
-    const int64_t e0 = tile_first + lane * VEC;
-    const bool live = e0 < a.numel;
-    const int64_t group = e0 / G;
-    const int k0 = static_cast<int>(e0 - group * G);
-    const int start = scan_start<T, G>(group);
-    // The draws depend on the element's place only.
-    float uniform[VEC];
+        const int64_t e0 = tile_first + lane * VEC;
+        const bool live = e0 < a.numel;
+        const int64_t group = e0 / G;
+        const int k0 = static_cast<int>(e0 - group * G);
+        const int start = scan_start<T, G>(group);
+        // The draws depend on the element's place only: they are computed while its value is still on its way.
+        float uniform[VEC];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) uniform[i] = 0.0f;
-    auto draw = [&]() __attribute__((always_inline)) {
-    if (stochastic) {
-        const uint32_t key0 = static_cast<uint32_t>(a.seed), key1 = static_cast<uint32_t>(a.seed >> 32);
-        const uint32_t sub0 = static_cast<uint32_t>(group), sub1 = static_cast<uint32_t>(static_cast<uint64_t>(group) >> 32);
-        const int phase = static_cast<int>(a.offset & 3);
-        auto to_uniform = [](uint32_t x) { return static_cast<float>(x) * 0x1p-32f + 0x1p-33f; };   // curand_uniform: (0, 1]
-        uint64_t block[VEC / 4];
-#pragma unroll
-        for (int q = 0; q < VEC / 4; ++q)
-            block[q] = (a.offset + static_cast<uint64_t>((k0 + 4 * q - start) & (G - 1))) >> 2;   // positions are multiples of 4
-        uint32_t lo[VEC / 4][4];
-#pragma unroll
-        for (int q = 0; q < VEC / 4; ++q)
-            philox_block(static_cast<uint32_t>(block[q]), static_cast<uint32_t>(block[q] >> 32), sub0, sub1, key0, key1, lo[q]);
-        if (phase == 0) {   // uniform; the offsets torch hands out are multiples of four: one block a quad
+        for (int i = 0; i < VEC; ++i) uniform[i] = 0.0f;
+        if (stochastic) {
+            const uint32_t key0 = static_cast<uint32_t>(a.seed), key1 = static_cast<uint32_t>(a.seed >> 32);
+            const uint32_t sub0 = static_cast<uint32_t>(group), sub1 = static_cast<uint32_t>(static_cast<uint64_t>(group) >> 32);
+            const int phase = static_cast<int>(a.offset & 3);
+            auto to_uniform = [](uint32_t x) { return static_cast<float>(x) * 0x1p-32f + 0x1p-33f; };   // curand_uniform: (0, 1]
+            uint64_t block[VEC / 4];
 #pragma unroll
             for (int q = 0; q < VEC / 4; ++q)
+                block[q] = (a.offset + static_cast<uint64_t>((k0 + 4 * q - start) & (G - 1))) >> 2;   // positions are multiples of 4
+            uint32_t lo[VEC / 4][4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) uniform[4 * q + e] = to_uniform(lo[q][e]);
-        } else {            // a quad's draws lie across two blocks
+            for (int q = 0; q < VEC / 4; ++q)
+                philox_block(static_cast<uint32_t>(block[q]), static_cast<uint32_t>(block[q] >> 32), sub0, sub1, key0, key1, lo[q]);
+            if (phase == 0) {   // uniform; the offsets torch hands out are multiples of four: one block a quad
 #pragma unroll
-            for (int q = 0; q < VEC / 4; ++q) {
-                uint32_t hi[4];
-                philox_block(static_cast<uint32_t>(block[q] + 1), static_cast<uint32_t>((block[q] + 1) >> 32), sub0, sub1,
-                             key0, key1, hi);
-                const uint32_t w[8] = {lo[q][0], lo[q][1], lo[q][2], lo[q][3], hi[0], hi[1], hi[2], hi[3]};
+                for (int q = 0; q < VEC / 4; ++q)
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    uniform[4 * q + e] = to_uniform(phase == 1 ? w[e + 1] : (phase == 2 ? w[e + 2] : w[e + 3]));
+                    for (int e = 0; e < 4; ++e) uniform[4 * q + e] = to_uniform(lo[q][e]);
+            } else {            // a quad's draws lie across two blocks
+#pragma unroll
+                for (int q = 0; q < VEC / 4; ++q) {
+                    uint32_t hi[4];
+                    philox_block(static_cast<uint32_t>(block[q] + 1), static_cast<uint32_t>((block[q] + 1) >> 32), sub0, sub1,
+                                 key0, key1, hi);
+                    const uint32_t w[8] = {lo[q][0], lo[q][1], lo[q][2], lo[q][3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        uniform[4 * q + e] = to_uniform(phase == 1 ? w[e + 1] : (phase == 2 ? w[e + 2] : w[e + 3]));
+                }
             }
         }
-    }
-    };
-    draw();   // while the element's value is still on its way
 
-    float v[VEC];
-    uint32_t mag[VEC];
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-        v[i] = value_of<T>(raw[i]);
-        mag[i] = raw[i] & RB::ABS;
-    }
-
-    uint8_t *group_codes = a.payload + (a.compact ? group * (CB + meta_bytes) : group * CB);
-    uint8_t *group_meta = a.compact ? group_codes + CB : a.payload + groups * CB + group * meta_bytes;
-
-    uint32_t scale_raw;
-    if (topk == 0) {
-        scale_raw = running_max_raw<T, G, VEC>(mag, k0, start);
-    } else {
-        // Three rounds of "largest remaining candidate": the group maximum of the magnitude keys, then, among
-        // the elements that hold it, the maximum of the tie-break ranks (1..G, unique inside a group).
-        // A 16-bit magnitude and its rank share one 32-bit key, so a round is a single reduction there.
-        uint32_t key[VEC], rank[VEC];
+        float v[VEC];
+        uint32_t mag[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
-            const int pos = (k0 + i - start) & (G - 1);
-            const bool candidate = WIDE ? mag[i] <= RB::INF : (mag[i] != 0 && mag[i] <= RB::INF);
-            rank[i] = static_cast<uint32_t>(WIDE ? k0 + i + 1 : G - pos);     // the larger rank wins a tie
-            const uint32_t joined = WIDE ? mag[i] : ((mag[i] << 7) | (rank[i] - 1));
-            key[i] = candidate ? joined + 1 : 0;                              // 0 stands for "none"
+            v[i] = value_of<T>(raw[i]);
+            mag[i] = raw[i] & RB::ABS;
         }
-        uint32_t best_key[3] = {0, 0, 0}, best_rank[2] = {0, 0};              // magnitude + 1, rank
+
+        uint8_t *group_codes = a.payload + (a.compact ? group * (CB + meta_bytes) : group * CB);
+        uint8_t *group_meta = a.compact ? group_codes + CB : a.payload + groups * CB + group * meta_bytes;
+
+        uint32_t scale_raw;
+        if (topk == 0) {
+            scale_raw = running_max_raw<T, G, VEC>(mag, k0, start);
+        } else {
+            // Three rounds of "largest remaining candidate": the group maximum of the magnitude keys, then, among
+            // the elements that hold it, the maximum of the tie-break ranks (1..G, unique inside a group).
+            // A 16-bit magnitude and its rank share one 32-bit key, so a round is a single reduction there.
+            uint32_t key[VEC], rank[VEC];
 #pragma unroll
-        for (int round = 0; round < 3; ++round) {
-            if (round == 2 && topk == 1) break;                             // uniform
-            uint32_t m = 0;
+            for (int i = 0; i < VEC; ++i) {
+                const int pos = (k0 + i - start) & (G - 1);
+                const bool candidate = WIDE ? mag[i] <= RB::INF : (mag[i] != 0 && mag[i] <= RB::INF);
+                rank[i] = static_cast<uint32_t>(WIDE ? k0 + i + 1 : G - pos);     // the larger rank wins a tie
+                const uint32_t joined = WIDE ? mag[i] : ((mag[i] << 7) | (rank[i] - 1));
+                key[i] = candidate ? joined + 1 : 0;                              // 0 stands for "none"
+            }
+            uint32_t best_key[3] = {0, 0, 0}, best_rank[2] = {0, 0};              // magnitude + 1, rank
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) m = key[i] > m ? key[i] : m;
-            m = group_max_bits<LPG>(m);
-            if constexpr (WIDE) {
-                best_key[round] = m;
-                if (round == 2) break;
-                uint32_t r = 0;
+            for (int round = 0; round < 3; ++round) {
+                if (round == 2 && topk == 1) break;                             // uniform
+                uint32_t m = 0;
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) r = (key[i] == m && rank[i] > r) ? rank[i] : r;
-                r = group_max_bits<LPG>(r);
-                r = m == 0 ? 0 : r;
-                best_rank[round] = r;
+                for (int i = 0; i < VEC; ++i) m = key[i] > m ? key[i] : m;
+                m = group_max_bits<LPG>(m);
+                if constexpr (WIDE) {
+                    best_key[round] = m;
+                    if (round == 2) break;
+                    uint32_t r = 0;
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) key[i] = (key[i] == m && rank[i] == r) ? 0 : key[i];   // taken
+                    for (int i = 0; i < VEC; ++i) r = (key[i] == m && rank[i] > r) ? rank[i] : r;
+                    r = group_max_bits<LPG>(r);
+                    r = m == 0 ? 0 : r;
+                    best_rank[round] = r;
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) key[i] = (key[i] == m && rank[i] == r) ? 0 : key[i];   // taken
+                } else {
+                    best_key[round] = m == 0 ? 0 : ((m - 1) >> 7) + 1;
+                    if (round == 2) break;
+                    best_rank[round] = m == 0 ? 0 : ((m - 1) & 0x7Fu) + 1;
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) key[i] = (key[i] == m && m != 0) ? 0 : key[i];          // taken
+                }
+            }
+            auto index_of = [&](uint32_t r) {
+                return WIDE ? static_cast<int>(r) - 1 : ((G - static_cast<int>(r)) + start) & (G - 1);
+            };
+            const bool none = best_key[0] == 0;
+            const int index1 = none ? 0 : index_of(best_rank[0]);
+            int index2 = -1;
+            if (topk == 1) {
+                // nothing comparable: the reference falls back to element 1 (as stored for fp32, its magnitude otherwise)
+                const uint32_t element1 = WIDE ? static_cast<uint32_t>(raw[1]) : mag[1];
+                const uint32_t fallback = static_cast<uint32_t>(__shfl(static_cast<int>(element1), lane & ~(LPG - 1)));
+                scale_raw = none ? fallback : (best_key[1] == 0 ? 0u : best_key[1] - 1);
             } else {
-                best_key[round] = m == 0 ? 0 : ((m - 1) >> 7) + 1;
-                if (round == 2) break;
-                best_rank[round] = m == 0 ? 0 : ((m - 1) & 0x7Fu) + 1;
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) key[i] = (key[i] == m && m != 0) ? 0 : key[i];          // taken
+                const bool lonely = !none && best_key[1] == 0;
+                index2 = none ? 1 : (lonely ? ((index1 + 1) & (G - 1)) : index_of(best_rank[1]));
+                scale_raw = (none || lonely || best_key[2] == 0) ? 0u : best_key[2] - 1;
             }
-        }
-        auto index_of = [&](uint32_t r) {
-            return WIDE ? static_cast<int>(r) - 1 : ((G - static_cast<int>(r)) + start) & (G - 1);
-        };
-        const bool none = best_key[0] == 0;
-        const int index1 = none ? 0 : index_of(best_rank[0]);
-        int index2 = -1;
-        if (topk == 1) {
-            // nothing comparable: the reference falls back to element 1 (as stored for fp32, its magnitude otherwise)
-            const uint32_t element1 = WIDE ? static_cast<uint32_t>(raw[1]) : mag[1];
-            const uint32_t fallback = static_cast<uint32_t>(__shfl(static_cast<int>(element1), lane & ~(LPG - 1)));
-            scale_raw = none ? fallback : (best_key[1] == 0 ? 0u : best_key[1] - 1);
-        } else {
-            const bool lonely = !none && best_key[1] == 0;
-            index2 = none ? 1 : (lonely ? ((index1 + 1) & (G - 1)) : index_of(best_rank[1]));
-            scale_raw = (none || lonely || best_key[2] == 0) ? 0u : best_key[2] - 1;
-        }
-        Raw top1_raw = 0, top2_raw = 0;
-        bool own1 = false, own2 = false;
+            Raw top1_raw = 0, top2_raw = 0;
+            bool own1 = false, own2 = false;
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            const bool first = k0 + i == index1, second = k0 + i == index2;
-            top1_raw = first ? raw[i] : top1_raw;
-            top2_raw = second ? raw[i] : top2_raw;
-            own1 |= first;
-            own2 |= second;
-            if (first || second) v[i] = 0.0f;
+            for (int i = 0; i < VEC; ++i) {
+                const bool first = k0 + i == index1, second = k0 + i == index2;
+                top1_raw = first ? raw[i] : top1_raw;
+                top2_raw = second ? raw[i] : top2_raw;
+                own1 |= first;
+                own2 |= second;
+                if (first || second) v[i] = 0.0f;
+            }
+            if (live && own1) *reinterpret_cast<Raw *>(group_meta + 2 * ITEM) = top1_raw;   // the owner lanes store
+            if (live && own2) *reinterpret_cast<Raw *>(group_meta + 3 * ITEM) = top2_raw;   // the outliers as they are
+            if (live && k0 == 0)
+                *reinterpret_cast<Raw *>(group_meta + ITEM) =
+                    static_cast<Raw>(topk == 1 ? index1 : (index1 | (index2 << 8)));
         }
-        if (live && own1) *reinterpret_cast<Raw *>(group_meta + 2 * ITEM) = top1_raw;   // the owner lanes store
-        if (live && own2) *reinterpret_cast<Raw *>(group_meta + 3 * ITEM) = top2_raw;   // the outliers as they are
-        if (live && k0 == 0)
-            *reinterpret_cast<Raw *>(group_meta + ITEM) =
-                static_cast<Raw>(topk == 1 ? index1 : (index1 | (index2 << 8)));
-    }
-    if (live && k0 == 0) *reinterpret_cast<Raw *>(group_meta) = static_cast<Raw>(scale_raw);
+        if (live && k0 == 0) *reinterpret_cast<Raw *>(group_meta) = static_cast<Raw>(scale_raw);
 
-    float scale = value_of<T>(scale_raw);
-    scale = scale < 1.0e-6f ? 1.0e-6f : scale;   // a NaN scale stays NaN and encodes every element as 0
+        float scale = value_of<T>(scale_raw);
+        scale = scale < 1.0e-6f ? 1.0e-6f : scale;   // a NaN scale stays NaN and encodes every element as 0
 
-    int c[VEC];
-    if (kind == 0) {
-        const float multiplier = W::LEVELS / scale;
-        constexpr int L = static_cast<int>(W::LEVELS);
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            // nvcc contracts v * m + noise into one FMA; without noise the product is rounded alone
-            const float t = stochastic ? __builtin_fmaf(v[i], multiplier, uniform[i] - 0.5f) : v[i] * multiplier;
-            const int r = cvt_i32(__builtin_rintf(t));
-            c[i] = r < -L ? -L : (r > L ? L : r);
-        }
-    } else {
-        // t = v / scale, the IEEE quotient.  A lane's elements share the divisor, so the reciprocal part of the
-        // division is done once: v_rcp_f32 and one Newton step, then per element the product and two corrections.
-        // These are the very operations the compiler emits for `v / scale`, minus its operand scaling and
-        // special-case fix-up (v_div_scale / v_div_fmas / v_div_fixup), which change nothing while the divisor
-        // lies in [2^-60, 2^60], |v| <= scale, and the dividend is not so small (below 2^-103) that the division
-        // would rescale it.  The scale is at least 1e-6 here, so such a dividend means a quotient below 2^-80, and a
-        // quotient below 2^-30 encodes as the book's zero whatever its last bits are: it is closer to that entry
-        // than the rounding error of the comparisons with its neighbours.  A wavefront with any other divisor,
-        // or with an element above its scale (only a group that holds a NaN has one) or not a number, takes the
-        // division.  tests/native/quotient_check.hip compares the two forms on the device.
-        float t[VEC];
-        const uint32_t scale_exponent = (as_u32(scale) >> 23) & 0xFFu;
-        bool unusual = scale_exponent < 127u - 60u || scale_exponent > 127u + 60u;
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) unusual |= !(__builtin_fabsf(v[i]) <= scale);
-        const bool usual = __ballot(unusual) == 0;   // wavefront-uniform
-        if (usual) {
-            float reciprocal = __builtin_amdgcn_rcpf(scale);
-            reciprocal = __builtin_fmaf(__builtin_fmaf(-scale, reciprocal, 1.0f), reciprocal, reciprocal);
+        int c[VEC];
+        if (kind == 0) {
+            const float multiplier = W::LEVELS / scale;
+            constexpr int L = static_cast<int>(W::LEVELS);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
-                float q = v[i] * reciprocal;
-                q = __builtin_fmaf(__builtin_fmaf(-scale, q, v[i]), reciprocal, q);
-                t[i] = __builtin_fmaf(__builtin_fmaf(-scale, q, v[i]), reciprocal, q);
+                // nvcc contracts v * m + noise into one FMA; without noise the product is rounded alone
+                const float t = stochastic ? __builtin_fmaf(v[i], multiplier, uniform[i] - 0.5f) : v[i] * multiplier;
+                const int r = cvt_i32(__builtin_rintf(t));
+                c[i] = r < -L ? -L : (r > L ? L : r);
             }
         } else {
+            // t = v / scale, the IEEE quotient.  A lane's elements share the divisor, so the reciprocal part of the
+            // division is done once: v_rcp_f32 and one Newton step, then per element the product and two corrections.
+            // These are the very operations the compiler emits for `v / scale`, minus its operand scaling and
+            // special-case fix-up (v_div_scale / v_div_fmas / v_div_fixup), which change nothing while the divisor
+            // lies in [2^-60, 2^60], |v| <= scale, and the dividend is not so small (below 2^-103) that the division
+            // would rescale it.  The scale is at least 1e-6 here, so such a dividend means a quotient below 2^-80, and a
+            // quotient below 2^-30 encodes as the book's zero whatever its last bits are: it is closer to that entry
+            // than the rounding error of the comparisons with its neighbours.  A wavefront with any other divisor,
+            // or with an element above its scale (only a group that holds a NaN has one) or not a number, takes the
+            // division.  tests/native/quotient_check.hip compares the two forms on the device.
+            float t[VEC];
+            const uint32_t scale_exponent = (as_u32(scale) >> 23) & 0xFFu;
+            bool unusual = scale_exponent < 127u - 60u || scale_exponent > 127u + 60u;
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) t[i] = v[i] / scale;
-        }
-        if (usual && by_cells) {
-            // Every t is a number in [-1, 1]: search and rounding are one table lookup (code_book_cells.h).
+            for (int i = 0; i < VEC; ++i) unusual |= !(__builtin_fabsf(v[i]) <= scale);
+            const bool usual = __ballot(unusual) == 0;   // wavefront-uniform
+            if (usual) {
+                float reciprocal = __builtin_amdgcn_rcpf(scale);
+                reciprocal = __builtin_fmaf(__builtin_fmaf(-scale, reciprocal, 1.0f), reciprocal, reciprocal);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    float q = v[i] * reciprocal;
+                    q = __builtin_fmaf(__builtin_fmaf(-scale, q, v[i]), reciprocal, q);
+                    t[i] = __builtin_fmaf(__builtin_fmaf(-scale, q, v[i]), reciprocal, q);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) t[i] = v[i] / scale;
+            }
+            if (usual && by_cells) {
+                // Every t is a number in [-1, 1]: search and rounding are one table lookup (code_book_cells.h).
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const book_cells::Cell cell = cells[static_cast<uint32_t>(__builtin_fmaf(t[i], 128.0f, 128.0f))];
+                    c[i] = static_cast<int>(cell.base) + (t[i] >= cell.threshold ? 1 : 0);
+                }
+            } else {
+            // The largest entry in [0, 14] with not (t < book[entry]); a NaN ends at 14.  Four halving steps, each
+            // over all of the lane's elements so that their LDS reads are in flight together; positions are kept as
+            // byte offsets into the book.
+            const char *book_bytes = reinterpret_cast<const char *>(book);
+            int at[VEC];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) at[i] = 0;
+#pragma unroll
+            for (int step = 8 * 4; step >= 4; step >>= 1) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const int mid = at[i] + step;
+                    const float entry = *reinterpret_cast<const float *>(book_bytes + mid);
+                    at[i] = (mid < 15 * 4 && !(t[i] < entry)) ? mid : at[i];
+                }
+            }
+            float excess[VEC], gap[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
-                const book_cells::Cell cell = cells[static_cast<uint32_t>(__builtin_fmaf(t[i], 128.0f, 128.0f))];
-                c[i] = static_cast<int>(cell.base) + (t[i] >= cell.threshold ? 1 : 0);
+                const float low = *reinterpret_cast<const float *>(book_bytes + at[i]);
+                gap[i] = *reinterpret_cast<const float *>(book_bytes + at[i] + 4) - low;
+                excess[i] = t[i] - low;
+                c[i] = at[i] >> 2;
             }
-        } else {
-        // The largest entry in [0, 14] with not (t < book[entry]); a NaN ends at 14.  Four halving steps, each
-        // over all of the lane's elements so that their LDS reads are in flight together; positions are kept as
-        // byte offsets into the book.
-        const char *book_bytes = reinterpret_cast<const char *>(book);
-        int at[VEC];
+            if (stochastic) {   // uniform: the second division only runs when it is needed
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) at[i] = 0;
+                for (int i = 0; i < VEC; ++i) c[i] += uniform[i] < excess[i] / gap[i] ? 1 : 0;
+            } else {
 #pragma unroll
-        for (int step = 8 * 4; step >= 4; step >>= 1) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                const int mid = at[i] + step;
-                const float entry = *reinterpret_cast<const float *>(book_bytes + mid);
-                at[i] = (mid < 15 * 4 && !(t[i] < entry)) ? mid : at[i];
+                for (int i = 0; i < VEC; ++i) c[i] += excess[i] > gap[i] * 0.5f ? 1 : 0;
+            }
             }
         }
-        float excess[VEC], gap[VEC];
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            const float low = *reinterpret_cast<const float *>(book_bytes + at[i]);
-            gap[i] = *reinterpret_cast<const float *>(book_bytes + at[i] + 4) - low;
-            excess[i] = t[i] - low;
-            c[i] = at[i] >> 2;
+        if (live) {
+            uint32_t words[W::WORDS];
+            pack_codes<T, BIT, VEC, W::WORDS>(c, words);
+            store_piece<T, BIT, kPlain, W::WORDS>(group_codes + piece_offset<T, BIT>(k0), words);
         }
-        if (stochastic) {   // uniform: the second division only runs when it is needed
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) c[i] += uniform[i] < excess[i] / gap[i] ? 1 : 0;
-        } else {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) c[i] += excess[i] > gap[i] * 0.5f ? 1 : 0;
-        }
-        }
-    }
-    if (live) {
-        uint32_t words[W::WORDS];
-        pack_codes<T, BIT, VEC, W::WORDS>(c, words);
-        store_piece<T, BIT, kPlain, W::WORDS>(group_codes + piece_offset<T, BIT>(k0), words);
-    }
     };
 #pragma unroll
     for (int tile = 0; tile < TILES; ++tile) {
