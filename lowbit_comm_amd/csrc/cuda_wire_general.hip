@@ -403,12 +403,16 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
     const float step = a.kind == 0 ? step_of<BIT>(scale) : scale;
 
     Raw decoded[VEC];
+    if (BIT == 4 && a.kind != 0) {   // uniform: the code's four bits, as they are, index the book
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-        const float code = unpack_code<T, BIT, W::WORDS>(words, i);
-        float value = code * step;
-        if (a.kind != 0) value = book[static_cast<int>(code) & 15] * step;
-        decoded[i] = static_cast<Raw>(raw_from<T>(value));
+        for (int i = 0; i < VEC; ++i) {
+            const int top = 16 - 16 * (i / 4) + 4 * (i % 4);   // left shift that puts the nibble on top, as in unpack_code
+            decoded[i] = static_cast<Raw>(raw_from<T>(book[(words[0] << top) >> 28] * step));
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+            decoded[i] = static_cast<Raw>(raw_from<T>(unpack_code<T, BIT, W::WORDS>(words, i) * step));
     }
     if (a.topk >= 1) {
         const uint32_t indices = meta[1];
