@@ -160,7 +160,7 @@ int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, i
  * quantize writes: nothing orders the two inside the launch.
  * One side with nothing to do (numel == 0) launches the other alone.  LBC_UNSUPPORTED - issue the two calls
  * yourself - unless: group_size 64; every operand aligned for the vector kernels and numel/world * element
- * size a multiple of 16; residual absent (fp32 input only) or fp32; out_dtype fp32 or x_dtype; reduce_world
+ * size a multiple of 16; residual absent or fp32; out_dtype fp32 or x_dtype; reduce_world
  * 2, 4 or 8.  Argument errors are reported as by the two calls.
  */
 int lbc_quant_pack_chunks_and_dequant_reduce(

@@ -12,19 +12,26 @@
 //
 // Every workgroup runs exactly the code of the separate kernels (quant_pack_block.h, dequant_reduce_block.h), so
 // the results are bit-identical to lbc_quant_pack_chunks followed by lbc_dequant_reduce.
+#include <type_traits>
+
 #include "dequant_reduce_block.h"
 #include "quant_pack_block.h"
 
 namespace lbc {
 namespace {
 
+// VEC elements of the bucket per lane, as the separate quantize kernel has them: 8 for a 16-bit bucket without a
+// residual, 4 for everything that touches an fp32 tensor.
+template <typename XT, typename RT> constexpr int quant_vec() { return (sizeof(XT) == 2 && is_void_t<RT>::value) ? 8 : 4; }
+
 template <typename XT, typename RT, typename OT, int W, int MODE>
 __global__ __launch_bounds__(kBlock) void bucket_step_kernel(const QuantArgs q, const ReduceArgs r, unsigned quant_grid_x,
                                                             unsigned quant_blocks, unsigned reduce_blocks) {
-    constexpr int G = 64;
+    constexpr int G = 64, VEC = quant_vec<XT, RT>();
+    using DT = typename std::conditional<VEC == 8, XT, float>::type;   // the type `restored` would have; not written here
     const unsigned b = blockIdx.x;      // wavefront-uniform: no divergence between the two bodies
     if (b < quant_blocks) {
-        quant::quant_pack_block<XT, RT, float, G, 4, MODE>(q, b % quant_grid_x, quant_grid_x, b / quant_grid_x);
+        quant::quant_pack_block<XT, RT, DT, G, VEC, MODE>(q, b % quant_grid_x, quant_grid_x, b / quant_grid_x);
     } else {
         reduce::dequant_reduce_block<OT, G, W, MODE>(r, b - quant_blocks, reduce_blocks);
     }
@@ -32,7 +39,7 @@ __global__ __launch_bounds__(kBlock) void bucket_step_kernel(const QuantArgs q, 
 
 template <typename XT, typename RT, typename OT, int W>
 hipError_t launch_w(int mode, const QuantArgs &q, int quant_world, const ReduceArgs &r, hipStream_t stream) {
-    using QT = quant::quant_tiling<4>;
+    using QT = quant::quant_tiling<quant_vec<XT, RT>()>;
     using RTile = reduce::decode_tiling<OT, W>;
     const int64_t padded = (q.shard_numel + 63) / 64 * 64;
     const int64_t quant_grid_x = (padded + QT::BLOCK_ELEMS - 1) / QT::BLOCK_ELEMS;
@@ -70,10 +77,7 @@ hipError_t launch_r(int x_dtype, int out_dtype, int reduce_world, int mode, cons
 template <typename XT>
 hipError_t launch_x(int x_dtype, int r_dtype, int out_dtype, int reduce_world, int mode, const QuantArgs &q,
                     int quant_world, const ReduceArgs &r, hipStream_t s) {
-    // 16-bit input without a residual is the 8-elements-per-lane quantizer, which has no shared grid
-    if constexpr (sizeof(XT) == 4) {
-        if (r_dtype == kNone) return launch_r<XT, void>(x_dtype, out_dtype, reduce_world, mode, q, quant_world, r, s);
-    }
+    if (r_dtype == kNone) return launch_r<XT, void>(x_dtype, out_dtype, reduce_world, mode, q, quant_world, r, s);
     if (r_dtype == kF32) return launch_r<XT, float>(x_dtype, out_dtype, reduce_world, mode, q, quant_world, r, s);
     return hipErrorNotSupported;
 }

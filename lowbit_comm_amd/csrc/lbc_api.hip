@@ -342,7 +342,7 @@ int lbc_quant_pack_chunks_and_dequant_reduce(
     if (r.empty) return launch_quant(q, "lbc_quant_pack_chunks_and_dequant_reduce", access, stream);
     // one grid exists for aligned operands, whole 16-byte chunks, group 64, a residual that is absent or fp32 and
     // 2, 4 or 8 payloads; everything else is for the caller to issue as the two separate calls
-    if (!q.aligned || !r.aligned || group_size != 64 || lbc::quant_pack_vec(q.x_dtype, q.r_dtype, q.d_dtype, q.outputs) != 4)
+    if (!q.aligned || !r.aligned || group_size != 64 || (q.r_dtype != LBC_NONE && q.r_dtype != LBC_F32))
         return LBC_UNSUPPORTED;
     return finish(lbc::launch_bucket_step(q.x_dtype, q.r_dtype, r.out_dtype, r.world, pick_mode(true, access), q.args,
                                           q.world, r.args, static_cast<hipStream_t>(stream)),

@@ -646,6 +646,7 @@ def test_reduce_requantize_contract(ops, hip_device):
 # --------------------------------------------------------------------------- #
 @pytest.mark.parametrize("grad_dtype,with_residual,out_dtype", [
     ("bf16", True, "fp32"), ("bf16", True, "bf16"), ("fp16", True, "fp32"), ("fp32", True, "fp32"), ("fp32", False, "fp32"),
+    ("bf16", False, "bf16"), ("bf16", False, "fp32"), ("fp16", False, "fp16"),
 ])
 @pytest.mark.parametrize("world,payloads", [(8, 8), (4, 2), (2, 4)])
 @pytest.mark.parametrize("n,reduce_n", [(64 * 8 * 640, 64 * 640), (64 * 8 * 64 * 3 + 64 * 8, 50_048), (64 * 8 * 30, 4096 * 3)])
@@ -748,8 +749,10 @@ def test_shared_launch_reports_what_it_has_no_grid_for(ops, hip_device):
     reduce3 = ops.bind_dequant_reduce(peers8[:3], out)
     bf16 = gradient_like(n, torch.bfloat16, 3301, hip_device)
     fp32 = gradient_like(n, torch.float32, 3302, hip_device)
-    # 16-bit input without a residual, three payloads, another group size: valid requests, no shared grid
-    assert ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(bf16, rows, world), reduce8)() is False
+    # a 16-bit residual, three payloads, another group size: valid requests, no shared grid
+    half_residual = gradient_like(n, torch.bfloat16, 3304, hip_device, sigma=1e-5, outliers=False)
+    assert ops.bind_quant_chunks_and_reduce(
+        ops.bind_quant_pack_chunks(bf16, rows, world, residual=half_residual), reduce8)() is False
     assert ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(fp32, rows, world), reduce3)() is False
     rows32 = torch.zeros(world, (ops.payload_nbytes(shard, 32) + 255) // 256 * 256, dtype=torch.uint8, device=hip_device)
     peers32 = [ops.quant_pack(gradient_like(4096, torch.float32, 3310 + r, hip_device), group_size=32) for r in range(8)]
