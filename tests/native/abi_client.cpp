@@ -1,5 +1,6 @@
-// A host program with no Python and no torch in it: allocates with the HIP runtime, calls the codec through the
-// C ABI of include/lbc.h on a stream of its own, and compares every byte with the scalar C oracle
+// A host program with no Python and no torch in it: allocates with the HIP runtime, calls every entry point of the
+// portable payload format through the C ABI of include/lbc.h on a stream of its own, and compares every byte with
+// the scalar C oracle
 // (oracle/codec_scalar.c, linked from oracle/_build).  Built by __graft_entry__.build(), run by
 // tests/test_abi_client.py on the GPU box.  Prints "OK <checks>" or the first mismatch.
 #include <hip/hip_runtime.h>
@@ -13,8 +14,11 @@
 
 extern "C" {
 void lbo_quantize_f32(const float *x, int64_t n, int group_size, int8_t *codes, float *scales);
+void lbo_dequantize_f32(const int8_t *codes, const float *scales, int64_t n, int group_size, float *out);
 void lbo_reduce_f32(const int8_t *const *codes, const float *const *scales, int world, int64_t n, int group_size,
                     float divisor, float *out);
+void lbo_ef_step_f32(const float *grad, const float *residual_in, int64_t n, int group_size, int8_t *codes, float *scales,
+                     float *residual_out, float *restored_out);
 }
 
 #define HIP_OK(call)                                                                       \
@@ -142,6 +146,137 @@ int main() {
         return 6;
     }
     checks += 3;
+
+    // decode of one payload
+    LBC_OK_OR_FAIL(lbc_dequant(d_codes[0], d_scales[0], n, g, d_out, LBC_F32, LBC_REDUCE_NONE, LBC_ACCESS_AUTO, stream));
+    HIP_OK(hipMemcpyAsync(got.data(), d_out, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    lbo_dequantize_f32(want_codes[0].data(), want_scales[0].data(), n, g, want.data());
+    if (memcmp(got.data(), want.data(), n * sizeof(float)) != 0) {
+        printf("FAIL decoded payload differs from the oracle\n");
+        return 8;
+    }
+    ++checks;
+
+    // error-feedback step: quantize x + residual, residual updated in place, the decoded value as a second output;
+    // then the same residual once more from lbc_ef_update
+    std::vector<float> residual(n), want_residual(n), want_restored(n), prepared(n);
+    fill(residual, 99u, 1e-5f);
+    for (int64_t i = 0; i < n; ++i) {
+        volatile float sum = x[0][i] + residual[i];
+        prepared[i] = sum;
+    }
+    std::vector<int8_t> ef_codes(padded), want_ef_codes(padded);
+    std::vector<float> ef_scales(groups), want_ef_scales(groups);
+    lbo_ef_step_f32(x[0].data(), residual.data(), n, g, want_ef_codes.data(), want_ef_scales.data(), want_residual.data(),
+                    want_restored.data());
+    float *d_residual = nullptr, *d_restored = nullptr, *d_prepared = nullptr;
+    HIP_OK(hipMalloc(&d_residual, n * sizeof(float)));
+    HIP_OK(hipMalloc(&d_restored, n * sizeof(float)));
+    HIP_OK(hipMalloc(&d_prepared, n * sizeof(float)));
+    HIP_OK(hipMemcpyAsync(d_x, x[0].data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
+    HIP_OK(hipMemcpyAsync(d_residual, residual.data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
+    HIP_OK(hipMemcpyAsync(d_prepared, prepared.data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
+    LBC_OK_OR_FAIL(lbc_quant_pack(d_x, LBC_F32, d_residual, LBC_F32, n, g, d_send_codes, d_send_scales, d_residual, LBC_F32,
+                                  d_restored, LBC_F32, LBC_ACCESS_AUTO, stream));
+    std::vector<float> got_residual(n), got_restored(n);
+    HIP_OK(hipMemcpyAsync(ef_codes.data(), d_send_codes, padded, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(ef_scales.data(), d_send_scales, groups * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(got_residual.data(), d_residual, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(got_restored.data(), d_restored, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    if (memcmp(ef_codes.data(), want_ef_codes.data(), padded) != 0 ||
+        memcmp(ef_scales.data(), want_ef_scales.data(), groups * sizeof(float)) != 0 ||
+        memcmp(got_residual.data(), want_residual.data(), n * sizeof(float)) != 0 ||
+        memcmp(got_restored.data(), want_restored.data(), n * sizeof(float)) != 0) {
+        printf("FAIL error-feedback step differs from the oracle\n");
+        return 9;
+    }
+    checks += 4;
+    LBC_OK_OR_FAIL(lbc_ef_update(d_prepared, LBC_F32, d_restored, LBC_F32, d_residual, LBC_F32, n, LBC_ACCESS_AUTO, stream));
+    HIP_OK(hipMemcpyAsync(got_residual.data(), d_residual, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    if (memcmp(got_residual.data(), want_residual.data(), n * sizeof(float)) != 0) {
+        printf("FAIL residual update differs from the oracle\n");
+        return 9;
+    }
+    ++checks;
+
+    // the bucket as `world` chunks in one launch, and the chunks decoded back in one launch
+    const int64_t shard = (n + world - 1) / world, shard_groups = (shard + g - 1) / g, shard_padded = shard_groups * g;
+    const int64_t stride = (shard_padded + shard_groups * 4 + 255) / 256 * 256;
+    uint8_t *d_rows = nullptr;
+    HIP_OK(hipMalloc(&d_rows, world * stride));
+    HIP_OK(hipMemsetAsync(d_rows, 0xEE, world * stride, stream));
+    LBC_OK_OR_FAIL(lbc_quant_pack_chunks(d_x, LBC_F32, nullptr, LBC_NONE, n, world, g, d_rows, stride, nullptr, LBC_NONE, nullptr,
+                                         LBC_NONE, LBC_ACCESS_AUTO, stream));
+    LBC_OK_OR_FAIL(lbc_dequant_chunks(d_rows, stride, world, shard, n, g, d_out, LBC_F32, LBC_ACCESS_AUTO, stream));
+    std::vector<uint8_t> rows(world * stride);
+    HIP_OK(hipMemcpyAsync(rows.data(), d_rows, world * stride, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(got.data(), d_out, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<std::vector<int8_t>> chunk_codes(world, std::vector<int8_t>(shard_padded));
+    std::vector<std::vector<float>> chunk_scales(world, std::vector<float>(shard_groups));
+    for (int d = 0; d < world; ++d) {
+        std::vector<float> piece(shard, 0.0f);   // the bucket counts as zero padded to world * shard
+        for (int64_t i = 0; i < shard && d * shard + i < n; ++i) piece[i] = x[0][d * shard + i];
+        lbo_quantize_f32(piece.data(), shard, g, chunk_codes[d].data(), chunk_scales[d].data());
+        if (memcmp(rows.data() + d * stride, chunk_codes[d].data(), shard_padded) != 0 ||
+            memcmp(rows.data() + d * stride + shard_padded, chunk_scales[d].data(), shard_groups * sizeof(float)) != 0) {
+            printf("FAIL payload of chunk %d differs from the oracle\n", d);
+            return 10;
+        }
+        std::vector<float> decoded(shard);
+        lbo_dequantize_f32(chunk_codes[d].data(), chunk_scales[d].data(), shard, g, decoded.data());
+        for (int64_t i = 0; i < shard && d * shard + i < n; ++i) want[d * shard + i] = decoded[i];
+        ++checks;
+    }
+    if (memcmp(got.data(), want.data(), n * sizeof(float)) != 0) {
+        printf("FAIL decoded chunks differ from the oracle\n");
+        return 10;
+    }
+    ++checks;
+
+    // reduce (mean) and requantize in one launch: the payload of quantize(reduce(payloads))
+    LBC_OK_OR_FAIL(lbc_dequant_reduce_quant(code_ptrs.data(), scale_ptrs.data(), world, n, g, static_cast<float>(world), LBC_F32,
+                                            d_send_codes, d_send_scales, LBC_ACCESS_AUTO, stream));
+    HIP_OK(hipMemcpyAsync(send_codes.data(), d_send_codes, padded, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(send_scales.data(), d_send_scales, groups * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    lbo_reduce_f32(host_codes.data(), host_scales.data(), world, n, g, static_cast<float>(world), want.data());
+    lbo_quantize_f32(want.data(), n, g, want_send_codes.data(), want_send_scales.data());
+    if (memcmp(send_codes.data(), want_send_codes.data(), padded) != 0 ||
+        memcmp(send_scales.data(), want_send_scales.data(), groups * sizeof(float)) != 0) {
+        printf("FAIL reduce + requantize differs from the oracle\n");
+        return 11;
+    }
+    checks += 2;
+
+    // quantize of one bucket (as chunks) and reduce of another bucket's payloads in one launch
+    const int64_t even = 64 * world * 40, even_shard = even / world, even_groups = even_shard / g;
+    const int64_t even_stride = (even_shard + even_groups * 4 + 255) / 256 * 256, reduce_n = 64 * 100;
+    HIP_OK(hipMemsetAsync(d_rows, 0xEE, world * stride, stream));
+    LBC_OK_OR_FAIL(lbc_quant_pack_chunks_and_dequant_reduce(d_x, LBC_F32, nullptr, LBC_NONE, even, world, g, d_rows, even_stride,
+                                                            nullptr, LBC_NONE, code_ptrs.data(), scale_ptrs.data(), world, reduce_n,
+                                                            static_cast<float>(world), d_out, LBC_F32, nullptr, nullptr,
+                                                            LBC_ACCESS_AUTO, stream));
+    HIP_OK(hipMemcpyAsync(rows.data(), d_rows, world * even_stride, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(got.data(), d_out, reduce_n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    for (int d = 0; d < world; ++d) {
+        lbo_quantize_f32(x[0].data() + d * even_shard, even_shard, g, chunk_codes[d].data(), chunk_scales[d].data());
+        if (memcmp(rows.data() + d * even_stride, chunk_codes[d].data(), even_shard) != 0 ||
+            memcmp(rows.data() + d * even_stride + even_shard, chunk_scales[d].data(), even_groups * sizeof(float)) != 0) {
+            printf("FAIL shared launch: payload of chunk %d differs from the oracle\n", d);
+            return 12;
+        }
+    }
+    lbo_reduce_f32(host_codes.data(), host_scales.data(), world, reduce_n, g, static_cast<float>(world), want.data());
+    if (memcmp(got.data(), want.data(), reduce_n * sizeof(float)) != 0) {
+        printf("FAIL shared launch: reduced shard differs from the oracle\n");
+        return 12;
+    }
+    checks += 2;
 
     // contract: a bad argument is refused with a message, an unsupported group size is "unsupported", not an error
     if (lbc_quant_pack(d_x, LBC_F32, nullptr, LBC_NONE, -1, g, d_codes[0], d_scales[0], nullptr, LBC_NONE, nullptr, LBC_NONE,
