@@ -1,7 +1,7 @@
 // A host program with no Python and no torch in it: allocates with the HIP runtime, calls every entry point of the
-// portable payload format through the C ABI of include/lbc.h on a stream of its own, and compares every byte with
-// the scalar C oracle
-// (oracle/codec_scalar.c, linked from oracle/_build).  Built by __graft_entry__.build(), run by
+// portable payload format and of the CUDA extension's byte format through the C ABI of include/lbc.h on a stream of
+// its own, and compares every byte with the scalar C oracles (oracle/codec_scalar.c, oracle/cuda_wire_scalar.c,
+// oracle/cuda_wire_general_scalar.c, linked from oracle/_build).  Built by __graft_entry__.build(), run by
 // tests/test_abi_client.py on the GPU box.  Prints "OK <checks>" or the first mismatch.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -19,6 +19,15 @@ void lbo_reduce_f32(const int8_t *const *codes, const float *const *scales, int 
                     float divisor, float *out);
 void lbo_ef_step_f32(const float *grad, const float *residual_in, int64_t n, int group_size, int8_t *codes, float *scales,
                      float *residual_out, float *restored_out);
+// the byte format of the reference's CUDA extension (oracle/cuda_wire_scalar.c, oracle/cuda_wire_general_scalar.c)
+void lbw_quantize(const void *x, const void *residual, int dtype, int64_t numel, int g, int compact, int bit, uint8_t *payload);
+void lbw_dequantize(const uint8_t *payload, int64_t numel, int g, int compact, int dtype, int op, int bit, void *out);
+void lbw_reduce(const uint8_t *const *payloads, int world, int64_t numel, int g, int compact, int dtype, float inv_divisor,
+                int use_fma, const void *prepared, void *out, void *residual);
+void lbg_quantize(const void *x, int dtype, int64_t numel, int g, int bit, int kind, int topk, int stochastic, uint64_t seed,
+                  uint64_t offset, int compact, uint8_t *payload);
+void lbg_dequantize(const uint8_t *payload, int64_t numel, int g, int bit, int kind, int topk, int compact, int dtype, int op,
+                    void *out);
 }
 
 #define HIP_OK(call)                                                                       \
@@ -53,6 +62,154 @@ static void fill(std::vector<float> &x, uint32_t seed, float sigma) {
         x[i] = u * 1.7320508f * sigma;
         if ((lcg(s) & 1023u) == 0u) x[i] *= 100.0f;
     }
+}
+
+static uint16_t to_bf16(float f) {   // round to nearest even; the inputs here are finite
+    uint32_t bits;
+    memcpy(&bits, &f, 4);
+    return static_cast<uint16_t>((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
+}
+
+// Every entry point of the CUDA extension's byte format, on whole groups, against its scalar C restatement.
+static int wire_format_checks(hipStream_t stream, long &checks) {
+    const int world = 4, g = 64;
+    const int64_t n = 64 * 4 * 750;   // whole groups, whole shards
+    std::vector<std::vector<float>> x(world, std::vector<float>(n));
+    for (int r = 0; r < world; ++r) fill(x[r], 4321u + 31u * r, 2e-3f * (r + 1));
+    std::vector<uint16_t> half(n);
+    for (int64_t i = 0; i < n; ++i) half[i] = to_bf16(x[0][i]);
+    void *d_x = nullptr, *d_out = nullptr;
+    HIP_OK(hipMalloc(&d_x, n * sizeof(float)));
+    HIP_OK(hipMalloc(&d_out, n * sizeof(float)));
+    const int64_t room = n + n / g * 16 + 256;   // the largest payload here: 8-bit codes and four fp32 words a group
+    std::vector<uint8_t *> d_payload(world, nullptr);
+    for (int r = 0; r < world; ++r) HIP_OK(hipMalloc(&d_payload[r], room));
+    std::vector<uint8_t> got(room), want(room);
+    std::vector<float> out(n), want_out(n);
+
+    // quantize + pack and decode: fp32 and bf16, interleaved and appended scales, 8 and 4 bits
+    for (int dtype : {LBC_F32, LBC_BF16}) {
+        const void *host = dtype == LBC_F32 ? static_cast<const void *>(x[0].data()) : static_cast<const void *>(half.data());
+        const size_t item = dtype == LBC_F32 ? 4 : 2;
+        HIP_OK(hipMemcpyAsync(d_x, host, n * item, hipMemcpyHostToDevice, stream));
+        for (int compact : {1, 0}) {
+            for (int bit : {8, 4}) {
+                const int64_t bytes = lbc_wire_payload_nbytes(n, g, dtype, bit);
+                if (bytes <= 0 || bytes > room) {
+                    printf("FAIL payload size %lld\n", static_cast<long long>(bytes));
+                    return 20;
+                }
+                LBC_OK_OR_FAIL(lbc_wire_quant_pack(d_x, nullptr, dtype, n, g, bit, compact, d_payload[0], LBC_ACCESS_AUTO, stream));
+                LBC_OK_OR_FAIL(lbc_wire_dequant(d_payload[0], n, g, bit, compact, d_out, dtype, LBC_REDUCE_NONE, LBC_ACCESS_AUTO, stream));
+                HIP_OK(hipMemcpyAsync(got.data(), d_payload[0], bytes, hipMemcpyDeviceToHost, stream));
+                HIP_OK(hipMemcpyAsync(out.data(), d_out, n * item, hipMemcpyDeviceToHost, stream));
+                HIP_OK(hipStreamSynchronize(stream));
+                lbw_quantize(host, nullptr, dtype, n, g, compact, bit, want.data());
+                lbw_dequantize(want.data(), n, g, compact, dtype, 0, bit, want_out.data());
+                if (memcmp(got.data(), want.data(), bytes) != 0 || memcmp(out.data(), want_out.data(), n * item) != 0) {
+                    printf("FAIL wire format: dtype %d compact %d bit %d differs from the oracle\n", dtype, compact, bit);
+                    return 21;
+                }
+                checks += 2;
+            }
+        }
+    }
+
+    // the payloads of four ranks (fp32, interleaved scales), their fused mean, and one ring step on them
+    const int64_t bytes = lbc_wire_payload_nbytes(n, g, LBC_F32, 8);
+    std::vector<std::vector<uint8_t>> host_payload(world, std::vector<uint8_t>(bytes));
+    std::vector<const uint8_t *> d_ptrs(world), h_ptrs(world);
+    for (int r = 0; r < world; ++r) {
+        HIP_OK(hipMemcpyAsync(d_x, x[r].data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
+        LBC_OK_OR_FAIL(lbc_wire_quant_pack(d_x, nullptr, LBC_F32, n, g, 8, 1, d_payload[r], LBC_ACCESS_AUTO, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        lbw_quantize(x[r].data(), nullptr, LBC_F32, n, g, 1, 8, host_payload[r].data());
+        d_ptrs[r] = d_payload[r];
+        h_ptrs[r] = host_payload[r].data();
+    }
+    LBC_OK_OR_FAIL(lbc_wire_dequant_reduce(d_ptrs.data(), world, n, g, 1, 0.25f, 1, d_out, LBC_F32, nullptr, nullptr,
+                                           LBC_ACCESS_AUTO, stream));
+    HIP_OK(hipMemcpyAsync(out.data(), d_out, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    lbw_reduce(h_ptrs.data(), world, n, g, 1, LBC_F32, 0.25f, 1, nullptr, want_out.data(), nullptr);
+    if (memcmp(out.data(), want_out.data(), n * sizeof(float)) != 0) {
+        printf("FAIL wire format: fused mean differs from the oracle\n");
+        return 22;
+    }
+    ++checks;
+    uint8_t *d_send = nullptr;
+    HIP_OK(hipMalloc(&d_send, room));
+    HIP_OK(hipMemcpyAsync(d_out, x[0].data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
+    LBC_OK_OR_FAIL(lbc_wire_ring_step(d_payload[1], d_out, LBC_F32, n, g, 1, LBC_REDUCE_SUM, 1.0f, d_send, LBC_ACCESS_AUTO, stream));
+    HIP_OK(hipMemcpyAsync(out.data(), d_out, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(got.data(), d_send, bytes, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    want_out = x[0];
+    lbw_dequantize(host_payload[1].data(), n, g, 1, LBC_F32, 1, 8, want_out.data());
+    lbw_quantize(want_out.data(), nullptr, LBC_F32, n, g, 1, 8, want.data());
+    if (memcmp(out.data(), want_out.data(), n * sizeof(float)) != 0 || memcmp(got.data(), want.data(), bytes) != 0) {
+        printf("FAIL wire format: ring step differs from the oracle\n");
+        return 23;
+    }
+    checks += 2;
+
+    // the bucket as four chunks in one launch, and the chunks decoded back in one launch
+    const int64_t shard = n / world, shard_bytes = lbc_wire_payload_nbytes(shard, g, LBC_F32, 8);
+    const int64_t stride = (shard_bytes + 255) / 256 * 256;
+    uint8_t *d_rows = nullptr;
+    HIP_OK(hipMalloc(&d_rows, world * stride));
+    HIP_OK(hipMemcpyAsync(d_x, x[0].data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
+    LBC_OK_OR_FAIL(lbc_wire_quant_pack_chunks(d_x, nullptr, LBC_F32, n, world, g, 8, 1, d_rows, stride, LBC_ACCESS_AUTO, stream));
+    LBC_OK_OR_FAIL(lbc_wire_dequant_chunks(d_rows, stride, world, shard, n, g, 8, 1, d_out, LBC_F32, LBC_REDUCE_NONE,
+                                           LBC_ACCESS_AUTO, stream));
+    std::vector<uint8_t> rows(world * stride);
+    HIP_OK(hipMemcpyAsync(rows.data(), d_rows, world * stride, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(out.data(), d_out, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    for (int d = 0; d < world; ++d) {
+        lbw_quantize(x[0].data() + d * shard, nullptr, LBC_F32, shard, g, 1, 8, want.data());
+        lbw_dequantize(want.data(), shard, g, 1, LBC_F32, 0, 8, want_out.data() + d * shard);
+        if (memcmp(rows.data() + d * stride, want.data(), shard_bytes) != 0) {
+            printf("FAIL wire format: payload of chunk %d differs from the oracle\n", d);
+            return 24;
+        }
+    }
+    if (memcmp(out.data(), want_out.data(), n * sizeof(float)) != 0) {
+        printf("FAIL wire format: decoded chunks differ from the oracle\n");
+        return 24;
+    }
+    checks += 2;
+
+    // the general policies: two outliers, stochastic rounding, a code book
+    struct Policy { int dtype, bit, kind, topk, stochastic; };
+    const Policy policies[] = {{LBC_F32, 8, LBC_QUANT_LINEAR, 2, 0}, {LBC_F32, 8, LBC_QUANT_LINEAR, 0, 1},
+                               {LBC_BF16, 4, LBC_QUANT_NORMAL, 0, 0}, {LBC_BF16, 4, LBC_QUANT_E2M1, 1, 1}};
+    for (const Policy &p : policies) {
+        const void *host = p.dtype == LBC_F32 ? static_cast<const void *>(x[0].data()) : static_cast<const void *>(half.data());
+        const size_t item = p.dtype == LBC_F32 ? 4 : 2;
+        const uint64_t seed = 0x1234567887654321ULL, offset = 12;
+        const int64_t size = lbc_wire_general_payload_nbytes(n, g, p.dtype, p.bit, p.topk);
+        if (size <= 0 || size > room) {
+            printf("FAIL general payload size %lld\n", static_cast<long long>(size));
+            return 25;
+        }
+        HIP_OK(hipMemcpyAsync(d_x, host, n * item, hipMemcpyHostToDevice, stream));
+        LBC_OK_OR_FAIL(lbc_wire_quant_general(d_x, p.dtype, n, g, p.bit, p.kind, p.topk, p.stochastic, seed, offset, 1,
+                                              d_payload[0], stream));
+        LBC_OK_OR_FAIL(lbc_wire_dequant_general(d_payload[0], n, g, p.bit, p.kind, p.topk, 1, d_out, p.dtype, LBC_REDUCE_NONE, stream));
+        HIP_OK(hipMemcpyAsync(got.data(), d_payload[0], size, hipMemcpyDeviceToHost, stream));
+        HIP_OK(hipMemcpyAsync(out.data(), d_out, n * item, hipMemcpyDeviceToHost, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        lbg_quantize(host, p.dtype, n, g, p.bit, p.kind, p.topk, p.stochastic, seed, offset, 1, want.data());
+        lbg_dequantize(want.data(), n, g, p.bit, p.kind, p.topk, 1, p.dtype, 0, want_out.data());
+        if (memcmp(got.data(), want.data(), size) != 0 || memcmp(out.data(), want_out.data(), n * item) != 0) {
+            printf("FAIL wire format: policy (dtype %d, %d bit, kind %d, top-%d, stochastic %d) differs from the oracle\n", p.dtype,
+                   p.bit, p.kind, p.topk, p.stochastic);
+            return 26;
+        }
+        checks += 2;
+    }
+    return 0;
 }
 
 int main() {
@@ -290,6 +447,7 @@ int main() {
         return 7;
     }
     checks += 2;
+    if (const int status = wire_format_checks(stream, checks)) return status;
     printf("OK %ld\n", checks);
     return 0;
 }

@@ -19,14 +19,15 @@ def test_client_source_uses_only_the_header_and_the_hip_runtime():
 
 
 @pytest.mark.gpu
-def test_client_runs_every_entry_point_of_the_portable_format_bit_exact_against_the_c_oracle(hip_device):
-    """quantize, decode, fused reduce, ring step, the error-feedback step and the residual update, the bucket as chunks
-    and the chunks decoded back, reduce + requantize, and the shared launch of a quantize and a reduce: 29 byte
-    comparisons with the scalar C oracle and the two contract checks."""
+def test_client_runs_every_entry_point_bit_exact_against_the_c_oracles(hip_device):
+    """Portable format: quantize, decode, fused reduce, ring step, the error-feedback step and the residual update, the
+    bucket as chunks and the chunks decoded back, reduce + requantize, the shared launch of a quantize and a reduce,
+    and two contract checks (29).  The CUDA extension's byte format: quantize and decode for fp32 / bf16, interleaved /
+    appended scales, 8 / 4 bits; fused mean of four payloads; ring step; chunks; four general policies (29)."""
     done = subprocess.run([str(CLIENT)], capture_output=True, text=True, timeout=120)
     assert done.returncode == 0, (done.stdout, done.stderr[-2000:])
     assert done.stdout.strip().startswith("OK "), done.stdout
-    assert int(done.stdout.split()[1]) == 29
+    assert int(done.stdout.split()[1]) == 58
 
 
 @pytest.mark.gpu
