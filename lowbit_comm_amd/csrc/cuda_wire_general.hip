@@ -86,7 +86,7 @@ __device__ __forceinline__ int meta_words_of(int topk) { return topk == 0 ? 1 : 
 // ---------------------------------------------------------------------------------------------
 // quantize: a wavefront works on tiles of 64 * VEC elements (64 lanes x 16 bytes of the tensor)
 // ---------------------------------------------------------------------------------------------
-// Tiles per wavefront: 32 bytes of the tensor per lane either way.  A 32-bit tensor's wavefront asks for both of
+// Tiles per wavefront: eight elements per lane either way.  A 32-bit tensor's wavefront asks for both of
 // its tiles before it does anything else and encodes one while the other is on its way (26.2 M fp32 elements:
 // stochastic rounding 28.8 instead of 37.4 us, top-2 30.3 instead of 30.8, a code book 28.2 instead of 30.0);
 // four tiles are slower again (32.7 us top-2), and so are two tiles of eight 16-bit elements a lane (bf16 top-2
