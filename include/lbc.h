@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define LBC_ABI_VERSION 7
+#define LBC_ABI_VERSION 8
 
 enum { LBC_OK = 0, LBC_UNSUPPORTED = 1, LBC_EINVAL = -1, LBC_ELAUNCH = -2 };
 
@@ -82,6 +82,15 @@ enum { LBC_ACCESS_AUTO = 0, LBC_ACCESS_CACHED = 1, LBC_ACCESS_STREAM = 2 };
  *   scale_g  = max(absmax_g(p)/127, 2^-23);  code = sat8(rint(p/scale_g)), NaN -> 0
  *   restored = code*scale_g rounded to restored_dtype          (written if restored != NULL)
  *   new_residual = p - restored, rounded to new_residual_dtype (written if new_residual != NULL)
+ *   prepared = p                                               (written if prepared != NULL)
+ *
+ * `prepared` is for the caller whose residual update comes later, from the reduced result of
+ * all ranks instead of the local round trip: the reference's all_gather hook keeps
+ * prepared = bucket + residual for `residual = prepared - restored` after the gather
+ * (ccdl_comm/communication/ddp_hook.py:196,224-241; ErrorFeedbackState.compensate,
+ * ccdl_comm/quantization/error_feedback.py:27-36), which costs it a kernel of its own before the
+ * quantize.  prepared_dtype must be p's type (x_dtype without a residual, else the torch promotion
+ * of x_dtype and residual_dtype); prepared must not alias another tensor of the call.
  *
  * new_residual may alias residual (in-place update).  codes must hold G*g bytes
  * and scales G floats (4-byte aligned).  Supported: group_size in {16,32,64};
@@ -92,7 +101,7 @@ enum { LBC_ACCESS_AUTO = 0, LBC_ACCESS_CACHED = 1, LBC_ACCESS_STREAM = 2 };
 int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residual_dtype,
                    int64_t numel, int group_size, int8_t *codes, float *scales,
                    void *new_residual, int new_residual_dtype, void *restored, int restored_dtype,
-                   int access, void *stream);
+                   void *prepared, int prepared_dtype, int access, void *stream);
 
 /*
  * Quantize `world` equal destination chunks of one flat bucket in a single
@@ -107,12 +116,13 @@ int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residua
  * element.  Payload d is written packed at payloads + d*payload_stride:
  * int8 codes[Gs*g] then float scales[Gs], Gs = ceil(shard_numel/g).
  * payload_stride >= Gs*(g+4) and a multiple of 4.  Pass residual =
- * new_residual = restored = NULL (dtypes ignored) for a plain quantize.
+ * new_residual = restored = prepared = NULL (dtypes ignored) for a plain quantize.
  */
 int lbc_quant_pack_chunks(const void *x, int x_dtype, const void *residual, int residual_dtype,
                           int64_t numel, int world, int group_size, uint8_t *payloads,
                           int64_t payload_stride, void *new_residual, int new_residual_dtype,
-                          void *restored, int restored_dtype, int access, void *stream);
+                          void *restored, int restored_dtype, void *prepared, int prepared_dtype,
+                          int access, void *stream);
 
 /*
  * Decode one payload: out[i] (op)= float(code[i]) * scale[i/g], rounded to out_dtype.
@@ -195,6 +205,63 @@ int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int worl
 int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *scales, int world,
                              int64_t numel, int group_size, float divisor, int mid_dtype,
                              int8_t *out_codes, float *out_scales, int access, void *stream);
+
+/*
+ * One launch for the three compute stages that a stream of buckets has in flight together under the
+ * compressed reduce-scatter + all-gather plan: the chunked quantize of bucket k (its all-to-all follows),
+ * the reduce + requantize of the payloads that arrived for bucket k-1's shard (its all-gather follows) and
+ * the decode of the gathered shard payloads of bucket k-2.  In the reference these are the compute steps
+ * between the collectives of ccdl_comm/communication/reduce_scatter_transport.py:252-347 (quantize the
+ * chunks, reduce what arrived) and ccdl_comm/communication/topology_transport.py:866-894 (requantize,
+ * gather, decode every shard), one kernel each and one bucket at a time; consecutive DDP buckets are
+ * independent, so stage s of bucket k-s is ready when the exchanges of the earlier buckets have been
+ * handed to the stream, and the shard-sized stages, which are mostly launch ramp on their own, ride in
+ * the grid of the quantize.
+ *
+ * Each stage structure carries the arguments of the call it stands for - lbc_quant_pack_chunks (without
+ * `restored` and `prepared`), lbc_dequant_reduce_quant, lbc_dequant_chunks - with the same meaning and
+ * the same validation; a NULL stage is absent, and a stage with nothing to do (numel == 0) counts as
+ * absent.  Results are bit-identical to those calls in any order.  Nothing orders the stages inside the
+ * launch: no stage may read or write what another writes (decoding bucket k-2 in place is fine, its
+ * quantize ran two launches earlier).
+ *
+ * With one stage present its own kernel runs.  With two or three: LBC_UNSUPPORTED - issue the calls
+ * yourself - unless group_size is 64, every operand is aligned for the vector kernels (16 bytes for
+ * tensors and shard boundaries, 4 for payload rows; 8 for 16-bit output), the residual is absent or
+ * fp32, the reduce has 2, 4 or 8 payloads, and x_dtype, mid_dtype and out_dtype are one type.
+ */
+typedef struct lbc_quant_chunks_stage {
+    const void *x;
+    const void *residual;       /* may be NULL */
+    uint8_t *payloads;
+    void *new_residual;         /* may be NULL; may alias residual */
+    int64_t numel;
+    int64_t payload_stride;
+    int x_dtype, residual_dtype, new_residual_dtype, world;
+} lbc_quant_chunks_stage;
+
+typedef struct lbc_reduce_quant_stage {
+    const int8_t *const *codes;  /* HOST arrays of `world` device pointers */
+    const float *const *scales;
+    int8_t *out_codes;
+    float *out_scales;
+    int64_t numel;
+    float divisor;
+    int world, mid_dtype;
+} lbc_reduce_quant_stage;
+
+typedef struct lbc_dequant_chunks_stage {
+    const uint8_t *payloads;
+    void *out;
+    int64_t payload_stride;
+    int64_t shard_numel;
+    int64_t total_numel;
+    int world, out_dtype;
+} lbc_dequant_chunks_stage;
+
+int lbc_bucket_pipeline_step(const lbc_quant_chunks_stage *quant, const lbc_reduce_quant_stage *reduce,
+                             const lbc_dequant_chunks_stage *decode, int group_size, int access,
+                             void *stream);
 
 /*
  * One compute step of the quantized ring all-reduce on one chunk of the bucket, in place:

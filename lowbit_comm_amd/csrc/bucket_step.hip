@@ -16,81 +16,89 @@
 
 #include "dequant_reduce_block.h"
 #include "quant_pack_block.h"
+#include "step_grid.h"
 
 namespace lbc {
 namespace {
 
-// VEC elements of the bucket per lane, as the separate quantize kernel has them: 8 for a 16-bit bucket without a
-// residual, 4 for everything that touches an fp32 tensor.
-template <typename XT, typename RT> constexpr int quant_vec() { return (sizeof(XT) == 2 && is_void_t<RT>::value) ? 8 : 4; }
-
-template <typename XT, typename RT, typename OT, int W, int MODE>
-__global__ __launch_bounds__(kBlock) void bucket_step_kernel(const QuantArgs q, const ReduceArgs r, unsigned quant_grid_x,
-                                                            unsigned quant_blocks, unsigned reduce_blocks) {
-    constexpr int G = 64, VEC = quant_vec<XT, RT>();
-    using DT = typename std::conditional<VEC == 8, XT, float>::type;   // the type `restored` would have; not written here
-    const unsigned b = blockIdx.x;      // wavefront-uniform: no divergence between the two bodies
-    if (b < quant_blocks) {
-        quant::quant_pack_block<XT, RT, DT, G, VEC, MODE>(q, b % quant_grid_x, quant_grid_x, b / quant_grid_x);
-    } else {
-        reduce::dequant_reduce_block<OT, G, W, MODE>(r, b - quant_blocks, reduce_blocks);
+// The quantize half is the instantiation the separate kernel would run for the same call (quant_pack_vec): VEC
+// elements of the bucket per lane - 8 for a call in which every tensor is 16 bits wide, 4 as soon as an fp32 tensor
+// takes part (an fp32 residual, or a 16-bit bucket without a residual whose new residual is asked for: `restored` is
+// rounded to fp32 there, so the new residual is an fp32 tensor) - and DT, the type `restored` is rounded to before
+// the subtraction, which fixes the new residual's type.
+template <typename XT, typename RT, int VEC, typename OT, int W, int MODE>
+__global__ __launch_bounds__(kBlock) void bucket_step_kernel(const QuantArgs q, const ReduceArgs r, const StepSegment quant_part,
+                                                            const StepSegment reduce_part) {
+    constexpr int G = 64;
+    static_assert(VEC == 4 || (VEC == 8 && sizeof(XT) == 2 && is_void_t<RT>::value), "no such quantize instantiation");
+    using DT = typename std::conditional<VEC == 8, XT, float>::type;
+    unsigned block_x, row;              // wavefront-uniform: no divergence between the two bodies
+    if (step_segment_holds(quant_part, blockIdx.x, block_x, row)) {
+        if (block_x < quant_part.grid_x) quant::quant_pack_block<XT, RT, DT, G, VEC, MODE>(q, block_x, quant_part.grid_x, row);
+    } else if (step_segment_holds(reduce_part, blockIdx.x, block_x, row)) {
+        if (block_x < reduce_part.grid_x) reduce::dequant_reduce_block<OT, G, W, MODE>(r, block_x, reduce_part.grid_x);
     }
 }
 
-template <typename XT, typename RT, typename OT, int W>
+template <typename XT, typename RT, int VEC, typename OT, int W>
 hipError_t launch_w(int mode, const QuantArgs &q, int quant_world, const ReduceArgs &r, hipStream_t stream) {
-    using QT = quant::quant_tiling<quant_vec<XT, RT>()>;
+    using QT = quant::quant_tiling<VEC>;
     using RTile = reduce::decode_tiling<OT, W>;
     const int64_t padded = (q.shard_numel + 63) / 64 * 64;
     const int64_t quant_grid_x = (padded + QT::BLOCK_ELEMS - 1) / QT::BLOCK_ELEMS;
-    const int64_t quant_blocks = quant_grid_x * quant_world;
     const int64_t reduce_blocks = (r.numel + RTile::BLOCK_ELEMS - 1) / RTile::BLOCK_ELEMS;
-    if (quant_blocks + reduce_blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-    const dim3 grid(static_cast<unsigned>(quant_blocks + reduce_blocks));
+    if (step_segment_slots(quant_grid_x, quant_world) + step_segment_slots(reduce_blocks, 1) > 0x7FFFFFFFLL)
+        return hipErrorInvalidValue;
+    int64_t cursor = 0;                 // the quantize's blocks first, the reduce's behind them
+    const StepSegment quant_part = step_segment_at(cursor, quant_grid_x, quant_world);
+    const StepSegment reduce_part = step_segment_at(cursor, reduce_blocks, 1);
+    const dim3 grid(static_cast<unsigned>(cursor));
     if (mode == kVector)
-        hipLaunchKernelGGL((bucket_step_kernel<XT, RT, OT, W, kVector>), grid, dim3(kBlock), 0, stream, q, r,
-                           static_cast<unsigned>(quant_grid_x), static_cast<unsigned>(quant_blocks), static_cast<unsigned>(reduce_blocks));
+        hipLaunchKernelGGL((bucket_step_kernel<XT, RT, VEC, OT, W, kVector>), grid, dim3(kBlock), 0, stream, q, r, quant_part, reduce_part);
     else
-        hipLaunchKernelGGL((bucket_step_kernel<XT, RT, OT, W, kStream>), grid, dim3(kBlock), 0, stream, q, r,
-                           static_cast<unsigned>(quant_grid_x), static_cast<unsigned>(quant_blocks), static_cast<unsigned>(reduce_blocks));
+        hipLaunchKernelGGL((bucket_step_kernel<XT, RT, VEC, OT, W, kStream>), grid, dim3(kBlock), 0, stream, q, r, quant_part, reduce_part);
     return hipGetLastError();
 }
 
-template <typename XT, typename RT, typename OT>
+template <typename XT, typename RT, int VEC, typename OT>
 hipError_t launch_o(int reduce_world, int mode, const QuantArgs &q, int quant_world, const ReduceArgs &r, hipStream_t s) {
     switch (reduce_world) {
-        case 2: return launch_w<XT, RT, OT, 2>(mode, q, quant_world, r, s);
-        case 4: return launch_w<XT, RT, OT, 4>(mode, q, quant_world, r, s);
-        case 8: return launch_w<XT, RT, OT, 8>(mode, q, quant_world, r, s);
+        case 2: return launch_w<XT, RT, VEC, OT, 2>(mode, q, quant_world, r, s);
+        case 4: return launch_w<XT, RT, VEC, OT, 4>(mode, q, quant_world, r, s);
+        case 8: return launch_w<XT, RT, VEC, OT, 8>(mode, q, quant_world, r, s);
         default: return hipErrorNotSupported;
     }
 }
 
-template <typename XT, typename RT>
+template <typename XT, typename RT, int VEC>
 hipError_t launch_r(int x_dtype, int out_dtype, int reduce_world, int mode, const QuantArgs &q, int quant_world,
                     const ReduceArgs &r, hipStream_t s) {
-    if (out_dtype == kF32) return launch_o<XT, RT, float>(reduce_world, mode, q, quant_world, r, s);
-    if (out_dtype == x_dtype) return launch_o<XT, RT, XT>(reduce_world, mode, q, quant_world, r, s);
+    if (out_dtype == kF32) return launch_o<XT, RT, VEC, float>(reduce_world, mode, q, quant_world, r, s);
+    if (out_dtype == x_dtype) return launch_o<XT, RT, VEC, XT>(reduce_world, mode, q, quant_world, r, s);
     return hipErrorNotSupported;
 }
 
 template <typename XT>
-hipError_t launch_x(int x_dtype, int r_dtype, int out_dtype, int reduce_world, int mode, const QuantArgs &q,
+hipError_t launch_x(int x_dtype, int r_dtype, int quant_vec, int out_dtype, int reduce_world, int mode, const QuantArgs &q,
                     int quant_world, const ReduceArgs &r, hipStream_t s) {
-    if (r_dtype == kNone) return launch_r<XT, void>(x_dtype, out_dtype, reduce_world, mode, q, quant_world, r, s);
-    if (r_dtype == kF32) return launch_r<XT, float>(x_dtype, out_dtype, reduce_world, mode, q, quant_world, r, s);
+    if (r_dtype == kF32 && quant_vec == 4) return launch_r<XT, float, 4>(x_dtype, out_dtype, reduce_world, mode, q, quant_world, r, s);
+    if (r_dtype != kNone) return hipErrorNotSupported;
+    if (quant_vec == 4) return launch_r<XT, void, 4>(x_dtype, out_dtype, reduce_world, mode, q, quant_world, r, s);
+    if constexpr (sizeof(XT) == 2) {
+        if (quant_vec == 8) return launch_r<XT, void, 8>(x_dtype, out_dtype, reduce_world, mode, q, quant_world, r, s);
+    }
     return hipErrorNotSupported;
 }
 
 }  // namespace
 
-hipError_t launch_bucket_step(int x_dtype, int r_dtype, int out_dtype, int reduce_world, int mode, const QuantArgs &quant,
-                              int quant_world, const ReduceArgs &reduce, hipStream_t stream) {
+hipError_t launch_bucket_step(int x_dtype, int r_dtype, int quant_vec, int out_dtype, int reduce_world, int mode,
+                              const QuantArgs &quant, int quant_world, const ReduceArgs &reduce, hipStream_t stream) {
     if (mode != kVector && mode != kStream) return hipErrorNotSupported;
     switch (x_dtype) {
-        case kF32: return launch_x<float>(x_dtype, r_dtype, out_dtype, reduce_world, mode, quant, quant_world, reduce, stream);
-        case kF16: return launch_x<f16>(x_dtype, r_dtype, out_dtype, reduce_world, mode, quant, quant_world, reduce, stream);
-        case kBF16: return launch_x<bf16>(x_dtype, r_dtype, out_dtype, reduce_world, mode, quant, quant_world, reduce, stream);
+        case kF32: return launch_x<float>(x_dtype, r_dtype, quant_vec, out_dtype, reduce_world, mode, quant, quant_world, reduce, stream);
+        case kF16: return launch_x<f16>(x_dtype, r_dtype, quant_vec, out_dtype, reduce_world, mode, quant, quant_world, reduce, stream);
+        case kBF16: return launch_x<bf16>(x_dtype, r_dtype, quant_vec, out_dtype, reduce_world, mode, quant, quant_world, reduce, stream);
         default: return hipErrorNotSupported;
     }
 }

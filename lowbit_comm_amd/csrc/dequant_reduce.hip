@@ -24,10 +24,6 @@ namespace {
 
 using namespace reduce;
 
-// Elements per lane of the fused reduce + requantize: 4 (one dword of codes per payload, 16 lanes per group
-// of 64) measured 3-4 % faster on a full bucket than 8 and the same on shards.
-constexpr int kReduceQuantVec = 4;
-
 template <typename OT, int G, int W, int MODE>
 __global__ __launch_bounds__(kBlock) void dequant_reduce_kernel(const ReduceArgs a) {
     dequant_reduce_block<OT, G, W, MODE>(a, blockIdx.x, gridDim.x);
@@ -74,76 +70,16 @@ hipError_t launch_reduce_t(int g, int world, int mode, const ReduceArgs &a, hipS
 }
 
 // ---------------------------------------------------------------------------
-// fused dequant-reduce + requantize (reduce-scatter shard -> all-gather payload)
+// fused dequant-reduce + requantize (reduce-scatter shard -> all-gather payload): dequant_reduce_quant_block
 // ---------------------------------------------------------------------------
-// The reduced shard never reaches memory: each lane folds its 4 elements over the W payloads exactly as
-// dequant_reduce_kernel does for an output of type MT (every partial sum rounded to MT, true division for
-// the mean), the group maximum is taken across the lanes of the group and the codes and the scale of the
-// new payload are written.  Elements past numel count as zeros, as the zero padding of a separate
-// quantize would.  Reads W*(g+4)/g bytes and writes (g+4)/g bytes per element.
 template <typename MT, int G, int W, int MODE>
 __global__ __launch_bounds__(kBlock) void dequant_reduce_quant_kernel(const ReduceQuantArgs a) {
-    constexpr int VEC = kReduceQuantVec;
-    constexpr int LPG = G / VEC;
-    constexpr int TILE = kWave * VEC;
-    constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock;
-    static_assert(LPG >= 1 && LPG <= 16, "a group must fit one DPP row");
-
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x >> 6;
-    const int64_t padded = (a.numel + G - 1) / G * G;
-    const int64_t e0 = static_cast<int64_t>(xcd_contiguous_block<true>(BLOCK_ELEMS)) * BLOCK_ELEMS + static_cast<int64_t>(wave) * TILE + lane * VEC;
-    const bool live = e0 < padded;     // whole lanes: padded and e0 are multiples of VEC
-    const bool mean = a.divisor != 1.0f;
-
-    float p[VEC];
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) p[i] = 0.0f;
-    if (live) {
-        uint32_t words[W][VEC / 4];
-        float scale[W];
-        const int64_t g = e0 / G;
-#pragma unroll
-        for (int r = 0; r < W; ++r) {
-            load_codes<VEC, code_load_mode<W>(MODE)>(a.codes[r] + e0, words[r]);
-            scale[r] = a.scales[r][g];
-        }
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) p[i] = round_through<MT>(code_to_float(words[0][i / 4], i % 4) * scale[0]);
-#pragma unroll
-        for (int r = 1; r < W; ++r) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                const float t = round_through<MT>(code_to_float(words[r][i / 4], i % 4) * scale[r]);
-                p[i] = round_through<MT>(p[i] + t);
-            }
-        }
-        if (mean) divide_all<MT, VEC>(p, a.divisor);
-        if (e0 + VEC > a.numel) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) p[i] = e0 + i < a.numel ? p[i] : 0.0f;
-        }
-    }
-    // every lane of the row takes part in the butterfly; lanes past the end contribute zeros
-    const float out_scale = group_scale<VEC, LPG>(p);
-    if (!live) return;
-    int c[VEC];
-    encode_group<VEC>(p, out_scale, c);
-    uint32_t out_words[VEC / 4];
-#pragma unroll
-    for (int k = 0; k < VEC / 4; ++k) out_words[k] = pack4(c[4 * k], c[4 * k + 1], c[4 * k + 2], c[4 * k + 3]);
-    if constexpr (MODE != kScalar) {
-        store_vec<uint32_t, VEC / 4, kVector>(reinterpret_cast<uint32_t *>(a.out_codes + e0), out_words);
-    } else {
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) a.out_codes[e0 + i] = static_cast<int8_t>(c[i]);
-    }
-    if ((lane & (LPG - 1)) == 0) a.out_scales[e0 / G] = out_scale;
+    dequant_reduce_quant_block<MT, G, W, MODE>(a, blockIdx.x, gridDim.x);
 }
 
 template <typename MT, int G, int W>
 hipError_t launch_reduce_quant_w(int mode, const ReduceQuantArgs &a, hipStream_t stream) {
-    constexpr int BLOCK_ELEMS = kWave * kReduceQuantVec * kWavesPerBlock;
+    constexpr int BLOCK_ELEMS = kReduceQuantBlockElems;
     const int64_t padded = (a.numel + G - 1) / G * G;
     const int64_t blocks = (padded + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
     if (blocks == 0) return hipSuccess;
@@ -183,78 +119,11 @@ hipError_t launch_reduce_quant_t(int g, int world, int mode, const ReduceQuantAr
 }
 
 // ---------------------------------------------------------------------------
-// decode of one payload, or of `world` shard payloads into consecutive shards
+// decode of one payload, or of `world` shard payloads into consecutive shards: decode_block
 // ---------------------------------------------------------------------------
-template <int OP> __device__ __forceinline__ float combine(float old, float v) {
-    if constexpr (OP == 1) return old + v;
-    else if constexpr (OP == 2) return old > v ? old : v;
-    else if constexpr (OP == 3) return old < v ? old : v;
-    else return v;
-}
-
-#ifndef LBC_DECODE1_UNROLL
-#define LBC_DECODE1_UNROLL 2
-#endif
-template <typename OT> struct decode1_tiling {
-    static constexpr int VEC = decode_tiling<OT>::VEC;
-    static constexpr int TILE = kWave * VEC;
-    static constexpr int UNROLL = LBC_DECODE1_UNROLL;   // a single payload has few loads per tile: keep more tiles in flight
-    static constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock * UNROLL;
-};
-
 template <typename OT, int G, int OP, int MODE>
 __global__ __launch_bounds__(kBlock) void decode_kernel(const DecodeArgs a) {
-    using T = decode1_tiling<OT>;
-    constexpr int VEC = T::VEC;
-    constexpr int UNROLL = T::UNROLL;
-
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x >> 6;
-    const int64_t chunk = blockIdx.y;
-    const int64_t chunk_start = chunk * a.shard_numel;
-    int64_t valid = a.total_numel - chunk_start;
-    valid = valid < 0 ? 0 : (valid > a.shard_numel ? a.shard_numel : valid);
-    const int8_t *__restrict__ codes = reinterpret_cast<const int8_t *>(a.codes_base + chunk * a.payload_stride);
-    const float *__restrict__ scales = reinterpret_cast<const float *>(a.scales_base + chunk * a.payload_stride);
-    OT *__restrict__ out = static_cast<OT *>(a.out) + chunk_start;
-    const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(T::BLOCK_ELEMS)) * T::BLOCK_ELEMS;
-    if (block_first >= valid) return;
-
-    if (MODE != kScalar && block_first + T::BLOCK_ELEMS <= valid) {
-        uint32_t words[UNROLL][VEC / 4];
-        float scale[UNROLL];
-        int64_t e0[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            e0[u] = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
-            load_codes<VEC, code_load_mode<1>(MODE)>(codes + e0[u], words[u]);
-            scale[u] = scales[e0[u] / G];
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            OT o[VEC];
-            if constexpr (OP != 0) load_vec<OT, VEC, MODE>(out + e0[u], o);
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                float v = round_through<OT>(code_to_float(words[u][i / 4], i % 4) * scale[u]);
-                if constexpr (OP != 0) v = round_through<OT>(combine<OP>(widen(o[i]), v));
-                o[i] = narrow<OT>(v);
-            }
-            store_vec<OT, VEC, MODE>(out + e0[u], o);
-        }
-        return;
-    }
-
-    for (int u = 0; u < UNROLL; ++u) {
-        const int64_t e0 = block_first + static_cast<int64_t>(tile_in_block<UNROLL>(u, wave)) * T::TILE + lane * VEC;
-        for (int i = 0; i < VEC; ++i) {
-            const int64_t e = e0 + i;
-            if (e >= valid) break;
-            float v = round_through<OT>(static_cast<float>(codes[e]) * scales[e / G]);
-            if constexpr (OP != 0) v = round_through<OT>(combine<OP>(widen(out[e]), v));
-            out[e] = narrow<OT>(v);
-        }
-    }
+    decode_block<OT, G, OP, MODE>(a, blockIdx.x, gridDim.x, blockIdx.y);
 }
 
 template <typename OT, int G, int OP>

@@ -19,6 +19,7 @@ struct QuantArgs {
     uint8_t *scales_base;    // chunk d: scales at scales_base + d * payload_stride
     void *new_residual;      // may be null
     void *restored;          // may be null
+    void *prepared;          // may be null: x + residual in its own type, for a caller that needs it later
     int64_t numel;           // valid elements in the whole tensor
     int64_t shard_numel;     // elements per chunk (== numel for a single payload)
     int64_t payload_stride;  // bytes
@@ -142,10 +143,17 @@ hipError_t launch_quant_pack(int x_dtype, int r_dtype, int d_dtype, bool outputs
 int quant_pack_vec(int x_dtype, int r_dtype, int d_dtype, bool outputs);
 hipError_t launch_dequant_reduce(int out_dtype, int group_size, int world, int mode,
                                  const ReduceArgs &args, hipStream_t stream);
-// Both of the above in one grid (group size 64; restored rounded to fp32; residual none or fp32; output fp32 or the
-// input's type; 2, 4 or 8 payloads; vector or streaming mode).  hipErrorNotSupported for anything else.
-hipError_t launch_bucket_step(int x_dtype, int r_dtype, int out_dtype, int reduce_world, int mode, const QuantArgs &quant,
-                              int quant_world, const ReduceArgs &reduce, hipStream_t stream);
+// Both of the above in one grid (group size 64; residual none or fp32; `quant_vec` = quant_pack_vec() of the quantize
+// call, which also fixes the new residual's type; output fp32 or the input's type; 2, 4 or 8 payloads; vector or
+// streaming mode).  hipErrorNotSupported for anything else.
+hipError_t launch_bucket_step(int x_dtype, int r_dtype, int quant_vec, int out_dtype, int reduce_world, int mode,
+                              const QuantArgs &quant, int quant_world, const ReduceArgs &reduce, hipStream_t stream);
+// Up to three stages of a bucket stream in one grid: chunked quantize (residual none or fp32, `quant_vec` as above),
+// reduce + requantize (2, 4 or 8 payloads) and decode of `decode_world` shard payloads, all in element type `dtype`,
+// group size 64, vector or streaming mode.  A null stage is absent.  hipErrorNotSupported for anything else.
+hipError_t launch_pipeline_step(int dtype, int r_dtype, int quant_vec, int mode, const QuantArgs *quant, int quant_world,
+                                const ReduceQuantArgs *reduce, int reduce_world, const DecodeArgs *decode, int decode_world,
+                                hipStream_t stream);
 // Reduce of `world` payloads in `mid_dtype` arithmetic, requantized without leaving the chip.
 hipError_t launch_dequant_reduce_quant(int mid_dtype, int group_size, int world, int mode,
                                        const ReduceQuantArgs &args, hipStream_t stream);

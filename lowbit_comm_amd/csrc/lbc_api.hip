@@ -74,7 +74,25 @@ struct ReduceCall {
     bool aligned = false;
 };
 
+struct ReduceQuantCall {
+    int status = LBC_OK;
+    bool empty = false;
+    lbc::ReduceQuantArgs args{};
+    int mid_dtype = LBC_F32, world = 0;
+    bool aligned = false;
+};
+
+struct DecodeCall {
+    int status = LBC_OK;
+    bool empty = false;
+    lbc::DecodeArgs args{};
+    int out_dtype = LBC_F32, world = 0;
+    bool aligned = false;
+};
+
 QuantCall refuse_quant(int status) { QuantCall c; c.status = status; return c; }
+ReduceQuantCall refuse_reduce_quant(int status) { ReduceQuantCall c; c.status = status; return c; }
+DecodeCall refuse_decode(int status) { DecodeCall c; c.status = status; return c; }
 ReduceCall refuse_reduce(int status) { ReduceCall c; c.status = status; return c; }
 
 // Shared body of lbc_quant_pack (world == 1, separate codes/scales pointers) and
@@ -82,9 +100,15 @@ ReduceCall refuse_reduce(int status) { ReduceCall c; c.status = status; return c
 QuantCall quant_pack_common(const void *x, int x_dtype, const void *residual, int residual_dtype,
                             int64_t numel, int world, int group_size, uint8_t *codes_base, uint8_t *scales_base,
                             int64_t payload_stride, int64_t shard_numel, void *new_residual, int new_residual_dtype,
-                            void *restored, int restored_dtype) {
+                            void *restored, int restored_dtype, void *prepared, int prepared_dtype) {
     const int r_dtype = residual ? residual_dtype : LBC_NONE;
     const int p_dtype = residual ? promote(x_dtype, r_dtype) : x_dtype;
+    if (prepared != nullptr && prepared_dtype != p_dtype)
+        return refuse_quant(fail(LBC_EINVAL, "prepared must have the promoted dtype of input and residual"));
+    if (prepared != nullptr && (prepared == x || prepared == residual || prepared == new_residual || prepared == restored))
+        return refuse_quant(fail(LBC_EINVAL, "prepared must not alias another tensor of the call"));
+    if (prepared != nullptr && !aligned_to(prepared, dtype_size(p_dtype)))
+        return refuse_quant(fail(LBC_EINVAL, "prepared is not aligned to its element size"));
     const bool wants_outputs = new_residual != nullptr || restored != nullptr;
     int d_dtype = LBC_F32;
     if (wants_outputs) {
@@ -110,6 +134,7 @@ QuantCall quant_pack_common(const void *x, int x_dtype, const void *residual, in
     side(residual, r_dtype);
     side(new_residual, new_residual_dtype);
     side(restored, d_dtype);
+    side(prepared, p_dtype);
 
     QuantCall c;
     c.args.x = x;
@@ -118,6 +143,7 @@ QuantCall quant_pack_common(const void *x, int x_dtype, const void *residual, in
     c.args.scales_base = scales_base;
     c.args.new_residual = new_residual;
     c.args.restored = restored;
+    c.args.prepared = prepared;
     c.args.numel = numel;
     c.args.shard_numel = shard_numel;
     c.args.payload_stride = payload_stride;
@@ -141,7 +167,8 @@ int launch_quant(const QuantCall &c, const char *what, int access, void *stream)
 // Validation of lbc_quant_pack_chunks, shared with the entry point that carries a reduce in the same launch.
 QuantCall prepare_quant_chunks(const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel,
                                int world, int group_size, uint8_t *payloads, int64_t payload_stride, void *new_residual,
-                               int new_residual_dtype, void *restored, int restored_dtype) {
+                               int new_residual_dtype, void *restored, int restored_dtype, void *prepared,
+                               int prepared_dtype) {
     if (numel < 0) return refuse_quant(fail(LBC_EINVAL, "numel must be >= 0"));
     if (world <= 0) return refuse_quant(fail(LBC_EINVAL, "world must be > 0"));
     if (!valid_dtype(x_dtype)) return refuse_quant(fail(LBC_EINVAL, "unsupported input dtype %d", x_dtype));
@@ -164,7 +191,7 @@ QuantCall prepare_quant_chunks(const void *x, int x_dtype, const void *residual,
     if (!aligned_to(x, dtype_size(x_dtype))) return refuse_quant(fail(LBC_EINVAL, "input is not aligned to its element size"));
     return quant_pack_common(x, x_dtype, residual, residual_dtype, numel, world, group_size, payloads,
                              payloads + groups * group_size, payload_stride, shard, new_residual, new_residual_dtype,
-                             restored, restored_dtype);
+                             restored, restored_dtype, prepared, prepared_dtype);
 }
 
 // Validation of lbc_dequant_reduce, shared in the same way.
@@ -212,6 +239,77 @@ ReduceCall prepare_reduce(const int8_t *const *codes, const float *const *scales
     return c;
 }
 
+// Validation of lbc_dequant_reduce_quant, shared with the pipeline step.
+ReduceQuantCall prepare_reduce_quant(const int8_t *const *codes, const float *const *scales, int world, int64_t numel,
+                                     int group_size, float divisor, int mid_dtype, int8_t *out_codes, float *out_scales) {
+    if (world <= 0) return refuse_reduce_quant(fail(LBC_EINVAL, "inputs must not be empty"));
+    if (numel < 0) return refuse_reduce_quant(fail(LBC_EINVAL, "numel must be >= 0"));
+    if (!(divisor > 0.0f)) return refuse_reduce_quant(fail(LBC_EINVAL, "divisor must be > 0"));
+    if (!valid_dtype(mid_dtype)) return refuse_reduce_quant(fail(LBC_EINVAL, "unsupported intermediate dtype %d", mid_dtype));
+    if (world > LBC_MAX_PAYLOADS || !valid_group(group_size)) return refuse_reduce_quant(LBC_UNSUPPORTED);
+    ReduceQuantCall c;
+    if (numel == 0) {
+        c.empty = true;
+        return c;
+    }
+    if (codes == nullptr || scales == nullptr || out_codes == nullptr || out_scales == nullptr)
+        return refuse_reduce_quant(fail(LBC_EINVAL, "codes, scales, out_codes and out_scales must not be null"));
+    if (!aligned_to(out_scales, 4)) return refuse_reduce_quant(fail(LBC_EINVAL, "out_scales must be 4-byte aligned"));
+    bool aligned = aligned_to(out_codes, 4);
+    for (int r = 0; r < world; ++r) {
+        if (codes[r] == nullptr || scales[r] == nullptr) return refuse_reduce_quant(fail(LBC_EINVAL, "payload %d has a null pointer", r));
+        if (!aligned_to(scales[r], 4)) return refuse_reduce_quant(fail(LBC_EINVAL, "scales of payload %d must be 4-byte aligned", r));
+        if (codes[r] == out_codes || scales[r] == out_scales)
+            return refuse_reduce_quant(fail(LBC_EINVAL, "the output payload must not alias input payload %d", r));
+        aligned = aligned && aligned_to(codes[r], 4);
+        c.args.codes[r] = codes[r];
+        c.args.scales[r] = scales[r];
+    }
+    c.args.out_codes = out_codes;
+    c.args.out_scales = out_scales;
+    c.args.numel = numel;
+    c.args.divisor = divisor;
+    c.mid_dtype = mid_dtype;
+    c.world = world;
+    c.aligned = aligned;
+    return c;
+}
+
+// Validation of lbc_dequant_chunks, shared in the same way.
+DecodeCall prepare_decode_chunks(const uint8_t *payloads, int64_t payload_stride, int world, int64_t shard_numel,
+                                 int64_t total_numel, int group_size, void *out, int out_dtype) {
+    if (shard_numel < 0 || total_numel < 0) return refuse_decode(fail(LBC_EINVAL, "element counts must be >= 0"));
+    if (world <= 0) return refuse_decode(fail(LBC_EINVAL, "world must be > 0"));
+    if (total_numel > shard_numel * world) return refuse_decode(fail(LBC_EINVAL, "total_numel exceeds world * shard_numel"));
+    if (!valid_dtype(out_dtype)) return refuse_decode(fail(LBC_EINVAL, "unsupported output dtype %d", out_dtype));
+    if (!valid_group(group_size)) return refuse_decode(LBC_UNSUPPORTED);
+    if (world > 65535) return refuse_decode(LBC_UNSUPPORTED);
+    DecodeCall c;
+    if (shard_numel == 0 || total_numel == 0) {
+        c.empty = true;
+        return c;
+    }
+    const int64_t groups = (shard_numel + group_size - 1) / group_size;
+    const int64_t payload_bytes = groups * (group_size + 4);
+    if (payloads == nullptr || out == nullptr) return refuse_decode(fail(LBC_EINVAL, "payloads and out must not be null"));
+    if (payload_stride < payload_bytes || (payload_stride & 3) != 0)
+        return refuse_decode(fail(LBC_EINVAL, "payload_stride must be a multiple of 4 and >= %lld", (long long)payload_bytes));
+    if (!aligned_to(payloads, 4)) return refuse_decode(fail(LBC_EINVAL, "payloads must be 4-byte aligned"));
+    if (!aligned_to(out, dtype_size(out_dtype))) return refuse_decode(fail(LBC_EINVAL, "out is not aligned to its element size"));
+    const int vec = out_dtype == LBC_F32 ? 4 : 8;
+    c.aligned = aligned_to(payloads, vec) && payload_stride % vec == 0 && aligned_to(out, 16) &&
+                (shard_numel * dtype_size(out_dtype)) % 16 == 0;
+    c.args.codes_base = payloads;
+    c.args.scales_base = payloads + groups * group_size;
+    c.args.out = out;
+    c.args.shard_numel = shard_numel;
+    c.args.total_numel = total_numel;
+    c.args.payload_stride = payload_stride;
+    c.out_dtype = out_dtype;
+    c.world = world;
+    return c;
+}
+
 int launch_reduce(const ReduceCall &c, int access, void *stream) {
     if (c.status != LBC_OK || c.empty) return c.status;
     return finish(lbc::launch_dequant_reduce(c.out_dtype, c.group_size, c.world,
@@ -230,7 +328,7 @@ const char *lbc_last_error(void) { return g_error; }
 
 int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel,
                    int group_size, int8_t *codes, float *scales, void *new_residual, int new_residual_dtype,
-                   void *restored, int restored_dtype, int access, void *stream) {
+                   void *restored, int restored_dtype, void *prepared, int prepared_dtype, int access, void *stream) {
     if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
     if (!valid_dtype(x_dtype)) return fail(LBC_EINVAL, "unsupported input dtype %d", x_dtype);
@@ -244,16 +342,18 @@ int lbc_quant_pack(const void *x, int x_dtype, const void *residual, int residua
     if (!aligned_to(x, dtype_size(x_dtype))) return fail(LBC_EINVAL, "input is not aligned to its element size");
     return launch_quant(quant_pack_common(x, x_dtype, residual, residual_dtype, numel, 1, group_size,
                                           reinterpret_cast<uint8_t *>(codes), reinterpret_cast<uint8_t *>(scales), 0, numel,
-                                          new_residual, new_residual_dtype, restored, restored_dtype),
+                                          new_residual, new_residual_dtype, restored, restored_dtype, prepared, prepared_dtype),
                         "lbc_quant_pack", access, stream);
 }
 
 int lbc_quant_pack_chunks(const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel,
                           int world, int group_size, uint8_t *payloads, int64_t payload_stride, void *new_residual,
-                          int new_residual_dtype, void *restored, int restored_dtype, int access, void *stream) {
+                          int new_residual_dtype, void *restored, int restored_dtype, void *prepared, int prepared_dtype,
+                          int access, void *stream) {
     if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     return launch_quant(prepare_quant_chunks(x, x_dtype, residual, residual_dtype, numel, world, group_size, payloads,
-                                             payload_stride, new_residual, new_residual_dtype, restored, restored_dtype),
+                                             payload_stride, new_residual, new_residual_dtype, restored, restored_dtype,
+                                             prepared, prepared_dtype),
                         "lbc_quant_pack_chunks", access, stream);
 }
 
@@ -287,32 +387,10 @@ int lbc_dequant(const int8_t *codes, const float *scales, int64_t numel, int gro
 int lbc_dequant_chunks(const uint8_t *payloads, int64_t payload_stride, int world, int64_t shard_numel,
                        int64_t total_numel, int group_size, void *out, int out_dtype, int access, void *stream) {
     if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
-    if (shard_numel < 0 || total_numel < 0) return fail(LBC_EINVAL, "element counts must be >= 0");
-    if (world <= 0) return fail(LBC_EINVAL, "world must be > 0");
-    if (total_numel > shard_numel * world) return fail(LBC_EINVAL, "total_numel exceeds world * shard_numel");
-    if (!valid_dtype(out_dtype)) return fail(LBC_EINVAL, "unsupported output dtype %d", out_dtype);
-    if (!valid_group(group_size)) return LBC_UNSUPPORTED;
-    if (world > 65535) return LBC_UNSUPPORTED;
-    if (shard_numel == 0 || total_numel == 0) return LBC_OK;
-    const int64_t groups = (shard_numel + group_size - 1) / group_size;
-    const int64_t payload_bytes = groups * (group_size + 4);
-    if (payloads == nullptr || out == nullptr) return fail(LBC_EINVAL, "payloads and out must not be null");
-    if (payload_stride < payload_bytes || (payload_stride & 3) != 0)
-        return fail(LBC_EINVAL, "payload_stride must be a multiple of 4 and >= %lld", (long long)payload_bytes);
-    if (!aligned_to(payloads, 4)) return fail(LBC_EINVAL, "payloads must be 4-byte aligned");
-    if (!aligned_to(out, dtype_size(out_dtype))) return fail(LBC_EINVAL, "out is not aligned to its element size");
-    const int vec = out_dtype == LBC_F32 ? 4 : 8;
-    const bool aligned = aligned_to(payloads, vec) && payload_stride % vec == 0 && aligned_to(out, 16) &&
-                         (shard_numel * dtype_size(out_dtype)) % 16 == 0;
-    lbc::DecodeArgs a{};
-    a.codes_base = payloads;
-    a.scales_base = payloads + groups * group_size;
-    a.out = out;
-    a.shard_numel = shard_numel;
-    a.total_numel = total_numel;
-    a.payload_stride = payload_stride;
-    return finish(lbc::launch_decode(out_dtype, group_size, LBC_REDUCE_NONE,
-                                     pick_mode(aligned, access), a, world,
+    const DecodeCall c = prepare_decode_chunks(payloads, payload_stride, world, shard_numel, total_numel, group_size, out,
+                                               out_dtype);
+    if (c.status != LBC_OK || c.empty) return c.status;
+    return finish(lbc::launch_decode(c.out_dtype, group_size, LBC_REDUCE_NONE, pick_mode(c.aligned, access), c.args, c.world,
                                      static_cast<hipStream_t>(stream)),
                   "lbc_dequant_chunks");
 }
@@ -333,7 +411,8 @@ int lbc_quant_pack_chunks_and_dequant_reduce(
     void *out, int out_dtype, const void *prepared, void *reduce_new_residual, int access, void *stream) {
     if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
     const QuantCall q = prepare_quant_chunks(x, x_dtype, residual, residual_dtype, numel, world, group_size, payloads,
-                                             payload_stride, new_residual, new_residual_dtype, nullptr, LBC_F32);
+                                             payload_stride, new_residual, new_residual_dtype, nullptr, LBC_F32, nullptr,
+                                             LBC_NONE);
     if (q.status != LBC_OK) return q.status;
     const ReduceCall r = prepare_reduce(codes, scales, reduce_world, reduce_numel, group_size, divisor, out, out_dtype,
                                         prepared, reduce_new_residual);
@@ -344,7 +423,9 @@ int lbc_quant_pack_chunks_and_dequant_reduce(
     // 2, 4 or 8 payloads; everything else is for the caller to issue as the two separate calls
     if (!q.aligned || !r.aligned || group_size != 64 || (q.r_dtype != LBC_NONE && q.r_dtype != LBC_F32))
         return LBC_UNSUPPORTED;
-    return finish(lbc::launch_bucket_step(q.x_dtype, q.r_dtype, r.out_dtype, r.world, pick_mode(true, access), q.args,
+    // the quantize half is the instantiation the separate call would run: its lane width also decided q.aligned
+    const int vec = lbc::quant_pack_vec(q.x_dtype, q.r_dtype, q.d_dtype, q.outputs);
+    return finish(lbc::launch_bucket_step(q.x_dtype, q.r_dtype, vec, r.out_dtype, r.world, pick_mode(true, access), q.args,
                                           q.world, r.args, static_cast<hipStream_t>(stream)),
                   "lbc_quant_pack_chunks_and_dequant_reduce");
 }
@@ -352,33 +433,62 @@ int lbc_quant_pack_chunks_and_dequant_reduce(
 int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *scales, int world, int64_t numel,
                              int group_size, float divisor, int mid_dtype, int8_t *out_codes, float *out_scales, int access, void *stream) {
     if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
-    if (world <= 0) return fail(LBC_EINVAL, "inputs must not be empty");
-    if (numel < 0) return fail(LBC_EINVAL, "numel must be >= 0");
-    if (!(divisor > 0.0f)) return fail(LBC_EINVAL, "divisor must be > 0");
-    if (!valid_dtype(mid_dtype)) return fail(LBC_EINVAL, "unsupported intermediate dtype %d", mid_dtype);
-    if (world > LBC_MAX_PAYLOADS || !valid_group(group_size)) return LBC_UNSUPPORTED;
-    if (numel == 0) return LBC_OK;
-    if (codes == nullptr || scales == nullptr || out_codes == nullptr || out_scales == nullptr)
-        return fail(LBC_EINVAL, "codes, scales, out_codes and out_scales must not be null");
-    if (!aligned_to(out_scales, 4)) return fail(LBC_EINVAL, "out_scales must be 4-byte aligned");
-    bool aligned = aligned_to(out_codes, 4);
-    lbc::ReduceQuantArgs a{};
-    for (int r = 0; r < world; ++r) {
-        if (codes[r] == nullptr || scales[r] == nullptr) return fail(LBC_EINVAL, "payload %d has a null pointer", r);
-        if (!aligned_to(scales[r], 4)) return fail(LBC_EINVAL, "scales of payload %d must be 4-byte aligned", r);
-        if (codes[r] == out_codes || scales[r] == out_scales)
-            return fail(LBC_EINVAL, "the output payload must not alias input payload %d", r);
-        aligned = aligned && aligned_to(codes[r], 4);
-        a.codes[r] = codes[r];
-        a.scales[r] = scales[r];
-    }
-    a.out_codes = out_codes;
-    a.out_scales = out_scales;
-    a.numel = numel;
-    a.divisor = divisor;
-    return finish(lbc::launch_dequant_reduce_quant(mid_dtype, group_size, world, pick_mode(aligned, access),
-                                                   a, static_cast<hipStream_t>(stream)),
+    const ReduceQuantCall c = prepare_reduce_quant(codes, scales, world, numel, group_size, divisor, mid_dtype, out_codes,
+                                                   out_scales);
+    if (c.status != LBC_OK || c.empty) return c.status;
+    return finish(lbc::launch_dequant_reduce_quant(c.mid_dtype, group_size, c.world, pick_mode(c.aligned, access), c.args,
+                                                   static_cast<hipStream_t>(stream)),
                   "lbc_dequant_reduce_quant");
+}
+
+int lbc_bucket_pipeline_step(const lbc_quant_chunks_stage *quant, const lbc_reduce_quant_stage *reduce,
+                             const lbc_dequant_chunks_stage *decode, int group_size, int access, void *stream) {
+    if (!valid_access(access)) return fail(LBC_EINVAL, "unknown access mode %d", access);
+    QuantCall q;
+    q.empty = true;
+    if (quant != nullptr) {
+        q = prepare_quant_chunks(quant->x, quant->x_dtype, quant->residual, quant->residual_dtype, quant->numel, quant->world,
+                                 group_size, quant->payloads, quant->payload_stride, quant->new_residual,
+                                 quant->new_residual_dtype, nullptr, LBC_F32, nullptr, LBC_NONE);
+        if (q.status != LBC_OK) return q.status;
+    }
+    ReduceQuantCall r;
+    r.empty = true;
+    if (reduce != nullptr) {
+        r = prepare_reduce_quant(reduce->codes, reduce->scales, reduce->world, reduce->numel, group_size, reduce->divisor,
+                                 reduce->mid_dtype, reduce->out_codes, reduce->out_scales);
+        if (r.status != LBC_OK) return r.status;
+    }
+    DecodeCall d;
+    d.empty = true;
+    if (decode != nullptr) {
+        d = prepare_decode_chunks(decode->payloads, decode->payload_stride, decode->world, decode->shard_numel,
+                                  decode->total_numel, group_size, decode->out, decode->out_dtype);
+        if (d.status != LBC_OK) return d.status;
+    }
+    const int stages = (q.empty ? 0 : 1) + (r.empty ? 0 : 1) + (d.empty ? 0 : 1);
+    if (stages == 0) return LBC_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (stages == 1) {          // one stage with work: its own kernel
+        if (!q.empty) return launch_quant(q, "lbc_bucket_pipeline_step", access, stream);
+        if (!r.empty)
+            return finish(lbc::launch_dequant_reduce_quant(r.mid_dtype, group_size, r.world, pick_mode(r.aligned, access), r.args, s),
+                          "lbc_bucket_pipeline_step");
+        return finish(lbc::launch_decode(d.out_dtype, group_size, LBC_REDUCE_NONE, pick_mode(d.aligned, access), d.args, d.world, s),
+                      "lbc_bucket_pipeline_step");
+    }
+    // one grid exists for group 64, operands aligned for the vector kernels, a residual that is absent or fp32,
+    // 2, 4 or 8 payloads to reduce, and one element type for the bucket, the reduce and the decoded output
+    if (group_size != 64 || (!q.empty && !q.aligned) || (!r.empty && !r.aligned) || (!d.empty && !d.aligned))
+        return LBC_UNSUPPORTED;
+    if (!q.empty && q.r_dtype != LBC_NONE && q.r_dtype != LBC_F32) return LBC_UNSUPPORTED;
+    const int dtype = !q.empty ? q.x_dtype : (!r.empty ? r.mid_dtype : d.out_dtype);
+    if ((!r.empty && r.mid_dtype != dtype) || (!d.empty && d.out_dtype != dtype)) return LBC_UNSUPPORTED;
+    const int vec = q.empty ? 4 : lbc::quant_pack_vec(q.x_dtype, q.r_dtype, q.d_dtype, q.outputs);
+    return finish(lbc::launch_pipeline_step(dtype, q.empty ? LBC_NONE : q.r_dtype, vec, pick_mode(true, access),
+                                            q.empty ? nullptr : &q.args, q.world, r.empty ? nullptr : &r.args, r.world,
+                                            d.empty ? nullptr : &d.args, d.world, s),
+                  "lbc_bucket_pipeline_step");
 }
 
 int lbc_ring_step(const int8_t *recv_codes, const float *recv_scales, void *chunk, int dtype, int64_t numel,

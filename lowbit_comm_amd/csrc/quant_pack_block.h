@@ -41,7 +41,8 @@ template <int VEC> struct quant_tiling {
     static constexpr int BLOCK_ELEMS = TILE * kWavesPerBlock * UNROLL;
 };
 
-// XT input, RT residual (void = none), DT type `restored` is rounded to.
+// XT input, RT residual (void = none), DT type `restored` is rounded to.  Optional outputs besides the payload:
+// `restored` (DT), `new_residual` = p - restored (promotion of p's type and DT) and `prepared` = p itself (p's type).
 // One workgroup's share: block `block_x` of `grid_x` along the chunk, destination chunk `chunk`.
 template <typename XT, typename RT, typename DT, int G, int VEC, int MODE>
 __device__ __forceinline__ void quant_pack_block(const QuantArgs &a, unsigned block_x, unsigned grid_x, unsigned chunk_index) {
@@ -69,6 +70,7 @@ __device__ __forceinline__ void quant_pack_block(const QuantArgs &a, unsigned bl
     float *__restrict__ scales = reinterpret_cast<float *>(a.scales_base + chunk * a.payload_stride);
     NT *new_r = a.new_residual ? static_cast<NT *>(a.new_residual) + chunk_start : nullptr;
     DT *__restrict__ restored = a.restored ? static_cast<DT *>(a.restored) + chunk_start : nullptr;
+    PT *__restrict__ prepared = a.prepared ? static_cast<PT *>(a.prepared) + chunk_start : nullptr;
 
     const int64_t block_first = static_cast<int64_t>(xcd_contiguous_block(block_x, grid_x, T::BLOCK_ELEMS)) * T::BLOCK_ELEMS;
     if (block_first >= padded) return;
@@ -148,6 +150,12 @@ __device__ __forceinline__ void quant_pack_block(const QuantArgs &a, unsigned bl
             }
             buffer_store<uint32_t, VEC / 4, kCodeStore>(codes_b, at[u], words);
 
+            if (prepared != nullptr) {
+                PT prep_out[VEC];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) prep_out[i] = narrow<PT>(p[u][i]);
+                buffer_store<PT, VEC, kSideStore>(buffer_over(prepared + block_first, T::BLOCK_ELEMS * sizeof(PT)), at[u] * sizeof(PT), prep_out);
+            }
             if (new_r != nullptr || restored != nullptr) {
                 DT rest_out[VEC];
                 NT diff_out[VEC];
@@ -191,6 +199,7 @@ __device__ __forceinline__ void quant_pack_block(const QuantArgs &a, unsigned bl
             const int c = encode(p[i], scale);
             if (e < padded) codes[e] = static_cast<int8_t>(c);
             if (e < valid) {
+                if (prepared != nullptr) prepared[e] = narrow<PT>(p[i]);
                 const float rest = round_through<DT>(static_cast<float>(c) * scale);
                 if (restored != nullptr) restored[e] = narrow<DT>(rest);
                 if (new_r != nullptr) new_r[e] = narrow<NT>(p[i] - rest);

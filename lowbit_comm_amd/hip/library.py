@@ -11,7 +11,7 @@ from pathlib import Path
 from lowbit_comm_amd.exceptions import CCDLUnavailableError
 
 LIBRARY_PATH = Path(__file__).resolve().parent.parent / "liblbc_hip.so"
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 LBC_OK = 0
 LBC_UNSUPPORTED = 1
@@ -25,9 +25,9 @@ SIGNATURES = {
     "lbc_abi_version": (_c_int, []),
     "lbc_last_error": (ctypes.c_char_p, []),
     "lbc_quant_pack": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_ptr, _c_ptr,
-                                _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
+                                _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
     "lbc_quant_pack_chunks": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_ptr, _c_i64,
-                                       _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
+                                       _c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
     "lbc_dequant": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]),
     "lbc_dequant_chunks": (_c_int, [_c_ptr, _c_i64, _c_int, _c_i64, _c_i64, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]),
     "lbc_dequant_reduce": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_ptr, _c_int,
@@ -37,6 +37,7 @@ SIGNATURES = {
         _c_ptr, _c_ptr, _c_int, _c_i64, ctypes.c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr]),
     "lbc_dequant_reduce_quant": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, ctypes.c_float, _c_int, _c_ptr,
                                           _c_ptr, _c_int, _c_ptr]),
+    "lbc_bucket_pipeline_step": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr]),
     "lbc_ring_step": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, ctypes.c_float, _c_ptr, _c_ptr,
                                _c_int, _c_ptr]),
     "lbc_ef_update": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_ptr]),
@@ -56,6 +57,30 @@ SIGNATURES = {
     "lbc_wire_dequant_general": (_c_int, [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int,
                                           _c_int, _c_ptr]),
 }
+
+
+
+class QuantChunksStage(ctypes.Structure):
+    """``lbc_quant_chunks_stage`` of include/lbc.h."""
+
+    _fields_ = [("x", _c_ptr), ("residual", _c_ptr), ("payloads", _c_ptr), ("new_residual", _c_ptr),
+                ("numel", _c_i64), ("payload_stride", _c_i64),
+                ("x_dtype", _c_int), ("residual_dtype", _c_int), ("new_residual_dtype", _c_int), ("world", _c_int)]
+
+
+class ReduceQuantStage(ctypes.Structure):
+    """``lbc_reduce_quant_stage`` of include/lbc.h."""
+
+    _fields_ = [("codes", _c_ptr), ("scales", _c_ptr), ("out_codes", _c_ptr), ("out_scales", _c_ptr),
+                ("numel", _c_i64), ("divisor", ctypes.c_float), ("world", _c_int), ("mid_dtype", _c_int)]
+
+
+class DequantChunksStage(ctypes.Structure):
+    """``lbc_dequant_chunks_stage`` of include/lbc.h."""
+
+    _fields_ = [("payloads", _c_ptr), ("out", _c_ptr), ("payload_stride", _c_i64), ("shard_numel", _c_i64),
+                ("total_numel", _c_i64), ("world", _c_int), ("out_dtype", _c_int)]
+
 
 _library: ctypes.CDLL | None = None
 

@@ -175,15 +175,17 @@ class BoundLaunch:
     the per-bucket fast path: a DDP hook binds once per bucket shape and replays every step.
     """
 
-    __slots__ = ("_fn", "_args", "_device", "_lib", "_keep", "_kind")
+    __slots__ = ("_fn", "_args", "_device", "_lib", "_keep", "_kind", "_hold")
 
-    def __init__(self, fn, args: tuple, device: torch.device, lib, keep: tuple, kind: str | None = None) -> None:
+    def __init__(self, fn, args: tuple, device: torch.device, lib, keep: tuple, kind: str | None = None,
+                 hold: tuple = ()) -> None:
         self._fn = fn
         self._args = args
         self._device = device
         self._lib = lib
         self._keep = keep
         self._kind = kind      # which entry point the arguments belong to, for launches that can share a grid
+        self._hold = hold      # host memory the arguments point into (argument structures, pointer arrays)
 
     def forget_tensors(self) -> "BoundLaunch":
         """Stop keeping the bound tensors alive.  For a cache keyed by everything the binding depends on (addresses,
@@ -212,7 +214,7 @@ def _finish(rc: int, lib) -> bool:
     raise RuntimeError(last_error(lib) or f"lbc call failed with code {rc}")
 
 
-def _side_tensors(x: torch.Tensor, residual, new_residual, restored, restored_dtype):
+def _side_tensors(x: torch.Tensor, residual, new_residual, restored, restored_dtype, prepared_out=None):
     """Validate the optional error-feedback tensors of a quantize call; returns their dtype codes."""
     device, n = x.device, x.numel()
     r_code = _NONE
@@ -232,7 +234,13 @@ def _side_tensors(x: torch.Tensor, residual, new_residual, restored, restored_dt
         _require(new_residual.numel() == n, "input and new_residual must have the same number of elements")
         _require(new_residual.dtype == promote(p_dtype, d_dtype),
                  f"new_residual must have dtype {promote(p_dtype, d_dtype)}")
-    return r_code, n_code, d_code
+    p_code = _NONE
+    if prepared_out is not None:
+        p_code = _float_tensor(prepared_out, "prepared_out", device)
+        _require(prepared_out.numel() >= n, "prepared_out must have at least input.numel() elements")
+        _require(prepared_out.dtype == p_dtype, f"prepared_out must have dtype {p_dtype}")
+    return r_code, n_code, d_code, p_code
+
 
 
 # --------------------------------------------------------------------------- #
@@ -241,16 +249,17 @@ def _side_tensors(x: torch.Tensor, residual, new_residual, restored, restored_dt
 def quant_pack_into(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, *, group_size: int = 64,
                     residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
                     restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None,
-                    access: str | None = None) -> bool:
-    """``codes, scales <- quant(x + residual)``; optionally ``restored`` and ``new_residual = p - restored``."""
+                    prepared_out: torch.Tensor | None = None, access: str | None = None) -> bool:
+    """``codes, scales <- quant(p)``, ``p = x + residual``; optionally ``restored``, ``new_residual = p - restored``
+    and ``prepared_out = p``."""
     return bind_quant_pack(x, codes, scales, group_size=group_size, residual=residual, new_residual=new_residual,
-                           restored=restored, restored_dtype=restored_dtype, access=access)()
+                           restored=restored, restored_dtype=restored_dtype, prepared_out=prepared_out, access=access)()
 
 
 def bind_quant_pack(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, *, group_size: int = 64,
                     residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
                     restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None,
-                    access: str | None = None) -> BoundLaunch:
+                    prepared_out: torch.Tensor | None = None, access: str | None = None) -> BoundLaunch:
     """Validate once; the returned :class:`BoundLaunch` replays :func:`quant_pack_into` on the same tensors."""
     lib = load_library()
     x_code = _float_tensor(x, "input")
@@ -263,26 +272,27 @@ def bind_quant_pack(x: torch.Tensor, codes: torch.Tensor, scales: torch.Tensor, 
     _require(scales.dtype == torch.float32, "scales must have float32 dtype")
     _require(codes.numel() == groups * group_size, "codes has an invalid quantized payload size")
     _require(scales.numel() == groups, "scales has an invalid group count")
-    r_code, n_code, d_code = _side_tensors(x, residual, new_residual, restored, restored_dtype)
+    r_code, n_code, d_code, p_code = _side_tensors(x, residual, new_residual, restored, restored_dtype, prepared_out)
     args = (_ptr(x), x_code, _ptr(residual), r_code, n, group_size, _ptr(codes), _ptr(scales),
-            _ptr(new_residual), n_code, _ptr(restored), d_code)
+            _ptr(new_residual), n_code, _ptr(restored), d_code, _ptr(prepared_out), p_code)
     return BoundLaunch(lib.lbc_quant_pack, args + (access_code(access),), device, lib,
-                       (x, codes, scales, residual, new_residual, restored))
+                       (x, codes, scales, residual, new_residual, restored, prepared_out))
 
 
 def bind_quant_pack_payload(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64,
                             residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
                             restored: torch.Tensor | None = None,
-                            restored_dtype: torch.dtype | None = None, access: str | None = None) -> BoundLaunch:
+                            restored_dtype: torch.dtype | None = None, prepared_out: torch.Tensor | None = None,
+                            access: str | None = None) -> BoundLaunch:
     """:func:`bind_quant_pack` writing the packed ``uint8[codes || scales]`` wire layout into ``payload``."""
     lib = load_library()
     x_code = _float_tensor(x, "input")
     codes_at, scales_at = payload_addresses(payload, x.numel(), group_size, name="output", device=x.device)
-    r_code, n_code, d_code = _side_tensors(x, residual, new_residual, restored, restored_dtype)
+    r_code, n_code, d_code, p_code = _side_tensors(x, residual, new_residual, restored, restored_dtype, prepared_out)
     args = (_ptr(x), x_code, _ptr(residual), r_code, x.numel(), group_size, ctypes.c_void_p(codes_at),
-            ctypes.c_void_p(scales_at), _ptr(new_residual), n_code, _ptr(restored), d_code)
+            ctypes.c_void_p(scales_at), _ptr(new_residual), n_code, _ptr(restored), d_code, _ptr(prepared_out), p_code)
     return BoundLaunch(lib.lbc_quant_pack, args + (access_code(access),), x.device, lib,
-                       (x, payload, residual, new_residual, restored))
+                       (x, payload, residual, new_residual, restored, prepared_out))
 
 
 def quant_pack_payload_into(x: torch.Tensor, payload: torch.Tensor, *, group_size: int = 64, **kwargs) -> bool:
@@ -303,19 +313,20 @@ def quant_pack(x: torch.Tensor, *, group_size: int = 64, residual: torch.Tensor 
 def quant_pack_chunks_into(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64,
                            residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
                            restored: torch.Tensor | None = None, restored_dtype: torch.dtype | None = None,
-                           access: str | None = None) -> bool:
+                           prepared_out: torch.Tensor | None = None, access: str | None = None) -> bool:
     """Quantize the ``world`` destination chunks of ``x`` (+ ``residual``) into the rows of ``payloads``
     (uint8 ``[world, stride]``) in one launch; optional fused error-feedback outputs as in
     :func:`quant_pack_into`."""
     return bind_quant_pack_chunks(x, payloads, world, group_size=group_size, residual=residual,
                                   new_residual=new_residual, restored=restored, restored_dtype=restored_dtype,
-                                  access=access)()
+                                  prepared_out=prepared_out, access=access)()
 
 
 def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, *, group_size: int = 64,
                            residual: torch.Tensor | None = None, new_residual: torch.Tensor | None = None,
                            restored: torch.Tensor | None = None,
-                           restored_dtype: torch.dtype | None = None, access: str | None = None) -> BoundLaunch:
+                           restored_dtype: torch.dtype | None = None, prepared_out: torch.Tensor | None = None,
+                           access: str | None = None) -> BoundLaunch:
     lib = load_library()
     x_code = _float_tensor(x, "input")
     device = x.device
@@ -325,11 +336,11 @@ def bind_quant_pack_chunks(x: torch.Tensor, payloads: torch.Tensor, world: int, 
     _require(payloads.shape[0] == world, "payloads must have one row per destination rank")
     shard = -(-n // world)
     _require(payloads.shape[1] >= payload_nbytes(shard, group_size), "payload rows are too small")
-    r_code, n_code, d_code = _side_tensors(x, residual, new_residual, restored, restored_dtype)
+    r_code, n_code, d_code, p_code = _side_tensors(x, residual, new_residual, restored, restored_dtype, prepared_out)
     args = (_ptr(x), x_code, _ptr(residual), r_code, n, world, group_size, _ptr(payloads), payloads.stride(0),
-            _ptr(new_residual), n_code, _ptr(restored), d_code)
+            _ptr(new_residual), n_code, _ptr(restored), d_code, _ptr(prepared_out), p_code)
     return BoundLaunch(lib.lbc_quant_pack_chunks, args + (access_code(access),), device, lib,
-                       (x, payloads, residual, new_residual, restored), kind="quant_pack_chunks")
+                       (x, payloads, residual, new_residual, restored, prepared_out), kind="quant_pack_chunks")
 
 
 # --------------------------------------------------------------------------- #
@@ -398,7 +409,8 @@ def bind_dequant_chunks(payloads: torch.Tensor, out: torch.Tensor, shard_numel: 
     _require(payloads.shape[1] >= payload_nbytes(shard_numel, group_size), "payload rows are too small")
     _require(out.numel() <= world * shard_numel, "output is larger than world * shard_numel")
     args = (_ptr(payloads), payloads.stride(0), world, shard_numel, out.numel(), group_size, _ptr(out), o_code)
-    return BoundLaunch(lib.lbc_dequant_chunks, args + (access_code(access),), out.device, lib, (payloads, out))
+    return BoundLaunch(lib.lbc_dequant_chunks, args + (access_code(access),), out.device, lib, (payloads, out),
+                       kind="dequant_chunks")
 
 
 def dequant_reduce_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out: torch.Tensor, *,
@@ -475,8 +487,8 @@ def bind_quant_chunks_and_reduce(quant: BoundLaunch, reduce: BoundLaunch) -> Bou
              "reduce must come from bind_dequant_reduce")
     _require(quant._device == reduce._device, "both launches must be on the same device")
     (x, x_code, residual, r_code, n, world, group_size, payloads, stride, new_residual, n_code, restored, _d_code,
-     access) = quant._args
-    _require(restored is None, "the shared launch does not write `restored`")
+     prepared_out, _p_code, access) = quant._args
+    _require(restored is None and prepared_out is None, "the shared launch does not write `restored` or `prepared_out`")
     code_ptrs, scale_ptrs, r_world, r_n, r_group, divisor, out, o_code, prepared, r_new_residual, _r_access = reduce._args
     _require(group_size == r_group, "both launches must use the same group size")
     args = (x, x_code, residual, r_code, n, world, group_size, payloads, stride, new_residual, n_code,
@@ -520,7 +532,59 @@ def bind_dequant_reduce_quant(payloads: Sequence[tuple[torch.Tensor, torch.Tenso
     args = (code_ptrs, scale_ptrs, world, n, group_size, float(divisor), DTYPE_CODES[mid_dtype], _ptr(out_codes),
             _ptr(out_scales))
     return BoundLaunch(lib.lbc_dequant_reduce_quant, args + (access_code(access),), device, lib,
-                       (tuple(payloads), out_codes, out_scales))
+                       (tuple(payloads), out_codes, out_scales), kind="dequant_reduce_quant")
+
+
+def bind_bucket_pipeline_step(quant: BoundLaunch | None = None, reduce: BoundLaunch | None = None,
+                              decode: BoundLaunch | None = None) -> BoundLaunch:
+    """One launch for up to three stages of a bucket stream (``lbc_bucket_pipeline_step``): ``quant`` from
+    :func:`bind_quant_pack_chunks` (bucket k, without ``restored`` / ``prepared_out``), ``reduce`` from
+    :func:`bind_dequant_reduce_quant` (bucket k-1) and ``decode`` from :func:`bind_dequant_chunks` (bucket k-2); any
+    may be ``None``.  The stages must not touch each other's outputs.  The access mode is that of the first stage
+    given.  Calling the result returns ``False`` when the combination has no shared grid (then call the stages
+    themselves); the results are bit-identical either way."""
+    from lowbit_comm_amd.hip.library import DequantChunksStage, QuantChunksStage, ReduceQuantStage
+
+    given = [stage for stage in (quant, reduce, decode) if stage is not None]
+    _require(len(given) > 0, "at least one stage must be given")
+    for stage, kind, maker in ((quant, "quant_pack_chunks", "bind_quant_pack_chunks"),
+                               (reduce, "dequant_reduce_quant", "bind_dequant_reduce_quant"),
+                               (decode, "dequant_chunks", "bind_dequant_chunks")):
+        _require(stage is None or (isinstance(stage, BoundLaunch) and stage._kind == kind),
+                 f"the {kind} stage must come from {maker}")
+    _require(all(stage._device == given[0]._device for stage in given), "all stages must be on the same device")
+    value = lambda p: None if p is None else (p.value if isinstance(p, ctypes.c_void_p) else p)  # noqa: E731
+    hold: list = []
+    group_size = None
+    q_ref = r_ref = d_ref = None
+    if quant is not None:
+        (x, x_code, residual, r_code, n, world, group_size, payloads, stride, new_residual, n_code, restored, _d_code,
+         prepared_out, _p_code, _access) = quant._args
+        _require(restored is None and prepared_out is None,
+                 "the shared launch does not write `restored` or `prepared_out`")
+        q_stage = QuantChunksStage(value(x), value(residual), value(payloads), value(new_residual), n, stride,
+                                   x_code, r_code, n_code, world)
+        hold.append(q_stage)
+        q_ref = ctypes.c_void_p(ctypes.addressof(q_stage))
+    if reduce is not None:
+        code_ptrs, scale_ptrs, r_world, r_n, r_group, divisor, mid_code, out_codes, out_scales, _r_access = reduce._args
+        _require(group_size in (None, r_group), "all stages must use the same group size")
+        group_size = r_group
+        r_stage = ReduceQuantStage(ctypes.addressof(code_ptrs), ctypes.addressof(scale_ptrs), value(out_codes),
+                                   value(out_scales), r_n, divisor, r_world, mid_code)
+        hold.extend((r_stage, code_ptrs, scale_ptrs))
+        r_ref = ctypes.c_void_p(ctypes.addressof(r_stage))
+    if decode is not None:
+        d_payloads, d_stride, d_world, d_shard, d_total, d_group, d_out, o_code, _d_access = decode._args
+        _require(group_size in (None, d_group), "all stages must use the same group size")
+        group_size = d_group
+        d_stage = DequantChunksStage(value(d_payloads), value(d_out), d_stride, d_shard, d_total, d_world, o_code)
+        hold.append(d_stage)
+        d_ref = ctypes.c_void_p(ctypes.addressof(d_stage))
+    lib = given[0]._lib
+    args = (q_ref, r_ref, d_ref, group_size, given[0]._args[-1])
+    return BoundLaunch(lib.lbc_bucket_pipeline_step, args, given[0]._device, lib, tuple(stage._keep for stage in given),
+                       kind="bucket_pipeline_step", hold=tuple(hold))
 
 
 def dequant_reduce_quant_into(payloads: Sequence[tuple[torch.Tensor, torch.Tensor]], out_codes: torch.Tensor,

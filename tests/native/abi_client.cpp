@@ -239,7 +239,7 @@ int main() {
         HIP_OK(hipMalloc(&d_scales[r], groups * sizeof(float)));
         HIP_OK(hipMemcpyAsync(d_x, x[r].data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
         LBC_OK_OR_FAIL(lbc_quant_pack(d_x, LBC_F32, nullptr, LBC_NONE, n, g, d_codes[r], d_scales[r], nullptr, LBC_NONE,
-                                      nullptr, LBC_NONE, LBC_ACCESS_AUTO, stream));
+                                      nullptr, LBC_NONE, nullptr, LBC_NONE, LBC_ACCESS_AUTO, stream));
         std::vector<int8_t> codes(padded);
         std::vector<float> scales(groups);
         HIP_OK(hipMemcpyAsync(codes.data(), d_codes[r], padded, hipMemcpyDeviceToHost, stream));
@@ -327,16 +327,18 @@ int main() {
     std::vector<float> ef_scales(groups), want_ef_scales(groups);
     lbo_ef_step_f32(x[0].data(), residual.data(), n, g, want_ef_codes.data(), want_ef_scales.data(), want_residual.data(),
                     want_restored.data());
-    float *d_residual = nullptr, *d_restored = nullptr, *d_prepared = nullptr;
+    float *d_residual = nullptr, *d_restored = nullptr, *d_prepared = nullptr, *d_prepared_out = nullptr;
     HIP_OK(hipMalloc(&d_residual, n * sizeof(float)));
     HIP_OK(hipMalloc(&d_restored, n * sizeof(float)));
     HIP_OK(hipMalloc(&d_prepared, n * sizeof(float)));
+    HIP_OK(hipMalloc(&d_prepared_out, n * sizeof(float)));
     HIP_OK(hipMemcpyAsync(d_x, x[0].data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
     HIP_OK(hipMemcpyAsync(d_residual, residual.data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
     HIP_OK(hipMemcpyAsync(d_prepared, prepared.data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
     LBC_OK_OR_FAIL(lbc_quant_pack(d_x, LBC_F32, d_residual, LBC_F32, n, g, d_send_codes, d_send_scales, d_residual, LBC_F32,
-                                  d_restored, LBC_F32, LBC_ACCESS_AUTO, stream));
-    std::vector<float> got_residual(n), got_restored(n);
+                                  d_restored, LBC_F32, d_prepared_out, LBC_F32, LBC_ACCESS_AUTO, stream));
+    std::vector<float> got_residual(n), got_restored(n), got_prepared(n);
+    HIP_OK(hipMemcpyAsync(got_prepared.data(), d_prepared_out, n * sizeof(float), hipMemcpyDeviceToHost, stream));
     HIP_OK(hipMemcpyAsync(ef_codes.data(), d_send_codes, padded, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipMemcpyAsync(ef_scales.data(), d_send_scales, groups * sizeof(float), hipMemcpyDeviceToHost, stream));
     HIP_OK(hipMemcpyAsync(got_residual.data(), d_residual, n * sizeof(float), hipMemcpyDeviceToHost, stream));
@@ -345,11 +347,12 @@ int main() {
     if (memcmp(ef_codes.data(), want_ef_codes.data(), padded) != 0 ||
         memcmp(ef_scales.data(), want_ef_scales.data(), groups * sizeof(float)) != 0 ||
         memcmp(got_residual.data(), want_residual.data(), n * sizeof(float)) != 0 ||
-        memcmp(got_restored.data(), want_restored.data(), n * sizeof(float)) != 0) {
+        memcmp(got_restored.data(), want_restored.data(), n * sizeof(float)) != 0 ||
+        memcmp(got_prepared.data(), prepared.data(), n * sizeof(float)) != 0) {
         printf("FAIL error-feedback step differs from the oracle\n");
         return 9;
     }
-    checks += 4;
+    checks += 5;
     LBC_OK_OR_FAIL(lbc_ef_update(d_prepared, LBC_F32, d_restored, LBC_F32, d_residual, LBC_F32, n, LBC_ACCESS_AUTO, stream));
     HIP_OK(hipMemcpyAsync(got_residual.data(), d_residual, n * sizeof(float), hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
@@ -366,7 +369,7 @@ int main() {
     HIP_OK(hipMalloc(&d_rows, world * stride));
     HIP_OK(hipMemsetAsync(d_rows, 0xEE, world * stride, stream));
     LBC_OK_OR_FAIL(lbc_quant_pack_chunks(d_x, LBC_F32, nullptr, LBC_NONE, n, world, g, d_rows, stride, nullptr, LBC_NONE, nullptr,
-                                         LBC_NONE, LBC_ACCESS_AUTO, stream));
+                                         LBC_NONE, nullptr, LBC_NONE, LBC_ACCESS_AUTO, stream));
     LBC_OK_OR_FAIL(lbc_dequant_chunks(d_rows, stride, world, shard, n, g, d_out, LBC_F32, LBC_ACCESS_AUTO, stream));
     std::vector<uint8_t> rows(world * stride);
     HIP_OK(hipMemcpyAsync(rows.data(), d_rows, world * stride, hipMemcpyDeviceToHost, stream));
@@ -435,14 +438,77 @@ int main() {
     }
     checks += 2;
 
+    // three stages of a bucket stream in one launch: chunked quantize of one bucket, reduce + requantize of the payloads
+    // that arrived for another, decode of a third one's gathered shard payloads
+    uint8_t *d_gathered = nullptr;
+    float *d_decoded = nullptr;
+    HIP_OK(hipMalloc(&d_gathered, world * even_stride));
+    HIP_OK(hipMalloc(&d_decoded, even * sizeof(float)));
+    HIP_OK(hipMemcpyAsync(d_gathered, d_rows, world * even_stride, hipMemcpyDeviceToDevice, stream));   // verified above
+    HIP_OK(hipMemsetAsync(d_rows, 0xEE, world * even_stride, stream));
+    HIP_OK(hipMemsetAsync(d_send_codes, 0xEE, padded, stream));
+    {
+        lbc_quant_chunks_stage quant_stage{};
+        quant_stage.x = d_x;
+        quant_stage.x_dtype = LBC_F32;
+        quant_stage.residual_dtype = quant_stage.new_residual_dtype = LBC_NONE;
+        quant_stage.numel = even;
+        quant_stage.world = world;
+        quant_stage.payloads = d_rows;
+        quant_stage.payload_stride = even_stride;
+        lbc_reduce_quant_stage reduce_stage{};
+        reduce_stage.codes = code_ptrs.data();
+        reduce_stage.scales = scale_ptrs.data();
+        reduce_stage.world = world;
+        reduce_stage.numel = reduce_n;
+        reduce_stage.divisor = static_cast<float>(world);
+        reduce_stage.mid_dtype = LBC_F32;
+        reduce_stage.out_codes = d_send_codes;
+        reduce_stage.out_scales = d_send_scales;
+        lbc_dequant_chunks_stage decode_stage{};
+        decode_stage.payloads = d_gathered;
+        decode_stage.payload_stride = even_stride;
+        decode_stage.world = world;
+        decode_stage.shard_numel = even_shard;
+        decode_stage.total_numel = even;
+        decode_stage.out = d_decoded;
+        decode_stage.out_dtype = LBC_F32;
+        LBC_OK_OR_FAIL(lbc_bucket_pipeline_step(&quant_stage, &reduce_stage, &decode_stage, g, LBC_ACCESS_AUTO, stream));
+    }
+    HIP_OK(hipMemcpyAsync(rows.data(), d_rows, world * even_stride, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(send_codes.data(), d_send_codes, reduce_n, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(send_scales.data(), d_send_scales, reduce_n / g * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(got.data(), d_decoded, even * sizeof(float), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    lbo_quantize_f32(want.data(), reduce_n, g, want_send_codes.data(), want_send_scales.data());   // want: the mean of reduce_n
+    for (int d = 0; d < world; ++d) {
+        if (memcmp(rows.data() + d * even_stride, chunk_codes[d].data(), even_shard) != 0 ||
+            memcmp(rows.data() + d * even_stride + even_shard, chunk_scales[d].data(), even_groups * sizeof(float)) != 0) {
+            printf("FAIL pipeline step: payload of chunk %d differs from the oracle\n", d);
+            return 13;
+        }
+        std::vector<float> decoded(even_shard);
+        lbo_dequantize_f32(chunk_codes[d].data(), chunk_scales[d].data(), even_shard, g, decoded.data());
+        if (memcmp(got.data() + d * even_shard, decoded.data(), even_shard * sizeof(float)) != 0) {
+            printf("FAIL pipeline step: decoded shard %d differs from the oracle\n", d);
+            return 13;
+        }
+    }
+    if (memcmp(send_codes.data(), want_send_codes.data(), reduce_n) != 0 ||
+        memcmp(send_scales.data(), want_send_scales.data(), reduce_n / g * sizeof(float)) != 0) {
+        printf("FAIL pipeline step: reduce + requantize differs from the oracle\n");
+        return 13;
+    }
+    checks += 3;
+
     // contract: a bad argument is refused with a message, an unsupported group size is "unsupported", not an error
     if (lbc_quant_pack(d_x, LBC_F32, nullptr, LBC_NONE, -1, g, d_codes[0], d_scales[0], nullptr, LBC_NONE, nullptr, LBC_NONE,
-                       LBC_ACCESS_AUTO, stream) != LBC_EINVAL || strstr(lbc_last_error(), "numel") == nullptr) {
+                       nullptr, LBC_NONE, LBC_ACCESS_AUTO, stream) != LBC_EINVAL || strstr(lbc_last_error(), "numel") == nullptr) {
         printf("FAIL negative numel was not refused\n");
         return 7;
     }
     if (lbc_quant_pack(d_x, LBC_F32, nullptr, LBC_NONE, n, 48, d_codes[0], d_scales[0], nullptr, LBC_NONE, nullptr, LBC_NONE,
-                       LBC_ACCESS_AUTO, stream) != LBC_UNSUPPORTED) {
+                       nullptr, LBC_NONE, LBC_ACCESS_AUTO, stream) != LBC_UNSUPPORTED) {
         printf("FAIL group size 48 should be unsupported\n");
         return 7;
     }

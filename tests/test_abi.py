@@ -33,18 +33,18 @@ def test_library_loads_on_the_cpu_and_exports_every_declared_symbol():
 def test_argument_validation_happens_before_any_device_work():
     lib = library.load_library()
     none = ctypes.c_void_p(None)
-    assert lib.lbc_quant_pack(none, 0, none, -1, -5, 64, none, none, none, -1, none, 0, 0, none) == -1
+    assert lib.lbc_quant_pack(none, 0, none, -1, -5, 64, none, none, none, -1, none, 0, none, -1, 0, none) == -1
     assert library.last_error(lib) == "numel must be >= 0"
-    assert lib.lbc_quant_pack(none, 7, none, -1, 64, 64, none, none, none, -1, none, 0, 0, none) == -1
+    assert lib.lbc_quant_pack(none, 7, none, -1, 64, 64, none, none, none, -1, none, 0, none, -1, 0, none) == -1
     assert "unsupported input dtype" in library.last_error(lib)
-    assert lib.lbc_quant_pack(none, 0, none, -1, 0, 64, none, none, none, -1, none, 0, 0, none) == 0      # empty: no-op
-    assert lib.lbc_quant_pack(none, 0, none, -1, 64, 48, none, none, none, -1, none, 0, 0, none) == 1     # unsupported group
+    assert lib.lbc_quant_pack(none, 0, none, -1, 0, 64, none, none, none, -1, none, 0, none, -1, 0, none) == 0      # empty: no-op
+    assert lib.lbc_quant_pack(none, 0, none, -1, 64, 48, none, none, none, -1, none, 0, none, -1, 0, none) == 1     # unsupported group
     assert lib.lbc_dequant_reduce(none, none, 0, 64, 64, 1.0, none, 0, none, none, 0, none) == -1
     assert library.last_error(lib) == "inputs must not be empty"
     assert lib.lbc_dequant_reduce(none, none, 9, 64, 64, 1.0, none, 0, none, none, 0, none) == 1          # > 8 payloads
     assert lib.lbc_dequant_reduce(none, none, 2, 64, 64, 0.0, none, 0, none, none, 0, none) == -1
     assert library.last_error(lib) == "divisor must be > 0"
-    assert lib.lbc_quant_pack_chunks(none, 0, none, -1, 640, 0, 64, none, 0, none, -1, none, 0, 0, none) == -1
+    assert lib.lbc_quant_pack_chunks(none, 0, none, -1, 640, 0, 64, none, 0, none, -1, none, 0, none, -1, 0, none) == -1
     assert library.last_error(lib) == "world must be > 0"
     assert lib.lbc_dequant(none, none, 64, 64, none, 0, 9, 0, none) == -1
     # ring / tree hops: (recv codes, recv scales, chunk, dtype, numel, g, op, divisor, send codes, send scales, access,
@@ -69,8 +69,8 @@ def test_argument_validation_happens_before_any_device_work():
     assert lib.lbc_wire_ring_step(none, none, 0, 0, 64, 1, 1, 1.0, none, 0, none) == 0
     assert lib.lbc_wire_ring_step(none, none, 0, 128, 64, 1, 1, -2.0, none, 0, none) == -1
     # the access mode is an argument of the call (0 auto, 1 cached, 2 stream); there is no process-wide setting
-    assert lib.lbc_quant_pack(none, 0, none, -1, 0, 64, none, none, none, -1, none, 0, 2, none) == 0
-    assert lib.lbc_quant_pack(none, 0, none, -1, 0, 64, none, none, none, -1, none, 0, 3, none) == -1
+    assert lib.lbc_quant_pack(none, 0, none, -1, 0, 64, none, none, none, -1, none, 0, none, -1, 2, none) == 0
+    assert lib.lbc_quant_pack(none, 0, none, -1, 0, 64, none, none, none, -1, none, 0, none, -1, 3, none) == -1
     assert library.last_error(lib) == "unknown access mode 3"
     assert lib.lbc_dequant(none, none, 0, 64, none, 0, 0, -1, none) == -1
     assert not hasattr(lib, "lbc_set_stream_min_bytes")

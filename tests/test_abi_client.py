@@ -22,12 +22,13 @@ def test_client_source_uses_only_the_header_and_the_hip_runtime():
 def test_client_runs_every_entry_point_bit_exact_against_the_c_oracles(hip_device):
     """Portable format: quantize, decode, fused reduce, ring step, the error-feedback step and the residual update, the
     bucket as chunks and the chunks decoded back, reduce + requantize, the shared launch of a quantize and a reduce,
-    and two contract checks (29).  The CUDA extension's byte format: quantize and decode for fp32 / bf16, interleaved /
+    the sum of bucket and residual as an output of the quantize, the three-stage pipeline step, and two contract
+    checks (33).  The CUDA extension's byte format: quantize and decode for fp32 / bf16, interleaved /
     appended scales, 8 / 4 bits; fused mean of four payloads; ring step; chunks; four general policies (29)."""
     done = subprocess.run([str(CLIENT)], capture_output=True, text=True, timeout=120)
     assert done.returncode == 0, (done.stdout, done.stderr[-2000:])
     assert done.stdout.strip().startswith("OK "), done.stdout
-    assert int(done.stdout.split()[1]) == 58
+    assert int(done.stdout.split()[1]) == 62
 
 
 @pytest.mark.gpu

@@ -687,6 +687,192 @@ def test_shared_launch_of_quantize_and_reduce_equals_the_two_launches_and_the_or
     assert_same_bits(got_out, want, "reduced shard against the oracle")
 
 
+@pytest.mark.parametrize("grad_dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("n", [64 * 8 * 640, 64 * 8 * 64 * 3 + 64 * 8])
+def test_shared_launch_with_a_16_bit_bucket_that_starts_a_residual_writes_an_fp32_residual(ops, hip_device, grad_dtype, n):
+    """A 16-bit bucket without a residual whose new residual is asked for: `restored` is rounded to fp32, so the new
+    residual is an fp32 tensor and the quantize half is the four-elements-per-lane instantiation - the shared launch
+    has to run that one, not the pure 16-bit one."""
+    world, reduce_n = 8, 64 * 640
+    grad = gradient_like(n, DTYPES[grad_dtype], 3300 + n, hip_device)
+    shard = -(-n // world)
+    stride = (ops.payload_nbytes(shard) + 255) // 256 * 256
+    rows = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+    guard = 4096
+    arena = torch.full((n + 2 * guard,), 7.0, dtype=torch.float32, device=hip_device)     # catches a write past either end
+    new_residual = arena[guard:guard + n]
+    peers = [ops.quant_pack(gradient_like(reduce_n, torch.float32, 3400 + r, hip_device)) for r in range(world)]
+    out = torch.empty(reduce_n, dtype=torch.float32, device=hip_device)
+    quant = ops.bind_quant_pack_chunks(grad, rows, world, new_residual=new_residual)
+    reduce = ops.bind_dequant_reduce(peers, out, divisor=float(world))
+    assert ops.bind_quant_chunks_and_reduce(quant, reduce)() is True
+    got_rows, got_out, got_residual = rows.clone(), out.clone(), new_residual.clone()
+    assert torch.equal(arena[:guard].cpu(), torch.full((guard,), 7.0)) and torch.equal(arena[guard + n:].cpu(), torch.full((guard,), 7.0))
+    rows.zero_(); out.zero_(); new_residual.zero_()
+    assert quant() and reduce()
+    assert torch.equal(got_rows, rows)
+    assert_same_bits(got_out, out.cpu(), "reduced shard")
+    assert_same_bits(got_residual, new_residual.cpu(), "new residual against the separate launch")
+    nbytes = ops.payload_nbytes(shard)
+    for d in range(world):
+        chunk = grad.cpu()[d * shard:(d + 1) * shard]
+        w_codes, w_scales, _w_restored, w_residual = codec_torch.ef_round_trip(chunk, None, 64, "fp32")
+        assert torch.equal(got_rows[d, :nbytes].cpu(), codec_torch.pack(w_codes, w_scales)), f"chunk {d}"
+        assert w_residual.dtype == torch.float32
+        assert_same_bits(got_residual[d * shard:(d + 1) * shard], w_residual, f"new residual of chunk {d} against the oracle")
+
+
+# --------------------------------------------------------------------------- #
+# the sum of bucket and residual as an output of the quantize
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("grad_dtype,res_dtype,restored_dtype", [
+    ("bf16", "fp32", "fp32"), ("bf16", "fp32", "bf16"), ("fp16", "fp32", "fp16"), ("fp32", "fp32", "fp32"),
+    ("bf16", "bf16", "bf16"), ("bf16", None, "bf16"), ("fp32", None, "fp32"), ("fp16", "fp16", "fp32"),
+])
+@pytest.mark.parametrize("n", [2048 * 5, 30_011])
+@pytest.mark.parametrize("with_feedback_outputs", [False, True])
+def test_quantize_also_writes_prepared(ops, hip_device, grad_dtype, res_dtype, restored_dtype, n, with_feedback_outputs):
+    """``prepared_out = bucket + residual`` in the torch promotion of their types - what
+    ``ErrorFeedbackState.compensate`` returns (ccdl_comm/quantization/error_feedback.py:27-36) - from the launch that
+    quantizes it; payload and the other outputs are those of the call without it."""
+    grad = gradient_like(n, DTYPES[grad_dtype], 1100 + n, hip_device)
+    residual = None if res_dtype is None else gradient_like(n, DTYPES[res_dtype], 1101, hip_device, sigma=1e-5,
+                                                             outliers=False)
+    p_dtype = grad.dtype if residual is None else ops.promote(grad.dtype, residual.dtype)
+    groups = ops.num_groups(n, 64)
+    codes = torch.empty(groups * 64, dtype=torch.int8, device=hip_device)
+    scales = torch.empty(groups, dtype=torch.float32, device=hip_device)
+    prepared = torch.full((n + 64,), 3.0, dtype=p_dtype, device=hip_device)
+    restored = new_residual = None
+    if with_feedback_outputs:
+        restored = torch.empty(n, dtype=DTYPES[restored_dtype], device=hip_device)
+        new_residual = torch.empty(n, dtype=ops.promote(p_dtype, DTYPES[restored_dtype]), device=hip_device)
+    assert ops.quant_pack_into(grad, codes, scales, residual=residual, new_residual=new_residual, restored=restored,
+                               restored_dtype=DTYPES[restored_dtype], prepared_out=prepared)
+    want_prepared = grad.cpu() if residual is None else grad.cpu() + residual.cpu()
+    assert want_prepared.dtype == p_dtype
+    assert_same_bits(prepared[:n], want_prepared, "prepared")
+    assert torch.equal(prepared[n:].cpu(), torch.full((64,), 3.0, dtype=p_dtype)), "written past the end"
+    w_codes, w_scales, w_restored, w_residual = codec_torch.ef_round_trip(
+        grad.cpu(), None if residual is None else residual.cpu(), 64, restored_dtype)
+    assert torch.equal(codes.cpu(), w_codes)
+    assert_same_bits(scales, w_scales, "scales")
+    if with_feedback_outputs:
+        assert_same_bits(restored, w_restored, "restored")
+        assert_same_bits(new_residual, w_residual, "residual")
+
+
+def test_quantize_chunks_also_write_prepared_and_refuse_a_wrong_type(ops, hip_device):
+    world, n = 8, 64 * 8 * 100 + 8 * 5
+    grad = gradient_like(n, torch.bfloat16, 1200, hip_device)
+    residual = gradient_like(n, torch.float32, 1201, hip_device, sigma=1e-5, outliers=False)
+    shard = -(-n // world)
+    rows = torch.zeros(world, (ops.payload_nbytes(shard) + 255) // 256 * 256, dtype=torch.uint8, device=hip_device)
+    plain = rows.clone()
+    prepared = torch.empty(n, dtype=torch.float32, device=hip_device)
+    assert ops.quant_pack_chunks_into(grad, rows, world, residual=residual, prepared_out=prepared)
+    assert ops.quant_pack_chunks_into(grad, plain, world, residual=residual)
+    assert torch.equal(rows, plain)
+    assert_same_bits(prepared, grad.cpu() + residual.cpu(), "prepared")
+    with pytest.raises(RuntimeError, match="prepared_out must have dtype"):
+        ops.quant_pack_chunks_into(grad, rows, world, residual=residual, prepared_out=prepared.to(torch.bfloat16))
+    with pytest.raises(RuntimeError, match="alias"):
+        ops.quant_pack_chunks_into(grad.float(), rows, world, residual=residual, prepared_out=residual)
+
+
+# --------------------------------------------------------------------------- #
+# three stages of a bucket stream in one launch
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("dtype,with_residual,track_residual", [
+    ("bf16", True, True), ("fp16", True, True), ("fp32", True, True), ("fp32", False, False), ("bf16", False, False),
+    ("fp16", False, False), ("bf16", False, True),
+])
+@pytest.mark.parametrize("world", [8, 4, 2])
+@pytest.mark.parametrize("stages", ["qrd", "qr", "qd", "rd", "q", "r", "d"])
+@pytest.mark.parametrize("n", [64 * 8 * 640, 64 * 8 * 64 * 3 + 64 * 8 * 5])
+def test_pipeline_step_equals_its_three_launches_and_the_oracle(ops, hip_device, dtype, with_residual, track_residual,
+                                                                world, stages, n):
+    """Quantize of bucket k, reduce + requantize for bucket k-1, decode of bucket k-2 in one grid: every output equal to
+    the separate launches' and to the oracle's."""
+    kind = DTYPES[dtype]
+    shard = -(-n // world)
+    nbytes = ops.payload_nbytes(shard)
+    stride = (nbytes + 255) // 256 * 256
+    grad = gradient_like(n, kind, 5100 + n, hip_device)
+    residual = gradient_like(n, torch.float32, 5101, hip_device, sigma=1e-5, outliers=False) if with_residual else None
+    new_residual = residual if with_residual else (torch.zeros(n, dtype=torch.float32, device=hip_device) if track_residual else None)
+    keep = None if residual is None else residual.clone()
+    send = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+    received = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+    for r in range(world):
+        ops.quant_pack_payload_into(gradient_like(shard, kind, 5200 + r, hip_device), received[r, :nbytes])
+    mine = torch.zeros(nbytes, dtype=torch.uint8, device=hip_device)
+    gathered = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+    for r in range(world):
+        ops.quant_pack_payload_into(gradient_like(shard, kind, 5300 + r, hip_device), gathered[r, :nbytes])
+    decoded = torch.zeros(n, dtype=kind, device=hip_device)
+    pairs = [ops.split_payload(received[r, :nbytes], shard) for r in range(world)]
+    quant = ops.bind_quant_pack_chunks(grad, send, world, residual=residual, new_residual=new_residual)
+    reduce = ops.bind_dequant_reduce_quant(pairs, *ops.split_payload(mine, shard), shard, divisor=float(world), mid_dtype=kind)
+    decode = ops.bind_dequant_chunks(gathered, decoded, shard)
+    step = ops.bind_bucket_pipeline_step(quant if "q" in stages else None, reduce if "r" in stages else None,
+                                         decode if "d" in stages else None)
+    assert step() is True
+    got = [t.clone() for t in (send, mine, decoded)] + [None if new_residual is None else new_residual.clone()]
+    for t in (send, mine, decoded):
+        t.zero_()
+    if residual is not None:
+        residual.copy_(keep)
+    elif new_residual is not None:
+        new_residual.zero_()
+    if "q" in stages:
+        assert quant()
+    if "r" in stages:
+        assert reduce()
+    if "d" in stages:
+        assert decode()
+    assert torch.equal(got[0], send), "payload rows"
+    assert torch.equal(got[1], mine), "requantized shard payload"
+    assert_same_bits(got[2], decoded.cpu(), "decoded bucket")
+    if new_residual is not None:
+        assert_same_bits(got[3], new_residual.cpu(), "residual")
+    if "q" in stages:
+        prepared = grad.cpu() if keep is None else grad.cpu() + keep.cpu()
+        for d in range(world):
+            chunk = prepared[d * shard:(d + 1) * shard]
+            if chunk.numel() < shard:
+                chunk = torch.cat([chunk, torch.zeros(shard - chunk.numel(), dtype=chunk.dtype)])
+            assert torch.equal(got[0][d, :nbytes].cpu(), codec_torch.pack(*codec_torch.quantize(chunk, 64))), f"chunk {d}"
+    if "r" in stages:
+        reduced = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in pairs], shard, 64, dtype, "mean")
+        assert torch.equal(got[1].cpu(), codec_torch.pack(*codec_torch.quantize(reduced, 64))), "reduce + requantize"
+    if "d" in stages:
+        for d in range(world):
+            codes, scales = ops.split_payload(gathered[d, :nbytes], shard)
+            want = codec_torch.dequantize(codes.cpu(), scales.cpu(), shard, 64, dtype)
+            stop = min(n, (d + 1) * shard)
+            assert_same_bits(got[2][d * shard:stop], want[:stop - d * shard], f"decoded shard {d}")
+
+
+def test_pipeline_step_without_a_shared_grid_says_so(ops, hip_device):
+    """Group 32, an odd payload count or operands that are not aligned have no shared grid: the bound step returns
+    False and the caller issues the stages themselves."""
+    world, n = 3, 64 * 3 * 50
+    shard = n // world
+    grad = gradient_like(n, torch.float32, 1, hip_device)
+    send = torch.zeros(world, ops.payload_nbytes(shard), dtype=torch.uint8, device=hip_device)
+    pairs = [ops.quant_pack(gradient_like(shard, torch.float32, 2 + r, hip_device)) for r in range(world)]
+    mine = torch.zeros(ops.payload_nbytes(shard), dtype=torch.uint8, device=hip_device)
+    quant = ops.bind_quant_pack_chunks(grad, send, world)
+    reduce = ops.bind_dequant_reduce_quant(pairs, *ops.split_payload(mine, shard), shard)
+    assert ops.bind_bucket_pipeline_step(quant, reduce)() is False          # three payloads
+    assert ops.bind_bucket_pipeline_step(quant, None, None)() is True       # one stage: its own kernel
+    with pytest.raises(RuntimeError, match="at least one stage"):
+        ops.bind_bucket_pipeline_step()
+    with pytest.raises(RuntimeError, match="must come from bind_dequant_reduce_quant"):
+        ops.bind_bucket_pipeline_step(quant, quant)
+
+
 def test_bucket_steps_dealt_to_two_streams_in_turn_equal_the_one_stream_schedule(ops, hip_device):
     """Consecutive buckets are independent: their launches (quantize of bucket k + reduce of bucket k-1) may alternate
     between two streams, each with its own send matrix and shard output, and must leave the same residuals, payloads
