@@ -271,12 +271,23 @@ def create_ddp_comm_hook(
     if effective in injected:
         transport = injected[effective]
 
+        # A transport that pipelines the stream of buckets (``transport.pipelined``) returns a future per bucket and
+        # holds the last stages of the newest buckets back until the next one arrives; the iteration's last bucket
+        # has no next one, so it is followed by a flush.
+        flush = getattr(transport, "flush", None) if getattr(transport, "pipelined", False) else None
+
         def process_bucket(bucket: Any) -> Any:
             tensor = bucket.buffer()
+            last = callable(flush) and callable(getattr(bucket, "is_last", None)) and bucket.is_last()
             if small(tensor):
+                if last:
+                    flush()
                 return uncompressed(clone(tensor), reduce)
-            return transport(tensor, config=config, op=reduce, async_op=False, dtype=resolve_dtype(dtype, tensor),
-                             extension_status=extension_status)
+            result = transport(tensor, config=config, op=reduce, async_op=False, dtype=resolve_dtype(dtype, tensor),
+                               extension_status=extension_status)
+            if last:
+                flush()
+            return result
 
     elif effective == "all_gather":
         if all_gather is None and not async_gather:

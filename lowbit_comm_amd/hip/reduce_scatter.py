@@ -18,6 +18,7 @@ one by an event, and a plan whose asynchronous exchange has not been waited for 
 """
 from __future__ import annotations
 
+import threading
 from collections import OrderedDict
 from collections.abc import Callable
 from typing import Any
@@ -66,20 +67,28 @@ class ReduceScatterPlan:
         # the callers' tensors alive (the key holds everything a binding depends on, and every step is handed the
         # live tensors), so it pins no memory beyond the plan's own buffers.
         self._bound: OrderedDict[Any, ops.BoundLaunch] = OrderedDict()
+        self._bound_lock = threading.Lock()   # DDP calls its hook from the autograd thread, a user may call from another
         self._last_stream: Any | None = None
         self._last_stream_handle: int | None = None
         self.exchange_in_flight: Any | None = None     # work object of an exchange that nobody has waited for yet
 
-    _BOUND_LAUNCHES = 256
+    # Every bucket of one shape shares the plan, and every bucket has its own addresses: a transformer's stream of
+    # 25 MiB buckets has hundreds of them (613 for an 8 B-parameter model), each with up to three stages.  A cache
+    # smaller than one pass over them would miss on every bucket.
+    _BOUND_LAUNCHES = 4096
 
     def _remember(self, key: Any, make: Callable[[], ops.BoundLaunch]) -> ops.BoundLaunch:
-        bound = self._bound.get(key)
-        if bound is None:
-            bound = self._bound[key] = make().forget_tensors()
+        with self._bound_lock:
+            bound = self._bound.get(key)
+            if bound is not None:
+                self._bound.move_to_end(key)
+                return bound
+        made = make().forget_tensors()           # binding validates tensors: outside the lock
+        with self._bound_lock:
+            bound = self._bound.setdefault(key, made)
+            self._bound.move_to_end(key)
             while len(self._bound) > self._BOUND_LAUNCHES:
                 self._bound.popitem(last=False)
-        else:
-            self._bound.move_to_end(key)
         return bound
 
     def _order_after_previous_use(self) -> None:
@@ -114,22 +123,28 @@ class ReduceScatterPlan:
 
         With ``new_residual`` the same launch also stores what quantization dropped,
         ``(tensor + residual) - decode(payload)``; it may be the ``residual`` tensor itself."""
+        bound = self.bound_quantize(tensor, residual=residual, new_residual=new_residual)
+        self._order_after_previous_use()
+        if self.numel and not bound():
+            raise ValueError(f"no HIP quantize kernel for dtype {tensor.dtype} with this residual")
+        return self.send
+
+    def bound_quantize(self, tensor: torch.Tensor, *, residual: torch.Tensor | None = None,
+                       new_residual: torch.Tensor | None = None) -> ops.BoundLaunch:
+        """The launch of :meth:`quantize_chunks`, bound and remembered but not issued (a caller that merges the stages of
+        several buckets into one launch takes it from here)."""
         flat = tensor.reshape(-1)
         if flat.numel() != self.numel or flat.dtype != self.dtype:
             raise ValueError("tensor does not match the planned bucket")
         if self.exchange_in_flight is not None:
             raise RuntimeError("this plan's send and receive buffers belong to an exchange that has not been waited for: "
                                "wait for the previous bucket's work first, or give every bucket in flight its own plan")
-        self._order_after_previous_use()
         key = ("q", flat.data_ptr(), None if residual is None else (residual.data_ptr(), residual.dtype, residual.numel()),
                None if new_residual is None else (new_residual.data_ptr(), new_residual.dtype, new_residual.numel()))
-        bound = self._remember(key, lambda: ops.bind_quant_pack_chunks(
+        return self._remember(key, lambda: ops.bind_quant_pack_chunks(
             flat, self.send, self.world_size, group_size=self.config.group_size,
             residual=None if residual is None else residual.reshape(-1),
             new_residual=None if new_residual is None else new_residual.reshape(-1)))
-        if self.numel and not bound():
-            raise ValueError(f"no HIP quantize kernel for dtype {flat.dtype} with this residual")
-        return self.send
 
     def reduce_received(self, received: torch.Tensor | None = None, *, op: str = "sum",
                         out: torch.Tensor | None = None) -> ReducedShard:
@@ -143,20 +158,35 @@ class ReduceScatterPlan:
         self._order_after_previous_use()
         if shard:
             if fused:
-                bound = self._remember(("r", rows.data_ptr(), rows.numel(), target.data_ptr(), target.dtype, target.numel(), op), lambda: ops.bind_dequant_reduce(
-                    self._pairs(rows), target, numel=shard, group_size=self.config.group_size,
-                    divisor=float(self.world_size) if op == "mean" else 1.0))
-                fused = bool(bound())
+                fused = bool(self.bound_reduce(rows, op=op, out=target)())
             if not fused:
                 for r, (codes, scales) in enumerate(self._pairs(rows)):
                     ops.dequant_into(codes, scales, target, numel=shard, group_size=self.config.group_size,
                                      reduce_op="none" if r == 0 else "sum")
                 if op == "mean":
                     ops.true_divide_(target, self.world_size)
+        return self.reduced_shard(target, op=op, fused=fused, caller_owned=out is not None)
+
+    def bound_reduce(self, received: torch.Tensor | None = None, *, op: str = "sum",
+                     out: torch.Tensor | None = None) -> ops.BoundLaunch:
+        """The fused launch of :meth:`reduce_received` (at most 8 ranks), bound and remembered but not issued."""
+        if op not in ("sum", "mean"):
+            raise ValueError(f"unsupported reduce-scatter mode: {op}")
+        rows = self.received if received is None else received
+        target = self.shard if out is None else out
+        shard = self.chunks.shard_numel
+        return self._remember(
+            ("r", rows.data_ptr(), rows.numel(), target.data_ptr(), target.dtype, target.numel(), op),
+            lambda: ops.bind_dequant_reduce(self._pairs(rows), target, numel=shard, group_size=self.config.group_size,
+                                            divisor=float(self.world_size) if op == "mean" else 1.0))
+
+    def reduced_shard(self, target: torch.Tensor, *, op: str, fused: bool = True, caller_owned: bool = False) -> ReducedShard:
+        """The :class:`ReducedShard` record for this rank's shard held in ``target``."""
+        shard = self.chunks.shard_numel
         metadata = {
             "compression_bit": self.config.bit, "group_size": self.config.group_size, "workspace_output": True,
             "workspace_shape": (shard,), "quantized_workspace_output": True, "received_workspace_output": True,
-            "workspace_cache": True, "output_ownership": "plan" if out is None else "caller",
+            "workspace_cache": True, "output_ownership": "caller" if caller_owned else "plan",
             "fused_dequant_reduce": fused, "chunk_plan_precompiled": True,
             "received_payload_numel": self.world_size * self.payload_bytes,
         }
@@ -199,6 +229,17 @@ class ReduceScatterPlan:
             self.reduce_received(rows, op=op)
             return self.requantize_shard()
         self._order_after_previous_use()
+        if not self.bound_reduce_requantize(rows, op=op)():
+            raise ValueError(f"no HIP reduce-requantize kernel for dtype {self.reduced_dtype}")
+        return row
+
+    def bound_reduce_requantize(self, received: torch.Tensor | None = None, *, op: str = "sum") -> ops.BoundLaunch:
+        """The launch of :meth:`reduce_and_requantize` (at most 8 ranks), bound and remembered but not issued."""
+        if op not in ("sum", "mean"):
+            raise ValueError(f"unsupported reduce-scatter mode: {op}")
+        rows = self.received if received is None else received
+        row = self.payload(self.gathered, self.rank)
+        shard = self.chunks.shard_numel
 
         def make() -> ops.BoundLaunch:
             codes, scales = ops.split_payload(row, shard, self.config.group_size)
@@ -207,21 +248,27 @@ class ReduceScatterPlan:
                                                  divisor=float(self.world_size) if op == "mean" else 1.0,
                                                  mid_dtype=self.reduced_dtype)
 
-        if not self._remember(("rq", rows.data_ptr(), rows.numel(), op), make)():
-            raise ValueError(f"no HIP reduce-requantize kernel for dtype {self.reduced_dtype}")
-        return row
+        return self._remember(("rq", rows.data_ptr(), rows.numel(), op), make)
 
     def decode_gathered(self, gathered: torch.Tensor | None = None, *, out: torch.Tensor | None = None) -> torch.Tensor:
         """Decode the ``W`` gathered shard payloads into one flat tensor of the bucket's size (one launch)."""
-        rows = self.gathered if gathered is None else gathered
         target = out if out is not None else torch.empty(self.numel, dtype=self.reduced_dtype, device=self.device)
-        make = lambda: ops.bind_dequant_chunks(rows, target.reshape(-1), self.chunks.shard_numel,  # noqa: E731
-                                               group_size=self.config.group_size)
+        bound = self.bound_decode(target, gathered, remember=out is not None)
         self._order_after_previous_use()
-        bound = self._remember(("d", rows.data_ptr(), rows.numel(), target.data_ptr(), target.dtype, target.numel()), make) if out is not None else make()
         if self.numel and not bound():
             raise ValueError(f"no HIP decode kernel for dtype {target.dtype}")
         return target.reshape(self.shape)
+
+    def bound_decode(self, target: torch.Tensor, gathered: torch.Tensor | None = None, *,
+                     remember: bool = True) -> ops.BoundLaunch:
+        """The launch of :meth:`decode_gathered` into ``target``, bound (and remembered, for a tensor that will come
+        back) but not issued."""
+        rows = self.gathered if gathered is None else gathered
+        make = lambda: ops.bind_dequant_chunks(rows, target.reshape(-1), self.chunks.shard_numel,  # noqa: E731
+                                               group_size=self.config.group_size)
+        if not remember:
+            return make()
+        return self._remember(("d", rows.data_ptr(), rows.numel(), target.data_ptr(), target.dtype, target.numel()), make)
 
 
 def compressed_reduce_scatter_shard(tensor: torch.Tensor, *, config: CompressionConfig, world_size: int, rank: int,
@@ -230,7 +277,8 @@ def compressed_reduce_scatter_shard(tensor: torch.Tensor, *, config: Compression
                                     future_factory: Callable[[], Any] | None = None,
                                     completion_manager: Any | None = None,
                                     update_feedback: Callable[[ReducedShard], None] | None = None,
-                                    advance_policy: Callable[[], None] | None = None) -> Any:
+                                    advance_policy: Callable[[], None] | None = None, pipeline: Any | None = None,
+                                    out: torch.Tensor | None = None) -> Any:
     """Quantize per-destination chunks, exchange, reduce: returns this rank's :class:`ReducedShard`.
 
     ``all_to_all(received_rows, send_rows)`` must fill row ``r`` of ``received_rows`` with rank ``r``'s
@@ -241,14 +289,27 @@ def compressed_reduce_scatter_shard(tensor: torch.Tensor, *, config: Compression
     :class:`~lowbit_comm_amd.communication.AsyncShardPipeline` that reduces the shard when the exchange is over
     and completes a future (``future_factory``, default ``torch.futures.Future``) with it
     (``ccdl_comm/communication/reduce_scatter_transport.py:286-333``).
+
+    ``pipeline`` (with ``async_op``): a :class:`~lowbit_comm_amd.hip.bucket_pipeline.BucketPipeline` built without an
+    all-gather, shared by the buckets of a stream.  The bucket's quantize then shares one launch with the reduce of the
+    bucket handed over before it, and its own reduce goes out with the next bucket (or when the returned pipeline
+    object is waited for, or at ``pipeline.flush()``); ``all_to_all``, ``world_size`` and ``rank`` are the pipeline's.
+    ``out``: where this rank's shard is to be written (default: the plan's shard buffer, or a fresh tensor under a
+    pipeline).
     """
+    if pipeline is not None:
+        if not async_op:
+            raise ValueError("a bucket pipeline completes its buckets later: it needs async_op=True")
+        return _shard_through_pipeline(tensor, config=config, op=op, pipeline=pipeline, out=out,
+                                       future_factory=future_factory, completion_manager=completion_manager,
+                                       update_feedback=update_feedback, advance_policy=advance_policy)
     if plan is None:
         plan = ReduceScatterPlan(tensor.numel(), tensor.dtype, world_size=world_size, rank=rank, config=config,
                                  device=tensor.device, shape=tuple(tensor.shape))
     send = plan.quantize_chunks(tensor)
     if not async_op:
         all_to_all(plan.received, send)
-        return plan.reduce_received(op=op)
+        return plan.reduce_received(op=op, out=out)
     from lowbit_comm_amd.communication.async_shard_pipeline import AsyncShardPipeline
 
     exchange = all_to_all(plan.received, send)
@@ -259,7 +320,7 @@ def compressed_reduce_scatter_shard(tensor: torch.Tensor, *, config: Compression
 
     def reduce_shard(_received: Any) -> ReducedShard:   # runs once the exchange has been waited for
         plan.exchange_in_flight = None
-        return plan.reduce_received(op=op)
+        return plan.reduce_received(op=op, out=out)
 
     def release_plan(_done: Any) -> None:               # also when the exchange failed and the reduce never ran
         if plan.exchange_in_flight is exchange:
@@ -272,6 +333,39 @@ def compressed_reduce_scatter_shard(tensor: torch.Tensor, *, config: Compression
                               update_feedback=update_feedback or (lambda _shard: None),
                               advance_policy=advance_policy or (lambda: None),
                               completion_manager=completion_manager, resources=(tensor, plan, send)).run()
+
+
+class _ReduceEnqueued:
+    """The 'exchange' an :class:`AsyncShardPipeline` sees for a bucket that went through a :class:`BucketPipeline`: it
+    is over when the bucket's reduce has been enqueued, and what it delivers is the reduced shard itself."""
+
+    def __init__(self, enqueued: Any) -> None:
+        self._enqueued = enqueued
+
+    def get_future(self) -> Any:
+        return self._enqueued
+
+    def wait(self) -> Any:
+        return self._enqueued.wait()
+
+
+def _shard_through_pipeline(tensor: torch.Tensor, *, config: CompressionConfig, op: str, pipeline: Any,
+                            out: torch.Tensor | None, future_factory: Callable[[], Any] | None,
+                            completion_manager: Any | None, update_feedback: Callable[[ReducedShard], None] | None,
+                            advance_policy: Callable[[], None] | None) -> Any:
+    from lowbit_comm_amd.communication.async_shard_pipeline import AsyncShardPipeline
+
+    if pipeline.all_gather is not None:
+        raise ValueError("the shard of a reduce-scatter comes from a pipeline built without all_gather")
+    enqueued = pipeline.submit(tensor, config=config, op=op, out=out)
+    # the outer future flushes the pipeline when somebody waits for it: the reduce of the stream's last bucket has no
+    # later bucket to ride with
+    outer = future_factory() if future_factory is not None else pipeline.make_future()
+    return AsyncShardPipeline(communication_work=_ReduceEnqueued(enqueued), future=outer,
+                              reduce_shard=lambda shard: shard,
+                              update_feedback=update_feedback or (lambda _shard: None),
+                              advance_policy=advance_policy or (lambda: None),
+                              completion_manager=completion_manager, resources=(tensor, pipeline)).run()
 
 
 def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: CompressionConfig, world_size: int,
@@ -346,7 +440,8 @@ def make_reduce_scatter_transport(*, world_size: int, rank: int,
                                   all_to_all: Callable[[torch.Tensor, torch.Tensor], None],
                                   all_gather: Callable[[torch.Tensor, torch.Tensor], None],
                                   max_plans: int = 64, manager: Any | None = None,
-                                  inplace: bool = True, error_feedback: bool = False) -> Callable[..., Any]:
+                                  inplace: bool = True, error_feedback: bool = False, pipelined: bool = False,
+                                  lanes: int = 1, future_factory: Callable[[], Any] | None = None) -> Callable[..., Any]:
     """The callable ``create_ddp_comm_hook(reduce_scatter_all_gather=...)`` expects, over pre-bound plans.
 
     ``transport(tensor, *, config, op, async_op=False, dtype=None, extension_status=None)`` runs the compressed
@@ -359,8 +454,18 @@ def make_reduce_scatter_transport(*, world_size: int, rank: int,
     quantize launch adds before encoding and refreshes with what the encoding dropped, in the same launch - the
     local error feedback of ``DDPBucketProcessor`` (``ccdl_comm/communication/ddp.py:69-97``); ``transport.residuals``
     exposes them, ``transport.reset()`` drops them.  Counterpart of ``compressed_reduce_scatter_all_gather``
-    (``ccdl_comm/communication/reduce_scatter_transport.py:186-377``) with the exchanges injected."""
-    from collections import OrderedDict
+    (``ccdl_comm/communication/reduce_scatter_transport.py:186-377``) with the exchanges injected.
+
+    ``pipelined``: the buckets go through a :class:`~lowbit_comm_amd.hip.bucket_pipeline.BucketPipeline` - one launch
+    per bucket carries the quantize of that bucket, the reduce + requantize of the one before and the decode of the
+    one before that; the transport then returns a future per bucket, ``transport.flush()`` issues what the last two
+    buckets still wait for, and ``transport.pipelined`` is true (the comm hook flushes after the iteration's last
+    bucket).  ``lanes`` deals the buckets to that many streams in turn.  More than eight ranks, and ``async_op``, take
+    the unpipelined plan."""
+    if pipelined and world_size <= ops.MAX_PAYLOADS:
+        return _pipelined_transport(world_size=world_size, rank=rank, all_to_all=all_to_all, all_gather=all_gather,
+                                    max_plans=max_plans, manager=manager, inplace=inplace, error_feedback=error_feedback,
+                                    lanes=lanes, future_factory=future_factory)
 
     plans: OrderedDict = OrderedDict()
     residuals: dict = {}
@@ -406,4 +511,40 @@ def make_reduce_scatter_transport(*, world_size: int, rank: int,
     transport.plans = plans
     transport.residuals = residuals
     transport.reset = residuals.clear
+    transport.pipelined = False
+    transport.flush = lambda: None
+    return transport
+
+
+def _pipelined_transport(*, world_size: int, rank: int, all_to_all: Callable[..., Any], all_gather: Callable[..., Any],
+                         max_plans: int, manager: Any | None, inplace: bool, error_feedback: bool, lanes: int,
+                         future_factory: Callable[[], Any] | None) -> Callable[..., Any]:
+    from lowbit_comm_amd.hip.bucket_pipeline import BucketPipeline
+
+    pipeline = BucketPipeline(world_size=world_size, rank=rank, all_to_all=all_to_all, all_gather=all_gather,
+                              error_feedback=error_feedback, inplace=inplace, lanes=lanes, max_plans=max_plans,
+                              future_factory=future_factory)
+    unpipelined = make_reduce_scatter_transport(world_size=world_size, rank=rank, all_to_all=all_to_all,
+                                                all_gather=all_gather, max_plans=max_plans, manager=manager,
+                                                inplace=inplace, error_feedback=False)
+
+    def transport(tensor: torch.Tensor, *, config: CompressionConfig, op: str = "sum", async_op: bool = False,
+                  dtype: str | None = None, extension_status: Any | None = None) -> Any:
+        del extension_status                      # the plans call the C ABI directly
+        if dtype is not None and torch_dtype(dtype) != tensor.dtype:
+            raise ValueError(f"the reduce-scatter plan reduces in the bucket's dtype; got dtype={dtype!r} for {tensor.dtype}")
+        if async_op:
+            if error_feedback:
+                raise ValueError("the pipelined transport keeps the residuals; async_op is served by the unpipelined plan, "
+                                 "which would not see them")
+            pipeline.flush()
+            return unpipelined(tensor, config=config, op=op, async_op=True)
+        return pipeline.submit(tensor, config=config, op=op)
+
+    transport.pipeline = pipeline
+    transport.plans = pipeline._plans
+    transport.residuals = pipeline.residuals
+    transport.reset = pipeline.reset
+    transport.pipelined = True
+    transport.flush = pipeline.flush
     return transport
