@@ -946,6 +946,40 @@ def main() -> int:
             host, wall = host_and_wall(lambda i: hook(None, buckets[i % 4]), 60)
             host_row(f"hook, reduce_scatter strategy over pre-bound plans, 25 MiB bf16 bucket, W=8, error feedback {feedback}",
                      host, wall)
+        # the same strategy over the pipelined transport: one launch per bucket carries the quantize of bucket k, the
+        # reduce + requantize of bucket k-1 and the decode of bucket k-2; the hook flushes after the last bucket
+        class StreamBucket(Bucket):
+            def __init__(self, tensor, index, last):
+                super().__init__(tensor, index)
+                self._last = last
+
+            def is_last(self):
+                return self._last
+
+        stream_count = 16
+        stream_buckets = [StreamBucket(gen(SEED + 7500 + i, n, 1e-3, torch.bfloat16), i, i == stream_count - 1)
+                          for i in range(stream_count)]
+        for feedback in (False, True):
+            for lane_count in (1, 2):
+                filled = set()
+                transport = make_reduce_scatter_transport(world_size=world, rank=0, all_to_all=all_to_all,
+                                                          all_gather=all_gather, error_feedback=feedback, pipelined=True,
+                                                          lanes=lane_count, future_factory=Slot)
+                hook = create_ddp_comm_hook(CompressionConfig(error_feedback=False), strategy="reduce_scatter",
+                                            reduce="mean", reduce_scatter_all_gather=transport, future_factory=Slot)
+
+                def one_iteration(_i=0):
+                    for bucket in stream_buckets:
+                        hook(None, bucket)
+
+                host, wall = host_and_wall(one_iteration, 12)
+                stats = transport.pipeline.stats
+                host_row(f"hook, reduce_scatter strategy over the pipelined transport ({lane_count} stream"
+                         f"{'s' if lane_count > 1 else ''}), stream of {stream_count} 25 MiB bf16 buckets, W=8, error feedback "
+                         f"{feedback}, per bucket", host / stream_count, wall / stream_count,
+                         merged_launches_per_bucket=stats["merged_launches"] / stats["buckets"],
+                         separate_launches_per_bucket=stats["separate_launches"] / stats["buckets"])
+        del stream_buckets
         # one pre-bound launch
         x = gen(SEED + 7100, n, 1e-3, torch.bfloat16)
         payload = torch.empty(ops.payload_nbytes(n, G), dtype=torch.uint8, device=dev)

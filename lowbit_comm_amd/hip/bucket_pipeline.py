@@ -70,13 +70,15 @@ def _wait_for(work: Any) -> None:
 class _Lane:
     """The buckets of one stream: at most one awaiting its reduce and one awaiting its decode."""
 
-    __slots__ = ("stream", "handle", "reduce_next", "decode_next")
+    __slots__ = ("stream", "handle", "reduce_next", "decode_next", "ready", "recorded")
 
     def __init__(self, stream: Any | None) -> None:
         self.stream = stream
         self.handle = None if stream is None else stream.cuda_stream
         self.reduce_next: _Bucket | None = None
         self.decode_next: _Bucket | None = None
+        self.ready = None if stream is None else torch.cuda.Event()    # "the caller's stream has got this far", reused
+        self.recorded: set = set()          # storages the caching allocator has been told this lane uses
 
 
 class BucketPipeline:
@@ -251,8 +253,7 @@ class BucketPipeline:
             arriving.exchange = self.all_to_all(arriving.plan.received, arriving.plan.send)
         if reducing is not None:
             if full:
-                plan = reducing.plan
-                reducing.gather = self.all_gather(plan.gathered, plan.payload(plan.gathered, plan.rank))
+                reducing.gather = self.all_gather(reducing.plan.gathered, reducing.plan.my_row)
             else:
                 self._complete(reducing, reducing.plan.reduced_shard(reducing.out, op=reducing.op, caller_owned=True))
         if decoding is not None:
@@ -309,11 +310,20 @@ class BucketPipeline:
                 self._advance(lane, bucket, residual)
             else:
                 current = torch.cuda.current_stream(tensor.device)
-                lane.stream.wait_stream(current)              # the bucket's gradients are ready on the caller's stream
-                with torch.cuda.stream(lane.stream):          # the exchanges and the future see the lane as current
+                lane.ready.record(current)                    # the bucket's gradients are ready on the caller's stream
+                lane.stream.wait_event(lane.ready)
+                torch.cuda.set_stream(lane.stream)            # the exchanges and the future see the lane as current
+                try:
                     self._advance(lane, bucket, residual)
+                finally:
+                    torch.cuda.set_stream(current)
                 for held in (tensor, out) + (() if residual is None else (residual,)):
-                    held.record_stream(lane.stream)
+                    seen = (held.data_ptr(), held.numel())
+                    if seen not in lane.recorded:             # a DDP bucket comes back every iteration: told once
+                        if len(lane.recorded) > 65536:
+                            lane.recorded.clear()
+                        lane.recorded.add(seen)
+                        held.record_stream(lane.stream)
             return future
 
     def flush(self) -> None:
@@ -330,14 +340,18 @@ class BucketPipeline:
             self._next_lane = 0
             self.stats["flushes"] += 1
             for lane in lanes:
-                while lane.reduce_next is not None or lane.decode_next is not None:
-                    if lane.stream is None:
+                if lane.stream is None:
+                    while lane.reduce_next is not None or lane.decode_next is not None:
                         self._advance(lane, None, None)
-                    else:
-                        with torch.cuda.stream(lane.stream):
-                            self._advance(lane, None, None)
-                if lane.stream is not None:
-                    torch.cuda.current_stream(lane.stream.device).wait_stream(lane.stream)
+                    continue
+                current = torch.cuda.current_stream(lane.stream.device)
+                torch.cuda.set_stream(lane.stream)
+                try:
+                    while lane.reduce_next is not None or lane.decode_next is not None:
+                        self._advance(lane, None, None)
+                finally:
+                    torch.cuda.set_stream(current)
+                current.wait_stream(lane.stream)
 
 
 class _FlushingFuture(torch.futures.Future):

@@ -62,6 +62,7 @@ class ReduceScatterPlan:
         self.received = torch.empty(rows, dtype=torch.uint8, device=self.device)   # every rank's chunk for me
         self.gathered = torch.empty(rows, dtype=torch.uint8, device=self.device)   # every rank's requantized shard
         self.shard = torch.empty(shard, dtype=self.reduced_dtype, device=self.device)
+        self.my_row = self.gathered[rank, :self.payload_bytes]      # where this rank's requantized shard payload goes
         # Launches bound to the tensor addresses seen so far, least recently used dropped first.  Many buckets of one
         # shape share a plan (the layers of a transformer), so the cache is sized for them; its entries do not keep
         # the callers' tensors alive (the key holds everything a binding depends on, and every step is handed the
@@ -238,11 +239,10 @@ class ReduceScatterPlan:
         if op not in ("sum", "mean"):
             raise ValueError(f"unsupported reduce-scatter mode: {op}")
         rows = self.received if received is None else received
-        row = self.payload(self.gathered, self.rank)
         shard = self.chunks.shard_numel
 
         def make() -> ops.BoundLaunch:
-            codes, scales = ops.split_payload(row, shard, self.config.group_size)
+            codes, scales = ops.split_payload(self.my_row, shard, self.config.group_size)
             return ops.bind_dequant_reduce_quant(self._pairs(rows), codes, scales, shard,
                                                  group_size=self.config.group_size,
                                                  divisor=float(self.world_size) if op == "mean" else 1.0,

@@ -40,6 +40,7 @@ class FakePlan:
         self.send = ("send", self.tag)
         self.received = ("received", self.tag)
         self.gathered = ("gathered", self.tag)
+        self.my_row = ("row", self.gathered, rank)
         self.log = log
         self.chunks = type("Chunks", (), {"shard_numel": -(-numel // world_size)})()
         self._launches = {}

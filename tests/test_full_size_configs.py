@@ -264,3 +264,96 @@ def test_config5_llama_3_8b_shaped_stream_through_the_workspace_pool(ops, hip_de
     for index in sample:
         assert torch.equal(got_shards[index].view(torch.int32), want_shards[index].view(torch.int32)), f"shard of bucket {index}"
     assert pool.stats.misses == misses
+
+
+def test_config5_stream_through_the_comm_hook_over_the_pipelined_transport(ops, hip_device):
+    """The 613-bucket Llama-3-8B-shaped bf16 stream through ``create_ddp_comm_hook(strategy="reduce_scatter")`` over the
+    pipelined reduce-scatter transport with local error feedback, W=8, two iterations: every bucket and every residual
+    bit-identical to the hook over the unpipelined transport, buckets 0 / 306 / 612 bit-identical to the CPU oracle,
+    and one launch per bucket on the device (612 shared launches while the stream arrives + 1 at the flush).  The
+    exchanges are stand-ins on the one GPU (this rank's own chunk payloads come back from the all-to-all, its own
+    requantized shard fills every row of the all-gather)."""
+    from torch.profiler import ProfilerActivity, profile
+
+    from lowbit_comm_amd import CompressionConfig
+    from lowbit_comm_amd.communication.ddp_hook import create_ddp_comm_hook
+    from lowbit_comm_amd.hip.reduce_scatter import make_reduce_scatter_transport
+
+    dev, world = hip_device, 8
+    total, bucket_numel = 8_030_261_248, 13_107_200
+    bounds = [(a, min(a + bucket_numel, total)) for a in range(0, total, bucket_numel)]
+    assert len(bounds) == 613
+    sample = (0, 306, 612)
+
+    class Bucket:
+        def __init__(self, tensor, index):
+            self._tensor, self._index = tensor, index
+
+        def buffer(self):
+            return self._tensor
+
+        def index(self):
+            return self._index
+
+        def is_last(self):
+            return self._index == len(bounds) - 1
+
+    def all_to_all(received, send):
+        received.copy_(send)
+
+    def all_gather(gathered, mine):
+        gathered[1:, :mine.numel()] = mine
+
+    common = dict(world_size=world, rank=0, all_to_all=all_to_all, all_gather=all_gather, error_feedback=True)
+    piped = make_reduce_scatter_transport(pipelined=True, **common)
+    plain = make_reduce_scatter_transport(**common)
+    cfg = CompressionConfig(bit=8, group_size=G)
+    hooks = [create_ddp_comm_hook(cfg, strategy="reduce_scatter", reduce="mean", reduce_scatter_all_gather=t)
+             for t in (piped, plain)]
+    mine = torch.empty(total, dtype=torch.bfloat16, device=dev)
+    theirs = torch.empty(total, dtype=torch.bfloat16, device=dev)
+    cpu_residual = {index: None for index in sample}
+    for step in range(2):
+        inputs = {}
+        for index, (a, b) in enumerate(bounds):
+            mine[a:b] = gen(SEED + 5 + index + 10_000 * step, b - a, 1e-3, dev, torch.bfloat16)
+            if index in sample:
+                inputs[index] = mine[a:b].cpu()
+        theirs.copy_(mine)
+        torch.cuda.synchronize()
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            futures = [hooks[0](None, Bucket(mine[a:b], index)) for index, (a, b) in enumerate(bounds)]
+            torch.cuda.synchronize()
+        assert all(f.done() for f in futures)                              # the hook flushed after bucket 612
+        names = [e.name for e in prof.events() if e.device_type == torch.autograd.DeviceType.CUDA and "lbc" in e.name]
+        assert sum("bucket_pipeline_step_kernel" in name for name in names) == 613
+        assert len(names) == 615                                           # + the first quantize and the last decode
+        for index, (a, b) in enumerate(bounds):
+            assert futures[index].wait().data_ptr() == mine[a:b].data_ptr()
+            hooks[1](None, Bucket(theirs[a:b], index)).wait()
+        torch.cuda.synchronize()
+        assert torch.equal(mine.view(torch.int16), theirs.view(torch.int16)), f"reduced buckets, iteration {step}"
+        for index, (a, b) in enumerate(bounds):
+            got = piped.residuals[(mine[a:b].data_ptr(), b - a, torch.bfloat16)]
+            want = plain.residuals[(theirs[a:b].data_ptr(), b - a, torch.bfloat16)]
+            assert torch.equal(got.view(torch.int32), want.view(torch.int32)), f"residual of bucket {index}, iteration {step}"
+        for index in sample:
+            a, b = bounds[index]
+            size = b - a
+            shard = -(-size // world)
+            prepared = inputs[index] if cpu_residual[index] is None else inputs[index] + cpu_residual[index]
+            padded = torch.cat([prepared, prepared.new_zeros(shard * world - size)])
+            payloads, dropped = [], []
+            for d in range(world):
+                chunk = padded[d * shard:(d + 1) * shard]
+                codes, scales = codec_torch.quantize(chunk, G)
+                payloads.append((codes, scales))
+                dropped.append(chunk - codec_torch.dequantize(codes, scales, shard, G, "fp32"))
+            reduced = codec_torch.reduce_payloads(payloads, shard, G, "bf16", "mean")
+            again = codec_torch.dequantize(*codec_torch.quantize(reduced, G), shard, G, "bf16")
+            assert same_bits(mine[a:b], again.repeat(world)[:size]), f"bucket {index}, iteration {step}, against the oracle"
+            cpu_residual[index] = torch.cat(dropped)[:size]
+            got = piped.residuals[(mine[a:b].data_ptr(), size, torch.bfloat16)]
+            assert same_bits(got, cpu_residual[index]), f"residual of bucket {index}, iteration {step}, against the oracle"
+    stats = piped.pipeline.stats
+    assert stats["buckets"] == 2 * 613 and stats["merged_launches"] == 2 * 613 and stats["separate_launches"] == 4
