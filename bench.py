@@ -46,7 +46,10 @@ GROUP = 64
 SEED = 1234
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # what the kernel of the step is built from
-KERNEL_SOURCES = ("bucket_step.hip", "quant_pack_block.h", "dequant_reduce_block.h", "device_utils.h", "launch.h", "lbc_api.hip")
+KERNEL_SOURCES = ("bucket_step.hip", "step_grid.h", "quant_pack_block.h", "dequant_reduce_block.h", "device_utils.h", "launch.h",
+                  "lbc_api.hip")
+BATCHES = 5                # every figure is the median of this many timed batches of --steps launches
+WARM_SECONDS = 0.05        # launches go on for at least this long before a leg is timed (clocks settle after idling)
 SHARD_SETS = 16            # payload sets of the shard-reduce leg: 16 x 41 MB
 
 
@@ -99,7 +102,7 @@ def record_traffic(fetch_db: str, write_db: str) -> int:
     find = lambda table, part: next(v for k, v in table.items() if part in k)
     copy_kib = BUCKET_NUMEL * 4 / 1024
     fetch_factor, write_factor = copy_kib / find(fetch, "copyBuffer.kd"), copy_kib / find(write, "copyBuffer.kd")
-    step_kernel = "bucket_step_kernelIfvfLi8ELi2E"     # mangled <float, void, float, 8 payloads, streaming>
+    step_kernel = "bucket_step_kernelIfvLi4EfLi8ELi2E"     # mangled <float, void, 4 per lane, float, 8 payloads, streaming>
     step_fetch, step_write = find(fetch, step_kernel), find(write, step_kernel)
     traffic = (step_fetch * fetch_factor + step_write * write_factor) * 1024
     shard = BUCKET_NUMEL // WORLD
@@ -111,7 +114,7 @@ def record_traffic(fetch_db: str, write_db: str) -> int:
                      "python3 bench.py --record-traffic <dir>/f_results.db <dir>/w_results.db"],
         "calibration": {"kernel": "__amd_rocclr_copyBuffer of 100 MiB (102400 KiB read, 102400 KiB written)",
                         "FETCH_SIZE_factor": fetch_factor, "WRITE_SIZE_factor": write_factor},
-        "bucket_step": {"kernel": "bucket_step_kernel<float, void, float, 8, 2>: quantize+pack of a 100 MiB fp32 bucket as 8 "
+        "bucket_step": {"kernel": "bucket_step_kernel<float, void, 4, float, 8, 2>: quantize+pack of a 100 MiB fp32 bucket as 8 "
                                   "chunks and the W=8 reduce of a 3,276,800-element shard in one launch",
                         "FETCH_SIZE_KiB_median": step_fetch, "WRITE_SIZE_KiB_median": step_write,
                         "traffic_bytes": round(traffic),
@@ -196,49 +199,91 @@ def main() -> int:
         sets[i % len(sets)]["quant"]()
         sets[i % len(sets) - 1]["reduce"]()
 
+    class Seconds(float):
+        """Median of the timed batches, in seconds per call; ``low`` and ``high`` are the fastest and slowest batch."""
+
+        low = high = None
+
+    def spread(per_call):
+        ordered = sorted(per_call)
+        value = Seconds(ordered[len(ordered) // 2])
+        value.low, value.high = ordered[0], ordered[-1]
+        return value
+
+    def warm(fn, warmup):
+        """`warmup` calls and at least WARM_SECONDS of calls: the memory clock of an idle GPU takes tens of
+        milliseconds to come up, and a 20-step warm-up is over in well under one."""
+        begun, i = time.perf_counter(), 0
+        while i < warmup or time.perf_counter() - begun < WARM_SECONDS:
+            fn(i)
+            i += 1
+            if i % 64 == 0:
+                torch.cuda.synchronize()
+        torch.cuda.synchronize()
+
     def timed(fn, count, warmup):
-        for i in range(warmup):
-            fn(i)
+        """Seconds per call: BATCHES batches of exactly `count` calls, each bracketed by events on the launch stream
+        and a device synchronisation on both sides."""
+        warm(fn, warmup)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        per_call = []
+        for _ in range(BATCHES):
+            start.record(stream)
+            for i in range(count):
+                fn(i)
+            stop.record(stream)
+            torch.cuda.synchronize()
+            per_call.append(start.elapsed_time(stop) * 1e-3 / count)
+        return spread(per_call)
+
+    def timed_on_lanes(fn, lanes, count, warmup):
+        """The same for calls dealt to the streams of `lanes` in turn (``fn(i, handle)``).  The lanes are forked from
+        the launch stream once, before the warm-up; a batch is bracketed by one event pair per lane and lasts from the
+        earliest start to the latest stop, so no fork, join or stream creation falls inside a timed region."""
+        lanes.fork()
+        warm(lambda i: fn(i, lanes.handle(i)), warmup)
+        starts = [torch.cuda.Event(enable_timing=True) for _ in lanes.streams]
+        stops = [torch.cuda.Event(enable_timing=True) for _ in lanes.streams]
+        per_call = []
+        for _ in range(BATCHES):
+            for event, lane in zip(starts, lanes.streams):
+                event.record(lane)
+            for i in range(count):
+                fn(i, lanes.handle(i))
+            for event, lane in zip(stops, lanes.streams):
+                event.record(lane)
+            torch.cuda.synchronize()
+            per_call.append(max(a.elapsed_time(b) for a in starts for b in stops) * 1e-3 / count)
+        lanes.join()
         torch.cuda.synchronize()
-        start = torch.cuda.Event(enable_timing=True)
-        stop = torch.cuda.Event(enable_timing=True)
-        start.record(stream)
-        for i in range(count):
-            fn(i)
-        stop.record(stream)
-        torch.cuda.synchronize()
-        return start.elapsed_time(stop) * 1e-3  # seconds
+        return spread(per_call)
+
+    def milliseconds(seconds):
+        return {"median": seconds * 1e3, "min": seconds.low * 1e3, "max": seconds.high * 1e3}
 
     # ---- the step ---------------------------------------------------------------------------------
     result = {}
     if not only or "step" in only:
-        total = timed(step, args.steps, args.warmup)
-        result["ms_per_step"] = total / args.steps * 1e3
-        result["value"] = n * 4 * args.steps / total / 1e9
-        result["ms_per_step_two_launches"] = timed(step_two_launches, args.steps, args.warmup) / args.steps * 1e3
+        seconds = timed(step, args.steps, args.warmup)
+        result["ms_per_step"] = seconds * 1e3
+        result["ms_per_step_spread"] = milliseconds(seconds)
+        result["value"] = n * 4 / seconds / 1e9
+        two = timed(step_two_launches, args.steps, args.warmup)
+        result["ms_per_step_two_launches"] = two * 1e3
+        result["ms_per_step_two_launches_spread"] = milliseconds(two)
         if len(sets) % 2 == 0:
             # Consecutive steps touch different buffer sets, so they may also be dealt to two streams in turn: the
             # ramp-up of one launch then overlaps the drain of the one before.  Reported next to the headline, which
             # stays on one stream so that a step is one kernel's duration.
             from lowbit_comm_amd.hip.lanes import StreamLanes
 
-            lanes = StreamLanes(2, dev)
+            def step_on(i, handle):
+                if not sets[i % len(sets)]["step"](handle):
+                    raise RuntimeError("the library has no shared launch for this quantize and reduce")
 
-            def run_lanes(count):
-                lanes.fork()
-                for i in range(count):
-                    if not sets[i % len(sets)]["step"](lanes.handle(i)):
-                        raise RuntimeError("the library has no shared launch for this quantize and reduce")
-                lanes.join()
-
-            run_lanes(args.warmup)
-            torch.cuda.synchronize()
-            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record(stream)
-            run_lanes(args.steps)
-            stop.record(stream)
-            torch.cuda.synchronize()
-            result["ms_per_step_two_streams"] = start.elapsed_time(stop) / args.steps
+            lanes = timed_on_lanes(step_on, StreamLanes(2, dev), args.steps, args.warmup)
+            result["ms_per_step_two_streams"] = lanes * 1e3
+            result["ms_per_step_two_streams_spread"] = milliseconds(lanes)
 
     # ---- per-kernel launch durations ---------------------------------------------------------------
     kernels = {}
@@ -247,9 +292,10 @@ def main() -> int:
         if only and name not in only:
             return
         launches = launches or args.steps
-        seconds = timed(fn, launches, warmup if warmup is not None else args.warmup) / launches
+        seconds = timed(fn, launches, warmup if warmup is not None else args.warmup)
         kernels[name] = {
-            "us_per_launch": seconds * 1e6, "algorithmic_bytes": algorithmic_bytes,
+            "us_per_launch": seconds * 1e6, "us_min": seconds.low * 1e6, "us_max": seconds.high * 1e6,
+            "algorithmic_bytes": algorithmic_bytes,
             "achieved_GBps": algorithmic_bytes / seconds / 1e9, "frac_of_hbm_peak": algorithmic_bytes / seconds / HBM_PEAK,
         }
 
@@ -257,12 +303,45 @@ def main() -> int:
     reduce_bytes = world * payload_bytes + shard * 4
     if "ms_per_step" in result:
         seconds = result["ms_per_step"] * 1e-3
+        spread_ms = result["ms_per_step_spread"]
         kernels["bucket_step"] = {
-            "us_per_launch": seconds * 1e6, "algorithmic_bytes": quant_bytes + reduce_bytes,
+            "us_per_launch": seconds * 1e6, "us_min": spread_ms["min"] * 1e3, "us_max": spread_ms["max"] * 1e3,
+            "algorithmic_bytes": quant_bytes + reduce_bytes,
             "achieved_GBps": (quant_bytes + reduce_bytes) / seconds / 1e9,
             "frac_of_hbm_peak": (quant_bytes + reduce_bytes) / seconds / HBM_PEAK,
         }
     leg("quant_pack_chunks", lambda i: sets[i % len(sets)]["quant"](), quant_bytes)
+    if not only or "bucket_pipeline_step" in only or "pipeline_three_launches" in only:
+        # the whole reduce-scatter + all-gather plan as the drop-in transport runs it on a stream of buckets: one launch
+        # carries the quantize of bucket k, the reduce + requantize of the payloads that arrived for bucket k-1 and the
+        # decode of the gathered shard payloads of bucket k-2 into that bucket (lbc_bucket_pipeline_step)
+        for k, s in enumerate(sets):
+            s["gathered"] = s["received"].clone()
+            s["mine"] = torch.empty(payload_bytes, dtype=torch.uint8, device=dev)
+            s["decoded"] = torch.empty(n, dtype=torch.float32, device=dev)
+            s["reduce_requant"] = ops.bind_dequant_reduce_quant(
+                [ops.split_payload(s["received"][r, :payload_bytes], shard, g) for r in range(world)],
+                *ops.split_payload(s["mine"], shard, g), shard, group_size=g, divisor=float(world))
+            s["decode"] = ops.bind_dequant_chunks(s["gathered"], s["decoded"], shard, group_size=g)
+        for k, s in enumerate(sets):
+            s["pipeline_step"] = ops.bind_bucket_pipeline_step(s["quant"], sets[k - 1]["reduce_requant"], sets[k - 2]["decode"])
+        plan_bytes = quant_bytes + (world + 1) * payload_bytes + world * payload_bytes + n * 4
+
+        def pipeline_step(i):
+            if not sets[i % len(sets)]["pipeline_step"]():
+                raise RuntimeError("the library has no shared launch for these three stages")
+
+        def pipeline_three_launches(i):
+            sets[i % len(sets)]["quant"]()
+            sets[i % len(sets) - 1]["reduce_requant"]()
+            sets[i % len(sets) - 2]["decode"]()
+
+        leg("bucket_pipeline_step", pipeline_step, plan_bytes)
+        leg("pipeline_three_launches", pipeline_three_launches, plan_bytes)
+        for s in sets:
+            for name in ("gathered", "mine", "decoded", "reduce_requant", "decode", "pipeline_step"):
+                del s[name]
+        torch.cuda.empty_cache()
     if not only or "dequant_reduce_shard" in only:
         # the shard reduce alone moves 41 MB a launch: it gets payload sets of its own, enough of them (656 MB) that
         # no launch finds its operands in the memory-side cache
@@ -386,9 +465,16 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "batches": BATCHES,
+        "timing": f"every figure is the median of {BATCHES} batches of exactly `steps` launches, each batch bracketed by HIP "
+                  f"events and a device synchronisation, after `warmup` launches and at least {WARM_SECONDS * 1e3:.0f} ms of "
+                  "launches; *_spread and us_min / us_max give the fastest and slowest batch",
         "ms_per_step": result.get("ms_per_step"),
+        "ms_per_step_spread": result.get("ms_per_step_spread"),
         "ms_per_step_two_launches": result.get("ms_per_step_two_launches"),
+        "ms_per_step_two_launches_spread": result.get("ms_per_step_two_launches_spread"),
         "ms_per_step_two_streams": result.get("ms_per_step_two_streams"),
+        "ms_per_step_two_streams_spread": result.get("ms_per_step_two_streams_spread"),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

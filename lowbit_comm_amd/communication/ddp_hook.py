@@ -27,11 +27,13 @@ from lowbit_comm_amd.config import CompressionConfig
 from lowbit_comm_amd.exceptions import UnsupportedCollective
 from lowbit_comm_amd.quantization.codec import (
     allocate_dequantized_buffer,
+    allocate_quantized_buffer,
     dequantize_reduce_tensors,
     dequantize_reduce_update_error_feedback,
     dequantize_tensor,
     inplace_dequantize_reduce_mean_update_error_feedback,
     quantize_tensor,
+    writes_prepared,
 )
 from lowbit_comm_amd.quantization.error_feedback import ErrorFeedbackState
 from lowbit_comm_amd.quantization.error_feedback_policy import ErrorFeedbackPolicy
@@ -261,6 +263,38 @@ def create_ddp_comm_hook(
     workspaces = DequantizedWorkspaceCache(
         allocator=allocate_dequantized_workspace or allocate_dequantized_buffer,
         max_entries=workspace_cache_max_entries, max_cached_bytes=workspace_cache_max_bytes)
+    # With a native module whose fused quantize also writes ``bucket + residual`` the compensate step needs no kernel
+    # and no allocation of its own: the sum lands in a cached workspace and the payload in a cached buffer, both
+    # under the budgets of the decode workspaces.
+    fuse_compensate = quantize is None and writes_prepared(extension_status)
+    prepared_workspaces = DequantizedWorkspaceCache(
+        allocator=allocate_dequantized_buffer, max_entries=workspace_cache_max_entries,
+        max_cached_bytes=workspace_cache_max_bytes)
+    payload_buffers = DequantizedWorkspaceCache(
+        allocator=lambda tensor, shape, active: allocate_quantized_buffer(tensor.reshape(shape), active,
+                                                                         dtype=resolve_dtype("auto", tensor)),
+        max_entries=workspace_cache_max_entries, max_cached_bytes=workspace_cache_max_bytes)
+
+    def compensate_and_quantize(key: Any, original: Any) -> tuple[Any, Any] | None:
+        """``(bucket + residual, its quantized payload)`` from one launch, or ``None`` when that launch is not to be
+        had (no residual yet, another shape, types without a common fused kernel, a policy it declines)."""
+        residual = feedback.get(key) if callable(getattr(feedback, "get", None)) else None
+        if residual is None or tuple(getattr(residual, "shape", ())) != tuple(original.shape):
+            return None
+        if not (getattr(original, "is_cuda", False) and original.is_contiguous() and residual.is_contiguous()):
+            return None
+        like = original if residual.dtype == original.dtype else residual     # the sum has the promoted type
+        if str(like.dtype) != "torch.float32" and like.dtype != original.dtype:
+            return None
+        shape = tuple(original.shape)
+        prepared = _shaped(prepared_workspaces.get(key, like, shape, config), shape)
+        buffer = payload_buffers.get(key, like, shape, config)
+        try:
+            quantize_tensor(original, config, extension_status=extension_status, output=buffer, residual=residual,
+                            prepared_out=prepared)
+        except (ValueError, RuntimeError):
+            return None
+        return prepared, buffer
 
     def small(tensor: Any) -> bool:
         return min_compress_numel > 0 and _numel(tensor) < min_compress_numel
@@ -359,14 +393,20 @@ def create_ddp_comm_hook(
             if small(original):
                 return uncompressed(clone(original), reduce)
             decision = policy.decide(key, numel=_numel(original))
-            prepared = feedback.compensate(key, original) if decision.apply else original
+            facade = dequantize is None and reduce in ("mean", "sum")
+            fused = compensate_and_quantize(key, original) if decision.apply and facade and fuse_compensate else None
+            if fused is not None:
+                prepared = fused[0]
+            else:
+                prepared = feedback.compensate(key, original) if decision.apply else original
             active_dtype = resolve_dtype(dtype, prepared)
             shape = tuple(prepared.shape)
             gather = (packed_gather if should_fuse_payload(prepared, enabled=fuse_payload,
                                                            min_numel=fuse_payload_min_numel) else plain_gather)
-            if dequantize is None and reduce in ("mean", "sum"):
+            if facade:
                 # facade path: flat uint8 buffers, fused decode+reduce (+ residual update) on the GPU
-                local = coerce_payload(active_quantize(prepared, config), shape=shape, dtype=active_dtype)
+                local = coerce_payload(fused[1] if fused is not None else active_quantize(prepared, config),
+                                       shape=shape, dtype=active_dtype)
                 needs_feedback = decision.apply or decision.update
                 if async_gather and (async_error_feedback or not needs_feedback):
                     return gather_asynchronously(key, prepared, local, shape, active_dtype, decision)

@@ -16,6 +16,7 @@ from __future__ import annotations
 
 import enum
 import operator
+import threading
 from collections import OrderedDict
 from typing import Sequence
 
@@ -102,22 +103,34 @@ class HipNativeModule:
         # call is one key lookup and one ABI call.  The key holds everything a binding depends on (addresses,
         # dtypes, element counts, policy), the entries do not keep the tensors alive, least recently used go first.
         self._launches: OrderedDict = OrderedDict()
+        # DistributedDataParallel calls its hook from the autograd thread while the training script may call the
+        # codec from its own (the reference guards its pool and caches the same way, ccdl_comm/cuda/workspace.py:294).
+        self._launches_lock = threading.Lock()
+        self.launch_memo_entries = self.LAUNCH_MEMO_ENTRIES
 
-    _LAUNCH_MEMO_ENTRIES = 256
+    # One pass over a model's buckets must fit: an 8 B-parameter model in 25 MiB buckets has 613 of them, each with
+    # a quantize and a reduce.  A smaller cache, walked cyclically, would miss on every call.  An entry is a few
+    # hundred bytes of host memory; ``launch_memo_entries`` can be raised per instance.
+    LAUNCH_MEMO_ENTRIES = 4096
 
     def _memoized(self, key: tuple, bind):
         """The launch remembered under ``key``, else ``bind()`` (which validates and may raise; nothing is then
-        stored).  ``bind`` may return ``None`` for a call that has no single launch."""
+        stored).  ``bind`` may return ``None`` for a call that has no single launch.  The key is completed with the
+        access mode in force: a launch bound under one mode is not replayed for a call made under another."""
+        key = key + (ops.access_code(None),)
         launches = self._launches
-        bound = launches.get(key)
+        with self._launches_lock:
+            bound = launches.get(key)
+            if bound is not None:
+                launches.move_to_end(key)
+                return bound
+        bound = bind()                       # validates tensors and marshals arguments: outside the lock
         if bound is not None:
-            launches.move_to_end(key)
-            return bound
-        bound = bind()
-        if bound is not None:
-            launches[key] = bound.forget_tensors()
-            while len(launches) > self._LAUNCH_MEMO_ENTRIES:
-                launches.popitem(last=False)
+            with self._launches_lock:
+                bound = launches.setdefault(key, bound.forget_tensors())
+                launches.move_to_end(key)
+                while len(launches) > self.launch_memo_entries:
+                    launches.popitem(last=False)
         return bound
 
     @staticmethod
@@ -160,9 +173,17 @@ class HipNativeModule:
         if not self.inplace_quantize_pack(input, output, None, group_size, topk, stochastic, bit, quant_type, compact):
             raise RuntimeError(f"no HIP quantize kernel for input dtype {input.dtype}")
 
+    # The fused quantize can also hand back ``input + residual`` (keyword ``prepared_out``); the codec facade looks
+    # for this flag before it passes the keyword, which the reference's extension does not know.
+    QUANTIZE_PACK_WRITES_PREPARED = True
+
     def inplace_quantize_pack(self, input, output, residual, group_size, topk, stochastic, bit, quant_type,
-                              compact) -> bool:
-        """Fused ``(input + residual) -> quantize -> pack`` into ``output``; ``False`` for unsupported policy."""
+                              compact, *, prepared_out=None) -> bool:
+        """Fused ``(input + residual) -> quantize -> pack`` into ``output``; ``False`` for unsupported policy.
+
+        ``prepared_out`` (no counterpart in the reference's extension): a tensor of the promoted type of input and
+        residual that receives ``input + residual`` from the same launch - what ``ErrorFeedbackState.compensate``
+        would have computed in a kernel of its own (ccdl_comm/quantization/error_feedback.py:27-36)."""
         if not _policy_supported(group_size, topk, stochastic, bit, quant_type):
             return False
         if not isinstance(input, torch.Tensor) or not input.is_cuda:
@@ -180,15 +201,12 @@ class HipNativeModule:
             return True
         # payload dtype / contiguity / size are checked where the addresses are taken
         bind = lambda: ops.bind_quant_pack_payload(input.reshape(-1), output, group_size=group_size,  # noqa: E731
-                                                   residual=None if residual is None else residual.reshape(-1))
-        out_spec, r_spec = self._spec(output), self._spec(residual)
-        if out_spec is None or r_spec is None:
+                                                   residual=None if residual is None else residual.reshape(-1),
+                                                   prepared_out=None if prepared_out is None else prepared_out.reshape(-1))
+        out_spec, r_spec, p_spec = self._spec(output), self._spec(residual), self._spec(prepared_out)
+        if out_spec is None or r_spec is None or p_spec is None:
             return bind()()
-        key = ("quant_pack", input.data_ptr(), input.dtype, input.numel(), out_spec, r_spec, group_size)
-        bound = self._launches.get(key)         # the steady state: same addresses as last step
-        if bound is not None:
-            self._launches.move_to_end(key)
-            return bound()
+        key = ("quant_pack", input.data_ptr(), input.dtype, input.numel(), out_spec, r_spec, p_spec, group_size)
         return self._memoized(key, bind)()
 
     # ---- dequantize -----------------------------------------------------------------------------

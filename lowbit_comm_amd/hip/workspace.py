@@ -79,7 +79,7 @@ class WorkspaceStats:
 
 
 class _Slot:
-    __slots__ = ("ident", "key", "buffer", "size_bytes", "completion")
+    __slots__ = ("ident", "key", "buffer", "size_bytes", "completion", "sweeps")
 
     def __init__(self, ident: int, key: WorkspaceKey, buffer: Any, size_bytes: int) -> None:
         self.ident = ident
@@ -87,6 +87,7 @@ class _Slot:
         self.buffer = buffer
         self.size_bytes = size_bytes
         self.completion: Any | None = None
+        self.sweeps = 0          # polls that found the completion pending since the release
 
 
 def _nbytes(buffer: Any, fallback: int) -> int:
@@ -99,11 +100,20 @@ def _nbytes(buffer: Any, fallback: int) -> int:
     return fallback
 
 
-def _is_done(completion: Any) -> bool:
+# A completion that offers peek() may never turn true by itself: a StreamOrderedCompletion records its event only when
+# somebody asks with query().  A released buffer that no acquire has taken over after this many polls is therefore
+# settled by the pool itself, with query(): the event is recorded once, late, and the following peeks see it.  The
+# usual case - the next bucket acquires the same key on the same stream within a few acquires - never gets here and
+# pays for no event.
+_SETTLE_AFTER_SWEEPS = 8
+
+
+def _is_done(completion: Any, *, settle: bool = False) -> bool:
     """Has the work behind ``completion`` finished?  A completion may offer ``peek()``, a form of ``query()`` that
-    costs the device nothing (see :class:`StreamOrderedCompletion`); the pool's own polling uses it when it is there."""
+    costs the device nothing (see :class:`StreamOrderedCompletion`); the pool's own polling uses it when it is there,
+    unless ``settle`` asks for the real answer."""
     peek = getattr(completion, "peek", None)
-    if callable(peek):
+    if callable(peek) and not settle:
         return bool(peek())
     query = getattr(completion, "query", None)
     return callable(query) and bool(query())
@@ -222,6 +232,7 @@ class HipWorkspacePool:
             if slot.ident not in self._busy:
                 raise RuntimeError("workspace lease is not owned by this pool")
             slot.completion = completion
+            slot.sweeps = 0
             if _is_done(completion):
                 self._become_idle(slot)
             else:
@@ -231,7 +242,10 @@ class HipWorkspacePool:
         for pending in list(self._pending_of_key.values()):
             for ident in list(pending):
                 slot = self._busy.get(ident)
-                if slot is not None and slot.completion is not None and _is_done(slot.completion):
+                if slot is None or slot.completion is None:
+                    continue
+                slot.sweeps += 1
+                if _is_done(slot.completion, settle=slot.sweeps == _SETTLE_AFTER_SWEEPS):
                     self._become_idle(slot)
 
     def _forget_pending(self, slot: _Slot) -> None:

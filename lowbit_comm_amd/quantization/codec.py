@@ -133,13 +133,21 @@ def allocate_dequantized_buffer(tensor: Any, shape: tuple[int, ...], config: Com
 # --------------------------------------------------------------------------- #
 # quantize
 # --------------------------------------------------------------------------- #
+def writes_prepared(extension_status: Any | None) -> bool:
+    """Can the native module's fused quantize also write ``tensor + residual`` (``prepared_out=``)?  The reference's
+    extension cannot; the HIP module says so with ``QUANTIZE_PACK_WRITES_PREPARED``."""
+    module = getattr(extension_status, "module", None)
+    return bool(getattr(extension_status, "available", False) and getattr(module, "QUANTIZE_PACK_WRITES_PREPARED", False))
+
+
 def _try_quantize_pack(module: object, tensor: Any, output: Any, residual: Any | None, config: CompressionConfig,
-                       metadata: dict[str, Any] | None, quant_type: Any) -> bool:
+                       metadata: dict[str, Any] | None, quant_type: Any, prepared_out: Any | None = None) -> bool:
     fused = False
     native = getattr(module, "inplace_quantize_pack", None)
     if native is not None:
+        extra = {} if prepared_out is None else {"prepared_out": prepared_out}     # a keyword only this build's module has
         fused = bool(native(tensor, output, residual, config.group_size, config.topk, config.stochastic,
-                            config.bit, quant_type, config.compact))
+                            config.bit, quant_type, config.compact, **extra))
     if metadata is not None:
         numel = int(tensor.numel())
         padded = _padded_numel(numel, config.group_size)
@@ -150,15 +158,25 @@ def _try_quantize_pack(module: object, tensor: Any, output: Any, residual: Any |
 
 def quantize_tensor(tensor: object, config: CompressionConfig, *, extension_status: Any | None = None,
                     output: object | None = None, residual: object | None = None,
-                    metadata: dict[str, Any] | None = None) -> object:
+                    metadata: dict[str, Any] | None = None, prepared_out: object | None = None) -> object:
     """Quantize ``tensor`` (plus ``residual``) into ``output`` or a fresh buffer; returns the buffer.
 
     With ``output`` the fused allocation-free call is tried first; if the native module declines, the
     padded ``inplace_quantize`` chain runs.  Raises :class:`CCDLUnavailableError` when the native
     module is missing or incomplete.
+
+    ``prepared_out`` (an addition to the reference's signature, needs ``output`` and a module for which
+    :func:`writes_prepared` is true): receives ``tensor + residual`` from the quantize launch, for the caller that
+    needs it after the collective (``ccdl_comm/communication/ddp_hook.py:196,224-241``).
     """
     module = _module_of(extension_status)
     quant_type = _quant_type(module, config)
+    if prepared_out is not None:
+        if output is None or not getattr(module, "QUANTIZE_PACK_WRITES_PREPARED", False):
+            raise ValueError("prepared_out needs output= and a native module whose fused quantize writes it")
+        if not _try_quantize_pack(module, tensor, output, residual, config, metadata, quant_type, prepared_out):
+            raise ValueError("the fused quantize declined this policy; quantize without prepared_out")
+        return output
     if output is not None and _try_quantize_pack(module, tensor, output, residual, config, metadata, quant_type):
         return output
     prepared = _zero_padded(tensor if residual is None else tensor + residual, config.group_size)

@@ -10,6 +10,9 @@ if str(ROOT) not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    config.addinivalue_line("markers", "gpu_perf: timing gates on a real MI355X (run with -m gpu_perf); kept apart from the "
+                                       "parity suite so that a clock or occupancy wobble on a shared box cannot turn "
+                                       "correctness red")
 
 
 @pytest.fixture(scope="session")

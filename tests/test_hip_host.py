@@ -190,8 +190,17 @@ def test_native_module_remembers_launches_by_address_without_pinning_or_going_st
     torch.cuda.synchronize()
     del fresh
     assert alive() is None
-    limit = type(module)._LAUNCH_MEMO_ENTRIES
-    assert len(module._launches) <= limit
+    assert len(module._launches) <= module.launch_memo_entries
+    # a launch bound under one access mode is not replayed for a call made under another
+    from lowbit_comm_amd.hip import ops
+
+    count = len(module._launches)
+    with ops.access_mode("cached"):
+        assert module.inplace_quantize_pack(x, payload, None, 64, 0, False, 8, linear, False)
+        assert len(module._launches) == count + 1
+        assert module.inplace_quantize_pack(x, payload, None, 64, 0, False, 8, linear, False)
+        assert len(module._launches) == count + 1
+    assert torch.equal(payload.cpu(), oracle_packed(x.cpu()))
 
 
 def test_unsupported_policies_decline_instead_of_failing(status, dev):
@@ -292,6 +301,57 @@ def test_all_gather_hook_facade_path_uses_the_fused_kernels(status, dev):
         assert same_bits(restored, want), f"step {step}"
         assert same_bits(state.get(1), cpu_residual), f"residual step {step}"
     assert outputs[1] == outputs[2] == outputs[3]          # cached decode workspace from step 1 on
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_all_gather_hook_takes_bucket_plus_residual_from_the_quantize_launch(status, dev, dtype):
+    """With error feedback the reference's hook first forms ``prepared = bucket + residual`` in a kernel of its own
+    (ccdl_comm/communication/ddp_hook.py:196; error_feedback.py:27-36) and needs it again after the gather.  Here
+    the quantize launch writes it: same results as the hook with the compensate step left to torch (an injected
+    quantizer switches the fusion off), two codec launches per bucket and no other kernel, nothing allocated from the
+    third step on."""
+    from torch.profiler import ProfilerActivity, profile
+
+    n, world, buckets = 64 * 900, 4, 3
+    peers = [[codec.quantize_tensor(grad(n, dtype, 800 + 10 * b + r, dev), CFG, extension_status=status)
+              for r in range(world - 1)] for b in range(buckets)]
+    current = [0]
+
+    def all_gather(local):
+        return GatheredPayloads([local.buffer] + peers[current[0]], world)
+
+    states = [ErrorFeedbackState(), ErrorFeedbackState()]
+    fused = create_ddp_comm_hook(CFG, strategy="all_gather", reduce="mean", all_gather=all_gather, error_feedback=states[0],
+                                 extension_status=status, workspace_cache_max_entries=8)
+    plain = create_ddp_comm_hook(CFG, strategy="all_gather", reduce="mean", all_gather=all_gather, error_feedback=states[1],
+                                 extension_status=status, workspace_cache_max_entries=8,
+                                 quantize=lambda tensor, active: codec.quantize_tensor(tensor, active, extension_status=status))
+    grads = [grad(n, dtype, 850 + b, dev) for b in range(buckets)]
+    allocated = None
+    for step in range(5):
+        for b in range(buckets):
+            grads[b].copy_(grad(n, dtype, 900 + 10 * step + b, dev))
+        torch.cuda.synchronize()
+        if step == 3:
+            allocated = torch.cuda.memory_allocated()
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            got = []
+            for b in range(buckets):
+                current[0] = b
+                got.append(fused(None, Bucket(grads[b], index=b)).wait())
+            torch.cuda.synchronize()
+        kernels = [e.name for e in prof.events() if e.device_type == torch.autograd.DeviceType.CUDA
+                   and "Memcpy" not in e.name and "Memset" not in e.name]
+        if step >= 2:            # step 0 has no residual yet, step 1 creates the workspaces
+            assert len(kernels) == 2 * buckets and all("lbc" in name for name in kernels), kernels
+        if step == 4:
+            assert torch.cuda.memory_allocated() == allocated
+        for b in range(buckets):
+            current[0] = b
+            want = plain(None, Bucket(grads[b].clone(), index=b)).wait()
+            assert got[b].dtype == want.dtype
+            assert same_bits(got[b], want), f"bucket {b}, step {step}"
+            assert same_bits(states[0].get(b), states[1].get(b)), f"residual {b}, step {step}"
 
 
 def test_fused_all_gather_adapter_ships_one_packed_tensor(dev):

@@ -196,8 +196,15 @@ def _payload(codes, scales, dtype=torch.float16):
                              metadata={"scales": torch.tensor(scales, dtype=dtype), "original_numel": len(codes)})
 
 
-def test_fused_payload_all_gather_packs_once_and_round_trips():
-    local, remote = _payload([-2, 3, 7, 11], [0.25, 0.5]), _payload([1, 2, 3, 4], [1.0, 2.0])
+def test_fused_payload_all_gather_packs_once_and_round_trips(golden_vectors):
+    """The reference's own packer case (tests/test_payload_packing.py:12-57): float16 scales, a round trip, one byte
+    collective; it asserts no packed bytes."""
+    case = golden_vectors["packer"]
+    assert case["scales_dtype"] == "float16"
+    assert (case["local"]["codes"], case["local"]["scales"]) == ([-2, 3, 7, 11], [0.25, 0.5])
+    assert (case["remote"]["codes"], case["remote"]["scales"]) == ([1, 2, 3, 4], [1.0, 2.0])
+    local = _payload(case["local"]["codes"], case["local"]["scales"])
+    remote = _payload(case["remote"]["codes"], case["remote"]["scales"])
     calls = []
 
     def byte_all_gather(packed):
@@ -206,7 +213,7 @@ def test_fused_payload_all_gather_packs_once_and_round_trips():
 
     fused = make_fused_payload_all_gather(byte_all_gather)
     gathered = fused(local)
-    assert calls == [(torch.uint8, (8,))]
+    assert calls == [(torch.uint8, (case["packed_numel"],))]
     assert gathered.world_size == 2
     assert [p.buffer.tolist() for p in gathered.payloads] == [[-2, 3, 7, 11], [1, 2, 3, 4]]
     assert [p.metadata["scales"].tolist() for p in gathered.payloads] == [[0.25, 0.5], [1.0, 2.0]]
@@ -670,3 +677,88 @@ def test_payload_conveniences():
     q = Quantizer(CompressionConfig(), dtype="bf16")
     assert q.payload_bytes(128) == 136 and q.payload_bytes(128, wire_format="native") == 132
     assert "group_size=64" in repr(q)
+
+
+# --------------------------------------------------------------------------- #
+# the native module's launch memo under two threads
+# --------------------------------------------------------------------------- #
+def test_launch_memo_survives_two_threads_on_a_four_entry_cache():
+    """DistributedDataParallel calls the hook from the autograd thread while the script may use the codec from its
+    own: lookups, insertions and evictions of the launch memo interleave.  The reference guards its caches with a lock
+    (ccdl_comm/cuda/workspace.py:84,149,294; two-thread release test tests/cuda/test_cuda_workspace_pool.py:413-450);
+    without one, ``get`` followed by ``move_to_end`` raises KeyError when the other thread's eviction lands between."""
+    import threading
+
+    from lowbit_comm_amd.hip.native_module import HipNativeModule
+
+    module = HipNativeModule()
+    module.launch_memo_entries = 4
+
+    class Launch:
+        def __init__(self, key):
+            self.key = key
+
+        def forget_tensors(self):
+            return self
+
+    failures, served = [], [0, 0]
+
+    def hammer(who, keys):
+        try:
+            for i in range(20_000):
+                key = ("k", keys[i % len(keys)])
+                got = module._memoized(key, lambda key=key: Launch(key))
+                assert got.key == key
+                served[who] += 1
+        except BaseException as failure:      # noqa: BLE001
+            failures.append(failure)
+
+    threads = [threading.Thread(target=hammer, args=(0, list(range(7)))),
+               threading.Thread(target=hammer, args=(1, list(range(3, 12))))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert failures == [] and served == [20_000, 20_000]
+    assert len(module._launches) <= 4
+    # a binder that declines (no single launch) stores nothing, one that raises stores nothing either
+    before = dict(module._launches)
+    assert module._memoized(("none",), lambda: None) is None
+
+    def refuse():
+        raise RuntimeError("bad tensor")
+
+    with pytest.raises(RuntimeError, match="bad tensor"):
+        module._memoized(("raises",), refuse)
+    assert dict(module._launches) == before
+
+
+def test_reduce_scatter_plan_memo_is_locked_and_sized_for_a_model():
+    """The plan's cache of bound launches: same guard, and room for every bucket of a large model (three stages each)."""
+    import threading
+
+    from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
+
+    assert ReduceScatterPlan._BOUND_LAUNCHES >= 3 * 613
+    plan = ReduceScatterPlan(64 * 8, torch.float32, world_size=8, rank=0, config=CompressionConfig(), device="cpu")
+    plan._BOUND_LAUNCHES = 4
+
+    class Launch:
+        def forget_tensors(self):
+            return self
+
+    failures = []
+
+    def hammer(keys):
+        try:
+            for i in range(20_000):
+                plan._remember(("q", keys[i % len(keys)]), Launch)
+        except BaseException as failure:      # noqa: BLE001
+            failures.append(failure)
+
+    threads = [threading.Thread(target=hammer, args=(list(range(7)),)), threading.Thread(target=hammer, args=(list(range(3, 12)),))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert failures == [] and len(plan._bound) <= 4

@@ -320,10 +320,12 @@ def test_empty_payload_list_and_bad_mode_are_rejected():
 
 
 # --------------------------------------------------------------------------- #
-# wire format: literal vectors from the reference's packer test
+# wire format: a byte vector worked by hand from the two's-complement and IEEE-754 little-endian definitions (the
+# reference's packer test checks a round trip and holds no bytes; that case is in tests/test_host_api.py)
 # --------------------------------------------------------------------------- #
 def test_pack_layout_literal_bytes(golden_vectors):
-    vector = golden_vectors["packer"]
+    vector = golden_vectors["packer_bytes_hand_computed"]
+    assert vector["source"].startswith("NOT from the reference")
     codes = np.array(vector["codes"], dtype=np.int8)
     scales = np.array(vector["scales"], dtype=np.float32)
     packed = codec_np.pack(codes, scales)

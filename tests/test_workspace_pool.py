@@ -320,3 +320,49 @@ def test_shard_session_reuses_send_recv_and_reduced_buffers():
                                                          rank=0) is None
     with pytest.raises(TypeError, match="pool"):
         ShardWorkspaceProvider(object(), backend="hip", collective="c", strategy="s", device="cuda")
+
+
+def test_a_released_buffer_nobody_adopts_is_settled_by_the_pool_itself():
+    """A completion whose ``peek()`` only turns true after someone has asked ``query()`` (the stream-ordered kind:
+    no event until it is needed) must not keep its buffer out of the idle set for ever: after a few polls the pool
+    asks the real question once, the buffer becomes idle, and the LRU limits see it."""
+    from lowbit_comm_amd.hip import workspace as ws
+
+    class Lazy:
+        """No event until query() is called; that call records it and finds it unfinished, every later look finds it
+        finished."""
+
+        def __init__(self):
+            self.queries = self.peeks = 0
+
+        def peek(self):
+            self.peeks += 1
+            return self.queries >= 1
+
+        def query(self):
+            self.queries += 1
+            return self.queries >= 2
+
+    made = []
+    pool = ws.HipWorkspacePool(allocator=lambda key, stream: made.append(key) or bytearray(64), max_entries=2)
+    keys = [ws.WorkspaceKey(backend="hip", collective="rs", strategy="s", shape_class=(64,), dtype="uint8", world_size=8,
+                            bit=8, group_size=64, chunk_config=(i,), workspace_kind="send", device="cpu") for i in range(12)]
+    completions = []
+    for key in keys[:4]:                        # four shapes that never come back
+        lease = pool.acquire(key, None)
+        completions.append(Lazy())
+        lease.release(completion=completions[-1])
+    assert pool.stats.in_flight_bytes == 4 * 64 and pool.stats.cached_bytes == 0
+    for key in keys[4:]:                        # other traffic: every acquire polls the pending ones
+        pool.acquire(key, None)
+    stats = pool.stats
+    assert all(c.queries == 1 for c in completions)              # asked by the pool, once, not by a caller
+    assert stats.in_flight_bytes == 8 * 64                       # only the eight live leases
+    assert stats.cached_bytes == 2 * 64 and stats.evictions == 2  # the four settled buffers met max_entries=2
+    # the usual case pays for no query: released and taken over by the next acquire of the same key
+    quick = Lazy()
+    lease = pool.acquire(keys[0], None)
+    lease.release(completion=quick)
+    quick.wait_stream = lambda stream: None
+    again = pool.acquire(keys[0], None)
+    assert quick.queries == 0 and again.buffer is lease.buffer

@@ -11,7 +11,7 @@ from pathlib import Path
 import pytest
 import torch
 
-pytestmark = pytest.mark.gpu
+pytestmark = pytest.mark.gpu_perf      # a timing gate: run with -m gpu_perf, apart from the parity suite
 
 PROBE = Path(__file__).resolve().parent / "native" / "_build" / "stream_probe"
 ROTATE = 640_000_000

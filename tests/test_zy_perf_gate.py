@@ -16,7 +16,7 @@ from pathlib import Path
 import pytest
 import torch
 
-pytestmark = pytest.mark.gpu
+# the launch-count test is exact and belongs to the parity suite; the timing gate has a marker of its own
 
 ROOT = Path(__file__).resolve().parent.parent
 
@@ -33,6 +33,7 @@ def kernel_names(run):
             and "Memset" not in e.name]
 
 
+@pytest.mark.gpu
 def test_every_entry_point_is_exactly_one_kernel_launch(hip_device):
     from lowbit_comm_amd.hip import cuda_wire, ops
 
@@ -59,6 +60,16 @@ def test_every_entry_point_is_exactly_one_kernel_launch(hip_device):
     wire_peers = [cuda_wire.quant_pack(torch.randn(n, device=dev) * 1e-3) for _ in range(world)]
     whole = x[:aligned].clone()
     general = torch.empty(cuda_wire.general_payload_nbytes(aligned, x.dtype, 64, 4, 2), dtype=torch.uint8, device=dev)
+    # three stages of a bucket stream: the quantize above, a reduce + requantize and a decode in the bucket's type
+    part = aligned // world
+    arrived = [ops.quant_pack(torch.randn(part, device=dev) * 1e-3) for _ in range(world)]
+    mine = ops.quant_pack(torch.zeros(part, device=dev))
+    shards = torch.zeros_like(rows)
+    assert ops.quant_pack_chunks_into(half[:aligned], shards, world)
+    decoded = torch.empty(aligned, dtype=half.dtype, device=dev)
+    pipeline_step = ops.bind_bucket_pipeline_step(
+        quant_chunks, ops.bind_dequant_reduce_quant(arrived, *mine, part, divisor=8.0, mid_dtype=half.dtype),
+        ops.bind_dequant_chunks(shards, decoded, part))
     calls = {
         "lbc_quant_pack": lambda: ops.quant_pack_into(x, codes, scales),
         "lbc_quant_pack (error feedback)": lambda: ops.quant_pack_into(half, codes, scales, residual=residual, new_residual=residual),
@@ -69,6 +80,7 @@ def test_every_entry_point_is_exactly_one_kernel_launch(hip_device):
         "lbc_dequant_reduce (error feedback)": lambda: ops.dequant_reduce_into(peers, out, divisor=8.0, prepared=x, new_residual=residual),
         "lbc_dequant_reduce_quant": lambda: ops.dequant_reduce_quant_into(peers, *requant, n, divisor=8.0),
         "lbc_quant_pack_chunks_and_dequant_reduce": lambda: ops.bind_quant_chunks_and_reduce(quant_chunks, reduce_shard)(),
+        "lbc_bucket_pipeline_step": pipeline_step,
         "lbc_ring_step": lambda: ops.ring_step_into(packed, out, send, reduce_op="sum", divisor=8.0),
         "lbc_ef_update": lambda: ops.ef_update_into(x, out, residual),
         "lbc_wire_quant_pack": lambda: cuda_wire.quant_pack_into(x, wire, residual=residual),
@@ -87,10 +99,11 @@ def test_every_entry_point_is_exactly_one_kernel_launch(hip_device):
             received, target = cuda_wire.quant_pack(whole), torch.empty_like(cuda_wire.quant_pack(whole))
             call = lambda: cuda_wire.ring_step_into(received, whole, target)
         launched = kernel_names(call)
-        ours = [k for k in launched if "lbc::" in k]
+        ours = [k for k in launched if "lbc" in k]          # some names arrive mangled (_ZN3lbc...)
         assert len(ours) == 1 and len(launched) == 1, f"{name}: {launched}"
 
 
+@pytest.mark.gpu_perf
 def test_hot_path_launches_hold_the_frozen_baseline(hip_device):
     import bench_configs
 
