@@ -46,8 +46,8 @@ GROUP = 64
 SEED = 1234
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # what the kernel of the step is built from
-KERNEL_SOURCES = ("bucket_step.hip", "step_grid.h", "quant_pack_block.h", "dequant_reduce_block.h", "device_utils.h", "launch.h",
-                  "lbc_api.hip")
+KERNEL_SOURCES = ("bucket_step.hip", "pipeline_step.hip", "step_grid.h", "quant_pack_block.h", "dequant_reduce_block.h",
+                  "device_utils.h", "launch.h", "lbc_api.hip")
 BATCHES = 5                # every figure is the median of this many timed batches of --steps launches
 WARM_SECONDS = 0.05        # launches go on for at least this long before a leg is timed (clocks settle after idling)
 SHARD_SETS = 16            # payload sets of the shard-reduce leg: 16 x 41 MB
@@ -73,6 +73,18 @@ def recorded_traffic():
     if record.get("kernel_sources_sha256_16") != kernel_sources_hash():
         return None, "profiles/hbm_traffic.json was measured on other kernel sources; record it again"
     return record["bucket_step"]["traffic_bytes"], "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated)"
+
+
+def recorded_pipeline_traffic():
+    """The same for the three-stage pipeline step, when the record holds it."""
+    try:
+        with open(TRAFFIC_FILE) as handle:
+            record = json.load(handle)
+    except (OSError, ValueError):
+        return None
+    if record.get("kernel_sources_sha256_16") != kernel_sources_hash():
+        return None
+    return record.get("bucket_pipeline_step", {}).get("traffic_bytes")
 
 
 def record_traffic(fetch_db: str, write_db: str) -> int:
@@ -107,10 +119,12 @@ def record_traffic(fetch_db: str, write_db: str) -> int:
     traffic = (step_fetch * fetch_factor + step_write * write_factor) * 1024
     shard = BUCKET_NUMEL // WORLD
     payload = shard // GROUP * (GROUP + 4)
+    pipeline_kernel = "bucket_pipeline_step_kernelIfvLi4ELi8ELi2E"   # mangled <float, void, 4 per lane, 8 payloads, streaming>
+    pipe_fetch, pipe_write = find(fetch, pipeline_kernel), find(write, pipeline_kernel)
     record = {
         "kernel_sources_sha256_16": kernel_sources_hash(), "kernel_sources": list(KERNEL_SOURCES),
-        "commands": ["rocprofv3 --pmc FETCH_SIZE -d <dir> -o f -- python3 bench.py --steps 20 --warmup 2 --only step,copy_calibration",
-                     "rocprofv3 --pmc WRITE_SIZE -d <dir> -o w -- python3 bench.py --steps 20 --warmup 2 --only step,copy_calibration",
+        "commands": ["rocprofv3 --pmc FETCH_SIZE -d <dir> -o f -- python3 bench.py --steps 20 --warmup 2 --only step,bucket_pipeline_step,copy_calibration",
+                     "rocprofv3 --pmc WRITE_SIZE -d <dir> -o w -- python3 bench.py --steps 20 --warmup 2 --only step,bucket_pipeline_step,copy_calibration",
                      "python3 bench.py --record-traffic <dir>/f_results.db <dir>/w_results.db"],
         "calibration": {"kernel": "__amd_rocclr_copyBuffer of 100 MiB (102400 KiB read, 102400 KiB written)",
                         "FETCH_SIZE_factor": fetch_factor, "WRITE_SIZE_factor": write_factor},
@@ -119,6 +133,13 @@ def record_traffic(fetch_db: str, write_db: str) -> int:
                         "FETCH_SIZE_KiB_median": step_fetch, "WRITE_SIZE_KiB_median": step_write,
                         "traffic_bytes": round(traffic),
                         "algorithmic_bytes": BUCKET_NUMEL * 4 + WORLD * payload + WORLD * payload + shard * 4},
+        "bucket_pipeline_step": {"kernel": "bucket_pipeline_step_kernel<float, void, 4, 8, 2>: quantize+pack of a 100 MiB fp32 bucket as "
+                                           "8 chunks, W=8 reduce + requantize of a 3,276,800-element shard and decode of 8 shard "
+                                           "payloads into a 100 MiB bucket in one launch",
+                                 "FETCH_SIZE_KiB_median": pipe_fetch, "WRITE_SIZE_KiB_median": pipe_write,
+                                 "traffic_bytes": round((pipe_fetch * fetch_factor + pipe_write * write_factor) * 1024),
+                                 "algorithmic_bytes": BUCKET_NUMEL * 4 + WORLD * payload + (WORLD + 1) * payload
+                                                      + WORLD * payload + BUCKET_NUMEL * 4},
     }
     with open(TRAFFIC_FILE, "w") as handle:
         json.dump(record, handle, indent=1)
@@ -337,6 +358,8 @@ def main() -> int:
             sets[i % len(sets) - 2]["decode"]()
 
         leg("bucket_pipeline_step", pipeline_step, plan_bytes)
+        if "bucket_pipeline_step" in kernels:
+            kernels["bucket_pipeline_step"]["traffic"] = recorded_pipeline_traffic()
         leg("pipeline_three_launches", pipeline_three_launches, plan_bytes)
         for s in sets:
             for name in ("gathered", "mine", "decoded", "reduce_requant", "decode", "pipeline_step"):

@@ -60,11 +60,17 @@ def _torch_future() -> Any:
     return torch.futures.Future()
 
 
+_TORCH_DTYPE_NAMES = {"torch.bfloat16": "bf16", "torch.float16": "fp16", "torch.float32": "fp32"}
+
+
 def resolve_dtype(dtype: str, tensor: Any) -> str:
     """``"auto"`` -> ``fp16`` / ``bf16`` / ``fp32`` from the bucket tensor's dtype."""
     if dtype != "auto":
         return dtype
     text = str(getattr(tensor, "dtype", ""))
+    known = _TORCH_DTYPE_NAMES.get(text)
+    if known is not None:
+        return known
     if "bfloat16" in text:
         return "bf16"
     if "float16" in text or text.endswith("half"):
@@ -106,6 +112,9 @@ def _shaped(workspace: Any, shape: tuple[int, ...]) -> Any:
     count = 1
     for dim in shape:
         count *= int(dim)
+    numel = getattr(workspace, "numel", None)
+    if callable(numel) and numel() == count:            # nothing to trim (whole groups): at most one view
+        return workspace if tuple(getattr(workspace, "shape", ())) == tuple(shape) else workspace.reshape(shape)
     flat = workspace.reshape((-1,))
     try:
         flat = flat[:count]

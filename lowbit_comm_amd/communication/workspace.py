@@ -93,8 +93,8 @@ class DequantizedWorkspaceCache:
         g = config.group_size
         numel = prod(shape) if shape else 0
         padded = -(-numel // g) * g if numel else 0
-        dtype = str(getattr(tensor, "dtype", ""))
-        layout = (tuple(shape), dtype, str(getattr(tensor, "device", "")), padded)
+        dtype = getattr(tensor, "dtype", "")
+        layout = (tuple(shape), dtype, getattr(tensor, "device", ""), padded)     # the objects themselves: no str() per call
         found = self._store.lookup(key, layout)
         if found is not None:
             return found

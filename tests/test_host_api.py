@@ -437,9 +437,11 @@ def test_loader_wire_format_choice():
     native = load_hip_extension(factory=HipCudaWireModule)
     assert portable.module.NATIVE_WIRE_FORMAT == "portable" and native.module.NATIVE_WIRE_FORMAT == "native"
     names = [n for n in dir(HipNativeModule) if not n.startswith("_")]
-    # same surface as the reference's pybind module, plus the one optional symbol the facade probes for: the
-    # portable format's sum-and-divide in one launch (the CUDA byte format divides the way torch does instead)
-    assert set(names) - set(dir(HipCudaWireModule)) == {"dequantize_reduce_mean"}
+    # same surface as the reference's pybind module, plus what the facade probes for - the portable format's
+    # sum-and-divide in one launch (the CUDA byte format divides the way torch does instead) and the flag that the
+    # fused quantize also writes bucket + residual - and the size of the launch memo
+    assert set(names) - set(dir(HipCudaWireModule)) == {"dequantize_reduce_mean", "QUANTIZE_PACK_WRITES_PREPARED",
+                                                        "LAUNCH_MEMO_ENTRIES"}
 
 
 def test_workspace_allocators():
