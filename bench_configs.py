@@ -47,12 +47,12 @@ MANIFEST = os.path.join(ROOT, "profiles", "baseline_manifest.json")
 
 
 def gate_rows(quads: int = 3, only=None):
-    """The five hot-path launches a later change is held to, each timed against a plain 100 MiB device copy in
+    """The six hot-path launches a later change is held to, each timed against a plain 100 MiB device copy in
     A-B-B-A order (copy, kernel, kernel, copy; the reference's gate alternates baseline and candidate the same way,
     tests/benchmarks/fused_dequant_executor_gate.py:16-33) so that clock and thermal drift cancel in the ratio.
     Returns ``{name: {"us", "copy_us", "ratio", "algorithmic_bytes", "frac_of_hbm_peak"}}``; ``ratio`` is the smallest
     kernel/copy ratio over ``quads`` A-B-B-A rounds.  Buffers rotate through more than 600 MB per row.  ``only``: a
-    collection of row names to measure instead of all five."""
+    collection of row names to measure instead of all six."""
     import torch
 
     from lowbit_comm_amd.hip import ops
@@ -131,10 +131,32 @@ def gate_rows(quads: int = 3, only=None):
                 assert both() is True
                 sets.append(both)
             return sets, n * 10 + 2 * world * ops.payload_nbytes(shard, G) + shard * 4
+        if name == "pipeline_step_25MiB_bf16_ef_W8":
+            # what the comm hook's reduce_scatter strategy launches per bucket: error-feedback quantize of bucket k,
+            # reduce + requantize of bucket k-1's shard, decode of bucket k-2's eight gathered shards, one grid
+            n, shard = 13_107_200, 1_638_400
+            nbytes = ops.payload_nbytes(shard, G)
+            stride = -(-nbytes // 256) * 256
+            sets = []
+            for s in range(5):
+                residual = gen(800 + s, n, 1e-5)
+                quant = ops.bind_quant_pack_chunks(gen(810 + s, n, 1e-3, torch.bfloat16), torch.empty(world, stride, dtype=torch.uint8, device=dev),
+                                                   world, residual=residual, new_residual=residual)
+                received, gathered = payload_rows(shard, world, 820 + 8 * s), payload_rows(shard, world, 860 + 8 * s)
+                mine = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+                reduce = ops.bind_dequant_reduce_quant([ops.split_payload(received[r], shard, G) for r in range(world)],
+                                                       *ops.split_payload(mine, shard, G), shard, divisor=float(world),
+                                                       mid_dtype=torch.bfloat16)
+                decode = ops.bind_dequant_chunks(gathered, torch.empty(n, dtype=torch.bfloat16, device=dev), shard)
+                step = ops.bind_bucket_pipeline_step(quant, reduce, decode)
+                assert step() is True
+                sets.append(step)
+            return sets, n * 10 + world * nbytes + (world + 1) * nbytes + world * nbytes + n * 2
         raise KeyError(name)
 
     names = ["quant_pack_chunks_100MiB_fp32_W8", "dequant_reduce_shard_3276800_W8", "dequant_reduce_full_26214400_W8",
-             "ef_quant_pack_100MiB_bf16_fp32_residual", "bucket_step_25MiB_bf16_ef_plus_shard_reduce_W8"]
+             "ef_quant_pack_100MiB_bf16_fp32_residual", "bucket_step_25MiB_bf16_ef_plus_shard_reduce_W8",
+             "pipeline_step_25MiB_bf16_ef_W8"]
     rows = {}
     for name in names:
         if only is not None and name not in only:

@@ -1108,7 +1108,7 @@ def test_bucket_step_replays_from_a_hip_graph(dev):
         assert same_bits(plan.shard, codec_torch.reduce_payloads(received, shard, 64, "fp32", "mean")), step
 
 
-@pytest.mark.parametrize("wire_format", ["portable", "native", "reduce_scatter"])
+@pytest.mark.parametrize("wire_format", ["portable", "native", "reduce_scatter", "reduce_scatter_pipelined"])
 def test_hook_on_a_real_distributed_data_parallel_model(hip_device, wire_format):
     """register_comm_hook on torch's own DDP (one rank, RCCL): real GradBucket objects and futures, gradients within
     the quantization error of the uncompressed model.  Runs in a child process under a time limit so that trouble in
@@ -1124,3 +1124,6 @@ def test_hook_on_a_real_distributed_data_parallel_model(hip_device, wire_format)
     report = json.loads([line for line in done.stdout.splitlines() if line.startswith("{")][-1])
     assert report["finite"] and report["buckets"] >= 3
     assert all(0.0 < e < 0.02 for e in report["errors"]), report
+    if wire_format == "reduce_scatter_pipelined":       # three iterations: flushed after each one's last bucket
+        assert report["pipeline"]["flushes"] == 3 and report["pipeline"]["pending"] == 0, report
+        assert report["pipeline"]["buckets"] == report["buckets"]

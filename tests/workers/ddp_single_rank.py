@@ -3,7 +3,9 @@
 One process, one GPU, a one-rank RCCL process group.  Modes "portable" / "native": the all_gather strategy in that
 wire format, the packed payload bytes moved by a real RCCL ``all_gather_into_tensor``.  Mode "reduce_scatter": the
 pre-bound reduce-scatter plan with its two exchanges as real RCCL calls (all_to_all_single, all_gather_into_tensor)
-and local error feedback.  Prints one JSON line with the gradient errors against an unwrapped copy of the model.
+and local error feedback; "reduce_scatter_pipelined": the same transport with the bucket pipeline behind it (futures
+completed by later buckets, the hook's flush after ``GradBucket.is_last()``).  Prints one JSON line with the gradient
+errors against an unwrapped copy of the model.
 """
 from __future__ import annotations
 
@@ -46,7 +48,7 @@ def main() -> int:
         model, plain = make(), make()
         plain.load_state_dict(model.state_dict())
         wrapped = DistributedDataParallel(model, device_ids=[0], bucket_cap_mb=1)
-        status = load_hip_extension(wire_format="portable" if wire_format == "reduce_scatter" else wire_format)
+        status = load_hip_extension(wire_format="portable" if wire_format.startswith("reduce_scatter") else wire_format)
         assert status.available, status.reason
         seen = []
 
@@ -61,7 +63,8 @@ def main() -> int:
             dist.all_gather_into_tensor(rows, mine)
             return GatheredPayloads(payloads=[replace(payload, buffer=rows[r]) for r in range(world)], world_size=world)
 
-        if wire_format == "reduce_scatter":
+        transport = None
+        if wire_format.startswith("reduce_scatter"):
             from lowbit_comm_amd.hip.reduce_scatter import make_reduce_scatter_transport
 
             def all_to_all(received, send):
@@ -72,7 +75,8 @@ def main() -> int:
                 dist.all_gather_into_tensor(gathered, gathered[0])
 
             transport = make_reduce_scatter_transport(world_size=1, rank=0, all_to_all=all_to_all,
-                                                      all_gather=all_gather, error_feedback=True)
+                                                      all_gather=all_gather, error_feedback=True,
+                                                      pipelined=wire_format == "reduce_scatter_pipelined")
             hook = create_ddp_comm_hook(CompressionConfig(error_feedback=False), strategy="reduce_scatter",
                                         reduce="mean", reduce_scatter_all_gather=transport)
         else:
@@ -89,8 +93,10 @@ def main() -> int:
             torch.cuda.synchronize()
             errors.append(max(float((a.grad - b.grad).norm() / (b.grad.norm() + 1e-12))
                               for a, b in zip(model.parameters(), plain.parameters())))
+        pipeline = getattr(transport, "pipeline", None)
         print(json.dumps({"errors": errors, "buckets": len(seen), "payload_bytes": sorted(set(seen)),
-                          "finite": all(bool(torch.isfinite(p.grad).all()) for p in model.parameters())}))
+                          "finite": all(bool(torch.isfinite(p.grad).all()) for p in model.parameters()),
+                          "pipeline": None if pipeline is None else dict(pipeline.stats, pending=pipeline.pending)}))
     finally:
         dist.destroy_process_group()
     return 0
