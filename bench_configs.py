@@ -483,6 +483,34 @@ def main() -> int:
             p.decode_gathered(out=outs[i % 2])
 
         t_plan_fused = timed(whole_fused, 24)
+        # the same plan on a stream of such buckets: one launch carries the quantize of bucket k, the reduce +
+        # requantize of bucket k-1 and the decode of bucket k-2 (lbc_bucket_pipeline_step); the eight plans stand for
+        # eight consecutive buckets
+        steps = []
+        for k in range(world):
+            quant = plans[k].bound_quantize(peers[k])
+            reduce = plans[k - 1].bound_reduce_requantize(op="sum")
+            decode = plans[k - 2].bound_decode(outs[k % 2])
+            steps.append(ops.bind_bucket_pipeline_step(quant, reduce, decode))
+        pipeline_check = None
+        if parity:
+            want_row = plans[0].payload(plans[0].gathered, 0).clone()
+            want_send = plans[1].send.clone()
+            plans[7].decode_gathered(out=outs[0])
+            want_out = outs[0].clone()
+            plans[0].gathered[0].zero_(); plans[1].send.zero_(); outs[1].zero_()
+            ok = steps[1]() is True           # quantize of bucket 1, reduce + requantize of bucket 0, decode of bucket 7
+            torch.cuda.synchronize()
+            ok = ok and torch.equal(plans[0].payload(plans[0].gathered, 0), want_row) and torch.equal(plans[1].send, want_send)
+            ok = ok and bits_equal(outs[1], want_out)
+            pipeline_check = "bit-exact vs the three launches" if ok else "MISMATCH"
+            del want_row, want_send, want_out
+
+        def pipeline_step(i):
+            if not steps[i % world]():
+                raise RuntimeError("no shared launch for the three stages")
+
+        t_pipeline = timed(pipeline_step, 24)
         emit(4, "(i) quant-pack 8 chunks of 200 MiB fp32", b_quant, t_quant, n * 4, check)
         emit(4, "(ii) fused dequant-reduce W=8 -> 25 MiB shard", b_reduce, t_reduce, world * pb, check)
         emit(4, "(iii) requantize shard", b_requant, t_requant, shard * 4, check)
@@ -491,6 +519,9 @@ def main() -> int:
         emit(4, "(ii+iii) fused reduce + requantize, shard not written", world * pb + pb, t_fused, world * pb, fused_check)
         emit(4, "whole plan, fused variant (3 launches)", b_quant + world * pb + pb + b_decode, t_plan_fused, n * 4,
              fused_check)
+        emit(4, "whole plan on a stream of buckets, one launch per bucket (quantize of bucket k + reduce and requantize of "
+                "bucket k-1 + decode of bucket k-2)", b_quant + world * pb + pb + b_decode, t_pipeline, n * 4, pipeline_check)
+        del steps
         del peers, plans, outs, out
         torch.cuda.empty_cache()
 
@@ -745,7 +776,80 @@ def main() -> int:
         emit(5, "same stream, one launch per bucket, the buckets dealt to two HIP streams in turn (each with its own send "
                 "matrix and shard output)", nbytes, seconds, total * 2, lanes_check, buckets=len(bounds),
              us_per_bucket=seconds / len(bounds) * 1e6, host_enqueue_s=host1 - host0)
-        del grads, residuals, lane_launches, lane_buffers
+        del residuals, lane_launches, lane_buffers
+        torch.cuda.empty_cache()
+        # The whole reduce-scatter + all-gather plan over the same stream, as the comm hook runs it: through
+        # create_ddp_comm_hook(strategy="reduce_scatter") over the transport with local error feedback, unpipelined
+        # (three launches per bucket) and pipelined (one launch per bucket: quantize of bucket k, reduce + requantize
+        # of bucket k-1, decode of bucket k-2).  The exchanges are stand-ins that fill their rows once; parity of this
+        # path at full size is tests/test_full_size_configs.py.
+        from lowbit_comm_amd.communication.ddp_hook import create_ddp_comm_hook
+        from lowbit_comm_amd.hip.reduce_scatter import make_reduce_scatter_transport
+
+        class StreamBucket:
+            def __init__(self, tensor, index, last):
+                self._tensor, self._index, self._last = tensor, index, last
+
+            def buffer(self):
+                return self._tensor
+
+            def index(self):
+                return self._index
+
+            def is_last(self):
+                return self._last
+
+        class Slot:
+            def set_result(self, value):
+                self.value = value
+
+        hook_buckets = [StreamBucket(grads[a:b], index, index == len(bounds) - 1) for index, (a, b) in enumerate(bounds)]
+        plan_bytes = 0
+        for a, b in bounds:
+            size = b - a
+            payload = ops.payload_nbytes(-(-size // world), G)
+            plan_bytes += size * (2 + 4 + 4) + world * payload + (world + 1) * payload + world * payload + size * 2
+        for pipelined in (False, True):
+            filled = set()
+
+            def all_to_all(received, send):
+                if received.data_ptr() not in filled:
+                    received.copy_(send)
+                    filled.add(received.data_ptr())
+
+            def all_gather(gathered, mine):
+                if gathered.data_ptr() not in filled:
+                    gathered[1:, :mine.numel()] = mine
+                    filled.add(gathered.data_ptr())
+
+            transport = make_reduce_scatter_transport(world_size=world, rank=0, all_to_all=all_to_all, all_gather=all_gather,
+                                                      error_feedback=True, pipelined=pipelined, future_factory=Slot)
+            hook = create_ddp_comm_hook(CompressionConfig(), strategy="reduce_scatter", reduce="mean",
+                                        reduce_scatter_all_gather=transport, future_factory=Slot)
+
+            def hook_pass():
+                for bucket in hook_buckets:
+                    hook(None, bucket)
+
+            hook_pass()
+            hook_pass()
+            torch.cuda.synchronize()
+            host0 = time.perf_counter()
+            a_ev.record(stream)
+            hook_pass()
+            b_ev.record(stream)
+            host1 = time.perf_counter()
+            torch.cuda.synchronize()
+            seconds = a_ev.elapsed_time(b_ev) * 1e-3
+            emit(5, "same stream through the comm hook, reduce_scatter strategy, whole plan with error feedback (quantize, "
+                    "reduce + requantize, decode of 8 shards per bucket), " +
+                    ("pipelined transport: one launch per bucket" if pipelined else "unpipelined transport: three launches per bucket"),
+                 plan_bytes, seconds, total * 2, None, buckets=len(bounds), us_per_bucket=seconds / len(bounds) * 1e6,
+                 host_enqueue_s=host1 - host0)
+            transport.reset()
+            del transport, hook
+            torch.cuda.empty_cache()
+        del grads, hook_buckets
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------------------------------ 6

@@ -23,6 +23,12 @@
 #include "launch.h"
 #include "wire_common.h"
 
+// Chunk size (log2 of the element count) from which the gather hop of interleaved 16-bit payloads stores group pairs
+// as shifted dwords; below it the misaligned 8-byte stores measured faster (see wire_ring_step_kernel).
+#ifndef LBC_PAIR_STORE_MIN_LOG2
+#define LBC_PAIR_STORE_MIN_LOG2 22
+#endif
+
 
 namespace lbc {
 namespace {
@@ -134,6 +140,10 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
             if (wide_codes) clamp_codes(c);
             uint32_t words[W::WORDS];
             pack_codes<T, BIT, VEC, W::WORDS>(c, words);
+            // Interleaved 16-bit payloads leave as misaligned 8-byte stores here.  Re-slicing a pair of 66-byte groups
+            // into aligned dwords across lanes (store_group_pair16, what the ring's gather hop does) measured slower in
+            // this kernel at every size, with operands rotated through 700 MB: 26.2 M bf16 elements 15.8 us as it is,
+            // 17.7 us with non-temporal pair stores, 16.1 us with cached ones; 52.4 M 27.4 / 32.8 / 27.6 us.
             store_piece<T, BIT, PNT, W::WORDS>(payload + at.codes(group) + piece_offset<T, BIT>(k0), words);
             if ((lane & (LPG - 1)) == 0) *reinterpret_cast<Raw *>(payload + at.scale(group)) = stored;
         }
@@ -621,11 +631,16 @@ __global__ __launch_bounds__(kBlock) void wire_ring_step_kernel(const WireRingSt
         uint32_t out_words[W::WORDS];
         pack_codes<T, 8, VEC, W::WORDS>(c, out_words);
         if constexpr (WINDOWS) {
-            // The hop that only decodes and requantizes, from 16 Mi elements on (uniform): the payload leaves as
-            // whole dwords shifted across lanes, with the non-temporal hint (52 M bf16 elements 38.8 instead of
-            // 43.3 us, 26 M 19.8 instead of 21.5; 13 M 11.4 against 10.9 us; the accumulating hop and the quantize
-            // kernel lost 1-20 % with the same stores).
-            if ((reinterpret_cast<uintptr_t>(a.send) & 3u) == 0 && a.numel >= (int64_t{1} << 24)) {
+            // The hop that only decodes and requantizes, from 4 Mi elements on (uniform): the payload leaves as
+            // whole dwords shifted across lanes, with the non-temporal hint.  Measured with operands rotated through
+            // 700 MB, bf16: 52 M elements 38.8 instead of 43.3 us, 26 M 19.8 instead of 21.5, 13.1 M 11.4 instead
+            // of 12.9, 6.5 M 7.3 instead of 8.3; 3.3 M 6.3 against 5.3 and 1.6 M 4.5 either way, hence the bound.
+            // (With only a few buffer sets, i.e. payloads that stay in the last-level cache, 13.1 M read 11.4
+            // against 10.9 us, which is where an earlier bound of 16 Mi came from.)  Both forms write exactly the
+            // chunk and the payload (rocprofv3 WRITE_SIZE 38,800 KiB against 39,082 KiB on 13.1 M elements) and read
+            // exactly the payload: the gain is in the store instructions, not in traffic.  The accumulating hop and
+            // the quantize kernel lost 1-20 % with the same stores.
+            if ((reinterpret_cast<uintptr_t>(a.send) & 3u) == 0 && a.numel >= (int64_t{1} << LBC_PAIR_STORE_MIN_LOG2)) {
                 store_group_pair16<kNonTemporal>(a.send + at.codes(group & ~int64_t{1}), lane, out_words, kept, live[u],
                                               (group | 1) < groups);
                 continue;

@@ -611,10 +611,15 @@ def check_wire_step(device, dtype, g, n, compact, reduce_op, divisor, emit, seed
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 def test_wire_gather_hop_of_a_large_chunk_bit_exact(hip_device, dtype):
-    """From 16 Mi elements on, the hop that only decodes and requantizes writes a 16-bit payload with interleaved
+    """From 4 Mi elements on, the hop that only decodes and requantizes writes a 16-bit payload with interleaved
     scales as whole dwords shifted across lanes.  An odd number of groups (the last group has no partner), an even
     one with NaNs and an infinity in the chunk, and an outgoing payload at a 2-byte aligned address (the kernel's
-    other store path at this size); bytes around the payload stay untouched."""
+    other store path at this size); bytes around the payload stay untouched.  Sizes on both sides of the bound."""
+    bound = 1 << 16                                    # groups of 64: 4 Mi elements
+    check_wire_step(hip_device, dtype, 64, 64 * bound, True, "none", 1.0, True, 80_990)
+    check_wire_step(hip_device, dtype, 64, 64 * (bound - 1), True, "none", 1.0, True, 80_992)
+    check_wire_step(hip_device, dtype, 64, 64 * (bound + 1), True, "none", 1.0, True, 80_994, poison=True)
+    check_wire_step(hip_device, dtype, 64, 64 * (bound + 2), True, "none", 1.0, True, 80_996, lead=2, send_lead=2)
     groups = 1 << 18
     check_wire_step(hip_device, dtype, 64, 64 * (groups + 1), True, "none", 1.0, True, 81_000)
     check_wire_step(hip_device, dtype, 64, 64 * (groups + 2), True, "none", 1.0, True, 81_002, poison=True)
