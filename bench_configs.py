@@ -1185,6 +1185,9 @@ def main() -> int:
                                          torch.bfloat16, 3)):
             eb = 4 if dtype == torch.float32 else 2
             pb = ops.payload_nbytes(n, G)
+            # at least 700 MB between two uses of a buffer: a rotation of one and a half times the 256 MiB memory-side
+            # cache is still partly served by it (plain stores are absorbed, the figures read up to 15 % better)
+            sets_n = max(sets_n, -(-700_000_000 // (n * eb + 2 * pb)))
             sets = []
             for k in range(sets_n):
                 received = torch.empty(pb, dtype=torch.uint8, device=dev)
@@ -1260,6 +1263,7 @@ def main() -> int:
                 ("bf16 chunk of 52,428,800, appended scales", 52_428_800, torch.bfloat16, 3, False)):
             eb = 4 if dtype == torch.float32 else 2
             pb = cw.payload_nbytes(n, dtype)
+            sets_n = max(sets_n, -(-700_000_000 // (n * eb + 2 * pb)))      # as above
             sets = []
             for k in range(sets_n):
                 received = cw.quant_pack(gen(SEED + 8500 + k, n, 1e-3, dtype), compact=compact)
