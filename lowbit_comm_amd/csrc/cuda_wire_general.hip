@@ -33,7 +33,13 @@ namespace {
 __constant__ book_cells::Books kCodeBooks = book_cells::kBookSet;
 __constant__ book_cells::Tables kBookCells = book_cells::kTables;
 
-// Philox4x32-10: one block of four 32-bit words.
+// Philox4x32-10: one block of four 32-bit words.  A round is two 32x32->64 multiplies and two three-way
+// exclusive-ors; gfx950 has the latter as one instruction (v_bitop3_b32 with the truth table 0x96), which the
+// compiler does not choose by itself for `a ^ b ^ c`.
+__device__ __forceinline__ uint32_t xor3(uint32_t x, uint32_t y, uint32_t z) {
+    return __builtin_amdgcn_bitop3_b32(x, y, z, 0x96);
+}
+
 __device__ __forceinline__ void philox_block(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
                                              uint32_t (&out)[4]) {
 #pragma unroll
@@ -43,7 +49,7 @@ __device__ __forceinline__ void philox_block(uint32_t c0, uint32_t c1, uint32_t 
             k1 += 0xBB67AE85u;
         }
         const uint64_t p0 = static_cast<uint64_t>(0xD2511F53u) * c0, p1 = static_cast<uint64_t>(0xCD9E8D57u) * c2;
-        const uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c1 ^ k0, n2 = static_cast<uint32_t>(p0 >> 32) ^ c3 ^ k1;
+        const uint32_t n0 = xor3(static_cast<uint32_t>(p1 >> 32), c1, k0), n2 = xor3(static_cast<uint32_t>(p0 >> 32), c3, k1);
         c0 = n0;
         c1 = static_cast<uint32_t>(p1);
         c2 = n2;
@@ -86,17 +92,34 @@ __device__ __forceinline__ int meta_words_of(int topk) { return topk == 0 ? 1 : 
 // ---------------------------------------------------------------------------------------------
 // quantize: a wavefront works on tiles of 64 * VEC elements (64 lanes x 16 bytes of the tensor)
 // ---------------------------------------------------------------------------------------------
-// Tiles per wavefront: eight elements per lane either way.  A 32-bit tensor's wavefront asks for both of
-// its tiles before it does anything else and encodes one while the other is on its way (26.2 M fp32 elements:
-// stochastic rounding 28.8 instead of 37.4 us, top-2 30.3 instead of 30.8, a code book 28.2 instead of 30.0);
-// four tiles are slower again (32.7 us top-2), and so are two tiles of eight 16-bit elements a lane (bf16 top-2
-// 25.9 instead of 23.2 us): the kernels are bound by instruction issue and need their eight wavefronts per SIMD.
-template <typename T> constexpr int general_quant_tiles() { return sizeof(T) == 4 ? 2 : 1; }
+// Elements per lane: 32 bytes of the tensor, twice what the other kernels of this format give a lane.  What a
+// policy costs per group - addresses, the NaN rule of the running maximum, the outlier searches, the division behind
+// the scale - is spread over twice the elements, and a group's reductions cross half the lanes.  These kernels are
+// bound by instruction issue, not by memory, so that is what counts (26.2 M elements, 16 against 32 bytes a lane:
+// see the measurements at launch_general_quant_g).
+template <typename T> constexpr int general_quant_elems() { return 32 / static_cast<int>(sizeof(T)); }
+
+// The EL 4-bit codes of one lane -> its 32-bit words.  Four codes make one 16-bit unit with the first code on top; a
+// 16-bit tensor's word holds two units, low half first, an fp32 tensor's word holds elements 0-3 in its upper half.
+template <typename T, int EL>
+__device__ __forceinline__ void pack_nibbles(const int (&c)[EL], uint32_t (&words)[EL / 8]) {
+#pragma unroll
+    for (int k = 0; k < EL / 8; ++k) {
+        uint32_t unit[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            unit[h] = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) unit[h] |= (static_cast<uint32_t>(c[8 * k + 4 * h + i]) & 0xFu) << (12 - 4 * i);
+        }
+        words[k] = sizeof(T) == 4 ? (unit[0] << 16) | unit[1] : unit[0] | (unit[1] << 16);
+    }
+}
 
 // FIXED names what the launch knows about the policy at compile time, so that the code of the other policies
 // is not part of the kernel: bit 0 "no outlier channel", bit 1 "round to nearest", bit 2 "linear codes".
-// 0 is the kernel for every policy.
-template <typename T, int G, int BIT, int FIXED>
+// 0 is the kernel for every policy.  EL: elements per lane, a multiple of 8 that divides G.
+template <typename T, int G, int BIT, int FIXED, int EL>
 __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGeneralQuantArgs a) {
     const int topk = (FIXED & 1) ? 0 : a.topk;
     const bool stochastic = (FIXED & 2) ? false : a.stochastic != 0;
@@ -104,36 +127,41 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     using W = wire<T, BIT>;
     using RB = raw_bits<T>;
     using Raw = typename RB::type;
-    constexpr int VEC = W::VEC, LPG = G / VEC, ITEM = sizeof(T), CB = G * BIT / 8;
+    constexpr int VEC = EL, LPG = G / VEC, ITEM = sizeof(T), CB = G * BIT / 8, WORDS = EL * BIT / 32;
     constexpr bool WIDE = ITEM == 4;
-    static_assert(LPG >= 2 && LPG <= 16, "a group must span 2..16 lanes of one DPP row");
+    static_assert(EL % 8 == 0 && EL % W::VEC == 0 && G % EL == 0 && LPG <= 16, "a group lies in 1..16 lanes of one DPP row");
 
-    constexpr int TILES = general_quant_tiles<T>();
     const int lane = threadIdx.x & (kWave - 1);
     const int meta_bytes = meta_words_of(topk) * ITEM;
     const int64_t groups = a.numel / G;
-    const int64_t first = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * (TILES * W::TILE);
+    const int64_t first = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * (kWave * EL);
 
-    // all of the wavefront's elements are asked for before anything else
-    Raw raws[TILES][VEC];
+    // all of the lane's elements are asked for before anything else
+    Raw raw[VEC];
 #pragma unroll
-    for (int tile = 0; tile < TILES; ++tile) {
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) raws[tile][i] = 0;
-        const int64_t e0 = first + tile * W::TILE + lane * VEC;
+    for (int i = 0; i < VEC; ++i) raw[i] = 0;
+    {
+        const int64_t e0 = first + lane * VEC;
         // numel is a multiple of G: dead lanes form whole dead groups.  Instruction-bound: a cache hint only costs.
-        if (e0 < a.numel) load_elems<Raw, VEC, kPlain>(static_cast<const Raw *>(a.x) + e0, raws[tile]);
+        if (e0 < a.numel) {
+#pragma unroll
+            for (int part = 0; part < EL / W::VEC; ++part) {
+                Raw piece[W::VEC];
+                load_elems<Raw, W::VEC, kPlain>(static_cast<const Raw *>(a.x) + e0 + part * W::VEC, piece);
+#pragma unroll
+                for (int i = 0; i < W::VEC; ++i) raw[part * W::VEC + i] = piece[i];
+            }
+        }
     }
     // After the loads were issued: the waits of the tables cover theirs.  The cell table pays for its copy and its
-    // barrier with the eight elements a lane has here (26.2 M bf16 elements: 20.1 us against 24.6 us with the
-    // search and rounding; fp32, two tiles: 28.0 against 30.0 us); with four it did not (33.3 against 32.2 us).
+    // barrier from eight elements a lane on.
     const bool by_cells = kind != 0 && !stochastic;   // uniform over the grid
     const book_cells::Cell *cells = by_cells ? block_book_cells(kind) : nullptr;
     if (first >= a.numel) return;   // wavefront-uniform, behind the workgroup's barrier
     const float *book = wave_code_book(kind, lane);
 
-    auto encode_tile = [&](const int64_t tile_first, const Raw (&raw)[VEC]) __attribute__((always_inline)) {
-        const int64_t e0 = tile_first + lane * VEC;
+    {
+        const int64_t e0 = first + lane * VEC;
         const bool live = e0 < a.numel;
         const int64_t group = e0 / G;
         const int k0 = static_cast<int>(e0 - group * G);
@@ -146,7 +174,8 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
             const uint32_t key0 = static_cast<uint32_t>(a.seed), key1 = static_cast<uint32_t>(a.seed >> 32);
             const uint32_t sub0 = static_cast<uint32_t>(group), sub1 = static_cast<uint32_t>(static_cast<uint64_t>(group) >> 32);
             const int phase = static_cast<int>(a.offset & 3);
-            auto to_uniform = [](uint32_t x) { return static_cast<float>(x) * 0x1p-32f + 0x1p-33f; };   // curand_uniform: (0, 1]
+            // curand_uniform, (0, 1]: x * 2^-32 + 2^-33.  The product is exact, so the fused form rounds as the two steps do.
+            auto to_uniform = [](uint32_t x) { return __builtin_fmaf(static_cast<float>(x), 0x1p-32f, 0x1p-33f); };
             uint64_t block[VEC / 4];
 #pragma unroll
             for (int q = 0; q < VEC / 4; ++q)
@@ -349,16 +378,11 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
             }
         }
         if (live) {
-            uint32_t words[W::WORDS];
-            pack_codes<T, BIT, VEC, W::WORDS>(c, words);
-            store_piece<T, BIT, kPlain, W::WORDS>(group_codes + piece_offset<T, BIT>(k0), words);
+            uint32_t words[WORDS];
+            if constexpr (BIT == 8) pack_codes<T, 8, VEC, WORDS>(c, words);
+            else pack_nibbles<T, EL>(c, words);
+            store_words<WORDS, ITEM, kPlain>(group_codes + k0 * BIT / 8, words);
         }
-    };
-#pragma unroll
-    for (int tile = 0; tile < TILES; ++tile) {
-        const int64_t tile_first = first + tile * W::TILE;
-        if (tile_first >= a.numel) return;   // wavefront-uniform
-        encode_tile(tile_first, raws[tile]);
     }
 }
 
@@ -442,31 +466,38 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
     store_elems<Raw, VEC, kNonTemporal>(out, decoded);
 }
 
-template <typename T, int G>
-hipError_t launch_general_quant_g(int bit, const WireGeneralQuantArgs &a, hipStream_t stream) {
-    const int64_t tile = wire<T, 8>::TILE * kWavesPerBlock * general_quant_tiles<T>();
+template <typename T, int G, int BIT, int FIXED, int EL>
+hipError_t launch_general_quant_as(const WireGeneralQuantArgs &a, hipStream_t stream) {
+    const int64_t tile = static_cast<int64_t>(kWave) * EL * kWavesPerBlock;
     const int64_t blocks = (a.numel + tile - 1) / tile;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-    const dim3 grid(static_cast<unsigned>(blocks));
+    hipLaunchKernelGGL((wire_general_quant_kernel<T, G, BIT, FIXED, EL>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0,
+                       stream, a);
+    return hipGetLastError();
+}
+
+template <typename T, int G>
+hipError_t launch_general_quant_g(int bit, const WireGeneralQuantArgs &a, hipStream_t stream) {
     // Policies that round to nearest run a kernel without the code of the others (26.2 M fp32 elements: top-2
     // 30.8 instead of 32.3 us, a code book 30.0 instead of 31.7 us); stochastic rounding is faster in the kernel
     // for every policy (37.4 against 38.6 us), whose Philox rounds leave the compiler less room to reorder.
+    //
+    // 32 bytes a lane against 16 (26.2 M elements, group 64, us): fp32 top-2 27.4 / 30.5, stochastic 24.3 / 26.6,
+    // a code book 25.5 / 27.9; bf16 top-2 22.1 / 23.3, stochastic 21.5 / 22.6, a code book through the cell table
+    // 19.8 / 19.3 - the one case that keeps 16 bytes.
+    constexpr int WIDE = general_quant_elems<T>() <= G ? general_quant_elems<T>() : G;
+    constexpr int CELLS = sizeof(T) == 4 ? WIDE : 8;
     const int fixed = a.stochastic ? 0 : ((a.topk == 0 ? 1 : 0) | 2 | (a.kind == 0 ? 4 : 0));
     if (bit != 8 && bit != 4) return hipErrorNotSupported;
     if (bit == 8 && a.kind != 0) return hipErrorNotSupported;   // eight bits: linear codes only
-#define LBC_GENERAL_QUANT(BIT, FIXED) \
-    hipLaunchKernelGGL((wire_general_quant_kernel<T, G, BIT, FIXED>), grid, dim3(kBlock), 0, stream, a)
     if (bit == 8) {
-        if (fixed == 6) LBC_GENERAL_QUANT(8, 6);
-        else LBC_GENERAL_QUANT(8, 0);
-    } else {
-        if (fixed == 2 || fixed == 6) LBC_GENERAL_QUANT(4, 2);
-        else if (fixed == 3) LBC_GENERAL_QUANT(4, 3);
-        else LBC_GENERAL_QUANT(4, 0);
+        if (fixed == 6) return launch_general_quant_as<T, G, 8, 6, WIDE>(a, stream);
+        return launch_general_quant_as<T, G, 8, 0, WIDE>(a, stream);
     }
-#undef LBC_GENERAL_QUANT
-    return hipGetLastError();
+    if (fixed == 2 || fixed == 6) return launch_general_quant_as<T, G, 4, 2, WIDE>(a, stream);
+    if (fixed == 3) return launch_general_quant_as<T, G, 4, 3, CELLS>(a, stream);
+    return launch_general_quant_as<T, G, 4, 0, WIDE>(a, stream);
 }
 
 template <typename T> hipError_t launch_general_quant_t(int g, int bit, const WireGeneralQuantArgs &a, hipStream_t s) {
