@@ -46,6 +46,12 @@ G = 64
 MANIFEST = os.path.join(ROOT, "profiles", "baseline_manifest.json")
 
 
+GATE_ROWS = ("quant_pack_chunks_100MiB_fp32_W8", "dequant_reduce_shard_3276800_W8", "dequant_reduce_full_26214400_W8",
+             "ef_quant_pack_100MiB_bf16_fp32_residual", "bucket_step_25MiB_bf16_ef_plus_shard_reduce_W8",
+             "pipeline_step_25MiB_bf16_ef_W8")
+GATE_ROW_NAMES = frozenset(GATE_ROWS)
+
+
 def gate_rows(quads: int = 3, only=None):
     """The six hot-path launches a later change is held to, each timed against a plain 100 MiB device copy in
     A-B-B-A order (copy, kernel, kernel, copy; the reference's gate alternates baseline and candidate the same way,
@@ -154,11 +160,8 @@ def gate_rows(quads: int = 3, only=None):
             return sets, n * 10 + world * nbytes + (world + 1) * nbytes + world * nbytes + n * 2
         raise KeyError(name)
 
-    names = ["quant_pack_chunks_100MiB_fp32_W8", "dequant_reduce_shard_3276800_W8", "dequant_reduce_full_26214400_W8",
-             "ef_quant_pack_100MiB_bf16_fp32_residual", "bucket_step_25MiB_bf16_ef_plus_shard_reduce_W8",
-             "pipeline_step_25MiB_bf16_ef_W8"]
     rows = {}
-    for name in names:
+    for name in GATE_ROWS:
         if only is not None and name not in only:
             continue
         sets_rows = []
@@ -181,10 +184,19 @@ def gate_rows(quads: int = 3, only=None):
     return rows
 
 
-def write_manifest(path: str = MANIFEST) -> int:
+def write_manifest(path: str = MANIFEST, refreeze: bool = False) -> int:
+    """Freeze the gate rows.  Rows the committed manifest already holds keep their frozen figures - a baseline that
+    moved with every measurement would hold nothing - and only rows it lacks are measured and added; ``refreeze``
+    measures all of them anew."""
     import subprocess
 
-    rows = gate_rows(quads=5)
+    frozen = {}
+    if not refreeze and os.path.exists(MANIFEST):
+        with open(MANIFEST) as handle:
+            frozen = json.load(handle).get("rows", {})
+    rows = dict(frozen)
+    measured = gate_rows(quads=5, only=None if not frozen else GATE_ROW_NAMES - set(frozen))
+    rows.update(measured)
     try:
         commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
     except OSError:
@@ -212,10 +224,12 @@ def main() -> int:
     ap.add_argument("--llama-layers", type=int, default=32, help="config 5: number of transformer layers (32 = full model)")
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--write-manifest", nargs="?", const=MANIFEST, default=None, metavar="PATH",
-                    help="measure the gate rows and freeze them (default: profiles/baseline_manifest.json), then exit")
+                    help="measure the gate rows the committed manifest lacks and write it with them added (default: "
+                         "profiles/baseline_manifest.json), then exit")
+    ap.add_argument("--refreeze", action="store_true", help="with --write-manifest: measure every gate row anew")
     args = ap.parse_args()
     if args.write_manifest:
-        return write_manifest(args.write_manifest)
+        return write_manifest(args.write_manifest, refreeze=args.refreeze)
     wanted = {int(c) for c in args.configs.split(",") if c}
 
     import torch
