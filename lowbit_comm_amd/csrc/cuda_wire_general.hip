@@ -116,6 +116,39 @@ __device__ __forceinline__ void pack_nibbles(const int (&c)[EL], uint32_t (&word
     }
 }
 
+__device__ __forceinline__ uint32_t umed3(uint32_t x, uint32_t y, uint32_t z) {
+    uint32_t m;
+    asm("v_med3_u32 %0, %1, %2, %3" : "=v"(m) : "v"(x), "v"(y), "v"(z));
+    return m;
+}
+
+// first >= second >= third are the three largest keys a lane knows (0 = none; nonzero keys are unique inside a
+// group).  Afterwards every lane of the group's LANES adjacent lanes holds the three largest of the group.  With
+// p, q = max, min of the two firsts, r, s = max, min of the seconds and t = max of the thirds, the union's first is
+// p, its second max(q, r) and its third max(min(q, r), s, t).  row_half_mirror and row_mirror act as xor 4 / xor 8
+// because the lanes they pair within a quad (half) already agree.
+template <int CTRL> __device__ __forceinline__ void merge_top3_step(uint32_t &first, uint32_t &second, uint32_t &third) {
+    auto partner = [](uint32_t v) {
+        return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xF, 0xF, true));
+    };
+    const uint32_t f = partner(first), g = partner(second), h = partner(third);
+    const uint32_t p = first > f ? first : f, q = first > f ? f : first;
+    const uint32_t r = second > g ? second : g, s = second > g ? g : second;
+    const uint32_t t = third > h ? third : h;
+    const uint32_t low = q < r ? q : r;
+    first = p;
+    second = q > r ? q : r;
+    third = low > s ? (low > t ? low : t) : (s > t ? s : t);
+}
+
+template <int LANES> __device__ __forceinline__ void merge_top3(uint32_t &first, uint32_t &second, uint32_t &third) {
+    static_assert(LANES == 1 || LANES == 2 || LANES == 4 || LANES == 8 || LANES == 16, "row-sized groups only");
+    if constexpr (LANES >= 2) merge_top3_step<0xB1>(first, second, third);    // quad_perm [1,0,3,2]
+    if constexpr (LANES >= 4) merge_top3_step<0x4E>(first, second, third);    // quad_perm [2,3,0,1]
+    if constexpr (LANES >= 8) merge_top3_step<0x141>(first, second, third);   // row_half_mirror
+    if constexpr (LANES >= 16) merge_top3_step<0x140>(first, second, third);  // row_mirror
+}
+
 // FIXED names what the launch knows about the policy at compile time, so that the code of the other policies
 // is not part of the kernel: bit 0 "no outlier channel", bit 1 "round to nearest", bit 2 "linear codes".
 // 0 is the kernel for every policy.  EL: elements per lane, a multiple of 8 that divides G.
@@ -215,30 +248,30 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
         uint8_t *group_meta = a.compact ? group_codes + CB : a.payload + groups * CB + group * meta_bytes;
 
         uint32_t scale_raw;
+        Raw meta[4] = {0, 0, 0, 0};   // [scale][indices][top1][top2]
+        bool any_nan = true;   // "not known": the outlier path does not look
         if (topk == 0) {
-            scale_raw = running_max_raw<T, G, VEC>(mag, k0, start);
+            scale_raw = running_max_raw<T, G, VEC>(mag, k0, start, &any_nan);
         } else {
-            // Three rounds of "largest remaining candidate": the group maximum of the magnitude keys, then, among
-            // the elements that hold it, the maximum of the tie-break ranks (1..G, unique inside a group).
-            // A 16-bit magnitude and its rank share one 32-bit key, so a round is a single reduction there.
-            uint32_t key[VEC], rank[VEC];
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                const int pos = (k0 + i - start) & (G - 1);
-                const bool candidate = WIDE ? mag[i] <= RB::INF : (mag[i] != 0 && mag[i] <= RB::INF);
-                rank[i] = static_cast<uint32_t>(WIDE ? k0 + i + 1 : G - pos);     // the larger rank wins a tie
-                const uint32_t joined = WIDE ? mag[i] : ((mag[i] << 7) | (rank[i] - 1));
-                key[i] = candidate ? joined + 1 : 0;                              // 0 stands for "none"
-            }
+            // The three largest candidates of the group, a candidate's key being its magnitude and a tie-break rank
+            // (1..G, unique inside a group; the larger rank wins).
             uint32_t best_key[3] = {0, 0, 0}, best_rank[2] = {0, 0};              // magnitude + 1, rank
+            if constexpr (WIDE) {
+                // Three rounds of "largest remaining candidate": the group maximum of the magnitude keys, then, among
+                // the elements that hold it, the maximum of the ranks.
+                uint32_t key[VEC], rank[VEC];
 #pragma unroll
-            for (int round = 0; round < 3; ++round) {
-                if (round == 2 && topk == 1) break;                             // uniform
-                uint32_t m = 0;
+                for (int i = 0; i < VEC; ++i) {
+                    rank[i] = static_cast<uint32_t>(k0 + i + 1);
+                    key[i] = mag[i] <= RB::INF ? mag[i] + 1 : 0;                  // 0 stands for "none"
+                }
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) m = key[i] > m ? key[i] : m;
-                m = group_max_bits<LPG>(m);
-                if constexpr (WIDE) {
+                for (int round = 0; round < 3; ++round) {
+                    if (round == 2 && topk == 1) break;                         // uniform
+                    uint32_t m = 0;
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) m = key[i] > m ? key[i] : m;
+                    m = group_max_bits<LPG>(m);
                     best_key[round] = m;
                     if (round == 2) break;
                     uint32_t r = 0;
@@ -248,13 +281,47 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
                     r = m == 0 ? 0 : r;
                     best_rank[round] = r;
 #pragma unroll
-                    for (int i = 0; i < VEC; ++i) key[i] = (key[i] == m && rank[i] == r) ? 0 : key[i];   // taken
-                } else {
-                    best_key[round] = m == 0 ? 0 : ((m - 1) >> 7) + 1;
-                    if (round == 2) break;
-                    best_rank[round] = m == 0 ? 0 : ((m - 1) & 0x7Fu) + 1;
+                    for (int i = 0; i < VEC; ++i) key[i] = rank[i] == r ? 0 : key[i];   // taken (r = 0 matches nobody)
+                }
+            } else {
+                // A 16-bit magnitude and its rank share one 32-bit key, (magnitude << 7) + rank, unique inside the
+                // group.  A lane keeps the three largest of its own keys in order (three instructions an element), and
+                // the group's lanes merge their triples over the DPP butterfly (eight instructions a step): no rounds
+                // over the elements.  Zeros are no candidates: their keys are below 128, under every candidate's, and
+                // are dropped from the result.  NaNs are no candidates either and their keys are above every
+                // candidate's: the first pass does not look for them, and when one tops any group of the wavefront
+                // (rare) the pass is repeated with every element checked.  Scan positions do not wrap inside four
+                // adjacent elements (a lane's first element and the scan's start are multiples of four).
+                constexpr uint32_t kBelow = 128, kAbove = (RB::INF << 7) + G;
+                uint32_t largest, runner_up, bronze;
+                auto search = [&](const bool checked) __attribute__((always_inline)) {
+                    largest = runner_up = bronze = 0;
+                    const uint32_t p0 = static_cast<uint32_t>(k0 - start) & (G - 1);
 #pragma unroll
-                    for (int i = 0; i < VEC; ++i) key[i] = (key[i] == m && m != 0) ? 0 : key[i];          // taken
+                    for (int q = 0; q < VEC / 4; ++q) {
+                        const uint32_t rank0 = G - ((p0 + 4 * q) & (G - 1));      // rank = G - scan position
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int i = 4 * q + j;
+                            uint32_t key = (mag[i] << 7) + (rank0 - j);
+                            if (checked) key = (mag[i] - 1u) < RB::INF ? key : 0;
+                            bronze = umed3(runner_up, bronze, key);
+                            runner_up = umed3(largest, runner_up, key);
+                            largest = key > largest ? key : largest;
+                        }
+                    }
+                    merge_top3<LPG>(largest, runner_up, bronze);
+                };
+                search(false);
+                if (__ballot(largest > kAbove) != 0) search(true);   // wavefront-uniform
+                largest = largest < kBelow ? 0 : largest;
+                runner_up = runner_up < kBelow ? 0 : runner_up;
+                bronze = bronze < kBelow ? 0 : bronze;
+                const uint32_t found[3] = {largest, runner_up, bronze};
+#pragma unroll
+                for (int round = 0; round < 3; ++round) {   // rank 1..G <= 64 never carries into the magnitude
+                    best_key[round] = found[round] == 0 ? 0 : ((found[round] - 1) >> 7) + 1;
+                    if (round < 2) best_rank[round] = found[round] == 0 ? 0 : ((found[round] - 1) & 0x7Fu) + 1;
                 }
             }
             auto index_of = [&](uint32_t r) {
@@ -273,24 +340,20 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
                 index2 = none ? 1 : (lonely ? ((index1 + 1) & (G - 1)) : index_of(best_rank[1]));
                 scale_raw = (none || lonely || best_key[2] == 0) ? 0u : best_key[2] - 1;
             }
-            Raw top1_raw = 0, top2_raw = 0;
-            bool own1 = false, own2 = false;
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                const bool first = k0 + i == index1, second = k0 + i == index2;
-                top1_raw = first ? raw[i] : top1_raw;
-                top2_raw = second ? raw[i] : top2_raw;
-                own1 |= first;
-                own2 |= second;
-                if (first || second) v[i] = 0.0f;
+            for (int i = 0; i < VEC; ++i)
+                if (k0 + i == index1 || k0 + i == index2) v[i] = 0.0f;
+            // The outliers travel as they are stored.  The group's first lane fetches them from the tensor once more
+            // (its wavefront has just read those lines) instead of every lane selecting among its elements; the
+            // metadata words leave together at the end of the tile, when the values have long arrived.
+            meta[1] = static_cast<Raw>(topk == 1 ? index1 : (index1 | (index2 << 8)));
+            if (live && k0 == 0) {
+                const Raw *members = static_cast<const Raw *>(a.x) + group * G;
+                meta[2] = members[index1];
+                if (topk == 2) meta[3] = members[index2];
             }
-            if (live && own1) *reinterpret_cast<Raw *>(group_meta + 2 * ITEM) = top1_raw;   // the owner lanes store
-            if (live && own2) *reinterpret_cast<Raw *>(group_meta + 3 * ITEM) = top2_raw;   // the outliers as they are
-            if (live && k0 == 0)
-                *reinterpret_cast<Raw *>(group_meta + ITEM) =
-                    static_cast<Raw>(topk == 1 ? index1 : (index1 | (index2 << 8)));
         }
-        if (live && k0 == 0) *reinterpret_cast<Raw *>(group_meta) = static_cast<Raw>(scale_raw);
+        meta[0] = static_cast<Raw>(scale_raw);
 
         float scale = value_of<T>(scale_raw);
         scale = scale < 1.0e-6f ? 1.0e-6f : scale;   // a NaN scale stays NaN and encodes every element as 0
@@ -320,8 +383,12 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
             float t[VEC];
             const uint32_t scale_exponent = (as_u32(scale) >> 23) & 0xFFu;
             bool unusual = scale_exponent < 127u - 60u || scale_exponent > 127u + 60u;
+            // Without outliers the scale is the group's largest magnitude unless a NaN reset the running maximum, and
+            // the wavefront is known to hold no NaN: no element needs to be looked at.
+            if (any_nan) {   // wavefront-uniform
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) unusual |= !(__builtin_fabsf(v[i]) <= scale);
+                for (int i = 0; i < VEC; ++i) unusual |= !(__builtin_fabsf(v[i]) <= scale);
+            }
             const bool usual = __ballot(unusual) == 0;   // wavefront-uniform
             if (usual) {
                 float reciprocal = __builtin_amdgcn_rcpf(scale);
@@ -382,6 +449,18 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
             if constexpr (BIT == 8) pack_codes<T, 8, VEC, WORDS>(c, words);
             else pack_nibbles<T, EL>(c, words);
             store_words<WORDS, ITEM, kPlain>(group_codes + k0 * BIT / 8, words);
+        }
+        if (live && k0 == 0) {
+            Raw *words = reinterpret_cast<Raw *>(group_meta);
+            if (topk == 2) {
+                store_elems<Raw, 4, kPlain>(words, meta);
+            } else if (topk == 1) {
+                const Raw pair[2] = {meta[0], meta[1]};
+                store_elems<Raw, 2, kPlain>(words, pair);
+                words[2] = meta[2];
+            } else {
+                words[0] = meta[0];
+            }
         }
     }
 }

@@ -270,19 +270,18 @@ template <typename T, int G> __device__ __forceinline__ int scan_start(int64_t g
 // the next element replaces the NaN, so the result is the maximum of what follows the group's last NaN, or that
 // NaN when it ends the scan.  `mag` are the magnitude bits of the lane's elements as stored, `k0` the lane's
 // first element inside its group, `start` the element the scan begins at.  Returns the scale as stored.
+// `any_nan` (optional) receives whether any lane of the wavefront holds a NaN.
 template <typename T, int G, int VEC>
-__device__ __forceinline__ uint32_t running_max_raw(const uint32_t (&mag)[VEC], int k0, int start) {
+__device__ __forceinline__ uint32_t running_max_raw(const uint32_t (&mag)[VEC], int k0, int start, bool *any_nan = nullptr) {
     constexpr int LPG = G / VEC;
     using RB = raw_bits<T>;
+    // A NaN's magnitude bits lie above those of every number, so the lane's plain maximum says whether it holds one.
     uint32_t m = 0;
-    bool has_nan = false;
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-        const bool nan = mag[i] > RB::INF;
-        has_nan |= nan;
-        m = (!nan && mag[i] > m) ? mag[i] : m;
-    }
-    if (__ballot(has_nan) != 0) {   // wavefront-uniform, rare
+    for (int i = 0; i < VEC; ++i) m = mag[i] > m ? mag[i] : m;
+    const bool nans = __ballot(m > RB::INF) != 0;   // wavefront-uniform, rare
+    if (any_nan) *any_nan = nans;
+    if (nans) {
         uint32_t last = 0;          // 1 + scan position of the group's last NaN
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
