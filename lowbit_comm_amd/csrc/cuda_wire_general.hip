@@ -152,7 +152,7 @@ template <int LANES> __device__ __forceinline__ void merge_top3(uint32_t &first,
 // FIXED names what the launch knows about the policy at compile time, so that the code of the other policies
 // is not part of the kernel: bit 0 "no outlier channel", bit 1 "round to nearest", bit 2 "linear codes".
 // 0 is the kernel for every policy.  EL: elements per lane, a multiple of 8 that divides G.
-template <typename T, int G, int BIT, int FIXED, int EL>
+template <typename T, int G, int BIT, int FIXED, int EL, int TILES>
 __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGeneralQuantArgs a) {
     const int topk = (FIXED & 1) ? 0 : a.topk;
     const bool stochastic = (FIXED & 2) ? false : a.stochastic != 0;
@@ -167,14 +167,16 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     const int lane = threadIdx.x & (kWave - 1);
     const int meta_bytes = meta_words_of(topk) * ITEM;
     const int64_t groups = a.numel / G;
-    const int64_t first = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * (kWave * EL);
+    constexpr int TILE = kWave * EL;
+    const int64_t first = (static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + (threadIdx.x >> 6)) * (TILES * TILE);
 
-    // all of the lane's elements are asked for before anything else
-    Raw raw[VEC];
+    // all of the wavefront's elements are asked for before anything else
+    Raw raws[TILES][VEC];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) raw[i] = 0;
-    {
-        const int64_t e0 = first + lane * VEC;
+    for (int tile = 0; tile < TILES; ++tile) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) raws[tile][i] = 0;
+        const int64_t e0 = first + tile * TILE + lane * VEC;
         // numel is a multiple of G: dead lanes form whole dead groups.  Instruction-bound: a cache hint only costs.
         if (e0 < a.numel) {
 #pragma unroll
@@ -182,7 +184,7 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
                 Raw piece[W::VEC];
                 load_elems<Raw, W::VEC, kPlain>(static_cast<const Raw *>(a.x) + e0 + part * W::VEC, piece);
 #pragma unroll
-                for (int i = 0; i < W::VEC; ++i) raw[part * W::VEC + i] = piece[i];
+                for (int i = 0; i < W::VEC; ++i) raws[tile][part * W::VEC + i] = piece[i];
             }
         }
     }
@@ -193,8 +195,8 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
     if (first >= a.numel) return;   // wavefront-uniform, behind the workgroup's barrier
     const float *book = wave_code_book(kind, lane);
 
-    {
-        const int64_t e0 = first + lane * VEC;
+    auto encode_tile = [&](const int64_t tile_first, const Raw (&raw)[VEC]) __attribute__((always_inline)) {
+        const int64_t e0 = tile_first + lane * VEC;
         const bool live = e0 < a.numel;
         const int64_t group = e0 / G;
         const int k0 = static_cast<int>(e0 - group * G);
@@ -462,6 +464,12 @@ __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGe
                 words[0] = meta[0];
             }
         }
+    };
+#pragma unroll
+    for (int tile = 0; tile < TILES; ++tile) {
+        const int64_t tile_first = first + tile * TILE;
+        if (tile_first >= a.numel) return;   // wavefront-uniform
+        encode_tile(tile_first, raws[tile]);
     }
 }
 
@@ -545,13 +553,13 @@ __global__ __launch_bounds__(kBlock) void wire_general_decode_kernel(const WireG
     store_elems<Raw, VEC, kNonTemporal>(out, decoded);
 }
 
-template <typename T, int G, int BIT, int FIXED, int EL>
+template <typename T, int G, int BIT, int FIXED, int EL, int TILES = 1>
 hipError_t launch_general_quant_as(const WireGeneralQuantArgs &a, hipStream_t stream) {
-    const int64_t tile = static_cast<int64_t>(kWave) * EL * kWavesPerBlock;
+    const int64_t tile = static_cast<int64_t>(kWave) * EL * kWavesPerBlock * TILES;
     const int64_t blocks = (a.numel + tile - 1) / tile;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((wire_general_quant_kernel<T, G, BIT, FIXED, EL>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0,
+    hipLaunchKernelGGL((wire_general_quant_kernel<T, G, BIT, FIXED, EL, TILES>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0,
                        stream, a);
     return hipGetLastError();
 }
@@ -564,9 +572,10 @@ hipError_t launch_general_quant_g(int bit, const WireGeneralQuantArgs &a, hipStr
     //
     // 32 bytes a lane against 16 (26.2 M elements, group 64, us): fp32 top-2 27.4 / 30.5, stochastic 24.3 / 26.6,
     // a code book 25.5 / 27.9; bf16 top-2 22.1 / 23.3, stochastic 21.5 / 22.6, a code book through the cell table
-    // 19.8 / 19.3 - the one case that keeps 16 bytes.
+    // 19.8 / 19.3 - the one case that keeps 16 bytes, and the one case that gains from two such tiles a wavefront,
+    // both asked for before either is encoded (18.2 against 19.4 us; the others lose 8-20 % with two tiles).
     constexpr int WIDE = general_quant_elems<T>() <= G ? general_quant_elems<T>() : G;
-    constexpr int CELLS = sizeof(T) == 4 ? WIDE : 8;
+    constexpr int CELLS = sizeof(T) == 4 ? WIDE : 8, CELL_TILES = sizeof(T) == 4 ? 1 : 2;
     const int fixed = a.stochastic ? 0 : ((a.topk == 0 ? 1 : 0) | 2 | (a.kind == 0 ? 4 : 0));
     if (bit != 8 && bit != 4) return hipErrorNotSupported;
     if (bit == 8 && a.kind != 0) return hipErrorNotSupported;   // eight bits: linear codes only
@@ -575,7 +584,7 @@ hipError_t launch_general_quant_g(int bit, const WireGeneralQuantArgs &a, hipStr
         return launch_general_quant_as<T, G, 8, 0, WIDE>(a, stream);
     }
     if (fixed == 2 || fixed == 6) return launch_general_quant_as<T, G, 4, 2, WIDE>(a, stream);
-    if (fixed == 3) return launch_general_quant_as<T, G, 4, 3, CELLS>(a, stream);
+    if (fixed == 3) return launch_general_quant_as<T, G, 4, 3, CELLS, CELL_TILES>(a, stream);
     return launch_general_quant_as<T, G, 4, 0, WIDE>(a, stream);
 }
 
