@@ -222,8 +222,8 @@ int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *sca
  * `restored` and `prepared`), lbc_dequant_reduce_quant, lbc_dequant_chunks - with the same meaning and
  * the same validation; a NULL stage is absent, and a stage with nothing to do (numel == 0) counts as
  * absent.  Results are bit-identical to those calls in any order.  Nothing orders the stages inside the
- * launch: no stage may read or write what another writes (decoding bucket k-2 in place is fine, its
- * quantize ran two launches earlier).
+ * launch: no stage may read or write what another writes (LBC_EINVAL otherwise; decoding bucket k-2 in
+ * place is fine, its quantize ran two launches earlier).
  *
  * With one stage present its own kernel runs.  With two or three: LBC_UNSUPPORTED - issue the calls
  * yourself - unless group_size is 64, every operand is aligned for the vector kernels (16 bytes for

@@ -468,6 +468,41 @@ int lbc_bucket_pipeline_step(const lbc_quant_chunks_stage *quant, const lbc_redu
     }
     const int stages = (q.empty ? 0 : 1) + (r.empty ? 0 : 1) + (d.empty ? 0 : 1);
     if (stages == 0) return LBC_OK;
+    if (stages > 1) {
+        // Nothing orders the stages inside the launch: what one writes, no other may read or write.
+        struct Span { const char *low, *high; int stage; bool written; };
+        Span spans[24];
+        int count = 0;
+        auto add = [&](const void *p, int64_t bytes, int stage, bool written) {
+            if (p != nullptr && bytes > 0) spans[count++] = {static_cast<const char *>(p), static_cast<const char *>(p) + bytes, stage, written};
+        };
+        const int64_t groups_of_r = r.empty ? 0 : (reduce->numel + group_size - 1) / group_size;
+        auto payload_bytes = [&](int64_t numel) { return (numel + group_size - 1) / group_size * (group_size + 4); };
+        if (!q.empty) {
+            add(quant->x, quant->numel * dtype_size(quant->x_dtype), 0, false);
+            if (quant->residual != nullptr) add(quant->residual, quant->numel * dtype_size(quant->residual_dtype), 0, false);
+            add(quant->payloads, (quant->world - 1) * quant->payload_stride + payload_bytes((quant->numel + quant->world - 1) / quant->world), 0, true);
+            if (quant->new_residual != nullptr) add(quant->new_residual, quant->numel * dtype_size(quant->new_residual_dtype), 0, true);
+        }
+        if (!r.empty) {
+            for (int i = 0; i < reduce->world; ++i) {
+                add(reduce->codes[i], reduce->numel, 1, false);
+                add(reduce->scales[i], groups_of_r * 4, 1, false);
+            }
+            add(reduce->out_codes, groups_of_r * group_size, 1, true);
+            add(reduce->out_scales, groups_of_r * 4, 1, true);
+        }
+        if (!d.empty) {
+            add(decode->payloads, (decode->world - 1) * decode->payload_stride + payload_bytes(decode->shard_numel), 2, false);
+            add(decode->out, decode->total_numel * dtype_size(decode->out_dtype), 2, true);
+        }
+        for (int i = 0; i < count; ++i) {
+            if (!spans[i].written) continue;
+            for (int j = 0; j < count; ++j)
+                if (spans[i].stage != spans[j].stage && spans[i].low < spans[j].high && spans[j].low < spans[i].high)
+                    return fail(LBC_EINVAL, "a stage writes memory that another stage of the same launch reads or writes");
+        }
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (stages == 1) {          // one stage with work: its own kernel
         if (!q.empty) return launch_quant(q, "lbc_bucket_pipeline_step", access, stream);

@@ -39,13 +39,13 @@ import torch
 
 from lowbit_comm_amd.config import CompressionConfig
 from lowbit_comm_amd.hip import ops
-from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan
+from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan, ResidualStore
 
 
 class _Bucket:
     """One bucket in flight: its plan (send / received / gathered rows), tensors, future and pending exchanges."""
 
-    __slots__ = ("plan", "tensor", "out", "op", "future", "exchange", "gather", "result", "lane", "lasting_out")
+    __slots__ = ("plan", "tensor", "out", "op", "future", "exchange", "gather", "result", "lane", "lasting_out", "spans")
 
     def __init__(self, plan: ReduceScatterPlan, tensor: torch.Tensor, out: torch.Tensor | None, op: str, future: Any,
                  lane: int, lasting_out: bool) -> None:
@@ -59,6 +59,12 @@ class _Bucket:
         self.gather: Any | None = None        # work object of the all-gather, if it returned one
         self.result: Any | None = None
         self.lane = lane
+        self.spans = (_span(tensor), _span(out))   # byte ranges this bucket reads and writes while it is in flight
+
+
+def _span(tensor: torch.Tensor) -> tuple[int, int]:
+    start = tensor.data_ptr()
+    return start, start + tensor.numel() * tensor.element_size()
 
 
 def _wait_for(work: Any) -> None:
@@ -92,7 +98,8 @@ class BucketPipeline:
     contiguous, else into a fresh tensor.
 
     ``error_feedback``: every bucket (keyed by storage address, element count and dtype) keeps an fp32 residual that
-    its quantize adds before encoding and refreshes, in the same launch, with what the encoding dropped.
+    its quantize adds before encoding and refreshes, in the same launch, with what the encoding dropped; beyond
+    ``max_residuals`` buckets the least recently used residual is dropped.
 
     ``lanes`` > 1 deals the buckets to that many streams of default priority in turn, each with its own buckets in
     flight: the ramp-up of one bucket's launch overlaps the drain of the one before.  A lane waits for the caller's
@@ -107,7 +114,7 @@ class BucketPipeline:
                  all_gather: Callable[[torch.Tensor, torch.Tensor], Any] | None = None, error_feedback: bool = False,
                  inplace: bool = True, lanes: int = 1, max_plans: int = 64, max_steps: int = 4096,
                  future_factory: Callable[[], Any] | None = None, plan_factory: Callable[..., Any] | None = None,
-                 merge_stages: Callable[..., Any] | None = None) -> None:
+                 merge_stages: Callable[..., Any] | None = None, max_residuals: int = 4096) -> None:
         if not 0 <= rank < world_size:
             raise ValueError(f"rank must be in [0, {world_size})")
         if lanes < 1:
@@ -121,7 +128,7 @@ class BucketPipeline:
         self.depth = 3 if all_gather is not None else 2
         self.max_plans = max_plans
         self.max_steps = max_steps
-        self.residuals: dict[Any, torch.Tensor] = {}
+        self.residuals = ResidualStore(max_residuals)
         self.stats = {"buckets": 0, "merged_launches": 0, "separate_launches": 0, "flushes": 0}
         self._future_factory = future_factory
         self._plan_factory = plan_factory or ReduceScatterPlan     # replaceable: the scheduling is testable without a GPU
@@ -163,13 +170,20 @@ class BucketPipeline:
         return self._lanes
 
     def _residual_for(self, tensor: torch.Tensor) -> torch.Tensor | None:
-        if not self.error_feedback:
-            return None
-        key = (tensor.data_ptr(), tensor.numel(), tensor.dtype)
-        residual = self.residuals.get(key)
-        if residual is None:
-            residual = self.residuals[key] = torch.zeros(tensor.numel(), dtype=torch.float32, device=tensor.device)
-        return residual
+        return self.residuals.for_tensor(tensor) if self.error_feedback else None
+
+    def _touches_a_bucket_in_flight(self, tensor: torch.Tensor, out: torch.Tensor) -> bool:
+        mine = None
+        for lane in self._lanes or ():
+            for bucket in (lane.reduce_next, lane.decode_next):
+                if bucket is None:
+                    continue
+                if mine is None:
+                    mine = (_span(tensor), _span(out))
+                for low, high in bucket.spans:
+                    if any(low < b and a < high for a, b in mine):
+                        return True
+        return False
 
     def _plan_for(self, tensor: torch.Tensor, config: CompressionConfig, lane: int) -> ReduceScatterPlan:
         key = (tensor.numel(), tensor.dtype, tensor.device, config.bit, config.group_size, config.topk,
@@ -303,6 +317,12 @@ class BucketPipeline:
                     out = torch.empty(plan.chunks.shard_numel, dtype=plan.reduced_dtype, device=tensor.device)
                 elif out.numel() != plan.chunks.shard_numel or out.dtype != plan.reduced_dtype:
                     raise ValueError("out does not match this rank's shard")
+            if self._touches_a_bucket_in_flight(tensor, out):
+                # The same memory again before its earlier bucket has been decoded (not a DDP iteration, where every
+                # bucket is handed over once): finish the earlier one first, so that this quantize reads its result
+                # and no launch both reads and writes the tensor.
+                self.flush()
+                plan = self._plan_for(tensor, config, index)
             bucket = _Bucket(plan, tensor, out, op, future, index, lasting_out)
             self._dirty = True
             residual = self._residual_for(tensor)
@@ -335,7 +355,6 @@ class BucketPipeline:
                 return
             if not self._dirty:
                 return
-            self._dirty = False
             self._turn.clear()
             self._next_lane = 0
             self.stats["flushes"] += 1
@@ -352,6 +371,7 @@ class BucketPipeline:
                 finally:
                     torch.cuda.set_stream(current)
                 current.wait_stream(lane.stream)
+            self._dirty = False                   # only now: a flush that raised half-way is retried by the next one
 
 
 class _FlushingFuture(torch.futures.Future):

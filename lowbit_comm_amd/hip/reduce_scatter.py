@@ -436,12 +436,37 @@ def compressed_all_reduce_async(tensor: torch.Tensor, *, config: CompressionConf
     return manager.create_work(result=result, completion=stream_work, resources=(tensor, plan, result, residual))
 
 
+class ResidualStore(OrderedDict):
+    """fp32 error-feedback residuals of a transport, one per bucket, keyed by the bucket's storage address, element
+    count and dtype (a DDP bucket comes back at the same address every iteration).  Bounded: beyond ``max_entries`` the
+    least recently used residual is dropped, and a bucket that returns after that starts from zero again - a caller
+    that hands over fresh tensors every step would otherwise grow the store by one bucket-sized tensor per call."""
+
+    def __init__(self, max_entries: int = 4096) -> None:
+        super().__init__()
+        if max_entries < 1:
+            raise ValueError("max_entries must be at least 1")
+        self.max_entries = max_entries
+
+    def for_tensor(self, tensor: torch.Tensor) -> torch.Tensor:
+        key = (tensor.data_ptr(), tensor.numel(), tensor.dtype)
+        residual = self.get(key)
+        if residual is None:
+            residual = self[key] = torch.zeros(tensor.numel(), dtype=torch.float32, device=tensor.device)
+            while len(self) > self.max_entries:
+                self.popitem(last=False)
+        else:
+            self.move_to_end(key)
+        return residual
+
+
 def make_reduce_scatter_transport(*, world_size: int, rank: int,
                                   all_to_all: Callable[[torch.Tensor, torch.Tensor], None],
                                   all_gather: Callable[[torch.Tensor, torch.Tensor], None],
                                   max_plans: int = 64, manager: Any | None = None,
                                   inplace: bool = True, error_feedback: bool = False, pipelined: bool = False,
-                                  lanes: int = 1, future_factory: Callable[[], Any] | None = None) -> Callable[..., Any]:
+                                  lanes: int = 1, future_factory: Callable[[], Any] | None = None,
+                                  max_residuals: int = 4096) -> Callable[..., Any]:
     """The callable ``create_ddp_comm_hook(reduce_scatter_all_gather=...)`` expects, over pre-bound plans.
 
     ``transport(tensor, *, config, op, async_op=False, dtype=None, extension_status=None)`` runs the compressed
@@ -453,7 +478,8 @@ def make_reduce_scatter_transport(*, world_size: int, rank: int,
     With ``error_feedback`` every bucket (keyed by its storage address and size) keeps an fp32 residual that the
     quantize launch adds before encoding and refreshes with what the encoding dropped, in the same launch - the
     local error feedback of ``DDPBucketProcessor`` (``ccdl_comm/communication/ddp.py:69-97``); ``transport.residuals``
-    exposes them, ``transport.reset()`` drops them.  Counterpart of ``compressed_reduce_scatter_all_gather``
+    exposes them (a :class:`ResidualStore`: the least recently used one is dropped beyond ``max_residuals``),
+    ``transport.reset()`` drops them.  Counterpart of ``compressed_reduce_scatter_all_gather``
     (``ccdl_comm/communication/reduce_scatter_transport.py:186-377``) with the exchanges injected.
 
     ``pipelined``: the buckets go through a :class:`~lowbit_comm_amd.hip.bucket_pipeline.BucketPipeline` - one launch
@@ -465,19 +491,15 @@ def make_reduce_scatter_transport(*, world_size: int, rank: int,
     if pipelined and world_size <= ops.MAX_PAYLOADS:
         return _pipelined_transport(world_size=world_size, rank=rank, all_to_all=all_to_all, all_gather=all_gather,
                                     max_plans=max_plans, manager=manager, inplace=inplace, error_feedback=error_feedback,
-                                    lanes=lanes, future_factory=future_factory)
+                                    lanes=lanes, future_factory=future_factory, max_residuals=max_residuals)
 
     plans: OrderedDict = OrderedDict()
-    residuals: dict = {}
+    residuals = ResidualStore(max_residuals)
 
     def residual_for(tensor: torch.Tensor) -> torch.Tensor | None:
         if not error_feedback or tensor.numel() == 0:
             return None
-        key = (tensor.data_ptr(), tensor.numel(), tensor.dtype)
-        residual = residuals.get(key)
-        if residual is None:
-            residual = residuals[key] = torch.zeros(tensor.numel(), dtype=torch.float32, device=tensor.device)
-        return residual
+        return residuals.for_tensor(tensor)
 
     def plan_for(tensor: torch.Tensor, config: CompressionConfig) -> ReduceScatterPlan:
         key = (tensor.numel(), tensor.dtype, tensor.device, config.bit, config.group_size, config.topk,
@@ -518,12 +540,12 @@ def make_reduce_scatter_transport(*, world_size: int, rank: int,
 
 def _pipelined_transport(*, world_size: int, rank: int, all_to_all: Callable[..., Any], all_gather: Callable[..., Any],
                          max_plans: int, manager: Any | None, inplace: bool, error_feedback: bool, lanes: int,
-                         future_factory: Callable[[], Any] | None) -> Callable[..., Any]:
+                         future_factory: Callable[[], Any] | None, max_residuals: int) -> Callable[..., Any]:
     from lowbit_comm_amd.hip.bucket_pipeline import BucketPipeline
 
     pipeline = BucketPipeline(world_size=world_size, rank=rank, all_to_all=all_to_all, all_gather=all_gather,
                               error_feedback=error_feedback, inplace=inplace, lanes=lanes, max_plans=max_plans,
-                              future_factory=future_factory)
+                              future_factory=future_factory, max_residuals=max_residuals)
     unpipelined = make_reduce_scatter_transport(world_size=world_size, rank=rank, all_to_all=all_to_all,
                                                 all_gather=all_gather, max_plans=max_plans, manager=manager,
                                                 inplace=inplace, error_feedback=False)

@@ -225,6 +225,65 @@ def test_error_feedback_residuals_are_kept_per_bucket_and_dropped_by_reset():
     assert pipe.residuals == {}
 
 
+def test_residual_store_is_bounded_and_drops_the_least_recently_used():
+    log = []
+    pipe = make_pipeline(log, error_feedback=True, max_residuals=2)
+    a, b, c = bucket_tensor(0), bucket_tensor(1), bucket_tensor(2)
+    key = lambda t: (t.data_ptr(), t.numel(), t.dtype)
+    pipe.submit(a, config=CFG)
+    pipe.submit(b, config=CFG)
+    first_a = pipe.residuals[key(a)]
+    pipe.submit(a, config=CFG)                       # a is the most recently used now
+    pipe.submit(c, config=CFG)                       # ... so b's residual is the one that goes
+    pipe.flush()
+    assert set(pipe.residuals) == {key(a), key(c)}
+    assert pipe.residuals[key(a)] is first_a         # a residual that stays is the same tensor, not a new zero one
+    with pytest.raises(ValueError, match="max_entries"):
+        make_pipeline(log, error_feedback=True, max_residuals=0)
+
+
+def test_the_same_memory_again_while_in_flight_finishes_the_earlier_bucket_first():
+    log = []
+    pipe = make_pipeline(log)
+    a, b = bucket_tensor(0), bucket_tensor(1)
+    first = pipe.submit(a, config=CFG)
+    pipe.submit(b, config=CFG)
+    assert not first.done()
+    again = pipe.submit(a, config=CFG)               # would be quantized while its earlier result is decoded into it
+    assert first.done() and not again.done() and pipe.pending == 1
+    decodes = [i for i, entry in enumerate(log) if entry[0] == "D" or (entry[0] == "MERGED" and any(p[0] == "D" for p in entry[1:]))]
+    quantizes = [i for i, entry in enumerate(log) if entry == ("Q", 0, False)]
+    assert len(quantizes) == 2 and max(decodes) < quantizes[1]    # every earlier decode precedes the second quantize
+    view = a[:320]                                    # an overlapping view counts as the same memory
+    view.bucket_id = 2
+    pipe.submit(view, config=CFG)
+    assert again.done()
+    pipe.flush()
+
+
+def test_a_flush_that_raised_is_retried_by_the_next_one():
+    log = []
+    pipe = make_pipeline(log)
+    failures = [RuntimeError("link down")]
+    inner = pipe.all_gather
+
+    def flaky_all_gather(gathered, mine):
+        if failures:
+            raise failures.pop()
+        return inner(gathered, mine)
+
+    futures = [pipe.submit(bucket_tensor(k), config=CFG) for k in range(2)]
+    pipe.all_gather = flaky_all_gather               # the first exchange of the flush fails
+    with pytest.raises(RuntimeError, match="link down"):
+        pipe.flush()
+    assert pipe.pending == 2 and not any(f.done() for f in futures)
+    pipe.flush()                                     # the stages of the failed step go out again, then the rest
+    assert pipe.pending == 0 and all(f.done() for f in futures)
+    issued = len(log)
+    pipe.flush()                                     # nothing is left: nothing is issued
+    assert len(log) == issued
+
+
 def test_empty_buckets_complete_at_once_and_invalid_requests_are_refused():
     log = []
     pipe = make_pipeline(log)

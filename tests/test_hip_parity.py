@@ -873,6 +873,27 @@ def test_pipeline_step_without_a_shared_grid_says_so(ops, hip_device):
         ops.bind_bucket_pipeline_step(quant, quant)
 
 
+def test_pipeline_step_refuses_stages_that_write_into_each_other(ops, hip_device):
+    """Nothing orders the stages inside the launch, so a stage that writes what another reads or writes is an error."""
+    world, n = 8, 64 * 8 * 40
+    shard = n // world
+    nbytes = ops.payload_nbytes(shard)
+    grad = gradient_like(n, torch.float32, 11, hip_device)
+    send = torch.zeros(world, nbytes, dtype=torch.uint8, device=hip_device)
+    gathered = torch.zeros(world, nbytes, dtype=torch.uint8, device=hip_device)
+    mine = torch.zeros(nbytes, dtype=torch.uint8, device=hip_device)
+    pairs = [ops.split_payload(send[r], shard) for r in range(world)]           # the reduce reads what the quantize writes
+    quant = ops.bind_quant_pack_chunks(grad, send, world)
+    reduce = ops.bind_dequant_reduce_quant(pairs, *ops.split_payload(mine, shard), shard)
+    with pytest.raises(RuntimeError, match="another stage of the same launch"):
+        ops.bind_bucket_pipeline_step(quant, reduce)()
+    decode_into_the_input = ops.bind_dequant_chunks(gathered, grad, shard)      # the decode writes what the quantize reads
+    with pytest.raises(RuntimeError, match="another stage of the same launch"):
+        ops.bind_bucket_pipeline_step(quant, None, decode_into_the_input)()
+    elsewhere = torch.zeros(n, device=hip_device)
+    assert ops.bind_bucket_pipeline_step(quant, None, ops.bind_dequant_chunks(gathered, elsewhere, shard))() is True
+
+
 def test_bucket_steps_dealt_to_two_streams_in_turn_equal_the_one_stream_schedule(ops, hip_device):
     """Consecutive buckets are independent: their launches (quantize of bucket k + reduce of bucket k-1) may alternate
     between two streams, each with its own send matrix and shard output, and must leave the same residuals, payloads
