@@ -474,6 +474,14 @@ int main() {
         decode_stage.out = d_decoded;
         decode_stage.out_dtype = LBC_F32;
         LBC_OK_OR_FAIL(lbc_bucket_pipeline_step(&quant_stage, &reduce_stage, &decode_stage, g, LBC_ACCESS_AUTO, stream));
+        // a decode into the tensor the quantize reads: the stages of one launch are not ordered, so this is refused
+        lbc_dequant_chunks_stage clash = decode_stage;
+        clash.out = d_x;
+        if (lbc_bucket_pipeline_step(&quant_stage, nullptr, &clash, g, LBC_ACCESS_AUTO, stream) != LBC_EINVAL) {
+            printf("FAIL pipeline step: stages that write into each other were not refused\n");
+            return 13;
+        }
+        ++checks;
     }
     HIP_OK(hipMemcpyAsync(rows.data(), d_rows, world * even_stride, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipMemcpyAsync(send_codes.data(), d_send_codes, reduce_n, hipMemcpyDeviceToHost, stream));

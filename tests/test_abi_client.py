@@ -28,7 +28,7 @@ def test_client_runs_every_entry_point_bit_exact_against_the_c_oracles(hip_devic
     done = subprocess.run([str(CLIENT)], capture_output=True, text=True, timeout=120)
     assert done.returncode == 0, (done.stdout, done.stderr[-2000:])
     assert done.stdout.strip().startswith("OK "), done.stdout
-    assert int(done.stdout.split()[1]) == 62
+    assert int(done.stdout.split()[1]) == 63
 
 
 @pytest.mark.gpu
