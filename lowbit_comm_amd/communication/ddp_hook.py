@@ -321,7 +321,8 @@ def create_ddp_comm_hook(
 
         def process_bucket(bucket: Any) -> Any:
             tensor = bucket.buffer()
-            last = callable(flush) and callable(getattr(bucket, "is_last", None)) and bucket.is_last()
+            # a bucket object that cannot say whether it is the last one is treated as the last: correct, unpipelined
+            last = callable(flush) and (not callable(getattr(bucket, "is_last", None)) or bucket.is_last())
             if small(tensor):
                 if last:
                     flush()

@@ -381,6 +381,35 @@ def test_hook_flushes_a_pipelined_transport_after_the_last_bucket():
     assert calls == []
 
 
+def test_hook_flushes_after_every_bucket_that_cannot_say_whether_it_is_the_last():
+    """DistributedDataParallel waits for a hook's futures where a Python override of wait() is not seen: a bucket
+    object without is_last() must not leave its future behind in the pipeline."""
+    log = []
+    pipe = make_pipeline(log)
+
+    def transport(tensor, *, config, op, async_op, dtype, extension_status):
+        return pipe.submit(tensor, config=config, op=op)
+
+    transport.pipelined = True
+    transport.flush = pipe.flush
+
+    class Anonymous:
+        def __init__(self, tensor, index):
+            self._tensor, self._index = tensor, index
+
+        def buffer(self):
+            return self._tensor
+
+        def index(self):
+            return self._index
+
+    hook = create_ddp_comm_hook(CFG, strategy="reduce_scatter", reduce="mean", reduce_scatter_all_gather=transport,
+                                dtype="fp32")
+    for k in range(3):
+        assert hook(None, Anonymous(bucket_tensor(k), k)).done() and pipe.pending == 0
+    assert pipe.stats["flushes"] == 3
+
+
 def test_hook_flushes_when_the_last_bucket_is_too_small_to_compress():
     log = []
     pipe = make_pipeline(log)
