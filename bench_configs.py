@@ -1119,6 +1119,15 @@ def main() -> int:
                          f"{feedback}, per bucket", host / stream_count, wall / stream_count,
                          merged_launches_per_bucket=stats["merged_launches"] / stats["buckets"],
                          separate_launches_per_bucket=stats["separate_launches"] / stats["buckets"])
+                # the same iteration - every bucket through the hook, the exchanges, the flush - as one HIP-graph replay
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    one_iteration()
+                host, wall = host_and_wall(lambda i: graph.replay(), 12)
+                host_row(f"the same iteration ({lane_count} stream{'s' if lane_count > 1 else ''}, error feedback {feedback}) "
+                         "as one HIP-graph replay, per bucket", host / stream_count, wall / stream_count)
+                del graph
         del stream_buckets
         # one pre-bound launch
         x = gen(SEED + 7100, n, 1e-3, torch.bfloat16)

@@ -251,3 +251,55 @@ def test_hook_with_the_pipelined_transport_on_a_stream_of_buckets(hip_device):
         for k, (future, want) in enumerate(zip(futures, wanted)):
             assert same_bits(future.wait(), want), f"bucket {k}, step {step}"
     assert piped.pipeline.stats["flushes"] == 2
+
+
+@pytest.mark.parametrize("error_feedback", [False, True])
+@pytest.mark.parametrize("lanes", [1, 2])
+def test_an_iteration_of_the_pipeline_captured_in_a_hip_graph_replays_like_eager(hip_device, error_feedback, lanes):
+    """No entry point allocates, clears memory or synchronises, so one iteration of the pipelined stream - every
+    bucket's launch, the exchanges, the flush, with two lanes the forks and joins of their streams - can be captured
+    once and replayed.  Every replay, with the program's own eager work and synchronisations in between, must leave what
+    an eager iteration leaves from the same state."""
+    world, count = 8, 6
+    sizes = [G * world * 48] * 4 + [G * world * 20, G * world * 48]
+    piped, _plain = transports(world, error_feedback=error_feedback, lanes=lanes)
+    source = [grad(n, torch.bfloat16, 9100 + k, hip_device) for k, n in enumerate(sizes)]
+    buckets = [s.clone() for s in source]
+
+    def restore():
+        for bucket, s in zip(buckets, source):
+            bucket.copy_(s)
+        for residual in piped.residuals.values():
+            residual.zero_()
+
+    def iteration():
+        for bucket in buckets:
+            piped(bucket, config=CFG, op="mean")
+        piped.flush()
+
+    for _ in range(2):                    # plans, bound launches, residuals and lane streams exist before the capture
+        iteration()
+    restore()
+    iteration()
+    torch.cuda.synchronize()
+    want = [bucket.clone() for bucket in buckets]
+    want_residuals = [r.clone() for r in piped.residuals.values()]
+    assert len(want_residuals) == (count if error_feedback else 0)
+    restore()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        iteration()
+    for replay in range(4):
+        restore()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for k, (bucket, expected) in enumerate(zip(buckets, want)):
+            assert same_bits(bucket, expected), f"bucket {k}, replay {replay}"
+        for k, (residual, expected) in enumerate(zip(piped.residuals.values(), want_residuals)):
+            assert same_bits(residual, expected), f"residual {k}, replay {replay}"
+        # eager work of the same program between the replays: an iteration outside the graph, and a host read-back
+        restore()
+        iteration()
+        assert same_bits(buckets[0], want[0])
