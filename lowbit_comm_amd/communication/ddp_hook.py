@@ -276,6 +276,9 @@ def create_ddp_comm_hook(
     # and no allocation of its own: the sum lands in a cached workspace and the payload in a cached buffer, both
     # under the budgets of the decode workspaces.
     fuse_compensate = quantize is None and writes_prepared(extension_status)
+    # Same condition for keeping a bucket's payload buffer from one iteration to the next: a DDP iteration is over
+    # (its futures waited for) before the bucket comes back, so the gather has long read the payload.
+    reuse_payload_buffers = fuse_compensate
     prepared_workspaces = DequantizedWorkspaceCache(
         allocator=allocate_dequantized_buffer, max_entries=workspace_cache_max_entries,
         max_cached_bytes=workspace_cache_max_bytes)
@@ -415,8 +418,16 @@ def create_ddp_comm_hook(
                                                            min_numel=fuse_payload_min_numel) else plain_gather)
             if facade:
                 # facade path: flat uint8 buffers, fused decode+reduce (+ residual update) on the GPU
-                local = coerce_payload(fused[1] if fused is not None else active_quantize(prepared, config),
-                                       shape=shape, dtype=active_dtype)
+                if fused is not None:
+                    packed = fused[1]
+                elif reuse_payload_buffers and getattr(prepared, "is_cuda", False) and prepared.is_contiguous():
+                    # the bucket's payload goes into the buffer its key had last iteration: nothing is allocated and
+                    # the native module meets the addresses it has bound launches for
+                    packed = quantize_tensor(prepared, config, extension_status=extension_status,
+                                             output=payload_buffers.get(key, prepared, shape, config))
+                else:
+                    packed = active_quantize(prepared, config)
+                local = coerce_payload(packed, shape=shape, dtype=active_dtype)
                 needs_feedback = decision.apply or decision.update
                 if async_gather and (async_error_feedback or not needs_feedback):
                     return gather_asynchronously(key, prepared, local, shape, active_dtype, decision)

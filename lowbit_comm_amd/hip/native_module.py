@@ -113,17 +113,26 @@ class HipNativeModule:
     # hundred bytes of host memory; ``launch_memo_entries`` can be raised per instance.
     LAUNCH_MEMO_ENTRIES = 4096
 
+    def _recall(self, key: tuple | None):
+        """The launch remembered under ``key`` for the access mode in force, or ``None``."""
+        if key is None:
+            return None
+        key = key + (ops.access_code(None),)
+        with self._launches_lock:
+            bound = self._launches.get(key)
+            if bound is not None:
+                self._launches.move_to_end(key)
+        return bound
+
     def _memoized(self, key: tuple, bind):
         """The launch remembered under ``key``, else ``bind()`` (which validates and may raise; nothing is then
         stored).  ``bind`` may return ``None`` for a call that has no single launch.  The key is completed with the
         access mode in force: a launch bound under one mode is not replayed for a call made under another."""
+        bound = self._recall(key)
+        if bound is not None:
+            return bound
         key = key + (ops.access_code(None),)
         launches = self._launches
-        with self._launches_lock:
-            bound = launches.get(key)
-            if bound is not None:
-                launches.move_to_end(key)
-                return bound
         bound = bind()                       # validates tensors and marshals arguments: outside the lock
         if bound is not None:
             with self._launches_lock:
@@ -281,9 +290,8 @@ class HipNativeModule:
         flat = output.reshape(-1)
         numel = min(flat.numel(), _padded_numel_of(inputs[0], group_size))
         key = self._reduce_key("reduce", inputs, (flat,), (group_size, topk, bit, int(quant_type), numel))
-        bound = self._launches.get(key) if key is not None else None
+        bound = self._recall(key)
         if bound is not None:
-            self._launches.move_to_end(key)
             if not bound():
                 raise RuntimeError(f"no HIP dequantize-reduce kernel for output dtype {output.dtype}")
             return
@@ -323,7 +331,7 @@ class HipNativeModule:
             raise RuntimeError("divisor must be > 0")
         key = self._reduce_key("reduce_mean", inputs, (output,),
                                (group_size, topk, bit, int(quant_type), float(divisor)))
-        bound = self._launches.get(key) if key is not None else None
+        bound = self._recall(key)
         if bound is None:
             if not self._fused_eligible(inputs, output, group_size, topk, bit, quant_type):
                 return False
@@ -365,9 +373,8 @@ class HipNativeModule:
             raise RuntimeError("divisor must be > 0")
         key = self._reduce_key("reduce_mean_feedback", inputs, (prepared, restored, residual),
                                (group_size, topk, bit, int(quant_type), float(divisor)))
-        bound = self._launches.get(key) if key is not None else None
+        bound = self._recall(key)
         if bound is not None:
-            self._launches.move_to_end(key)
             return bound()
         for name, t in (("prepared", prepared), ("restored", restored), ("residual", residual)):
             if not isinstance(t, torch.Tensor) or not t.is_cuda:
