@@ -167,8 +167,15 @@ def test_native_module_remembers_launches_by_address_without_pinning_or_going_st
     assert len(module._launches) == before + 1
     peers = [codec.quantize_tensor(grad(n, torch.float32, 40 + r, dev), CFG, extension_status=status) for r in range(world)]
     out = torch.empty(n, device=dev)
-    for _ in range(2):
-        assert module.inplace_dequantize_reduce_mean(peers, out, 64, 0, 8, linear, False, world)
+    checked = []
+    eligible = module._fused_eligible
+    module._fused_eligible = lambda *args: checked.append(1) or eligible(*args)
+    try:
+        for _ in range(3):
+            assert module.inplace_dequantize_reduce_mean(peers, out, 64, 0, 8, linear, False, world)
+    finally:
+        del module._fused_eligible
+    assert len(checked) == 1, "the second and third call replay the remembered launch without looking at the tensors again"
     want = codec_torch.reduce_payloads([unpack(p) for p in peers], n, 64, "fp32", "mean")
     assert same_bits(out, want)
     assert module.inplace_dequantize_reduce_mean(peers[::-1], out, 64, 0, 8, linear, False, world)   # another order: another key
