@@ -48,7 +48,7 @@ class _Bucket:
     __slots__ = ("plan", "tensor", "out", "op", "future", "exchange", "gather", "result", "lane", "lasting_out", "spans")
 
     def __init__(self, plan: ReduceScatterPlan, tensor: torch.Tensor, out: torch.Tensor | None, op: str, future: Any,
-                 lane: int, lasting_out: bool) -> None:
+                 lane: int, lasting_out: bool, spans: tuple) -> None:
         self.plan = plan
         self.tensor = tensor
         self.out = out
@@ -59,7 +59,7 @@ class _Bucket:
         self.gather: Any | None = None        # work object of the all-gather, if it returned one
         self.result: Any | None = None
         self.lane = lane
-        self.spans = (_span(tensor), _span(out))   # byte ranges this bucket reads and writes while it is in flight
+        self.spans = spans                    # byte ranges this bucket reads and writes while it is in flight
 
 
 def _span(tensor: torch.Tensor) -> tuple[int, int]:
@@ -172,17 +172,15 @@ class BucketPipeline:
     def _residual_for(self, tensor: torch.Tensor) -> torch.Tensor | None:
         return self.residuals.for_tensor(tensor) if self.error_feedback else None
 
-    def _touches_a_bucket_in_flight(self, tensor: torch.Tensor, out: torch.Tensor) -> bool:
-        mine = None
+    def _touches_a_bucket_in_flight(self, mine: tuple) -> bool:
         for lane in self._lanes or ():
             for bucket in (lane.reduce_next, lane.decode_next):
                 if bucket is None:
                     continue
-                if mine is None:
-                    mine = (_span(tensor), _span(out))
                 for low, high in bucket.spans:
-                    if any(low < b and a < high for a, b in mine):
-                        return True
+                    for a, b in mine:
+                        if low < b and a < high:
+                            return True
         return False
 
     def _plan_for(self, tensor: torch.Tensor, config: CompressionConfig, lane: int) -> ReduceScatterPlan:
@@ -317,13 +315,16 @@ class BucketPipeline:
                     out = torch.empty(plan.chunks.shard_numel, dtype=plan.reduced_dtype, device=tensor.device)
                 elif out.numel() != plan.chunks.shard_numel or out.dtype != plan.reduced_dtype:
                     raise ValueError("out does not match this rank's shard")
-            if self._touches_a_bucket_in_flight(tensor, out):
+            spans = (_span(tensor),)
+            if out.data_ptr() != spans[0][0] or out.numel() * out.element_size() != spans[0][1] - spans[0][0]:
+                spans += (_span(out),)            # not the bucket itself: a second range
+            if self._touches_a_bucket_in_flight(spans):
                 # The same memory again before its earlier bucket has been decoded (not a DDP iteration, where every
                 # bucket is handed over once): finish the earlier one first, so that this quantize reads its result
                 # and no launch both reads and writes the tensor.
                 self.flush()
                 plan = self._plan_for(tensor, config, index)
-            bucket = _Bucket(plan, tensor, out, op, future, index, lasting_out)
+            bucket = _Bucket(plan, tensor, out, op, future, index, lasting_out, spans)
             self._dirty = True
             residual = self._residual_for(tensor)
             if lane.stream is None:
