@@ -90,13 +90,13 @@ __device__ __forceinline__ const book_cells::Cell *block_book_cells(int kind) {
 __device__ __forceinline__ int meta_words_of(int topk) { return topk == 0 ? 1 : topk + 2; }
 
 // ---------------------------------------------------------------------------------------------
-// quantize: a wavefront works on tiles of 64 * VEC elements (64 lanes x 16 bytes of the tensor)
+// quantize: a wavefront works on tiles of 64 * EL elements (64 lanes x 32 bytes of the tensor, 16 for one policy)
 // ---------------------------------------------------------------------------------------------
 // Elements per lane: 32 bytes of the tensor, twice what the other kernels of this format give a lane.  What a
 // policy costs per group - addresses, the NaN rule of the running maximum, the outlier searches, the division behind
 // the scale - is spread over twice the elements, and a group's reductions cross half the lanes.  These kernels are
-// bound by instruction issue, not by memory, so that is what counts (26.2 M elements, 16 against 32 bytes a lane:
-// see the measurements at launch_general_quant_g).
+// bound by instruction work and latency, not by memory, so that is what counts (26.2 M elements, 16 against 32 bytes a
+// lane: see the measurements at launch_general_quant_g).
 template <typename T> constexpr int general_quant_elems() { return 32 / static_cast<int>(sizeof(T)); }
 
 // The EL 4-bit codes of one lane -> its 32-bit words.  Four codes make one 16-bit unit with the first code on top; a
