@@ -151,7 +151,8 @@ template <int LANES> __device__ __forceinline__ void merge_top3(uint32_t &first,
 
 // FIXED names what the launch knows about the policy at compile time, so that the code of the other policies
 // is not part of the kernel: bit 0 "no outlier channel", bit 1 "round to nearest", bit 2 "linear codes".
-// 0 is the kernel for every policy.  EL: elements per lane, a multiple of 8 that divides G.
+// 0 is the kernel for every policy.  EL: elements per lane, a multiple of 8 that divides G.  TILES: tiles of 64 * EL
+// elements a wavefront owns, all of them asked for before the first is encoded.
 template <typename T, int G, int BIT, int FIXED, int EL, int TILES>
 __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGeneralQuantArgs a) {
     const int topk = (FIXED & 1) ? 0 : a.topk;
