@@ -76,7 +76,7 @@ def _wait_for(work: Any) -> None:
 class _Lane:
     """The buckets of one stream: at most one awaiting its reduce and one awaiting its decode."""
 
-    __slots__ = ("stream", "handle", "reduce_next", "decode_next", "ready", "recorded")
+    __slots__ = ("stream", "handle", "reduce_next", "decode_next", "ready")
 
     def __init__(self, stream: Any | None) -> None:
         self.stream = stream
@@ -84,7 +84,6 @@ class _Lane:
         self.reduce_next: _Bucket | None = None
         self.decode_next: _Bucket | None = None
         self.ready = None if stream is None else torch.cuda.Event()    # "the caller's stream has got this far", reused
-        self.recorded: set = set()          # storages the caching allocator has been told this lane uses
 
 
 class BucketPipeline:
@@ -338,13 +337,10 @@ class BucketPipeline:
                     self._advance(lane, bucket, residual)
                 finally:
                     torch.cuda.set_stream(current)
+                # Every time, not once per address: a tensor that was freed and whose block was handed out again is a
+                # new block to the caching allocator, which has to hear of the lane's use of it too.
                 for held in (tensor, out) + (() if residual is None else (residual,)):
-                    seen = (held.data_ptr(), held.numel())
-                    if seen not in lane.recorded:             # a DDP bucket comes back every iteration: told once
-                        if len(lane.recorded) > 65536:
-                            lane.recorded.clear()
-                        lane.recorded.add(seen)
-                        held.record_stream(lane.stream)
+                    held.record_stream(lane.stream)
             return future
 
     def flush(self) -> None:
