@@ -404,7 +404,7 @@ def compressed_all_reduce_via_reduce_scatter(tensor: torch.Tensor, *, config: Co
     return plan.decode_gathered(out=out)
 
 
-__all__ = ["ReduceScatterPlan", "compressed_all_reduce_async", "compressed_all_reduce_via_reduce_scatter",
+__all__ = ["ReduceScatterPlan", "ResidualStore", "compressed_all_reduce_async", "compressed_all_reduce_via_reduce_scatter",
            "compressed_reduce_scatter_shard", "make_reduce_scatter_transport", "ccdl_dtype", "torch_dtype"]
 
 
