@@ -143,7 +143,10 @@ __global__ __launch_bounds__(kBlock) void wire_quant_kernel(const WireQuantArgs 
             // Interleaved 16-bit payloads leave as misaligned 8-byte stores here.  Re-slicing a pair of 66-byte groups
             // into aligned dwords across lanes (store_group_pair16, what the ring's gather hop does) measured slower in
             // this kernel at every size, with operands rotated through 700 MB: 26.2 M bf16 elements 15.8 us as it is,
-            // 17.7 us with non-temporal pair stores, 16.1 us with cached ones; 52.4 M 27.4 / 32.8 / 27.6 us.
+            // 17.7 us with non-temporal pair stores, 16.1 us with cached ones; 52.4 M 27.4 / 32.8 / 27.6 us.  Nor does
+            // it pay to stage a wavefront's run of eight groups (528 bytes, 16-byte aligned) in LDS and carry it out
+            // as 33 aligned 16-byte stores: 16.2 us (16.4 us non-temporal) against 15.6 us on 26.2 M elements, no
+            // workgroup barrier involved.  The misaligned stores are not what this layout costs.
             store_piece<T, BIT, PNT, W::WORDS>(payload + at.codes(group) + piece_offset<T, BIT>(k0), words);
             if ((lane & (LPG - 1)) == 0) *reinterpret_cast<Raw *>(payload + at.scale(group)) = stored;
         }
