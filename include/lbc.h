@@ -170,8 +170,8 @@ int lbc_dequant_reduce(const int8_t *const *codes, const float *const *scales, i
  * quantize writes: nothing orders the two inside the launch.
  * One side with nothing to do (numel == 0) launches the other alone.  LBC_UNSUPPORTED - issue the two calls
  * yourself - unless: group_size 64; every operand aligned for the vector kernels and numel/world * element
- * size a multiple of 16; residual absent or fp32; out_dtype fp32 or x_dtype; reduce_world
- * 2, 4 or 8.  Argument errors are reported as by the two calls.
+ * size a multiple of 16; residual absent or fp32; out_dtype fp32 or x_dtype (reduce_world is at most
+ * 8, as for lbc_dequant_reduce).  Argument errors are reported as by the two calls.
  */
 int lbc_quant_pack_chunks_and_dequant_reduce(
     const void *x, int x_dtype, const void *residual, int residual_dtype, int64_t numel, int world, int group_size,
@@ -228,7 +228,7 @@ int lbc_dequant_reduce_quant(const int8_t *const *codes, const float *const *sca
  * With one stage present its own kernel runs.  With two or three: LBC_UNSUPPORTED - issue the calls
  * yourself - unless group_size is 64, every operand is aligned for the vector kernels (16 bytes for
  * tensors and shard boundaries, 4 for payload rows; 8 for 16-bit output), the residual is absent or
- * fp32, the reduce has 2, 4 or 8 payloads, and x_dtype, mid_dtype and out_dtype are one type.
+ * fp32, and x_dtype, mid_dtype and out_dtype are one type (the reduce has at most 8 payloads, as always).
  */
 typedef struct lbc_quant_chunks_stage {
     const void *x;

@@ -63,8 +63,13 @@ hipError_t launch_w(int mode, const QuantArgs &q, int quant_world, const ReduceA
 template <typename XT, typename RT, int VEC, typename OT>
 hipError_t launch_o(int reduce_world, int mode, const QuantArgs &q, int quant_world, const ReduceArgs &r, hipStream_t s) {
     switch (reduce_world) {
+        case 1: return launch_w<XT, RT, VEC, OT, 1>(mode, q, quant_world, r, s);
         case 2: return launch_w<XT, RT, VEC, OT, 2>(mode, q, quant_world, r, s);
+        case 3: return launch_w<XT, RT, VEC, OT, 3>(mode, q, quant_world, r, s);
         case 4: return launch_w<XT, RT, VEC, OT, 4>(mode, q, quant_world, r, s);
+        case 5: return launch_w<XT, RT, VEC, OT, 5>(mode, q, quant_world, r, s);
+        case 6: return launch_w<XT, RT, VEC, OT, 6>(mode, q, quant_world, r, s);
+        case 7: return launch_w<XT, RT, VEC, OT, 7>(mode, q, quant_world, r, s);
         case 8: return launch_w<XT, RT, VEC, OT, 8>(mode, q, quant_world, r, s);
         default: return hipErrorNotSupported;
     }

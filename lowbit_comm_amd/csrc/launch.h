@@ -144,12 +144,12 @@ int quant_pack_vec(int x_dtype, int r_dtype, int d_dtype, bool outputs);
 hipError_t launch_dequant_reduce(int out_dtype, int group_size, int world, int mode,
                                  const ReduceArgs &args, hipStream_t stream);
 // Both of the above in one grid (group size 64; residual none or fp32; `quant_vec` = quant_pack_vec() of the quantize
-// call, which also fixes the new residual's type; output fp32 or the input's type; 2, 4 or 8 payloads; vector or
+// call, which also fixes the new residual's type; output fp32 or the input's type; 1 to 8 payloads; vector or
 // streaming mode).  hipErrorNotSupported for anything else.
 hipError_t launch_bucket_step(int x_dtype, int r_dtype, int quant_vec, int out_dtype, int reduce_world, int mode,
                               const QuantArgs &quant, int quant_world, const ReduceArgs &reduce, hipStream_t stream);
 // Up to three stages of a bucket stream in one grid: chunked quantize (residual none or fp32, `quant_vec` as above),
-// reduce + requantize (2, 4 or 8 payloads) and decode of `decode_world` shard payloads, all in element type `dtype`,
+// reduce + requantize (1 to 8 payloads) and decode of `decode_world` shard payloads, all in element type `dtype`,
 // group size 64, vector or streaming mode.  A null stage is absent.  hipErrorNotSupported for anything else.
 hipError_t launch_pipeline_step(int dtype, int r_dtype, int quant_vec, int mode, const QuantArgs *quant, int quant_world,
                                 const ReduceQuantArgs *reduce, int reduce_world, const DecodeArgs *decode, int decode_world,

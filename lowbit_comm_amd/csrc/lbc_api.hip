@@ -419,8 +419,8 @@ int lbc_quant_pack_chunks_and_dequant_reduce(
     if (r.status != LBC_OK) return r.status;
     if (q.empty) return launch_reduce(r, access, stream);
     if (r.empty) return launch_quant(q, "lbc_quant_pack_chunks_and_dequant_reduce", access, stream);
-    // one grid exists for aligned operands, whole 16-byte chunks, group 64, a residual that is absent or fp32 and
-    // 2, 4 or 8 payloads; everything else is for the caller to issue as the two separate calls
+    // one grid exists for aligned operands, whole 16-byte chunks, group 64 and a residual that is absent or fp32;
+    // everything else is for the caller to issue as the two separate calls
     if (!q.aligned || !r.aligned || group_size != 64 || (q.r_dtype != LBC_NONE && q.r_dtype != LBC_F32))
         return LBC_UNSUPPORTED;
     // the quantize half is the instantiation the separate call would run: its lane width also decided q.aligned
@@ -513,7 +513,7 @@ int lbc_bucket_pipeline_step(const lbc_quant_chunks_stage *quant, const lbc_redu
                       "lbc_bucket_pipeline_step");
     }
     // one grid exists for group 64, operands aligned for the vector kernels, a residual that is absent or fp32,
-    // 2, 4 or 8 payloads to reduce, and one element type for the bucket, the reduce and the decoded output
+    // and one element type for the bucket, the reduce and the decoded output
     if (group_size != 64 || (!q.empty && !q.aligned) || (!r.empty && !r.aligned) || (!d.empty && !d.aligned))
         return LBC_UNSUPPORTED;
     if (!q.empty && q.r_dtype != LBC_NONE && q.r_dtype != LBC_F32) return LBC_UNSUPPORTED;

@@ -79,8 +79,13 @@ template <typename T, typename RT, int VEC>
 hipError_t launch_v(int reduce_world, int mode, const QuantArgs *q, int quant_world, const ReduceQuantArgs *r,
                     const DecodeArgs *d, int decode_world, hipStream_t s) {
     switch (r ? reduce_world : 8) {       // without a reduce stage any instantiation serves
+        case 1: return launch_w<T, RT, VEC, 1>(mode, q, quant_world, r, d, decode_world, s);
         case 2: return launch_w<T, RT, VEC, 2>(mode, q, quant_world, r, d, decode_world, s);
+        case 3: return launch_w<T, RT, VEC, 3>(mode, q, quant_world, r, d, decode_world, s);
         case 4: return launch_w<T, RT, VEC, 4>(mode, q, quant_world, r, d, decode_world, s);
+        case 5: return launch_w<T, RT, VEC, 5>(mode, q, quant_world, r, d, decode_world, s);
+        case 6: return launch_w<T, RT, VEC, 6>(mode, q, quant_world, r, d, decode_world, s);
+        case 7: return launch_w<T, RT, VEC, 7>(mode, q, quant_world, r, d, decode_world, s);
         case 8: return launch_w<T, RT, VEC, 8>(mode, q, quant_world, r, d, decode_world, s);
         default: return hipErrorNotSupported;
     }

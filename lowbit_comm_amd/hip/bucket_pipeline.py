@@ -14,7 +14,7 @@ independent of each other, so at any moment three compute stages of three differ
 ``lbc_quant_pack_chunks_and_dequant_reduce`` for the reduce-scatter leg alone): on this part the shard-sized stages
 are mostly launch ramp on their own, and behind a quantize that fills the chip that ramp is hidden (25 MiB bf16 buckets
 with error feedback, W = 8: 31 us per bucket in one grid against 37 us as three launches).  When a combination has no
-shared grid (an odd rank count, unaligned tensors, more than eight ranks) the same stages go out as separate launches,
+shared grid (unaligned tensors, a group size other than 64, more than eight ranks) the same stages go out as separate launches,
 in the same order, with the same results.
 
 Ordering.  Everything is enqueued on the caller's current stream (or on the pipeline's lanes, see ``lanes``), so a

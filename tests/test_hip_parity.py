@@ -648,7 +648,7 @@ def test_reduce_requantize_contract(ops, hip_device):
     ("bf16", True, "fp32"), ("bf16", True, "bf16"), ("fp16", True, "fp32"), ("fp32", True, "fp32"), ("fp32", False, "fp32"),
     ("bf16", False, "bf16"), ("bf16", False, "fp32"), ("fp16", False, "fp16"),
 ])
-@pytest.mark.parametrize("world,payloads", [(8, 8), (4, 2), (2, 4)])
+@pytest.mark.parametrize("world,payloads", [(8, 8), (4, 2), (2, 4), (8, 3), (4, 5), (2, 7), (8, 6), (4, 1)])
 @pytest.mark.parametrize("n,reduce_n", [(64 * 8 * 640, 64 * 640), (64 * 8 * 64 * 3 + 64 * 8, 50_048), (64 * 8 * 30, 4096 * 3)])
 def test_shared_launch_of_quantize_and_reduce_equals_the_two_launches_and_the_oracle(
         ops, hip_device, grad_dtype, with_residual, out_dtype, world, payloads, n, reduce_n):
@@ -787,7 +787,7 @@ def test_quantize_chunks_also_write_prepared_and_refuse_a_wrong_type(ops, hip_de
     ("bf16", True, True), ("fp16", True, True), ("fp32", True, True), ("fp32", False, False), ("bf16", False, False),
     ("fp16", False, False), ("bf16", False, True),
 ])
-@pytest.mark.parametrize("world", [8, 4, 2])
+@pytest.mark.parametrize("world", [8, 4, 2, 3, 5, 6, 7, 1])
 @pytest.mark.parametrize("stages", ["qrd", "qr", "qd", "rd", "q", "r", "d"])
 @pytest.mark.parametrize("n", [64 * 8 * 640, 64 * 8 * 64 * 3 + 64 * 8 * 5])
 def test_pipeline_step_equals_its_three_launches_and_the_oracle(ops, hip_device, dtype, with_residual, track_residual,
@@ -795,6 +795,7 @@ def test_pipeline_step_equals_its_three_launches_and_the_oracle(ops, hip_device,
     """Quantize of bucket k, reduce + requantize for bucket k-1, decode of bucket k-2 in one grid: every output equal to
     the separate launches' and to the oracle's."""
     kind = DTYPES[dtype]
+    n -= n % (64 * world)                 # shard boundaries on whole groups: the shared grid wants them 16-byte aligned
     shard = -(-n // world)
     nbytes = ops.payload_nbytes(shard)
     stride = (nbytes + 255) // 256 * 256
@@ -855,9 +856,9 @@ def test_pipeline_step_equals_its_three_launches_and_the_oracle(ops, hip_device,
 
 
 def test_pipeline_step_without_a_shared_grid_says_so(ops, hip_device):
-    """Group 32, an odd payload count or operands that are not aligned have no shared grid: the bound step returns
-    False and the caller issues the stages themselves."""
-    world, n = 3, 64 * 3 * 50
+    """Another group size than 64, or operands that are not aligned for the vector kernels, have no shared grid: the
+    bound step returns False and the caller issues the stages themselves."""
+    world, n = 4, 64 * 4 * 50
     shard = n // world
     grad = gradient_like(n, torch.float32, 1, hip_device)
     send = torch.zeros(world, ops.payload_nbytes(shard), dtype=torch.uint8, device=hip_device)
@@ -865,7 +866,17 @@ def test_pipeline_step_without_a_shared_grid_says_so(ops, hip_device):
     mine = torch.zeros(ops.payload_nbytes(shard), dtype=torch.uint8, device=hip_device)
     quant = ops.bind_quant_pack_chunks(grad, send, world)
     reduce = ops.bind_dequant_reduce_quant(pairs, *ops.split_payload(mine, shard), shard)
-    assert ops.bind_bucket_pipeline_step(quant, reduce)() is False          # three payloads
+    assert ops.bind_bucket_pipeline_step(quant, reduce)() is True
+    # group 32
+    send32 = torch.zeros(world, ops.payload_nbytes(shard, 32), dtype=torch.uint8, device=hip_device)
+    pairs32 = [ops.quant_pack(gradient_like(shard, torch.float32, 2 + r, hip_device), group_size=32) for r in range(world)]
+    mine32 = torch.zeros(ops.payload_nbytes(shard, 32), dtype=torch.uint8, device=hip_device)
+    quant32 = ops.bind_quant_pack_chunks(grad, send32, world, group_size=32)
+    reduce32 = ops.bind_dequant_reduce_quant(pairs32, *ops.split_payload(mine32, shard, 32), shard, group_size=32)
+    assert ops.bind_bucket_pipeline_step(quant32, reduce32)() is False
+    # a bucket that does not start on a 16-byte boundary
+    shifted = torch.zeros(n + 1, device=hip_device)[1:]
+    assert ops.bind_bucket_pipeline_step(ops.bind_quant_pack_chunks(shifted, send, world), reduce)() is False
     assert ops.bind_bucket_pipeline_step(quant, None, None)() is True       # one stage: its own kernel
     with pytest.raises(RuntimeError, match="at least one stage"):
         ops.bind_bucket_pipeline_step()
@@ -956,11 +967,11 @@ def test_shared_launch_reports_what_it_has_no_grid_for(ops, hip_device):
     reduce3 = ops.bind_dequant_reduce(peers8[:3], out)
     bf16 = gradient_like(n, torch.bfloat16, 3301, hip_device)
     fp32 = gradient_like(n, torch.float32, 3302, hip_device)
-    # a 16-bit residual, three payloads, another group size: valid requests, no shared grid
+    # a 16-bit residual, another group size: valid requests, no shared grid; any payload count up to eight has one
     half_residual = gradient_like(n, torch.bfloat16, 3304, hip_device, sigma=1e-5, outliers=False)
     assert ops.bind_quant_chunks_and_reduce(
         ops.bind_quant_pack_chunks(bf16, rows, world, residual=half_residual), reduce8)() is False
-    assert ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(fp32, rows, world), reduce3)() is False
+    assert ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(fp32, rows, world), reduce3)() is True
     rows32 = torch.zeros(world, (ops.payload_nbytes(shard, 32) + 255) // 256 * 256, dtype=torch.uint8, device=hip_device)
     peers32 = [ops.quant_pack(gradient_like(4096, torch.float32, 3310 + r, hip_device), group_size=32) for r in range(8)]
     assert ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(fp32, rows32, world, group_size=32),
