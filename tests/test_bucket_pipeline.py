@@ -94,7 +94,7 @@ def kernel_counts(run):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("error_feedback", [False, True])
-@pytest.mark.parametrize("world,lanes", [(8, 1), (8, 2), (4, 1), (2, 3)])
+@pytest.mark.parametrize("world,lanes", [(8, 1), (8, 2), (4, 1), (2, 3), (6, 1), (3, 2), (1, 1)])
 def test_pipelined_transport_equals_the_unpipelined_one_and_the_oracle(hip_device, dtype, error_feedback, world, lanes):
     sizes = [G * world * 40, G * world * 40, G * world * 24, G * world * 40 + 8 * world, 70_001, G * world * 40, 640]
     piped, plain = transports(world, error_feedback=error_feedback, lanes=lanes)
