@@ -51,6 +51,7 @@ KERNEL_SOURCES = ("bucket_step.hip", "pipeline_step.hip", "step_grid.h", "quant_
 BATCHES = 5                # every figure is the median of this many timed batches of --steps launches
 WARM_SECONDS = 0.05        # launches go on for at least this long before a leg is timed (clocks settle after idling)
 SHARD_SETS = 16            # payload sets of the shard-reduce leg: 16 x 41 MB
+CPU_SAMPLE_SECONDS = 10.0  # CPU work of the cpu_baseline leg on all threads (half of it again on one thread)
 
 
 def kernel_sources_hash() -> str:
@@ -440,30 +441,30 @@ def main() -> int:
         ok = all(torch.equal(sent_cpu[d, :payload_bytes], codec_torch.pack(*payloads[d])) for d in range(world))
         ok = ok and torch.equal(s0["out"].cpu().view(torch.int32), reduced.view(torch.int32))
         parity = "bit-exact" if ok else "MISMATCH"
+        # A bounded sample of the same step: repeats for about ten seconds of CPU work (a host's first repeats, with its
+        # thread pool and caches cold, are several times slower than its steady state, and a dozen repeats gave figures
+        # between 3 and 16 GB/s from one box to the next).
         times = []
-        deadline = time.perf_counter() + 25.0
-        for i in range(12):
+        deadline = time.perf_counter() + CPU_SAMPLE_SECONDS
+        while len(times) < 3 or (time.perf_counter() < deadline and len(times) < 5000):
             t0 = time.perf_counter()
             cpu_step()
             times.append(time.perf_counter() - t0)
-            if time.perf_counter() > deadline:
-                break
-        times = sorted(times[2:] or times)
+        times = sorted(times[3:] or times)
         median = times[len(times) // 2]
         threads = torch.get_num_threads()
         single = None
         if threads > 1:                                   # the same step on one thread, a few repeats
             torch.set_num_threads(1)
             one = []
-            stop_at = time.perf_counter() + 8.0
-            for i in range(4):
+            stop_at = time.perf_counter() + CPU_SAMPLE_SECONDS / 2
+            while len(one) < 2 or (time.perf_counter() < stop_at and len(one) < 1000):
                 t0 = time.perf_counter()
                 cpu_step()
                 one.append(time.perf_counter() - t0)
-                if time.perf_counter() > stop_at:
-                    break
             torch.set_num_threads(threads)
-            single = sorted(one[1:] or one)[0]
+            one = sorted(one[1:] or one)
+            single = one[len(one) // 2]
         model = "unknown"
         try:
             with open("/proc/cpuinfo") as info:
@@ -472,8 +473,8 @@ def main() -> int:
             pass
         cpu_baseline = {
             "value": n * 4 / median / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": f"{len(times)} timed repeats of the full step (8x quantize of 3,276,800-element chunks + "
-                      f"8-payload left-fold reduce of one shard) with torch CPU ops, median {median * 1e3:.1f} ms; "
+            "sample": f"{len(times)} timed repeats ({sum(times):.1f} s) of the full step (8x quantize of 3,276,800-element "
+                      f"chunks + 8-payload left-fold reduce of one shard) with torch CPU ops, median {median * 1e3:.1f} ms; "
                       f"host has {os.cpu_count()} logical CPUs",
             "single_thread_value": None if single is None else n * 4 / single / 1e9,
             "cpu_model": model,
