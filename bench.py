@@ -441,9 +441,8 @@ def main() -> int:
         ok = all(torch.equal(sent_cpu[d, :payload_bytes], codec_torch.pack(*payloads[d])) for d in range(world))
         ok = ok and torch.equal(s0["out"].cpu().view(torch.int32), reduced.view(torch.int32))
         parity = "bit-exact" if ok else "MISMATCH"
-        # A bounded sample of the same step: repeats for about ten seconds of CPU work (a host's first repeats, with its
-        # thread pool and caches cold, are several times slower than its steady state, and a dozen repeats gave figures
-        # between 3 and 16 GB/s from one box to the next).
+        # A bounded sample of the same step: repeats for about ten seconds of CPU work, so that the figure is the
+        # host's steady state and not that of a cold thread pool (hosts still differ: 2.6 to 12 GB/s were seen).
         times = []
         deadline = time.perf_counter() + CPU_SAMPLE_SECONDS
         while len(times) < 3 or (time.perf_counter() < deadline and len(times) < 5000):
