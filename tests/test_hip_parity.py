@@ -992,3 +992,58 @@ def test_shared_launch_reports_what_it_has_no_grid_for(ops, hip_device):
     restored = torch.empty(n, device=hip_device)
     with pytest.raises(RuntimeError, match="restored"):
         ops.bind_quant_chunks_and_reduce(ops.bind_quant_pack_chunks(fp32, rows, world, restored=restored), reduce8)
+
+
+# --------------------------------------------------------------------------- #
+# seeded random sweep: sizes, start offsets, dtypes, rank counts and access modes nobody picked by hand
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shapes_and_offsets_against_the_oracle(hip_device, seed):
+    """Every case: a bucket view at a random element offset (so every alignment class of the kernels is met), split
+    into a random number of chunks with or without a residual, quantized; then the same number of payloads reduced into
+    a shard view - both against the oracle, bit for bit."""
+    from lowbit_comm_amd.hip import ops as hip_ops
+
+    rng = np.random.default_rng(4000 + seed)
+    for case in range(40):
+        dtype = str(rng.choice(["fp32", "bf16", "fp16"]))
+        kind = DTYPES[dtype]
+        world = int(rng.integers(1, 9))
+        n = int(rng.choice([rng.integers(1, 200), rng.integers(200, 70_000), 64 * world * int(rng.integers(1, 400))]))
+        offset = int(rng.integers(0, 9))
+        group = int(rng.choice([64, 64, 64, 32, 16]))
+        mode = str(rng.choice(["cached", "stream", "auto"]))
+        with_residual = bool(rng.integers(0, 2))
+        what = f"seed {seed} case {case}: {dtype} n={n} offset={offset} world={world} group={group} {mode} residual={with_residual}"
+        grad = gradient_like(n + offset, kind, 9000 + 100 * seed + case, hip_device)[offset:]
+        residual = None
+        if with_residual:
+            residual = gradient_like(n + offset, torch.float32, 9500 + case, hip_device, sigma=1e-5, outliers=False)[offset:]
+        keep = None if residual is None else residual.clone()
+        shard = -(-n // world)
+        nbytes = hip_ops.payload_nbytes(shard, group)
+        stride = (nbytes + 3) // 4 * 4 + 4 * int(rng.integers(0, 3))
+        rows = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+        with hip_ops.access_mode(mode):
+            assert hip_ops.quant_pack_chunks_into(grad, rows, world, group_size=group, residual=residual,
+                                                  new_residual=residual), what
+        prepared = grad.cpu() if keep is None else grad.cpu() + keep.cpu()
+        dropped = []
+        for d in range(world):
+            chunk = prepared[d * shard:(d + 1) * shard]
+            if chunk.numel() < shard:
+                chunk = torch.cat([chunk, torch.zeros(shard - chunk.numel(), dtype=chunk.dtype)])
+            codes, scales = codec_torch.quantize(chunk, group)
+            assert torch.equal(rows[d, :nbytes].cpu(), codec_torch.pack(codes, scales)), f"{what}: chunk {d}"
+            dropped.append(chunk.float() - codec_torch.dequantize(codes, scales, shard, group, "fp32"))
+        if residual is not None:
+            assert_same_bits(residual, torch.cat(dropped)[:n], f"{what}: residual")
+        # the chunk payloads, taken as what `world` peers sent for one shard, reduced into a view at another offset
+        out_offset = int(rng.integers(0, 5))
+        out = torch.zeros(shard + out_offset, dtype=kind, device=hip_device)[out_offset:]
+        pairs = [hip_ops.split_payload(rows[d, :nbytes], shard, group) for d in range(world)]
+        op = str(rng.choice(["sum", "mean"]))
+        with hip_ops.access_mode(mode):
+            assert hip_ops.dequant_reduce_into(pairs, out, group_size=group, divisor=float(world) if op == "mean" else 1.0), what
+        want = codec_torch.reduce_payloads([(c.cpu(), s.cpu()) for c, s in pairs], shard, group, dtype, op)
+        assert_same_bits(out, want, f"{what}: reduced shard ({op})")
