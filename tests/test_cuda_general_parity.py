@@ -438,3 +438,45 @@ def test_code_books_on_every_16_bit_quotient(hip, hip_device, name, quant_type):
         payload = torch.empty(hip.general_payload_nbytes(n, x.dtype, g, 4, 0), dtype=torch.uint8, device=hip_device)
         assert hip.quant_general_into(x, payload, group_size=g, bit=4, quant_type=quant_type, compact=True)
         same(payload, general.quantize(x_np, name, g, 4, quant_type, 0, None, True), f"{name} {quant_type} top={top}")
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_policies_sizes_and_values_against_the_oracle(hip, hip_device, seed):
+    """A seeded random walk over what the systematic sweep fixes by hand: group counts from one to a few tens of
+    thousands, magnitudes over twelve decades, NaN / Inf sprinkled in, many ties and zeros, every policy, both layouts,
+    random Philox seeds and offsets (all four phases of a block), decode with every reduce op."""
+    rng = np.random.default_rng(7100 + seed)
+    for case in range(60):
+        name = str(rng.choice(list(NAMES)))
+        g = int(rng.choice([16, 32, 64]))
+        bit = int(rng.choice([4, 8]))
+        quant_type = "linear" if bit == 8 else str(rng.choice(general.QUANT_TYPES))
+        topk = int(rng.choice([0, 1, 2]))
+        stochastic = None if rng.random() < 0.4 else (int(rng.integers(0, 2**63)), int(rng.integers(0, 2**40)))
+        compact = bool(rng.integers(0, 2))
+        groups = int(rng.choice([1, 3, 17, 64, 65, 255, 1024, 4097, 20000]))
+        n = g * groups
+        values = (rng.standard_normal(n) * 10.0 ** rng.integers(-8, 4)).astype(np.float32)
+        mode = int(rng.integers(0, 4))
+        if mode == 1:
+            values[rng.integers(0, n, max(1, n // 50))] = np.nan
+            values[rng.integers(0, n, 2)] = np.inf
+        elif mode == 2:
+            values = np.round(values * 4) / 4           # many ties and zeros
+        elif mode == 3:
+            values[rng.integers(0, n, max(1, n // 3))] = 0
+        what = (f"seed {seed} case {case}: {name} g={g} bit={bit} {quant_type} topk={topk} stochastic={stochastic} "
+                f"compact={compact} groups={groups} mode={mode}")
+        x_np = wire.from_f32(values, name)
+        x = from_numpy(x_np, name, hip_device)
+        payload = torch.empty(hip.general_payload_nbytes(n, x.dtype, g, bit, topk), dtype=torch.uint8, device=hip_device)
+        policy = dict(group_size=g, bit=bit, quant_type=quant_type, topk=topk, compact=compact)
+        hip.quant_general_into(x, payload, stochastic=stochastic, **policy)
+        want = general.quantize(x_np, name, g, bit, quant_type, topk, stochastic, compact)
+        assert to_numpy(payload).tobytes() == want.tobytes(), f"{what}: payload bytes"
+        op = str(rng.choice(["none", "sum", "max", "min"]))
+        old_np = wire.from_f32(rng.standard_normal(n).astype(np.float32), name)
+        out = from_numpy(old_np, name, hip_device)
+        hip.dequant_general_into(payload, out, reduce_op=op, **policy)
+        decoded = general.dequantize(want, n, name, g, bit, quant_type, topk, compact, op, old_np)
+        assert to_numpy(out).tobytes() == decoded.tobytes(), f"{what}: decoded values ({op})"
