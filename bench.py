@@ -155,6 +155,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--sets", type=int, default=6, help="distinct buffer sets rotated through (defeats the LLC)")
+    ap.add_argument("--deep-sets", type=int, default=24,
+                    help="buffer sets of the deep-rotation legs (0 leaves them out); every set holds 0.5 GB")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma list of kernel legs to time (for profiling one kernel)")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_DB", "WRITE_DB"),
@@ -193,8 +195,7 @@ def main() -> int:
         return (torch.randn(numel, generator=gen_, device=dev) * sigma).to(dtype)
 
     # ---- synthetic inputs, resident in HBM before any timing -----------------------------------
-    sets = []
-    for s in range(args.sets):
+    def make_set(s):
         bucket = gen(SEED + 100 * s, n, 1e-3)                       # this rank's bucket
         sent = torch.empty(world, stride, dtype=torch.uint8, device=dev)
         received = torch.empty(world, stride, dtype=torch.uint8, device=dev)
@@ -203,11 +204,23 @@ def main() -> int:
             assert ops.quant_pack_payload_into(peer_chunk, received[r, :payload_bytes], group_size=g)
         out = torch.empty(shard, dtype=torch.float32, device=dev)
         pairs = [ops.split_payload(received[r, :payload_bytes], shard, g) for r in range(world)]
-        sets.append({
+        return {
             "bucket": bucket, "sent": sent, "received": received, "out": out,
             "quant": ops.bind_quant_pack_chunks(bucket, sent, world, group_size=g),
             "reduce": ops.bind_dequant_reduce(pairs, out, group_size=g),
-        })
+        }
+
+    def add_plan_stages(s):
+        """The stages of the reduce-scatter + all-gather plan that follow the quantize, on buffers of this set."""
+        s["gathered"] = s["received"].clone()
+        s["mine"] = torch.empty(payload_bytes, dtype=torch.uint8, device=dev)
+        s["decoded"] = torch.empty(n, dtype=torch.float32, device=dev)
+        s["reduce_requant"] = ops.bind_dequant_reduce_quant(
+            [ops.split_payload(s["received"][r, :payload_bytes], shard, g) for r in range(world)],
+            *ops.split_payload(s["mine"], shard, g), shard, group_size=g, divisor=float(world))
+        s["decode"] = ops.bind_dequant_chunks(s["gathered"], s["decoded"], shard, group_size=g)
+
+    sets = [make_set(s) for s in range(args.sets)]
     # the step: the quantize of one set's bucket and the reduce of the previous set's payloads, one launch
     for k, s in enumerate(sets):
         s["step"] = ops.bind_quant_chunks_and_reduce(s["quant"], sets[k - 1]["reduce"])
@@ -337,14 +350,8 @@ def main() -> int:
         # the whole reduce-scatter + all-gather plan as the drop-in transport runs it on a stream of buckets: one launch
         # carries the quantize of bucket k, the reduce + requantize of the payloads that arrived for bucket k-1 and the
         # decode of the gathered shard payloads of bucket k-2 into that bucket (lbc_bucket_pipeline_step)
-        for k, s in enumerate(sets):
-            s["gathered"] = s["received"].clone()
-            s["mine"] = torch.empty(payload_bytes, dtype=torch.uint8, device=dev)
-            s["decoded"] = torch.empty(n, dtype=torch.float32, device=dev)
-            s["reduce_requant"] = ops.bind_dequant_reduce_quant(
-                [ops.split_payload(s["received"][r, :payload_bytes], shard, g) for r in range(world)],
-                *ops.split_payload(s["mine"], shard, g), shard, group_size=g, divisor=float(world))
-            s["decode"] = ops.bind_dequant_chunks(s["gathered"], s["decoded"], shard, group_size=g)
+        for s in sets:
+            add_plan_stages(s)
         for k, s in enumerate(sets):
             s["pipeline_step"] = ops.bind_bucket_pipeline_step(s["quant"], sets[k - 1]["reduce_requant"], sets[k - 2]["decode"])
         plan_bytes = quant_bytes + (world + 1) * payload_bytes + world * payload_bytes + n * 4
@@ -365,6 +372,34 @@ def main() -> int:
         for s in sets:
             for name in ("gathered", "mine", "decoded", "reduce_requant", "decode", "pipeline_step"):
                 del s[name]
+        torch.cuda.empty_cache()
+    if (not only or "deep_rotation" in only) and args.deep_sets > len(sets):
+        # The same two launches with four times as many buffer sets in rotation (4 GB and 7 GB instead of 1 GB and
+        # 1.8 GB between two uses of a buffer): launches that write much read a few percent slower this way although
+        # the traffic that leaves the L2 is the same, so both figures are in the line.
+        deep = sets + [make_set(s) for s in range(len(sets), args.deep_sets)]
+        for s in deep:
+            add_plan_stages(s)
+        deep_steps = [ops.bind_quant_chunks_and_reduce(s["quant"], deep[k - 1]["reduce"]) for k, s in enumerate(deep)]
+        deep_plans = [ops.bind_bucket_pipeline_step(s["quant"], deep[k - 1]["reduce_requant"], deep[k - 2]["decode"])
+                      for k, s in enumerate(deep)]
+
+        def run_deep(launches):
+            def call(i):
+                if not launches[i % len(launches)]():
+                    raise RuntimeError("the library has no shared launch for these stages")
+            return call
+
+        leg("bucket_step_deep_rotation", run_deep(deep_steps), quant_bytes + reduce_bytes, launches=max(args.steps, 48))
+        leg("bucket_pipeline_step_deep_rotation", run_deep(deep_plans),
+            quant_bytes + (2 * world + 1) * payload_bytes + n * 4, launches=max(args.steps, 48))
+        for name in ("bucket_step_deep_rotation", "bucket_pipeline_step_deep_rotation"):
+            if name in kernels:
+                kernels[name]["buffer_sets"] = len(deep)
+        for s in deep:
+            for name in ("gathered", "mine", "decoded", "reduce_requant", "decode"):
+                del s[name]
+        del deep, deep_steps, deep_plans
         torch.cuda.empty_cache()
     if not only or "dequant_reduce_shard" in only:
         # the shard reduce alone moves 41 MB a launch: it gets payload sets of its own, enough of them (656 MB) that
@@ -516,6 +551,9 @@ def main() -> int:
             "achieved": dominant["achieved_GBps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
             "frac": dominant["frac_of_hbm_peak"], "traffic": traffic, "traffic_source": traffic_source,
             "algorithmic_bytes": dominant["algorithmic_bytes"], "us_per_launch": dominant["us_per_launch"],
+            "buffer_sets": args.sets,
+            # the same kernel with four times as many buffer sets in rotation (see kernels.bucket_step_deep_rotation)
+            "frac_deep_rotation": kernels.get("bucket_step_deep_rotation", {}).get("frac_of_hbm_peak"),
         },
         "cpu_baseline": cpu_baseline,
         "parity": parity,
