@@ -3,11 +3,15 @@
 // its own, and compares every byte with the scalar C oracles (oracle/codec_scalar.c, oracle/cuda_wire_scalar.c,
 // oracle/cuda_wire_general_scalar.c, linked from oracle/_build).  Built by __graft_entry__.build(), run by
 // tests/test_abi_client.py on the GPU box.  Prints "OK <checks>" or the first mismatch.
+// `abi_client ring-host-cost` instead measures what the calls of one rank's ring schedule cost a native caller: the
+// host time of 15 consecutive lbc_ring_step calls (the launches of a W=8 ring on one 200 MiB fp32 bucket) and the time
+// the device takes for them back to back - the floor under any submission loop written above this ABI.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
 
+#include <chrono>
 #include <vector>
 
 #include "../../include/lbc.h"
@@ -212,7 +216,40 @@ static int wire_format_checks(hipStream_t stream, long &checks) {
     return 0;
 }
 
-int main() {
+static int ring_host_cost() {
+    const int64_t n = 6553600, groups = n / 64;   // a 200 MiB fp32 bucket over 8 ranks
+    const int buckets = 12, launches = 15;
+    int8_t *recv_codes, *send_codes;
+    float *recv_scales, *send_scales, *chunk;
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+    HIP_OK(hipMalloc(&recv_codes, n));
+    HIP_OK(hipMalloc(&send_codes, n));
+    HIP_OK(hipMalloc(&recv_scales, groups * sizeof(float)));
+    HIP_OK(hipMalloc(&send_scales, groups * sizeof(float)));
+    HIP_OK(hipMalloc(&chunk, n * sizeof(float)));
+    HIP_OK(hipMemset(recv_codes, 1, n));
+    HIP_OK(hipMemset(recv_scales, 0, groups * sizeof(float)));
+    HIP_OK(hipMemset(chunk, 0, n * sizeof(float)));
+    for (int rep = 0; rep < 5; ++rep) {           // the first repetition warms up
+        const auto begin = std::chrono::steady_clock::now();
+        for (int i = 0; i < buckets * launches; ++i)
+            LBC_OK_OR_FAIL(lbc_ring_step(recv_codes, recv_scales, chunk, LBC_F32, n, 64, LBC_REDUCE_SUM, 1.0f, send_codes,
+                                         send_scales, LBC_ACCESS_AUTO, stream));
+        const auto enqueued = std::chrono::steady_clock::now();
+        HIP_OK(hipStreamSynchronize(stream));
+        const auto done = std::chrono::steady_clock::now();
+        if (rep > 0)
+            printf("%d calls of lbc_ring_step (6,553,600 fp32): host %.1f us (%.2f us a call), device %.1f us\n", launches,
+                   std::chrono::duration<double, std::micro>(enqueued - begin).count() / buckets,
+                   std::chrono::duration<double, std::micro>(enqueued - begin).count() / (buckets * launches),
+                   std::chrono::duration<double, std::micro>(done - begin).count() / buckets);
+    }
+    return 0;
+}
+
+int main(int argc, char **argv) {
+    if (argc > 1 && strcmp(argv[1], "ring-host-cost") == 0) return ring_host_cost();
     if (lbc_abi_version() != LBC_ABI_VERSION) {
         printf("FAIL abi version %d, header %d\n", lbc_abi_version(), LBC_ABI_VERSION);
         return 1;
