@@ -150,13 +150,15 @@ template <int LANES> __device__ __forceinline__ void merge_top3(uint32_t &first,
 }
 
 // FIXED names what the launch knows about the policy at compile time, so that the code of the other policies
-// is not part of the kernel: bit 0 "no outlier channel", bit 1 "round to nearest", bit 2 "linear codes".
-// 0 is the kernel for every policy.  EL: elements per lane, a multiple of 8 that divides G.  TILES: tiles of 64 * EL
-// elements a wavefront owns, all of them asked for before the first is encoded.
+// is not part of the kernel: bit 0 "no outlier channel", bit 1 "round to nearest", bit 2 "linear codes", bit 3
+// "stochastic rounding" (13: plain linear codes rounded stochastically, 12: the same with outliers, 9: a code book
+// with stochastic rounding).  0 is the kernel for every policy.
+// EL: elements per lane, a multiple of 8 that divides G.  TILES: tiles of 64 * EL elements a wavefront owns, all of
+// them asked for before the first is encoded.
 template <typename T, int G, int BIT, int FIXED, int EL, int TILES>
 __global__ __launch_bounds__(kBlock) void wire_general_quant_kernel(const WireGeneralQuantArgs a) {
     const int topk = (FIXED & 1) ? 0 : a.topk;
-    const bool stochastic = (FIXED & 2) ? false : a.stochastic != 0;
+    const bool stochastic = (FIXED & 2) ? false : ((FIXED & 8) ? true : a.stochastic != 0);
     const int kind = (FIXED & 4) ? 0 : a.kind;
     using W = wire<T, BIT>;
     using RB = raw_bits<T>;
@@ -567,9 +569,12 @@ hipError_t launch_general_quant_as(const WireGeneralQuantArgs &a, hipStream_t st
 
 template <typename T, int G>
 hipError_t launch_general_quant_g(int bit, const WireGeneralQuantArgs &a, hipStream_t stream) {
-    // Policies that round to nearest run a kernel without the code of the others (26.2 M fp32 elements: top-2
-    // 30.8 instead of 32.3 us, a code book 30.0 instead of 31.7 us); stochastic rounding is faster in the kernel
-    // for every policy (37.4 against 38.6 us), whose Philox rounds leave the compiler less room to reorder.
+    // Each common policy runs a kernel without the code of the others (26.2 M fp32 elements: top-2 30.8 instead of
+    // 32.3 us, a code book 30.0 instead of 31.7 us).  Stochastic rounding of plain linear codes gains most: in the
+    // kernel for every policy it holds 126 vector registers for sixteen 16-bit elements a lane (four wavefronts a
+    // SIMD), on its own 65 (seven): 26.2 M bf16 elements 17.0 instead of 20.4 us, fp32 23.7 instead of 24.2 us.
+    // With outliers 32.4 / 26.8 instead of 35.3 / 28.5 us (fp32 / bf16), with a code book 36.5 / 34.5 instead of
+    // 40.8 / 38.8 us.
     //
     // 32 bytes a lane against 16 (26.2 M elements, group 64, us): fp32 top-2 27.4 / 30.5, stochastic 24.3 / 26.6,
     // a code book 25.5 / 27.9; bf16 top-2 22.1 / 23.3, stochastic 21.5 / 22.6, a code book through the cell table
@@ -581,10 +586,14 @@ hipError_t launch_general_quant_g(int bit, const WireGeneralQuantArgs &a, hipStr
     if (bit != 8 && bit != 4) return hipErrorNotSupported;
     if (bit == 8 && a.kind != 0) return hipErrorNotSupported;   // eight bits: linear codes only
     if (bit == 8) {
-        if (fixed == 6) return launch_general_quant_as<T, G, 8, 6, WIDE>(a, stream);
-        return launch_general_quant_as<T, G, 8, 0, WIDE>(a, stream);
+        if (a.stochastic && a.topk == 0) return launch_general_quant_as<T, G, 8, 13, WIDE>(a, stream);
+        if (a.stochastic) return launch_general_quant_as<T, G, 8, 12, WIDE>(a, stream);
+        return launch_general_quant_as<T, G, 8, 6, WIDE>(a, stream);   // round to nearest, outliers or none
     }
-    if (fixed == 2 || fixed == 6) return launch_general_quant_as<T, G, 4, 2, WIDE>(a, stream);
+    if (fixed == 6) return launch_general_quant_as<T, G, 4, 6, WIDE>(a, stream);
+    if (fixed == 2) return launch_general_quant_as<T, G, 4, 2, WIDE>(a, stream);
+    if (a.stochastic && a.topk == 0 && a.kind == 0) return launch_general_quant_as<T, G, 4, 13, WIDE>(a, stream);
+    if (a.stochastic && a.topk == 0) return launch_general_quant_as<T, G, 4, 9, WIDE>(a, stream);
     if (fixed == 3) return launch_general_quant_as<T, G, 4, 3, CELLS, CELL_TILES>(a, stream);
     return launch_general_quant_as<T, G, 4, 0, WIDE>(a, stream);
 }
