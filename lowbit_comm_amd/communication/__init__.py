@@ -1,4 +1,5 @@
 """Adapters between DDP buckets, the codec and injected collectives."""
+from .async_pipeline import AsyncBucketPipeline
 from .async_shard_pipeline import AsyncShardPipeline
 from .collectives import CompressedAllReduce, CompressedPayload, PackedPayload
 from .gather_reduce import CompressedAllGatherReduce, GatheredPayloads
@@ -13,7 +14,7 @@ from .payload_packing import (
 )
 
 __all__ = [
-    "AsyncShardPipeline", "CompressedAllGatherReduce", "CompressedAllReduce", "CompressedPayload", "DEFAULT_FUSED_PAYLOAD_MIN_NUMEL",
+    "AsyncBucketPipeline", "AsyncShardPipeline", "CompressedAllGatherReduce", "CompressedAllReduce", "CompressedPayload", "DEFAULT_FUSED_PAYLOAD_MIN_NUMEL",
     "FusedPayloadAllGather", "FusedPayloadPacker", "GatheredPayloads", "PackedPayload", "TensorFieldSchema",
     "make_fused_payload_all_gather", "make_payload_all_gather", "should_fuse_payload",
 ]

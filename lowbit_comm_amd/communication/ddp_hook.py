@@ -14,6 +14,7 @@ from collections.abc import Callable
 from dataclasses import dataclass, field
 from typing import Any
 
+from lowbit_comm_amd.communication.async_pipeline import AsyncBucketPipeline, chain_after
 from lowbit_comm_amd.communication.collectives import CompressedPayload
 from lowbit_comm_amd.communication.ddp import DDPBucketProcessor
 from lowbit_comm_amd.communication.gather_reduce import CompressedAllGatherReduce, GatheredPayloads
@@ -121,52 +122,6 @@ def _shaped(workspace: Any, shape: tuple[int, ...]) -> Any:
     except TypeError:
         pass
     return flat.reshape(shape)
-
-
-def _chain_after(work: Any, finish: Callable[[Any], Any]) -> None:
-    """Run ``finish`` once the asynchronous gather is done: behind the work's own future when it offers one
-    (``get_future().then``), immediately otherwise."""
-    get_future = getattr(work, "get_future", None)
-    inner = get_future() if callable(get_future) else None
-    if inner is not None and hasattr(inner, "then"):
-        inner.then(finish)
-    else:
-        finish(None)
-
-
-def _finish_feedback_bucket(work: Any, bucket_future: Any, *, decode: Callable[[Any], Any],
-                            update: Callable[[Any], None], advance: Callable[[], None], completions: Any,
-                            host_wait: bool) -> Any:
-    """Completion of a bucket with error feedback whose gather ran asynchronously: decode and reduce, update the
-    residual, advance the feedback policy, order the result on the device (and, unless switched off, on the host)
-    and resolve the bucket's future; an exception goes to the future when it can carry one
-    (sequence of ccdl_comm/communication/async_pipeline.py:49-65)."""
-    if completions is None:
-        from lowbit_comm_amd.hip.workspace import EventCompletionManager
-
-        completions = EventCompletionManager()
-
-    def finish(_unused: Any = None) -> Any:
-        try:
-            restored = decode(work.wait())
-            update(restored)
-            advance()
-            done = completions.record_for(restored)
-            done.wait()
-            block_host = getattr(done, "synchronize", None)
-            if host_wait and callable(block_host):
-                block_host()
-        except Exception as exc:
-            carry = getattr(bucket_future, "set_exception", None)
-            if not callable(carry):
-                raise
-            carry(exc)
-            return None
-        bucket_future.set_result(restored)
-        return restored
-
-    _chain_after(work, finish)
-    return bucket_future
 
 
 def _single_process_all_reduce(tensor: Any, reduce: str) -> Any:
@@ -387,9 +342,9 @@ def create_ddp_comm_hook(
                     feedback.update(key, original=prepared, transmitted=restored)
 
             if decision.apply or decision.update:
-                return _finish_feedback_bucket(work, outer, decode=decode, update=update,
-                                               advance=lambda: policy.advance(key), completions=completion_manager,
-                                               host_wait=synchronize_async_feedback_completion)
+                return AsyncBucketPipeline(gather_work=work, future=outer, dequantize_reduce=decode, update_feedback=update,
+                                           advance_policy=lambda: policy.advance(key), completion_manager=completion_manager,
+                                           synchronize_completion=synchronize_async_feedback_completion).run()
 
             def complete(_unused: Any = None) -> Any:
                 restored = decode(work.wait())
@@ -397,7 +352,7 @@ def create_ddp_comm_hook(
                 outer.set_result(restored)
                 return restored
 
-            _chain_after(work, complete)
+            chain_after(work, complete)
             return outer
 
         def process_bucket(bucket: Any) -> Any:
