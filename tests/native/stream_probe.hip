@@ -140,6 +140,94 @@ double run(F launch, int iters, int nbuf) {
     return ms * 1e-3 / iters;
 }
 
+// "shape" mode: the fp32 quantize's traffic on 100 MiB against (a) the workgroups that fit a CU, limited through
+// an LDS allocation, with one, two or four tiles a lane in flight, and (b) a grid whose last part is cut into one-tile
+// workgroups - what occupancy and the drain of coarse workgroups are worth for such a launch.
+template <int UNROLL>
+__global__ __launch_bounds__(256) void quantlike_lds_kernel(const float4v* __restrict__ in, unsigned* __restrict__ out, size_t n4) {
+    extern __shared__ char lds[];
+    size_t base = (size_t)blockIdx.x * 256 * UNROLL + threadIdx.x;
+    float4v v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) { size_t i = base + (size_t)u * 256; if (i < n4) v[u] = __builtin_nontemporal_load(in + i); }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        size_t i = base + (size_t)u * 256;
+        if (i < n4) __builtin_nontemporal_store(__builtin_bit_cast(unsigned, v[u].x + v[u].y + v[u].z + v[u].w), out + i);
+    }
+    if (n4 == 1) lds[threadIdx.x] = 1;   // keeps the allocation
+}
+
+__global__ __launch_bounds__(256) void quantlike_tail_kernel(const float4v* __restrict__ in, unsigned* __restrict__ out, size_t n4,
+                                                            unsigned split) {
+    if (blockIdx.x < split) {            // four tiles a lane
+        size_t base = (size_t)blockIdx.x * 1024 + threadIdx.x;
+        float4v v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(in + base + u * 256);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            __builtin_nontemporal_store(__builtin_bit_cast(unsigned, v[u].x + v[u].y + v[u].z + v[u].w), out + base + u * 256);
+    } else {                             // one tile a lane behind them
+        size_t i = (size_t)split * 1024 + (size_t)(blockIdx.x - split) * 256 + threadIdx.x;
+        if (i < n4) {
+            float4v v = __builtin_nontemporal_load(in + i);
+            __builtin_nontemporal_store(__builtin_bit_cast(unsigned, v.x + v.y + v.z + v.w), out + i);
+        }
+    }
+}
+
+template <typename F>
+static double best_of(F launch, int nbuf) {
+    Timer t;
+    for (int i = 0; i < 300; ++i) launch(i % nbuf);
+    CK(hipDeviceSynchronize());
+    double best = 1e9;
+    for (int rep = 0; rep < 7; ++rep) {
+        CK(hipEventRecord(t.a));
+        for (int i = 0; i < 60; ++i) launch(i % nbuf);
+        CK(hipEventRecord(t.b));
+        CK(hipEventSynchronize(t.b));
+        float ms; CK(hipEventElapsedTime(&ms, t.a, t.b));
+        if (ms / 60 < best) best = ms / 60;
+    }
+    return best * 1e-3;
+}
+
+static int shape_mode() {
+    const size_t bytes = (size_t)100 << 20, n4 = bytes / 16;
+    const int nbuf = 6;
+    std::vector<float4v*> in(nbuf); std::vector<unsigned*> out(nbuf);
+    for (int i = 0; i < nbuf; ++i) { CK(hipMalloc(&in[i], bytes)); CK(hipMalloc(&out[i], bytes / 4)); CK(hipMemset(in[i], 1, bytes)); }
+    const int lds_sizes[] = {0, 26 * 1024, 40 * 1024, 80 * 1024};
+    CK(hipFuncSetAttribute((const void*)quantlike_lds_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024));
+    CK(hipFuncSetAttribute((const void*)quantlike_lds_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024));
+    CK(hipFuncSetAttribute((const void*)quantlike_lds_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024));
+    for (int lds : lds_sizes)
+        for (int U : {1, 2, 4}) {
+            const unsigned grid = (unsigned)((n4 + 256 * U - 1) / (256 * U));
+            double t = best_of([&](int k) {
+                if (U == 1) hipLaunchKernelGGL(quantlike_lds_kernel<1>, dim3(grid), dim3(256), lds, 0, in[k], out[k], n4);
+                if (U == 2) hipLaunchKernelGGL(quantlike_lds_kernel<2>, dim3(grid), dim3(256), lds, 0, in[k], out[k], n4);
+                if (U == 4) hipLaunchKernelGGL(quantlike_lds_kernel<4>, dim3(grid), dim3(256), lds, 0, in[k], out[k], n4);
+            }, nbuf);
+            printf("SHAPE lds %6d B a workgroup, %d tile(s) a lane: %.2f us (%.1f %% of 8 TB/s)\n", lds, U, t * 1e6,
+                   bytes * 1.25 / t / 8e12 * 100);
+            fflush(stdout);
+        }
+    const unsigned full = (unsigned)(n4 / 1024);
+    for (int pct : {100, 97, 90, 75, 50, 0}) {
+        const unsigned split = (unsigned)((size_t)full * pct / 100);
+        const unsigned rest = (unsigned)((n4 - (size_t)split * 1024 + 255) / 256);
+        double t = best_of([&](int k) { hipLaunchKernelGGL(quantlike_tail_kernel, dim3(split + rest), dim3(256), 0, 0, in[k], out[k], n4, split); },
+                           nbuf);
+        printf("SHAPE four-tile workgroups for %3d %% of the data, one-tile workgroups behind: %.2f us (%.1f %% of 8 TB/s)\n", pct, t * 1e6,
+               bytes * 1.25 / t / 8e12 * 100);
+        fflush(stdout);
+    }
+    return 0;
+}
+
 // "rows" mode: the two traffic mixes the hot kernels are held to, at the caller's sizes, over > 600 MB of buffers
 static int rows_mode(size_t reduce_elems, size_t quant_elems) {
     {
@@ -176,6 +264,7 @@ static int rows_mode(size_t reduce_elems, size_t quant_elems) {
 
 int main(int argc, char** argv) {
     if (argc > 3 && std::string(argv[1]) == "rows") return rows_mode((size_t)atoll(argv[2]), (size_t)atoll(argv[3]));
+    if (argc > 1 && std::string(argv[1]) == "shape") return shape_mode();
     size_t bytes = (argc > 1 ? atol(argv[1]) : 100) * (size_t)1048576;
     int nbuf = 6;
     std::vector<float4v*> in(nbuf), out(nbuf);
