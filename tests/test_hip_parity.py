@@ -855,6 +855,76 @@ def test_pipeline_step_equals_its_three_launches_and_the_oracle(ops, hip_device,
             assert_same_bits(got[2][d * shard:stop], want[:stop - d * shard], f"decoded shard {d}")
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_shared_grids_equal_their_separate_launches(ops, hip_device, seed):
+    """Random bucket sizes, ranks, payload counts, types and stage subsets through both shared-grid entry points: every
+    byte they write equals what the separate launches write.  (A stage's place in the grid - its row and its position
+    in the row - comes out of a division by a run-time stride; sizes that are no round numbers walk that arithmetic.)"""
+    rng = np.random.default_rng(8800 + seed)
+    merged = 0
+    for case in range(40):
+        dtype = str(rng.choice(["fp32", "bf16", "fp16"]))
+        kind = DTYPES[dtype]
+        world = int(rng.integers(1, 9))
+        n = 64 * world * int(rng.choice([rng.integers(1, 40), rng.integers(40, 3000)]))
+        shard = n // world
+        with_residual = bool(rng.integers(0, 2))
+        what = f"seed {seed} case {case}: {dtype} n {n} world {world} residual {with_residual}"
+        nbytes = ops.payload_nbytes(shard)
+        stride = (nbytes + 255) // 256 * 256
+        grad = gradient_like(n, kind, 8900 + 50 * seed + case, hip_device)
+        residual = gradient_like(n, torch.float32, 8901 + case, hip_device, sigma=1e-5, outliers=False) if with_residual else None
+        keep = None if residual is None else residual.clone()
+        send = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+        quant = ops.bind_quant_pack_chunks(grad, send, world, residual=residual, new_residual=residual)
+
+        def restore():
+            send.zero_()
+            if residual is not None:
+                residual.copy_(keep)
+
+        # the two-stage entry point: quantize + reduce of `payloads` payloads of another length
+        payloads = int(rng.integers(1, 9))
+        reduce_n = 64 * int(rng.integers(1, 1200)) + int(rng.choice([0, 0, 17]))
+        peers = [ops.quant_pack(gradient_like(reduce_n, torch.float32, 9000 + r, hip_device)) for r in range(payloads)]
+        out = torch.zeros(reduce_n, dtype=kind if rng.integers(0, 2) else torch.float32, device=hip_device)
+        reduce = ops.bind_dequant_reduce(peers, out, divisor=float(payloads))
+        if ops.bind_quant_chunks_and_reduce(quant, reduce)():
+            merged += 1
+            got = (send.clone(), out.clone(), None if residual is None else residual.clone())
+            restore(); out.zero_()
+            assert quant() and reduce(), what
+            assert torch.equal(got[0], send) and torch.equal(got[1].view(torch.uint8), out.view(torch.uint8)), what
+            assert residual is None or torch.equal(got[2].view(torch.uint8), residual.view(torch.uint8)), what
+        restore()
+
+        # the three-stage entry point on a random subset of its stages
+        received = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+        gathered = torch.zeros(world, stride, dtype=torch.uint8, device=hip_device)
+        for r in range(world):
+            ops.quant_pack_payload_into(gradient_like(shard, kind, 9100 + r, hip_device), received[r, :nbytes])
+            ops.quant_pack_payload_into(gradient_like(shard, kind, 9200 + r, hip_device), gathered[r, :nbytes])
+        mine = torch.zeros(nbytes, dtype=torch.uint8, device=hip_device)
+        decoded = torch.zeros(n, dtype=kind, device=hip_device)
+        pairs = [ops.split_payload(received[r, :nbytes], shard) for r in range(world)]
+        requant = ops.bind_dequant_reduce_quant(pairs, *ops.split_payload(mine, shard), shard, divisor=float(world), mid_dtype=kind)
+        decode = ops.bind_dequant_chunks(gathered, decoded, shard)
+        stages = str(rng.choice(["qrd", "qr", "qd", "rd"]))
+        step = ops.bind_bucket_pipeline_step(quant if "q" in stages else None, requant if "r" in stages else None,
+                                             decode if "d" in stages else None)
+        if step():
+            merged += 1
+            got = (send.clone(), mine.clone(), decoded.clone(), None if residual is None else residual.clone())
+            restore(); mine.zero_(); decoded.zero_()
+            for name, launch in (("q", quant), ("r", requant), ("d", decode)):
+                if name in stages:
+                    assert launch(), what
+            assert torch.equal(got[0], send) and torch.equal(got[1], mine), f"{what} stages {stages}"
+            assert torch.equal(got[2].view(torch.uint8), decoded.view(torch.uint8)), f"{what} stages {stages}"
+            assert residual is None or torch.equal(got[3].view(torch.uint8), residual.view(torch.uint8)), f"{what} stages {stages}"
+    assert merged >= 40, "most of these combinations have a shared grid"
+
+
 def test_pipeline_step_without_a_shared_grid_says_so(ops, hip_device):
     """Another group size than 64, or operands that are not aligned for the vector kernels, have no shared grid: the
     bound step returns False and the caller issues the stages themselves."""
