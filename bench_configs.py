@@ -1128,6 +1128,53 @@ def main() -> int:
                 host_row(f"the same iteration ({lane_count} stream{'s' if lane_count > 1 else ''}, error feedback {feedback}) "
                          "as one HIP-graph replay, per bucket", host / stream_count, wall / stream_count)
                 del graph
+        # the all-gather form of the all-reduce over pre-bound plans, behind the hook's whole-collective seam: a bucket
+        # is quantized into one payload, the W payloads are gathered (W - 1 stand-in peers resident in HBM) and one
+        # fused launch reduces them into the bucket.  Sixteen buckets of sixteen sizes, so that every bucket has
+        # its own peers' payloads (1.6 GB in all) and no row reads them out of the last-level cache; the facade's own
+        # all_gather strategy runs over the same stream for comparison.
+        from lowbit_comm_amd.hip.reduce_scatter import make_all_gather_transport
+
+        varied = [StreamBucket(gen(SEED + 7600 + i, n - 64 * world * 8 * i, 1e-3, torch.bfloat16), i, i == stream_count - 1)
+                  for i in range(stream_count)]
+        whole_filled = set()
+
+        def whole_gather(received, mine):
+            if received.data_ptr() not in whole_filled:     # the peers' payloads stay where they are; row 0 is `mine`
+                for r in range(1, world):
+                    received[r, :mine.numel()].copy_(mine)
+                whole_filled.add(received.data_ptr())
+
+        for feedback in (False, True):
+            peers.clear()
+            hook = create_ddp_comm_hook(CompressionConfig(error_feedback=feedback), strategy="all_gather", reduce="mean",
+                                        all_gather=gather, extension_status=status, future_factory=Slot,
+                                        workspace_cache_max_entries=2 * stream_count)
+
+            def facade_iteration(_i=0):
+                for bucket in varied:
+                    hook(None, bucket)
+
+            host, wall = host_and_wall(facade_iteration, 12)
+            host_row(f"hook, all_gather strategy through the facade, stream of {stream_count} bf16 buckets of 22-25 MiB with their "
+                     f"own peers, W=8, error feedback {feedback}, per bucket", host / stream_count, wall / stream_count)
+            for pipelined in (False, True):
+                transport = make_all_gather_transport(world_size=world, rank=0, all_gather=whole_gather,
+                                                      error_feedback=feedback, pipelined=pipelined, future_factory=Slot)
+                hook = create_ddp_comm_hook(CompressionConfig(error_feedback=False), strategy="topology", reduce="mean",
+                                            topology_all_reduce=transport, future_factory=Slot)
+
+                def gather_iteration(_i=0):
+                    for bucket in varied:
+                        hook(None, bucket)
+
+                host, wall = host_and_wall(gather_iteration, 12)
+                host_row(f"hook, all-gather form over pre-bound plans ({'pipelined: one launch per bucket' if pipelined else 'two launches per bucket'}), "
+                         f"the same stream, W=8, {'local ' if feedback else ''}error feedback {feedback}, per bucket",
+                         host / stream_count, wall / stream_count)
+                del transport, hook
+        peers.clear()
+        del varied
         del stream_buckets
         # one pre-bound launch
         x = gen(SEED + 7100, n, 1e-3, torch.bfloat16)

@@ -39,7 +39,7 @@ import torch
 
 from lowbit_comm_amd.config import CompressionConfig
 from lowbit_comm_amd.hip import ops
-from lowbit_comm_amd.hip.reduce_scatter import ReduceScatterPlan, ResidualStore
+from lowbit_comm_amd.hip.reduce_scatter import AllGatherPlan, ReduceScatterPlan, ResidualStore
 
 
 class _Bucket:
@@ -96,6 +96,12 @@ class BucketPipeline:
     future resolves to the reduced bucket - decoded in place into ``tensor`` when ``inplace`` and the tensor is
     contiguous, else into a fresh tensor.
 
+    ``whole_gather(received_rows, my_payload)`` instead of ``all_to_all`` selects the all-gather form of the all-reduce
+    (the comm hook's ``all_gather`` strategy, ``ccdl_comm/communication/ddp_hook.py:190-330``): a bucket is quantized
+    into one payload, the ``W`` payloads are all-gathered and one fused launch reduces them into the bucket.  The
+    quantize of bucket k then shares its launch with the reduce of bucket k-1, and a future resolves to the reduced
+    bucket (in place under the same condition as above).
+
     ``error_feedback``: every bucket (keyed by storage address, element count and dtype) keeps an fp32 residual that
     its quantize adds before encoding and refreshes, in the same launch, with what the encoding dropped; beyond
     ``max_residuals`` buckets the least recently used residual is dropped.
@@ -109,19 +115,25 @@ class BucketPipeline:
     Calls from several threads are serialised by a lock; the buckets of one iteration still have to arrive in one
     order."""
 
-    def __init__(self, *, world_size: int, rank: int, all_to_all: Callable[[torch.Tensor, torch.Tensor], Any],
+    def __init__(self, *, world_size: int, rank: int, all_to_all: Callable[[torch.Tensor, torch.Tensor], Any] | None = None,
                  all_gather: Callable[[torch.Tensor, torch.Tensor], Any] | None = None, error_feedback: bool = False,
                  inplace: bool = True, lanes: int = 1, max_plans: int = 64, max_steps: int = 4096,
                  future_factory: Callable[[], Any] | None = None, plan_factory: Callable[..., Any] | None = None,
-                 merge_stages: Callable[..., Any] | None = None, max_residuals: int = 4096) -> None:
+                 merge_stages: Callable[..., Any] | None = None, max_residuals: int = 4096,
+                 whole_gather: Callable[[torch.Tensor, torch.Tensor], Any] | None = None) -> None:
         if not 0 <= rank < world_size:
             raise ValueError(f"rank must be in [0, {world_size})")
         if lanes < 1:
             raise ValueError("lanes must be at least 1")
+        if (all_to_all is None) == (whole_gather is None):
+            raise ValueError("give either all_to_all (reduce-scatter form) or whole_gather (all-gather form)")
+        if whole_gather is not None and all_gather is not None:
+            raise ValueError("the all-gather form has one exchange: whole_gather")
         self.world_size = world_size
         self.rank = rank
         self.all_to_all = all_to_all
         self.all_gather = all_gather
+        self.whole_gather = whole_gather
         self.error_feedback = bool(error_feedback)
         self.inplace = bool(inplace)
         self.depth = 3 if all_gather is not None else 2
@@ -130,7 +142,8 @@ class BucketPipeline:
         self.residuals = ResidualStore(max_residuals)
         self.stats = {"buckets": 0, "merged_launches": 0, "separate_launches": 0, "flushes": 0}
         self._future_factory = future_factory
-        self._plan_factory = plan_factory or ReduceScatterPlan     # replaceable: the scheduling is testable without a GPU
+        # replaceable: the scheduling is testable without a GPU
+        self._plan_factory = plan_factory or (AllGatherPlan if whole_gather is not None else ReduceScatterPlan)
         self._merge_stages = merge_stages or self._bind_merged
         self._dirty = False                                        # something was submitted since the last flush
         self._lock = threading.RLock()
@@ -261,10 +274,15 @@ class BucketPipeline:
             decode = decoding.plan.bound_decode(decoding.out, remember=decoding.lasting_out)
         self._launch(lane, quant, reduce, decode)
         if arriving is not None:
-            arriving.exchange = self.all_to_all(arriving.plan.received, arriving.plan.send)
+            if self.whole_gather is not None:
+                arriving.exchange = self.whole_gather(arriving.plan.received, arriving.plan.my_payload)
+            else:
+                arriving.exchange = self.all_to_all(arriving.plan.received, arriving.plan.send)
         if reducing is not None:
             if full:
                 reducing.gather = self.all_gather(reducing.plan.gathered, reducing.plan.my_row)
+            elif self.whole_gather is not None:
+                self._complete(reducing, reducing.out.reshape(reducing.tensor.shape))
             else:
                 self._complete(reducing, reducing.plan.reduced_shard(reducing.out, op=reducing.op, caller_owned=True))
         if decoding is not None:
@@ -287,8 +305,9 @@ class BucketPipeline:
             future = self.make_future()
             self.stats["buckets"] += 1
             full = self.all_gather is not None
+            whole = full or self.whole_gather is not None       # the result is the reduced bucket, not a shard
             if tensor.numel() == 0:           # nothing to exchange on any rank
-                future.set_result(tensor if full else
+                future.set_result(tensor if whole else
                                   self._plan_factory(0, tensor.dtype, world_size=self.world_size, rank=self.rank, config=config,
                                                      device=tensor.device, shape=tuple(tensor.shape))
                                   .reduced_shard(tensor.reshape(-1), op=op, fused=False, caller_owned=True))
@@ -302,7 +321,7 @@ class BucketPipeline:
             lane = lanes[index]
             plan = self._plan_for(tensor, config, index)
             lasting_out = out is not None
-            if full:
+            if whole:
                 if out is None:
                     lasting_out = self.inplace and tensor.is_contiguous()
                     out = tensor.reshape(-1) if lasting_out else torch.empty(

@@ -425,3 +425,60 @@ def test_hook_flushes_when_the_last_bucket_is_too_small_to_compress():
     assert pipe.pending == 1
     hook(None, Bucket(bucket_tensor(1, 10), 1, last=True))
     assert pipe.pending == 0 and first.done()
+
+
+# ---- the all-gather form: one payload per bucket, gathered whole, reduced into the bucket ------------------------------
+def make_gather_pipeline(log, **kwargs):
+    def merge(quant, reduce, decode):
+        assert decode is None
+        return FakeLaunch(log, ("MERGED",) + tuple(p.what for p in (quant, reduce) if p is not None))
+
+    def whole_gather(received, mine):
+        log.append(("gather", received, mine))
+
+    def plan(*a, **k):
+        made = FakePlan(*a, log=log, **k)
+        made.my_payload = ("payload", made.tag)
+        return made
+
+    FakePlan.made = 0
+    return BucketPipeline(world_size=8, rank=0, whole_gather=whole_gather, plan_factory=plan, merge_stages=merge,
+                          future_factory=torch.futures.Future, **kwargs)
+
+
+def test_all_gather_form_merges_the_quantize_with_the_previous_buckets_reduce():
+    log = []
+    pipe = make_gather_pipeline(log)
+    tensors = [bucket_tensor(k) for k in range(3)]
+    futures = [pipe.submit(t, config=CFG, op="mean") for t in tensors]
+    assert log == [
+        ("Q", 0, False), ("gather", ("received", 1), ("payload", 1)),
+        ("MERGED", ("Q", 1, False), ("R", 1, "mean")), ("gather", ("received", 2), ("payload", 2)),
+        ("MERGED", ("Q", 2, False), ("R", 2, "mean")), ("gather", ("received", 1), ("payload", 1)),   # two plans per shape
+    ]
+    assert [f.done() for f in futures] == [True, True, False] and pipe.pending == 1
+    pipe.flush()
+    assert log[-1] == ("R", 1, "mean") and futures[2].done() and pipe.pending == 0
+    for tensor, future in zip(tensors, futures):
+        assert future.wait().data_ptr() == tensor.data_ptr() and future.wait().shape == tensor.shape   # reduced in place
+
+
+def test_all_gather_form_with_error_feedback_hands_the_buckets_residual_to_the_quantize():
+    log = []
+    pipe = make_gather_pipeline(log, error_feedback=True)
+    first, second = bucket_tensor(0), bucket_tensor(1)
+    for _ in range(2):
+        pipe.submit(first, config=CFG)
+        pipe.submit(second, config=CFG)
+        pipe.flush()
+    assert [entry for entry in log if entry[0] == "Q"] == [("Q", 0, True), ("Q", 0, True)]
+    assert len(pipe.residuals) == 2
+
+
+def test_the_two_forms_exclude_each_other():
+    with pytest.raises(ValueError, match="either all_to_all"):
+        BucketPipeline(world_size=2, rank=0)
+    with pytest.raises(ValueError, match="either all_to_all"):
+        BucketPipeline(world_size=2, rank=0, all_to_all=lambda r, s: None, whole_gather=lambda r, m: None)
+    with pytest.raises(ValueError, match="one exchange"):
+        BucketPipeline(world_size=2, rank=0, whole_gather=lambda r, m: None, all_gather=lambda g, m: None)
