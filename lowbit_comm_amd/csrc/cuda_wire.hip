@@ -595,13 +595,22 @@ __global__ __launch_bounds__(kBlock) void wire_ring_step_kernel(const WireRingSt
         if (live[u]) {
             const float step = step_of<8>(widen(stored[u]));
 #pragma unroll
+            for (int i = 0; i < VEC; ++i) p[i] = unpack_code<T, 8, W::WORDS>(words[u], i) * step;
+            round_through_all<T, VEC>(p);
+            if constexpr (ACC) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) p[i] = widen(xv[u][i]) + p[i];
+                round_through_all<T, VEC>(p);
+            }
+            if (scaled) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) p[i] = p[i] * a.inv_divisor;
+                round_through_all<T, VEC>(p);
+            }
+            narrow_all<T, VEC>(p, held);
+#pragma unroll
             for (int i = 0; i < VEC; ++i) {
-                float v = round_through<T>(unpack_code<T, 8, W::WORDS>(words[u], i) * step);
-                if constexpr (ACC) v = add_in<T>(widen(xv[u][i]), v);
-                if (scaled) v = round_through<T>(v * a.inv_divisor);
-                held[i] = narrow<T>(v);
-                p[i] = v;
-                const uint32_t bits = as_u32(v) & 0x7FFFFFFFu;
+                const uint32_t bits = as_u32(p[i]) & 0x7FFFFFFFu;
                 m = bits > m ? bits : m;
             }
             store_elems<T, VEC, NT>(chunk + e0[u], held);

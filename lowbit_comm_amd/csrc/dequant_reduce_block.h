@@ -117,19 +117,21 @@ __device__ __forceinline__ void dequant_reduce_block(const ReduceArgs &a, unsign
         for (int u = 0; u < UNROLL; ++u) {
             float acc[VEC];
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[i] = round_through<OT>(code_to_float(words[u][0][i / 4], i % 4) * scale[u][0]);
+            for (int i = 0; i < VEC; ++i) acc[i] = code_to_float(words[u][0][i / 4], i % 4) * scale[u][0];
+            round_through_all<OT, VEC>(acc);
 #pragma unroll
             for (int r = 1; r < W; ++r) {
+                float t[VEC];
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) {
-                    const float t = round_through<OT>(code_to_float(words[u][r][i / 4], i % 4) * scale[u][r]);
-                    acc[i] = round_through<OT>(acc[i] + t);
-                }
+                for (int i = 0; i < VEC; ++i) t[i] = code_to_float(words[u][r][i / 4], i % 4) * scale[u][r];
+                round_through_all<OT, VEC>(t);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[i] += t[i];
+                round_through_all<OT, VEC>(acc);
             }
             if (mean) divide_all<OT, VEC>(acc, a.divisor);
             OT o[VEC];
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) o[i] = narrow<OT>(acc[i]);
+            narrow_all<OT, VEC>(acc, o);
             buffer_store<OT, VEC, kStore>(out_b, at[u] * sizeof(OT), o);
             if (new_r != nullptr) {
                 OT pv[VEC], d[VEC];
@@ -204,14 +206,17 @@ __device__ __forceinline__ void dequant_reduce_quant_block(const ReduceQuantArgs
             scale[r] = a.scales[r][g];
         }
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) p[i] = round_through<MT>(code_to_float(words[0][i / 4], i % 4) * scale[0]);
+        for (int i = 0; i < VEC; ++i) p[i] = code_to_float(words[0][i / 4], i % 4) * scale[0];
+        round_through_all<MT, VEC>(p);
 #pragma unroll
         for (int r = 1; r < W; ++r) {
+            float t[VEC];
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                const float t = round_through<MT>(code_to_float(words[r][i / 4], i % 4) * scale[r]);
-                p[i] = round_through<MT>(p[i] + t);
-            }
+            for (int i = 0; i < VEC; ++i) t[i] = code_to_float(words[r][i / 4], i % 4) * scale[r];
+            round_through_all<MT, VEC>(t);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) p[i] += t[i];
+            round_through_all<MT, VEC>(p);
         }
         if (mean) divide_all<MT, VEC>(p, a.divisor);
         if (e0 + VEC > a.numel) {

@@ -84,6 +84,46 @@ template <typename T> __device__ __forceinline__ float round_through(float v) {
     else return static_cast<float>(static_cast<T>(v));
 }
 
+// round_through<T> on every element of an array.  gfx950 rounds two floats to a bf16 pair in one instruction
+// (v_cvt_pk_bf16_f32); element by element the compiler spends one such instruction per value, pair by pair half as
+// many - same rounding, same results.
+template <typename T, int N> __device__ __forceinline__ void round_through_all(float (&v)[N]) {
+    if constexpr (same_t<T, float>::value) {
+        return;
+    } else if constexpr (same_t<T, bf16>::value && N % 2 == 0) {
+        using float2v = vec_t<float, 2>;
+        using bf16x2 = vec_t<bf16, 2>;
+#pragma unroll
+        for (int i = 0; i < N; i += 2) {
+            const float2v pair = {v[i], v[i + 1]};
+            const float2v back = __builtin_convertvector(__builtin_convertvector(pair, bf16x2), float2v);
+            v[i] = back.x;
+            v[i + 1] = back.y;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = round_through<T>(v[i]);
+    }
+}
+
+// narrow<T> of every element, pair by pair for bf16 for the same reason: the pair comes out packed in one register.
+template <typename T, int N> __device__ __forceinline__ void narrow_all(const float (&v)[N], T (&out)[N]) {
+    if constexpr (same_t<T, bf16>::value && N % 2 == 0) {
+        using float2v = vec_t<float, 2>;
+        using bf16x2 = vec_t<bf16, 2>;
+#pragma unroll
+        for (int i = 0; i < N; i += 2) {
+            const float2v pair = {v[i], v[i + 1]};
+            const bf16x2 packed = __builtin_convertvector(pair, bf16x2);
+            out[i] = packed.x;
+            out[i + 1] = packed.y;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) out[i] = narrow<T>(v[i]);
+    }
+}
+
 // ---- N-element contiguous load / store --------------------------------------
 template <typename T, int N, int MODE>
 __device__ __forceinline__ void load_vec(const T *__restrict__ p, T (&dst)[N]) {
@@ -307,11 +347,12 @@ template <typename T, int N> __device__ __forceinline__ void divide_all(float (&
     if ((bits & 0x007FFFFFu) == 0 && exponent >= 2 && exponent <= 252) {
         const float reciprocal = as_f32((254u - exponent) << 23);
 #pragma unroll
-        for (int i = 0; i < N; ++i) v[i] = round_through<T>(v[i] * reciprocal);
+        for (int i = 0; i < N; ++i) v[i] = v[i] * reciprocal;
     } else {
 #pragma unroll
-        for (int i = 0; i < N; ++i) v[i] = round_through<T>(v[i] / divisor);
+        for (int i = 0; i < N; ++i) v[i] = v[i] / divisor;
     }
+    round_through_all<T, N>(v);
 }
 
 // codes[i] = rint(p[i] / scale) as the reference computes it (IEEE division, then round-half-even), a NaN

@@ -73,14 +73,15 @@ __global__ __launch_bounds__(kBlock) void ring_step_kernel(const RingStepArgs a)
             float p[VEC];
             T out[VEC];
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                float v = round_through<T>(code_to_float(words[u][i / 4], i % 4) * rscale[u]);
-                if constexpr (ACC) v = round_through<T>(widen(xv[u][i]) + v);
-                p[i] = v;
+            for (int i = 0; i < VEC; ++i) p[i] = code_to_float(words[u][i / 4], i % 4) * rscale[u];
+            round_through_all<T, VEC>(p);
+            if constexpr (ACC) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) p[i] = widen(xv[u][i]) + p[i];
+                round_through_all<T, VEC>(p);
             }
             if (mean) divide_all<T, VEC>(p, a.divisor);
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) out[i] = narrow<T>(p[i]);
+            narrow_all<T, VEC>(p, out);
             store_wide<T, VEC, MODE>(chunk + e0[u], out);
             if (emit) {
                 const float scale = group_scale<VEC, LPG>(p);

@@ -628,8 +628,8 @@ def make_all_gather_transport(*, world_size: int, rank: int, all_gather: Callabl
     is true, so the comm hook flushes after the iteration's last bucket.  ``error_feedback`` keeps an fp32 residual per
     bucket (local error feedback, fused into the quantize launch; at most ``max_residuals`` of them).  More than eight
     ranks take the unpipelined plan, whose reduce then decodes payload by payload.  The form is bound by its reduce,
-    which reads ``W`` payloads: pipelining saves host time (15 against 19 us per 25 MiB bf16 bucket; 26 us through the
-    codec facade), not GPU time (36.6 us either way at W = 8)."""
+    which reads ``W`` payloads: pipelining saves host time (14 against 17 us per 25 MiB bf16 bucket; 24 us through the
+    codec facade), not GPU time (33-35 us either way at W = 8)."""
     residuals = ResidualStore(max_residuals)
     plans: OrderedDict[Any, AllGatherPlan] = OrderedDict()
     lock = threading.Lock()
