@@ -157,6 +157,10 @@ def parse_args():
     ap.add_argument("--sets", type=int, default=6, help="distinct buffer sets rotated through (defeats the LLC)")
     ap.add_argument("--deep-sets", type=int, default=24,
                     help="buffer sets of the deep-rotation legs (0 leaves them out); every set holds 0.5 GB")
+    ap.add_argument("--wide-sets", type=int, default=2,
+                    help="buffer sets of the whole-bucket reduce (0.33 GB a set) and error-feedback (0.58 GB a set) legs")
+    ap.add_argument("--wide-deep-sets", type=int, default=6,
+                    help="buffer sets of those two legs' deep-rotation variants (0 leaves them out)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma list of kernel legs to time (for profiling one kernel)")
     ap.add_argument("--record-traffic", nargs=2, metavar=("FETCH_DB", "WRITE_DB"),
@@ -323,8 +327,11 @@ def main() -> int:
     # ---- per-kernel launch durations ---------------------------------------------------------------
     kernels = {}
 
+    def wanted(name):
+        return not only or name in only or ("deep_rotation" in only and name.endswith("_deep_rotation"))
+
     def leg(name, fn, algorithmic_bytes, launches=None, warmup=None):
-        if only and name not in only:
+        if not wanted(name):
             return
         launches = launches or args.steps
         seconds = timed(fn, launches, warmup if warmup is not None else args.warmup)
@@ -373,7 +380,7 @@ def main() -> int:
             for name in ("gathered", "mine", "decoded", "reduce_requant", "decode", "pipeline_step"):
                 del s[name]
         torch.cuda.empty_cache()
-    if (not only or "deep_rotation" in only) and args.deep_sets > len(sets):
+    if (wanted("bucket_step_deep_rotation") or wanted("bucket_pipeline_step_deep_rotation")) and args.deep_sets > len(sets):
         # The same two launches with four times as many buffer sets in rotation (4 GB and 7 GB instead of 1 GB and
         # 1.8 GB between two uses of a buffer): launches that write much read a few percent slower this way although
         # the traffic that leaves the L2 is the same, so both figures are in the line.
@@ -422,32 +429,48 @@ def main() -> int:
         leg("copy_calibration", lambda i: dsts[i % 2].copy_(srcs[i % len(srcs)]), 2 * n * 4)
         del dsts
 
-    if not only or "dequant_reduce_full" in only or "ef_quant_pack" in only:
+    if any(wanted(k + d) for k in ("dequant_reduce_full", "ef_quant_pack") for d in ("", "_deep_rotation")):
+        # Both legs are timed twice: over --wide-sets buffer sets (two: 0.66 and 1.16 GB in rotation, past the
+        # last-level cache, within what the address-translation caches still cover) and over --wide-deep-sets (six),
+        # where every launch also pays for translation misses, as a stream of gradient buckets does.
+        def rotations(name):
+            for count, suffix in ((args.wide_sets, ""), (args.wide_deep_sets, "_deep_rotation")):
+                if count > 0 and (suffix == "" or count > args.wide_sets) and wanted(name + suffix):
+                    yield count, name + suffix
+
+        def run_over(launches):
+            return lambda i: launches[i % len(launches)]()
+
         # all-gather-reduce shape: 8 payloads of the whole bucket -> fp32 bucket
         full_sets = []
-        if not only or "dequant_reduce_full" in only:
-            for s in range(2):
+        for count, name in rotations("dequant_reduce_full"):
+            for s in range(len(full_sets), count):
                 pairs = [ops.quant_pack(gen(SEED + 7000 + 10 * s + r, n, 1e-3), group_size=g) for r in range(world)]
                 out = torch.empty(n, dtype=torch.float32, device=dev)
                 full_sets.append(ops.bind_dequant_reduce(pairs, out, group_size=g))
-            leg("dequant_reduce_full", lambda i: full_sets[i % 2](), world * ops.payload_nbytes(n, g) + n * 4,
-                launches=max(20, args.steps // 4), warmup=5)
-            del full_sets
-        if not only or "ef_quant_pack" in only:
-            # config 3: 100 MiB bf16 gradient + fp32 residual, residual updated in place
-            n3 = 52_428_800
-            groups3 = ops.num_groups(n3, g)
-            ef_sets = []
-            for s in range(2):
+            leg(name, run_over(full_sets[:count]), world * ops.payload_nbytes(n, g) + n * 4,
+                launches=max(24, args.steps // 4), warmup=6)
+            if name in kernels:
+                kernels[name]["buffer_sets"] = count
+        del full_sets
+        torch.cuda.empty_cache()
+        # config 3: 100 MiB bf16 gradient + fp32 residual, residual updated in place
+        n3 = 52_428_800
+        groups3 = ops.num_groups(n3, g)
+        ef_sets = []
+        for count, name in rotations("ef_quant_pack"):
+            for s in range(len(ef_sets), count):
                 grad = gen(SEED + 9000 + s, n3, 1e-3, torch.bfloat16)
                 residual = gen(SEED + 9100 + s, n3, 1e-5)
                 codes = torch.empty(groups3 * g, dtype=torch.int8, device=dev)
                 scales = torch.empty(groups3, dtype=torch.float32, device=dev)
                 ef_sets.append(ops.bind_quant_pack(grad, codes, scales, group_size=g, residual=residual,
                                                    new_residual=residual))
-            leg("ef_quant_pack", lambda i: ef_sets[i % 2](), n3 * (2 + 4 + 4) + groups3 * (g + 4),
-                launches=max(20, args.steps // 4), warmup=5)
-            del ef_sets
+            leg(name, run_over(ef_sets[:count]), n3 * (2 + 4 + 4) + groups3 * (g + 4),
+                launches=max(24, args.steps // 4), warmup=6)
+            if name in kernels:
+                kernels[name]["buffer_sets"] = count
+        del ef_sets
         torch.cuda.empty_cache()
 
     # ---- parity of the timed workload + CPU baseline (oracle, checker only) -------------------
