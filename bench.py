@@ -417,7 +417,9 @@ def main() -> int:
             out = torch.empty(shard, dtype=torch.float32, device=dev)
             pairs = [ops.split_payload(rows[r, :payload_bytes], shard, g) for r in range(world)]
             shard_sets.append(ops.bind_dequant_reduce(pairs, out, group_size=g))
-        leg("dequant_reduce_shard", lambda i: shard_sets[i % SHARD_SETS](), reduce_bytes)
+        # a launch of 8-9 us: batches of at least 96, so that the first launch after the synchronisation (which meets
+        # an idle GPU) does not weigh a twentieth of the figure
+        leg("dequant_reduce_shard", lambda i: shard_sets[i % SHARD_SETS](), reduce_bytes, launches=max(args.steps, 96))
         del shard_sets
         torch.cuda.empty_cache()
 
