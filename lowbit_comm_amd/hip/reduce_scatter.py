@@ -326,6 +326,24 @@ class AllGatherPlan(ReduceScatterPlan):
         del op, fused, caller_owned
         return target.reshape(self.shape)
 
+    def reduce_received(self, received: torch.Tensor | None = None, *, op: str = "sum",
+                        out: torch.Tensor | None = None) -> torch.Tensor:
+        if out is None:
+            raise ValueError("the all-gather plan keeps no output buffer: pass out= (the bucket, or a tensor of its size)")
+        return super().reduce_received(received, op=op, out=out)
+
+    def bound_reduce(self, received: torch.Tensor | None = None, *, op: str = "sum",
+                     out: torch.Tensor | None = None) -> ops.BoundLaunch:
+        if out is None:
+            raise ValueError("the all-gather plan keeps no output buffer: pass out= (the bucket, or a tensor of its size)")
+        return super().bound_reduce(received, op=op, out=out)
+
+    def _no_second_leg(self, *args: Any, **kwargs: Any) -> Any:
+        raise TypeError("the all-gather form ends with the reduce of the gathered payloads: it has no requantize, "
+                        "shard gather or decode step (those belong to ReduceScatterPlan)")
+
+    requantize_shard = reduce_and_requantize = bound_reduce_requantize = decode_gathered = bound_decode = _no_second_leg
+
     def run(self, tensor: torch.Tensor, all_gather: Callable[[torch.Tensor, torch.Tensor], Any], *, op: str = "mean",
             out: torch.Tensor | None = None, residual: torch.Tensor | None = None) -> torch.Tensor:
         """The three steps one after the other: quantize, ``all_gather(received_rows, my_payload)``, fused reduce into

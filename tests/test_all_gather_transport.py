@@ -175,3 +175,36 @@ def test_all_gather_transport_behind_the_comm_hook(hip_device, error_feedback, p
         want, _ = oracle(inputs[k], torch.zeros(sizes[k]) if error_feedback else None,
                          [t.cpu() for t in peers.tensors[sizes[k]]], "mean")
         assert same_bits(future.value().reshape(-1), want), f"bucket {k}"
+
+
+def test_all_gather_plan_refuses_the_steps_of_the_other_form(hip_device):
+    """The plan inherits the reduce-scatter plan's buffers and steps only as far as they apply: the reduce needs an
+    output from the caller (the plan keeps none), and the second leg's steps say that they do not exist here."""
+    from lowbit_comm_amd.hip.reduce_scatter import AllGatherPlan
+
+    n, world, rank = 64 * 40 + 17, 3, 1
+    plan = AllGatherPlan(n, torch.float32, world_size=world, rank=rank, config=CompressionConfig(), device=hip_device)
+    with pytest.raises(ValueError, match="pass out="):
+        plan.reduce_received(op="sum")
+    with pytest.raises(ValueError, match="pass out="):
+        plan.bound_reduce(op="sum")
+    for step in (plan.requantize_shard, plan.reduce_and_requantize, plan.bound_reduce_requantize, plan.decode_gathered):
+        with pytest.raises(TypeError, match="no requantize"):
+            step()
+    with pytest.raises(TypeError, match="no requantize"):
+        plan.bound_decode(torch.empty(n, device=hip_device))
+
+    # and the steps that do apply still give the oracle's result
+    bucket = grad(n, torch.float32, 31, hip_device)
+    peers = {r: grad(n, torch.float32, 40 + r, hip_device) for r in range(world) if r != rank}
+
+    def all_gather(received, mine):
+        for r, peer in peers.items():
+            codes, scales = codec_torch.quantize(peer.cpu(), 64)
+            received[r, :plan.payload_bytes].copy_(codec_torch.pack(codes, scales))
+
+    out = torch.empty(n, device=hip_device)
+    reduced = plan.run(bucket, all_gather, op="sum", out=out)
+    payloads = [codec_torch.quantize((bucket if r == rank else peers[r]).cpu(), 64) for r in range(world)]
+    want = codec_torch.reduce_payloads(payloads, n, 64, "fp32", "sum")
+    assert same_bits(reduced.cpu().reshape(-1), want)
