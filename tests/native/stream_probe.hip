@@ -5,8 +5,8 @@
 // these figures as well as against the 8 TB/s on the data sheet, and tests/test_zx_streaming_ceiling.py holds the hot
 // kernels to 0.9 of the row with their traffic mix.
 // Usage: stream_probe [MiB per buffer, default 100]           the table
-//        stream_probe rows <elements of a W=8 reduce> <elements of an fp32 quantize>
-//                                                             two machine-readable rows: "ROW name microseconds bytes"
+//        stream_probe rows <elements of a W=8 reduce> <elements of an fp32 quantize> [<elements of a 16-bit quantize>]
+//                                                             machine-readable rows: "ROW name microseconds bytes"
 // Not part of the product.
 #include <hip/hip_runtime.h>
 #include <cstdio>
@@ -98,6 +98,23 @@ __global__ __launch_bounds__(256) void quantlike_nt_kernel(const float4v* __rest
     for (int u = 0; u < UNROLL; ++u) {
         size_t i = base + (size_t)u * 256;
         if (i < n4) __builtin_nontemporal_store(__builtin_bit_cast(unsigned, v[u].x + v[u].y + v[u].z + v[u].w), out + i);
+    }
+}
+
+// 2:1 read:write, the traffic of an 8-bit quantize of 16-bit elements (read 16 B, write 8 B per lane)
+typedef unsigned uint2v __attribute__((ext_vector_type(2)));
+template <int UNROLL, bool NT_STORE>
+__global__ __launch_bounds__(256) void quantlike16_kernel(const float4v* __restrict__ in, uint2v* __restrict__ out, size_t n4) {
+    size_t base = (size_t)blockIdx.x * 256 * UNROLL + threadIdx.x;
+    float4v v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) { size_t i = base + (size_t)u * 256; if (i < n4) v[u] = __builtin_nontemporal_load(in + i); }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        size_t i = base + (size_t)u * 256;
+        if (i >= n4) continue;
+        const uint2v o = {__builtin_bit_cast(unsigned, v[u].x + v[u].y), __builtin_bit_cast(unsigned, v[u].z + v[u].w)};
+        if (NT_STORE) __builtin_nontemporal_store(o, out + i); else out[i] = o;
     }
 }
 
@@ -229,7 +246,7 @@ static int shape_mode() {
 }
 
 // "rows" mode: the two traffic mixes the hot kernels are held to, at the caller's sizes, over > 600 MB of buffers
-static int rows_mode(size_t reduce_elems, size_t quant_elems) {
+static int rows_mode(size_t reduce_elems, size_t quant_elems, size_t quant16_elems) {
     {
         const size_t n4 = reduce_elems / 4, groups = reduce_elems / 64;
         const size_t per_set = 8 * (reduce_elems + groups * 4) + reduce_elems * 4;
@@ -258,12 +275,24 @@ static int rows_mode(size_t reduce_elems, size_t quant_elems) {
         const unsigned grid = (unsigned)((n4 + 1023) / 1024);
         double t = run([&](int b) { quantlike_nt_kernel<4><<<grid, 256>>>(in[b], out[b], n4); }, 10 * sets, sets);
         printf("ROW quant_like_fp32 %.3f %zu\n", t * 1e6, per_set);
+        for (int i = 0; i < sets; ++i) { CK(hipFree(in[i])); CK(hipFree(out[i])); }
+    }
+    if (quant16_elems) {   // optional third row: 16-bit elements, 8-bit codes
+        const size_t n4 = quant16_elems / 8, per_set = quant16_elems * 2 + quant16_elems;
+        const int sets = (int)((size_t)640000000 / per_set) + 1;
+        std::vector<float4v*> in(sets); std::vector<uint2v*> out(sets);
+        for (int i = 0; i < sets; ++i) { CK(hipMalloc(&in[i], quant16_elems * 2)); CK(hipMalloc(&out[i], quant16_elems)); CK(hipMemset(in[i], 1, quant16_elems * 2)); }
+        const unsigned grid = (unsigned)((n4 + 1023) / 1024);
+        double plain = run([&](int b) { quantlike16_kernel<4, false><<<grid, 256>>>(in[b], out[b], n4); }, 10 * sets, sets);
+        double hinted = run([&](int b) { quantlike16_kernel<4, true><<<grid, 256>>>(in[b], out[b], n4); }, 10 * sets, sets);
+        printf("ROW quant_like_16bit %.3f %zu\n", plain * 1e6, per_set);
+        printf("ROW quant_like_16bit_nt_store %.3f %zu\n", hinted * 1e6, per_set);
     }
     return 0;
 }
 
 int main(int argc, char** argv) {
-    if (argc > 3 && std::string(argv[1]) == "rows") return rows_mode((size_t)atoll(argv[2]), (size_t)atoll(argv[3]));
+    if (argc > 3 && std::string(argv[1]) == "rows") return rows_mode((size_t)atoll(argv[2]), (size_t)atoll(argv[3]), argc > 4 ? (size_t)atoll(argv[4]) : 0);
     if (argc > 1 && std::string(argv[1]) == "shape") return shape_mode();
     size_t bytes = (argc > 1 ? atol(argv[1]) : 100) * (size_t)1048576;
     int nbuf = 6;
