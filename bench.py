@@ -502,7 +502,7 @@ def main() -> int:
         ok = ok and torch.equal(s0["out"].cpu().view(torch.int32), reduced.view(torch.int32))
         parity = "bit-exact" if ok else "MISMATCH"
         # A bounded sample of the same step: repeats for about ten seconds of CPU work, so that the figure is the
-        # host's steady state and not that of a cold thread pool (hosts still differ: 2.6 to 12 GB/s were seen).
+        # host's steady state and not that of a cold thread pool (hosts still differ: 2.0 to 14 GB/s were seen).
         times = []
         deadline = time.perf_counter() + CPU_SAMPLE_SECONDS
         while len(times) < 3 or (time.perf_counter() < deadline and len(times) < 5000):
