@@ -7,6 +7,7 @@
 // Usage: stream_probe [MiB per buffer, default 100]           the table
 //        stream_probe rows <elements of a W=8 reduce> <elements of an fp32 quantize> [<elements of a 16-bit quantize>]
 //                                                             machine-readable rows: "ROW name microseconds bytes"
+//        stream_probe depth                                   the plain kernels against the number of buffers in rotation
 // Not part of the product.
 #include <hip/hip_runtime.h>
 #include <cstdio>
@@ -291,7 +292,30 @@ static int rows_mode(size_t reduce_elems, size_t quant_elems, size_t quant16_ele
     return 0;
 }
 
+// "depth" mode: the plain read, write, copy and quantize-like kernels on 100 MiB buffers while the number of buffers
+// (pairs) in rotation grows from 2 to 32: how much of a launch's time depends on how long ago its pages were last
+// touched, for kernels that do nothing but move bytes.
+static int depth_mode() {
+    const size_t bytes = (size_t)100 << 20, n4 = bytes / 16;
+    const int most = 32;
+    std::vector<float4v*> in(most), out(most);
+    for (int i = 0; i < most; ++i) { CK(hipMalloc(&in[i], bytes)); CK(hipMalloc(&out[i], bytes)); CK(hipMemset(in[i], 1, bytes)); CK(hipMemset(out[i], 0, bytes)); }
+    float* flag; CK(hipMalloc(&flag, 4));
+    printf("buffers in rotation (100 MiB each, a read and a write buffer per step)   read U=2   write U=4 nt   copy U=4 nt   16B in / 4B out nt   us\n");
+    for (int nbuf : {2, 3, 4, 6, 8, 12, 16, 24, 32}) {
+        const int iters = nbuf * 4 < 48 ? 48 : nbuf * 4;
+        auto best_of3 = [&](auto launch) { double best = 1e9; for (int r = 0; r < 3; ++r) { const double t = run(launch, iters, nbuf); best = t < best ? t : best; } return best; };
+        const double r = best_of3([&](int b){ read_kernel<2,false><<<(unsigned)((n4 + 511) / 512),256>>>(in[b], flag, n4); });
+        const double w = best_of3([&](int b){ write_kernel<4,true><<<(unsigned)((n4 + 1023) / 1024),256>>>(out[b], n4); });
+        const double c = best_of3([&](int b){ copy_kernel<4,true><<<(unsigned)((n4 + 1023) / 1024),256>>>(in[b], out[b], n4); });
+        const double q = best_of3([&](int b){ quantlike_nt_kernel<4><<<(unsigned)((n4 + 1023) / 1024),256>>>(in[b], (unsigned*)out[b], n4); });
+        printf("DEPTH %2d   %8.2f   %8.2f   %8.2f   %8.2f\n", nbuf, r * 1e6, w * 1e6, c * 1e6, q * 1e6); fflush(stdout);
+    }
+    return 0;
+}
+
 int main(int argc, char** argv) {
+    if (argc > 1 && std::string(argv[1]) == "depth") return depth_mode();
     if (argc > 3 && std::string(argv[1]) == "rows") return rows_mode((size_t)atoll(argv[2]), (size_t)atoll(argv[3]), argc > 4 ? (size_t)atoll(argv[4]) : 0);
     if (argc > 1 && std::string(argv[1]) == "shape") return shape_mode();
     size_t bytes = (argc > 1 ? atol(argv[1]) : 100) * (size_t)1048576;
